@@ -1,0 +1,280 @@
+/*
+ * C ABI of libnfn_mi355_tile_ops.so — the K-Quant packed-linear operators of
+ * NeuralFn's tile-ops sidecar, implemented for AMD MI355X (gfx950).
+ *
+ * Every `nfn_native_tile_*` entry point below keeps the name, argument order
+ * and meaning of the declaration it replaces in the reference's
+ * neuralfn/csrc/native_train/tile_ops.h (cited per function), so the
+ * reference's resident engine can dlopen this library through its
+ * `tile_ops_lib` option.  `nfn_mi355_*` entry points are additions; each says
+ * what it adds and that no reference counterpart exists.
+ *
+ * Conventions (reference: tile_ops.cu:4504-4713, glimmer_k_mmq.cu:2349-2649):
+ *  - Return `int`: 0 on success, 1 (invalid value) for every argument or
+ *    descriptor violation, any other value is a HIP runtime error code that
+ *    nfn_native_tile_ops_error_string() turns into text.
+ *  - All data pointers are device pointers.  Descriptor structs and arrays of
+ *    descriptor/output pointers are host memory, read during the call only.
+ *  - The caller owns every buffer.  No entry point allocates, frees,
+ *    synchronises or keeps a pointer after it returns.
+ *  - `cuda_stream` is an opaque stream handle: here a hipStream_t.  Null is the
+ *    default stream.  Entry points without a stream argument use
+ *    descriptor->cuda_stream.
+ *  - Work is enqueued; the status reflects argument checks and the launch.
+ *  - Tensors: input [rows, input_dim] row-major float; each output
+ *    [rows, output_dim] row-major float; bias [output_dim] float, added after
+ *    the reduction.
+ */
+#ifndef NFN_MI355_TILE_OPS_H
+#define NFN_MI355_TILE_OPS_H
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Encoding ids (tile_ops.h:11-26).  8 = ggml Q8_0 is an addition: the reference
+ * accepts only 0, 12, 13, 14, 30 (and a training-only 31, rejected here). */
+enum {
+    NFN_NATIVE_TILE_PACKED_WEIGHT_V1 = 1,
+    NFN_NATIVE_TILE_K_QUANT_MMQ_V1 = 1,
+    NFN_NATIVE_TILE_PACKED_WEIGHT_F32 = 0,
+    NFN_MI355_PACKED_WEIGHT_Q8_0 = 8,
+    NFN_NATIVE_TILE_PACKED_WEIGHT_Q4_K = 12,
+    NFN_NATIVE_TILE_PACKED_WEIGHT_Q5_K = 13,
+    NFN_NATIVE_TILE_PACKED_WEIGHT_Q6_K = 14,
+    NFN_NATIVE_TILE_PACKED_WEIGHT_BF16 = 30
+};
+
+/* One [output_dim, input_dim] row-major packed matrix (tile_ops.h:293-307).
+ * 72 bytes.  Row r starts at data + r*row_stride_bytes; rows are unpadded:
+ * row_stride_bytes == input_dim/block_elements*block_bytes and
+ * data_nbytes == output_dim*row_stride_bytes, or validation fails. */
+typedef struct NfnNativeTilePackedWeightDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version;   /* NFN_NATIVE_TILE_PACKED_WEIGHT_V1 */
+    uint32_t encoding;
+    uint32_t flags;     /* 0 */
+    const uint8_t* data;
+    int64_t data_nbytes;
+    int64_t output_dim;
+    int64_t input_dim;
+    int64_t row_stride_bytes;
+    uint32_t reserved0; /* 0 */
+    uint32_t reserved1; /* 0 */
+    void* cuda_stream;
+} NfnNativeTilePackedWeightDescriptorV1;
+
+/* ---- versions (tile_ops.h:601-606; engine requires the first four == 1,
+ *      resident_glimmer_cuda.cpp:496-501) -------------------------------- */
+int nfn_native_tile_ops_abi_version(void);
+int nfn_native_tile_strict_math_abi_version(void);
+int nfn_native_tile_packed_weight_abi_version(void);
+int nfn_native_tile_glimmer_inference_abi_version(void);
+int nfn_native_tile_k_quant_mmq_abi_version(void);
+
+/* tile_ops.h:1096.  Never returns null. */
+const char* nfn_native_tile_ops_error_string(int code);
+
+/* ---- validation and dequantization (tile_ops.h:609-613) ----------------- */
+int nfn_native_tile_packed_weight_validate_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor);
+/* output: [output_dim, input_dim] float, bit-exact with the reference's
+ * packed_weight_value_device (kernels.cu:1225-1322). */
+int nfn_native_tile_packed_weight_dequantize_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    float* output);
+
+/* ---- generic float-activation linear, any row count (tile_ops.h:614-620).
+ *      rows <= 16 run a float GEMV; larger row counts with a K-quant weight
+ *      run the MFMA dequant-GEMM. ------------------------------------------ */
+int nfn_native_tile_linear_packed_weight_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const float* input,
+    const float* bias,
+    float* output,
+    int64_t rows,
+    bool has_bias);
+
+/* ---- public Q8_1 activation path (tile_ops.h:624-640, 743-756) ----------
+ * q8_values: rows*width int8; q8_scales, q8_sums: rows*(width/32) float. */
+int nfn_native_tile_quantize_q8_1_float32_v1(
+    const float* input,
+    int8_t* q8_values,
+    float* q8_scales,
+    float* q8_sums,
+    int64_t rows,
+    int64_t width,
+    void* cuda_stream);
+int nfn_native_tile_linear_packed_weight_q8_1_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const int8_t* q8_values,
+    const float* q8_scales,
+    const float* q8_sums,
+    const float* bias,
+    float* output,
+    int64_t rows,
+    bool has_bias);
+int nfn_native_tile_linear_packed_weight_q8_1_multi_decode_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor0,
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor1,
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor2,
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor3,
+    const int8_t* q8_values,
+    const float* q8_scales,
+    const float* q8_sums,
+    float* output0,
+    float* output1,
+    float* output2,
+    float* output3,
+    int64_t projection_count,
+    void* cuda_stream);
+
+/* ---- decode / small-batch K-quant path (tile_ops.h:647-739) --------------
+ * 1..4 projections that share one input, rows 1..16, Q4_K/Q5_K/Q6_K (and
+ * Q8_0 here).  `workspace` is caller-owned scratch whose layout is private to
+ * this library; its size comes from the query.  The query returns 0 when rows
+ * is outside 1..16 or input_dim is not a multiple of 128. */
+int64_t nfn_native_tile_k_quant_mmq_workspace_bytes_v1(int64_t rows, int64_t input_dim);
+int nfn_native_tile_k_quant_mmq_multi_linear_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* input,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+/* input := input / (1 + expf(-gate)), fused (tile_ops.h:659-672). */
+int nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* input,
+    const float* gate,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+/* input := (up * gate) * (1 / (1 + expf(-gate))), fused (tile_ops.h:673-684). */
+int nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* gate,
+    const float* up,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+/* Verifier variants: every row gets exactly the one-row arithmetic
+ * (tile_ops.h:685-729). */
+int nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* input,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* input,
+    const float* gate,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+int nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* gate,
+    const float* up,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+/* One-row decode GEMV (tile_ops.h:730-739). */
+int nfn_native_tile_k_quant_mmvq_linear_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const float* input,
+    float* output,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+
+/* ---- row argmax, ties to the lowest column (tile_ops.h:757-764) --------- */
+int nfn_native_tile_argmax_rows_float32_v1(
+    const float* values,
+    int64_t* output_indices,
+    float* output_values,
+    int64_t rows,
+    int64_t width,
+    void* cuda_stream);
+
+/* ---- element-wise operators the fused prologues must equal bit for bit
+ *      (tile_ops.h:998-1003, 3251-3256) ----------------------------------- */
+int nfn_native_tile_glimmer_sigmoid_gate_float32_v1(
+    const float* values,
+    const float* gate,
+    float* output,
+    int64_t count,
+    void* cuda_stream);
+int nfn_native_tile_swiglu_float32(
+    const float* gate,
+    const float* up,
+    float* out,
+    int64_t n,
+    void* cuda_stream);
+
+/* ==== additions: no counterpart in the reference ========================= */
+
+int nfn_mi355_abi_version(void);
+
+/* lm_head GEMV with the argmax fused in: logits never reach memory.  The
+ * reference runs mmvq_linear into an 808 KB logits buffer and then
+ * argmax_rows over it (resident_glimmer_cuda.cpp:4087-4151, 2661-2704); this
+ * is both in one call.  rows 1..8.  Ties go to the lowest index; NaN never
+ * wins.  output_indices: int64[rows]; output_values: float[rows]. */
+int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(int64_t rows, int64_t output_dim);
+int nfn_mi355_lm_head_argmax_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const float* input,
+    int64_t* output_indices,
+    float* output_values,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+
+/* Prefill dequant-GEMM for any row count: output[rows, output_dim] =
+ * input[rows, input_dim] * W^T.  The reference's small-batch entry points stop
+ * at 16 rows (glimmer_k_mmq.cu:1326-1328) and its only route for more rows is
+ * the generic linear above.  mode selects the MFMA operand type. */
+enum {
+    NFN_MI355_GEMM_BF16 = 0, /* weights dequantized to bf16 in LDS, bf16 MFMA */
+    NFN_MI355_GEMM_INT8 = 1  /* activations int8 per 32 values, int8 MFMA     */
+};
+int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+    int64_t rows, int64_t input_dim, int64_t output_dim, int mode);
+int nfn_mi355_k_quant_gemm_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const float* input,
+    float* output,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    int mode,
+    void* cuda_stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NFN_MI355_TILE_OPS_H */

@@ -1,0 +1,359 @@
+// extern "C" surface of libnfn_mi355_tile_ops.so: argument checks, then one or
+// two launches on the caller's stream.  Nothing here allocates, synchronises
+// or keeps state between calls.  Reference wrappers:
+// neuralfn/csrc/native_train/tile_ops.cu:4504-4713 and
+// neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:2349-2649.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "lm_head.hpp"
+
+#include <limits>
+
+namespace nfn {
+
+namespace {
+
+constexpr std::int64_t kMaxSmallRows = 16;
+constexpr std::int64_t kMaxOperations = 4;
+// Private activation record of the small-batch path: per 32 values two int8
+// planes (high and low byte of a 16-bit fixed-point code), a float scale and
+// the float sum of the 32 inputs.
+constexpr std::int64_t kActivationGroupBytes = 72;
+
+std::int64_t small_batch_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
+    if (rows < 1 || rows > kMaxSmallRows || input_dim <= 0 || input_dim % 128 != 0) return 0;
+    const std::int64_t groups = (input_dim + 31) / 32;
+    if (groups > std::numeric_limits<std::int64_t>::max() / (kActivationGroupBytes * rows)) {
+        return 0;
+    }
+    const std::int64_t raw = rows * groups * kActivationGroupBytes;
+    return (raw + 255) & ~std::int64_t(255);
+}
+
+Projection make_projection(const Descriptor& descriptor, float* output) {
+    Projection op{};
+    op.data = descriptor.data;
+    op.output = output;
+    op.output_dim = descriptor.output_dim;
+    op.row_stride = descriptor.row_stride_bytes;
+    op.encoding = descriptor.encoding;
+    op.first_tile = 0;
+    return op;
+}
+
+// Shared body of the small-batch entry points.
+int run_small_batch(const Descriptor* const* descriptors, const float* first,
+                    const float* second, int prologue, float* const* outputs,
+                    std::int64_t operation_count, std::int64_t rows, void* workspace,
+                    std::int64_t workspace_nbytes, void* stream) {
+    if (descriptors == nullptr || first == nullptr || outputs == nullptr ||
+        operation_count < 1 || operation_count > kMaxOperations || workspace == nullptr ||
+        workspace_nbytes <= 0 || (prologue != kPlain && second == nullptr)) {
+        return kInvalid;
+    }
+    const std::int64_t input_dim = descriptors[0] == nullptr ? 0 : descriptors[0]->input_dim;
+    ProjectionSet set{};
+    set.count = static_cast<int>(operation_count);
+    set.input_dim = input_dim;
+    for (std::int64_t index = 0; index < operation_count; ++index) {
+        if (outputs[index] == nullptr ||
+            !validate_k_descriptor(descriptors[index], input_dim, stream, true)) {
+            return kInvalid;
+        }
+        set.op[index] = make_projection(*descriptors[index], outputs[index]);
+    }
+    const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    launch_gemv_f32(set, first, second, prologue, nullptr, rows, as_stream(stream));
+    return launch_status();
+}
+
+}  // namespace
+
+}  // namespace nfn
+
+using namespace nfn;
+
+extern "C" {
+
+int nfn_native_tile_ops_abi_version(void) { return 1; }
+// Strict math: no fast-math flags, correctly rounded division and square root,
+// no contraction of the reference's two-rounding weight decode.
+int nfn_native_tile_strict_math_abi_version(void) { return 1; }
+int nfn_native_tile_packed_weight_abi_version(void) { return NFN_NATIVE_TILE_PACKED_WEIGHT_V1; }
+int nfn_native_tile_glimmer_inference_abi_version(void) { return 1; }
+int nfn_native_tile_k_quant_mmq_abi_version(void) { return NFN_NATIVE_TILE_K_QUANT_MMQ_V1; }
+int nfn_mi355_abi_version(void) { return 1; }
+
+const char* nfn_native_tile_ops_error_string(int code) {
+    const char* text = hipGetErrorString(static_cast<hipError_t>(code));
+    return text != nullptr ? text : "unknown error";
+}
+
+int nfn_native_tile_packed_weight_validate_v1(const Descriptor* descriptor) {
+    Descriptor normalized{};
+    return normalize_descriptor(descriptor, &normalized) ? 0 : kInvalid;
+}
+
+int nfn_native_tile_packed_weight_dequantize_float32_v1(const Descriptor* descriptor,
+                                                        float* output) {
+    Descriptor normalized{};
+    if (!normalize_descriptor(descriptor, &normalized) || output == nullptr) return kInvalid;
+    launch_dequantize(normalized, output, as_stream(normalized.cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_linear_packed_weight_float32_v1(const Descriptor* descriptor,
+                                                    const float* input, const float* bias,
+                                                    float* output, std::int64_t rows,
+                                                    bool has_bias) {
+    Descriptor normalized{};
+    if (!normalize_descriptor(descriptor, &normalized) || input == nullptr ||
+        output == nullptr || rows <= 0 || (has_bias && bias == nullptr)) {
+        return kInvalid;
+    }
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = normalized.input_dim;
+    set.op[0] = make_projection(normalized, output);
+    const hipStream_t stream = as_stream(normalized.cuda_stream);
+    constexpr std::int64_t kChunk = 65535 * 8;
+    for (std::int64_t row = 0; row < rows; row += kChunk) {
+        const std::int64_t count = rows - row < kChunk ? rows - row : kChunk;
+        set.op[0].output = output + row * normalized.output_dim;
+        launch_gemv_f32(set, input + row * normalized.input_dim, nullptr, kPlain,
+                        has_bias ? bias : nullptr, count, stream);
+    }
+    return launch_status();
+}
+
+int nfn_native_tile_quantize_q8_1_float32_v1(const float* input, std::int8_t* q8_values,
+                                             float* q8_scales, float* q8_sums,
+                                             std::int64_t rows, std::int64_t width,
+                                             void* cuda_stream) {
+    if (input == nullptr || q8_values == nullptr || q8_scales == nullptr ||
+        q8_sums == nullptr || rows <= 0 || width <= 0 || width % 32 != 0) {
+        return kInvalid;
+    }
+    launch_quantize_q8_1(input, q8_values, q8_scales, q8_sums, rows, width,
+                         as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_linear_packed_weight_q8_1_float32_v1(
+    const Descriptor* descriptor, const std::int8_t* q8_values, const float* q8_scales,
+    const float* q8_sums, const float* bias, float* output, std::int64_t rows, bool has_bias) {
+    Descriptor normalized{};
+    if (!normalize_descriptor(descriptor, &normalized) || q8_values == nullptr ||
+        q8_scales == nullptr || q8_sums == nullptr || output == nullptr || rows <= 0 ||
+        (has_bias && bias == nullptr) || normalized.input_dim % 256 != 0 ||
+        !is_k_quant(normalized.encoding)) {
+        return kInvalid;
+    }
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = normalized.input_dim;
+    const hipStream_t stream = as_stream(normalized.cuda_stream);
+    const std::int64_t groups = normalized.input_dim / 32;
+    constexpr std::int64_t kChunk = 65535;
+    for (std::int64_t row = 0; row < rows; row += kChunk) {
+        const std::int64_t count = rows - row < kChunk ? rows - row : kChunk;
+        set.op[0] = make_projection(normalized, output + row * normalized.output_dim);
+        launch_linear_q8_1(set, q8_values + row * normalized.input_dim, q8_scales + row * groups,
+                           q8_sums + row * groups, has_bias ? bias : nullptr, count, stream);
+    }
+    return launch_status();
+}
+
+int nfn_native_tile_linear_packed_weight_q8_1_multi_decode_float32_v1(
+    const Descriptor* descriptor0, const Descriptor* descriptor1, const Descriptor* descriptor2,
+    const Descriptor* descriptor3, const std::int8_t* q8_values, const float* q8_scales,
+    const float* q8_sums, float* output0, float* output1, float* output2, float* output3,
+    std::int64_t projection_count, void* cuda_stream) {
+    const Descriptor* descriptors[4] = {descriptor0, descriptor1, descriptor2, descriptor3};
+    float* outputs[4] = {output0, output1, output2, output3};
+    if (projection_count < 2 || projection_count > 4 || q8_values == nullptr ||
+        q8_scales == nullptr || q8_sums == nullptr) {
+        return kInvalid;
+    }
+    ProjectionSet set{};
+    set.count = static_cast<int>(projection_count);
+    for (int index = 0; index < 4; ++index) {
+        if (index >= projection_count) {
+            // Unused slots must be null (tile_ops.cu:4669-4683).
+            if (descriptors[index] != nullptr || outputs[index] != nullptr) return kInvalid;
+            continue;
+        }
+        Descriptor normalized{};
+        if (descriptors[index] == nullptr || outputs[index] == nullptr ||
+            !normalize_descriptor(descriptors[index], &normalized) ||
+            normalized.input_dim % 256 != 0 || !is_k_quant(normalized.encoding)) {
+            return kInvalid;
+        }
+        if (index == 0) set.input_dim = normalized.input_dim;
+        if (normalized.input_dim != set.input_dim) return kInvalid;
+        set.op[index] = make_projection(normalized, outputs[index]);
+    }
+    launch_linear_q8_1(set, q8_values, q8_scales, q8_sums, nullptr, 1, as_stream(cuda_stream));
+    return launch_status();
+}
+
+std::int64_t nfn_native_tile_k_quant_mmq_workspace_bytes_v1(std::int64_t rows,
+                                                            std::int64_t input_dim) {
+    return small_batch_workspace_bytes(rows, input_dim);
+}
+
+int nfn_native_tile_k_quant_mmq_multi_linear_float32_v1(
+    const Descriptor* const* descriptors, const float* input, float* const* outputs,
+    std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1(
+    const Descriptor* const* descriptors, const float* input, const float* gate,
+    float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    if (gate == nullptr) return kInvalid;
+    return run_small_batch(descriptors, input, gate, kGated, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1(
+    const Descriptor* const* descriptors, const float* gate, const float* up,
+    float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    if (gate == nullptr || up == nullptr) return kInvalid;
+    return run_small_batch(descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1(
+    const Descriptor* const* descriptors, const float* input, float* const* outputs,
+    std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
+    const Descriptor* const* descriptors, const float* input, const float* gate,
+    float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    if (gate == nullptr) return kInvalid;
+    return run_small_batch(descriptors, input, gate, kGated, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1(
+    const Descriptor* const* descriptors, const float* gate, const float* up,
+    float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
+    std::int64_t workspace_nbytes, void* cuda_stream) {
+    if (gate == nullptr || up == nullptr) return kInvalid;
+    return run_small_batch(descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
+                           workspace, workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_k_quant_mmvq_linear_float32_v1(const Descriptor* descriptor,
+                                                   const float* input, float* output,
+                                                   void* workspace,
+                                                   std::int64_t workspace_nbytes,
+                                                   void* cuda_stream) {
+    const Descriptor* descriptors[1] = {descriptor};
+    float* outputs[1] = {output};
+    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, 1, 1, workspace,
+                           workspace_nbytes, cuda_stream);
+}
+
+int nfn_native_tile_argmax_rows_float32_v1(const float* values, std::int64_t* output_indices,
+                                           float* output_values, std::int64_t rows,
+                                           std::int64_t width, void* cuda_stream) {
+    if (values == nullptr || output_indices == nullptr || output_values == nullptr ||
+        rows <= 0 || width <= 0 || rows > 0x7fffffff) {
+        return kInvalid;
+    }
+    launch_argmax_rows(values, output_indices, output_values, rows, width,
+                       as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_sigmoid_gate_float32_v1(const float* values, const float* gate,
+                                                    float* output, std::int64_t count,
+                                                    void* cuda_stream) {
+    if (values == nullptr || gate == nullptr || output == nullptr || count <= 0) return kInvalid;
+    launch_sigmoid_gate(values, gate, output, count, as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_swiglu_float32(const float* gate, const float* up, float* out,
+                                   std::int64_t n, void* cuda_stream) {
+    if (gate == nullptr || up == nullptr || out == nullptr || n <= 0) return kInvalid;
+    launch_swiglu(gate, up, out, n, as_stream(cuda_stream));
+    return launch_status();
+}
+
+std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
+                                                         std::int64_t output_dim) {
+    if (rows < 1 || rows > 8 || output_dim <= 0) return 0;
+    const std::int64_t raw =
+        rows * lm_head_f32_blocks(output_dim) * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+    return (raw + 255) & ~std::int64_t(255);
+}
+
+int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input,
+                                std::int64_t* output_indices, float* output_values,
+                                std::int64_t rows, void* workspace,
+                                std::int64_t workspace_nbytes, void* cuda_stream) {
+    Descriptor normalized{};
+    if (!normalize_descriptor(descriptor, &normalized) || input == nullptr ||
+        output_indices == nullptr || output_values == nullptr || workspace == nullptr ||
+        (normalized.cuda_stream != nullptr && normalized.cuda_stream != cuda_stream)) {
+        return kInvalid;
+    }
+    const std::int64_t required =
+        nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    launch_lm_head_f32(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
+                       output_indices, output_values, as_stream(cuda_stream));
+    return launch_status();
+}
+
+std::int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(std::int64_t rows, std::int64_t input_dim,
+                                                       std::int64_t output_dim, int mode) {
+    if (rows <= 0 || input_dim <= 0 || input_dim % 256 != 0 || output_dim <= 0 ||
+        (mode != NFN_MI355_GEMM_BF16 && mode != NFN_MI355_GEMM_INT8)) {
+        return 0;
+    }
+    return 256;
+}
+
+int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float* input,
+                                      float* output, std::int64_t rows, void* workspace,
+                                      std::int64_t workspace_nbytes, int mode,
+                                      void* cuda_stream) {
+    Descriptor normalized{};
+    if (input == nullptr || output == nullptr || workspace == nullptr || rows <= 0 ||
+        !validate_k_descriptor(descriptor, descriptor == nullptr ? 0 : descriptor->input_dim,
+                               cuda_stream, true) ||
+        !normalize_descriptor(descriptor, &normalized)) {
+        return kInvalid;
+    }
+    const std::int64_t required = nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+        rows, normalized.input_dim, normalized.output_dim, mode);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = normalized.input_dim;
+    set.op[0] = make_projection(normalized, output);
+    constexpr std::int64_t kChunk = 65535 * 8;
+    for (std::int64_t row = 0; row < rows; row += kChunk) {
+        const std::int64_t count = rows - row < kChunk ? rows - row : kChunk;
+        set.op[0].output = output + row * normalized.output_dim;
+        launch_gemv_f32(set, input + row * normalized.input_dim, nullptr, kPlain, nullptr, count,
+                        as_stream(cuda_stream));
+    }
+    return launch_status();
+}
+
+}  // extern "C"

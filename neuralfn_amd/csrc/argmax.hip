@@ -1,0 +1,82 @@
+// Row argmax over float logits.  Ties select the lowest column, NaN never
+// wins, an all-NaN row yields index 0 and -inf: the behaviour of the
+// reference kernel (neuralfn/csrc/tile_cuda/kernels.cu:1564-1602), pinned by
+// tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1869-1904.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace nfn {
+
+namespace {
+
+constexpr int kArgmaxThreads = 1024;
+
+__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
+                                       std::int64_t& best_index) {
+    if (value > best_value || (value == best_value && index < best_index)) {
+        best_value = value;
+        best_index = index;
+    }
+}
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_rows_kernel(
+    const float* __restrict__ values, std::int64_t* __restrict__ indices,
+    float* __restrict__ maxima, std::int64_t width) {
+    __shared__ float wave_values[kArgmaxThreads / kWave];
+    __shared__ std::int64_t wave_indices[kArgmaxThreads / kWave];
+    const std::int64_t row = blockIdx.x;
+    const float* source = values + row * width;
+    float best_value = -INFINITY;
+    std::int64_t best_index = 0;
+    // Vector body where the row start is 16-byte aligned, scalar otherwise.
+    const bool aligned = (reinterpret_cast<std::uintptr_t>(source) & 15u) == 0;
+    const std::int64_t vector_count = aligned ? width / 4 : 0;
+    for (std::int64_t v = threadIdx.x; v < vector_count; v += kArgmaxThreads) {
+        const float4 x = reinterpret_cast<const float4*>(source)[v];
+        better(x.x, v * 4, best_value, best_index);
+        better(x.y, v * 4 + 1, best_value, best_index);
+        better(x.z, v * 4 + 2, best_value, best_index);
+        better(x.w, v * 4 + 3, best_value, best_index);
+    }
+    for (std::int64_t column = vector_count * 4 + threadIdx.x; column < width;
+         column += kArgmaxThreads) {
+        better(source[column], column, best_value, best_index);
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        const float other_value = __shfl_xor(best_value, offset, 64);
+        const std::int64_t other_index = __shfl_xor(best_index, offset, 64);
+        better(other_value, other_index, best_value, best_index);
+    }
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    if (lane == 0) {
+        wave_values[wave] = best_value;
+        wave_indices[wave] = best_index;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        best_value = lane < kArgmaxThreads / kWave ? wave_values[lane] : -INFINITY;
+        best_index = lane < kArgmaxThreads / kWave ? wave_indices[lane] : 0;
+#pragma unroll
+        for (int offset = 8; offset > 0; offset >>= 1) {
+            const float other_value = __shfl_xor(best_value, offset, 64);
+            const std::int64_t other_index = __shfl_xor(best_index, offset, 64);
+            better(other_value, other_index, best_value, best_index);
+        }
+        if (lane == 0) {
+            indices[row] = best_index;
+            maxima[row] = best_value;
+        }
+    }
+}
+
+}  // namespace
+
+void launch_argmax_rows(const float* values, std::int64_t* indices, float* maxima,
+                        std::int64_t rows, std::int64_t width, hipStream_t stream) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3(static_cast<unsigned>(rows)),
+                       dim3(kArgmaxThreads), 0, stream, values, indices, maxima, width);
+}
+
+}  // namespace nfn

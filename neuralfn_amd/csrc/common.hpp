@@ -1,0 +1,182 @@
+// Shared host/device definitions for the MI355X K-Quant packed-linear library.
+//
+// Formats follow ggml's block layouts as the reference states them
+// (neuralfn/csrc/tile_cuda/vendor/llama_mmq_62bf73d/ggml/src/ggml-common.h:251-368)
+// and the per-weight arithmetic of the reference's CPU engine
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:542-616), with the canonical
+// Q6_K sub-scale index (neuralfn/csrc/tile_cuda/kernels.cu:1320).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/nfn_mi355_tile_ops.h"
+
+namespace nfn {
+
+constexpr int kInvalid = 1;  // hipErrorInvalidValue; the reference returns cudaErrorInvalidValue (1)
+constexpr int kWave = 64;
+
+enum : std::uint32_t {
+    kEncF32 = NFN_NATIVE_TILE_PACKED_WEIGHT_F32,
+    kEncQ8_0 = NFN_MI355_PACKED_WEIGHT_Q8_0,
+    kEncQ4K = NFN_NATIVE_TILE_PACKED_WEIGHT_Q4_K,
+    kEncQ5K = NFN_NATIVE_TILE_PACKED_WEIGHT_Q5_K,
+    kEncQ6K = NFN_NATIVE_TILE_PACKED_WEIGHT_Q6_K,
+    kEncBF16 = NFN_NATIVE_TILE_PACKED_WEIGHT_BF16,
+};
+
+using Descriptor = NfnNativeTilePackedWeightDescriptorV1;
+
+__host__ __device__ constexpr std::int64_t block_bytes(std::uint32_t encoding) {
+    switch (encoding) {
+        case kEncF32: return 4;
+        case kEncBF16: return 2;
+        case kEncQ8_0: return 34;
+        case kEncQ4K: return 144;
+        case kEncQ5K: return 176;
+        case kEncQ6K: return 210;
+        default: return 0;
+    }
+}
+
+__host__ __device__ constexpr std::int64_t block_elements(std::uint32_t encoding) {
+    switch (encoding) {
+        case kEncF32: case kEncBF16: return 1;
+        case kEncQ8_0: return 32;
+        case kEncQ4K: case kEncQ5K: case kEncQ6K: return 256;
+        default: return 0;
+    }
+}
+
+__host__ __device__ constexpr bool is_k_quant(std::uint32_t encoding) {
+    return encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K;
+}
+
+// Host-side checks (descriptor.cpp).
+bool normalize_descriptor(const Descriptor* source, Descriptor* output);
+bool validate_k_descriptor(const Descriptor* descriptor, std::int64_t input_dim,
+                           void* stream, bool allow_q8_0);
+
+inline hipStream_t as_stream(void* stream) { return reinterpret_cast<hipStream_t>(stream); }
+inline int launch_status() { return static_cast<int>(hipPeekAtLastError()); }
+
+// What one projection of a multi-projection launch needs on the device.
+struct Projection {
+    const std::uint8_t* data;
+    float* output;
+    std::int64_t output_dim;
+    std::int64_t row_stride;
+    std::uint32_t encoding;
+    std::uint32_t first_tile;  // first tile index of this projection in the launch
+};
+
+struct ProjectionSet {
+    Projection op[4];
+    int count;
+    std::int64_t input_dim;
+};
+
+// Activation prologues of the fused entry points (glimmer_k_mmq.cu:299-317).
+enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2 };
+
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ float half_bits_to_float(std::uint32_t bits) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(bits)));
+}
+
+__device__ __forceinline__ float load_half(const std::uint8_t* p) {
+    return half_bits_to_float(static_cast<std::uint32_t>(p[0]) | (static_cast<std::uint32_t>(p[1]) << 8));
+}
+
+// 6-bit scale and minimum of sub-block `index` (resident_glimmer.cpp:178-186).
+__device__ __forceinline__ void k_scale_min(const std::uint8_t* scales, int index,
+                                            int* scale, int* minimum) {
+    if (index < 4) {
+        *scale = scales[index] & 63;
+        *minimum = scales[index + 4] & 63;
+        return;
+    }
+    *scale = (scales[index + 4] & 0x0f) | ((scales[index - 4] >> 6) << 4);
+    *minimum = (scales[index + 4] >> 4) | ((scales[index] >> 6) << 4);
+}
+
+// fused activation prologue; `first`/`second` follow the entry points'
+// argument order: gated (input, gate), swiglu (gate, up).
+template <int P>
+__device__ __forceinline__ float apply_prologue(float first, float second) {
+    if constexpr (P == kGated) {
+        return first / (1.0f + expf(-second));
+    } else if constexpr (P == kSwiGlu) {
+        return (second * first) * (1.0f / (1.0f + expf(-first)));
+    } else {
+        return first;
+    }
+}
+
+// One weight, decoded from scratch: the slow, obviously-right form used by the
+// dequantize entry point and by encodings without a tuned kernel.
+__device__ __forceinline__ float weight_value(std::uint32_t encoding,
+                                              const std::uint8_t* row_data,
+                                              std::int64_t col) {
+    if (encoding == kEncF32) {
+        return reinterpret_cast<const float*>(row_data)[col];
+    }
+    if (encoding == kEncBF16) {
+        const std::uint32_t bits = reinterpret_cast<const std::uint16_t*>(row_data)[col];
+        return __uint_as_float(bits << 16);
+    }
+    if (encoding == kEncQ8_0) {
+        const std::uint8_t* block = row_data + (col / 32) * 34;
+        const int quant = static_cast<std::int8_t>(block[2 + (col & 31)]);
+        return load_half(block) * static_cast<float>(quant);
+    }
+    const std::int64_t block_index = col >> 8;
+    const int within = static_cast<int>(col & 255);
+    if (encoding == kEncQ4K || encoding == kEncQ5K) {
+        const bool q5 = encoding == kEncQ5K;
+        const std::uint8_t* block = row_data + block_index * (q5 ? 176 : 144);
+        const float d = load_half(block);
+        const float dmin = load_half(block + 2);
+        const int group = within >> 6;
+        const int lane = within & 31;
+        const bool high = (within & 32) != 0;
+        int scale, minimum;
+        k_scale_min(block + 4, group * 2 + (high ? 1 : 0), &scale, &minimum);
+        const std::uint8_t packed = block[(q5 ? 48 : 16) + group * 32 + lane];
+        int quant = high ? (packed >> 4) : (packed & 0x0f);
+        if (q5) {
+            const int mask = (high ? 2 : 1) << (2 * group);
+            quant += (block[16 + lane] & mask) ? 16 : 0;
+        }
+        // Two roundings and a subtraction, never an FMA: the CPU engine's form.
+        return __fsub_rn(__fmul_rn(d, static_cast<float>(scale * quant)),
+                         __fmul_rn(dmin, static_cast<float>(minimum)));
+    }
+    const std::uint8_t* block = row_data + block_index * 210;
+    const int half = within >> 7;
+    const int position = within & 127;
+    const int quarter = position >> 5;
+    const int lane = position & 31;
+    const std::uint8_t low = block[half * 64 + lane + ((quarter & 1) ? 32 : 0)];
+    const std::uint8_t high = block[128 + half * 32 + lane];
+    const int nibble = quarter < 2 ? (low & 0x0f) : (low >> 4);
+    const int quant = (nibble | (((high >> (2 * quarter)) & 3) << 4)) - 32;
+    const int scale = static_cast<std::int8_t>(block[192 + half * 8 + quarter * 2 + (lane >> 4)]);
+    return __fmul_rn(__fmul_rn(load_half(block + 208), static_cast<float>(scale)),
+                     static_cast<float>(quant));
+}
+
+__device__ __forceinline__ float wave_sum(float value) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        value += __shfl_xor(value, offset, 64);
+    }
+    return value;
+}
+
+#endif  // __HIPCC__
+
+}  // namespace nfn

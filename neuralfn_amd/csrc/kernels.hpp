@@ -1,0 +1,32 @@
+// Launchers implemented by the .hip files; called by the C ABI in abi.cpp.
+#pragma once
+
+#include "common.hpp"
+
+namespace nfn {
+
+// dequant.hip
+void launch_dequantize(const Descriptor& descriptor, float* output, hipStream_t stream);
+
+// gemv_f32.hip — exact float-activation path, rows in tiles of up to 8.
+void launch_gemv_f32(ProjectionSet set, const float* first, const float* second, int prologue,
+                     const float* bias, std::int64_t rows, hipStream_t stream);
+
+// q8_1.hip — the public int8-activation path.
+void launch_quantize_q8_1(const float* input, std::int8_t* codes, float* scales, float* sums,
+                          std::int64_t rows, std::int64_t width, hipStream_t stream);
+void launch_linear_q8_1(ProjectionSet set, const std::int8_t* codes, const float* scales,
+                        const float* sums, const float* bias, std::int64_t rows,
+                        hipStream_t stream);
+
+// argmax.hip
+void launch_argmax_rows(const float* values, std::int64_t* indices, float* maxima,
+                        std::int64_t rows, std::int64_t width, hipStream_t stream);
+
+// elementwise.hip
+void launch_sigmoid_gate(const float* values, const float* gate, float* output,
+                         std::int64_t count, hipStream_t stream);
+void launch_swiglu(const float* gate, const float* up, float* output, std::int64_t count,
+                   hipStream_t stream);
+
+}  // namespace nfn

@@ -1,0 +1,21 @@
+// Workspace record and launchers of the fused lm_head argmax.
+#pragma once
+
+#include "common.hpp"
+
+namespace nfn {
+
+// Best logit of one workgroup for one input row; the workspace holds
+// [rows][workgroups] of these.
+struct LmHeadCandidate {
+    std::int64_t index;
+    float value;
+    std::uint32_t pad;
+};
+
+std::int64_t lm_head_f32_blocks(std::int64_t output_dim);
+void launch_lm_head_f32(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                        LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
+                        hipStream_t stream);
+
+}  // namespace nfn

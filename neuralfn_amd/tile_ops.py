@@ -1,0 +1,362 @@
+"""ctypes binding of libnfn_mi355_tile_ops.so and a small torch-tensor front end.
+
+The descriptor struct and the calling pattern mirror the reference's own ctypes
+harness for this ABI (tools/bench_muse_glimmer_packed_linear.py:28-43, 560-640):
+device pointers as integers, a 72-byte descriptor per packed matrix, an int
+status per call.  torch is used only to own device memory and streams.
+
+There is no CPU fallback: if the library is missing, loading raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Optional, Sequence
+
+from . import kquant
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libnfn_mi355_tile_ops.so"
+INVALID = 1
+
+GEMM_BF16 = 0
+GEMM_INT8 = 1
+
+
+class PackedWeightDescriptor(ctypes.Structure):
+    """NfnNativeTilePackedWeightDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:293-307)."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("version", ctypes.c_uint32),
+        ("encoding", ctypes.c_uint32),
+        ("flags", ctypes.c_uint32),
+        ("data", ctypes.c_void_p),
+        ("data_nbytes", ctypes.c_int64),
+        ("output_dim", ctypes.c_int64),
+        ("input_dim", ctypes.c_int64),
+        ("row_stride_bytes", ctypes.c_int64),
+        ("reserved0", ctypes.c_uint32),
+        ("reserved1", ctypes.c_uint32),
+        ("cuda_stream", ctypes.c_void_p),
+    ]
+
+
+_P = ctypes.c_void_p
+_I64 = ctypes.c_int64
+_DESC = ctypes.POINTER(PackedWeightDescriptor)
+_DESC_ARRAY = ctypes.POINTER(_DESC)
+_PTR_ARRAY = ctypes.POINTER(ctypes.c_void_p)
+
+#: every symbol include/nfn_mi355_tile_ops.h declares: name -> (restype, argtypes)
+SIGNATURES = {
+    "nfn_native_tile_ops_abi_version": (ctypes.c_int, []),
+    "nfn_native_tile_strict_math_abi_version": (ctypes.c_int, []),
+    "nfn_native_tile_packed_weight_abi_version": (ctypes.c_int, []),
+    "nfn_native_tile_glimmer_inference_abi_version": (ctypes.c_int, []),
+    "nfn_native_tile_k_quant_mmq_abi_version": (ctypes.c_int, []),
+    "nfn_mi355_abi_version": (ctypes.c_int, []),
+    "nfn_native_tile_ops_error_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "nfn_native_tile_packed_weight_validate_v1": (ctypes.c_int, [_DESC]),
+    "nfn_native_tile_packed_weight_dequantize_float32_v1": (ctypes.c_int, [_DESC, _P]),
+    "nfn_native_tile_linear_packed_weight_float32_v1": (
+        ctypes.c_int, [_DESC, _P, _P, _P, _I64, ctypes.c_bool]),
+    "nfn_native_tile_quantize_q8_1_float32_v1": (ctypes.c_int, [_P, _P, _P, _P, _I64, _I64, _P]),
+    "nfn_native_tile_linear_packed_weight_q8_1_float32_v1": (
+        ctypes.c_int, [_DESC, _P, _P, _P, _P, _P, _I64, ctypes.c_bool]),
+    "nfn_native_tile_linear_packed_weight_q8_1_multi_decode_float32_v1": (
+        ctypes.c_int, [_DESC, _DESC, _DESC, _DESC, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmq_workspace_bytes_v1": (_I64, [_I64, _I64]),
+    "nfn_native_tile_k_quant_mmq_multi_linear_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmvq_linear_float32_v1": (
+        ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P]),
+    "nfn_native_tile_argmax_rows_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
+    "nfn_native_tile_glimmer_sigmoid_gate_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
+    "nfn_native_tile_swiglu_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
+    "nfn_mi355_lm_head_argmax_workspace_bytes_v1": (_I64, [_I64, _I64]),
+    "nfn_mi355_lm_head_argmax_v1": (ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P, _I64, _P]),
+    "nfn_mi355_k_quant_gemm_workspace_bytes_v1": (_I64, [_I64, _I64, _I64, ctypes.c_int]),
+    "nfn_mi355_k_quant_gemm_float32_v1": (
+        ctypes.c_int, [_DESC, _P, _P, _I64, _P, _I64, ctypes.c_int, _P]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load(path: Optional[Path] = None) -> ctypes.CDLL:
+    """dlopen the library and bind every declared symbol; raises if absent."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    target = Path(path) if path is not None else LIB_PATH
+    if not target.exists():
+        raise RuntimeError(
+            f"{target} is not built; run `python -m neuralfn_amd.build` (there is no CPU fallback)")
+    lib = ctypes.CDLL(str(target), mode=ctypes.RTLD_LOCAL)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        function = getattr(lib, name)  # AttributeError if the symbol is missing
+        function.restype = restype
+        function.argtypes = argtypes
+    if path is None:
+        _lib = lib
+    return lib
+
+
+class TileOpsError(RuntimeError):
+    def __init__(self, operation: str, status: int):
+        text = load().nfn_native_tile_ops_error_string(status)
+        super().__init__(f"{operation} failed with status {status}: {text.decode() if text else '?'}")
+        self.status = status
+
+
+def check(status: int, operation: str) -> None:
+    if status != 0:
+        raise TileOpsError(operation, status)
+
+
+def make_descriptor(encoding: int, data_ptr: int, output_dim: int, input_dim: int,
+                    stream: int = 0) -> PackedWeightDescriptor:
+    stride = kquant.row_stride_bytes(encoding, input_dim)
+    return PackedWeightDescriptor(
+        struct_size=ctypes.sizeof(PackedWeightDescriptor), version=1, encoding=encoding, flags=0,
+        data=data_ptr, data_nbytes=output_dim * stride, output_dim=output_dim,
+        input_dim=input_dim, row_stride_bytes=stride, reserved0=0, reserved1=0,
+        cuda_stream=stream or None)
+
+
+def _stream_handle() -> int:
+    import torch
+    return int(torch.cuda.current_stream().cuda_stream)
+
+
+@dataclass
+class PackedWeight:
+    """A packed [output_dim, input_dim] matrix resident in device memory."""
+
+    encoding: int
+    output_dim: int
+    input_dim: int
+    data: "object"  # torch.uint8 tensor on the GPU, kept alive here
+
+    @classmethod
+    def from_numpy(cls, encoding: int, packed, output_dim: int, input_dim: int,
+                   device: str = "cuda:0") -> "PackedWeight":
+        import torch
+        expected = kquant.packed_nbytes(encoding, output_dim, input_dim)
+        if packed.size != expected:
+            raise ValueError(f"packed tensor has {packed.size} bytes, expected {expected}")
+        return cls(encoding, output_dim, input_dim, torch.from_numpy(packed).to(device))
+
+    @property
+    def nbytes(self) -> int:
+        return int(self.data.numel())
+
+    def descriptor(self, stream: int = 0) -> PackedWeightDescriptor:
+        return make_descriptor(self.encoding, self.data.data_ptr(), self.output_dim,
+                               self.input_dim, stream)
+
+
+def _descriptor_array(descriptors: Sequence[PackedWeightDescriptor]):
+    array = (_DESC * len(descriptors))()
+    for index, descriptor in enumerate(descriptors):
+        array[index] = ctypes.pointer(descriptor)
+    return array
+
+
+def _pointer_array(tensors) -> "ctypes.Array":
+    array = (ctypes.c_void_p * len(tensors))()
+    for index, tensor in enumerate(tensors):
+        array[index] = tensor.data_ptr()
+    return array
+
+
+def dequantize(weight: PackedWeight):
+    import torch
+    out = torch.empty((weight.output_dim, weight.input_dim), dtype=torch.float32,
+                      device=weight.data.device)
+    descriptor = weight.descriptor(_stream_handle())
+    check(load().nfn_native_tile_packed_weight_dequantize_float32_v1(
+        ctypes.byref(descriptor), out.data_ptr()), "dequantize")
+    return out
+
+
+def linear(weight: PackedWeight, x, bias=None):
+    """nfn_native_tile_linear_packed_weight_float32_v1: any row count."""
+    import torch
+    rows = x.shape[0]
+    out = torch.empty((rows, weight.output_dim), dtype=torch.float32, device=x.device)
+    descriptor = weight.descriptor(_stream_handle())
+    check(load().nfn_native_tile_linear_packed_weight_float32_v1(
+        ctypes.byref(descriptor), x.data_ptr(), bias.data_ptr() if bias is not None else None,
+        out.data_ptr(), rows, bias is not None), "linear_packed_weight")
+    return out
+
+
+def small_batch_workspace(rows: int, input_dim: int, device="cuda:0"):
+    import torch
+    nbytes = load().nfn_native_tile_k_quant_mmq_workspace_bytes_v1(rows, input_dim)
+    if nbytes <= 0:
+        raise ValueError(f"no small-batch workspace for rows={rows}, input_dim={input_dim}")
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+_MULTI = {
+    ("mmq", "plain"): "nfn_native_tile_k_quant_mmq_multi_linear_float32_v1",
+    ("mmq", "gated"): "nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1",
+    ("mmq", "swiglu"): "nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1",
+    ("mmvq", "plain"): "nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1",
+    ("mmvq", "gated"): "nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1",
+    ("mmvq", "swiglu"): "nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1",
+}
+
+
+def multi_linear(weights: Sequence[PackedWeight], x, workspace, second=None, family: str = "mmq",
+                 prologue: str = "plain", outputs=None):
+    """1..4 projections of one shared input, rows 1..16.
+
+    prologue "gated": x / (1 + exp(-second));  "swiglu": x is gate, second is up.
+    """
+    import torch
+    rows = x.shape[0]
+    stream = _stream_handle()
+    if outputs is None:
+        outputs = [torch.empty((rows, w.output_dim), dtype=torch.float32, device=x.device)
+                   for w in weights]
+    descriptors = [w.descriptor(stream) for w in weights]
+    function = getattr(load(), _MULTI[(family, prologue)])
+    args = [_descriptor_array(descriptors), x.data_ptr()]
+    if prologue != "plain":
+        args.append(second.data_ptr() if second is not None else None)
+    args += [_pointer_array(outputs), len(weights), rows, workspace.data_ptr(),
+             workspace.numel(), stream]
+    check(function(*args), _MULTI[(family, prologue)])
+    return outputs
+
+
+def mmvq_linear(weight: PackedWeight, x, workspace, out=None):
+    """nfn_native_tile_k_quant_mmvq_linear_float32_v1: the one-row decode GEMV."""
+    import torch
+    stream = _stream_handle()
+    if out is None:
+        out = torch.empty((1, weight.output_dim), dtype=torch.float32, device=x.device)
+    descriptor = weight.descriptor(stream)
+    check(load().nfn_native_tile_k_quant_mmvq_linear_float32_v1(
+        ctypes.byref(descriptor), x.data_ptr(), out.data_ptr(), workspace.data_ptr(),
+        workspace.numel(), stream), "mmvq_linear")
+    return out
+
+
+def quantize_q8_1(x):
+    import torch
+    rows, width = x.shape
+    codes = torch.empty((rows, width), dtype=torch.int8, device=x.device)
+    scales = torch.empty((rows, width // 32), dtype=torch.float32, device=x.device)
+    sums = torch.empty_like(scales)
+    check(load().nfn_native_tile_quantize_q8_1_float32_v1(
+        x.data_ptr(), codes.data_ptr(), scales.data_ptr(), sums.data_ptr(), rows, width,
+        _stream_handle()), "quantize_q8_1")
+    return codes, scales, sums
+
+
+def linear_q8_1(weight: PackedWeight, codes, scales, sums, bias=None):
+    import torch
+    rows = codes.shape[0]
+    out = torch.empty((rows, weight.output_dim), dtype=torch.float32, device=codes.device)
+    descriptor = weight.descriptor(_stream_handle())
+    check(load().nfn_native_tile_linear_packed_weight_q8_1_float32_v1(
+        ctypes.byref(descriptor), codes.data_ptr(), scales.data_ptr(), sums.data_ptr(),
+        bias.data_ptr() if bias is not None else None, out.data_ptr(), rows, bias is not None),
+        "linear_q8_1")
+    return out
+
+
+def linear_q8_1_multi_decode(weights: Sequence[PackedWeight], codes, scales, sums):
+    import torch
+    stream = _stream_handle()
+    outputs = [torch.empty((1, w.output_dim), dtype=torch.float32, device=codes.device)
+               for w in weights]
+    descriptors = [w.descriptor() for w in weights]
+    refs = [ctypes.byref(d) for d in descriptors] + [None] * (4 - len(weights))
+    outs = [o.data_ptr() for o in outputs] + [None] * (4 - len(weights))
+    check(load().nfn_native_tile_linear_packed_weight_q8_1_multi_decode_float32_v1(
+        *refs, codes.data_ptr(), scales.data_ptr(), sums.data_ptr(), *outs, len(weights),
+        stream), "q8_1_multi_decode")
+    return outputs
+
+
+def argmax_rows(values):
+    import torch
+    rows, width = values.shape
+    indices = torch.empty(rows, dtype=torch.int64, device=values.device)
+    maxima = torch.empty(rows, dtype=torch.float32, device=values.device)
+    check(load().nfn_native_tile_argmax_rows_float32_v1(
+        values.data_ptr(), indices.data_ptr(), maxima.data_ptr(), rows, width,
+        _stream_handle()), "argmax_rows")
+    return indices, maxima
+
+
+def sigmoid_gate(values, gate):
+    import torch
+    out = torch.empty_like(values)
+    check(load().nfn_native_tile_glimmer_sigmoid_gate_float32_v1(
+        values.data_ptr(), gate.data_ptr(), out.data_ptr(), values.numel(), _stream_handle()),
+        "sigmoid_gate")
+    return out
+
+
+def swiglu(gate, up):
+    import torch
+    out = torch.empty_like(gate)
+    check(load().nfn_native_tile_swiglu_float32(
+        gate.data_ptr(), up.data_ptr(), out.data_ptr(), gate.numel(), _stream_handle()), "swiglu")
+    return out
+
+
+def lm_head_argmax(weight: PackedWeight, x, workspace=None):
+    """nfn_mi355_lm_head_argmax_v1: GEMV + argmax, logits never stored."""
+    import torch
+    rows = x.shape[0]
+    stream = _stream_handle()
+    if workspace is None:
+        nbytes = load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, weight.output_dim)
+        if nbytes <= 0:
+            raise ValueError("lm_head_argmax supports 1..8 rows")
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    indices = torch.empty(rows, dtype=torch.int64, device=x.device)
+    maxima = torch.empty(rows, dtype=torch.float32, device=x.device)
+    descriptor = weight.descriptor(stream)
+    check(load().nfn_mi355_lm_head_argmax_v1(
+        ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), rows,
+        workspace.data_ptr(), workspace.numel(), stream), "lm_head_argmax")
+    return indices, maxima
+
+
+def gemm(weight: PackedWeight, x, mode: int = GEMM_BF16, workspace=None, out=None):
+    """nfn_mi355_k_quant_gemm_float32_v1: prefill dequant-GEMM, any row count."""
+    import torch
+    rows = x.shape[0]
+    stream = _stream_handle()
+    if workspace is None:
+        nbytes = load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+            rows, weight.input_dim, weight.output_dim, mode)
+        if nbytes <= 0:
+            raise ValueError("unsupported GEMM geometry or mode")
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    if out is None:
+        out = torch.empty((rows, weight.output_dim), dtype=torch.float32, device=x.device)
+    descriptor = weight.descriptor(stream)
+    check(load().nfn_mi355_k_quant_gemm_float32_v1(
+        ctypes.byref(descriptor), x.data_ptr(), out.data_ptr(), rows, workspace.data_ptr(),
+        workspace.numel(), mode, stream), "k_quant_gemm")
+    return out

@@ -1,0 +1,485 @@
+// CPU oracle for the K-Quant packed-linear path.  TEST INFRASTRUCTURE ONLY.
+//
+// This file restates, on the CPU, the arithmetic of the reference's C++
+// resident engine for packed K-Quant weights.  It is the checker that the GPU
+// library is compared against; nothing in the shipped library links, loads or
+// calls it.  Only the test suite, the smoke check and the benchmark's
+// cpu_baseline leg may use it.
+//
+// Reference files followed (paths relative to the reference checkout):
+//   fp16 decode      neuralfn/csrc/native_gpt2/resident_glimmer.cpp:159-176
+//   k_scale_min      neuralfn/csrc/native_gpt2/resident_glimmer.cpp:178-186
+//   parallel_for     neuralfn/csrc/native_gpt2/resident_glimmer.cpp:188-235
+//   weight value     neuralfn/csrc/native_gpt2/resident_glimmer.cpp:542-616
+//   linear           neuralfn/csrc/native_gpt2/resident_glimmer.cpp:655-679
+//   linear_rows      neuralfn/csrc/native_gpt2/resident_glimmer_assistant.cpp:459-483
+//   argmax           neuralfn/csrc/native_gpt2/resident_glimmer.cpp:250-254, 1957-1965
+//   Q8_1 quantize    neuralfn/csrc/tile_cuda/kernels.cu:1527-1562
+//   Q8_1 x K dot     neuralfn/csrc/tile_cuda/kernels.cu:1620-1731
+//   Q8_0 layout      neuralfn/csrc/tile_cuda/vendor/llama_mmq_62bf73d/ggml/src/ggml-common.h:251-256
+//
+// Pinning status (what checks each function besides its own formula):
+//   nfo_fp16_to_float   exhaustive 65,536-value sweep against numpy float16.
+//   nfo_k_scale_min     brute force against an independent bit-field statement.
+//   Q4_K / Q5_K / Q6_K  the reference's known-answer blocks
+//                       (tests/test_native_gguf.py:510-553) and, where the
+//                       reference build is available, element-for-element
+//                       equality with the compiled reference sources.
+//   Q6_K                canonical (ggml) sub-scale index is the contract; the
+//                       reference CPU engine's line 614 drops the `lane/16`
+//                       term, reproduced here by q6_as_written != 0.
+//   Q8_0                parity unpinned: the reference has no Q8_0 code or test;
+//                       pinned by the closed form w = d*q only.
+//   nfo_linear*         equals dequantize-then-double-dot; equals the compiled
+//                       reference linear() bit for bit where that builds.
+//   nfo_quantize_q8_1   exact-scale crafted input (scale exactly 1/32) and the
+//                       reference probe's equality rule
+//                       (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:968-1007).
+//   nfo_linear_q8_1     closed form over reconstructed activations, same rule
+//                       as tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1009-1023.
+//
+// Build: g++ -std=c++17 -O2 -pthread -ffp-contract=off -shared -fPIC.
+// -ffp-contract=off keeps `d*float(sc*q) - dmin*float(m)` as two roundings,
+// as the reference build (-O2, x86-64, no FMA contraction) produces.
+
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <thread>
+#include <vector>
+
+namespace {
+
+constexpr std::uint32_t kEncF32 = 0;
+constexpr std::uint32_t kEncQ8_0 = 8;
+constexpr std::uint32_t kEncQ4K = 12;
+constexpr std::uint32_t kEncQ5K = 13;
+constexpr std::uint32_t kEncQ6K = 14;
+constexpr std::uint32_t kEncBF16 = 30;
+
+// resident_glimmer.cpp:159-176 — IEEE half via ldexp in double, then to float.
+float fp16_to_float(const std::uint8_t* source) {
+    std::uint16_t bits = 0;
+    std::memcpy(&bits, source, sizeof(bits));
+    const bool negative = (bits & 0x8000u) != 0;
+    const int exponent = static_cast<int>((bits >> 10u) & 0x1fu);
+    const int mantissa = static_cast<int>(bits & 0x03ffu);
+    double value = 0.0;
+    if (exponent == 0) {
+        value = std::ldexp(static_cast<double>(mantissa), -24);
+    } else if (exponent == 31) {
+        value = mantissa == 0 ? std::numeric_limits<double>::infinity()
+                              : std::numeric_limits<double>::quiet_NaN();
+    } else {
+        value = std::ldexp(1.0 + static_cast<double>(mantissa) / 1024.0, exponent - 15);
+    }
+    return static_cast<float>(negative ? -value : value);
+}
+
+// resident_glimmer.cpp:152-157
+float bf16_to_float(const std::uint8_t* source) {
+    std::uint16_t bits = 0;
+    std::memcpy(&bits, source, sizeof(bits));
+    const std::uint32_t wide = static_cast<std::uint32_t>(bits) << 16u;
+    float result;
+    std::memcpy(&result, &wide, sizeof(result));
+    return result;
+}
+
+// resident_glimmer.cpp:178-186
+void k_scale_min(const std::uint8_t* scales, int index, int* scale, int* minimum) {
+    if (index < 4) {
+        *scale = scales[index] & 63;
+        *minimum = scales[index + 4] & 63;
+        return;
+    }
+    *scale = (scales[index + 4] & 0x0f) | ((scales[index - 4] >> 6) << 4);
+    *minimum = (scales[index + 4] >> 4) | ((scales[index] >> 6) << 4);
+}
+
+std::int64_t block_bytes(std::uint32_t encoding) {
+    switch (encoding) {
+        case kEncF32: return 4;
+        case kEncBF16: return 2;
+        case kEncQ8_0: return 34;
+        case kEncQ4K: return 144;
+        case kEncQ5K: return 176;
+        case kEncQ6K: return 210;
+        default: return 0;
+    }
+}
+
+std::int64_t block_elements(std::uint32_t encoding) {
+    switch (encoding) {
+        case kEncF32: return 1;
+        case kEncBF16: return 1;
+        case kEncQ8_0: return 32;
+        case kEncQ4K: case kEncQ5K: case kEncQ6K: return 256;
+        default: return 0;
+    }
+}
+
+// resident_glimmer.cpp:542-616 — one weight, decoded from scratch.
+float weight_value(std::uint32_t encoding, const std::uint8_t* row_data,
+                   std::int64_t col, bool q6_as_written) {
+    if (encoding == kEncF32) {
+        float result = 0.0f;
+        std::memcpy(&result, row_data + col * 4, sizeof(result));
+        return result;
+    }
+    if (encoding == kEncBF16) {
+        return bf16_to_float(row_data + col * 2);
+    }
+    if (encoding == kEncQ8_0) {
+        // ggml block_q8_0 {fp16 d; int8 qs[32]}; w = d * q.
+        const std::uint8_t* block = row_data + (col / 32) * 34;
+        const float d = fp16_to_float(block);
+        const int quant = static_cast<std::int8_t>(block[2 + col % 32]);
+        return d * static_cast<float>(quant);
+    }
+    const std::int64_t block_index = col / 256;
+    const int within = static_cast<int>(col % 256);
+    if (encoding == kEncQ4K) {
+        const std::uint8_t* block = row_data + block_index * 144;
+        const float d = fp16_to_float(block);
+        const float dmin = fp16_to_float(block + 2);
+        const int group = within / 64;
+        const int lane = within % 32;
+        const bool high = (within % 64) >= 32;
+        int scale = 0, minimum = 0;
+        k_scale_min(block + 4, group * 2 + (high ? 1 : 0), &scale, &minimum);
+        const std::uint8_t packed = block[16 + group * 32 + lane];
+        const int quant = high ? (packed >> 4) : (packed & 0x0f);
+        return d * static_cast<float>(scale * quant) - dmin * static_cast<float>(minimum);
+    }
+    if (encoding == kEncQ5K) {
+        const std::uint8_t* block = row_data + block_index * 176;
+        const float d = fp16_to_float(block);
+        const float dmin = fp16_to_float(block + 2);
+        const std::uint8_t* high_bits = block + 16;
+        const std::uint8_t* low_bits = block + 48;
+        const int group = within / 64;
+        const int lane = within % 32;
+        const bool high_half = (within % 64) >= 32;
+        int scale = 0, minimum = 0;
+        k_scale_min(block + 4, group * 2 + (high_half ? 1 : 0), &scale, &minimum);
+        const std::uint8_t packed = low_bits[group * 32 + lane];
+        const int low = high_half ? (packed >> 4) : (packed & 0x0f);
+        const int mask = (high_half ? 2 : 1) << (2 * group);
+        const int quant = low + ((high_bits[lane] & mask) ? 16 : 0);
+        return d * static_cast<float>(scale * quant) - dmin * static_cast<float>(minimum);
+    }
+    // Q6_K
+    const std::uint8_t* block = row_data + block_index * 210;
+    const std::uint8_t* low_bits = block;
+    const std::uint8_t* high_bits = block + 128;
+    const std::int8_t* scales = reinterpret_cast<const std::int8_t*>(block + 192);
+    const float d = fp16_to_float(block + 208);
+    const int half = within / 128;
+    const int position = within % 128;
+    const int quarter = position / 32;
+    const int lane = position % 32;
+    const std::uint8_t low = low_bits[half * 64 + lane + ((quarter & 1) ? 32 : 0)];
+    const std::uint8_t high = high_bits[half * 32 + lane];
+    const int nibble = quarter < 2 ? (low & 0x0f) : (low >> 4);
+    const int quant = nibble | (((high >> (2 * quarter)) & 3) << 4);
+    // Canonical ggml index (kernels.cu:1320, native_gguf.py:1698-1706) versus
+    // the CPU engine as written (resident_glimmer.cpp:614).
+    const int scale_index = q6_as_written ? half * 8 + 2 * quarter
+                                          : half * 8 + 2 * quarter + lane / 16;
+    return d * static_cast<float>(scales[scale_index]) * static_cast<float>(quant - 32);
+}
+
+// Decode one whole row with the same per-element arithmetic (same bits).
+void decode_row(std::uint32_t encoding, const std::uint8_t* row_data,
+                std::int64_t cols, bool q6_as_written, float* out) {
+    if (encoding == kEncQ4K || encoding == kEncQ5K) {
+        const std::int64_t bytes = encoding == kEncQ4K ? 144 : 176;
+        for (std::int64_t b = 0; b < cols / 256; ++b) {
+            const std::uint8_t* block = row_data + b * bytes;
+            const float d = fp16_to_float(block);
+            const float dmin = fp16_to_float(block + 2);
+            const std::uint8_t* high_bits = block + 16;
+            const std::uint8_t* low_bits = encoding == kEncQ4K ? block + 16 : block + 48;
+            for (int sub = 0; sub < 8; ++sub) {
+                int scale = 0, minimum = 0;
+                k_scale_min(block + 4, sub, &scale, &minimum);
+                const int group = sub / 2;
+                const bool high = (sub & 1) != 0;
+                const float offset = dmin * static_cast<float>(minimum);
+                for (int lane = 0; lane < 32; ++lane) {
+                    const std::uint8_t packed = low_bits[group * 32 + lane];
+                    int quant = high ? (packed >> 4) : (packed & 0x0f);
+                    if (encoding == kEncQ5K) {
+                        const int mask = (high ? 2 : 1) << (2 * group);
+                        quant += (high_bits[lane] & mask) ? 16 : 0;
+                    }
+                    out[b * 256 + sub * 32 + lane] =
+                        d * static_cast<float>(scale * quant) - offset;
+                }
+            }
+        }
+        return;
+    }
+    for (std::int64_t col = 0; col < cols; ++col) {
+        out[col] = weight_value(encoding, row_data, col, q6_as_written);
+    }
+}
+
+// resident_glimmer.cpp:188-235 — static partition over at most 32 threads.
+template <typename Function>
+void parallel_for(std::int64_t count, std::int64_t minimum_per_thread, int thread_cap,
+                  Function&& function) {
+    if (count <= 0) return;
+    const unsigned hardware = std::max(1u, std::thread::hardware_concurrency());
+    std::int64_t limit = std::min<std::int64_t>(hardware, 32);
+    if (thread_cap > 0) limit = std::min<std::int64_t>(limit, thread_cap);
+    const std::int64_t wanted = (count + minimum_per_thread - 1) / minimum_per_thread;
+    const std::int64_t workers =
+        std::max<std::int64_t>(1, std::min<std::int64_t>({count, wanted, limit}));
+    if (workers == 1) {
+        for (std::int64_t index = 0; index < count; ++index) function(index);
+        return;
+    }
+    std::vector<std::thread> threads;
+    threads.reserve(static_cast<std::size_t>(workers));
+    for (std::int64_t worker = 0; worker < workers; ++worker) {
+        const std::int64_t begin = count * worker / workers;
+        const std::int64_t end = count * (worker + 1) / workers;
+        threads.emplace_back([&, begin, end]() {
+            for (std::int64_t index = begin; index < end; ++index) function(index);
+        });
+    }
+    for (auto& thread : threads) thread.join();
+}
+
+}  // namespace
+
+extern "C" {
+
+float nfo_fp16_to_float(std::uint16_t bits) {
+    std::uint8_t bytes[2];
+    std::memcpy(bytes, &bits, 2);
+    return fp16_to_float(bytes);
+}
+
+void nfo_k_scale_min(const std::uint8_t* scales, int index, int* scale, int* minimum) {
+    k_scale_min(scales, index, scale, minimum);
+}
+
+std::int64_t nfo_block_bytes(std::uint32_t encoding) { return block_bytes(encoding); }
+std::int64_t nfo_block_elements(std::uint32_t encoding) { return block_elements(encoding); }
+
+// Threads parallel_for would use for `count` items (resident_glimmer.cpp:193-196).
+int nfo_worker_count(std::int64_t count, std::int64_t minimum_per_thread, int thread_cap) {
+    const unsigned hardware = std::max(1u, std::thread::hardware_concurrency());
+    std::int64_t limit = std::min<std::int64_t>(hardware, 32);
+    if (thread_cap > 0) limit = std::min<std::int64_t>(limit, thread_cap);
+    const std::int64_t wanted = (count + minimum_per_thread - 1) / minimum_per_thread;
+    return static_cast<int>(
+        std::max<std::int64_t>(1, std::min<std::int64_t>({count, wanted, limit})));
+}
+
+// Dequantize a whole [out_dim, in_dim] matrix, element by element.
+int nfo_dequantize(std::uint32_t encoding, const std::uint8_t* data,
+                   std::int64_t out_dim, std::int64_t in_dim, float* out,
+                   int q6_as_written) {
+    const std::int64_t elements = block_elements(encoding);
+    if (elements == 0 || in_dim % elements != 0) return 1;
+    const std::int64_t stride = in_dim / elements * block_bytes(encoding);
+    parallel_for(out_dim, 16, 0, [&](std::int64_t row) {
+        for (std::int64_t col = 0; col < in_dim; ++col) {
+            out[row * in_dim + col] =
+                weight_value(encoding, data + row * stride, col, q6_as_written != 0);
+        }
+    });
+    return 0;
+}
+
+// The reference's CPU matmul as written: every weight decoded from scratch,
+// product and accumulation in double in column order, one float rounding at
+// the end; a batch is a flat index over rows*out_dim (linear_rows).  bias, when
+// given, is added in float after the rounding, as the device ABI specifies
+// (kernels.cu:1521-1522).  Returns 2 when an output is not finite (the
+// reference throws).
+int nfo_linear_as_written(std::uint32_t encoding, const std::uint8_t* data,
+                          std::int64_t out_dim, std::int64_t in_dim,
+                          const float* input, std::int64_t rows, const float* bias,
+                          float* output, int thread_cap, int q6_as_written) {
+    const std::int64_t elements = block_elements(encoding);
+    if (elements == 0 || in_dim % elements != 0 || rows <= 0) return 1;
+    const std::int64_t stride = in_dim / elements * block_bytes(encoding);
+    std::atomic<int> status{0};
+    parallel_for(rows * out_dim, 128, thread_cap, [&](std::int64_t flat) {
+        const std::int64_t input_row = flat / out_dim;
+        const std::int64_t output_row = flat % out_dim;
+        const float* source = input + input_row * in_dim;
+        const std::uint8_t* row_data = data + output_row * stride;
+        double sum = 0.0;
+        for (std::int64_t col = 0; col < in_dim; ++col) {
+            sum += static_cast<double>(source[col]) *
+                weight_value(encoding, row_data, col, q6_as_written != 0);
+        }
+        float result = static_cast<float>(sum);
+        if (!std::isfinite(result)) status.store(2);
+        if (bias != nullptr) result += bias[output_row];
+        output[flat] = result;
+    });
+    return status.load();
+}
+
+// Same arithmetic, same bits, but each weight row is decoded once and reused
+// for every input row.  Used by tests at sizes where the as-written form is
+// too slow; never reported as the CPU baseline.
+int nfo_linear(std::uint32_t encoding, const std::uint8_t* data,
+               std::int64_t out_dim, std::int64_t in_dim, const float* input,
+               std::int64_t rows, const float* bias, float* output,
+               int thread_cap, int q6_as_written) {
+    const std::int64_t elements = block_elements(encoding);
+    if (elements == 0 || in_dim % elements != 0 || rows <= 0) return 1;
+    const std::int64_t stride = in_dim / elements * block_bytes(encoding);
+    std::atomic<int> status{0};
+    parallel_for(out_dim, 8, thread_cap, [&](std::int64_t output_row) {
+        std::vector<float> weights(static_cast<std::size_t>(in_dim));
+        decode_row(encoding, data + output_row * stride, in_dim, q6_as_written != 0,
+                   weights.data());
+        for (std::int64_t input_row = 0; input_row < rows; ++input_row) {
+            const float* source = input + input_row * in_dim;
+            double sum = 0.0;
+            for (std::int64_t col = 0; col < in_dim; ++col) {
+                sum += static_cast<double>(source[col]) * weights[col];
+            }
+            float result = static_cast<float>(sum);
+            if (!std::isfinite(result)) status.store(2);
+            if (bias != nullptr) result += bias[output_row];
+            output[input_row * out_dim + output_row] = result;
+        }
+    });
+    return status.load();
+}
+
+// std::max_element: the first maximum wins (resident_glimmer.cpp:250-254).
+std::int64_t nfo_argmax(const float* values, std::int64_t count) {
+    if (count <= 0) return -1;
+    return static_cast<std::int64_t>(
+        std::distance(values, std::max_element(values, values + count)));
+}
+
+// kernels.cu:1527-1562 — per 32 values: inverse = 127/max, scale = 1/inverse,
+// code = clamp(roundf(x*inverse)), sum = float sum of the inputs.  The device
+// kernel sums by a shuffle tree; the order of that float sum is not part of the
+// contract (the probe allows 2e-5), so a serial float sum is used here.
+int nfo_quantize_q8_1(const float* input, std::int64_t rows, std::int64_t width,
+                      std::int8_t* codes, float* scales, float* sums) {
+    if (rows <= 0 || width <= 0 || width % 32 != 0) return 1;
+    const std::int64_t blocks = rows * (width / 32);
+    for (std::int64_t block = 0; block < blocks; ++block) {
+        float maximum = 0.0f;
+        float sum = 0.0f;
+        for (int lane = 0; lane < 32; ++lane) {
+            const float value = input[block * 32 + lane];
+            maximum = std::max(maximum, std::fabs(value));
+            sum += value;
+        }
+        const float inverse = maximum > 0.0f ? 127.0f / maximum : 0.0f;
+        const float scale = inverse > 0.0f ? 1.0f / inverse : 0.0f;
+        for (int lane = 0; lane < 32; ++lane) {
+            int code = inverse > 0.0f
+                ? static_cast<int>(std::round(input[block * 32 + lane] * inverse))
+                : 0;
+            code = std::max(-127, std::min(127, code));
+            codes[block * 32 + lane] = static_cast<std::int8_t>(code);
+        }
+        scales[block] = scale;
+        sums[block] = sum;
+    }
+    return 0;
+}
+
+// Round a float through IEEE half (round to nearest even) and back.
+float nfo_round_through_fp16(float value) {
+    std::uint32_t bits;
+    std::memcpy(&bits, &value, sizeof(bits));
+    const std::uint32_t sign = bits & 0x80000000u;
+    const std::uint32_t magnitude = bits & 0x7fffffffu;
+    std::uint16_t half = 0;
+    if (magnitude >= 0x7f800000u) {
+        half = magnitude > 0x7f800000u ? 0x7e00u : 0x7c00u;  // NaN / inf
+    } else if (magnitude >= 0x477ff000u) {
+        half = 0x7c00u;  // rounds to or beyond 65520 -> inf
+    } else if (magnitude >= 0x38800000u) {
+        // normal half: drop 13 mantissa bits, round to nearest even
+        const std::uint32_t shifted = magnitude - 0x38000000u;
+        const std::uint32_t rounded = shifted + 0x0fffu + ((shifted >> 13) & 1u);
+        half = static_cast<std::uint16_t>(rounded >> 13);
+    } else if (magnitude >= 0x33000000u) {
+        // subnormal half: value * 2^24 rounded to nearest even integer
+        float scaled;
+        std::uint32_t positive = magnitude;
+        std::memcpy(&scaled, &positive, sizeof(scaled));
+        half = static_cast<std::uint16_t>(std::nearbyint(std::ldexp(scaled, 24)));
+    }
+    std::uint8_t bytes[2];
+    std::memcpy(bytes, &half, 2);
+    const float result = fp16_to_float(bytes);
+    return sign ? -result : result;
+}
+
+// Q8_1-activation oracle: y = sum_c double(scale'*code) * w(r,c) (+bias), where
+// scale' is the activation scale rounded through fp16 for Q4_K/Q5_K and kept
+// in float for Q6_K (kernels.cu:1697-1718; probe :996-1003).  This is the
+// closed form the reference's own probe compares the int8 path with; it leaves
+// out the fp16 rounding of the block sum, which the probe's tolerance absorbs.
+int nfo_linear_q8_1(std::uint32_t encoding, const std::uint8_t* data,
+                    std::int64_t out_dim, std::int64_t in_dim,
+                    const std::int8_t* codes, const float* scales,
+                    std::int64_t rows, const float* bias, float* output) {
+    if (encoding != kEncQ4K && encoding != kEncQ5K && encoding != kEncQ6K) return 1;
+    if (in_dim % 256 != 0 || rows <= 0) return 1;
+    const std::int64_t stride = in_dim / 256 * block_bytes(encoding);
+    std::vector<float> reconstructed(static_cast<std::size_t>(rows * in_dim));
+    for (std::int64_t index = 0; index < rows * in_dim; ++index) {
+        float scale = scales[index / 32];
+        if (encoding != kEncQ6K) scale = nfo_round_through_fp16(scale);
+        reconstructed[index] = scale * static_cast<float>(codes[index]);
+    }
+    parallel_for(out_dim, 8, 0, [&](std::int64_t output_row) {
+        std::vector<float> weights(static_cast<std::size_t>(in_dim));
+        decode_row(encoding, data + output_row * stride, in_dim, false, weights.data());
+        for (std::int64_t input_row = 0; input_row < rows; ++input_row) {
+            double sum = bias != nullptr ? bias[output_row] : 0.0;
+            for (std::int64_t col = 0; col < in_dim; ++col) {
+                sum += static_cast<double>(reconstructed[input_row * in_dim + col]) *
+                    weights[col];
+            }
+            output[input_row * out_dim + output_row] = static_cast<float>(sum);
+        }
+    });
+    return 0;
+}
+
+// Standalone float forms of the two fused prologues, as the reference's
+// element-wise operators compute them (glimmer_k_mmq.cu:299-317, 369-376):
+//   gated  : x / (1 + expf(-g))
+//   swiglu : (up * gate) * (1 / (1 + expf(-gate)))
+// expf here is the host libm's; the device uses its own expf, so tests compare
+// the fused GPU path against the GPU's materialised path bit for bit and
+// against this form only to a tolerance.
+void nfo_sigmoid_gate(const float* input, const float* gate, float* output,
+                      std::int64_t count) {
+    for (std::int64_t index = 0; index < count; ++index) {
+        output[index] = input[index] / (1.0f + std::exp(-gate[index]));
+    }
+}
+
+void nfo_swiglu(const float* gate, const float* up, float* output, std::int64_t count) {
+    for (std::int64_t index = 0; index < count; ++index) {
+        const float sigmoid = 1.0f / (1.0f + std::exp(-gate[index]));
+        output[index] = (up[index] * gate[index]) * sigmoid;
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,157 @@
+"""The C ABI without a GPU: the library loads, exports every symbol the header
+declares, and fails closed on bad arguments before touching the device.
+
+Negative cases follow the reference probe
+(tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1429-1433, 1740-1762, 1834-1866).
+"""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from neuralfn_amd import kquant, tile_ops
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "nfn_mi355_tile_ops.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return tile_ops.load()
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(nfn_(?:native_tile|mi355)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    names = declared_symbols()
+    assert len(names) >= 28
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared but not exported"
+    assert set(names) == set(tile_ops.SIGNATURES), "binding and header disagree"
+
+
+def test_versions(lib):
+    for name in ("nfn_native_tile_ops_abi_version", "nfn_native_tile_strict_math_abi_version",
+                 "nfn_native_tile_packed_weight_abi_version",
+                 "nfn_native_tile_glimmer_inference_abi_version",
+                 "nfn_native_tile_k_quant_mmq_abi_version"):
+        assert getattr(lib, name)() == 1
+
+
+def test_descriptor_is_72_bytes():
+    assert ctypes.sizeof(tile_ops.PackedWeightDescriptor) == 72
+    assert tile_ops.PackedWeightDescriptor.data.offset == 16
+    assert tile_ops.PackedWeightDescriptor.row_stride_bytes.offset == 48
+    assert tile_ops.PackedWeightDescriptor.cuda_stream.offset == 64
+
+
+def _descriptor(encoding=kquant.Q4_K, out_dim=5, in_dim=512):
+    return tile_ops.make_descriptor(encoding, 0x1000, out_dim, in_dim)
+
+
+def test_validate_accepts_canonical_layouts(lib):
+    for encoding in (kquant.F32, kquant.BF16, kquant.Q8_0, kquant.Q4_K, kquant.Q5_K, kquant.Q6_K):
+        d = _descriptor(encoding)
+        assert lib.nfn_native_tile_packed_weight_validate_v1(ctypes.byref(d)) == 0
+
+
+@pytest.mark.parametrize("mutate", [
+    lambda d: setattr(d, "data_nbytes", d.data_nbytes - 1),
+    lambda d: setattr(d, "row_stride_bytes", d.row_stride_bytes - 1),
+    lambda d: setattr(d, "encoding", 0xFFFF),
+    lambda d: setattr(d, "encoding", 31),
+    lambda d: setattr(d, "version", 2),
+    lambda d: setattr(d, "flags", 1),
+    lambda d: setattr(d, "reserved0", 1),
+    lambda d: setattr(d, "reserved1", 1),
+    lambda d: setattr(d, "struct_size", 64),
+    lambda d: setattr(d, "data", None),
+    lambda d: setattr(d, "output_dim", 0),
+    lambda d: setattr(d, "input_dim", 511),
+])
+def test_validate_fails_closed(lib, mutate):
+    d = _descriptor()
+    mutate(d)
+    assert lib.nfn_native_tile_packed_weight_validate_v1(ctypes.byref(d)) == tile_ops.INVALID
+    assert lib.nfn_native_tile_packed_weight_validate_v1(None) == tile_ops.INVALID
+
+
+def test_workspace_contract(lib):
+    query = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1
+    assert query(5, 512) > 0 and query(1, 512) > 0
+    assert query(17, 512) == 0
+    assert query(0, 512) == 0
+    assert query(5, 511) == 0
+    assert query(16, 6656) >= query(1, 6656)
+    assert query(1, 512) >= 512 // 32 * 36  # at least the reference's one-row need
+
+
+def test_small_batch_entry_points_fail_closed_without_launching(lib):
+    d = _descriptor()
+    descriptors = (ctypes.POINTER(tile_ops.PackedWeightDescriptor) * 1)(ctypes.pointer(d))
+    outputs = (ctypes.c_void_p * 1)(0x2000)
+    need = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(5, 512)
+    mmq = lib.nfn_native_tile_k_quant_mmq_multi_linear_float32_v1
+    good = dict(x=0x3000, count=1, rows=5, ws=0x4000, ws_bytes=need)
+
+    def call(desc=descriptors, **kw):
+        a = {**good, **kw}
+        return mmq(desc, a["x"], outputs, a["count"], a["rows"], a["ws"], a["ws_bytes"], None)
+
+    assert call(ws_bytes=need - 1) == tile_ops.INVALID      # short workspace
+    assert call(rows=17) == tile_ops.INVALID                # unsupported row count
+    assert call(rows=0) == tile_ops.INVALID
+    assert call(count=0) == tile_ops.INVALID
+    assert call(count=5) == tile_ops.INVALID
+    assert call(x=None) == tile_ops.INVALID
+    assert call(ws=None) == tile_ops.INVALID
+    for mutate in (lambda v: setattr(v, "data_nbytes", v.data_nbytes - 1),
+                   lambda v: setattr(v, "encoding", 0xFFFF),
+                   lambda v: setattr(v, "encoding", kquant.F32),
+                   lambda v: setattr(v, "row_stride_bytes", v.row_stride_bytes - 1),
+                   lambda v: setattr(v, "cuda_stream", 0x1234)):
+        bad = _descriptor()
+        mutate(bad)
+        array = (ctypes.POINTER(tile_ops.PackedWeightDescriptor) * 1)(ctypes.pointer(bad))
+        assert call(desc=array) == tile_ops.INVALID
+    gated = lib.nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1
+    assert gated(descriptors, 0x3000, None, outputs, 1, 5, 0x4000, need, None) == tile_ops.INVALID
+    swiglu = lib.nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1
+    assert swiglu(descriptors, 0x3000, None, outputs, 1, 5, 0x4000, need, None) == tile_ops.INVALID
+    mmvq = lib.nfn_native_tile_k_quant_mmvq_linear_float32_v1
+    one = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(1, 512)
+    assert mmvq(ctypes.byref(d), 0x3000, 0x2000, 0x4000, one - 1, None) == tile_ops.INVALID
+    assert mmvq(None, 0x3000, 0x2000, 0x4000, one, None) == tile_ops.INVALID
+
+
+def test_other_entry_points_fail_closed(lib):
+    d = _descriptor()
+    assert lib.nfn_native_tile_linear_packed_weight_float32_v1(
+        ctypes.byref(d), 0x3000, None, 0x2000, 0, False) == tile_ops.INVALID
+    assert lib.nfn_native_tile_linear_packed_weight_float32_v1(
+        ctypes.byref(d), 0x3000, None, 0x2000, 1, True) == tile_ops.INVALID  # bias promised, absent
+    assert lib.nfn_native_tile_packed_weight_dequantize_float32_v1(
+        ctypes.byref(d), None) == tile_ops.INVALID
+    assert lib.nfn_native_tile_quantize_q8_1_float32_v1(
+        0x1, 0x2, 0x3, 0x4, 1, 33, None) == tile_ops.INVALID
+    f32 = _descriptor(kquant.F32)
+    assert lib.nfn_native_tile_linear_packed_weight_q8_1_float32_v1(
+        ctypes.byref(f32), 0x1, 0x2, 0x3, None, 0x4, 1, False) == tile_ops.INVALID
+    multi = lib.nfn_native_tile_linear_packed_weight_q8_1_multi_decode_float32_v1
+    assert multi(ctypes.byref(d), ctypes.byref(d), None, None, 0x1, 0x2, 0x3, 0x4, 0x5, None,
+                 None, 1, None) == tile_ops.INVALID                      # fewer than two
+    assert multi(ctypes.byref(d), ctypes.byref(d), ctypes.byref(d), None, 0x1, 0x2, 0x3, 0x4,
+                 0x5, None, None, 2, None) == tile_ops.INVALID           # unused slot not null
+    assert lib.nfn_native_tile_argmax_rows_float32_v1(0x1, 0x2, 0x3, 0, 8, None) == tile_ops.INVALID
+    assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(9, 1000) == 0
+    assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(512, 6656, 16384, 7) == 0
+    assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(512, 100, 16384, 0) == 0
+
+
+def test_error_string_never_null(lib):
+    for code in (0, 1, 2, 98, 719, 12345):
+        assert lib.nfn_native_tile_ops_error_string(code)

@@ -1,0 +1,480 @@
+"""Parity of the HIP library with the CPU oracle, through the C ABI.
+
+Known-answer and cross-path checks follow the reference's device probe
+(tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:650-1904).  The bar, from the
+build's contract: dequantized weights bit-exact; float outputs within
+max|y - ref| / max|ref| <= 2e-3 of the CPU engine's double-accumulate matmul;
+argmax indices exact.
+"""
+import ctypes
+import struct
+
+import numpy as np
+import pytest
+
+from neuralfn_amd import kquant, tile_ops
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 2e-3  # max relative error allowed against the CPU oracle
+K_ENCODINGS = [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K]
+ALL_PACKED = K_ENCODINGS + [kquant.Q8_0]
+
+
+def torch_():
+    import torch
+    return torch
+
+
+def to_device(array, device):
+    return torch_().from_numpy(np.ascontiguousarray(array)).to(device)
+
+
+def normalised_error(actual, expected):
+    scale = np.max(np.abs(expected))
+    return float(np.max(np.abs(actual.astype(np.float64) - expected.astype(np.float64))) / scale)
+
+
+def assert_bits_equal(a, b, label=""):
+    a = a.detach().cpu().numpy() if hasattr(a, "detach") else a
+    b = b.detach().cpu().numpy() if hasattr(b, "detach") else b
+    assert a.shape == b.shape, label
+    mismatch = np.flatnonzero(a.reshape(-1).view(np.uint32) != b.reshape(-1).view(np.uint32))
+    assert mismatch.size == 0, f"{label}: {mismatch.size} values differ, first at {mismatch[:4]}"
+
+
+def random_packed(encoding, out_dim, in_dim, seed):
+    rng = np.random.default_rng(seed)
+    elements, nbytes = kquant.BLOCKS[encoding]
+    blocks = rng.integers(0, 256, (out_dim * in_dim // elements, nbytes), dtype=np.uint8)
+    offsets = {kquant.Q4_K: (0, 2), kquant.Q5_K: (0, 2), kquant.Q6_K: (208,), kquant.Q8_0: (0,)}
+    for offset in offsets[encoding]:
+        blocks[:, offset + 1] = (blocks[:, offset + 1] & 0x83) | 0x24
+    return blocks.reshape(-1)
+
+
+def probe_packed(encoding, out_dim, in_dim, seed):
+    """make_packed of the reference probe (:1290-1327): patterned bytes, fixed d/dmin."""
+    _, nbytes = kquant.BLOCKS[encoding]
+    total = kquant.packed_nbytes(encoding, out_dim, in_dim)
+    index = np.arange(total, dtype=np.uint64)
+    packed = ((index * np.uint64(seed * 2 + 17) + np.uint64(seed)) & np.uint64(0xFF)).astype(np.uint8)
+    blocks = packed.reshape(out_dim, in_dim // 256, nbytes)
+    rows = np.arange(out_dim)[:, None]
+    if encoding in (kquant.Q4_K, kquant.Q5_K):
+        blocks[:, :, 0], blocks[:, :, 1], blocks[:, :, 2], blocks[:, :, 3] = 0x00, 0x28, 0x00, 0x24
+        for scale in range(12):
+            blocks[:, :, 4 + scale] = (1 + (scale + rows + seed) % 4).astype(np.uint8)
+    else:
+        for scale in range(16):
+            blocks[:, :, 192 + scale] = (((scale + rows + seed) % 11 - 5) & 0xFF).astype(np.uint8)
+        blocks[:, :, 208], blocks[:, :, 209] = 0x00, 0x28
+    return packed
+
+
+# ---------------------------------------------------------------- dequantize
+
+@pytest.mark.parametrize("encoding", ALL_PACKED + [kquant.F32, kquant.BF16])
+def test_dequantize_bit_exact(cuda, oracle, encoding):
+    out_dim, in_dim = 37, 1024
+    if encoding in (kquant.F32, kquant.BF16):
+        packed = kquant.quantize(encoding, kquant.synthetic_weights(3, out_dim, in_dim))
+    else:
+        packed = random_packed(encoding, out_dim, in_dim, 21 + encoding)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    actual = tile_ops.dequantize(weight).cpu().numpy()
+    expected = oracle.dequantize(encoding, packed, out_dim, in_dim)
+    assert_bits_equal(actual, expected, kquant.NAMES[encoding])
+
+
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_dequantize_bit_exact_quantized_weights(cuda, oracle, encoding):
+    out_dim, in_dim = 64, 6656
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(17, out_dim, in_dim))
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    assert_bits_equal(tile_ops.dequantize(weight), oracle.dequantize(encoding, packed, out_dim, in_dim))
+
+
+def test_q4_k_known_answer_through_the_abi(cuda, oracle):
+    # probe :650-746
+    block = bytes([0x00, 0x3C, 0x00, 0x38]) + bytes(range(1, 9)) + bytes(4) + bytes([0x21] * 128)
+    packed = np.frombuffer(block, np.uint8).copy()
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, packed, 1, 256)
+    values = tile_ops.dequantize(weight).cpu().numpy()[0]
+    assert np.all(values[:32] == -1.5) and np.all(values[32:64] == 1.0)
+    assert np.all(values[64:96] == -0.5) and np.all(values[96:128] == 4.0)
+    x = ((np.arange(256) % 17 - 8) / 19.0).astype(np.float32)[None, :]
+    y = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
+    expected = float(np.dot(values.astype(np.float64), x[0].astype(np.float64)))
+    assert abs(y[0, 0] - expected) <= 2e-4
+
+
+# ------------------------------------------------------- generic float linear
+
+@pytest.mark.parametrize("encoding", ALL_PACKED + [kquant.F32, kquant.BF16])
+def test_generic_linear_rows5_with_bias(cuda, oracle, encoding):
+    # probe :748-897: rows 5, out 5, in 512, patterned bytes, bias, tol 5e-3 absolute
+    rows, out_dim, in_dim = 5, 5, 512
+    if encoding in (kquant.F32, kquant.BF16):
+        packed = kquant.quantize(encoding, kquant.synthetic_weights(4, out_dim, in_dim, 1.0))
+    else:
+        packed = kquant.patterned_bytes(encoding, out_dim, in_dim)
+    r, c = np.arange(rows)[:, None], np.arange(in_dim)[None, :]
+    x = (((r * 37 + c * 13) % 257 - 128) / 257.0).astype(np.float32)
+    bias = ((np.arange(out_dim) - 2) / 7.0).astype(np.float32)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.linear(weight, to_device(x, cuda), to_device(bias, cuda)).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x, bias=bias)
+    assert np.max(np.abs(y - expected)) <= 5e-3
+    assert normalised_error(y, expected) <= 1e-5
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 7, 16, 23])
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_generic_linear_against_oracle(cuda, oracle, encoding, rows):
+    out_dim, in_dim = 257, 1024
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(31 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(77 + rows, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    assert normalised_error(y, expected) <= TOLERANCE
+
+
+# ------------------------------------------------------------ public Q8_1 path
+
+def crafted_q8_input(rows, in_dim):
+    """probe :899-920: every 32-block has scale exactly 1/32."""
+    x = np.zeros((rows, in_dim), np.float32)
+    for row in range(rows):
+        for block in range(in_dim // 32):
+            for lane in range(32):
+                code = 0
+                if lane == 0:
+                    code = -127
+                elif lane == 1:
+                    code = 127
+                elif lane == 2:
+                    code = 64 - 2 * (row % 5)
+                elif lane >= 4:
+                    magnitude = 1 + (block * 11 + (lane // 2) * 7 + row * 3) % 96
+                    code = magnitude if lane % 2 == 0 else -magnitude
+                x[row, block * 32 + lane] = code * 0.03125
+    return x
+
+
+@pytest.mark.parametrize("encoding", K_ENCODINGS)
+def test_q8_1_quantize_and_linear(cuda, oracle, encoding):
+    rows, out_dim, in_dim = 5, 7, 512
+    _, nbytes = kquant.BLOCKS[encoding]
+    packed = kquant.patterned_bytes(encoding, out_dim, in_dim, multiplier=41, offset=23)
+    x = crafted_q8_input(rows, in_dim)
+    bias = ((np.arange(out_dim) - 3) / 9.0).astype(np.float32)
+    codes, scales, sums = tile_ops.quantize_q8_1(to_device(x, cuda))
+    o_codes, o_scales, o_sums = oracle.quantize_q8_1(x)
+    assert np.array_equal(codes.cpu().numpy(), o_codes)
+    assert np.max(np.abs(scales.cpu().numpy() - o_scales)) <= 1e-7
+    assert np.max(np.abs(sums.cpu().numpy() - o_sums)) <= 2e-5
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.linear_q8_1(weight, codes, scales, sums, to_device(bias, cuda)).cpu().numpy()
+    expected = oracle.linear_q8_1(encoding, packed, out_dim, in_dim, o_codes, o_scales, bias)
+    assert np.max(np.abs(y - expected)) <= 8e-3  # probe :1019-1022
+
+
+def test_q8_1_quantize_random_matches_oracle(cuda, oracle):
+    x = kquant.synthetic_activations(5, 4, 6656)
+    x[1, 64:96] = 0.0
+    codes, scales, sums = tile_ops.quantize_q8_1(to_device(x, cuda))
+    o_codes, o_scales, o_sums = oracle.quantize_q8_1(x)
+    assert np.array_equal(codes.cpu().numpy(), o_codes)
+    assert np.array_equal(scales.cpu().numpy(), o_scales)
+    assert np.max(np.abs(sums.cpu().numpy() - o_sums)) <= 2e-5
+
+
+def test_q8_1_multi_decode_bit_exact_with_single(cuda):
+    # probe :1026-1202
+    in_dim = 512
+    specs = [(kquant.Q4_K, 5, 3), (kquant.Q5_K, 7, 5), (kquant.Q6_K, 3, 7), (kquant.Q4_K, 9, 11)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, probe_packed(e, n, in_dim, s), n, in_dim)
+               for e, n, s in specs]
+    x = (((np.arange(in_dim) * 19 + 7) % 251 - 125) / 47.0).astype(np.float32)[None, :]
+    codes, scales, sums = tile_ops.quantize_q8_1(to_device(x, cuda))
+    singles = [tile_ops.linear_q8_1(w, codes, scales, sums) for w in weights]
+    fused = tile_ops.linear_q8_1_multi_decode(weights, codes, scales, sums)
+    for index, (a, b) in enumerate(zip(singles, fused)):
+        assert_bits_equal(a, b, f"projection {index}")
+    fused2 = tile_ops.linear_q8_1_multi_decode(weights[:2], codes, scales, sums)
+    assert_bits_equal(singles[0], fused2[0])
+    assert_bits_equal(singles[1], fused2[1])
+
+
+# ----------------------------------------------- small-batch K-quant entry points
+
+@pytest.fixture(scope="module")
+def mixed(cuda):
+    """probe :1278-1390: rows 5, K 512, Q4_K x129, Q5_K x17, Q6_K x33."""
+    in_dim, rows = 512, 5
+    specs = [(kquant.Q4_K, 129, 3), (kquant.Q5_K, 17, 5), (kquant.Q6_K, 33, 7)]
+    packed = [probe_packed(e, n, in_dim, s) for e, n, s in specs]
+    weights = [tile_ops.PackedWeight.from_numpy(e, p, n, in_dim)
+               for (e, n, _), p in zip(specs, packed)]
+    r, c = np.arange(rows)[:, None], np.arange(in_dim)[None, :]
+    x = (((c * 19 + r * 23 + 7) % 251 - 125) / 47.0).astype(np.float32)
+    gate = (((np.arange(rows * in_dim) * 13 + 11) % 101 - 50) / 17.0).astype(np.float32)
+    return dict(specs=specs, packed=packed, weights=weights, x=x, gate=gate.reshape(rows, in_dim),
+                rows=rows, in_dim=in_dim)
+
+
+def test_small_batch_against_both_oracles(cuda, oracle, mixed):
+    rows, in_dim = mixed["rows"], mixed["in_dim"]
+    x = to_device(mixed["x"], cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    outputs = tile_ops.multi_linear(mixed["weights"], x, workspace)
+    o_codes, o_scales, _ = oracle.quantize_q8_1(mixed["x"])
+    for (encoding, out_dim, _), packed, y in zip(mixed["specs"], mixed["packed"], outputs):
+        y = y.cpu().numpy()
+        exact = oracle.linear(encoding, packed, out_dim, in_dim, mixed["x"])
+        assert normalised_error(y, exact) <= TOLERANCE
+        q8 = oracle.linear_q8_1(encoding, packed, out_dim, in_dim, o_codes, o_scales)
+        assert np.all(np.abs(y - q8) <= 2e-2 + 4e-4 * np.abs(q8))  # probe :1444-1458
+
+
+def test_one_row_paths_agree_bit_for_bit(cuda, oracle, mixed):
+    in_dim = mixed["in_dim"]
+    x = to_device(mixed["x"][:1], cuda)
+    workspace = tile_ops.small_batch_workspace(1, in_dim)
+    grouped = tile_ops.multi_linear(mixed["weights"], x, workspace)
+    direct = tile_ops.mmvq_linear(mixed["weights"][0], x, workspace)
+    assert_bits_equal(grouped[0], direct, "dedicated vs grouped one-row")  # probe :1520-1529
+    for (encoding, out_dim, _), packed, y in zip(mixed["specs"], mixed["packed"], grouped):
+        exact = oracle.linear(encoding, packed, out_dim, in_dim, mixed["x"][:1])
+        assert normalised_error(y.cpu().numpy(), exact) <= TOLERANCE
+
+
+@pytest.mark.parametrize("prologue", ["plain", "gated", "swiglu"])
+def test_verifier_rows_equal_row_by_row(cuda, mixed, prologue):
+    # probe :1588-1640: batched verifier == the one-row call per row, bit for bit
+    rows, in_dim = mixed["rows"], mixed["in_dim"]
+    x = to_device(mixed["x"], cuda)
+    second = to_device(mixed["gate"], cuda) if prologue != "plain" else None
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    one = tile_ops.small_batch_workspace(1, in_dim)
+    batched = tile_ops.multi_linear(mixed["weights"], x, workspace, second, "mmvq", prologue)
+    for row in range(rows):
+        single = tile_ops.multi_linear(
+            mixed["weights"], x[row:row + 1], one,
+            second[row:row + 1] if second is not None else None, "mmq", prologue)
+        for b, s in zip(batched, single):
+            assert_bits_equal(b[row:row + 1], s, f"{prologue} row {row}")
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+@pytest.mark.parametrize("prologue", ["gated", "swiglu"])
+def test_fused_prologue_equals_materialised(cuda, oracle, mixed, prologue, rows):
+    # probe :1659-1692, 1764-1833
+    in_dim = mixed["in_dim"]
+    x = to_device(mixed["x"][:rows], cuda)
+    g = to_device(mixed["gate"][:rows], cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    if prologue == "gated":
+        materialised = tile_ops.sigmoid_gate(x, g)
+        host = oracle.sigmoid_gate(mixed["x"][:rows], mixed["gate"][:rows])
+    else:
+        materialised = tile_ops.swiglu(x, g)  # x is the gate operand, g is `up`
+        host = oracle.swiglu(mixed["x"][:rows], mixed["gate"][:rows])
+    np.testing.assert_allclose(materialised.cpu().numpy(), host, rtol=2e-6, atol=1e-7)
+    baseline = tile_ops.multi_linear(mixed["weights"], materialised, workspace)
+    fused = tile_ops.multi_linear(mixed["weights"], x, workspace, g, "mmq", prologue)
+    for b, f in zip(baseline, fused):
+        assert_bits_equal(b, f, prologue)
+
+
+def test_small_batch_fails_closed_on_device(cuda, mixed):
+    # probe :1834-1866 with real device buffers
+    rows, in_dim = mixed["rows"], mixed["in_dim"]
+    lib = tile_ops.load()
+    x = to_device(mixed["x"], cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    weight = mixed["weights"][0]
+    out = torch_().full((rows, weight.output_dim), 123.0, device=cuda)
+
+    def call(descriptor, test_rows, ws_bytes):
+        array = (ctypes.POINTER(tile_ops.PackedWeightDescriptor) * 1)(ctypes.pointer(descriptor))
+        outs = (ctypes.c_void_p * 1)(out.data_ptr())
+        return lib.nfn_native_tile_k_quant_mmq_multi_linear_float32_v1(
+            array, x.data_ptr(), outs, 1, test_rows, workspace.data_ptr(), ws_bytes, None)
+
+    good = weight.descriptor()
+    for field, value in (("data_nbytes", good.data_nbytes - 1), ("encoding", 0xFFFF),
+                         ("row_stride_bytes", good.row_stride_bytes - 1)):
+        bad = weight.descriptor()
+        setattr(bad, field, value)
+        assert call(bad, rows, workspace.numel()) == tile_ops.INVALID
+    need = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(rows, in_dim)
+    assert call(good, rows, need - 1) == tile_ops.INVALID
+    assert call(good, 17, workspace.numel()) == tile_ops.INVALID
+    torch_().cuda.synchronize()
+    assert bool((out == 123.0).all()), "a rejected call wrote to its output"
+    assert call(good, rows, need) == 0
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8, 16])
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_small_batch_quantized_weights(cuda, oracle, encoding, rows):
+    out_dim, in_dim = 272, 1024
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(50 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(60 + rows, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    y = tile_ops.multi_linear([weight], to_device(x, cuda), workspace)[0].cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    assert normalised_error(y, expected) <= TOLERANCE
+
+
+# ------------------------------------------------------------------- argmax
+
+def test_argmax_rows_tie_rule_at_vocabulary_width(cuda):
+    # probe :1869-1904
+    rows, width = 3, 202048
+    values = np.full((rows, width), -9.0, np.float32)
+    values[0, 17] = 10.0
+    values[0, 123] = 10.0
+    values[1, width - 1] = 5.5
+    values[2, 0] = -1.0
+    indices, maxima = tile_ops.argmax_rows(to_device(values, cuda))
+    assert indices.cpu().tolist() == [17, width - 1, 0]
+    assert maxima.cpu().tolist() == [10.0, 5.5, -1.0]
+
+
+def test_argmax_rows_random_and_nan(cuda, oracle):
+    rng = np.random.default_rng(1)
+    values = rng.standard_normal((4, 50001)).astype(np.float32)
+    values[1, 100] = np.nan
+    values[2, :] = np.nan
+    values[3, 7] = values[3].max()
+    indices, maxima = tile_ops.argmax_rows(to_device(values, cuda))
+    indices = indices.cpu().tolist()
+    assert indices[0] == oracle.argmax(values[0])
+    assert indices[1] == int(np.nanargmax(values[1]))
+    assert indices[2] == 0 and maxima.cpu()[2].item() == -np.inf
+    assert indices[3] == min(7, int(np.argmax(values[3])))
+
+
+@pytest.mark.parametrize("rows", [1, 3, 8])
+@pytest.mark.parametrize("encoding", [kquant.Q6_K, kquant.Q4_K, kquant.Q5_K])
+def test_lm_head_fused_argmax_against_oracle(cuda, oracle, encoding, rows):
+    out_dim, in_dim = 4099, 1024
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(80 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(90 + rows, rows, in_dim, rms_normalize=True)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    indices, maxima = tile_ops.lm_head_argmax(weight, to_device(x, cuda))
+    logits = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    scale = np.max(np.abs(logits))
+    for row in range(rows):
+        ordered = np.sort(logits[row])[::-1]
+        assert abs(maxima.cpu()[row].item() - ordered[0]) <= TOLERANCE * scale
+        if ordered[0] - ordered[1] > 2 * TOLERANCE * scale:  # argmax exact on non-tied rows
+            assert indices.cpu()[row].item() == oracle.argmax(logits[row])
+        else:
+            assert logits[row, indices.cpu()[row].item()] >= ordered[0] - 2 * TOLERANCE * scale
+
+
+def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda):
+    # Two identical vocabulary rows far apart: the lower index must win.
+    out_dim, in_dim = 3000, 512
+    w = kquant.synthetic_weights(5, out_dim, in_dim)
+    x = kquant.synthetic_activations(6, 1, in_dim)
+    best = w[100] * 0 + np.sign(x[0]) * 0.05
+    w[100] = best
+    w[2900] = best
+    packed = kquant.quantize(kquant.Q6_K, w)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q6_K, packed, out_dim, in_dim)
+    indices, _ = tile_ops.lm_head_argmax(weight, to_device(x, cuda))
+    assert indices.cpu().tolist() == [100]
+
+
+# ------------------------------------------------ the benchmark's geometries
+
+def config_layer(seed, encoding=kquant.Q4_K):
+    shapes = {"q": (4096, 6656), "k": (256, 6656), "v": (256, 6656), "o": (6656, 4096)}
+    return {name: (shape, kquant.quantize(encoding, kquant.synthetic_weights(seed + i, *shape)))
+            for i, (name, shape) in enumerate(shapes.items())}
+
+
+@pytest.mark.parametrize("rows", [1, 4, 8])
+def test_config1_attention_projections(cuda, oracle, rows):
+    layer = config_layer(1000)
+    x = kquant.synthetic_activations(2000 + rows, rows, 6656)
+    attn = kquant.synthetic_activations(3000 + rows, rows, 4096)
+    weights = {n: tile_ops.PackedWeight.from_numpy(kquant.Q4_K, p, *s) for n, (s, p) in layer.items()}
+    workspace = tile_ops.small_batch_workspace(16, 6656)
+    q, k, v = tile_ops.multi_linear([weights["q"], weights["k"], weights["v"]],
+                                    to_device(x, cuda), workspace)
+    (o,) = tile_ops.multi_linear([weights["o"]], to_device(attn, cuda), workspace)
+    for name, y, source in (("q", q, x), ("k", k, x), ("v", v, x), ("o", o, attn)):
+        (out_dim, in_dim), packed = layer[name]
+        expected = oracle.linear(kquant.Q4_K, packed, out_dim, in_dim, source)
+        assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE, name
+    if rows == 1:  # config 0 is the Q projection at M=1 through the decode GEMV
+        direct = tile_ops.mmvq_linear(weights["q"], to_device(x, cuda), workspace)
+        assert_bits_equal(direct, q, "config 0")
+
+
+def test_config4_mixed_formats_dispatch(cuda, oracle):
+    # per-tensor formats drawn by seed, V/O/down at least Q5_K; decode (M=1)
+    rng = np.random.default_rng(4)
+    low = [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0]
+    high = [kquant.Q5_K, kquant.Q6_K, kquant.Q8_0]
+    in_dim = 1024
+    names = {"q": (512, low), "k": (256, low), "v": (256, high), "gate": (768, low)}
+    x = kquant.synthetic_activations(41, 1, in_dim)
+    weights, packed_all = [], []
+    for index, (name, (out_dim, choices)) in enumerate(names.items()):
+        encoding = int(rng.choice(choices))
+        packed = kquant.quantize(encoding, kquant.synthetic_weights(400 + index, out_dim, in_dim))
+        packed_all.append((encoding, out_dim, packed))
+        weights.append(tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim))
+    workspace = tile_ops.small_batch_workspace(1, in_dim)
+    outputs = tile_ops.multi_linear(weights, to_device(x, cuda), workspace)
+    for (encoding, out_dim, packed), y in zip(packed_all, outputs):
+        expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+        assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE
+
+
+@pytest.mark.parametrize("mode", [tile_ops.GEMM_BF16, tile_ops.GEMM_INT8])
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_prefill_gemm_against_oracle(cuda, oracle, encoding, mode):
+    rows, out_dim, in_dim = 160, 384, 1024
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(70 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(71, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), mode).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    error = normalised_error(y, expected)
+    if mode == tile_ops.GEMM_BF16:
+        assert error <= TOLERANCE
+    else:
+        # int8 activations per 32 values are a separate numerics tier: compared
+        # with the Q8_1-activation oracle at the reference's own tolerance
+        # (probe :1444-1458), and reported against the float oracle.
+        codes, scales, _ = oracle.quantize_q8_1(x)
+        if encoding in K_ENCODINGS:
+            q8 = oracle.linear_q8_1(encoding, packed, out_dim, in_dim, codes, scales)
+            assert np.all(np.abs(y - q8) <= 2e-2 + 4e-4 * np.abs(q8))
+        assert error <= 2e-2
+
+
+def test_prefill_gemm_full_size_row_subset(cuda, oracle):
+    # BASELINE shape (M=512, 6656 -> 16384): check a slice of output columns.
+    rows, out_dim, in_dim = 512, 16384, 6656
+    torch = torch_()
+    generator = torch.Generator(device="cpu").manual_seed(5)
+    packed = random_packed(kquant.Q4_K, 256, in_dim, 91)
+    full = np.tile(packed.reshape(256, -1), (out_dim // 256, 1)).reshape(-1)
+    x = kquant.synthetic_activations(92, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, full, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_BF16).cpu().numpy()
+    expected = oracle.linear(kquant.Q4_K, packed, 256, in_dim, x)
+    assert normalised_error(y[:, :256], expected) <= TOLERANCE
+    # every 256-column stripe repeats the same weights
+    assert np.array_equal(y[:, :256], y[:, out_dim - 256:])
