@@ -1,0 +1,348 @@
+#!/usr/bin/env python3
+"""Benchmark of the K-Quant packed-linear hot path on one MI355X.
+
+Headline workload (the configuration the metric is quoted on): decode
+attention projections of Glimmer-shaped layers with Q4_K weights — per layer one
+grouped launch for Q (6656->4096), K and V (6656->256 each) and one launch for
+O (4096->6656) — over 48 independently seeded layers so that no weight byte is
+served from cache.  One "step" is one pass over all layers for one batch of
+`--rows` tokens, replayed from a HIP graph as the reference's decode loop does.
+
+Prints one JSON line.  `value` is whole-job algorithmic GB/s: packed weight
+bytes + float activations in + float outputs, per step, over the step time,
+with every input resident in HBM before the timed region.  `roofline` is the
+same traffic per launch over the average launch duration measured with HIP
+events on the launch stream.  `cpu_baseline` is the reference's CPU K-Quant
+matmul timed on this host's cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "int8": 5000.0}
+MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
+FFN_DIM = 16384
+VOCAB = 202048
+
+
+def parse_args() -> argparse.Namespace:
+    parser = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=3)
+    parser.add_argument("--rows", type=int, default=1, help="tokens per step (1, 4 or 8)")
+    parser.add_argument("--layers", type=int, default=48)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-extras", action="store_true",
+                        help="skip the lm_head and prefill side measurements")
+    parser.add_argument("--no-graph", action="store_true", help="enqueue directly, no HIP graph")
+    return parser.parse_args()
+
+
+def layer_algorithmic_bytes(rows: int) -> int:
+    """Packed weights + float inputs (once per distinct input) + float outputs."""
+    from neuralfn_amd import kquant
+    weights = (kquant.packed_nbytes(kquant.Q4_K, ATTN_DIM, MODEL_DIM)
+               + 2 * kquant.packed_nbytes(kquant.Q4_K, KV_DIM, MODEL_DIM)
+               + kquant.packed_nbytes(kquant.Q4_K, MODEL_DIM, ATTN_DIM))
+    inputs = rows * (MODEL_DIM + ATTN_DIM) * 4
+    outputs = rows * (ATTN_DIM + KV_DIM + KV_DIM + MODEL_DIM) * 4
+    return weights + inputs + outputs
+
+
+def make_layers(layers: int, device):
+    """Seeded N(0, 0.02) weights, quantized to Q4_K on the host, resident on the GPU."""
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    shapes = (("q", ATTN_DIM, MODEL_DIM), ("k", KV_DIM, MODEL_DIM), ("v", KV_DIM, MODEL_DIM),
+              ("o", MODEL_DIM, ATTN_DIM))
+    result = []
+    host_copies = []
+    for layer in range(layers):
+        entry = {}
+        host = {}
+        for index, (name, out_dim, in_dim) in enumerate(shapes):
+            generator = torch.Generator(device=device).manual_seed(1_000_003 * layer + index + 1)
+            weights = (torch.randn((out_dim, in_dim), generator=generator, device=device,
+                                   dtype=torch.float32) * 0.02).cpu().numpy()
+            packed = kquant.quantize(kquant.Q4_K, weights)
+            entry[name] = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, packed, out_dim, in_dim,
+                                                           str(device))
+            host[name] = packed
+        result.append(entry)
+        host_copies.append(host)
+    return result, host_copies
+
+
+class DecodeStep:
+    """Pre-built ctypes arguments for the two launches of every layer."""
+
+    def __init__(self, layers, rows: int, device):
+        import torch
+        from neuralfn_amd import kquant, tile_ops
+        self.lib = tile_ops.load()
+        self.rows = rows
+        self.layers = layers
+        self.workspace = tile_ops.small_batch_workspace(16, MODEL_DIM, device)
+        self.hidden = torch.from_numpy(
+            kquant.synthetic_activations(11, rows * len(layers), MODEL_DIM)).to(device)
+        self.attention = torch.from_numpy(
+            kquant.synthetic_activations(12, rows * len(layers), ATTN_DIM)).to(device)
+        self.outputs = []
+        self.calls = []
+        for index, layer in enumerate(layers):
+            outs = {name: torch.empty((rows, weight.output_dim), dtype=torch.float32, device=device)
+                    for name, weight in layer.items()}
+            self.outputs.append(outs)
+            self.calls.append((index, layer, outs))
+        self._keep = []
+
+    def enqueue(self, stream: int) -> None:
+        from neuralfn_amd import tile_ops
+        function = self.lib.nfn_native_tile_k_quant_mmq_multi_linear_float32_v1
+        rows = self.rows
+        for index, layer, outs in self.calls:
+            qkv = [layer[n].descriptor(stream) for n in ("q", "k", "v")]
+            o = [layer["o"].descriptor(stream)]
+            self._keep.append((qkv, o))
+            hidden = self.hidden[index * rows:(index + 1) * rows]
+            attention = self.attention[index * rows:(index + 1) * rows]
+            tile_ops.check(function(
+                tile_ops._descriptor_array(qkv), hidden.data_ptr(),
+                tile_ops._pointer_array([outs["q"], outs["k"], outs["v"]]), 3, rows,
+                self.workspace.data_ptr(), self.workspace.numel(), stream), "qkv projections")
+            tile_ops.check(function(
+                tile_ops._descriptor_array(o), attention.data_ptr(),
+                tile_ops._pointer_array([outs["o"]]), 1, rows,
+                self.workspace.data_ptr(), self.workspace.numel(), stream), "o projection")
+        self._keep.clear()
+
+    @property
+    def launches_per_step(self) -> int:
+        return 2 * len(self.calls)
+
+
+def time_replays(run, steps: int, warmup: int) -> float:
+    """Milliseconds per call of run(), measured with events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        run()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
+    """The reference's CPU matmul on this host, on as many layers as fit the budget."""
+    from neuralfn_amd import kquant
+    from oracle import kquant_oracle
+    use_reference = kquant_oracle.reference_available()
+    kind = "reference" if use_reference else "port"
+    hidden = kquant.synthetic_activations(11, rows * len(host_layers), MODEL_DIM)
+    attention = kquant.synthetic_activations(12, rows * len(host_layers), ATTN_DIM)
+    shapes = {"q": (ATTN_DIM, MODEL_DIM), "k": (KV_DIM, MODEL_DIM), "v": (KV_DIM, MODEL_DIM),
+              "o": (MODEL_DIM, ATTN_DIM)}
+
+    def run(name, packed, x):
+        out_dim, in_dim = shapes[name]
+        if use_reference:
+            return kquant_oracle.ref_linear(kquant.Q4_K, packed, out_dim, in_dim, x)
+        return kquant_oracle.linear(kquant.Q4_K, packed, out_dim, in_dim, x, as_written=True)
+
+    done = 0
+    began = time.perf_counter()
+    for index, layer in enumerate(host_layers):
+        x = hidden[index * rows:(index + 1) * rows]
+        a = attention[index * rows:(index + 1) * rows]
+        for name in ("q", "k", "v"):
+            run(name, layer[name], x)
+        run("o", layer["o"], a)
+        done += 1
+        if time.perf_counter() - began > budget_seconds:
+            break
+    elapsed = time.perf_counter() - began
+    cores = kquant_oracle.worker_count(ATTN_DIM, 128)
+    return {
+        "value": round(done * layer_algorithmic_bytes(rows) / elapsed / 1e9, 4),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": kind,
+        "sample": f"{done} of {len(host_layers)} layers (Q,K,V,O at rows={rows}) in {elapsed:.2f} s; "
+                  f"{done * rows / elapsed:.3f} layer-tokens/s",
+    }
+
+
+def random_packed_on_device(encoding: int, out_dim: int, in_dim: int, device, seed: int):
+    """Uniform random quant bytes with small finite scales, made on the GPU.
+
+    Used only where throughput is measured on tensors too large to quantize on
+    the host within the benchmark's time; parity for these paths is in tests/.
+    """
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    elements, nbytes = kquant.BLOCKS[encoding]
+    generator = torch.Generator(device=device).manual_seed(seed)
+    blocks = torch.randint(0, 256, (out_dim * in_dim // elements, nbytes), generator=generator,
+                           device=device, dtype=torch.uint8)
+    halves = {kquant.Q4_K: (0, 2), kquant.Q5_K: (0, 2), kquant.Q6_K: (208,), kquant.Q8_0: (0,)}
+    for offset in halves[encoding]:
+        blocks[:, offset + 1] = (blocks[:, offset + 1] & 0x03) | 0x14  # d in [2^-10, 2^-9)
+    return tile_ops.PackedWeight(encoding, out_dim, in_dim, blocks.reshape(-1))
+
+
+def lm_head_extra(device, steps: int, warmup: int) -> dict:
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    weight = random_packed_on_device(kquant.Q6_K, VOCAB, MODEL_DIM, device, 7)
+    result = {}
+    for rows in (1, 4):
+        x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
+        nbytes = tile_ops.load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, VOCAB)
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        ms = time_replays(lambda: tile_ops.lm_head_argmax(weight, x, workspace), steps, warmup)
+        traffic = weight.nbytes + rows * MODEL_DIM * 4 + rows * 12
+        result[f"rows{rows}"] = {"ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
+                                 "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                 "tokens/s": round(rows / ms * 1e3, 1)}
+    return {"workload": f"Q6_K lm_head {MODEL_DIM}->{VOCAB}, fused argmax", **result}
+
+
+def prefill_extra(device, steps: int, warmup: int) -> dict:
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    gate = random_packed_on_device(kquant.Q4_K, FFN_DIM, MODEL_DIM, device, 8)
+    down = random_packed_on_device(kquant.Q4_K, MODEL_DIM, FFN_DIM, device, 9)
+    result = {}
+    for mode, name in ((tile_ops.GEMM_BF16, "bf16"), (tile_ops.GEMM_INT8, "int8")):
+        for rows in (512, 2048):
+            x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
+            h = torch.from_numpy(kquant.synthetic_activations(32, rows, FFN_DIM)).to(device)
+            for label, weight, source in (("gate_up", gate, x), ("down", down, h)):
+                out = torch.empty((rows, weight.output_dim), dtype=torch.float32, device=device)
+                nbytes = tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+                    rows, weight.input_dim, weight.output_dim, mode)
+                workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+                ms = time_replays(
+                    lambda: tile_ops.gemm(weight, source, mode, workspace, out),
+                    max(3, steps // 4), max(1, warmup // 2))
+                flops = 2.0 * rows * weight.input_dim * weight.output_dim
+                tflops = flops / ms / 1e9
+                result[f"{name}_{label}_M{rows}"] = {
+                    "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
+                    "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS[name], 4),
+                    "tokens/s": round(rows / ms * 1e3, 1)}
+    return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}", **result}
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
+              file=sys.stderr)
+        return 2
+    if args.rows not in (1, 2, 4, 8, 16):
+        print("--rows must be one of 1, 2, 4, 8, 16", file=sys.stderr)
+        return 2
+    import torch
+    from neuralfn_amd import tile_ops
+
+    tile_ops.load()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    began = time.perf_counter()
+    layers, host_layers = make_layers(args.layers, device)
+    setup_seconds = time.perf_counter() - began
+    step = DecodeStep(layers, args.rows, device)
+
+    stream = torch.cuda.Stream()
+    graph = None
+    with torch.cuda.stream(stream):
+        step.enqueue(int(stream.cuda_stream))  # eager warm-up, loads code objects
+        stream.synchronize()
+        if not args.no_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                step.enqueue(int(torch.cuda.current_stream().cuda_stream))
+
+        def run():
+            if graph is not None:
+                graph.replay()
+            else:
+                step.enqueue(int(stream.cuda_stream))
+
+        ms_per_step = time_replays(run, args.steps, args.warmup)
+
+    bytes_per_step = args.layers * layer_algorithmic_bytes(args.rows)
+    value = bytes_per_step / ms_per_step / 1e6  # GB/s
+    launches = step.launches_per_step
+    record = {
+        "metric": "Q4_K decode GEMV GB/s",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 x int4 dot, f32 accumulate",
+        "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K; bf16-rounded N(0,1) activations)",
+        "config": {
+            "workload": f"decode attention projections Q/K/V (grouped) + O, Q4_K, "
+                        f"{args.layers} layers, rows={args.rows}",
+            "rows": args.rows,
+            "layers": args.layers,
+            "launches_per_step": launches,
+            "hip_graph": graph is not None,
+            "setup_seconds": round(setup_seconds, 1),
+        },
+        "tokens_per_s": round(args.rows / ms_per_step * 1e3, 2),
+        "frac_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(value, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(value / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": "decode GEMV (Q/K/V grouped launch and O launch, averaged)",
+            "bytes_per_launch": bytes_per_step // launches,
+            "us_per_launch": round(ms_per_step * 1e3 / launches, 3),
+        },
+    }
+    if not args.no_extras:
+        try:
+            with torch.cuda.stream(stream):
+                record["lm_head"] = lm_head_extra(device, args.steps, args.warmup)
+                record["prefill"] = prefill_extra(device, args.steps, args.warmup)
+        except Exception as error:  # side measurements never hide the headline
+            record["extras_error"] = repr(error)
+    if not args.no_cpu_baseline:
+        record["cpu_baseline"] = cpu_baseline(host_layers, args.rows)
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -235,8 +235,12 @@ def test_small_batch_against_both_oracles(cuda, oracle, mixed):
         y = y.cpu().numpy()
         exact = oracle.linear(encoding, packed, out_dim, in_dim, mixed["x"])
         assert normalised_error(y, exact) <= TOLERANCE
+        # The reference checks this entry point against its int8-activation
+        # path (probe :1444-1458).  This library keeps 16 bits of every
+        # activation here, so it has to sit closer to the float oracle than
+        # that int8 result does, not within the int8 path's own tolerance.
         q8 = oracle.linear_q8_1(encoding, packed, out_dim, in_dim, o_codes, o_scales)
-        assert np.all(np.abs(y - q8) <= 2e-2 + 4e-4 * np.abs(q8))  # probe :1444-1458
+        assert normalised_error(y, exact) <= normalised_error(q8, exact)
 
 
 def test_one_row_paths_agree_bit_for_bit(cuda, oracle, mixed):
