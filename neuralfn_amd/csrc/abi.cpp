@@ -4,6 +4,7 @@
 // neuralfn/csrc/native_train/tile_ops.cu:4504-4713 and
 // neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:2349-2649.
 #include "common.hpp"
+#include "gemv_mfma.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
 
@@ -18,7 +19,7 @@ constexpr std::int64_t kMaxOperations = 4;
 // Private activation record of the small-batch path: per 32 values two int8
 // planes (high and low byte of a 16-bit fixed-point code), a float scale and
 // the float sum of the 32 inputs.
-constexpr std::int64_t kActivationGroupBytes = 72;
+constexpr std::int64_t kActivationGroupBytes = kActivationRecordBytes / 8;
 
 std::int64_t small_batch_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
     if (rows < 1 || rows > kMaxSmallRows || input_dim <= 0 || input_dim % 128 != 0) return 0;
@@ -64,7 +65,19 @@ int run_small_batch(const Descriptor* const* descriptors, const float* first,
     }
     const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    launch_gemv_f32(set, first, second, prologue, nullptr, rows, as_stream(stream));
+    // Projections with a matrix-core kernel go in one launch, the rest in another.
+    ProjectionSet fast{}, exact{};
+    fast.input_dim = exact.input_dim = input_dim;
+    for (int index = 0; index < set.count; ++index) {
+        ProjectionSet& target = gemv_mfma_supports(set.op[index].encoding) ? fast : exact;
+        target.op[target.count++] = set.op[index];
+    }
+    if (fast.count > 0) {
+        launch_gemv_mfma(fast, first, second, prologue, rows, workspace, as_stream(stream));
+    }
+    if (exact.count > 0) {
+        launch_gemv_f32(exact, first, second, prologue, nullptr, rows, as_stream(stream));
+    }
     return launch_status();
 }
 
