@@ -69,7 +69,7 @@ int run_small_batch(const Descriptor* const* descriptors, const float* first,
     ProjectionSet fast{}, exact{};
     fast.input_dim = exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
-        ProjectionSet& target = gemv_mfma_supports(set.op[index].encoding) ? fast : exact;
+        ProjectionSet& target = gemv_mfma_supports(set.op[index].encoding, input_dim) ? fast : exact;
         target.op[target.count++] = set.op[index];
     }
     if (fast.count > 0) {

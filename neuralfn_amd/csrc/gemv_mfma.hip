@@ -1,41 +1,54 @@
 // Decode / small-batch GEMV on the int8 matrix cores.
 //
-// One workgroup (4 waves) owns a tile of 16 consecutive weight rows; the waves
-// split the K dimension by super-block ranges and meet once, at the end, in a
-// fixed-order sum.  Per 256-value super-block a wave
-//   1. copies its 16 x block_bytes of packed weights from HBM to a private LDS
-//      tile with fully coalesced 16-byte loads (prefetched DEPTH blocks ahead),
-//   2. turns the 256 activations of that block into two int8 planes (the high
-//      and low byte of a 16-bit fixed-point code, one scale per 32 values) —
-//      in this launch for one token, or read from the workspace for 2..8,
-//   3. unpacks 4/5/6/8-bit codes to int8 straight from LDS in the operand
-//      layout of v_mfma_i32_16x16x32_i8 (weights are the B operand: lane
-//      l holds row l%16, k-chunk l/16; the token planes are rows of A),
-//   4. scales the int32 dot products of each 32-value sub-block in float.
+// A workgroup of 8 waves owns tiles of 32 consecutive weight rows (persistent:
+// it walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...).  The waves split the
+// K dimension by super-block ranges and meet once per tile in a fixed-order
+// sum.  A wave first loads its share of the activations and starts the loads
+// of its first packed blocks, then — while those fly — turns the activations
+// into two int8 planes (high and low byte of a 16-bit fixed-point code, one
+// scale per 256 values) kept in LDS for every tile it will visit; for 2..16
+// tokens the planes come from the workspace, written by a small quantizer
+// launch.  Per 256-value super-block the wave then
+//   1. stores its 32 x block_bytes of packed weights, loaded with coalesced
+//      16-byte accesses several blocks ahead (across tile boundaries), into a
+//      private LDS tile,
+//   2. unpacks 4/5/6-bit codes to int8 straight from LDS in the operand layout
+//      of v_mfma_i32_32x32x32_i8 (weights are the B operand: lane l holds row
+//      l%32, k-half l/32; the token planes are rows of A),
+//   3. weights the int32 dot products of every sub-block with its integer
+//      sub-scale (24-bit multiply-add) and converts to float once per block.
 // Every weight byte is read from HBM exactly once per launch.
 //
 // Arithmetic it replaces: the reference's one-row and small-batch kernels
 // (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:714-890, 1174-1303), which
 // quantize activations to 8 bits; here 16 bits are kept so the result stays
 // within 2e-3 of the float-activation CPU engine
-// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:655-679).
-//   y[t][j] = sum_blocks d*sum_sub sc_sub*s[t][sub]*(256*dot(q,hi) + dot(q,lo))
-//                        - dmin*sum_sub m_sub*S[t][sub]
-// with s the activation scale and S the float sum of the 32 activations.
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:655-679).  With x = s*c,
+// c = 256*hi + lo the 16-bit code of an activation and s its block scale:
+//   Q4_K/Q5_K: y += s*(d*sum_sub sc*dot(q, c) - dmin*sum_sub m*sum(c))
+//   Q6_K:      y += s*d*sum_16 sc8*dot(q - 32, c)
 #include "common.hpp"
 #include "gemv_mfma.hpp"
+
+#include <type_traits>
 
 namespace nfn {
 
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kTileRows = 16;
-constexpr int kWaves = 4;
+constexpr int kTileRows = 32;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
-constexpr float kCodeRange = 32512.0f;  // 127*256: high byte stays in [-127, 127]
+constexpr float kCodeRange = 32512.0f;  // 127*256: the high byte stays in [-127, 127]
 constexpr int kActRecord = kActivationRecordBytes;
+// record layout: [0,256) high plane, [256,512) low plane, [512,544) eight int32
+// sums of the codes per 32 values, [544,548) float scale, rest padding
+constexpr int kRecordSums = 512;
+constexpr int kRecordScale = 544;
+constexpr int kEarlyBlocks = 4;  // activation blocks per wave loaded before the weights
 
 struct __attribute__((packed, aligned(2))) Chunk16 {
     std::uint32_t v[4];
@@ -47,9 +60,9 @@ template <>
 struct Format<kEncQ4K> {
     static constexpr int kBlockBytes = 144;
     static constexpr int kChunks = 9;    // 16-byte chunks copied per block
-    static constexpr int kLdsRow = 144;  // (kLdsRow/4) % 64 must be 4*odd: conflict-free reads
+    static constexpr int kLdsRow = 144;  // (kLdsRow/4) % 64 is 4*odd: conflict-free operand reads
     static constexpr bool kAligned = true;
-    static constexpr bool kHasMin = true;
+    static constexpr int kDepth = 4;     // packed blocks in flight per wave
 };
 template <>
 struct Format<kEncQ5K> {
@@ -57,7 +70,7 @@ struct Format<kEncQ5K> {
     static constexpr int kChunks = 11;
     static constexpr int kLdsRow = 176;
     static constexpr bool kAligned = true;
-    static constexpr bool kHasMin = true;
+    static constexpr int kDepth = 3;
 };
 template <>
 struct Format<kEncQ6K> {
@@ -65,242 +78,265 @@ struct Format<kEncQ6K> {
     static constexpr int kChunks = 14;  // 224 bytes: the tail reads into the next block
     static constexpr int kLdsRow = 240;
     static constexpr bool kAligned = false;
-    static constexpr bool kHasMin = false;
+    static constexpr int kDepth = 3;
 };
-template <>
-struct Format<kEncQ8_0> {
-    static constexpr int kBlockBytes = 272;  // eight 34-byte blocks
-    static constexpr int kChunks = 17;
-    static constexpr int kLdsRow = 272;
-    static constexpr bool kAligned = false;
-    static constexpr bool kHasMin = false;
-};
-
-constexpr int kMaxLdsTile = kTileRows * 272;
 
 template <int CTRL>
+__device__ __forceinline__ int dpp_move(int value) {
+    return __builtin_amdgcn_update_dpp(0, value, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
 __device__ __forceinline__ float dpp_move(float value) {
-    return __builtin_bit_cast(
-        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), CTRL, 0xF, 0xF, true));
+    return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, value)));
 }
 
-// Reductions over the 8 lanes that share one 32-value group: quad xor 1, quad
-// xor 2, then the mirrored half row (lane k <-> 7-k) brings in the other quad.
-__device__ __forceinline__ float group8_max(float v) {
-    v = fmaxf(v, dpp_move<0xB1>(v));
-    v = fmaxf(v, dpp_move<0x4E>(v));
-    v = fmaxf(v, dpp_move<0x141>(v));
-    return v;
+constexpr int kQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141;  // lane k <-> 7-k within 8 lanes
+constexpr int kRowMirror = 0x140;   // lane k <-> 15-k within 16 lanes
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
-__device__ __forceinline__ float group8_sum(float v) {
-    v += dpp_move<0xB1>(v);
-    v += dpp_move<0x4E>(v);
-    v += dpp_move<0x141>(v);
-    return v;
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_move<kQuadXor1>(v));
+    v = fmaxf(v, dpp_move<kQuadXor2>(v));
+    v = fmaxf(v, dpp_move<kHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kRowMirror>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
+                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
 __device__ __forceinline__ std::uint32_t perm(std::uint32_t hi, std::uint32_t lo, std::uint32_t sel) {
     return __builtin_amdgcn_perm(hi, lo, sel);
 }
 
-// Quantize four consecutive activations held by this lane; the 8 lanes of a
-// 32-value group agree on one scale.  Returns the packed high and low planes.
-struct QuantizedQuad {
-    std::uint32_t hi;
-    std::uint32_t lo;
-    float scale;  // activation = scale * (256*hi + lo)
-    float sum;    // float sum of the 32 inputs of the group
-    int isum;     // sum over the group of (256*hi + lo), for formats with an offset code
-};
-
-__device__ __forceinline__ QuantizedQuad quantize_quad(float x0, float x1, float x2, float x3) {
-    QuantizedQuad q;
-    const float local = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
-    const float maximum = group8_max(local);
-    q.sum = group8_sum((x0 + x1) + (x2 + x3));
-    const float inverse = maximum > 0.0f ? kCodeRange / maximum : 0.0f;
-    q.scale = maximum * (1.0f / kCodeRange);
+// Quantize the 256 activations of one block, four per lane, and write the
+// record (planes, per-32 code sums, scale) to `record` (LDS or workspace).
+__device__ __forceinline__ void quantize_block(float4 x, int lane, std::uint8_t* record) {
+    const float local = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+    const float maximum = wave_max(local);
+    const float inverse = maximum > 1.0e-30f ? kCodeRange * __builtin_amdgcn_rcpf(maximum) : 0.0f;
+    const float scale = maximum * (1.0f / kCodeRange);
     // 1.5*2^23 + 128: the low 16 bits of the sum's bit pattern are
     // round-to-nearest-even(x*inverse) + 128 in two's complement.
     constexpr float kMagic = 12582912.0f + 128.0f;
-    const std::uint32_t u0 = __float_as_uint(fmaf(x0, inverse, kMagic));
-    const std::uint32_t u1 = __float_as_uint(fmaf(x1, inverse, kMagic));
-    const std::uint32_t u2 = __float_as_uint(fmaf(x2, inverse, kMagic));
-    const std::uint32_t u3 = __float_as_uint(fmaf(x3, inverse, kMagic));
-    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped.
+    const std::uint32_t u0 = __float_as_uint(fmaf(x.x, inverse, kMagic));
+    const std::uint32_t u1 = __float_as_uint(fmaf(x.y, inverse, kMagic));
+    const std::uint32_t u2 = __float_as_uint(fmaf(x.z, inverse, kMagic));
+    const std::uint32_t u3 = __float_as_uint(fmaf(x.w, inverse, kMagic));
+    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped
     const std::uint32_t p01 = perm(u1, u0, 0x05010400u);  // [u0.b0, u1.b0, u0.b1, u1.b1]
     const std::uint32_t p23 = perm(u3, u2, 0x05010400u);
-    q.lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
-    q.hi = perm(p23, p01, 0x07060302u);
-    q.isum = 0;
-    return q;
+    const std::uint32_t lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
+    const std::uint32_t hi = perm(p23, p01, 0x07060302u);
+    // sum of the four codes, then over the 8 lanes of the 32-value group
+    int sum = (__builtin_amdgcn_sdot4(static_cast<int>(hi), 0x01010101, 0, false) << 8) +
+        __builtin_amdgcn_sdot4(static_cast<int>(lo), 0x01010101, 0, false);
+    sum += dpp_move<kQuadXor1>(sum);
+    sum += dpp_move<kQuadXor2>(sum);
+    sum += dpp_move<kHalfMirror>(sum);
+    *reinterpret_cast<std::uint32_t*>(record + lane * 4) = hi;
+    *reinterpret_cast<std::uint32_t*>(record + 256 + lane * 4) = lo;
+    if ((lane & 7) == 0) {
+        *reinterpret_cast<int*>(record + kRecordSums + (lane >> 3) * 4) = sum;
+    }
+    if (lane == 0) {
+        *reinterpret_cast<float*>(record + kRecordScale) = scale;
+    }
 }
 
-struct TileContext {
-    Projection op;
-    std::int64_t row0;
-    int valid_rows;
-};
+template <int P>
+__device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
+                                                   const float* __restrict__ second,
+                                                   std::int64_t column) {
+    float4 x = *reinterpret_cast<const float4*>(first + column);
+    if constexpr (P != kPlain) {
+        const float4 y = *reinterpret_cast<const float4*>(second + column);
+        x.x = apply_prologue<P>(x.x, y.x);
+        x.y = apply_prologue<P>(x.y, y.y);
+        x.z = apply_prologue<P>(x.z, y.z);
+        x.w = apply_prologue<P>(x.w, y.w);
+    }
+    return x;
+}
 
-// Per-lane float scale factors of one super-block of this lane's weight row.
-template <std::uint32_t ENC>
-struct BlockScales;
-
-template <>
-struct BlockScales<kEncQ4K> {
-    float d, dmin;
-    float sc[8];
-    float mn[8];
-    __device__ __forceinline__ void load(const std::uint8_t* row) {
-        const uint4 h = *reinterpret_cast<const uint4*>(row);
-        d = half_bits_to_float(h.x & 0xffffu);
-        dmin = half_bits_to_float(h.x >> 16);
-        const std::uint32_t sc_lo = h.y & 0x3f3f3f3fu;
-        const std::uint32_t mn_lo = h.z & 0x3f3f3f3fu;
-        const std::uint32_t sc_hi = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
-        const std::uint32_t mn_hi = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sc[i] = static_cast<float>((sc_lo >> (8 * i)) & 0xffu);
-            mn[i] = static_cast<float>((mn_lo >> (8 * i)) & 0xffu);
-            sc[4 + i] = static_cast<float>((sc_hi >> (8 * i)) & 0xffu);
-            mn[4 + i] = static_cast<float>((mn_hi >> (8 * i)) & 0xffu);
+// Token <-> operand-row bookkeeping of v_mfma_i32_32x32x32_i8.  Output register
+// r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 of column l%32.
+//  Q4_K/Q5_K: a token takes two A rows (high, low plane).  Token t = 2u + h sits
+//    in registers 2u, 2u+1 of lane half h: up to 16 tokens, S = ceil(tokens/2)
+//    register pairs per lane.
+//  Q6_K: a 32-wide MFMA spans two 16-value groups with different sub-scales,
+//    so a token takes four A rows (high/low x first/second 16) and a lane
+//    feeds zeros where its k-half is not the row's: token t = 2q + h sits in
+//    registers 4q..4q+3 of lane half h: up to 8 tokens.
+template <bool Q6>
+struct OperandRow {
+    int token;
+    int plane;
+    bool keep;  // false: this lane's k-half is outside the row, feed zeros
+    __device__ __forceinline__ OperandRow(int i, int kc) {
+        if constexpr (Q6) {
+            const int row4 = i >> 2;
+            const int within = i & 3;
+            plane = within & 1;
+            keep = (within >> 1) == kc;
+            token = 2 * (row4 >> 1) + (row4 & 1);
+        } else {
+            const int pair = i >> 1;
+            plane = i & 1;
+            keep = true;
+            const int u = 2 * (pair >> 2) + (pair & 1);
+            const int h = (pair >> 1) & 1;
+            token = 2 * u + h;
         }
     }
 };
-template <>
-struct BlockScales<kEncQ5K> : BlockScales<kEncQ4K> {};
 
-__device__ __forceinline__ long pack_long(std::uint32_t lo, std::uint32_t hi) {
-    return static_cast<long>((static_cast<unsigned long>(hi) << 32) | lo);
-}
-
-// Where one lane finds the activation planes and scales of (token, super-block).
-struct ActSource {
-    const std::uint8_t* planes;  // hi plane at +0, lo plane at +256
-    const float* scales;         // 8 scales then 8 sums
+// Activation side of one super-block as one lane sees it.
+template <int S>
+struct BlockActivation {
+    const std::uint8_t* operand_base;  // record + plane offset of this lane's A row
+    bool keep;
+    int kc;
+    float scale[S];
+    int sums[S][8];
+    __device__ __forceinline__ v4i operand(int sub) const {
+        v4i v = *reinterpret_cast<const v4i*>(operand_base + sub * 32 + kc * 16);
+        if (!keep) v = v4i{0, 0, 0, 0};
+        return v;
+    }
 };
 
-// Process one super-block: 8 sub-block MFMAs and their float post-scaling.
-// `tile` is this wave's LDS copy of the 16 rows of the block.
-template <std::uint32_t ENC, int TPG, typename ActFn>
-__device__ __forceinline__ void process_block(const std::uint8_t* tile, int j, int kq,
-                                              ActFn&& activation, float (&acc)[TPG]);
+__device__ __forceinline__ int byte_of(std::uint32_t packed, int index) {
+    return static_cast<int>((packed >> (8 * index)) & 0xffu);
+}
+__device__ __forceinline__ int signed_byte_of(std::uint32_t packed, int index) {
+    return static_cast<int>(static_cast<std::int32_t>(packed << (24 - 8 * index)) >> 24);
+}
 
-template <int TPG, bool Q5, typename ActFn>
-__device__ __forceinline__ void process_block_q45(const std::uint8_t* tile, int j, int kq,
-                                                  ActFn&& activation, float (&acc)[TPG]) {
+__device__ __forceinline__ v16i mfma32(v4i a, v4i b) {
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
+}
+
+// ---- Q4_K / Q5_K ------------------------------------------------------------
+template <int S, bool Q5>
+__device__ __forceinline__ void process_block_q45(const std::uint8_t* tile, int j, int kc,
+                                                  const BlockActivation<S>& act,
+                                                  float (&acc)[S]) {
     constexpr int kRow = Q5 ? 176 : 144;
     const std::uint8_t* row = tile + j * kRow;
-    BlockScales<kEncQ4K> scales;
-    scales.load(row);
-    std::uint32_t high0 = 0, high1 = 0;
-    if constexpr (Q5) {
-        const uint2 h = *reinterpret_cast<const uint2*>(row + 16 + kq * 8);
-        high0 = h.x;
-        high1 = h.y;
-    }
-    const std::uint8_t* quants = row + (Q5 ? 48 : 16) + kq * 8;
-    float block_acc[TPG];
-    float block_min[TPG];
+    const uint4 h = *reinterpret_cast<const uint4*>(row);
+    v4i high = {0, 0, 0, 0};
+    if constexpr (Q5) high = *reinterpret_cast<const v4i*>(row + 16 + kc * 16);
+    const std::uint8_t* quants = row + (Q5 ? 48 : 16) + kc * 16;
+    // 6-bit scales and minimums of the eight sub-blocks, packed four per word
+    const std::uint32_t sc_lo = h.y & 0x3f3f3f3fu;
+    const std::uint32_t mn_lo = h.z & 0x3f3f3f3fu;
+    const std::uint32_t sc_hi = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
+    const std::uint32_t mn_hi = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u);
+    int acc_hi[S], acc_lo[S], acc_min[S];
 #pragma unroll
-    for (int u = 0; u < TPG; ++u) {
-        block_acc[u] = 0.0f;
-        block_min[u] = 0.0f;
+    for (int u = 0; u < S; ++u) {
+        acc_hi[u] = 0;
+        acc_lo[u] = 0;
+        acc_min[u] = 0;
     }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        const uint2 packed = *reinterpret_cast<const uint2*>(quants + g * 32);
-        std::uint32_t lo0 = packed.x & 0x0f0f0f0fu;
-        std::uint32_t lo1 = packed.y & 0x0f0f0f0fu;
-        std::uint32_t hi0 = (packed.x >> 4) & 0x0f0f0f0fu;
-        std::uint32_t hi1 = (packed.y >> 4) & 0x0f0f0f0fu;
-        if constexpr (Q5) {
-            // bit 2g of the high-bit byte belongs to sub-block 2g, bit 2g+1 to 2g+1
-            lo0 |= ((high0 >> (2 * g)) & 0x01010101u) << 4;
-            lo1 |= ((high1 >> (2 * g)) & 0x01010101u) << 4;
-            hi0 |= ((high0 >> (2 * g + 1)) & 0x01010101u) << 4;
-            hi1 |= ((high1 >> (2 * g + 1)) & 0x01010101u) << 4;
+        const v4i packed = *reinterpret_cast<const v4i*>(quants + g * 32);
+        v4i low, upper;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const std::uint32_t word = static_cast<std::uint32_t>(packed[w]);
+            std::uint32_t lo = word & 0x0f0f0f0fu;
+            std::uint32_t up = (word >> 4) & 0x0f0f0f0fu;
+            if constexpr (Q5) {
+                // bit 2g of the high-bit byte belongs to sub-block 2g, bit 2g+1 to 2g+1
+                const std::uint32_t bits = static_cast<std::uint32_t>(high[w]);
+                lo |= (g < 2 ? bits << (4 - 2 * g) : bits >> (2 * g - 4)) & 0x10101010u;
+                up |= (g < 2 ? bits << (3 - 2 * g) : bits >> (2 * g - 3)) & 0x10101010u;
+            }
+            low[w] = static_cast<int>(lo);
+            upper[w] = static_cast<int>(up);
         }
 #pragma unroll
         for (int part = 0; part < 2; ++part) {
             const int sub = 2 * g + part;
-            const long b = part == 0 ? pack_long(lo0, lo1) : pack_long(hi0, hi1);
-            const long a = activation.operand(sub);
-            v4i dot = {0, 0, 0, 0};
-            dot = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, dot, 0, 0, 0);
+            const v16i dot = mfma32(act.operand(sub), part == 0 ? low : upper);
+            const int sc = byte_of(sub < 4 ? sc_lo : sc_hi, sub & 3);
+            const int mn = byte_of(sub < 4 ? mn_lo : mn_hi, sub & 3);
 #pragma unroll
-            for (int u = 0; u < TPG; ++u) {
-                const int code = (dot[2 * u] << 8) + dot[2 * u + 1];
-                block_acc[u] = fmaf(static_cast<float>(code),
-                                    scales.sc[sub] * activation.scale(u, sub), block_acc[u]);
-                block_min[u] = fmaf(scales.mn[sub], activation.sum(u, sub), block_min[u]);
+            for (int u = 0; u < S; ++u) {
+                acc_hi[u] += __mul24(sc, dot[2 * u]);
+                acc_lo[u] += __mul24(sc, dot[2 * u + 1]);
+                acc_min[u] += __mul24(mn, act.sums[u][sub]);
             }
         }
     }
+    const float d = half_bits_to_float(h.x & 0xffffu);
+    const float dmin = half_bits_to_float(h.x >> 16);
 #pragma unroll
-    for (int u = 0; u < TPG; ++u) {
-        acc[u] = fmaf(scales.d, block_acc[u], acc[u]);
-        acc[u] = fmaf(-scales.dmin, block_min[u], acc[u]);
+    for (int u = 0; u < S; ++u) {
+        const float codes = fmaf(static_cast<float>(acc_hi[u]), 256.0f, static_cast<float>(acc_lo[u]));
+        const float value = fmaf(-dmin, static_cast<float>(acc_min[u]), d * codes);
+        acc[u] = fmaf(act.scale[u], value, acc[u]);
     }
 }
 
-// Activations quantized by this wave into its own LDS record (one token).
-struct FusedActivation {
-    const std::uint8_t* record;  // LDS: hi[256] lo[256] scale[8] sum[8]
-    int plane_offset;            // which plane this lane feeds to the A operand
-    int kq;
-    float scales[8];
-    float sums[8];
-    __device__ __forceinline__ void load_scalars() {
-        const float4* p = reinterpret_cast<const float4*>(record + 512);
-        const float4 a = p[0], b = p[1], c = p[2], d = p[3];
-        scales[0] = a.x; scales[1] = a.y; scales[2] = a.z; scales[3] = a.w;
-        scales[4] = b.x; scales[5] = b.y; scales[6] = b.z; scales[7] = b.w;
-        sums[0] = c.x; sums[1] = c.y; sums[2] = c.z; sums[3] = c.w;
-        sums[4] = d.x; sums[5] = d.y; sums[6] = d.z; sums[7] = d.w;
-    }
-    __device__ __forceinline__ long operand(int sub) const {
-        const uint2 v = *reinterpret_cast<const uint2*>(record + plane_offset + sub * 32 + kq * 8);
-        return pack_long(v.x, v.y);
-    }
-    __device__ __forceinline__ float scale(int, int sub) const { return scales[sub]; }
-    __device__ __forceinline__ float sum(int, int sub) const { return sums[sub]; }
-};
-
-// Activations quantized earlier into the workspace (2..8 tokens per pass).
-template <int TPG>
-struct WorkspaceActivation {
-    const std::uint8_t* operand_base;  // this lane's plane of its A row, or a valid dummy
-    int kq;
-    float scales[TPG][8];
-    float sums[TPG][8];
-    __device__ __forceinline__ void load_scalars(const std::uint8_t* const (&records)[TPG]) {
+// ---- Q6_K ---------------------------------------------------------------------
+template <int S>
+__device__ __forceinline__ void process_block_q6(const std::uint8_t* tile, int j, int kc,
+                                                 const BlockActivation<S>& act, float (&acc)[S]) {
+    const std::uint8_t* row = tile + j * 240;
+    const uint4 sc = *reinterpret_cast<const uint4*>(row + 192);
+    const std::uint32_t scales[4] = {sc.x, sc.y, sc.z, sc.w};
+    int acc_hi[S], acc_lo[S];
 #pragma unroll
-        for (int u = 0; u < TPG; ++u) {
-            const float4* p = reinterpret_cast<const float4*>(records[u] + 512);
-            const float4 a = p[0], b = p[1], c = p[2], d = p[3];
-            scales[u][0] = a.x; scales[u][1] = a.y; scales[u][2] = a.z; scales[u][3] = a.w;
-            scales[u][4] = b.x; scales[u][5] = b.y; scales[u][6] = b.z; scales[u][7] = b.w;
-            sums[u][0] = c.x; sums[u][1] = c.y; sums[u][2] = c.z; sums[u][3] = c.w;
-            sums[u][4] = d.x; sums[u][5] = d.y; sums[u][6] = d.z; sums[u][7] = d.w;
+    for (int u = 0; u < S; ++u) {
+        acc_hi[u] = 0;
+        acc_lo[u] = 0;
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const v4i ql_a = *reinterpret_cast<const v4i*>(row + half * 64 + kc * 16);
+        const v4i ql_b = *reinterpret_cast<const v4i*>(row + half * 64 + 32 + kc * 16);
+        const v4i qh = *reinterpret_cast<const v4i*>(row + 128 + half * 32 + kc * 16);
+#pragma unroll
+        for (int quarter = 0; quarter < 4; ++quarter) {
+            v4i q;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const std::uint32_t ql = static_cast<std::uint32_t>((quarter & 1) ? ql_b[w] : ql_a[w]);
+                const std::uint32_t nib = (quarter < 2 ? ql : ql >> 4) & 0x0f0f0f0fu;
+                const std::uint32_t bits = static_cast<std::uint32_t>(qh[w]);
+                // bits 2q, 2q+1 of the high byte move to bits 4, 5
+                const std::uint32_t top =
+                    (quarter < 2 ? bits << (4 - 2 * quarter) : bits >> (2 * quarter - 4)) & 0x30303030u;
+                // q - 32 as signed bytes with no borrow between bytes:
+                // ((q | 0x80) - 0x20) ^ 0x80
+                q[w] = static_cast<int>(((nib | top | 0x80808080u) - 0x20202020u) ^ 0x80808080u);
+            }
+            const int sub = half * 4 + quarter;
+            const v16i dot = mfma32(act.operand(sub), q);
+            // a lane's k-half is one 16-value group: rows of the first group
+            // carry zeros in k-half 1 and the other way round
+            const int s0 = signed_byte_of(scales[sub >> 1], (2 * sub) & 3);
+            const int s1 = signed_byte_of(scales[sub >> 1], (2 * sub + 1) & 3);
+#pragma unroll
+            for (int u = 0; u < S; ++u) {
+                acc_hi[u] += __mul24(s0, dot[4 * u]) + __mul24(s1, dot[4 * u + 2]);
+                acc_lo[u] += __mul24(s0, dot[4 * u + 1]) + __mul24(s1, dot[4 * u + 3]);
+            }
         }
     }
-    __device__ __forceinline__ long operand(int sub) const {
-        const uint2 v = *reinterpret_cast<const uint2*>(operand_base + sub * 32 + kq * 8);
-        return pack_long(v.x, v.y);
-    }
-    __device__ __forceinline__ float scale(int u, int sub) const { return scales[u][sub]; }
-    __device__ __forceinline__ float sum(int u, int sub) const { return sums[u][sub]; }
-};
-
-template <std::uint32_t ENC, int TPG, typename Act>
-__device__ __forceinline__ void dispatch_block(const std::uint8_t* tile, int j, int kq, Act& act,
-                                               float (&acc)[TPG]) {
-    if constexpr (ENC == kEncQ4K) {
-        process_block_q45<TPG, false>(tile, j, kq, act, acc);
-    } else if constexpr (ENC == kEncQ5K) {
-        process_block_q45<TPG, true>(tile, j, kq, act, acc);
+    const float d = half_bits_to_float(*reinterpret_cast<const std::uint16_t*>(row + 208));
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+        const float codes = fmaf(static_cast<float>(acc_hi[u]), 256.0f, static_cast<float>(acc_lo[u]));
+        acc[u] = fmaf(act.scale[u], d * codes, acc[u]);
     }
 }
 
@@ -314,201 +350,302 @@ __device__ __forceinline__ uint4 load_chunk(const std::uint8_t* p) {
     }
 }
 
-// The whole K loop of one wave for one tile.
-template <std::uint32_t ENC, int TPG, bool FUSED, int P, int DEPTH>
-__device__ __forceinline__ void run_tile(const TileContext& ctx, std::int64_t input_dim,
-                                         const float* __restrict__ first,
-                                         const float* __restrict__ second,
-                                         const std::uint8_t* __restrict__ workspace,
-                                         int tokens, std::uint8_t* wave_tile,
-                                         std::uint8_t* wave_record, int lane, int wave,
-                                         float (&acc)[TPG]) {
+__device__ __forceinline__ void wave_lds_fence() {
+    // LDS traffic of one wave is in order; this only pins the compiler.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Where the chunks a lane copies for one tile come from and go to.
+template <std::uint32_t ENC>
+struct TileSource {
     using F = Format<ENC>;
-    constexpr int kTotalChunks = kTileRows * F::kChunks;
-    constexpr int kLoads = (kTotalChunks + kWave - 1) / kWave;
-    const int j = lane & 15;
-    const int kq = lane >> 4;
-    const std::int64_t blocks = input_dim >> 8;
-    const std::int64_t begin = blocks * wave / kWaves;
-    const std::int64_t end = blocks * (wave + 1) / kWaves;
+    static constexpr int kTotalChunks = kTileRows * F::kChunks;
+    static constexpr int kLoads = (kTotalChunks + kWave - 1) / kWave;
+    const std::uint8_t* base;      // first byte of the tile's first row (uniform)
+    const std::uint8_t* data_end;  // end of the tensor (uniform)
+    std::uint32_t offset[kLoads];  // byte offset of this lane's chunk i from base
+    float* output;
+    std::int64_t output_dim;
+    std::int64_t row0;
+    int valid_rows;
 
-    // Per-lane source pointers and LDS offsets of the chunks this lane copies.
-    const std::uint8_t* source[kLoads];
-    int target[kLoads];
-    const std::uint8_t* data_end = ctx.op.data + ctx.op.output_dim * ctx.op.row_stride;
+    __device__ __forceinline__ void setup(const ProjectionSet& set, std::uint32_t tile, int lane) {
+        int which = 0;
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-        const int chunk = i * kWave + lane;
-        const int row = chunk / F::kChunks;
-        const int col = chunk - row * F::kChunks;
-        const int clamped = min(row, ctx.valid_rows - 1);
-        source[i] = ctx.op.data + (ctx.row0 + clamped) * ctx.op.row_stride + col * 16;
-        target[i] = row * F::kLdsRow + col * 16;
-    }
-    (void)data_end;
-
-    uint4 staged[DEPTH][kLoads];
-    auto fetch = [&](int slot, std::int64_t block) {
+        for (int index = 1; index < 4; ++index) {
+            if (index < set.count && tile >= set.op[index].first_tile) which = index;
+        }
+        const Projection& op = set.op[which];
+        row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
+        valid_rows = static_cast<int>(min(static_cast<std::int64_t>(kTileRows), op.output_dim - row0));
+        base = op.data + row0 * op.row_stride;
+        data_end = op.data + op.output_dim * op.row_stride;
+        output = op.output;
+        output_dim = op.output_dim;
+        const std::uint32_t stride = static_cast<std::uint32_t>(op.row_stride);
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
-            if (i * kWave + lane < kTotalChunks) {
-                const std::uint8_t* p = source[i] + block * F::kBlockBytes;
-                if constexpr (!F::kAligned) {
-                    // the last chunk of a block reads past it; keep it inside the tensor
-                    p = p + 16 <= data_end ? p : data_end - 16;
-                }
-                staged[slot][i] = load_chunk<ENC>(p);
-            }
+            // lanes past the last chunk repeat it: same bytes to the same LDS
+            // address, and no lane-masked load to blur the load counters
+            const int chunk = min(i * kWave + lane, kTotalChunks - 1);
+            const int row = chunk / F::kChunks;
+            const int col = chunk - row * F::kChunks;
+            offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) * stride + col * 16;
         }
-    };
-
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-        if (begin + d < end) fetch(d, begin + d);
     }
+};
 
-    // Which activation plane this lane supplies as a row of the A operand.
-    const int a_group = j >> 2;          // which lane group's tokens
-    const int a_slot = (j & 3) >> 1;     // token slot within the group
-    const int a_term = j & 1;            // 0: high plane, 1: low plane
-    const int a_token = a_group * TPG + (a_slot < TPG ? a_slot : 0);
-    const bool a_valid = a_slot < TPG && a_token < tokens;
-
-    for (std::int64_t base = begin; base < end; base += DEPTH) {
+template <std::uint32_t ENC>
+__device__ __forceinline__ void fetch_block(const TileSource<ENC>& src, std::int64_t block,
+                                            int lane, uint4 (&staged)[TileSource<ENC>::kLoads]) {
+    using F = Format<ENC>;
+    const std::uint8_t* block_base = src.base + block * F::kBlockBytes;
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const std::int64_t block = base + d;
-            if (block < end) {
-                // (1) staged weights -> private LDS tile
-#pragma unroll
-                for (int i = 0; i < kLoads; ++i) {
-                    if (i * kWave + lane < kTotalChunks) {
-                        *reinterpret_cast<uint4*>(wave_tile + target[i]) = staged[d][i];
-                    }
-                }
-                if (block + DEPTH < end) fetch(d, block + DEPTH);
-
-                if constexpr (FUSED) {
-                    // (2) quantize this block's 256 activations of the one token
-                    const std::int64_t column = block * 256 + lane * 4;
-                    float4 x = *reinterpret_cast<const float4*>(first + column);
-                    if constexpr (P != kPlain) {
-                        const float4 y = *reinterpret_cast<const float4*>(second + column);
-                        x.x = apply_prologue<P>(x.x, y.x);
-                        x.y = apply_prologue<P>(x.y, y.y);
-                        x.z = apply_prologue<P>(x.z, y.z);
-                        x.w = apply_prologue<P>(x.w, y.w);
-                    }
-                    const QuantizedQuad q = quantize_quad(x.x, x.y, x.z, x.w);
-                    *reinterpret_cast<std::uint32_t*>(wave_record + lane * 4) = q.hi;
-                    *reinterpret_cast<std::uint32_t*>(wave_record + 256 + lane * 4) = q.lo;
-                    if ((lane & 7) == 0) {
-                        *reinterpret_cast<float*>(wave_record + 512 + (lane >> 3) * 4) = q.scale;
-                        *reinterpret_cast<float*>(wave_record + 544 + (lane >> 3) * 4) = q.sum;
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                    FusedActivation act;
-                    act.record = wave_record;
-                    act.plane_offset = a_term * 256;
-                    act.kq = kq;
-                    act.load_scalars();
-                    dispatch_block<ENC, TPG>(wave_tile, j, kq, act, acc);
-                } else {
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                    WorkspaceActivation<TPG> act;
-                    const std::uint8_t* records[TPG];
-#pragma unroll
-                    for (int u = 0; u < TPG; ++u) {
-                        const int token = min(kq * TPG + u, tokens - 1);
-                        records[u] = workspace + (token * blocks + block) * kActRecord;
-                    }
-                    const int token = a_valid ? a_token : 0;
-                    act.operand_base =
-                        workspace + (token * blocks + block) * kActRecord + a_term * 256;
-                    act.kq = kq;
-                    act.load_scalars(records);
-                    dispatch_block<ENC, TPG>(wave_tile, j, kq, act, acc);
-                }
-                // the next block's LDS writes must not pass this block's reads
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-            }
+    for (int i = 0; i < TileSource<ENC>::kLoads; ++i) {
+        const std::uint8_t* p = block_base + src.offset[i];
+        if constexpr (F::kAligned) {
+            staged[i] = load_chunk<ENC>(p);
+        } else {
+            // The last chunk of a block reads 14 bytes past it; only its first
+            // two bytes (the block's d) are used.  At the very end of the
+            // tensor read the 16 bytes before the end instead and move those
+            // two bytes into place.
+            const bool past = p + 16 > src.data_end;
+            uint4 v = load_chunk<ENC>(past ? src.data_end - 16 : p);
+            if (past) v.x = v.w >> 16;
+            staged[i] = v;
         }
     }
 }
 
-template <int TPG, bool FUSED, int P, int DEPTH>
+template <std::uint32_t ENC>
+__device__ __forceinline__ void store_block(const uint4 (&staged)[TileSource<ENC>::kLoads],
+                                            int lane, std::uint8_t* wave_tile) {
+    using F = Format<ENC>;
+#pragma unroll
+    for (int i = 0; i < TileSource<ENC>::kLoads; ++i) {
+        const int chunk = min(i * kWave + lane, TileSource<ENC>::kTotalChunks - 1);
+        const int row = chunk / F::kChunks;
+        const int col = chunk - row * F::kChunks;
+        *reinterpret_cast<uint4*>(wave_tile + row * F::kLdsRow + col * 16) = staged[i];
+    }
+}
+
+template <std::uint32_t ENC, int S, bool FUSED, int P>
 __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    const std::uint8_t* __restrict__ workspace, int tokens, int token_stride_tiles) {
-    __shared__ __attribute__((aligned(16))) std::uint8_t tiles[kWaves][kMaxLdsTile];
-    __shared__ __attribute__((aligned(16))) std::uint8_t records[kWaves][640];
-    __shared__ float partial[kWaves][kWave][TPG];
+    const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
+    int pass_capacity) {
+    using F = Format<ENC>;
+    using Source = TileSource<ENC>;
+    constexpr bool kQ6 = ENC == kEncQ6K;
+    constexpr int kDepth = F::kDepth;
+    constexpr int kTileBytes = kTileRows * F::kLdsRow;
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const std::uint32_t tile_index = blockIdx.x;
-    int which = 0;
-#pragma unroll
-    for (int index = 1; index < 4; ++index) {
-        if (index < set.count && tile_index >= set.op[index].first_tile) which = index;
-    }
-    TileContext ctx;
-    ctx.op = set.op[which];
-    ctx.row0 = static_cast<std::int64_t>(tile_index - ctx.op.first_tile) * kTileRows;
-    ctx.valid_rows =
-        static_cast<int>(min(static_cast<std::int64_t>(kTileRows), ctx.op.output_dim - ctx.row0));
-
-    // Passes over the tokens when there are more than one pass can hold.
-    const int token0 = blockIdx.y * 4 * TPG;
-    const int pass_tokens = min(tokens - token0, 4 * TPG);
+    // the wave index is uniform; saying so keeps tile bookkeeping in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31;
+    const int kc = lane >> 5;
     const std::int64_t blocks = set.input_dim >> 8;
+    const std::int64_t begin = blocks * wave / kWaves;
+    const std::int64_t end = blocks * (wave + 1) / kWaves;
+    const int count = static_cast<int>(end - begin);
+    const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
+
+    // LDS: [waves][tile] | [2][waves][lanes][S] partial sums | [waves][max_count] records
+    std::uint8_t* wave_tile = lds + wave * kTileBytes;
+    float* partial = reinterpret_cast<float*>(lds + kWaves * kTileBytes);
+    std::uint8_t* wave_records =
+        lds + kWaves * kTileBytes + 2 * kWaves * kWave * S * 4 + wave * max_count * kActRecord;
+
+    const int token0 = blockIdx.y * pass_capacity;
+    const int pass_tokens = min(tokens - token0, pass_capacity);
     const std::uint8_t* pass_workspace =
         FUSED ? nullptr : workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord;
-    const float* pass_first = first;
-    const float* pass_second = second;
 
-    float acc[TPG];
-#pragma unroll
-    for (int u = 0; u < TPG; ++u) acc[u] = 0.0f;
+    const std::uint32_t first_tile = blockIdx.x;
 
-    switch (ctx.op.encoding) {
-        case kEncQ4K:
-            run_tile<kEncQ4K, TPG, FUSED, P, DEPTH>(ctx, set.input_dim, pass_first, pass_second,
-                                                   pass_workspace, pass_tokens, tiles[wave],
-                                                   records[wave], lane, wave, acc);
-            break;
-        case kEncQ5K:
-            run_tile<kEncQ5K, TPG, FUSED, P, DEPTH>(ctx, set.input_dim, pass_first, pass_second,
-                                                   pass_workspace, pass_tokens, tiles[wave],
-                                                   records[wave], lane, wave, acc);
-            break;
-        default:
-            break;
-    }
-
+    // Every load below is unconditional (indices are clamped instead): with a
+    // fixed number of loads in flight the waits the compiler inserts are exact,
+    // so the quantizer only waits for the activations and a block only for its
+    // own chunks.
+    float4 x[FUSED ? kEarlyBlocks : 1];
+    if constexpr (FUSED) {
+        // activations first: their (short) latency must not queue behind the weights
 #pragma unroll
-    for (int u = 0; u < TPG; ++u) partial[wave][lane][u] = acc[u];
-    __syncthreads();
-    if (wave == 0) {
-        const int j = lane & 15;
-        const int kq = lane >> 4;
-#pragma unroll
-        for (int u = 0; u < TPG; ++u) {
-            const int token = kq * TPG + u;
-            const float total = ((partial[0][lane][u] + partial[1][lane][u]) +
-                                 partial[2][lane][u]) + partial[3][lane][u];
-            if (token < pass_tokens && j < ctx.valid_rows) {
-                ctx.op.output[static_cast<std::int64_t>(token0 + token) * ctx.op.output_dim +
-                              ctx.row0 + j] = total;
-            }
+        for (int b = 0; b < kEarlyBlocks; ++b) {
+            const int clamped = max(min(b, count - 1), 0);
+            x[b] = load_activations<P>(first, second, (begin + clamped) * 256 + lane * 4);
         }
     }
-    (void)token_stride_tiles;
+
+    // Flat stream of (tile, block) pairs this wave processes; the prefetch
+    // cursor runs kDepth pairs ahead of the processing cursor and stays on the
+    // last pair once the stream is exhausted.
+    Source fetch_source;
+    std::uint32_t fetch_tile = first_tile;
+    int fetch_index = 0;
+    fetch_source.setup(set, fetch_tile, lane);
+    uint4 staged[kDepth][Source::kLoads];
+    auto advance_fetch = [&]() {
+        if (fetch_index + 1 < count) {
+            ++fetch_index;
+        } else if (fetch_tile + gridDim.x < total_tiles) {
+            fetch_index = 0;
+            fetch_tile += gridDim.x;
+            fetch_source.setup(set, fetch_tile, lane);
+        } else {
+            // stream exhausted: the remaining (never used) fetches all hit one line
+#pragma unroll
+            for (int i = 0; i < Source::kLoads; ++i) fetch_source.offset[i] = 0;
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+        fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[d]);
+        advance_fetch();
+    }
+
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int b = 0; b < kEarlyBlocks; ++b) {
+#ifndef NFN_EXP_SKIP_QUANT
+            if (b < count) quantize_block(x[b], lane, wave_records + b * kActRecord);
+#endif
+        }
+        // more than kEarlyBlocks blocks per wave: quantize the rest now
+        for (int b = kEarlyBlocks; b < count; ++b) {
+            const float4 v = load_activations<P>(first, second, (begin + b) * 256 + lane * 4);
+            quantize_block(v, lane, wave_records + b * kActRecord);
+        }
+        wave_lds_fence();
+    }
+
+    // Which A row this lane supplies.
+    const OperandRow<kQ6> a_row(j, kc);
+    const bool a_valid = a_row.token < pass_tokens && a_row.token < 2 * S;
+
+    Source source;
+    int parity = 0;
+    int slot_base = 0;  // staging slot of the tile's first block, modulo kDepth
+    for (std::uint32_t tile = first_tile; tile < total_tiles; tile += gridDim.x) {
+        source.setup(set, tile, lane);
+        float acc[S];
+#pragma unroll
+        for (int u = 0; u < S; ++u) acc[u] = 0.0f;
+
+        for (int b = 0; b < count; ++b) {
+            {
+                {
+                    // staging slots rotate with the flat pair index
+                    const int slot = (slot_base + b) % kDepth;
+                    auto rotate = [&](auto slot_constant) {
+                        constexpr int kSlot = decltype(slot_constant)::value;
+#ifndef NFN_EXP_SKIP_STORE
+                        store_block<ENC>(staged[kSlot], lane, wave_tile);
+#else
+                        {
+                            std::uint32_t mix = 0;
+                            for (int i = 0; i < Source::kLoads; ++i) {
+                                mix ^= staged[kSlot][i].x ^ staged[kSlot][i].y ^ staged[kSlot][i].z ^ staged[kSlot][i].w;
+                            }
+                            if (mix == 0x12345u) wave_tile[lane] = 1;
+                        }
+#endif
+                        fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[kSlot]);
+                        advance_fetch();
+                    };
+                    if (slot == 0) {
+                        rotate(std::integral_constant<int, 0>{});
+                    } else if (slot == 1) {
+                        rotate(std::integral_constant<int, 1>{});
+                    } else if (slot == 2 || kDepth == 3) {
+                        rotate(std::integral_constant<int, 2>{});
+                    } else {
+                        rotate(std::integral_constant<int, kDepth - 1>{});
+                    }
+                    wave_lds_fence();
+
+                    BlockActivation<S> act;
+                    act.kc = kc;
+                    act.keep = a_row.keep;
+                    const std::int64_t block = begin + b;
+                    if constexpr (FUSED) {
+                        const std::uint8_t* record = wave_records + b * kActRecord;
+                        act.operand_base = record + a_row.plane * 256;
+                        act.scale[0] = *reinterpret_cast<const float*>(record + kRecordScale);
+                        if constexpr (!kQ6) {
+                            const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
+                            const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
+                            act.sums[0][0] = s0.x; act.sums[0][1] = s0.y;
+                            act.sums[0][2] = s0.z; act.sums[0][3] = s0.w;
+                            act.sums[0][4] = s1.x; act.sums[0][5] = s1.y;
+                            act.sums[0][6] = s1.z; act.sums[0][7] = s1.w;
+                        }
+                    } else {
+                        const int operand_token = a_valid ? a_row.token : 0;
+                        act.operand_base = pass_workspace +
+                            (operand_token * blocks + block) * kActRecord + a_row.plane * 256;
+#pragma unroll
+                        for (int u = 0; u < S; ++u) {
+                            const int token = min(2 * u + kc, pass_tokens - 1);
+                            const std::uint8_t* record =
+                                pass_workspace + (token * blocks + block) * kActRecord;
+                            act.scale[u] = *reinterpret_cast<const float*>(record + kRecordScale);
+                            if constexpr (!kQ6) {
+                                const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
+                                const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
+                                act.sums[u][0] = s0.x; act.sums[u][1] = s0.y;
+                                act.sums[u][2] = s0.z; act.sums[u][3] = s0.w;
+                                act.sums[u][4] = s1.x; act.sums[u][5] = s1.y;
+                                act.sums[u][6] = s1.z; act.sums[u][7] = s1.w;
+                            }
+                        }
+                    }
+#ifdef NFN_EXP_SKIP_COMPUTE
+                    acc[0] += act.scale[0] + static_cast<float>(wave_tile[lane * 36]);
+#else
+                    if constexpr (ENC == kEncQ4K) {
+                        process_block_q45<S, false>(wave_tile, j, kc, act, acc);
+                    } else if constexpr (ENC == kEncQ5K) {
+                        process_block_q45<S, true>(wave_tile, j, kc, act, acc);
+                    } else {
+                        process_block_q6<S>(wave_tile, j, kc, act, acc);
+                    }
+#endif
+                    wave_lds_fence();  // the next block's stores stay behind these reads
+                }
+            }
+        }
+        slot_base = (slot_base + count) % kDepth;
+
+        // Cross-wave sum in a fixed order; the two buffers alternate so one
+        // barrier per tile is enough.
+        float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * S;
+#pragma unroll
+        for (int u = 0; u < S; ++u) mine[u] = acc[u];
+        __syncthreads();
+        if (wave == (parity ? kWaves - 1 : 0)) {
+#pragma unroll
+            for (int u = 0; u < S; ++u) {
+                const int token = 2 * u + kc;
+                float total = partial[((parity * kWaves + 0) * kWave + lane) * S + u];
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w) {
+                    total += partial[((parity * kWaves + w) * kWave + lane) * S + u];
+                }
+                if (token < pass_tokens && j < source.valid_rows) {
+                    source.output[static_cast<std::int64_t>(token0 + token) * source.output_dim +
+                                  source.row0 + j] = total;
+                }
+            }
+        }
+        parity ^= 1;
+    }
 }
 
 // ---- activation quantizer for the multi-token passes -----------------------
@@ -521,84 +658,132 @@ __global__ __launch_bounds__(256) void quantize_activations_kernel(
     const int lane = threadIdx.x & 63;
     const std::int64_t record = static_cast<std::int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (record >= total_blocks) return;
-    const std::int64_t column = record * 256 + lane * 4;
-    float4 x = *reinterpret_cast<const float4*>(first + column);
-    if constexpr (P != kPlain) {
-        const float4 y = *reinterpret_cast<const float4*>(second + column);
-        x.x = apply_prologue<P>(x.x, y.x);
-        x.y = apply_prologue<P>(x.y, y.y);
-        x.z = apply_prologue<P>(x.z, y.z);
-        x.w = apply_prologue<P>(x.w, y.w);
-    }
-    const QuantizedQuad q = quantize_quad(x.x, x.y, x.z, x.w);
-    std::uint8_t* out = workspace + record * kActRecord;
-    *reinterpret_cast<std::uint32_t*>(out + lane * 4) = q.hi;
-    *reinterpret_cast<std::uint32_t*>(out + 256 + lane * 4) = q.lo;
-    if ((lane & 7) == 0) {
-        *reinterpret_cast<float*>(out + 512 + (lane >> 3) * 4) = q.scale;
-        *reinterpret_cast<float*>(out + 544 + (lane >> 3) * 4) = q.sum;
-    }
+    const float4 x = load_activations<P>(first, second, record * 256 + lane * 4);
+    quantize_block(x, lane, workspace + record * kActRecord);
 }
 
-template <int TPG, bool FUSED, int P>
-void launch_variant(const ProjectionSet& set, const float* first, const float* second,
-                    const std::uint8_t* workspace, int tokens, std::uint32_t tiles, int passes,
+int compute_units() {
+    static const int count = [] {
+        int device = 0;
+        int value = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            value <= 0) {
+            return 256;
+        }
+        return value;
+    }();
+    return count;
+}
+
+template <std::uint32_t ENC, int S, bool FUSED, int P>
+void launch_variant(ProjectionSet set, const float* first, const float* second,
+                    const std::uint8_t* workspace, int tokens, int pass_capacity,
                     hipStream_t stream) {
-    hipLaunchKernelGGL((gemv_mfma_kernel<TPG, FUSED, P, 4>), dim3(tiles, passes), dim3(kThreads),
-                       0, stream, set, first, second, workspace, tokens, 0);
-}
-
-}  // namespace
-
-bool gemv_mfma_supports(std::uint32_t encoding) {
-    return encoding == kEncQ4K || encoding == kEncQ5K;
-}
-
-void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second, int prologue,
-                      std::int64_t rows, void* workspace, hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
-    const int tokens = static_cast<int>(rows);
+    const std::int64_t blocks = set.input_dim >> 8;
+    const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
+    const std::size_t lds = static_cast<std::size_t>(kWaves) * kTileRows * Format<ENC>::kLdsRow +
+        2u * kWaves * kWave * S * 4 +
+        (FUSED ? static_cast<std::size_t>(kWaves) * max_count * kActRecord : 0);
+    auto kernel = gemv_mfma_kernel<ENC, S, FUSED, P>;
+    // More than 64 KB of dynamic LDS has to be allowed once per kernel.
+    static const bool raised =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+    (void)raised;
+    const int passes = (tokens + pass_capacity - 1) / pass_capacity;
+    // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
+    const std::uint32_t grid = tiles < static_cast<std::uint32_t>(compute_units())
+        ? tiles : static_cast<std::uint32_t>(compute_units());
+    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, stream, set, first, second,
+                       workspace, tokens, tiles, pass_capacity);
+}
+
+template <std::uint32_t ENC>
+void launch_encoding(const ProjectionSet& set, const float* first, const float* second,
+                     int prologue, const std::uint8_t* workspace, int tokens,
+                     hipStream_t stream) {
+    constexpr bool kQ6 = ENC == kEncQ6K;
     if (tokens == 1) {
         switch (prologue) {
             case kGated:
-                launch_variant<1, true, kGated>(set, first, second, nullptr, 1, tiles, 1, stream);
+                launch_variant<ENC, 1, true, kGated>(set, first, second, nullptr, 1, 2, stream);
                 break;
             case kSwiGlu:
-                launch_variant<1, true, kSwiGlu>(set, first, second, nullptr, 1, tiles, 1, stream);
+                launch_variant<ENC, 1, true, kSwiGlu>(set, first, second, nullptr, 1, 2, stream);
                 break;
             default:
-                launch_variant<1, true, kPlain>(set, first, second, nullptr, 1, tiles, 1, stream);
+                launch_variant<ENC, 1, true, kPlain>(set, first, second, nullptr, 1, 2, stream);
                 break;
         }
         return;
     }
-    // 2..16 tokens: quantize once into the workspace, then one or two passes.
-    const std::int64_t records = rows * (set.input_dim >> 8);
-    const dim3 grid(static_cast<unsigned>((records + 3) / 4));
-    std::uint8_t* ws = static_cast<std::uint8_t*>(workspace);
-    switch (prologue) {
-        case kGated:
-            hipLaunchKernelGGL((quantize_activations_kernel<kGated>), grid, dim3(256), 0, stream,
-                               first, second, ws, records);
-            break;
-        case kSwiGlu:
-            hipLaunchKernelGGL((quantize_activations_kernel<kSwiGlu>), grid, dim3(256), 0, stream,
-                               first, second, ws, records);
-            break;
-        default:
-            hipLaunchKernelGGL((quantize_activations_kernel<kPlain>), grid, dim3(256), 0, stream,
-                               first, second, ws, records);
-            break;
-    }
-    if (tokens <= 4) {
-        launch_variant<1, false, kPlain>(set, nullptr, nullptr, ws, tokens, tiles, 1, stream);
+    if (tokens <= 2) {
+        launch_variant<ENC, 1, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 2, stream);
+    } else if (tokens <= 4) {
+        launch_variant<ENC, 2, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 4, stream);
+    } else if (tokens <= 8 || kQ6) {
+        launch_variant<ENC, 4, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 8, stream);
     } else {
-        launch_variant<2, false, kPlain>(set, nullptr, nullptr, ws, tokens, tiles,
-                                         (tokens + 7) / 8, stream);
+        if constexpr (!kQ6) {
+            launch_variant<ENC, 8, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 16,
+                                                 stream);
+        }
+    }
+}
+
+}  // namespace
+
+bool gemv_mfma_supports(std::uint32_t encoding, std::int64_t input_dim) {
+    // the activation records of one wave's K range stay in LDS
+    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
+        input_dim % 256 == 0 && input_dim <= 65536;
+}
+
+void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second, int prologue,
+                      std::int64_t rows, void* workspace, hipStream_t stream) {
+    const int tokens = static_cast<int>(rows);
+    std::uint8_t* ws = static_cast<std::uint8_t*>(workspace);
+    if (tokens > 1) {
+        // 2..16 tokens: quantize once into the workspace
+        const std::int64_t records = rows * (set.input_dim >> 8);
+        const dim3 grid(static_cast<unsigned>((records + 3) / 4));
+        switch (prologue) {
+            case kGated:
+                hipLaunchKernelGGL((quantize_activations_kernel<kGated>), grid, dim3(256), 0,
+                                   stream, first, second, ws, records);
+                break;
+            case kSwiGlu:
+                hipLaunchKernelGGL((quantize_activations_kernel<kSwiGlu>), grid, dim3(256), 0,
+                                   stream, first, second, ws, records);
+                break;
+            default:
+                hipLaunchKernelGGL((quantize_activations_kernel<kPlain>), grid, dim3(256), 0,
+                                   stream, first, second, ws, records);
+                break;
+        }
+    }
+    // one launch per encoding present
+    const std::uint32_t encodings[3] = {kEncQ4K, kEncQ5K, kEncQ6K};
+    for (const std::uint32_t encoding : encodings) {
+        ProjectionSet group{};
+        group.input_dim = set.input_dim;
+        for (int index = 0; index < set.count; ++index) {
+            if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
+        }
+        if (group.count == 0) continue;
+        if (encoding == kEncQ4K) {
+            launch_encoding<kEncQ4K>(group, first, second, prologue, ws, tokens, stream);
+        } else if (encoding == kEncQ5K) {
+            launch_encoding<kEncQ5K>(group, first, second, prologue, ws, tokens, stream);
+        } else {
+            launch_encoding<kEncQ6K>(group, first, second, prologue, ws, tokens, stream);
+        }
     }
 }
 

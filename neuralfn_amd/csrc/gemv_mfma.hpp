@@ -9,8 +9,8 @@ namespace nfn {
 // [256], 8 float scales, 8 float sums.
 constexpr int kActivationRecordBytes = 576;
 
-// True when every projection of the set has a matrix-core kernel.
-bool gemv_mfma_supports(std::uint32_t encoding);
+// True when a projection of this encoding and width has a matrix-core kernel.
+bool gemv_mfma_supports(std::uint32_t encoding, std::int64_t input_dim);
 
 // rows == 1: one launch, activations quantized inside it.  rows 2..16: one
 // quantizer launch into `workspace`, then the GEMV.
