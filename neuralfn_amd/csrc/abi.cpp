@@ -4,6 +4,7 @@
 // neuralfn/csrc/native_train/tile_ops.cu:4504-4713 and
 // neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:2349-2649.
 #include "common.hpp"
+#include "gemv_dot.hpp"
 #include "gemv_mfma.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
@@ -43,7 +44,8 @@ Projection make_projection(const Descriptor& descriptor, float* output) {
 }
 
 // Shared body of the small-batch entry points.
-int run_small_batch(const Descriptor* const* descriptors, const float* first,
+// `verifier`: every row must get the one-row arithmetic bit for bit.
+int run_small_batch(bool verifier, const Descriptor* const* descriptors, const float* first,
                     const float* second, int prologue, float* const* outputs,
                     std::int64_t operation_count, std::int64_t rows, void* workspace,
                     std::int64_t workspace_nbytes, void* stream) {
@@ -65,15 +67,27 @@ int run_small_batch(const Descriptor* const* descriptors, const float* first,
     }
     const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    // Projections with a matrix-core kernel go in one launch, the rest in another.
-    ProjectionSet fast{}, exact{};
-    fast.input_dim = exact.input_dim = input_dim;
+    // One row, and the verifier entry points at any row count: the vector-ALU
+    // kernel.  2..16 rows otherwise: the matrix-core kernel.  Encodings without
+    // either: the float kernel.
+    const bool one_row_arithmetic = rows == 1 || verifier;
+    ProjectionSet dot{}, matrix{}, exact{};
+    dot.input_dim = matrix.input_dim = exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
-        ProjectionSet& target = gemv_mfma_supports(set.op[index].encoding, input_dim) ? fast : exact;
-        target.op[target.count++] = set.op[index];
+        const std::uint32_t encoding = set.op[index].encoding;
+        ProjectionSet* target = &exact;
+        if (one_row_arithmetic && gemv_dot_supports(encoding, input_dim)) {
+            target = &dot;
+        } else if (gemv_mfma_supports(encoding, input_dim)) {
+            target = &matrix;
+        }
+        target->op[target->count++] = set.op[index];
     }
-    if (fast.count > 0) {
-        launch_gemv_mfma(fast, first, second, prologue, rows, workspace, as_stream(stream));
+    if (dot.count > 0) {
+        launch_gemv_dot(dot, first, second, prologue, rows, as_stream(stream));
+    }
+    if (matrix.count > 0) {
+        launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));
     }
     if (exact.count > 0) {
         launch_gemv_f32(exact, first, second, prologue, nullptr, rows, as_stream(stream));
@@ -220,7 +234,7 @@ int nfn_native_tile_k_quant_mmq_multi_linear_float32_v1(
     const Descriptor* const* descriptors, const float* input, float* const* outputs,
     std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
-    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
+    return run_small_batch(false, descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -229,7 +243,7 @@ int nfn_native_tile_k_quant_mmq_multi_linear_gated_float32_v1(
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
     if (gate == nullptr) return kInvalid;
-    return run_small_batch(descriptors, input, gate, kGated, outputs, operation_count, rows,
+    return run_small_batch(false, descriptors, input, gate, kGated, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -238,7 +252,7 @@ int nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1(
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
     if (gate == nullptr || up == nullptr) return kInvalid;
-    return run_small_batch(descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
+    return run_small_batch(false, descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -246,7 +260,7 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1(
     const Descriptor* const* descriptors, const float* input, float* const* outputs,
     std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
-    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
+    return run_small_batch(true, descriptors, input, nullptr, kPlain, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -255,7 +269,7 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
     if (gate == nullptr) return kInvalid;
-    return run_small_batch(descriptors, input, gate, kGated, outputs, operation_count, rows,
+    return run_small_batch(true, descriptors, input, gate, kGated, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -264,7 +278,7 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1(
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
     std::int64_t workspace_nbytes, void* cuda_stream) {
     if (gate == nullptr || up == nullptr) return kInvalid;
-    return run_small_batch(descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
+    return run_small_batch(true, descriptors, gate, up, kSwiGlu, outputs, operation_count, rows,
                            workspace, workspace_nbytes, cuda_stream);
 }
 
@@ -275,7 +289,7 @@ int nfn_native_tile_k_quant_mmvq_linear_float32_v1(const Descriptor* descriptor,
                                                    void* cuda_stream) {
     const Descriptor* descriptors[1] = {descriptor};
     float* outputs[1] = {output};
-    return run_small_batch(descriptors, input, nullptr, kPlain, outputs, 1, 1, workspace,
+    return run_small_batch(true, descriptors, input, nullptr, kPlain, outputs, 1, 1, workspace,
                            workspace_nbytes, cuda_stream);
 }
 

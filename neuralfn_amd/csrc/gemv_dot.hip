@@ -1,0 +1,541 @@
+// One-token (and verifier) decode GEMV on the vector ALUs: v_dot4_i32_i8.
+//
+// One wave owns whole weight rows; its 64 lanes split a row into units of one
+// 64-value pair of sub-blocks (32 bytes of 4-bit codes = two 16-byte loads, so
+// consecutive lanes read consecutive bytes of the row).  A workgroup first
+// turns the activation vector into two int8 planes (high and low byte of a
+// 16-bit fixed-point code, one scale per 256 values) in LDS, laid out so that
+// consecutive units read consecutive 16-byte slots; the first weight loads of
+// every wave are already in flight while it does so.  Per unit a lane then
+// spends 24 logic operations on unpacking and 32 dot4 on the two planes, and
+// folds the 6-bit sub-scales in with 24-bit integer multiplies; one float
+// conversion per unit, one butterfly per row.  No LDS round trip for weights,
+// no synchronisation after the single barrier, small register footprint: the
+// latency of HBM is hidden by many resident waves.
+//
+// Every row gets the same arithmetic whatever the number of tokens in the
+// launch (T token planes are walked one after another against the same
+// unpacked weights), which is the contract of the reference's verifier entry
+// points (neuralfn/csrc/native_train/tile_ops.h:685-688) and of its one-row
+// kernel (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:714-890).  With x = s*c,
+// c = 256*hi + lo:  y += s*(d*sum_sub sc*dot(q, c) - dmin*sum_sub m*sum(c)).
+#include "common.hpp"
+#include "gemv_dot.hpp"
+
+namespace nfn {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+#ifndef NFN_DOT_WAVES
+#define NFN_DOT_WAVES 8
+#endif
+#ifndef NFN_DOT_OCC
+#define NFN_DOT_OCC 32
+#endif
+constexpr int kDotWaves = NFN_DOT_WAVES;
+constexpr int kDotThreads = kDotWaves * kWave;
+constexpr float kCodeRange = 32512.0f;  // 127*256: the high byte stays in [-127, 127]
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int value) {
+    return __builtin_amdgcn_update_dpp(0, value, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float value) {
+    return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, value)));
+}
+
+constexpr int kQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141;  // lane k <-> 7-k within 8 lanes
+constexpr int kRowMirror = 0x140;   // lane k <-> 15-k within 16 lanes
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_move<kQuadXor1>(v));
+    v = fmaxf(v, dpp_move<kQuadXor2>(v));
+    v = fmaxf(v, dpp_move<kHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kRowMirror>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
+                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
+// Sum over the wave in a fixed order; the total is returned in every lane.
+__device__ __forceinline__ float wave_total(float v) {
+    v += dpp_move<kQuadXor1>(v);
+    v += dpp_move<kQuadXor2>(v);
+    v += dpp_move<kHalfMirror>(v);
+    v += dpp_move<kRowMirror>(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+
+__device__ __forceinline__ std::uint32_t perm(std::uint32_t hi, std::uint32_t lo, std::uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+template <int P>
+__device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
+                                                   const float* __restrict__ second,
+                                                   std::int64_t column) {
+    float4 x = *reinterpret_cast<const float4*>(first + column);
+    if constexpr (P != kPlain) {
+        const float4 y = *reinterpret_cast<const float4*>(second + column);
+        x.x = apply_prologue<P>(x.x, y.x);
+        x.y = apply_prologue<P>(x.y, y.y);
+        x.z = apply_prologue<P>(x.z, y.z);
+        x.w = apply_prologue<P>(x.w, y.w);
+    }
+    return x;
+}
+
+// LDS image of one token's activations for a K of `blocks` super-blocks:
+//   planes: eight arrays of `units` 16-byte slots, units = 4*blocks; unit
+//           u = 4*block + pair reads slot u of every array:
+//           array = 4*part + 2*plane + half  (part: which sub-block of the pair,
+//           plane: 0 high / 1 low byte, half: which 16 of the 32 values)
+//   sums:   int32 per sub-block: sum of its 32 codes
+//   scale:  float per block
+struct TokenImage {
+    std::uint8_t* planes;
+    int* sums;
+    float* scale;
+};
+
+__device__ __forceinline__ int token_image_bytes(int blocks) {
+    return blocks * (4 * 128 + 8 * 4 + 4 + 12);  // keeps every image 16-byte aligned
+}
+constexpr int token_image_bytes_host(std::int64_t blocks) {
+    return static_cast<int>(blocks * (4 * 128 + 8 * 4 + 4 + 12));
+}
+
+__device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, int blocks) {
+    std::uint8_t* base = lds + token * token_image_bytes(blocks);
+    TokenImage image;
+    image.planes = base;
+    image.sums = reinterpret_cast<int*>(base + blocks * 512);
+    image.scale = reinterpret_cast<float*>(base + blocks * 544);
+    return image;
+}
+
+// Quantize the 256 activations of block `block`, four per lane.
+__device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
+                                               const TokenImage& image) {
+    const float local = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+    const float maximum = wave_max(local);
+    const float inverse = maximum > 1.0e-30f ? kCodeRange * __builtin_amdgcn_rcpf(maximum) : 0.0f;
+    // 1.5*2^23 + 128: the low 16 bits of the sum's bit pattern are
+    // round-to-nearest-even(x*inverse) + 128 in two's complement.
+    constexpr float kMagic = 12582912.0f + 128.0f;
+    const std::uint32_t u0 = __float_as_uint(fmaf(x.x, inverse, kMagic));
+    const std::uint32_t u1 = __float_as_uint(fmaf(x.y, inverse, kMagic));
+    const std::uint32_t u2 = __float_as_uint(fmaf(x.z, inverse, kMagic));
+    const std::uint32_t u3 = __float_as_uint(fmaf(x.w, inverse, kMagic));
+    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped
+    const std::uint32_t p01 = perm(u1, u0, 0x05010400u);  // [u0.b0, u1.b0, u0.b1, u1.b1]
+    const std::uint32_t p23 = perm(u3, u2, 0x05010400u);
+    const std::uint32_t lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
+    const std::uint32_t hi = perm(p23, p01, 0x07060302u);
+    int sum = (__builtin_amdgcn_sdot4(static_cast<int>(hi), 0x01010101, 0, false) << 8) +
+        __builtin_amdgcn_sdot4(static_cast<int>(lo), 0x01010101, 0, false);
+    sum += dpp_move<kQuadXor1>(sum);
+    sum += dpp_move<kQuadXor2>(sum);
+    sum += dpp_move<kHalfMirror>(sum);
+    // lane L holds values 4L..4L+3: sub-block L/8, 16-value half (L%8)/4, byte (L%4)*4
+    const int units = 4 * blocks;
+    const int sub = lane >> 3;
+    const int unit = 4 * block + (sub >> 1);
+    const int array_high = 4 * (sub & 1) + ((lane >> 2) & 1);
+    std::uint8_t* slot = image.planes + (array_high * units + unit) * 16 + (lane & 3) * 4;
+    *reinterpret_cast<std::uint32_t*>(slot) = hi;
+    *reinterpret_cast<std::uint32_t*>(slot + 2 * units * 16) = lo;
+    if ((lane & 7) == 0) image.sums[block * 8 + sub] = sum;
+    if (lane == 0) image.scale[block] = maximum * (1.0f / kCodeRange);
+}
+
+template <bool Q5>
+struct Stage {
+    uint4 header;  // d, dmin, 12 scale bytes
+    uint4 q0, q1;  // 32 bytes of 4-bit codes
+    uint4 h0, h1;  // Q5_K: the block's 32 high-bit bytes
+};
+
+// Projection `index` of the set, chosen with scalar selects from fields that
+// were all read with static offsets: a dynamically indexed read of the kernel
+// arguments is a dependent scalar load, and its first touch of a cache line
+// costs a trip to memory in the middle of the kernel.
+__device__ __forceinline__ Projection pick(const ProjectionSet& set, int index) {
+    Projection p = set.op[0];
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+        const bool take = index == k;
+        p.data = take ? set.op[k].data : p.data;
+        p.output = take ? set.op[k].output : p.output;
+        p.output_dim = take ? set.op[k].output_dim : p.output_dim;
+        p.row_stride = take ? set.op[k].row_stride : p.row_stride;
+        p.first_tile = take ? set.op[k].first_tile : p.first_tile;
+    }
+    return p;
+}
+
+// Walks the (row, iteration) pairs of one wave without divisions: everything
+// here is uniform and lives in scalar registers.
+struct PairCursor {
+    int op;                   // projection index
+    Projection current;       // its fields
+    std::int64_t local_row;   // row inside that projection
+    int iteration;            // which 64-unit slice of the row
+    const std::uint8_t* row;  // first byte of the row
+
+    __device__ __forceinline__ void start(const ProjectionSet& set, std::int64_t global_row) {
+        op = 0;
+#pragma unroll
+        for (int index = 1; index < 4; ++index) {
+            if (index < set.count && global_row >= set.op[index].first_tile) op = index;
+        }
+        current = pick(set, op);
+        local_row = global_row - current.first_tile;
+        iteration = 0;
+        row = current.data + local_row * current.row_stride;
+    }
+    __device__ __forceinline__ void advance(const ProjectionSet& set, int iterations) {
+        if (++iteration < iterations) return;
+        iteration = 0;
+        ++local_row;
+        row += current.row_stride;
+        if (local_row == current.output_dim && op + 1 < set.count) {
+            ++op;
+            current = pick(set, op);
+            local_row = 0;
+            row = current.data;
+        }
+    }
+};
+
+template <std::uint32_t ENC, int T, int P>
+__global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
+    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
+    int tokens, std::int64_t total_rows, int rows_per_wave, int token_base_stride) {
+    constexpr bool kQ5 = ENC == kEncQ5K;
+    constexpr int kBlockBytes = kQ5 ? 176 : 144;
+    constexpr int kQuants = kQ5 ? 48 : 16;
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
+
+#ifdef NFN_EXP_TIMELINE
+    unsigned long long stamp[8];
+    stamp[0] = __builtin_amdgcn_s_memrealtime();
+#define NFN_STAMP(i) stamp[i] = __builtin_amdgcn_s_memrealtime()
+#else
+#define NFN_STAMP(i)
+#endif
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int blocks = static_cast<int>(set.input_dim >> 8);
+    const int units = 4 * blocks;
+    const int iterations = (units + kWave - 1) / kWave;
+    const int token0 = blockIdx.y * T;
+    const int pass_tokens = min(tokens - token0, T);
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_second =
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+
+    // rows of this wave: a contiguous range
+    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kDotWaves + wave;
+    const std::int64_t row_begin = wave_index * rows_per_wave;
+    const int row_count = static_cast<int>(
+        max(static_cast<std::int64_t>(0), min(static_cast<std::int64_t>(rows_per_wave), total_rows - row_begin)));
+    const int total = row_count * iterations;
+
+    // (1) activations of the first records this wave quantizes: loaded first so
+    // that their short latency does not queue behind the weight loads.  All
+    // loads are unconditional (clamped indices) to keep the load counters exact.
+    const int records = pass_tokens * blocks;
+    constexpr int kEarly = 4;
+    float4 early[kEarly];
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = min(wave + e * kDotWaves, records - 1);
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        early[e] = load_activations<P>(pass_first, pass_second,
+                                       static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+    }
+
+    // (2) weight loads of the first two (row, iteration) pairs
+    PairCursor fetch;
+    fetch.start(set, min(row_begin, total_rows - 1));
+    int fetch_left = total;  // pairs not fetched yet; the cursor rests on the last one
+    auto issue = [&](Stage<kQ5>& stage) {
+        const int unit = min(fetch.iteration * kWave + lane, units - 1);
+        const std::uint8_t* block = fetch.row + (unit >> 2) * kBlockBytes;
+        stage.header = *reinterpret_cast<const uint4*>(block);
+        const std::uint8_t* quants = block + kQuants + (unit & 3) * 32;
+        stage.q0 = *reinterpret_cast<const uint4*>(quants);
+        stage.q1 = *reinterpret_cast<const uint4*>(quants + 16);
+        if constexpr (kQ5) {
+            stage.h0 = *reinterpret_cast<const uint4*>(block + 16);
+            stage.h1 = *reinterpret_cast<const uint4*>(block + 32);
+        }
+        if (--fetch_left > 0) fetch.advance(set, iterations);
+    };
+    Stage<kQ5> stage0, stage1;
+    NFN_STAMP(1);
+    issue(stage0);
+    issue(stage1);
+#ifdef NFN_EXP_TIMELINE
+    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    NFN_STAMP(2);
+#endif
+
+    // (3) quantize; one barrier; after it the workgroup never synchronises again
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = wave + e * kDotWaves;
+#ifndef NFN_EXP_SKIP_QUANT
+        if (record < records) {
+            const int token = record / blocks;
+            quantize_block(early[e], lane, record - token * blocks, blocks,
+                           token_image(lds, token, blocks));
+        }
+#endif
+    }
+    for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        const float4 x = load_activations<P>(
+            pass_first, pass_second,
+            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+    }
+    NFN_STAMP(3);
+    __syncthreads();
+    NFN_STAMP(4);
+#ifdef NFN_EXP_TIMELINE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    NFN_STAMP(5);
+#endif
+
+    float acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = 0.0f;
+
+    PairCursor work;
+    work.start(set, min(row_begin, total_rows - 1));
+    auto compute = [&](const Stage<kQ5>& stage) {
+        const int iteration = work.iteration;
+#ifdef NFN_EXP_SKIP_COMPUTE
+        acc[0] += __uint_as_float((stage.q0.x ^ stage.q0.y ^ stage.q0.z ^ stage.q0.w ^ stage.q1.x ^ stage.q1.y ^ stage.q1.z ^ stage.q1.w ^ stage.header.x ^ stage.header.y ^ stage.header.z ^ stage.header.w) & 0x3fffffffu);
+        if (acc[0] == 1.2345f) lds[lane] = 1;
+        work.advance(set, iterations);
+        return;
+#endif
+        const int raw_unit = iteration * kWave + lane;
+        const bool live = raw_unit < units;
+        const int unit = min(raw_unit, units - 1);
+        const int block = unit >> 2;
+        const int pair = unit & 3;
+
+        // unpack: the low nibbles are sub-block 2*pair, the high nibbles 2*pair+1
+        const std::uint32_t packed[8] = {stage.q0.x, stage.q0.y, stage.q0.z, stage.q0.w,
+                                         stage.q1.x, stage.q1.y, stage.q1.z, stage.q1.w};
+        std::uint32_t low[8], high[8];
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            low[w] = packed[w] & 0x0f0f0f0fu;
+            high[w] = (packed[w] >> 4) & 0x0f0f0f0fu;
+        }
+        if constexpr (kQ5) {
+            const std::uint32_t bits[8] = {stage.h0.x, stage.h0.y, stage.h0.z, stage.h0.w,
+                                           stage.h1.x, stage.h1.y, stage.h1.z, stage.h1.w};
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                // bit 2*pair of the high-bit byte belongs to the first sub-block, 2*pair+1 to the second
+                const std::uint32_t shifted = bits[w] >> (2 * pair);
+                low[w] |= (shifted & 0x01010101u) << 4;
+                high[w] |= (shifted & 0x02020202u) << 3;
+            }
+        }
+        // the pair's two 6-bit scales and minimums, packed [second:first] in 16 bits
+        const int shift = 16 * (pair & 1);
+        const std::uint32_t y = stage.header.y >> shift;
+        const std::uint32_t z = stage.header.z >> shift;
+        const std::uint32_t w = stage.header.w >> shift;
+        const bool upper = pair >= 2;
+        const std::uint32_t scales = upper ? ((w & 0x0f0fu) | ((y >> 2) & 0x3030u)) : (y & 0x3f3fu);
+        const std::uint32_t minimums =
+            upper ? (((w >> 4) & 0x0f0fu) | ((z >> 2) & 0x3030u)) : (z & 0x3f3fu);
+        // as floats: every product and sum below stays under 2^24, so the
+        // float arithmetic on the integer dot products is exact
+        const float scale_a = static_cast<float>(scales & 0xffu);
+        const float scale_b = static_cast<float>((scales >> 8) & 0xffu);
+        const float min_a = static_cast<float>(minimums & 0xffu);
+        const float min_b = static_cast<float>((minimums >> 8) & 0xffu);
+        const float d = half_bits_to_float(stage.header.x & 0xffffu);
+        const float dmin = half_bits_to_float(stage.header.x >> 16);
+
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const TokenImage image = token_image(lds, t, blocks);
+            const std::uint8_t* slot = image.planes + unit * 16;
+            const int stride = units * 16;
+            int dot_a_hi = 0, dot_a_lo = 0, dot_b_hi = 0, dot_b_lo = 0;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const v4i a_hi = *reinterpret_cast<const v4i*>(slot + (0 + half) * stride);
+                const v4i a_lo = *reinterpret_cast<const v4i*>(slot + (2 + half) * stride);
+                const v4i b_hi = *reinterpret_cast<const v4i*>(slot + (4 + half) * stride);
+                const v4i b_lo = *reinterpret_cast<const v4i*>(slot + (6 + half) * stride);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int lo_codes = static_cast<int>(low[half * 4 + v]);
+                    const int hi_codes = static_cast<int>(high[half * 4 + v]);
+                    dot_a_hi = __builtin_amdgcn_sdot4(lo_codes, a_hi[v], dot_a_hi, false);
+                    dot_a_lo = __builtin_amdgcn_sdot4(lo_codes, a_lo[v], dot_a_lo, false);
+                    dot_b_hi = __builtin_amdgcn_sdot4(hi_codes, b_hi[v], dot_b_hi, false);
+                    dot_b_lo = __builtin_amdgcn_sdot4(hi_codes, b_lo[v], dot_b_lo, false);
+                }
+            }
+            const int2 sums = *reinterpret_cast<const int2*>(image.sums + block * 8 + 2 * pair);
+            const float scale = image.scale[block];
+            const float weighted_hi = fmaf(scale_b, static_cast<float>(dot_b_hi),
+                                           scale_a * static_cast<float>(dot_a_hi));
+            const float weighted_lo = fmaf(scale_b, static_cast<float>(dot_b_lo),
+                                           scale_a * static_cast<float>(dot_a_lo));
+            const float weighted_min = fmaf(min_b, static_cast<float>(sums.y),
+                                            min_a * static_cast<float>(sums.x));
+            const float codes = fmaf(weighted_hi, 256.0f, weighted_lo);
+            const float value = fmaf(-dmin, weighted_min, d * codes);
+            acc[t] = fmaf(live ? scale : 0.0f, value, acc[t]);
+        }
+
+        if (iteration == iterations - 1) {
+            // the row is complete: fixed-order butterfly, lane 0 writes
+            float* output = work.current.output + work.local_row;
+            const std::int64_t output_dim = work.current.output_dim;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const float total_value = wave_total(acc[t]);
+                if (lane == 0 && t < pass_tokens) {
+                    output[static_cast<std::int64_t>(token0 + t) * output_dim] = total_value;
+                }
+                acc[t] = 0.0f;
+            }
+        }
+        work.advance(set, iterations);
+    };
+
+    for (int n = 0; n < total; n += 2) {
+        compute(stage0);
+        issue(stage0);
+        if (n + 1 < total) compute(stage1);
+        issue(stage1);
+    }
+#ifdef NFN_EXP_TIMELINE
+    NFN_STAMP(6);
+    if (lane == 0 && wave == 0 && blockIdx.x < 500) {
+        unsigned* out = reinterpret_cast<unsigned*>(const_cast<float*>(first));
+        for (int i = 0; i < 7; ++i) out[blockIdx.x * 8 + i] = static_cast<unsigned>(stamp[i]);
+    }
+#endif
+    (void)token_base_stride;
+}
+
+int compute_units() {
+    static const int count = [] {
+        int device = 0;
+        int value = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            value <= 0) {
+            return 256;
+        }
+        return value;
+    }();
+    return count;
+}
+
+template <std::uint32_t ENC, int T, int P>
+void launch_variant(ProjectionSet set, const float* first, const float* second, int tokens,
+                    hipStream_t stream) {
+    std::int64_t rows = 0;
+    for (int index = 0; index < set.count; ++index) {
+        set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
+        rows += set.op[index].output_dim;
+    }
+    const std::int64_t blocks = set.input_dim >> 8;
+    const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes_host(blocks);
+    auto kernel = gemv_dot_kernel<ENC, T, P>;
+    static const bool raised =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+    (void)raised;
+    // about one wave per SIMD lane group and row range: rows_per_wave keeps the
+    // activation quantization (done once per workgroup) a small part of the work
+    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * NFN_DOT_OCC;
+    std::int64_t rows_per_wave = rows / waves_wanted;
+    if (rows_per_wave < 1) rows_per_wave = 1;
+    const std::int64_t groups = (rows + rows_per_wave * kDotWaves - 1) / (rows_per_wave * kDotWaves);
+    const int passes = (tokens + T - 1) / T;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
+                       stream, set, first, second, tokens, rows, static_cast<int>(rows_per_wave), 0);
+}
+
+template <std::uint32_t ENC, int P>
+void launch_tokens(const ProjectionSet& set, const float* first, const float* second, int tokens,
+                   hipStream_t stream) {
+    // token planes of one pass must fit in LDS: four tokens up to K = 16384
+    const std::int64_t image = token_image_bytes_host(set.input_dim >> 8);
+    int capacity = static_cast<int>((150 * 1024) / image);
+    if (capacity > 4) capacity = 4;
+    const int per_pass = tokens < capacity ? tokens : capacity;
+    if (per_pass <= 1) {
+        launch_variant<ENC, 1, P>(set, first, second, tokens, stream);
+    } else if (per_pass == 2) {
+        launch_variant<ENC, 2, P>(set, first, second, tokens, stream);
+    } else if (capacity >= 4) {
+        launch_variant<ENC, 4, P>(set, first, second, tokens, stream);
+    } else {
+        launch_variant<ENC, 2, P>(set, first, second, tokens, stream);
+    }
+}
+
+template <std::uint32_t ENC>
+void launch_prologue(const ProjectionSet& set, const float* first, const float* second,
+                     int prologue, int tokens, hipStream_t stream) {
+    switch (prologue) {
+        case kGated: launch_tokens<ENC, kGated>(set, first, second, tokens, stream); break;
+        case kSwiGlu: launch_tokens<ENC, kSwiGlu>(set, first, second, tokens, stream); break;
+        default: launch_tokens<ENC, kPlain>(set, first, second, tokens, stream); break;
+    }
+}
+
+}  // namespace
+
+bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim) {
+    return (encoding == kEncQ4K || encoding == kEncQ5K) && input_dim % 256 == 0 &&
+        token_image_bytes_host(input_dim >> 8) <= 150 * 1024;
+}
+
+void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* second,
+                     int prologue, std::int64_t rows, hipStream_t stream) {
+    const std::uint32_t encodings[2] = {kEncQ4K, kEncQ5K};
+    for (const std::uint32_t encoding : encodings) {
+        ProjectionSet group{};
+        group.input_dim = set.input_dim;
+        for (int index = 0; index < set.count; ++index) {
+            if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
+        }
+        if (group.count == 0) continue;
+        if (encoding == kEncQ4K) {
+            launch_prologue<kEncQ4K>(group, first, second, prologue, static_cast<int>(rows), stream);
+        } else {
+            launch_prologue<kEncQ5K>(group, first, second, prologue, static_cast<int>(rows), stream);
+        }
+    }
+}
+
+}  // namespace nfn

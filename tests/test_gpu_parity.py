@@ -482,3 +482,15 @@ def test_prefill_gemm_full_size_row_subset(cuda, oracle):
     assert normalised_error(y[:, :256], expected) <= TOLERANCE
     # every 256-column stripe repeats the same weights
     assert np.array_equal(y[:, :256], y[:, out_dim - 256:])
+
+
+def test_decode_gemv_is_deterministic(cuda):
+    # the same call must return the same bits every time (fixed reduction order)
+    out_dim, in_dim = 520, 6656
+    packed = random_packed(kquant.Q4_K, out_dim, in_dim, 5)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, packed, out_dim, in_dim)
+    x = to_device(kquant.synthetic_activations(8, 1, in_dim), cuda)
+    workspace = tile_ops.small_batch_workspace(1, in_dim)
+    first = tile_ops.mmvq_linear(weight, x, workspace).cpu().numpy()
+    for _ in range(20):
+        assert_bits_equal(tile_ops.mmvq_linear(weight, x, workspace), first)
