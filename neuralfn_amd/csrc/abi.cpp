@@ -5,6 +5,7 @@
 // neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:2349-2649.
 #include "common.hpp"
 #include "gemv_dot.hpp"
+#include "gemm_mfma.hpp"
 #include "gemv_mfma.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
@@ -352,7 +353,7 @@ std::int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(std::int64_t rows, std::i
         (mode != NFN_MI355_GEMM_BF16 && mode != NFN_MI355_GEMM_INT8)) {
         return 0;
     }
-    return 256;
+    return mode == NFN_MI355_GEMM_BF16 ? gemm_bf16_workspace_bytes(rows, input_dim) : 256;
 }
 
 int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float* input,
@@ -369,6 +370,12 @@ int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float*
     const std::int64_t required = nfn_mi355_k_quant_gemm_workspace_bytes_v1(
         rows, normalized.input_dim, normalized.output_dim, mode);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
+    if (mode == NFN_MI355_GEMM_BF16 &&
+        gemm_bf16_supports(normalized.encoding, normalized.input_dim)) {
+        if (reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) return kInvalid;
+        launch_gemm_bf16(normalized, input, output, rows, workspace, as_stream(cuda_stream));
+        return launch_status();
+    }
     ProjectionSet set{};
     set.count = 1;
     set.input_dim = normalized.input_dim;
