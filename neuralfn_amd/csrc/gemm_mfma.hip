@@ -53,12 +53,15 @@ __device__ __forceinline__ std::uint32_t pack_bf16(float lo, float hi) {
 }
 
 // fp32 -> bf16 (round to nearest even) copy of the activations
+// into whole 256-row tiles: rows past the end are written as zeros
 __global__ __launch_bounds__(256) void convert_activations_kernel(
-    const float* __restrict__ input, std::uint32_t* __restrict__ output, std::int64_t pairs) {
+    const float* __restrict__ input, std::uint32_t* __restrict__ output, std::int64_t quads,
+    std::int64_t padded_quads) {
     const std::int64_t stride = static_cast<std::int64_t>(gridDim.x) * blockDim.x;
     for (std::int64_t i = static_cast<std::int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-         i < pairs / 2; i += stride) {
-        const float4 x = reinterpret_cast<const float4*>(input)[i];
+         i < padded_quads; i += stride) {
+        float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (i < quads) x = reinterpret_cast<const float4*>(input)[i];
         reinterpret_cast<uint2*>(output)[i] = make_uint2(pack_bf16(x.x, x.y), pack_bf16(x.z, x.w));
     }
 }
@@ -85,10 +88,13 @@ struct PackedSlice<kEncQ4K> {
         const std::uint32_t y = header.y, z = header.z, w = header.w;
         const int shift = 16 * (pair & 1);
         const std::uint32_t ys = y >> shift, zs = z >> shift, ws = w >> shift;
-        const bool upper = pair >= 2;
-        const std::uint32_t sc = upper ? ((ws & 0x0f0fu) | ((ys >> 2) & 0x3030u)) : (ys & 0x3f3fu);
-        const std::uint32_t mn =
-            upper ? (((ws >> 4) & 0x0f0fu) | ((zs >> 2) & 0x3030u)) : (zs & 0x3f3fu);
+        // sub-blocks 4..7 keep their 6-bit values split over two bytes; bit masks
+        // instead of a branch keep the K step one basic block
+        const std::uint32_t upper = 0u - static_cast<std::uint32_t>(pair >> 1);
+        const std::uint32_t sc = (((ws & 0x0f0fu) | ((ys >> 2) & 0x3030u)) & upper) |
+            ((ys & 0x3f3fu) & ~upper);
+        const std::uint32_t mn = ((((ws >> 4) & 0x0f0fu) | ((zs >> 2) & 0x3030u)) & upper) |
+            ((zs & 0x3f3fu) & ~upper);
         const float da = d * static_cast<float>(sc & 0xffu);
         const float db = d * static_cast<float>((sc >> 8) & 0xffu);
         const float ma = dmin * static_cast<float>(mn & 0xffu);
@@ -130,10 +136,13 @@ struct PackedSlice<kEncQ5K> {
         const float dmin = half_bits_to_float(header.x >> 16);
         const int shift = 16 * (pair & 1);
         const std::uint32_t ys = header.y >> shift, zs = header.z >> shift, ws = header.w >> shift;
-        const bool upper = pair >= 2;
-        const std::uint32_t sc = upper ? ((ws & 0x0f0fu) | ((ys >> 2) & 0x3030u)) : (ys & 0x3f3fu);
-        const std::uint32_t mn =
-            upper ? (((ws >> 4) & 0x0f0fu) | ((zs >> 2) & 0x3030u)) : (zs & 0x3f3fu);
+        // sub-blocks 4..7 keep their 6-bit values split over two bytes; bit masks
+        // instead of a branch keep the K step one basic block
+        const std::uint32_t upper = 0u - static_cast<std::uint32_t>(pair >> 1);
+        const std::uint32_t sc = (((ws & 0x0f0fu) | ((ys >> 2) & 0x3030u)) & upper) |
+            ((ys & 0x3f3fu) & ~upper);
+        const std::uint32_t mn = ((((ws >> 4) & 0x0f0fu) | ((zs >> 2) & 0x3030u)) & upper) |
+            ((zs & 0x3f3fu) & ~upper);
         const float da = d * static_cast<float>(sc & 0xffu);
         const float db = d * static_cast<float>((sc >> 8) & 0xffu);
         const float ma = dmin * static_cast<float>(mn & 0xffu);
@@ -182,7 +191,7 @@ struct PackedSlice<kEncQ6K> {
     }
     __device__ __forceinline__ void decode(int pair, int half, std::uint32_t (&out)[16]) const {
         const float d = half_bits_to_float(d_bits);
-        const bool upper = (pair & 1) != 0;  // quarters 2,3: high nibbles, high-bit pairs 4..7
+        const int upper = (pair & 1) * 4;  // quarters 2,3: high nibbles, high-bit pairs 4..7
         // sub-scale index = quarter*2 + lane/16: this thread's 16 values sit in one 16-group
         const int sa = static_cast<std::int8_t>((scale_bytes >> (8 * half)) & 0xffu);
         const int sb = static_cast<std::int8_t>((scale_bytes >> (8 * (2 + half))) & 0xffu);
@@ -193,9 +202,9 @@ struct PackedSlice<kEncQ6K> {
         const std::uint32_t hb[4] = {high.x, high.y, high.z, high.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const std::uint32_t na = (upper ? la[i] >> 4 : la[i]) & 0x0f0f0f0fu;
-            const std::uint32_t nb = (upper ? lb[i] >> 4 : lb[i]) & 0x0f0f0f0fu;
-            const std::uint32_t ha = (upper ? hb[i] >> 4 : hb[i]);        // bits 0,1 -> first quarter
+            const std::uint32_t na = (la[i] >> upper) & 0x0f0f0f0fu;
+            const std::uint32_t nb = (lb[i] >> upper) & 0x0f0f0f0fu;
+            const std::uint32_t ha = hb[i] >> upper;  // bits 0,1 -> first quarter
             const std::uint32_t qa = na | ((ha & 0x03030303u) << 4);
             const std::uint32_t qb = nb | (((ha >> 2) & 0x03030303u) << 4);
             float a[4], b[4];
@@ -247,6 +256,81 @@ struct PackedSlice<kEncQ8_0> {
     }
 };
 
+typedef std::uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// Eight 16-byte chunks of activations in named registers (an array here ends up
+// in scratch memory).
+struct ActivationSlice {
+    u32x4 c0, c1, c2, c3, c4, c5, c6, c7;
+};
+#define NFN_EACH_CHUNK(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7)
+
+__device__ __forceinline__ void load_slice(ActivationSlice& a, const std::uint8_t* source,
+                                           std::int64_t row_bytes) {
+#define NFN_LOAD_CHUNK(i) a.c##i = *reinterpret_cast<const u32x4*>(source + i * 32 * row_bytes);
+    NFN_EACH_CHUNK(NFN_LOAD_CHUNK)
+#undef NFN_LOAD_CHUNK
+}
+
+__device__ __forceinline__ void store_slice(const ActivationSlice& a, std::uint8_t* target) {
+#define NFN_STORE_CHUNK(i) *reinterpret_cast<u32x4*>(target + i * 32 * kRowBytes) = a.c##i;
+    NFN_EACH_CHUNK(NFN_STORE_CHUNK)
+#undef NFN_STORE_CHUNK
+}
+
+// One K step: the 32 matrix instructions of `stage`, the dequantization of the
+// slice held in (a_next, b_next) into `other`, and the loads that refill them.
+// The scheduling groups at the end ask for that work to be issued between the
+// matrix instructions rather than after them.
+template <std::uint32_t ENC>
+__device__ __forceinline__ void k_step(
+    v16f (&acc)[4][2], const std::uint8_t* a_read, const std::uint8_t* b_read,
+    std::uint8_t* a_write, std::uint8_t* b_write, ActivationSlice& a_next,
+    PackedSlice<ENC>& b_next, int decode_pair, int b_half,
+    const std::uint8_t* a_global, std::int64_t a_row_bytes, const std::uint8_t* b_global,
+    int fetch_step) {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+        bf16x8 a[4], b[2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            a[i] = *reinterpret_cast<const bf16x8*>(a_read + i * 32 * kRowBytes + kk * 32);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            b[j] = *reinterpret_cast<const bf16x8*>(b_read + j * 32 * kRowBytes + kk * 32);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+    // dequantize the held slice into the other stage
+    std::uint32_t w[16];
+    b_next.decode(decode_pair, b_half, w);
+    *reinterpret_cast<uint4*>(b_write) = make_uint4(w[0], w[1], w[2], w[3]);
+    *reinterpret_cast<uint4*>(b_write + 16) = make_uint4(w[4], w[5], w[6], w[7]);
+    *reinterpret_cast<uint4*>(b_write + 64) = make_uint4(w[8], w[9], w[10], w[11]);
+    *reinterpret_cast<uint4*>(b_write + 80) = make_uint4(w[12], w[13], w[14], w[15]);
+    store_slice(a_next, a_write);
+    // refill
+    load_slice(a_next, a_global + static_cast<std::int64_t>(fetch_step) * (kBK * 2), a_row_bytes);
+    b_next.load(b_global, fetch_step >> 2, fetch_step & 3, b_half);
+
+    // 32 x {1 matrix op, 1 LDS read, 4 vector ops}, LDS writes and global loads spread over them
+#pragma unroll
+    for (int g = 0; g < 32; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (g < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        if (g >= 12 && g < 24) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        if (g >= 22) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+}
+
 template <std::uint32_t ENC>
 __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(
     const std::uint8_t* __restrict__ weights, std::int64_t row_stride, std::int64_t output_dim,
@@ -256,54 +340,26 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_m = wave >> 1;  // 0..1: which 128 rows
-    const int wave_n = wave & 1;   // 0..1: which 64 columns
+    const int wave_m = wave >> 1;  // which 128 rows
+    const int wave_n = wave & 1;   // which 64 columns
     const int m_tile = blockIdx.x % m_tiles;
     const int n_tile = blockIdx.x / m_tiles;
     const std::int64_t m0 = static_cast<std::int64_t>(m_tile) * kBM;
     const std::int64_t n0 = static_cast<std::int64_t>(n_tile) * kBN;
-    const int steps = static_cast<int>(input_dim / kBK);
+    const int steps = static_cast<int>(input_dim / kBK);  // a multiple of 4
+    const int last = steps - 1;
 
-    // activation copy: 8 chunks of 16 bytes per thread and step
-    const std::uint16_t* a_source[8];
-    int a_target[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int chunk = tid + i * kThreads;
-        const int row = chunk >> 3;
-        const int col = chunk & 7;
-        const std::int64_t m = min(m0 + row, rows - 1);
-        a_source[i] = activations + m * input_dim + col * 8;
-        a_target[i] = row * kRowBytes + col * 16;
-    }
+    // activation copy: chunk c = tid + 256*i is row c/8 = tid/8 + 32*i, 16-byte column tid%8;
+    // the workspace holds whole 256-row tiles, so no row needs a bounds check
+    const std::int64_t a_row_bytes = input_dim * 2;
+    const std::uint8_t* a_global = reinterpret_cast<const std::uint8_t*>(activations) +
+        (m0 + (tid >> 3)) * a_row_bytes + (tid & 7) * 16;
+    const int a_target = (tid >> 3) * kRowBytes + (tid & 7) * 16;
     // weights: thread -> (row, which 16 positions of the two 32-value groups)
     const int b_row = tid >> 1;
     const int b_half = tid & 1;
-    const std::uint8_t* b_source = weights + min(n0 + b_row, output_dim - 1) * row_stride;
+    const std::uint8_t* b_global = weights + min(n0 + b_row, output_dim - 1) * row_stride;
     const int b_target = kTileA + b_row * kRowBytes + b_half * 32;
-
-    uint4 a_regs[8];
-    PackedSlice<ENC> b_regs;
-    auto fetch = [&](int step) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            a_regs[i] = *reinterpret_cast<const uint4*>(a_source[i] + step * kBK);
-        }
-        b_regs.load(b_source, step >> 2, step & 3, b_half);
-    };
-    auto stash = [&](int step, std::uint8_t* stage) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            *reinterpret_cast<uint4*>(stage + a_target[i]) = a_regs[i];
-        }
-        std::uint32_t w[16];
-        b_regs.decode(step & 3, b_half, w);
-        std::uint8_t* target = stage + b_target;
-        *reinterpret_cast<uint4*>(target) = make_uint4(w[0], w[1], w[2], w[3]);
-        *reinterpret_cast<uint4*>(target + 16) = make_uint4(w[4], w[5], w[6], w[7]);
-        *reinterpret_cast<uint4*>(target + 64) = make_uint4(w[8], w[9], w[10], w[11]);
-        *reinterpret_cast<uint4*>(target + 80) = make_uint4(w[12], w[13], w[14], w[15]);
-    };
 
     v16f acc[4][2];
 #pragma unroll
@@ -315,55 +371,64 @@ __global__ __launch_bounds__(kThreads) void gemm_bf16_kernel(
         }
     }
 
-    fetch(0);
-    stash(0, lds);
-    if (steps > 1) fetch(1);
+    ActivationSlice a_even, a_odd;  // hold steps s+2 (even s) and s+1 while step s computes
+    PackedSlice<ENC> b_even, b_odd;
+    auto fetch = [&](ActivationSlice& a, PackedSlice<ENC>& b, int step) {
+        load_slice(a, a_global + static_cast<std::int64_t>(step) * (kBK * 2), a_row_bytes);
+        b.load(b_global, step >> 2, step & 3, b_half);
+    };
+    fetch(a_even, b_even, 0);
+    fetch(a_odd, b_odd, 1);
+    {
+        std::uint32_t w[16];
+        b_even.decode(0, b_half, w);
+        std::uint8_t* target = lds + b_target;
+        *reinterpret_cast<uint4*>(target) = make_uint4(w[0], w[1], w[2], w[3]);
+        *reinterpret_cast<uint4*>(target + 16) = make_uint4(w[4], w[5], w[6], w[7]);
+        *reinterpret_cast<uint4*>(target + 64) = make_uint4(w[8], w[9], w[10], w[11]);
+        *reinterpret_cast<uint4*>(target + 80) = make_uint4(w[12], w[13], w[14], w[15]);
+        store_slice(a_even, lds + a_target);
+    }
+    fetch(a_even, b_even, 2);
     __syncthreads();
 
-    const int operand_row = lane & 31;
-    const int operand_k = (lane >> 5) * 16;
-    for (int step = 0; step < steps; ++step) {
-        const std::uint8_t* stage = lds + (step & 1) * kStageBytes;
-        const std::uint8_t* a_base = stage + (wave_m * 128 + operand_row) * kRowBytes + operand_k;
-        const std::uint8_t* b_base = stage + kTileA + (wave_n * 64 + operand_row) * kRowBytes + operand_k;
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            bf16x8 a[4], b[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                a[i] = *reinterpret_cast<const bf16x8*>(a_base + i * 32 * kRowBytes + kk * 32);
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                b[j] = *reinterpret_cast<const bf16x8*>(b_base + j * 32 * kRowBytes + kk * 32);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-                }
-            }
-        }
-        if (step + 1 < steps) {
-            stash(step + 1, lds + ((step + 1) & 1) * kStageBytes);
-            if (step + 2 < steps) fetch(step + 2);
-        }
+    const int operand = (lane & 31) * kRowBytes + (lane >> 5) * 16;
+    const std::uint8_t* a_read0 = lds + wave_m * 128 * kRowBytes + operand;
+    const std::uint8_t* b_read0 = lds + kTileA + wave_n * 64 * kRowBytes + operand;
+    for (int step = 0; step < steps; step += 2) {
+        // stage 0 computes; step+1 (odd slice) goes to stage 1; odd slice refills with step+3
+        k_step<ENC>(acc, a_read0, b_read0, lds + kStageBytes + a_target,
+                    lds + kStageBytes + b_target, a_odd, b_odd, (step + 1) & 3, b_half, a_global,
+                    a_row_bytes, b_global, min(step + 3, last));
+        __syncthreads();
+        // stage 1 computes; step+2 (even slice) goes to stage 0; even slice refills with step+4
+        k_step<ENC>(acc, a_read0 + kStageBytes, b_read0 + kStageBytes, lds + a_target,
+                    lds + b_target, a_even, b_even, (step + 2) & 3, b_half, a_global, a_row_bytes,
+                    b_global, min(step + 4, last));
         __syncthreads();
     }
 
     // D register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     const int column = lane & 31;
     const int row_base = (lane >> 5) * 4;
+    const bool whole = m0 + kBM <= rows && n0 + kBN <= output_dim;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const std::int64_t n = n0 + wave_n * 64 + j * 32 + column;
+            float* target = output + (m0 + wave_m * 128 + i * 32 + row_base) * output_dim + n;
+            if (whole) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const std::int64_t m = m0 + wave_m * 128 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
-                if (m < rows && n < output_dim) output[m * output_dim + n] = acc[i][j][r];
+                for (int r = 0; r < 16; ++r) {
+                    target[(8 * (r >> 2) + (r & 3)) * output_dim] = acc[i][j][r];
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const std::int64_t m = m0 + wave_m * 128 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
+                    if (m < rows && n < output_dim) output[m * output_dim + n] = acc[i][j][r];
+                }
             }
         }
     }
@@ -388,7 +453,8 @@ void launch_encoding(const Descriptor& descriptor, const std::uint16_t* activati
 }  // namespace
 
 std::int64_t gemm_bf16_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
-    return ((rows * input_dim * 2 + 255) & ~std::int64_t(255)) + 256;
+    const std::int64_t padded_rows = (rows + kBM - 1) / kBM * kBM;
+    return padded_rows * input_dim * 2 + 256;
 }
 
 bool gemm_bf16_supports(std::uint32_t encoding, std::int64_t input_dim) {
@@ -399,11 +465,13 @@ bool gemm_bf16_supports(std::uint32_t encoding, std::int64_t input_dim) {
 void launch_gemm_bf16(const Descriptor& descriptor, const float* input, float* output,
                       std::int64_t rows, void* workspace, hipStream_t stream) {
     std::uint16_t* activations = static_cast<std::uint16_t*>(workspace);
-    const std::int64_t pairs = rows * descriptor.input_dim / 2;
-    const std::int64_t blocks = (pairs / 2 + 255) / 256;
+    const std::int64_t quads = rows * descriptor.input_dim / 4;
+    const std::int64_t padded_quads = (rows + kBM - 1) / kBM * kBM * descriptor.input_dim / 4;
+    const std::int64_t blocks = (padded_quads + 255) / 256;
     hipLaunchKernelGGL(convert_activations_kernel,
                        dim3(static_cast<unsigned>(blocks < 65536 ? blocks : 65536)), dim3(256), 0,
-                       stream, input, reinterpret_cast<std::uint32_t*>(activations), pairs);
+                       stream, input, reinterpret_cast<std::uint32_t*>(activations), quads,
+                       padded_quads);
     switch (descriptor.encoding) {
         case kEncQ4K: launch_encoding<kEncQ4K>(descriptor, activations, output, rows, stream); break;
         case kEncQ5K: launch_encoding<kEncQ5K>(descriptor, activations, output, rows, stream); break;
