@@ -32,7 +32,7 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
-MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
 FFN_DIM = 16384
 VOCAB = 202048
@@ -232,7 +232,7 @@ def prefill_extra(device, steps: int, warmup: int) -> dict:
     gate = random_packed_on_device(kquant.Q4_K, FFN_DIM, MODEL_DIM, device, 8)
     down = random_packed_on_device(kquant.Q4_K, MODEL_DIM, FFN_DIM, device, 9)
     result = {}
-    for mode, name in ((tile_ops.GEMM_BF16, "bf16"), (tile_ops.GEMM_INT8, "int8")):
+    for mode, name in ((tile_ops.GEMM_F16, "f16"), (tile_ops.GEMM_INT8, "int8")):
         for rows in (512, 2048):
             x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
             h = torch.from_numpy(kquant.synthetic_activations(32, rows, FFN_DIM)).to(device)

@@ -258,8 +258,9 @@ int nfn_mi355_lm_head_argmax_v1(
  * at 16 rows (glimmer_k_mmq.cu:1326-1328) and its only route for more rows is
  * the generic linear above.  mode selects the MFMA operand type. */
 enum {
-    NFN_MI355_GEMM_BF16 = 0, /* weights dequantized to bf16 in LDS, bf16 MFMA */
-    NFN_MI355_GEMM_INT8 = 1  /* activations int8 per 32 values, int8 MFMA     */
+    NFN_MI355_GEMM_F16 = 0, /* weights dequantized to fp16 in LDS, activations
+                               row-scaled fp16, fp16 MFMA, float accumulate */
+    NFN_MI355_GEMM_INT8 = 1 /* activations int8 per 32 values, int8 MFMA      */
 };
 int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(
     int64_t rows, int64_t input_dim, int64_t output_dim, int mode);

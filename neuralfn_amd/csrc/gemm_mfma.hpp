@@ -1,15 +1,16 @@
-// Prefill dequant-GEMM on the bf16 matrix cores (gemm_mfma.hip).
+// Prefill dequant-GEMM on the fp16 matrix cores (gemm_mfma.hip).
 #pragma once
 
 #include "common.hpp"
 
 namespace nfn {
 
-// Bytes of device workspace the bf16 path needs: a bf16 copy of the activations.
-std::int64_t gemm_bf16_workspace_bytes(std::int64_t rows, std::int64_t input_dim);
-bool gemm_bf16_supports(std::uint32_t encoding, std::int64_t input_dim);
+// Bytes of device workspace the fp16 path needs: a row-scaled fp16 copy of the
+// activations in whole 256-row tiles and one inverse scale per row.
+std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim);
+bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim);
 // output[rows, output_dim] = input[rows, input_dim] * W^T, float accumulation.
-void launch_gemm_bf16(const Descriptor& descriptor, const float* input, float* output,
+void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,
                       std::int64_t rows, void* workspace, hipStream_t stream);
 
 }  // namespace nfn

@@ -19,7 +19,7 @@ from . import kquant
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libnfn_mi355_tile_ops.so"
 INVALID = 1
 
-GEMM_BF16 = 0
+GEMM_F16 = 0
 GEMM_INT8 = 1
 
 
@@ -342,7 +342,7 @@ def lm_head_argmax(weight: PackedWeight, x, workspace=None):
     return indices, maxima
 
 
-def gemm(weight: PackedWeight, x, mode: int = GEMM_BF16, workspace=None, out=None):
+def gemm(weight: PackedWeight, x, mode: int = GEMM_F16, workspace=None, out=None):
     """nfn_mi355_k_quant_gemm_float32_v1: prefill dequant-GEMM, any row count."""
     import torch
     rows = x.shape[0]

@@ -445,7 +445,7 @@ def test_config4_mixed_formats_dispatch(cuda, oracle):
         assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE
 
 
-@pytest.mark.parametrize("mode", [tile_ops.GEMM_BF16, tile_ops.GEMM_INT8])
+@pytest.mark.parametrize("mode", [tile_ops.GEMM_F16, tile_ops.GEMM_INT8])
 @pytest.mark.parametrize("encoding", ALL_PACKED)
 def test_prefill_gemm_against_oracle(cuda, oracle, encoding, mode):
     rows, out_dim, in_dim = 160, 384, 1024
@@ -455,7 +455,7 @@ def test_prefill_gemm_against_oracle(cuda, oracle, encoding, mode):
     y = tile_ops.gemm(weight, to_device(x, cuda), mode).cpu().numpy()
     expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
     error = normalised_error(y, expected)
-    if mode == tile_ops.GEMM_BF16:
+    if mode == tile_ops.GEMM_F16:
         assert error <= TOLERANCE
     else:
         # int8 activations per 32 values are a separate numerics tier: compared
@@ -477,7 +477,7 @@ def test_prefill_gemm_full_size_row_subset(cuda, oracle):
     full = np.tile(packed.reshape(256, -1), (out_dim // 256, 1)).reshape(-1)
     x = kquant.synthetic_activations(92, rows, in_dim)
     weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, full, out_dim, in_dim)
-    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_BF16).cpu().numpy()
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
     expected = oracle.linear(kquant.Q4_K, packed, 256, in_dim, x)
     assert normalised_error(y[:, :256], expected) <= TOLERANCE
     # every 256-column stripe repeats the same weights
