@@ -7,6 +7,7 @@
 #include "gemv_dot.hpp"
 #include "gemm_mfma.hpp"
 #include "gemv_mfma.hpp"
+#include "gemv_q6.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
 
@@ -72,13 +73,15 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // kernel.  2..16 rows otherwise: the matrix-core kernel.  Encodings without
     // either: the float kernel.
     const bool one_row_arithmetic = rows == 1 || verifier;
-    ProjectionSet dot{}, matrix{}, exact{};
-    dot.input_dim = matrix.input_dim = exact.input_dim = input_dim;
+    ProjectionSet dot{}, dot6{}, matrix{}, exact{};
+    dot.input_dim = dot6.input_dim = matrix.input_dim = exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
         const std::uint32_t encoding = set.op[index].encoding;
         ProjectionSet* target = &exact;
         if (one_row_arithmetic && gemv_dot_supports(encoding, input_dim)) {
             target = &dot;
+        } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
+            target = &dot6;
         } else if (gemv_mfma_supports(encoding, input_dim)) {
             target = &matrix;
         }
@@ -86,6 +89,9 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     }
     if (dot.count > 0) {
         launch_gemv_dot(dot, first, second, prologue, rows, as_stream(stream));
+    }
+    if (dot6.count > 0) {
+        launch_gemv_q6(dot6, first, second, prologue, rows, as_stream(stream));
     }
     if (matrix.count > 0) {
         launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));
@@ -324,8 +330,11 @@ int nfn_native_tile_swiglu_float32(const float* gate, const float* up, float* ou
 std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
                                                          std::int64_t output_dim) {
     if (rows < 1 || rows > 8 || output_dim <= 0) return 0;
-    const std::int64_t raw =
-        rows * lm_head_f32_blocks(output_dim) * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+    // room for either kernel's per-workgroup candidates
+    const std::int64_t f32_groups = lm_head_f32_blocks(output_dim);
+    const std::int64_t q6_groups = lm_head_q6_groups(output_dim);
+    const std::int64_t raw = rows * (f32_groups > q6_groups ? f32_groups : q6_groups) *
+        static_cast<std::int64_t>(sizeof(LmHeadCandidate));
     return (raw + 255) & ~std::int64_t(255);
 }
 
@@ -342,8 +351,13 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
     const std::int64_t required =
         nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    launch_lm_head_f32(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
-                       output_indices, output_values, as_stream(cuda_stream));
+    if (gemv_q6_supports(normalized.encoding, normalized.input_dim)) {
+        launch_lm_head_q6(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
+                          output_indices, output_values, as_stream(cuda_stream));
+    } else {
+        launch_lm_head_f32(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
+                           output_indices, output_values, as_stream(cuda_stream));
+    }
     return launch_status();
 }
 

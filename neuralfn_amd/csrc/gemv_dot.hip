@@ -21,6 +21,7 @@
 // c = 256*hi + lo:  y += s*(d*sum_sub sc*dot(q, c) - dmin*sum_sub m*sum(c)).
 #include "common.hpp"
 #include "gemv_dot.hpp"
+#include "wave_rows.hpp"
 
 namespace nfn {
 
@@ -28,70 +29,9 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-#ifndef NFN_DOT_WAVES
-#define NFN_DOT_WAVES 8
-#endif
-#ifndef NFN_DOT_OCC
-#define NFN_DOT_OCC 32
-#endif
-constexpr int kDotWaves = NFN_DOT_WAVES;
+constexpr int kDotWaves = 8;
 constexpr int kDotThreads = kDotWaves * kWave;
-constexpr float kCodeRange = 32512.0f;  // 127*256: the high byte stays in [-127, 127]
-
-template <int CTRL>
-__device__ __forceinline__ int dpp_move(int value) {
-    return __builtin_amdgcn_update_dpp(0, value, CTRL, 0xF, 0xF, true);
-}
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float value) {
-    return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, value)));
-}
-
-constexpr int kQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
-constexpr int kQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
-constexpr int kHalfMirror = 0x141;  // lane k <-> 7-k within 8 lanes
-constexpr int kRowMirror = 0x140;   // lane k <-> 15-k within 16 lanes
-
-__device__ __forceinline__ float lane_value(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_move<kQuadXor1>(v));
-    v = fmaxf(v, dpp_move<kQuadXor2>(v));
-    v = fmaxf(v, dpp_move<kHalfMirror>(v));
-    v = fmaxf(v, dpp_move<kRowMirror>(v));
-    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
-                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
-}
-
-// Sum over the wave in a fixed order; the total is returned in every lane.
-__device__ __forceinline__ float wave_total(float v) {
-    v += dpp_move<kQuadXor1>(v);
-    v += dpp_move<kQuadXor2>(v);
-    v += dpp_move<kHalfMirror>(v);
-    v += dpp_move<kRowMirror>(v);
-    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
-}
-
-__device__ __forceinline__ std::uint32_t perm(std::uint32_t hi, std::uint32_t lo, std::uint32_t sel) {
-    return __builtin_amdgcn_perm(hi, lo, sel);
-}
-
-template <int P>
-__device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
-                                                   const float* __restrict__ second,
-                                                   std::int64_t column) {
-    float4 x = *reinterpret_cast<const float4*>(first + column);
-    if constexpr (P != kPlain) {
-        const float4 y = *reinterpret_cast<const float4*>(second + column);
-        x.x = apply_prologue<P>(x.x, y.x);
-        x.y = apply_prologue<P>(x.y, y.y);
-        x.z = apply_prologue<P>(x.z, y.z);
-        x.w = apply_prologue<P>(x.w, y.w);
-    }
-    return x;
-}
+constexpr int kWavesPerUnit = 32;  // waves the grid aims at per compute unit
 
 // LDS image of one token's activations for a K of `blocks` super-blocks:
 //   planes: eight arrays of `units` 16-byte slots, units = 4*blocks; unit
@@ -125,23 +65,10 @@ __device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, 
 // Quantize the 256 activations of block `block`, four per lane.
 __device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
                                                const TokenImage& image) {
-    const float local = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
-    const float maximum = wave_max(local);
-    const float inverse = maximum > 1.0e-30f ? kCodeRange * __builtin_amdgcn_rcpf(maximum) : 0.0f;
-    // 1.5*2^23 + 128: the low 16 bits of the sum's bit pattern are
-    // round-to-nearest-even(x*inverse) + 128 in two's complement.
-    constexpr float kMagic = 12582912.0f + 128.0f;
-    const std::uint32_t u0 = __float_as_uint(fmaf(x.x, inverse, kMagic));
-    const std::uint32_t u1 = __float_as_uint(fmaf(x.y, inverse, kMagic));
-    const std::uint32_t u2 = __float_as_uint(fmaf(x.z, inverse, kMagic));
-    const std::uint32_t u3 = __float_as_uint(fmaf(x.w, inverse, kMagic));
-    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped
-    const std::uint32_t p01 = perm(u1, u0, 0x05010400u);  // [u0.b0, u1.b0, u0.b1, u1.b1]
-    const std::uint32_t p23 = perm(u3, u2, 0x05010400u);
-    const std::uint32_t lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
-    const std::uint32_t hi = perm(p23, p01, 0x07060302u);
-    int sum = (__builtin_amdgcn_sdot4(static_cast<int>(hi), 0x01010101, 0, false) << 8) +
-        __builtin_amdgcn_sdot4(static_cast<int>(lo), 0x01010101, 0, false);
+    const ActivationCodes codes = encode_activations(x);
+    const std::uint32_t hi = codes.hi, lo = codes.lo;
+    const float maximum = codes.maximum;
+    int sum = codes.sum;
     sum += dpp_move<kQuadXor1>(sum);
     sum += dpp_move<kQuadXor2>(sum);
     sum += dpp_move<kHalfMirror>(sum);
@@ -164,58 +91,6 @@ struct Stage {
     uint4 h0, h1;  // Q5_K: the block's 32 high-bit bytes
 };
 
-// Projection `index` of the set, chosen with scalar selects from fields that
-// were all read with static offsets: a dynamically indexed read of the kernel
-// arguments is a dependent scalar load, and its first touch of a cache line
-// costs a trip to memory in the middle of the kernel.
-__device__ __forceinline__ Projection pick(const ProjectionSet& set, int index) {
-    Projection p = set.op[0];
-#pragma unroll
-    for (int k = 1; k < 4; ++k) {
-        const bool take = index == k;
-        p.data = take ? set.op[k].data : p.data;
-        p.output = take ? set.op[k].output : p.output;
-        p.output_dim = take ? set.op[k].output_dim : p.output_dim;
-        p.row_stride = take ? set.op[k].row_stride : p.row_stride;
-        p.first_tile = take ? set.op[k].first_tile : p.first_tile;
-    }
-    return p;
-}
-
-// Walks the (row, iteration) pairs of one wave without divisions: everything
-// here is uniform and lives in scalar registers.
-struct PairCursor {
-    int op;                   // projection index
-    Projection current;       // its fields
-    std::int64_t local_row;   // row inside that projection
-    int iteration;            // which 64-unit slice of the row
-    const std::uint8_t* row;  // first byte of the row
-
-    __device__ __forceinline__ void start(const ProjectionSet& set, std::int64_t global_row) {
-        op = 0;
-#pragma unroll
-        for (int index = 1; index < 4; ++index) {
-            if (index < set.count && global_row >= set.op[index].first_tile) op = index;
-        }
-        current = pick(set, op);
-        local_row = global_row - current.first_tile;
-        iteration = 0;
-        row = current.data + local_row * current.row_stride;
-    }
-    __device__ __forceinline__ void advance(const ProjectionSet& set, int iterations) {
-        if (++iteration < iterations) return;
-        iteration = 0;
-        ++local_row;
-        row += current.row_stride;
-        if (local_row == current.output_dim && op + 1 < set.count) {
-            ++op;
-            current = pick(set, op);
-            local_row = 0;
-            row = current.data;
-        }
-    }
-};
-
 template <std::uint32_t ENC, int T, int P>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
@@ -225,13 +100,6 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     constexpr int kQuants = kQ5 ? 48 : 16;
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
 
-#ifdef NFN_EXP_TIMELINE
-    unsigned long long stamp[8];
-    stamp[0] = __builtin_amdgcn_s_memrealtime();
-#define NFN_STAMP(i) stamp[i] = __builtin_amdgcn_s_memrealtime()
-#else
-#define NFN_STAMP(i)
-#endif
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int blocks = static_cast<int>(set.input_dim >> 8);
@@ -283,25 +151,18 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         if (--fetch_left > 0) fetch.advance(set, iterations);
     };
     Stage<kQ5> stage0, stage1;
-    NFN_STAMP(1);
     issue(stage0);
     issue(stage1);
-#ifdef NFN_EXP_TIMELINE
-    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    NFN_STAMP(2);
-#endif
 
     // (3) quantize; one barrier; after it the workgroup never synchronises again
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kDotWaves;
-#ifndef NFN_EXP_SKIP_QUANT
         if (record < records) {
             const int token = record / blocks;
             quantize_block(early[e], lane, record - token * blocks, blocks,
                            token_image(lds, token, blocks));
         }
-#endif
     }
     for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
         const int token = record / blocks;
@@ -311,13 +172,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
             static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
         quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
     }
-    NFN_STAMP(3);
     __syncthreads();
-    NFN_STAMP(4);
-#ifdef NFN_EXP_TIMELINE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    NFN_STAMP(5);
-#endif
 
     float acc[T];
 #pragma unroll
@@ -327,12 +182,6 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     work.start(set, min(row_begin, total_rows - 1));
     auto compute = [&](const Stage<kQ5>& stage) {
         const int iteration = work.iteration;
-#ifdef NFN_EXP_SKIP_COMPUTE
-        acc[0] += __uint_as_float((stage.q0.x ^ stage.q0.y ^ stage.q0.z ^ stage.q0.w ^ stage.q1.x ^ stage.q1.y ^ stage.q1.z ^ stage.q1.w ^ stage.header.x ^ stage.header.y ^ stage.header.z ^ stage.header.w) & 0x3fffffffu);
-        if (acc[0] == 1.2345f) lds[lane] = 1;
-        work.advance(set, iterations);
-        return;
-#endif
         const int raw_unit = iteration * kWave + lane;
         const bool live = raw_unit < units;
         const int unit = min(raw_unit, units - 1);
@@ -434,28 +283,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         if (n + 1 < total) compute(stage1);
         issue(stage1);
     }
-#ifdef NFN_EXP_TIMELINE
-    NFN_STAMP(6);
-    if (lane == 0 && wave == 0 && blockIdx.x < 500) {
-        unsigned* out = reinterpret_cast<unsigned*>(const_cast<float*>(first));
-        for (int i = 0; i < 7; ++i) out[blockIdx.x * 8 + i] = static_cast<unsigned>(stamp[i]);
-    }
-#endif
     (void)token_base_stride;
-}
-
-int compute_units() {
-    static const int count = [] {
-        int device = 0;
-        int value = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-            value <= 0) {
-            return 256;
-        }
-        return value;
-    }();
-    return count;
 }
 
 template <std::uint32_t ENC, int T, int P>
@@ -475,7 +303,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     (void)raised;
     // about one wave per SIMD lane group and row range: rows_per_wave keeps the
     // activation quantization (done once per workgroup) a small part of the work
-    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * NFN_DOT_OCC;
+    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * kWavesPerUnit;
     std::int64_t rows_per_wave = rows / waves_wanted;
     if (rows_per_wave < 1) rows_per_wave = 1;
     const std::int64_t groups = (rows + rows_per_wave * kDotWaves - 1) / (rows_per_wave * kDotWaves);

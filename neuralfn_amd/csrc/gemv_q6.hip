@@ -1,0 +1,422 @@
+// Q6_K decode GEMV on the vector ALUs (v_dot4_i32_i8), with an optional fused
+// argmax for the lm_head.
+//
+// One wave owns whole weight rows.  Its lanes split a row into units of 64
+// values: unit (block, half, sixteen) covers positions 16*sixteen .. +15 of all
+// four 32-value quarters of one 128-value half of a 210-byte block, which is
+// exactly three 16-byte loads (low nibbles of quarters 0/2, of quarters 1/3,
+// and the 2-bit tops of all four), so consecutive lanes read neighbouring
+// bytes and every loaded byte is used.  The blocks are 2-byte aligned only;
+// the 16-byte loads are issued unaligned.  Four int8 sub-scales (one per
+// quarter, the format has one per 16 values) and the block's fp16 scale come
+// with two small loads from the same cache lines.
+//
+// Activations become two int8 planes in LDS (16-bit fixed-point codes, one
+// scale per 256 values, quantized by the workgroup in the same launch), laid
+// out per unit so that consecutive lanes read consecutive 16-byte slots.  The
+// format's offset of 32 is applied through the per-16 sums of the codes:
+//   y += s*d * sum_quarter sc * (256*dot(q, hi) + dot(q, lo) - 32*sum(codes)).
+// The bracket is exact integer arithmetic; one float conversion and one fused
+// multiply-add per quarter, one fixed-order butterfly per row.
+//
+// Every row gets the same arithmetic whatever the number of tokens in the
+// launch, the contract of the reference's verifier entry points
+// (neuralfn/csrc/native_train/tile_ops.h:685-688).  With the argmax fused in,
+// each workgroup keeps the best (value, index) per token and the logits never
+// reach memory; the reference runs a linear and an argmax with a logits buffer
+// in between (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:4087-4151),
+// ties to the lowest index and NaN never winning as in
+// neuralfn/csrc/tile_cuda/kernels.cu:1564-1602.  Block layout:
+// neuralfn/csrc/native_gpt2/resident_glimmer.cpp:591-616.
+#include "common.hpp"
+#include "gemv_q6.hpp"
+#include "lm_head.hpp"
+#include "wave_rows.hpp"
+
+namespace nfn {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kWavesPerUnit = 32;  // waves the grid aims at per compute unit
+constexpr int kBlockBytes = 210;
+
+struct __attribute__((packed, aligned(2))) Unaligned16 {
+    std::uint32_t v[4];
+};
+struct __attribute__((packed, aligned(2))) Unaligned8 {
+    std::uint32_t v[2];
+};
+
+// LDS image of one token's activations for a K of `blocks` blocks:
+//   planes: eight arrays of `units` 16-byte slots, units = 4*blocks; unit
+//           u = 4*block + 2*half + sixteen reads slot u of array 2*quarter + plane
+//           (plane 0: high byte, 1: low byte of the codes)
+//   sums:   int32[4] per unit: the sum of the 16 codes of each quarter
+//   scale:  float per block
+struct TokenImage {
+    std::uint8_t* planes;
+    int* sums;
+    float* scale;
+};
+
+constexpr int kImageBytesPerBlock = 4 * 128 + 4 * 16 + 16;
+
+__host__ __device__ constexpr int token_image_bytes(std::int64_t blocks) {
+    return static_cast<int>(blocks * kImageBytesPerBlock);
+}
+
+__device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, int blocks) {
+    std::uint8_t* base = lds + token * token_image_bytes(blocks);
+    TokenImage image;
+    image.planes = base;
+    image.sums = reinterpret_cast<int*>(base + blocks * 512);
+    image.scale = reinterpret_cast<float*>(base + blocks * 576);
+    return image;
+}
+
+// Quantize the 256 activations of block `block`, four per lane: lane L holds
+// positions 4L..4L+3 = half L/32, quarter (L/8)%4, sixteen (L/4)%2, bytes 4*(L%4)..
+__device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
+                                               const TokenImage& image) {
+    const ActivationCodes codes = encode_activations(x);
+    int sum = codes.sum;
+    sum += dpp_move<kQuadXor1>(sum);
+    sum += dpp_move<kQuadXor2>(sum);
+    const int units = 4 * blocks;
+    const int quarter = (lane >> 3) & 3;
+    const int unit = 4 * block + 2 * (lane >> 5) + ((lane >> 2) & 1);
+    std::uint8_t* slot = image.planes + (2 * quarter * units + unit) * 16 + (lane & 3) * 4;
+    *reinterpret_cast<std::uint32_t*>(slot) = codes.hi;
+    *reinterpret_cast<std::uint32_t*>(slot + units * 16) = codes.lo;
+    if ((lane & 3) == 0) image.sums[unit * 4 + quarter] = sum;
+    if (lane == 0) image.scale[block] = codes.maximum * (1.0f / kCodeRange);
+}
+
+struct Stage {
+    Unaligned16 low_a;   // low nibbles: quarter 0, high nibbles: quarter 2
+    Unaligned16 low_b;   // low nibbles: quarter 1, high nibbles: quarter 3
+    Unaligned16 top;     // two bits per quarter
+    Unaligned8 scales;   // the eight int8 sub-scales of the half
+    std::uint32_t d_bits;
+};
+
+__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
+                                       std::int64_t& best_index) {
+    if (value > best_value || (value == best_value && index < best_index)) {
+        best_value = value;
+        best_index = index;
+    }
+}
+
+template <int T, int P, bool ARGMAX>
+__global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
+    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
+    int tokens, std::int64_t total_rows, int rows_per_wave,
+    LmHeadCandidate* __restrict__ candidates) {
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int blocks = static_cast<int>(set.input_dim >> 8);
+    const int units = 4 * blocks;
+    const int iterations = (units + kWave - 1) / kWave;
+    const int token0 = blockIdx.y * T;
+    const int pass_tokens = min(tokens - token0, T);
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_second =
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+
+    // rows of this wave: a contiguous range
+    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kWaves + wave;
+    const std::int64_t row_begin = wave_index * rows_per_wave;
+    const int row_count = static_cast<int>(max(
+        static_cast<std::int64_t>(0),
+        min(static_cast<std::int64_t>(rows_per_wave), total_rows - row_begin)));
+    const int total = row_count * iterations;
+
+    // (1) activations of the first records this wave quantizes: loaded first so
+    // that their short latency does not queue behind the weight loads.  All
+    // loads are unconditional (clamped indices) to keep the load counters exact.
+    const int records = pass_tokens * blocks;
+    constexpr int kEarly = 4;
+    float4 early[kEarly];
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = min(wave + e * kWaves, records - 1);
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        early[e] = load_activations<P>(
+            pass_first, pass_second,
+            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+    }
+
+    // (2) weight loads of the first two (row, slice) pairs
+    PairCursor fetch;
+    fetch.start(set, min(row_begin, total_rows - 1));
+    int fetch_left = total;  // pairs not fetched yet; the cursor rests on the last one
+    auto issue = [&](Stage& stage) {
+        const int unit = min(fetch.iteration * kWave + lane, units - 1);
+        const std::uint8_t* block = fetch.row + (unit >> 2) * kBlockBytes;
+        const int half = (unit >> 1) & 1;
+        const int sixteen = unit & 1;
+        const std::uint8_t* low = block + half * 64 + sixteen * 16;
+        stage.low_a = *reinterpret_cast<const Unaligned16*>(low);
+        stage.low_b = *reinterpret_cast<const Unaligned16*>(low + 32);
+        stage.top = *reinterpret_cast<const Unaligned16*>(block + 128 + half * 32 + sixteen * 16);
+        stage.scales = *reinterpret_cast<const Unaligned8*>(block + 192 + half * 8);
+        stage.d_bits = *reinterpret_cast<const std::uint16_t*>(block + 208);
+        if (--fetch_left > 0) fetch.advance(set, iterations);
+    };
+    Stage stage0, stage1;
+    issue(stage0);
+    issue(stage1);
+
+    // (3) quantize; one barrier
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = wave + e * kWaves;
+        if (record < records) {
+            const int token = record / blocks;
+            quantize_block(early[e], lane, record - token * blocks, blocks,
+                           token_image(lds, token, blocks));
+        }
+    }
+    for (int record = wave + kEarly * kWaves; record < records; record += kWaves) {
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        const float4 x = load_activations<P>(
+            pass_first, pass_second,
+            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+    }
+    __syncthreads();
+
+    float acc[T];
+    float best_value[T];
+    std::int64_t best_index[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        acc[t] = 0.0f;
+        best_value[t] = -INFINITY;
+        best_index[t] = 0;
+    }
+
+    PairCursor work;
+    work.start(set, min(row_begin, total_rows - 1));
+    auto compute = [&](const Stage& stage) {
+        const int iteration = work.iteration;
+        const int raw_unit = iteration * kWave + lane;
+        const bool live = raw_unit < units;
+        const int unit = min(raw_unit, units - 1);
+        const int block = unit >> 2;
+        const int sixteen = unit & 1;
+
+        // 6-bit codes of the four quarters, four bytes per word
+        std::uint32_t q[4][4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const std::uint32_t a = stage.low_a.v[w], b = stage.low_b.v[w], h = stage.top.v[w];
+            q[0][w] = (a & 0x0f0f0f0fu) | ((h & 0x03030303u) << 4);
+            q[1][w] = (b & 0x0f0f0f0fu) | ((h & 0x0c0c0c0cu) << 2);
+            q[2][w] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+            q[3][w] = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+        }
+        // sub-scale of quarter k: byte 2*k + sixteen of the half's eight
+        const std::uint32_t s01 = stage.scales.v[0] >> (8 * sixteen);
+        const std::uint32_t s23 = stage.scales.v[1] >> (8 * sixteen);
+        const float scale_q[4] = {
+            static_cast<float>(static_cast<std::int8_t>(s01 & 0xffu)),
+            static_cast<float>(static_cast<std::int8_t>((s01 >> 16) & 0xffu)),
+            static_cast<float>(static_cast<std::int8_t>(s23 & 0xffu)),
+            static_cast<float>(static_cast<std::int8_t>((s23 >> 16) & 0xffu))};
+        const float d = half_bits_to_float(stage.d_bits);
+
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const TokenImage image = token_image(lds, t, blocks);
+            const std::uint8_t* slot = image.planes + unit * 16;
+            const int stride = units * 16;
+            const v4i sums = *reinterpret_cast<const v4i*>(image.sums + unit * 4);
+            float unit_value = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const v4i hi = *reinterpret_cast<const v4i*>(slot + (2 * k) * stride);
+                const v4i lo = *reinterpret_cast<const v4i*>(slot + (2 * k + 1) * stride);
+                int dot_hi = 0, dot_lo = 0;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    dot_hi = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), hi[w], dot_hi, false);
+                    dot_lo = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), lo[w], dot_lo, false);
+                }
+                // |256*dot_hi + dot_lo| < 2^26 and 32*|sum| < 2^25: exact in int32
+                const int bracket = (dot_hi << 8) + dot_lo - (sums[k] << 5);
+                unit_value = fmaf(scale_q[k], static_cast<float>(bracket), unit_value);
+            }
+            const float scale = image.scale[block];
+            acc[t] = fmaf(live ? scale * d : 0.0f, unit_value, acc[t]);
+        }
+
+        if (iteration == iterations - 1) {
+            // the row is complete: fixed-order butterfly
+            const std::int64_t output_dim = work.current.output_dim;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const float total_value = wave_total(acc[t]);
+                if constexpr (ARGMAX) {
+                    // rows come in increasing order: a strict comparison keeps the lowest index
+                    if (total_value > best_value[t]) {
+                        best_value[t] = total_value;
+                        best_index[t] = work.local_row;
+                    }
+                } else {
+                    float* output = work.current.output + work.local_row;
+                    if (lane == 0 && t < pass_tokens) {
+                        output[static_cast<std::int64_t>(token0 + t) * output_dim] = total_value;
+                    }
+                }
+                acc[t] = 0.0f;
+            }
+        }
+        work.advance(set, iterations);
+    };
+
+    for (int n = 0; n < total; n += 2) {
+        compute(stage0);
+        issue(stage0);
+        if (n + 1 < total) compute(stage1);
+        issue(stage1);
+    }
+
+    if constexpr (ARGMAX) {
+        // best of the workgroup per token: waves through LDS (the images are no longer needed)
+        __syncthreads();
+        float* values = reinterpret_cast<float*>(lds);
+        std::int64_t* indices = reinterpret_cast<std::int64_t*>(lds + kWaves * T * 4);
+        if (lane == 0) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                values[wave * T + t] = best_value[t];
+                indices[wave * T + t] = best_index[t];
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x < static_cast<unsigned>(pass_tokens)) {
+            const int t = threadIdx.x;
+            float value = values[t];
+            std::int64_t index = indices[t];
+            for (int w = 1; w < kWaves; ++w) better(values[w * T + t], indices[w * T + t], value, index);
+            LmHeadCandidate candidate;
+            candidate.index = index;
+            candidate.value = value;
+            candidate.pad = 0;
+            candidates[static_cast<std::int64_t>(token0 + t) * gridDim.x + blockIdx.x] = candidate;
+        }
+    }
+}
+
+struct Geometry {
+    std::int64_t rows_per_wave;
+    std::int64_t groups;
+};
+
+Geometry geometry(std::int64_t rows) {
+    // about kWavesPerUnit waves per compute unit: the activation quantization
+    // (done once per workgroup) stays a small part of a workgroup's work
+    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * kWavesPerUnit;
+    Geometry g;
+    g.rows_per_wave = rows / waves_wanted;
+    if (g.rows_per_wave < 1) g.rows_per_wave = 1;
+    g.groups = (rows + g.rows_per_wave * kWaves - 1) / (g.rows_per_wave * kWaves);
+    return g;
+}
+
+template <int T, int P, bool ARGMAX>
+void launch_variant(ProjectionSet set, const float* first, const float* second, int tokens,
+                    LmHeadCandidate* candidates, hipStream_t stream) {
+    std::int64_t rows = 0;
+    for (int index = 0; index < set.count; ++index) {
+        set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
+        rows += set.op[index].output_dim;
+    }
+    std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8);
+    if (lds < 1024) lds = 1024;  // room for the per-wave candidates
+    auto kernel = gemv_q6_kernel<T, P, ARGMAX>;
+    static const bool raised =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+    (void)raised;
+    const Geometry g = geometry(rows);
+    const int passes = (tokens + T - 1) / T;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(kThreads), lds,
+                       stream, set, first, second, tokens, rows, static_cast<int>(g.rows_per_wave),
+                       candidates);
+}
+
+template <int P, bool ARGMAX>
+void launch_tokens(const ProjectionSet& set, const float* first, const float* second, int tokens,
+                   LmHeadCandidate* candidates, hipStream_t stream) {
+    // the token images of one pass must fit in LDS
+    const std::int64_t image = token_image_bytes(set.input_dim >> 8);
+    int capacity = static_cast<int>((150 * 1024) / image);
+    if (capacity > 4) capacity = 4;
+    const int per_pass = tokens < capacity ? tokens : capacity;
+    if (per_pass <= 1) {
+        launch_variant<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    } else if (per_pass == 2 || capacity < 4) {
+        launch_variant<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    } else {
+        launch_variant<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    }
+}
+
+}  // namespace
+
+bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim) {
+    return encoding == kEncQ6K && input_dim % 256 == 0 &&
+        token_image_bytes(input_dim >> 8) <= 150 * 1024;
+}
+
+void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
+                    int prologue, std::int64_t rows, hipStream_t stream) {
+    ProjectionSet group{};
+    group.input_dim = set.input_dim;
+    for (int index = 0; index < set.count; ++index) {
+        if (set.op[index].encoding == kEncQ6K) group.op[group.count++] = set.op[index];
+    }
+    if (group.count == 0) return;
+    const int tokens = static_cast<int>(rows);
+    switch (prologue) {
+        case kGated:
+            launch_tokens<kGated, false>(group, first, second, tokens, nullptr, stream);
+            break;
+        case kSwiGlu:
+            launch_tokens<kSwiGlu, false>(group, first, second, tokens, nullptr, stream);
+            break;
+        default:
+            launch_tokens<kPlain, false>(group, first, second, tokens, nullptr, stream);
+            break;
+    }
+}
+
+std::int64_t lm_head_q6_groups(std::int64_t output_dim) { return geometry(output_dim).groups; }
+
+void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                       LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
+                       hipStream_t stream) {
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = descriptor.input_dim;
+    set.op[0].data = descriptor.data;
+    set.op[0].output = nullptr;
+    set.op[0].output_dim = descriptor.output_dim;
+    set.op[0].row_stride = descriptor.row_stride_bytes;
+    set.op[0].encoding = descriptor.encoding;
+    launch_tokens<kPlain, true>(set, input, nullptr, static_cast<int>(rows), candidates, stream);
+    launch_lm_head_final(candidates, lm_head_q6_groups(descriptor.output_dim), indices, maxima,
+                         rows, stream);
+}
+
+}  // namespace nfn

@@ -1,0 +1,22 @@
+// Q6_K decode GEMV on the vector ALUs and the lm_head with fused argmax (gemv_q6.hip).
+#pragma once
+
+#include "common.hpp"
+#include "lm_head.hpp"
+
+namespace nfn {
+
+bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim);
+
+// The Q6_K projections of `set`, rows 1..16; activations are quantized inside
+// the launch, no workspace.
+void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
+                    int prologue, std::int64_t rows, hipStream_t stream);
+
+// Workgroups of the fused lm_head launch = candidates per input row.
+std::int64_t lm_head_q6_groups(std::int64_t output_dim);
+void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                       LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
+                       hipStream_t stream);
+
+}  // namespace nfn

@@ -110,6 +110,13 @@ __global__ __launch_bounds__(256) void lm_head_final_kernel(
     }
 }
 
+void launch_lm_head_final(const LmHeadCandidate* candidates, std::int64_t candidate_count,
+                          std::int64_t* indices, float* maxima, std::int64_t rows,
+                          hipStream_t stream) {
+    hipLaunchKernelGGL(lm_head_final_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
+                       stream, candidates, candidate_count, indices, maxima);
+}
+
 std::int64_t lm_head_f32_blocks(std::int64_t output_dim) {
     // 16 vocabulary rows per wave, 64 per workgroup.
     return (output_dim + 63) / 64;
@@ -137,8 +144,7 @@ void launch_lm_head_f32(const Descriptor& descriptor, const float* input, std::i
         hipLaunchKernelGGL((lm_head_partial_kernel<8>), grid, block, 0, stream, op,
                            descriptor.input_dim, input, rows, 16, candidates);
     }
-    hipLaunchKernelGGL(lm_head_final_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
-                       stream, candidates, blocks, indices, maxima);
+    launch_lm_head_final(candidates, blocks, indices, maxima, rows, stream);
 }
 
 }  // namespace nfn

@@ -13,6 +13,11 @@ struct LmHeadCandidate {
     std::uint32_t pad;
 };
 
+// Pass 2: one workgroup per input row reduces `candidate_count` candidates.
+void launch_lm_head_final(const LmHeadCandidate* candidates, std::int64_t candidate_count,
+                          std::int64_t* indices, float* maxima, std::int64_t rows,
+                          hipStream_t stream);
+
 std::int64_t lm_head_f32_blocks(std::int64_t output_dim);
 void launch_lm_head_f32(const Descriptor& descriptor, const float* input, std::int64_t rows,
                         LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,

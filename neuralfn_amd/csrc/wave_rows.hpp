@@ -1,0 +1,165 @@
+// Pieces shared by the wave-per-row decode kernels (gemv_dot.hip, gemv_q6.hip):
+// fixed-order wave reductions on DPP, the activation load with its fused
+// prologue, and the cursor that walks a wave's (row, slice) pairs.
+#pragma once
+
+#include "common.hpp"
+
+namespace nfn {
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int value) {
+    return __builtin_amdgcn_update_dpp(0, value, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float value) {
+    return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, value)));
+}
+
+constexpr int kQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int kHalfMirror = 0x141;  // lane k <-> 7-k within 8 lanes
+constexpr int kRowMirror = 0x140;   // lane k <-> 15-k within 16 lanes
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_move<kQuadXor1>(v));
+    v = fmaxf(v, dpp_move<kQuadXor2>(v));
+    v = fmaxf(v, dpp_move<kHalfMirror>(v));
+    v = fmaxf(v, dpp_move<kRowMirror>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
+                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
+// Sum over the wave in a fixed order; the total is returned in every lane.
+__device__ __forceinline__ float wave_total(float v) {
+    v += dpp_move<kQuadXor1>(v);
+    v += dpp_move<kQuadXor2>(v);
+    v += dpp_move<kHalfMirror>(v);
+    v += dpp_move<kRowMirror>(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+
+__device__ __forceinline__ std::uint32_t perm(std::uint32_t hi, std::uint32_t lo, std::uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+constexpr float kCodeRange = 32512.0f;  // 127*256: the high byte stays in [-127, 127]
+
+// Four activations of one lane as 16-bit fixed-point codes, code = x * 32512 /
+// (largest magnitude among the wave's 256 values), rounded to nearest even and
+// split into two int8 planes: code = 256*hi + lo with lo in [-128, 127].
+struct ActivationCodes {
+    std::uint32_t hi, lo;  // four bytes each, value order
+    int sum;               // of this lane's four codes
+    float maximum;         // the wave's largest magnitude; scale = maximum / 32512
+};
+
+__device__ __forceinline__ ActivationCodes encode_activations(float4 x) {
+    const float local = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+    ActivationCodes codes;
+    codes.maximum = wave_max(local);
+    const float inverse =
+        codes.maximum > 1.0e-30f ? kCodeRange * __builtin_amdgcn_rcpf(codes.maximum) : 0.0f;
+    // 1.5*2^23 + 128: the low 16 bits of the sum's bit pattern are
+    // round-to-nearest-even(x*inverse) + 128 in two's complement.
+    constexpr float kMagic = 12582912.0f + 128.0f;
+    const std::uint32_t u0 = __float_as_uint(fmaf(x.x, inverse, kMagic));
+    const std::uint32_t u1 = __float_as_uint(fmaf(x.y, inverse, kMagic));
+    const std::uint32_t u2 = __float_as_uint(fmaf(x.z, inverse, kMagic));
+    const std::uint32_t u3 = __float_as_uint(fmaf(x.w, inverse, kMagic));
+    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped
+    const std::uint32_t p01 = perm(u1, u0, 0x05010400u);  // [u0.b0, u1.b0, u0.b1, u1.b1]
+    const std::uint32_t p23 = perm(u3, u2, 0x05010400u);
+    codes.lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
+    codes.hi = perm(p23, p01, 0x07060302u);
+    codes.sum = (__builtin_amdgcn_sdot4(static_cast<int>(codes.hi), 0x01010101, 0, false) << 8) +
+        __builtin_amdgcn_sdot4(static_cast<int>(codes.lo), 0x01010101, 0, false);
+    return codes;
+}
+
+template <int P>
+__device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
+                                                   const float* __restrict__ second,
+                                                   std::int64_t column) {
+    float4 x = *reinterpret_cast<const float4*>(first + column);
+    if constexpr (P != kPlain) {
+        const float4 y = *reinterpret_cast<const float4*>(second + column);
+        x.x = apply_prologue<P>(x.x, y.x);
+        x.y = apply_prologue<P>(x.y, y.y);
+        x.z = apply_prologue<P>(x.z, y.z);
+        x.w = apply_prologue<P>(x.w, y.w);
+    }
+    return x;
+}
+
+// Projection `index` of the set, chosen with scalar selects from fields that
+// were all read with static offsets: a dynamically indexed read of the kernel
+// arguments is a dependent scalar load, and its first touch of a cache line
+// costs a trip to memory in the middle of the kernel.
+__device__ __forceinline__ Projection pick(const ProjectionSet& set, int index) {
+    Projection p = set.op[0];
+#pragma unroll
+    for (int k = 1; k < 4; ++k) {
+        const bool take = index == k;
+        p.data = take ? set.op[k].data : p.data;
+        p.output = take ? set.op[k].output : p.output;
+        p.output_dim = take ? set.op[k].output_dim : p.output_dim;
+        p.row_stride = take ? set.op[k].row_stride : p.row_stride;
+        p.first_tile = take ? set.op[k].first_tile : p.first_tile;
+    }
+    return p;
+}
+
+// Walks the (row, iteration) pairs of one wave without divisions: everything
+// here is uniform and lives in scalar registers.
+struct PairCursor {
+    int op;                   // projection index
+    Projection current;       // its fields
+    std::int64_t local_row;   // row inside that projection
+    int iteration;            // which 64-unit slice of the row
+    const std::uint8_t* row;  // first byte of the row
+
+    __device__ __forceinline__ void start(const ProjectionSet& set, std::int64_t global_row) {
+        op = 0;
+#pragma unroll
+        for (int index = 1; index < 4; ++index) {
+            if (index < set.count && global_row >= set.op[index].first_tile) op = index;
+        }
+        current = pick(set, op);
+        local_row = global_row - current.first_tile;
+        iteration = 0;
+        row = current.data + local_row * current.row_stride;
+    }
+    __device__ __forceinline__ void advance(const ProjectionSet& set, int iterations) {
+        if (++iteration < iterations) return;
+        iteration = 0;
+        ++local_row;
+        row += current.row_stride;
+        if (local_row == current.output_dim && op + 1 < set.count) {
+            ++op;
+            current = pick(set, op);
+            local_row = 0;
+            row = current.data;
+        }
+    }
+};
+
+inline int compute_units() {
+    static const int count = [] {
+        int device = 0;
+        int value = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            value <= 0) {
+            return 256;
+        }
+        return value;
+    }();
+    return count;
+}
+
+}  // namespace nfn
