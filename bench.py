@@ -49,6 +49,9 @@ def parse_args() -> argparse.Namespace:
     parser.add_argument("--no-extras", action="store_true",
                         help="skip the lm_head and prefill side measurements")
     parser.add_argument("--no-graph", action="store_true", help="enqueue directly, no HIP graph")
+    parser.add_argument("--traffic-probe", action="store_true",
+                        help="for a counter run: one plain copy of 256 MiB, then one eager step; "
+                             "no timing, no JSON")
     return parser.parse_args()
 
 
@@ -151,6 +154,22 @@ def time_replays(run, steps: int, warmup: int) -> float:
     return start.elapsed_time(stop) / steps
 
 
+def time_graph(run, stream, steps: int, warmup: int) -> float:
+    """Milliseconds per call of run(), captured once into a HIP graph and replayed.
+
+    A call is a few dependent launches; replaying them from a graph takes the
+    host's launch latency between them out of the measurement, as the decode
+    loop's own graph replay does.
+    """
+    import torch
+    run()  # eager: loads code objects, and nothing is allocated during capture
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        run()
+    return time_replays(graph.replay, steps, warmup)
+
+
 def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
     """The reference's CPU matmul on this host, on as many layers as fit the budget."""
     from neuralfn_amd import kquant
@@ -170,14 +189,18 @@ def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
 
     done = 0
     began = time.perf_counter()
-    for index, layer in enumerate(host_layers):
-        x = hidden[index * rows:(index + 1) * rows]
-        a = attention[index * rows:(index + 1) * rows]
-        for name in ("q", "k", "v"):
-            run(name, layer[name], x)
-        run("o", layer["o"], a)
-        done += 1
-        if time.perf_counter() - began > budget_seconds:
+    minimum_seconds = 10.0
+    while True:
+        for index, layer in enumerate(host_layers):
+            x = hidden[index * rows:(index + 1) * rows]
+            a = attention[index * rows:(index + 1) * rows]
+            for name in ("q", "k", "v"):
+                run(name, layer[name], x)
+            run("o", layer["o"], a)
+            done += 1
+            if time.perf_counter() - began > budget_seconds:
+                break
+        if time.perf_counter() - began > minimum_seconds:
             break
     elapsed = time.perf_counter() - began
     cores = kquant_oracle.worker_count(ATTN_DIM, 128)
@@ -186,7 +209,8 @@ def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
         "unit": "GB/s",
         "cores": cores,
         "kind": kind,
-        "sample": f"{done} of {len(host_layers)} layers (Q,K,V,O at rows={rows}) in {elapsed:.2f} s; "
+        "sample": f"{done} layer passes (Q,K,V,O at rows={rows}) over the {len(host_layers)} "
+                  f"layers of the workload in {elapsed:.2f} s; "
                   f"{done * rows / elapsed:.3f} layer-tokens/s",
     }
 
@@ -209,7 +233,7 @@ def random_packed_on_device(encoding: int, out_dim: int, in_dim: int, device, se
     return tile_ops.PackedWeight(encoding, out_dim, in_dim, blocks.reshape(-1))
 
 
-def lm_head_extra(device, steps: int, warmup: int) -> dict:
+def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
     import torch
     from neuralfn_amd import kquant, tile_ops
     weight = random_packed_on_device(kquant.Q6_K, VOCAB, MODEL_DIM, device, 7)
@@ -218,7 +242,10 @@ def lm_head_extra(device, steps: int, warmup: int) -> dict:
         x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
         nbytes = tile_ops.load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, VOCAB)
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        ms = time_replays(lambda: tile_ops.lm_head_argmax(weight, x, workspace), steps, warmup)
+        indices = torch.empty(rows, dtype=torch.int64, device=device)
+        values = torch.empty(rows, dtype=torch.float32, device=device)
+        ms = time_graph(lambda: tile_ops.lm_head_argmax(weight, x, workspace, indices, values),
+                        stream, steps, warmup)
         traffic = weight.nbytes + rows * MODEL_DIM * 4 + rows * 12
         result[f"rows{rows}"] = {"ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
                                  "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
@@ -226,13 +253,13 @@ def lm_head_extra(device, steps: int, warmup: int) -> dict:
     return {"workload": f"Q6_K lm_head {MODEL_DIM}->{VOCAB}, fused argmax", **result}
 
 
-def prefill_extra(device, steps: int, warmup: int) -> dict:
+def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     import torch
     from neuralfn_amd import kquant, tile_ops
     gate = random_packed_on_device(kquant.Q4_K, FFN_DIM, MODEL_DIM, device, 8)
     down = random_packed_on_device(kquant.Q4_K, MODEL_DIM, FFN_DIM, device, 9)
     result = {}
-    for mode, name in ((tile_ops.GEMM_F16, "f16"), (tile_ops.GEMM_INT8, "int8")):
+    for mode, name in ((tile_ops.GEMM_F16, "f16"),):
         for rows in (512, 2048):
             x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
             h = torch.from_numpy(kquant.synthetic_activations(32, rows, FFN_DIM)).to(device)
@@ -241,16 +268,17 @@ def prefill_extra(device, steps: int, warmup: int) -> dict:
                 nbytes = tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
                     rows, weight.input_dim, weight.output_dim, mode)
                 workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-                ms = time_replays(
-                    lambda: tile_ops.gemm(weight, source, mode, workspace, out),
-                    max(3, steps // 4), max(1, warmup // 2))
+                ms = time_graph(
+                    lambda: tile_ops.gemm(weight, source, mode, workspace, out), stream,
+                    max(5, steps // 2), max(2, warmup // 2))
                 flops = 2.0 * rows * weight.input_dim * weight.output_dim
                 tflops = flops / ms / 1e9
                 result[f"{name}_{label}_M{rows}"] = {
                     "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
                     "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS[name], 4),
                     "tokens/s": round(rows / ms * 1e3, 1)}
-    return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}", **result}
+    return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}, dequant-GEMM "
+                        "incl. activation conversion", **result}
 
 
 def main() -> int:
@@ -273,6 +301,22 @@ def main() -> int:
     layers, host_layers = make_layers(args.layers, device)
     setup_seconds = time.perf_counter() - began
     step = DecodeStep(layers, args.rows, device)
+
+    if args.traffic_probe:
+        # a copy kernel of known size calibrates the byte counters, then the
+        # launches of one step follow as separate dispatches
+        source = torch.empty(256 << 20, dtype=torch.uint8, device=device)
+        target = torch.empty_like(source)
+        source.fill_(1)
+        torch.cuda.synchronize()
+        target.copy_(source)
+        torch.cuda.synchronize()
+        step.enqueue(int(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        print(f"traffic probe: copy of {source.numel()} bytes, then {step.launches_per_step} "
+              f"launches of {layer_algorithmic_bytes(args.rows) // 2} bytes on average",
+              file=sys.stderr)
+        return 0
 
     stream = torch.cuda.Stream()
     graph = None
@@ -334,8 +378,8 @@ def main() -> int:
     if not args.no_extras:
         try:
             with torch.cuda.stream(stream):
-                record["lm_head"] = lm_head_extra(device, args.steps, args.warmup)
-                record["prefill"] = prefill_extra(device, args.steps, args.warmup)
+                record["lm_head"] = lm_head_extra(device, stream, args.steps, args.warmup)
+                record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
             record["extras_error"] = repr(error)
     if not args.no_cpu_baseline:

@@ -260,7 +260,8 @@ int nfn_mi355_lm_head_argmax_v1(
 enum {
     NFN_MI355_GEMM_F16 = 0, /* weights dequantized to fp16 in LDS, activations
                                row-scaled fp16, fp16 MFMA, float accumulate */
-    NFN_MI355_GEMM_INT8 = 1 /* activations int8 per 32 values, int8 MFMA      */
+    NFN_MI355_GEMM_INT8 = 1 /* reserved: int8 activations per 32 values on the
+                               int8 MFMA; refused (workspace query returns 0) */
 };
 int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(
     int64_t rows, int64_t input_dim, int64_t output_dim, int mode);

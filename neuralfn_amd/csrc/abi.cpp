@@ -364,10 +364,10 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
 std::int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(std::int64_t rows, std::int64_t input_dim,
                                                        std::int64_t output_dim, int mode) {
     if (rows <= 0 || input_dim <= 0 || input_dim % 256 != 0 || output_dim <= 0 ||
-        (mode != NFN_MI355_GEMM_F16 && mode != NFN_MI355_GEMM_INT8)) {
+        mode != NFN_MI355_GEMM_F16) {
         return 0;
     }
-    return mode == NFN_MI355_GEMM_F16 ? gemm_f16_workspace_bytes(rows, input_dim) : 256;
+    return gemm_f16_workspace_bytes(rows, input_dim);
 }
 
 int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float* input,
@@ -384,8 +384,7 @@ int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float*
     const std::int64_t required = nfn_mi355_k_quant_gemm_workspace_bytes_v1(
         rows, normalized.input_dim, normalized.output_dim, mode);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    if (mode == NFN_MI355_GEMM_F16 &&
-        gemm_f16_supports(normalized.encoding, normalized.input_dim)) {
+    if (gemm_f16_supports(normalized.encoding, normalized.input_dim)) {
         if (reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) return kInvalid;
         launch_gemm_f16(normalized, input, output, rows, workspace, as_stream(cuda_stream));
         return launch_status();

@@ -41,7 +41,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
-constexpr int kWavesPerUnit = 32;  // waves the grid aims at per compute unit
+constexpr int kWavesPerUnit = 64;  // waves the grid aims at per compute unit
 constexpr int kBlockBytes = 210;
 
 struct __attribute__((packed, aligned(2))) Unaligned16 {

@@ -323,7 +323,7 @@ def swiglu(gate, up):
     return out
 
 
-def lm_head_argmax(weight: PackedWeight, x, workspace=None):
+def lm_head_argmax(weight: PackedWeight, x, workspace=None, indices=None, maxima=None):
     """nfn_mi355_lm_head_argmax_v1: GEMV + argmax, logits never stored."""
     import torch
     rows = x.shape[0]
@@ -333,8 +333,10 @@ def lm_head_argmax(weight: PackedWeight, x, workspace=None):
         if nbytes <= 0:
             raise ValueError("lm_head_argmax supports 1..8 rows")
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-    indices = torch.empty(rows, dtype=torch.int64, device=x.device)
-    maxima = torch.empty(rows, dtype=torch.float32, device=x.device)
+    if indices is None:
+        indices = torch.empty(rows, dtype=torch.int64, device=x.device)
+    if maxima is None:
+        maxima = torch.empty(rows, dtype=torch.float32, device=x.device)
     descriptor = weight.descriptor(stream)
     check(load().nfn_mi355_lm_head_argmax_v1(
         ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), rows,

@@ -445,27 +445,51 @@ def test_config4_mixed_formats_dispatch(cuda, oracle):
         assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE
 
 
-@pytest.mark.parametrize("mode", [tile_ops.GEMM_F16, tile_ops.GEMM_INT8])
 @pytest.mark.parametrize("encoding", ALL_PACKED)
-def test_prefill_gemm_against_oracle(cuda, oracle, encoding, mode):
+def test_prefill_gemm_against_oracle(cuda, oracle, encoding):
+    # 160 rows: one full and one ragged 256-row tile is not covered here but by
+    # the ragged test below; 384 columns = three 128-column tiles
     rows, out_dim, in_dim = 160, 384, 1024
     packed = kquant.quantize(encoding, kquant.synthetic_weights(70 + encoding, out_dim, in_dim))
     x = kquant.synthetic_activations(71, rows, in_dim)
     weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
-    y = tile_ops.gemm(weight, to_device(x, cuda), mode).cpu().numpy()
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
     expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
-    error = normalised_error(y, expected)
-    if mode == tile_ops.GEMM_F16:
-        assert error <= TOLERANCE
-    else:
-        # int8 activations per 32 values are a separate numerics tier: compared
-        # with the Q8_1-activation oracle at the reference's own tolerance
-        # (probe :1444-1458), and reported against the float oracle.
-        codes, scales, _ = oracle.quantize_q8_1(x)
-        if encoding in K_ENCODINGS:
-            q8 = oracle.linear_q8_1(encoding, packed, out_dim, in_dim, codes, scales)
-            assert np.all(np.abs(y - q8) <= 2e-2 + 4e-4 * np.abs(q8))
-        assert error <= 2e-2
+    assert normalised_error(y, expected) <= TOLERANCE
+
+
+@pytest.mark.parametrize("encoding", K_ENCODINGS)
+def test_prefill_gemm_ragged_tiles_and_odd_block_count(cuda, oracle, encoding):
+    # 300 rows (a full tile and a ragged one), 200 columns (ragged), K of three
+    # blocks (odd: the kernel's two-block loop runs its first block ahead)
+    rows, out_dim, in_dim = 300, 200, 768
+    packed = random_packed(encoding, out_dim, in_dim, 41)
+    x = kquant.synthetic_activations(72, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    assert normalised_error(y, expected) <= TOLERANCE
+
+
+def test_prefill_gemm_activation_range(cuda, oracle):
+    # rows scaled far outside the fp16 range, and a zero row: the per-row power
+    # of two keeps every row at the same relative accuracy
+    rows, out_dim, in_dim = 6, 128, 512
+    packed = kquant.quantize(kquant.Q4_K, kquant.synthetic_weights(77, out_dim, in_dim))
+    x = kquant.synthetic_activations(73, rows, in_dim)
+    x *= np.array([1.0, 1.0e6, 1.0e-6, 3.0e20, 2.0e-22, 0.0], dtype=np.float32)[:, None]
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
+    expected = oracle.linear(kquant.Q4_K, packed, out_dim, in_dim, x)
+    for row in range(rows - 1):
+        assert normalised_error(y[row:row + 1], expected[row:row + 1]) <= TOLERANCE
+    assert np.all(y[rows - 1] == 0.0)
+
+
+def test_prefill_gemm_reserved_mode_is_refused(cuda):
+    lib = tile_ops.load()
+    assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(64, 512, 128, tile_ops.GEMM_INT8) == 0
+    assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(64, 512, 128, tile_ops.GEMM_F16) > 0
 
 
 def test_prefill_gemm_full_size_row_subset(cuda, oracle):
