@@ -32,6 +32,11 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+# HBM bytes per launch of the default workload (rows=1), from the FETCH_SIZE and
+# WRITE_SIZE counters of a `--traffic-probe` run, each calibrated on a plain
+# copy of known size; the figures and commands are in
+# profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_615_834}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
 FFN_DIM = 16384
@@ -369,7 +374,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(value / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.rows),
             "kernel": "decode GEMV (Q/K/V grouped launch and O launch, averaged)",
             "bytes_per_launch": bytes_per_step // launches,
             "us_per_launch": round(ms_per_step * 1e3 / launches, 3),
