@@ -386,6 +386,7 @@ struct WeightFragments {
 #define NFN_LOAD_ACTIVATIONS(base, row_block, chunk) \
     (*reinterpret_cast<const f16x8*>((base) + (row_block) * row_block_bytes + (chunk) * kFragmentBytes))
 #define NFN_WRITE16(target, x, y, z, w) *reinterpret_cast<u32x4*>(target) = u32x4{x, y, z, w}
+#define NFN_WRITE8(target, pair) *reinterpret_cast<uint2*>(target) = make_uint2((pair)[0], (pair)[1])
 
 // One matrix instruction with the statements issued in its shadow.  A wave
 // issues in order and stalls at a matrix instruction while the previous one
@@ -413,38 +414,37 @@ __device__ __forceinline__ void k_step(
     const std::uint8_t* a_fetch, std::int64_t row_block_bytes, const std::uint8_t* b_global,
     int fetch_step) {
     WeightFragments ahead;
-    std::uint32_t wa[4][2], wb[4][2];
+    std::uint32_t w[2];
 
-    // K chunk 0: read chunk 1, decode
+    // K chunk 0: read chunk 1, decode; every decoded group of four values is
+    // written to the other stage at once (8 bytes), which keeps few registers live
     NFN_SLOT(a_now.r0k0, current.c0, acc[0][0], b_next.prepare_bits(header, decode_pair, b_half))
     NFN_SLOT(a_now.r0k0, current.c1, acc[0][1], b_next.prepare_scales(header);
              ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 1))
-    NFN_SLOT(a_now.r0k0, current.c2, acc[0][2], b_next.template group_a<0>(wa[0]);
-             ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
-    NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_b<0>(wb[0]))
-    NFN_SLOT(a_now.r1k0, current.c0, acc[1][0], b_next.template group_a<1>(wa[1]);
-             ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
+    NFN_SLOT(a_now.r0k0, current.c2, acc[0][2], b_next.template group_a<0>(w);
+             NFN_WRITE8(b_write, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
+    NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_b<0>(w);
+             NFN_WRITE8(b_write + 64, w))
+    NFN_SLOT(a_now.r1k0, current.c0, acc[1][0], b_next.template group_a<1>(w);
+             NFN_WRITE8(b_write + 8, w); ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
              a_now.r0k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 0))
-    NFN_SLOT(a_now.r1k0, current.c1, acc[1][1], b_next.template group_b<1>(wb[1]))
-    NFN_SLOT(a_now.r1k0, current.c2, acc[1][2], b_next.template group_a<2>(wa[2]);
-             ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
-    NFN_SLOT(a_now.r1k0, current.c3, acc[1][3], b_next.template group_b<2>(wb[2]))
-    // K chunk 1: read chunk 2, finish decoding, write the decoded weights
-    NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<3>(wa[3]);
-             current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
+    NFN_SLOT(a_now.r1k0, current.c1, acc[1][1], b_next.template group_b<1>(w);
+             NFN_WRITE8(b_write + 72, w))
+    NFN_SLOT(a_now.r1k0, current.c2, acc[1][2], b_next.template group_a<2>(w);
+             NFN_WRITE8(b_write + 16, w); ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
+    NFN_SLOT(a_now.r1k0, current.c3, acc[1][3], b_next.template group_b<2>(w);
+             NFN_WRITE8(b_write + 80, w))
+    // K chunk 1: read chunk 2, finish decoding
+    NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<3>(w);
+             NFN_WRITE8(b_write + 24, w); current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
              a_now.r1k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 1, 0))
-    NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<3>(wb[3]))
-    NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2],
-             NFN_WRITE16(b_write, wa[0][0], wa[0][1], wa[1][0], wa[1][1]);
-             current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
-    NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3],
-             NFN_WRITE16(b_write + 16, wa[2][0], wa[2][1], wa[3][0], wa[3][1]))
-    NFN_SLOT(a_now.r1k1, ahead.c0, acc[1][0],
-             NFN_WRITE16(b_write + 64, wb[0][0], wb[0][1], wb[1][0], wb[1][1]);
-             current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2);
+    NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<3>(w);
+             NFN_WRITE8(b_write + 88, w))
+    NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2], current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
+    NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3], (void)0)
+    NFN_SLOT(a_now.r1k1, ahead.c0, acc[1][0], current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2);
              a_now.r0k1 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 1))
-    NFN_SLOT(a_now.r1k1, ahead.c1, acc[1][1],
-             NFN_WRITE16(b_write + 80, wb[2][0], wb[2][1], wb[3][0], wb[3][1]))
+    NFN_SLOT(a_now.r1k1, ahead.c1, acc[1][1], (void)0)
     NFN_SLOT(a_now.r1k1, ahead.c2, acc[1][2], current.c3 = NFN_READ_WEIGHTS(b_read, 3, 2))
     NFN_SLOT(a_now.r1k1, ahead.c3, acc[1][3], (void)0)
     // K chunk 2: read chunk 3
@@ -482,8 +482,15 @@ __device__ __forceinline__ void k_step(
     NFN_FENCE();
 }
 
+// Two workgroups per compute unit (two waves per SIMD) where the registers
+// allow it: while one wave waits at the barrier or for LDS, the other keeps
+// the matrix pipe busy.  The Q6_K decode holds more live state and stays at one.
 template <std::uint32_t ENC>
-__global__ __launch_bounds__(kThreads) void gemm_f16_kernel(
+constexpr int kWavesPerSimd = ENC == kEncQ6K ? 1 : 2;
+
+template <std::uint32_t ENC>
+__global__ __launch_bounds__(kThreads)
+__attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) void gemm_f16_kernel(
     const std::uint8_t* __restrict__ weights, std::int64_t row_stride, std::int64_t output_dim,
     std::int64_t input_dim, const std::uint8_t* __restrict__ activations,
     const float* __restrict__ inverse_scale, float* __restrict__ output, std::int64_t rows,
