@@ -406,9 +406,9 @@ struct WeightFragments {
 //   b_next:   packed weights of the next step: dequantized into the other
 //             stage with the scales in `header`, then refilled with the packed
 //             bytes of `fetch_step`
-template <std::uint32_t ENC>
+template <std::uint32_t ENC, int RB>
 __device__ __forceinline__ void k_step(
-    v16f (&acc)[2][4], ActivationSlice& a_now, WeightFragments& current,
+    v16f (&acc)[RB][4], ActivationSlice& a_now, WeightFragments& current,
     const std::uint8_t* b_read, const std::uint8_t* b_read_next, std::uint8_t* b_write,
     PackedSlice<ENC>& b_next, const BlockHeader<ENC>& header, int decode_pair, int b_half,
     const std::uint8_t* a_fetch, std::int64_t row_block_bytes, const std::uint8_t* b_global,
@@ -416,6 +416,44 @@ __device__ __forceinline__ void k_step(
     WeightFragments ahead;
     std::uint32_t w[2];
 
+    if constexpr (RB == 1) {
+        // One row block per wave: 16 slots carry the same side work.
+        NFN_SLOT(a_now.r0k0, current.c0, acc[0][0], b_next.prepare_bits(header, decode_pair, b_half))
+        NFN_SLOT(a_now.r0k0, current.c1, acc[0][1], b_next.prepare_scales(header);
+                 ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 1))
+        NFN_SLOT(a_now.r0k0, current.c2, acc[0][2], b_next.template group_a<0>(w);
+                 NFN_WRITE8(b_write, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
+        NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_b<0>(w);
+                 NFN_WRITE8(b_write + 64, w); ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
+                 ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
+        NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<1>(w);
+                 NFN_WRITE8(b_write + 8, w); current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
+                 a_now.r0k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 0))
+        NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<1>(w);
+                 NFN_WRITE8(b_write + 72, w); current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
+        NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2], b_next.template group_a<2>(w);
+                 NFN_WRITE8(b_write + 16, w); current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2))
+        NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3], b_next.template group_b<2>(w);
+                 NFN_WRITE8(b_write + 80, w); current.c3 = NFN_READ_WEIGHTS(b_read, 3, 2))
+        NFN_SLOT(a_now.r0k2, current.c0, acc[0][0], b_next.template group_a<3>(w);
+                 NFN_WRITE8(b_write + 24, w); ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 3);
+                 a_now.r0k1 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 1))
+        NFN_SLOT(a_now.r0k2, current.c1, acc[0][1], b_next.template group_b<3>(w);
+                 NFN_WRITE8(b_write + 88, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 3))
+        NFN_SLOT(a_now.r0k2, current.c2, acc[0][2], ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 3))
+        NFN_SLOT(a_now.r0k2, current.c3, acc[0][3], ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 3))
+        __syncthreads();
+        NFN_SLOT(a_now.r0k3, ahead.c0, acc[0][0], current.c0 = NFN_READ_WEIGHTS(b_read_next, 0, 0);
+                 a_now.r0k2 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 2))
+        NFN_SLOT(a_now.r0k3, ahead.c1, acc[0][1], current.c1 = NFN_READ_WEIGHTS(b_read_next, 1, 0))
+        NFN_SLOT(a_now.r0k3, ahead.c2, acc[0][2], current.c2 = NFN_READ_WEIGHTS(b_read_next, 2, 0))
+        NFN_SLOT(a_now.r0k3, ahead.c3, acc[0][3], current.c3 = NFN_READ_WEIGHTS(b_read_next, 3, 0))
+        a_now.r0k3 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 3);
+        NFN_FENCE();
+        b_next.load(b_global, fetch_step >> 2, fetch_step & 3, b_half);
+        NFN_FENCE();
+        return;
+    } else {
     // K chunk 0: read chunk 1, decode; every decoded group of four values is
     // written to the other stage at once (8 bytes), which keeps few registers live
     NFN_SLOT(a_now.r0k0, current.c0, acc[0][0], b_next.prepare_bits(header, decode_pair, b_half))
@@ -480,17 +518,20 @@ __device__ __forceinline__ void k_step(
     NFN_FENCE();
     b_next.load(b_global, fetch_step >> 2, fetch_step & 3, b_half);
     NFN_FENCE();
+    }
 }
 
-// Two workgroups per compute unit (two waves per SIMD) where the registers
-// allow it: while one wave waits at the barrier or for LDS, the other keeps
-// the matrix pipe busy.  The Q6_K decode holds more live state and stays at one.
-template <std::uint32_t ENC>
-constexpr int kWavesPerSimd = ENC == kEncQ6K ? 1 : 2;
+// Workgroups per compute unit (= waves per SIMD): as many as the registers
+// allow; while one wave waits at the barrier or for LDS, another keeps the
+// matrix pipe busy.  With 256-row tiles the Q6_K decode holds too much live
+// state for two.
+template <std::uint32_t ENC, int RB>
+constexpr int kWavesPerSimd = ENC == kEncQ6K ? RB == 1 ? 2 : 1 : RB == 1 ? 3 : 2;
 
-template <std::uint32_t ENC>
+// RB: 32-row blocks per wave; the workgroup's tile is 128*RB rows by 128 columns.
+template <std::uint32_t ENC, int RB>
 __global__ __launch_bounds__(kThreads)
-__attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) void gemm_f16_kernel(
+__attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB>))) void gemm_f16_kernel(
     const std::uint8_t* __restrict__ weights, std::int64_t row_stride, std::int64_t output_dim,
     std::int64_t input_dim, const std::uint8_t* __restrict__ activations,
     const float* __restrict__ inverse_scale, float* __restrict__ output, std::int64_t rows,
@@ -501,7 +542,8 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // rows 64*wave .. +63 of the tile
     const int m_tile = blockIdx.x % m_tiles;
     const int n_tile = blockIdx.x / m_tiles;
-    const std::int64_t m0 = static_cast<std::int64_t>(m_tile) * kBM;
+    constexpr int kTileRows = 128 * RB;
+    const std::int64_t m0 = static_cast<std::int64_t>(m_tile) * kTileRows;
     const std::int64_t n0 = static_cast<std::int64_t>(n_tile) * kBN;
     const int steps = static_cast<int>(input_dim / kBK);  // a positive multiple of 4
     const int last = steps - 1;
@@ -509,7 +551,7 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     // activations: fragment (row block, K chunk) is 1 KB, a row block's chunks are consecutive
     const std::int64_t row_block_bytes = (input_dim / 16) * kFragmentBytes;
     const std::uint8_t* a_global =
-        activations + (m0 / 32 + wave * 2) * row_block_bytes + lane * 16;
+        activations + (m0 / 32 + wave * RB) * row_block_bytes + lane * 16;
     constexpr int kStepBytes = (kBK / 16) * kFragmentBytes;
     // weights: thread -> (row, which 16 positions of the two 32-value groups)
     const int b_row = tid >> 1;
@@ -517,9 +559,9 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     const std::uint8_t* b_global = weights + min(n0 + b_row, output_dim - 1) * row_stride;
     const int b_target = b_row * kRowBytes + b_half * 32;
 
-    v16f acc[2][4];
+    v16f acc[RB][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < RB; ++i) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -547,13 +589,15 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     b2.load(b_global, 0, 2, b_half);
     b3.load(b_global, 0, 3, b_half);
     a_now.r0k0 = NFN_LOAD_ACTIVATIONS(a_global, 0, 0);
-    a_now.r1k0 = NFN_LOAD_ACTIVATIONS(a_global, 1, 0);
     a_now.r0k1 = NFN_LOAD_ACTIVATIONS(a_global, 0, 1);
-    a_now.r1k1 = NFN_LOAD_ACTIVATIONS(a_global, 1, 1);
     a_now.r0k2 = NFN_LOAD_ACTIVATIONS(a_global, 0, 2);
-    a_now.r1k2 = NFN_LOAD_ACTIVATIONS(a_global, 1, 2);
     a_now.r0k3 = NFN_LOAD_ACTIVATIONS(a_global, 0, 3);
-    a_now.r1k3 = NFN_LOAD_ACTIVATIONS(a_global, 1, 3);
+    if constexpr (RB == 2) {
+        a_now.r1k0 = NFN_LOAD_ACTIVATIONS(a_global, 1, 0);
+        a_now.r1k1 = NFN_LOAD_ACTIVATIONS(a_global, 1, 1);
+        a_now.r1k2 = NFN_LOAD_ACTIVATIONS(a_global, 1, 2);
+        a_now.r1k3 = NFN_LOAD_ACTIVATIONS(a_global, 1, 3);
+    }
     {
         std::uint32_t wa[4][2], wb[4][2];
         b0.prepare_bits(header_even, 0, b_half);
@@ -599,13 +643,13 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     // this block, `next` those of the following one (needed by the fourth step,
     // which decodes the first step of that block).
     auto block_of_four = [&](int step, const BlockHeader<ENC>& now, const BlockHeader<ENC>& next) {
-        k_step<ENC>(acc, a_now, current, b_read0, b_read1, b_write1, b1, now, 1, b_half,
+        k_step<ENC, RB>(acc, a_now, current, b_read0, b_read1, b_write1, b1, now, 1, b_half,
                     activations_of(step + 1), row_block_bytes, b_global, min(step + 5, last));
-        k_step<ENC>(acc, a_now, current, b_read1, b_read0, b_write0, b2, now, 2, b_half,
+        k_step<ENC, RB>(acc, a_now, current, b_read1, b_read0, b_write0, b2, now, 2, b_half,
                     activations_of(step + 2), row_block_bytes, b_global, min(step + 6, last));
-        k_step<ENC>(acc, a_now, current, b_read0, b_read1, b_write1, b3, now, 3, b_half,
+        k_step<ENC, RB>(acc, a_now, current, b_read0, b_read1, b_write1, b3, now, 3, b_half,
                     activations_of(step + 3), row_block_bytes, b_global, min(step + 7, last));
-        k_step<ENC>(acc, a_now, current, b_read1, b_read0, b_write0, b0, next, 0, b_half,
+        k_step<ENC, RB>(acc, a_now, current, b_read1, b_read0, b_write0, b0, next, 0, b_half,
                     activations_of(step + 4), row_block_bytes, b_global, min(step + 8, last));
     };
     // The two header register sets swap roles every block; the loop body is two
@@ -636,10 +680,10 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     // D register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32
     const int column = lane & 31;
     const int row_base = (lane >> 5) * 4;
-    const bool whole = m0 + kBM <= rows && n0 + kBN <= output_dim;
+    const bool whole = m0 + kTileRows <= rows && n0 + kBN <= output_dim;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const std::int64_t tile_row = m0 + wave * 64 + i * 32 + row_base;
+    for (int i = 0; i < RB; ++i) {
+        const std::int64_t tile_row = m0 + wave * (32 * RB) + i * 32 + row_base;
         float inverse[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) inverse[r] = inverse_scale[tile_row + 8 * (r >> 2) + (r & 3)];
@@ -665,16 +709,42 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC>, kWavesPerSimd<ENC>))) voi
     }
 }
 
+int compute_unit_count() {
+    static const int count = [] {
+        int device = 0;
+        int value = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            value <= 0) {
+            return 256;
+        }
+        return value;
+    }();
+    return count;
+}
+
 template <std::uint32_t ENC>
 void launch_encoding(const Descriptor& descriptor, const std::uint8_t* activations,
                      const float* inverse_scale, float* output, std::int64_t rows,
                      hipStream_t stream) {
-    const int m_tiles = static_cast<int>((rows + kBM - 1) / kBM);
     const std::int64_t n_tiles = (descriptor.output_dim + kBN - 1) / kBN;
-    hipLaunchKernelGGL(gemm_f16_kernel<ENC>, dim3(static_cast<unsigned>(m_tiles * n_tiles)),
-                       dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,
-                       descriptor.row_stride_bytes, descriptor.output_dim, descriptor.input_dim,
-                       activations, inverse_scale, output, rows, m_tiles);
+    const std::int64_t tall_tiles = (rows + 255) / 256;
+    // 256-row tiles reuse each weight fragment twice as often and win whenever
+    // they give every compute unit a workgroup; 128-row tiles double the number
+    // of workgroups for the small problems that would leave units empty
+    if (tall_tiles * n_tiles >= compute_unit_count()) {
+        const int m_tiles = static_cast<int>(tall_tiles);
+        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 2>), dim3(static_cast<unsigned>(m_tiles * n_tiles)),
+                           dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,
+                           descriptor.row_stride_bytes, descriptor.output_dim,
+                           descriptor.input_dim, activations, inverse_scale, output, rows, m_tiles);
+    } else {
+        const int m_tiles = static_cast<int>((rows + 127) / 128);
+        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 1>), dim3(static_cast<unsigned>(m_tiles * n_tiles)),
+                           dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,
+                           descriptor.row_stride_bytes, descriptor.output_dim,
+                           descriptor.input_dim, activations, inverse_scale, output, rows, m_tiles);
+    }
 }
 
 std::int64_t padded_rows(std::int64_t rows) { return (rows + kBM - 1) / kBM * kBM; }

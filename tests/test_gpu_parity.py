@@ -471,6 +471,21 @@ def test_prefill_gemm_ragged_tiles_and_odd_block_count(cuda, oracle, encoding):
     assert normalised_error(y, expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_prefill_gemm_tall_tiles(cuda, oracle, encoding):
+    # 512 rows x 16384 columns = 2 x 128 tiles: enough workgroups for the
+    # 256-row tile variant (smaller problems run the 128-row one); K of two
+    # blocks (even count).  The oracle checks a spread of rows.
+    rows, out_dim, in_dim = 512, 16384, 512
+    packed = random_packed(encoding, out_dim, in_dim, 43)
+    x = kquant.synthetic_activations(74, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
+    picked = np.array([0, 1, 31, 32, 63, 64, 127, 128, 255, 256, 300, 383, 384, 447, 448, 511])
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, np.ascontiguousarray(x[picked]))
+    assert normalised_error(y[picked], expected) <= TOLERANCE
+
+
 def test_prefill_gemm_activation_range(cuda, oracle):
     # rows scaled far outside the fp16 range, and a zero row: the per-row power
     # of two keeps every row at the same relative accuracy
