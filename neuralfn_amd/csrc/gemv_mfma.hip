@@ -513,9 +513,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     if constexpr (FUSED) {
 #pragma unroll
         for (int b = 0; b < kEarlyBlocks; ++b) {
-#ifndef NFN_EXP_SKIP_QUANT
             if (b < count) quantize_block(x[b], lane, wave_records + b * kActRecord);
-#endif
         }
         // more than kEarlyBlocks blocks per wave: quantize the rest now
         for (int b = kEarlyBlocks; b < count; ++b) {
@@ -545,17 +543,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                     const int slot = (slot_base + b) % kDepth;
                     auto rotate = [&](auto slot_constant) {
                         constexpr int kSlot = decltype(slot_constant)::value;
-#ifndef NFN_EXP_SKIP_STORE
                         store_block<ENC>(staged[kSlot], lane, wave_tile);
-#else
-                        {
-                            std::uint32_t mix = 0;
-                            for (int i = 0; i < Source::kLoads; ++i) {
-                                mix ^= staged[kSlot][i].x ^ staged[kSlot][i].y ^ staged[kSlot][i].z ^ staged[kSlot][i].w;
-                            }
-                            if (mix == 0x12345u) wave_tile[lane] = 1;
-                        }
-#endif
                         fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[kSlot]);
                         advance_fetch();
                     };
@@ -606,9 +594,6 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                             }
                         }
                     }
-#ifdef NFN_EXP_SKIP_COMPUTE
-                    acc[0] += act.scale[0] + static_cast<float>(wave_tile[lane * 36]);
-#else
                     if constexpr (ENC == kEncQ4K) {
                         process_block_q45<S, false>(wave_tile, j, kc, act, acc);
                     } else if constexpr (ENC == kEncQ5K) {
@@ -616,7 +601,6 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                     } else {
                         process_block_q6<S>(wave_tile, j, kc, act, acc);
                     }
-#endif
                     wave_lds_fence();  // the next block's stores stay behind these reads
                 }
             }

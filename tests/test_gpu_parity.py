@@ -458,11 +458,12 @@ def test_prefill_gemm_against_oracle(cuda, oracle, encoding):
     assert normalised_error(y, expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("in_dim", [256, 768])
 @pytest.mark.parametrize("encoding", K_ENCODINGS)
-def test_prefill_gemm_ragged_tiles_and_odd_block_count(cuda, oracle, encoding):
-    # 300 rows (a full tile and a ragged one), 200 columns (ragged), K of three
-    # blocks (odd: the kernel's two-block loop runs its first block ahead)
-    rows, out_dim, in_dim = 300, 200, 768
+def test_prefill_gemm_ragged_tiles_and_odd_block_count(cuda, oracle, encoding, in_dim):
+    # 300 rows (full tiles and a ragged one), 200 columns (ragged), K of one or
+    # three blocks (odd: the kernel's two-block loop runs its first block ahead)
+    rows, out_dim = 300, 200
     packed = random_packed(encoding, out_dim, in_dim, 41)
     x = kquant.synthetic_activations(72, rows, in_dim)
     weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
