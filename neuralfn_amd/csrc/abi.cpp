@@ -332,7 +332,7 @@ std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
     if (rows < 1 || rows > 8 || output_dim <= 0) return 0;
     // room for either kernel's per-workgroup candidates
     const std::int64_t f32_groups = lm_head_f32_blocks(output_dim);
-    const std::int64_t q6_groups = lm_head_q6_groups(output_dim);
+    const std::int64_t q6_groups = lm_head_q6_max_groups(output_dim);
     const std::int64_t raw = rows * (f32_groups > q6_groups ? f32_groups : q6_groups) *
         static_cast<std::int64_t>(sizeof(LmHeadCandidate));
     return (raw + 255) & ~std::int64_t(255);

@@ -38,6 +38,7 @@ namespace nfn {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef std::uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
@@ -109,6 +110,70 @@ __device__ __forceinline__ void better(float value, std::int64_t index, float& b
     if (value > best_value || (value == best_value && index < best_index)) {
         best_value = value;
         best_index = index;
+    }
+}
+
+// The packed bytes of one unit: 64 values = positions 16*sixteen .. +15 of the
+// four quarters of one half of a block.
+struct UnitData {
+    std::uint32_t low_a[4];  // low nibbles: quarter 0, high nibbles: quarter 2
+    std::uint32_t low_b[4];  // low nibbles: quarter 1, high nibbles: quarter 3
+    std::uint32_t top[4];    // two bits per quarter
+    std::uint32_t scales_lo, scales_hi;  // the eight int8 sub-scales of the half
+    std::uint32_t d_bits;
+};
+
+// acc[t] += (activation scale * d) * sum_quarter sc * (256*dot(q,hi) + dot(q,lo) - 32*sum(codes))
+// for unit `unit` (= 4*block + 2*half + sixteen inside the row) and every token.
+template <int T>
+__device__ __forceinline__ void accumulate_unit(const UnitData& data, std::uint8_t* lds, int blocks,
+                                                int unit, bool live, float (&acc)[T]) {
+    const int units = 4 * blocks;
+    const int block = unit >> 2;
+    const int sixteen = unit & 1;
+    // 6-bit codes of the four quarters, four bytes per word
+    std::uint32_t q[4][4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const std::uint32_t a = data.low_a[w], b = data.low_b[w], h = data.top[w];
+        q[0][w] = (a & 0x0f0f0f0fu) | ((h & 0x03030303u) << 4);
+        q[1][w] = (b & 0x0f0f0f0fu) | ((h & 0x0c0c0c0cu) << 2);
+        q[2][w] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+        q[3][w] = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+    }
+    // sub-scale of quarter k: byte 2*k + sixteen of the half's eight
+    const std::uint32_t s01 = data.scales_lo >> (8 * sixteen);
+    const std::uint32_t s23 = data.scales_hi >> (8 * sixteen);
+    const float scale_q[4] = {
+        static_cast<float>(static_cast<std::int8_t>(s01 & 0xffu)),
+        static_cast<float>(static_cast<std::int8_t>((s01 >> 16) & 0xffu)),
+        static_cast<float>(static_cast<std::int8_t>(s23 & 0xffu)),
+        static_cast<float>(static_cast<std::int8_t>((s23 >> 16) & 0xffu))};
+    const float d = half_bits_to_float(data.d_bits);
+
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const TokenImage image = token_image(lds, t, blocks);
+        const std::uint8_t* slot = image.planes + unit * 16;
+        const int stride = units * 16;
+        const v4i sums = *reinterpret_cast<const v4i*>(image.sums + unit * 4);
+        float unit_value = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const v4i hi = *reinterpret_cast<const v4i*>(slot + (2 * k) * stride);
+            const v4i lo = *reinterpret_cast<const v4i*>(slot + (2 * k + 1) * stride);
+            int dot_hi = 0, dot_lo = 0;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                dot_hi = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), hi[w], dot_hi, false);
+                dot_lo = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), lo[w], dot_lo, false);
+            }
+            // |256*dot_hi + dot_lo| < 2^26 and 32*|sum| < 2^25: exact in int32
+            const int bracket = (dot_hi << 8) + dot_lo - (sums[k] << 5);
+            unit_value = fmaf(scale_q[k], static_cast<float>(bracket), unit_value);
+        }
+        const float scale = image.scale[block];
+        acc[t] = fmaf(live ? scale * d : 0.0f, unit_value, acc[t]);
     }
 }
 
@@ -211,53 +276,18 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
         const int raw_unit = iteration * kWave + lane;
         const bool live = raw_unit < units;
         const int unit = min(raw_unit, units - 1);
-        const int block = unit >> 2;
-        const int sixteen = unit & 1;
 
-        // 6-bit codes of the four quarters, four bytes per word
-        std::uint32_t q[4][4];
+        UnitData data;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const std::uint32_t a = stage.low_a.v[w], b = stage.low_b.v[w], h = stage.top.v[w];
-            q[0][w] = (a & 0x0f0f0f0fu) | ((h & 0x03030303u) << 4);
-            q[1][w] = (b & 0x0f0f0f0fu) | ((h & 0x0c0c0c0cu) << 2);
-            q[2][w] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
-            q[3][w] = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+            data.low_a[w] = stage.low_a.v[w];
+            data.low_b[w] = stage.low_b.v[w];
+            data.top[w] = stage.top.v[w];
         }
-        // sub-scale of quarter k: byte 2*k + sixteen of the half's eight
-        const std::uint32_t s01 = stage.scales.v[0] >> (8 * sixteen);
-        const std::uint32_t s23 = stage.scales.v[1] >> (8 * sixteen);
-        const float scale_q[4] = {
-            static_cast<float>(static_cast<std::int8_t>(s01 & 0xffu)),
-            static_cast<float>(static_cast<std::int8_t>((s01 >> 16) & 0xffu)),
-            static_cast<float>(static_cast<std::int8_t>(s23 & 0xffu)),
-            static_cast<float>(static_cast<std::int8_t>((s23 >> 16) & 0xffu))};
-        const float d = half_bits_to_float(stage.d_bits);
-
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const TokenImage image = token_image(lds, t, blocks);
-            const std::uint8_t* slot = image.planes + unit * 16;
-            const int stride = units * 16;
-            const v4i sums = *reinterpret_cast<const v4i*>(image.sums + unit * 4);
-            float unit_value = 0.0f;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const v4i hi = *reinterpret_cast<const v4i*>(slot + (2 * k) * stride);
-                const v4i lo = *reinterpret_cast<const v4i*>(slot + (2 * k + 1) * stride);
-                int dot_hi = 0, dot_lo = 0;
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    dot_hi = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), hi[w], dot_hi, false);
-                    dot_lo = __builtin_amdgcn_sdot4(static_cast<int>(q[k][w]), lo[w], dot_lo, false);
-                }
-                // |256*dot_hi + dot_lo| < 2^26 and 32*|sum| < 2^25: exact in int32
-                const int bracket = (dot_hi << 8) + dot_lo - (sums[k] << 5);
-                unit_value = fmaf(scale_q[k], static_cast<float>(bracket), unit_value);
-            }
-            const float scale = image.scale[block];
-            acc[t] = fmaf(live ? scale * d : 0.0f, unit_value, acc[t]);
-        }
+        data.scales_lo = stage.scales.v[0];
+        data.scales_hi = stage.scales.v[1];
+        data.d_bits = stage.d_bits;
+        accumulate_unit<T>(data, lds, blocks, unit, live, acc);
 
         if (iteration == iterations - 1) {
             // the row is complete: fixed-order butterfly
@@ -317,6 +347,247 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Streaming variant for rows of at least 16 blocks (K >= 4096).
+//
+// The kernel above gives every lane a coherent unit, which makes each load
+// instruction touch sixteen separate 32-byte runs; measured, that pattern tops
+// out near 4.4 TB/s whatever the arithmetic.  Here a wave copies its rows —
+// contiguous in memory, the descriptor allows no padding — through a private
+// LDS staging area instead: per pass 16 blocks, read as 224 consecutive 16-byte
+// pieces (four load instructions whose lanes touch neighbouring bytes) and
+// written to 224-byte slots, one per block, so that every piece of a block is
+// 16-byte aligned in LDS.  Piece 13 of a block is read from byte 194, not 208,
+// so that no load reaches past the block; it lands at slot offset 208 and puts
+// d at slot offset 222.  The 64 lanes then read one unit each from the slots
+// and run the same arithmetic as above.  Nothing but the first barrier (for
+// the activation image) synchronises the workgroup; a wave's own LDS accesses
+// execute in order.
+//
+// A pass can straddle two rows (never three: a row is at least 16 blocks), so
+// every lane keeps two running sums, for the wave's current row and the next.
+// ---------------------------------------------------------------------------
+constexpr int kPassBlocks = 16;
+constexpr int kSlotBytes = 224;
+constexpr int kPiecesPerBlock = 14;
+constexpr int kPassPieces = kPassBlocks * kPiecesPerBlock;  // 224 of 256 lane slots
+constexpr int kStagingBytes = kPassBlocks * kSlotBytes;
+
+struct PassLoads {
+    Unaligned16 piece[4];
+};
+
+// W: waves per workgroup (the activation images are shared by the workgroup,
+// so more tokens per pass want more waves behind each image).
+template <int T, int P, bool ARGMAX, int W>
+__global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
+    Projection op, std::int64_t input_dim, const float* __restrict__ first,
+    const float* __restrict__ second, int tokens, int rows_per_wave,
+    LmHeadCandidate* __restrict__ candidates) {
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int blocks = static_cast<int>(input_dim >> 8);  // per row, >= 16
+    const int token0 = blockIdx.y * T;
+    const int pass_tokens = min(tokens - token0, T);
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
+    const float* pass_second =
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
+    std::uint8_t* staging = lds + T * token_image_bytes(blocks) + wave * kStagingBytes;
+
+    // rows and blocks of this wave
+    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * W + wave;
+    const std::int64_t row_begin = wave_index * rows_per_wave;
+    const int row_count = static_cast<int>(max(
+        static_cast<std::int64_t>(0),
+        min(static_cast<std::int64_t>(rows_per_wave), op.output_dim - row_begin)));
+    const int wave_blocks = row_count * blocks;
+    const int passes = (wave_blocks + kPassBlocks - 1) / kPassBlocks;
+    // first byte of the wave's first block; a wave without rows points at the
+    // last row so that its (unused) loads stay inside the tensor
+    const std::uint8_t* stream = op.data +
+        min(row_begin, op.output_dim - 1) * op.row_stride;
+    const int stream_blocks = max(wave_blocks, 1);  // blocks that may be read from `stream`
+
+    // which piece of a pass each of this lane's four loads fetches: loop invariant
+    int source_offset[4], target_offset[4], piece_block[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int piece = min(k * kWave + lane, kPassPieces - 1);
+        const int block = piece / kPiecesPerBlock;
+        const int within = piece - block * kPiecesPerBlock;
+        piece_block[k] = block;
+        source_offset[k] = within == 13 ? 194 : within * 16;
+        target_offset[k] = block * kSlotBytes + within * 16;
+    }
+    auto issue = [&](PassLoads& loads, int pass) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            // blocks past the wave's range are read from its last block instead
+            const int block = min(pass * kPassBlocks + piece_block[k], stream_blocks - 1);
+            loads.piece[k] = *reinterpret_cast<const Unaligned16*>(
+                stream + static_cast<std::int64_t>(block) * kBlockBytes + source_offset[k]);
+        }
+    };
+
+    // (1) activations of the first records this wave quantizes, then (2) the
+    // packed bytes of the first two passes: all in flight together
+    const int records = pass_tokens * blocks;
+    constexpr int kEarly = 4;
+    float4 early[kEarly];
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = min(wave + e * W, records - 1);
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        early[e] = load_activations<P>(
+            pass_first, pass_second,
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
+    }
+    PassLoads loads0, loads1;
+    issue(loads0, 0);
+    issue(loads1, min(1, max(passes - 1, 0)));
+
+    // (3) quantize; one barrier
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e) {
+        const int record = wave + e * W;
+        if (record < records) {
+            const int token = record / blocks;
+            quantize_block(early[e], lane, record - token * blocks, blocks,
+                           token_image(lds, token, blocks));
+        }
+    }
+    for (int record = wave + kEarly * W; record < records; record += W) {
+        const int token = record / blocks;
+        const int block = record - token * blocks;
+        const float4 x = load_activations<P>(
+            pass_first, pass_second,
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
+        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+    }
+    __syncthreads();
+
+    float acc_current[T], acc_next[T];
+    float best_value[T];
+    std::int64_t best_index[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        acc_current[t] = 0.0f;
+        acc_next[t] = 0.0f;
+        best_value[t] = -INFINITY;
+        best_index[t] = 0;
+    }
+    int row = 0;                 // current row, relative to row_begin
+    int row_first_block = 0;     // its first block in the wave's stream
+    const int my_block = lane >> 2;  // block of this lane's unit inside a pass
+    const int my_unit = lane & 3;    // 2*half + sixteen
+    const std::uint8_t* my_slot = staging + my_block * kSlotBytes;
+    const int half = my_unit >> 1;
+    const int sixteen = my_unit & 1;
+
+    auto consume = [&](const PassLoads& loads, int pass) {
+        // stage: every lane writes its pieces (lanes 32..63 of the fourth load hold
+        // duplicates of the last piece and write the same bytes to the same place)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            *reinterpret_cast<u32x4*>(staging + target_offset[k]) =
+                u32x4{loads.piece[k].v[0], loads.piece[k].v[1], loads.piece[k].v[2],
+                      loads.piece[k].v[3]};
+        }
+        // read back this lane's unit
+        UnitData data;
+        const u32x4 a = *reinterpret_cast<const u32x4*>(my_slot + half * 64 + sixteen * 16);
+        const u32x4 b = *reinterpret_cast<const u32x4*>(my_slot + half * 64 + 32 + sixteen * 16);
+        const u32x4 h = *reinterpret_cast<const u32x4*>(my_slot + 128 + half * 32 + sixteen * 16);
+        const uint2 sc = *reinterpret_cast<const uint2*>(my_slot + 192 + half * 8);
+        data.d_bits = *reinterpret_cast<const std::uint16_t*>(my_slot + 222);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            data.low_a[w] = a[w];
+            data.low_b[w] = b[w];
+            data.top[w] = h[w];
+        }
+        data.scales_lo = sc.x;
+        data.scales_hi = sc.y;
+
+        const int stream_block = pass * kPassBlocks + my_block;
+        const bool live = stream_block < wave_blocks;
+        const int row_end_block = row_first_block + blocks;
+        const bool in_next = stream_block >= row_end_block;
+        // block inside its row, clamped for dead lanes
+        const int block_in_row =
+            min(stream_block - (in_next ? row_end_block : row_first_block), blocks - 1);
+        const int unit = 4 * block_in_row + my_unit;
+        float value[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) value[t] = 0.0f;
+        accumulate_unit<T>(data, lds, blocks, unit, live, value);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc_current[t] += in_next ? 0.0f : value[t];
+            acc_next[t] += in_next ? value[t] : 0.0f;
+        }
+
+        // the current row ends inside this pass: reduce and emit it
+        if (row_end_block <= (pass + 1) * kPassBlocks && row < row_count) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const float total_value = wave_total(acc_current[t]);
+                if constexpr (ARGMAX) {
+                    // rows come in increasing order: a strict comparison keeps the lowest index
+                    if (total_value > best_value[t]) {
+                        best_value[t] = total_value;
+                        best_index[t] = row_begin + row;
+                    }
+                } else {
+                    if (lane == 0 && t < pass_tokens) {
+                        op.output[static_cast<std::int64_t>(token0 + t) * op.output_dim +
+                                  row_begin + row] = total_value;
+                    }
+                }
+                acc_current[t] = acc_next[t];
+                acc_next[t] = 0.0f;
+            }
+            ++row;
+            row_first_block = row_end_block;
+        }
+    };
+
+    for (int pass = 0; pass < passes; pass += 2) {
+        consume(loads0, pass);
+        issue(loads0, min(pass + 2, passes - 1));
+        if (pass + 1 < passes) consume(loads1, pass + 1);
+        issue(loads1, min(pass + 3, passes - 1));
+    }
+
+    if constexpr (ARGMAX) {
+        // best of the workgroup per token: waves through LDS (the images are no longer needed)
+        __syncthreads();
+        float* values = reinterpret_cast<float*>(lds);
+        std::int64_t* indices = reinterpret_cast<std::int64_t*>(lds + W * T * 4);
+        if (lane == 0) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                values[wave * T + t] = best_value[t];
+                indices[wave * T + t] = best_index[t];
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x < static_cast<unsigned>(pass_tokens)) {
+            const int t = threadIdx.x;
+            float value = values[t];
+            std::int64_t index = indices[t];
+            for (int w = 1; w < W; ++w) better(values[w * T + t], indices[w * T + t], value, index);
+            LmHeadCandidate candidate;
+            candidate.index = index;
+            candidate.value = value;
+            candidate.pad = 0;
+            candidates[static_cast<std::int64_t>(token0 + t) * gridDim.x + blockIdx.x] = candidate;
+        }
+    }
+}
+
 struct Geometry {
     std::int64_t rows_per_wave;
     std::int64_t groups;
@@ -333,9 +604,11 @@ Geometry geometry(std::int64_t rows) {
     return g;
 }
 
+// The launchers return the number of workgroups along x of their (last)
+// launch: with the argmax fused in, that is the number of candidates per token.
 template <int T, int P, bool ARGMAX>
-void launch_variant(ProjectionSet set, const float* first, const float* second, int tokens,
-                    LmHeadCandidate* candidates, hipStream_t stream) {
+std::int64_t launch_variant(ProjectionSet set, const float* first, const float* second,
+                            int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
@@ -353,30 +626,81 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(kThreads), lds,
                        stream, set, first, second, tokens, rows, static_cast<int>(g.rows_per_wave),
                        candidates);
+    return g.groups;
 }
 
+// Rows per wave of the streaming kernel: whole multiples of eight rows once
+// there are enough rows, so that a wave's block count is a multiple of the 16
+// blocks of a pass for the common row lengths (26 blocks at K = 6656).
+Geometry stream_geometry(std::int64_t rows, int waves_per_group) {
+    Geometry g = geometry(rows);
+    if (g.rows_per_wave >= 8) g.rows_per_wave &= ~std::int64_t(7);
+    g.groups = (rows + g.rows_per_wave * waves_per_group - 1) / (g.rows_per_wave * waves_per_group);
+    return g;
+}
+
+// waves per workgroup of the streaming kernel for T tokens per pass
+constexpr int stream_waves(int tokens_per_pass) {
+    return tokens_per_pass <= 2 ? 8 : 16;
+}
+
+template <int T, int P, bool ARGMAX>
+std::int64_t launch_stream(const ProjectionSet& set, const float* first, const float* second,
+                           int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+    constexpr int W = stream_waves(T);
+    const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8) +
+        W * kStagingBytes;
+    auto kernel = gemv_q6_stream_kernel<T, P, ARGMAX, W>;
+    static const bool raised =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
+    (void)raised;
+    const int passes = (tokens + T - 1) / T;
+    // one launch per projection: a wave's rows must be contiguous in memory
+    std::int64_t groups = 0;
+    for (int index = 0; index < set.count; ++index) {
+        const Geometry g = stream_geometry(set.op[index].output_dim, W);
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(W * kWave),
+                           lds, stream, set.op[index], set.input_dim, first, second, tokens,
+                           static_cast<int>(g.rows_per_wave), candidates);
+        groups = g.groups;
+    }
+    return groups;
+}
+
+bool streams(std::int64_t input_dim) { return (input_dim >> 8) >= kPassBlocks; }
+
 template <int P, bool ARGMAX>
-void launch_tokens(const ProjectionSet& set, const float* first, const float* second, int tokens,
-                   LmHeadCandidate* candidates, hipStream_t stream) {
-    // the token images of one pass must fit in LDS
+std::int64_t launch_tokens(const ProjectionSet& set, const float* first, const float* second,
+                           int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+    // the token images of one pass (and the staging areas) must fit in LDS
     const std::int64_t image = token_image_bytes(set.input_dim >> 8);
-    int capacity = static_cast<int>((150 * 1024) / image);
+    int capacity = static_cast<int>((150 * 1024 - 16 * kStagingBytes) / image);
     if (capacity > 4) capacity = 4;
     const int per_pass = tokens < capacity ? tokens : capacity;
-    if (per_pass <= 1) {
-        launch_variant<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
-    } else if (per_pass == 2 || capacity < 4) {
-        launch_variant<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
-    } else {
-        launch_variant<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    if (streams(set.input_dim)) {
+        if (per_pass <= 1) {
+            return launch_stream<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+        }
+        if (per_pass == 2 || capacity < 4) {
+            return launch_stream<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+        }
+        return launch_stream<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
     }
+    if (per_pass <= 1) {
+        return launch_variant<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    }
+    if (per_pass == 2 || capacity < 4) {
+        return launch_variant<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    }
+    return launch_variant<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
 }
 
 }  // namespace
 
 bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim) {
     return encoding == kEncQ6K && input_dim % 256 == 0 &&
-        token_image_bytes(input_dim >> 8) <= 150 * 1024;
+        token_image_bytes(input_dim >> 8) <= 150 * 1024 - 16 * kStagingBytes;
 }
 
 void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
@@ -401,7 +725,12 @@ void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* s
     }
 }
 
-std::int64_t lm_head_q6_groups(std::int64_t output_dim) { return geometry(output_dim).groups; }
+std::int64_t lm_head_q6_max_groups(std::int64_t output_dim) {
+    // the eight-wave workgroups of the one- and two-token streaming kernel are the most numerous
+    const std::int64_t a = stream_geometry(output_dim, stream_waves(1)).groups;
+    const std::int64_t b = geometry(output_dim).groups;
+    return a > b ? a : b;
+}
 
 void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::int64_t rows,
                        LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
@@ -414,9 +743,9 @@ void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::in
     set.op[0].output_dim = descriptor.output_dim;
     set.op[0].row_stride = descriptor.row_stride_bytes;
     set.op[0].encoding = descriptor.encoding;
-    launch_tokens<kPlain, true>(set, input, nullptr, static_cast<int>(rows), candidates, stream);
-    launch_lm_head_final(candidates, lm_head_q6_groups(descriptor.output_dim), indices, maxima,
-                         rows, stream);
+    const std::int64_t groups =
+        launch_tokens<kPlain, true>(set, input, nullptr, static_cast<int>(rows), candidates, stream);
+    launch_lm_head_final(candidates, groups, indices, maxima, rows, stream);
 }
 
 }  // namespace nfn

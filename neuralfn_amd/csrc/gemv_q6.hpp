@@ -13,8 +13,9 @@ bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim);
 void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
                     int prologue, std::int64_t rows, hipStream_t stream);
 
-// Workgroups of the fused lm_head launch = candidates per input row.
-std::int64_t lm_head_q6_groups(std::int64_t output_dim);
+// Upper bound of the workgroups of a fused lm_head launch (= candidates per
+// input row) over all input widths and token counts, for sizing the workspace.
+std::int64_t lm_head_q6_max_groups(std::int64_t output_dim);
 void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::int64_t rows,
                        LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
                        hipStream_t stream);

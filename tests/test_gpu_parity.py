@@ -397,6 +397,47 @@ def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda):
     assert indices.cpu().tolist() == [100]
 
 
+# ------------------------------------------------ Q6_K rows of 16 blocks and more (streaming kernel)
+
+@pytest.mark.parametrize("shape", [(777, 4096), (1301, 6656), (64, 8192)])
+def test_q6_k_long_rows_one_token_and_verifier(cuda, oracle, shape):
+    # row counts that leave partial passes and waves without rows; K of exactly
+    # 16 blocks, of 26 (rows straddle passes) and of 32
+    out_dim, in_dim = shape
+    packed = random_packed(kquant.Q6_K, out_dim, in_dim, 51)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q6_K, packed, out_dim, in_dim)
+    x = kquant.synthetic_activations(52, 3, in_dim)
+    workspace = tile_ops.small_batch_workspace(3, in_dim)
+    expected = oracle.linear(kquant.Q6_K, packed, out_dim, in_dim, x)
+    batched = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family="mmvq")[0]
+    assert normalised_error(batched.cpu().numpy(), expected) <= TOLERANCE
+    for row in range(3):
+        single = tile_ops.mmvq_linear(weight, to_device(x[row:row + 1], cuda), workspace)
+        assert_bits_equal(single, batched[row:row + 1], f"row {row}")
+    one = tile_ops.multi_linear([weight], to_device(x[:1], cuda), workspace, family="mmq")[0]
+    assert_bits_equal(one, batched[:1], "mmq at one row")
+
+
+@pytest.mark.parametrize("rows", [1, 3])
+def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
+    out_dim, in_dim = 5003, 6656
+    packed = kquant.quantize(kquant.Q6_K, kquant.synthetic_weights(83, out_dim, in_dim))
+    x = kquant.synthetic_activations(93 + rows, rows, in_dim, rms_normalize=True)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q6_K, packed, out_dim, in_dim)
+    indices, maxima = tile_ops.lm_head_argmax(weight, to_device(x, cuda))
+    logits = oracle.linear(kquant.Q6_K, packed, out_dim, in_dim, x)
+    scale = np.max(np.abs(logits))
+    for row in range(rows):
+        ordered = np.sort(logits[row])[::-1]
+        assert abs(maxima.cpu()[row].item() - ordered[0]) <= TOLERANCE * scale
+        if ordered[0] - ordered[1] > 2 * TOLERANCE * scale:
+            assert indices.cpu()[row].item() == oracle.argmax(logits[row])
+    # the fused result equals argmax over the unfused logits of the same kernel
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    unfused = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family="mmvq")[0]
+    assert torch_().equal(unfused.max(dim=1).values.cpu(), maxima.cpu())
+
+
 # ------------------------------------------------ the benchmark's geometries
 
 def config_layer(seed, encoding=kquant.Q4_K):
