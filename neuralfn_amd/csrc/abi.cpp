@@ -8,6 +8,7 @@
 #include "gemm_mfma.hpp"
 #include "gemv_mfma.hpp"
 #include "gemv_q6.hpp"
+#include "gemv_q8.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
 
@@ -73,8 +74,8 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // kernel.  2..16 rows otherwise: the matrix-core kernel.  Encodings without
     // either: the float kernel.
     const bool one_row_arithmetic = rows == 1 || verifier;
-    ProjectionSet dot{}, dot6{}, matrix{}, exact{};
-    dot.input_dim = dot6.input_dim = matrix.input_dim = exact.input_dim = input_dim;
+    ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, exact{};
+    dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
         const std::uint32_t encoding = set.op[index].encoding;
         ProjectionSet* target = &exact;
@@ -82,6 +83,8 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
             target = &dot;
         } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
             target = &dot6;
+        } else if (one_row_arithmetic && gemv_q8_supports(encoding, input_dim)) {
+            target = &dot8;
         } else if (gemv_mfma_supports(encoding, input_dim)) {
             target = &matrix;
         }
@@ -92,6 +95,9 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     }
     if (dot6.count > 0) {
         launch_gemv_q6(dot6, first, second, prologue, rows, as_stream(stream));
+    }
+    if (dot8.count > 0) {
+        launch_gemv_q8(dot8, first, second, prologue, rows, as_stream(stream));
     }
     if (matrix.count > 0) {
         launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));

@@ -397,6 +397,23 @@ def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda):
     assert indices.cpu().tolist() == [100]
 
 
+@pytest.mark.parametrize("shape", [(130, 256), (515, 6656)])
+def test_q8_0_one_token_and_verifier(cuda, oracle, shape):
+    out_dim, in_dim = shape
+    packed = random_packed(kquant.Q8_0, out_dim, in_dim, 61)
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q8_0, packed, out_dim, in_dim)
+    x = kquant.synthetic_activations(62, 5, in_dim)
+    workspace = tile_ops.small_batch_workspace(5, in_dim)
+    expected = oracle.linear(kquant.Q8_0, packed, out_dim, in_dim, x)
+    batched = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family="mmvq")[0]
+    assert normalised_error(batched.cpu().numpy(), expected) <= TOLERANCE
+    for row in range(5):
+        single = tile_ops.mmvq_linear(weight, to_device(x[row:row + 1], cuda), workspace)
+        assert_bits_equal(single, batched[row:row + 1], f"row {row}")
+    one = tile_ops.multi_linear([weight], to_device(x[:1], cuda), workspace, family="mmq")[0]
+    assert_bits_equal(one, batched[:1], "mmq at one row")
+
+
 # ------------------------------------------------ Q6_K rows of 16 blocks and more (streaming kernel)
 
 @pytest.mark.parametrize("shape", [(777, 4096), (1301, 6656), (64, 8192)])
