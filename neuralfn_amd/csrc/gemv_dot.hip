@@ -31,7 +31,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kDotWaves = 8;
 constexpr int kDotThreads = kDotWaves * kWave;
-constexpr int kWavesPerUnit = 32;  // waves the grid aims at per compute unit
 
 // LDS image of one token's activations for a K of `blocks` super-blocks:
 //   planes: eight arrays of `units` 16-byte slots, units = 4*blocks; unit
@@ -94,7 +93,7 @@ struct Stage {
 template <std::uint32_t ENC, int T, int P>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows, int rows_per_wave, int token_base_stride) {
+    int tokens, std::int64_t total_rows) {
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
     constexpr int kQuants = kQ5 ? 48 : 16;
@@ -111,11 +110,13 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const float* pass_second =
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
 
-    // rows of this wave: a contiguous range
+    // rows of this wave: the rows are dealt out evenly over all waves of the grid
+    // (counts differ by at most one), each wave a contiguous range
     const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kDotWaves + wave;
-    const std::int64_t row_begin = wave_index * rows_per_wave;
-    const int row_count = static_cast<int>(
-        max(static_cast<std::int64_t>(0), min(static_cast<std::int64_t>(rows_per_wave), total_rows - row_begin)));
+    const std::int64_t wave_total_count = static_cast<std::int64_t>(gridDim.x) * kDotWaves;
+    const std::int64_t row_begin = wave_index * total_rows / wave_total_count;
+    const int row_count =
+        static_cast<int>((wave_index + 1) * total_rows / wave_total_count - row_begin);
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -283,7 +284,6 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         if (n + 1 < total) compute(stage1);
         issue(stage1);
     }
-    (void)token_base_stride;
 }
 
 template <std::uint32_t ENC, int T, int P>
@@ -301,15 +301,9 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
-    // about one wave per SIMD lane group and row range: rows_per_wave keeps the
-    // activation quantization (done once per workgroup) a small part of the work
-    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * kWavesPerUnit;
-    std::int64_t rows_per_wave = rows / waves_wanted;
-    if (rows_per_wave < 1) rows_per_wave = 1;
-    const std::int64_t groups = (rows + rows_per_wave * kDotWaves - 1) / (rows_per_wave * kDotWaves);
     const int passes = (tokens + T - 1) / T;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
-                       stream, set, first, second, tokens, rows, static_cast<int>(rows_per_wave), 0);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kDotWaves)), passes),
+                       dim3(kDotThreads), lds, stream, set, first, second, tokens, rows);
 }
 
 template <std::uint32_t ENC, int P>

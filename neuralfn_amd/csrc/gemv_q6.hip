@@ -180,8 +180,7 @@ __device__ __forceinline__ void accumulate_unit(const UnitData& data, std::uint8
 template <int T, int P, bool ARGMAX>
 __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows, int rows_per_wave,
-    LmHeadCandidate* __restrict__ candidates) {
+    int tokens, std::int64_t total_rows, LmHeadCandidate* __restrict__ candidates) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -194,12 +193,13 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     const float* pass_second =
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
 
-    // rows of this wave: a contiguous range
+    // rows of this wave: dealt out evenly over all waves of the grid, each wave
+    // a contiguous range
     const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kWaves + wave;
-    const std::int64_t row_begin = wave_index * rows_per_wave;
-    const int row_count = static_cast<int>(max(
-        static_cast<std::int64_t>(0),
-        min(static_cast<std::int64_t>(rows_per_wave), total_rows - row_begin)));
+    const std::int64_t wave_total_count = static_cast<std::int64_t>(gridDim.x) * kWaves;
+    const std::int64_t row_begin = wave_index * total_rows / wave_total_count;
+    const int row_count =
+        static_cast<int>((wave_index + 1) * total_rows / wave_total_count - row_begin);
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -621,12 +621,11 @@ std::int64_t launch_variant(ProjectionSet set, const float* first, const float* 
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
-    const Geometry g = geometry(rows);
+    const std::int64_t groups = decode_groups(rows, kWaves);
     const int passes = (tokens + T - 1) / T;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(kThreads), lds,
-                       stream, set, first, second, tokens, rows, static_cast<int>(g.rows_per_wave),
-                       candidates);
-    return g.groups;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
+                       stream, set, first, second, tokens, rows, candidates);
+    return groups;
 }
 
 // Rows per wave of the streaming kernel: whole multiples of eight rows once
@@ -728,7 +727,7 @@ void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* s
 std::int64_t lm_head_q6_max_groups(std::int64_t output_dim) {
     // the eight-wave workgroups of the one- and two-token streaming kernel are the most numerous
     const std::int64_t a = stream_geometry(output_dim, stream_waves(1)).groups;
-    const std::int64_t b = geometry(output_dim).groups;
+    const std::int64_t b = decode_groups(output_dim, kWaves);
     return a > b ? a : b;
 }
 

@@ -28,7 +28,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
-constexpr int kWavesPerUnit = 32;  // waves the grid aims at per compute unit
 constexpr int kUnitBytes = 68;     // two blocks
 
 struct __attribute__((packed, aligned(4))) Unaligned16 {
@@ -81,7 +80,7 @@ struct Stage {
 template <int T, int P>
 __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows, int rows_per_wave) {
+    int tokens, std::int64_t total_rows) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -94,12 +93,13 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const float* pass_second =
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
 
-    // rows of this wave: a contiguous range
+    // rows of this wave: dealt out evenly over all waves of the grid, each wave
+    // a contiguous range
     const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kWaves + wave;
-    const std::int64_t row_begin = wave_index * rows_per_wave;
-    const int row_count = static_cast<int>(max(
-        static_cast<std::int64_t>(0),
-        min(static_cast<std::int64_t>(rows_per_wave), total_rows - row_begin)));
+    const std::int64_t wave_total_count = static_cast<std::int64_t>(gridDim.x) * kWaves;
+    const std::int64_t row_begin = wave_index * total_rows / wave_total_count;
+    const int row_count =
+        static_cast<int>((wave_index + 1) * total_rows / wave_total_count - row_begin);
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -253,13 +253,9 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
-    const std::int64_t waves_wanted = static_cast<std::int64_t>(compute_units()) * kWavesPerUnit;
-    std::int64_t rows_per_wave = rows / waves_wanted;
-    if (rows_per_wave < 1) rows_per_wave = 1;
-    const std::int64_t groups = (rows + rows_per_wave * kWaves - 1) / (rows_per_wave * kWaves);
     const int passes = (tokens + T - 1) / T;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
-                       stream, set, first, second, tokens, rows, static_cast<int>(rows_per_wave));
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kWaves)), passes),
+                       dim3(kThreads), lds, stream, set, first, second, tokens, rows);
 }
 
 template <int P>
