@@ -80,15 +80,18 @@ __global__ __launch_bounds__(kWavesPerBlock * kWave) void lm_head_partial_kernel
 
 }  // namespace
 
-__global__ __launch_bounds__(256) void lm_head_final_kernel(
+constexpr int kFinalThreads = 1024;
+
+__global__ __launch_bounds__(kFinalThreads) void lm_head_final_kernel(
     const LmHeadCandidate* __restrict__ candidates, std::int64_t candidate_count,
     std::int64_t* __restrict__ indices, float* __restrict__ maxima) {
-    __shared__ float wave_values[4];
-    __shared__ std::int64_t wave_indices[4];
+    constexpr int kFinalWaves = kFinalThreads / kWave;
+    __shared__ float wave_values[kFinalWaves];
+    __shared__ std::int64_t wave_indices[kFinalWaves];
     const std::int64_t row = blockIdx.x;
     float best_value = -INFINITY;
     std::int64_t best_index = 0;
-    for (std::int64_t i = threadIdx.x; i < candidate_count; i += 256) {
+    for (std::int64_t i = threadIdx.x; i < candidate_count; i += kFinalThreads) {
         const LmHeadCandidate c = candidates[row * candidate_count + i];
         better(c.value, c.index, best_value, best_index);
     }
@@ -104,7 +107,9 @@ __global__ __launch_bounds__(256) void lm_head_final_kernel(
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) better(wave_values[w], wave_indices[w], best_value, best_index);
+        for (int w = 1; w < kFinalWaves; ++w) {
+            better(wave_values[w], wave_indices[w], best_value, best_index);
+        }
         indices[row] = best_index;
         maxima[row] = best_value;
     }
@@ -113,8 +118,9 @@ __global__ __launch_bounds__(256) void lm_head_final_kernel(
 void launch_lm_head_final(const LmHeadCandidate* candidates, std::int64_t candidate_count,
                           std::int64_t* indices, float* maxima, std::int64_t rows,
                           hipStream_t stream) {
-    hipLaunchKernelGGL(lm_head_final_kernel, dim3(static_cast<unsigned>(rows)), dim3(256), 0,
-                       stream, candidates, candidate_count, indices, maxima);
+    hipLaunchKernelGGL(lm_head_final_kernel, dim3(static_cast<unsigned>(rows)),
+                       dim3(kFinalThreads), 0, stream, candidates, candidate_count, indices,
+                       maxima);
 }
 
 std::int64_t lm_head_f32_blocks(std::int64_t output_dim) {
