@@ -59,6 +59,21 @@ bool normalize_descriptor(const Descriptor* source, Descriptor* output);
 bool validate_k_descriptor(const Descriptor* descriptor, std::int64_t input_dim,
                            void* stream, bool allow_q8_0);
 
+// Compute units of the current device (256 on MI355X), cached.
+inline int compute_units() {
+    static const int count = [] {
+        int device = 0;
+        int value = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            value <= 0) {
+            return 256;
+        }
+        return value;
+    }();
+    return count;
+}
+
 inline hipStream_t as_stream(void* stream) { return reinterpret_cast<hipStream_t>(stream); }
 inline int launch_status() { return static_cast<int>(hipPeekAtLastError()); }
 

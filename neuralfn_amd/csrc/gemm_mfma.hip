@@ -709,20 +709,6 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB
     }
 }
 
-int compute_unit_count() {
-    static const int count = [] {
-        int device = 0;
-        int value = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-            value <= 0) {
-            return 256;
-        }
-        return value;
-    }();
-    return count;
-}
-
 template <std::uint32_t ENC>
 void launch_encoding(const Descriptor& descriptor, const std::uint8_t* activations,
                      const float* inverse_scale, float* output, std::int64_t rows,
@@ -732,7 +718,7 @@ void launch_encoding(const Descriptor& descriptor, const std::uint8_t* activatio
     // 256-row tiles reuse each weight fragment twice as often and win whenever
     // they give every compute unit a workgroup; 128-row tiles double the number
     // of workgroups for the small problems that would leave units empty
-    if (tall_tiles * n_tiles >= compute_unit_count()) {
+    if (tall_tiles * n_tiles >= compute_units()) {
         const int m_tiles = static_cast<int>(tall_tiles);
         hipLaunchKernelGGL((gemm_f16_kernel<ENC, 2>), dim3(static_cast<unsigned>(m_tiles * n_tiles)),
                            dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,

@@ -1,14 +1,12 @@
-// Decode / small-batch GEMV on the int8 matrix cores.
+// Small-batch (2..16 rows) GEMV on the int8 matrix cores.
 //
-// A workgroup of 8 waves owns tiles of 32 consecutive weight rows (persistent:
-// it walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...).  The waves split the
-// K dimension by super-block ranges and meet once per tile in a fixed-order
-// sum.  A wave first loads its share of the activations and starts the loads
-// of its first packed blocks, then — while those fly — turns the activations
-// into two int8 planes (high and low byte of a 16-bit fixed-point code, one
-// scale per 256 values) kept in LDS for every tile it will visit; for 2..16
-// tokens the planes come from the workspace, written by a small quantizer
-// launch.  Per 256-value super-block the wave then
+// A small quantizer launch first turns the activations into two int8 planes
+// (high and low byte of a 16-bit fixed-point code, one scale per 256 values)
+// in the caller's workspace.  In the main kernel a workgroup of 8 waves owns
+// tiles of 32 consecutive weight rows (persistent: it walks tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ...).  The waves split the K dimension by
+// super-block ranges and meet once per tile in a fixed-order sum.  Per
+// 256-value super-block a wave
 //   1. stores its 32 x block_bytes of packed weights, loaded with coalesced
 //      16-byte accesses several blocks ahead (across tile boundaries), into a
 //      private LDS tile,
@@ -19,10 +17,10 @@
 //      sub-scale (24-bit multiply-add) and converts to float once per block.
 // Every weight byte is read from HBM exactly once per launch.
 //
-// Arithmetic it replaces: the reference's one-row and small-batch kernels
-// (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:714-890, 1174-1303), which
-// quantize activations to 8 bits; here 16 bits are kept so the result stays
-// within 2e-3 of the float-activation CPU engine
+// Arithmetic it replaces: the reference's small-batch kernel
+// (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:1174-1303), which quantizes
+// activations to 8 bits; here 16 bits are kept so the result stays within 2e-3
+// of the float-activation CPU engine
 // (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:655-679).  With x = s*c,
 // c = 256*hi + lo the 16-bit code of an activation and s its block scale:
 //   Q4_K/Q5_K: y += s*(d*sum_sub sc*dot(q, c) - dmin*sum_sub m*sum(c))
@@ -48,7 +46,6 @@ constexpr int kActRecord = kActivationRecordBytes;
 // sums of the codes per 32 values, [544,548) float scale, rest padding
 constexpr int kRecordSums = 512;
 constexpr int kRecordScale = 544;
-constexpr int kEarlyBlocks = 4;  // activation blocks per wave loaded before the weights
 
 struct __attribute__((packed, aligned(2))) Chunk16 {
     std::uint32_t v[4];
@@ -433,10 +430,9 @@ __device__ __forceinline__ void store_block(const uint4 (&staged)[TileSource<ENC
     }
 }
 
-template <std::uint32_t ENC, int S, bool FUSED, int P>
+template <std::uint32_t ENC, int S>
 __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
-    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
+    ProjectionSet set, const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
     int pass_capacity) {
     using F = Format<ENC>;
     using Source = TileSource<ENC>;
@@ -454,35 +450,21 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const std::int64_t begin = blocks * wave / kWaves;
     const std::int64_t end = blocks * (wave + 1) / kWaves;
     const int count = static_cast<int>(end - begin);
-    const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
 
-    // LDS: [waves][tile] | [2][waves][lanes][S] partial sums | [waves][max_count] records
+    // LDS: [waves][tile] | [2][waves][lanes][S] partial sums
     std::uint8_t* wave_tile = lds + wave * kTileBytes;
     float* partial = reinterpret_cast<float*>(lds + kWaves * kTileBytes);
-    std::uint8_t* wave_records =
-        lds + kWaves * kTileBytes + 2 * kWaves * kWave * S * 4 + wave * max_count * kActRecord;
 
     const int token0 = blockIdx.y * pass_capacity;
     const int pass_tokens = min(tokens - token0, pass_capacity);
     const std::uint8_t* pass_workspace =
-        FUSED ? nullptr : workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord;
+        workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord;
 
     const std::uint32_t first_tile = blockIdx.x;
 
     // Every load below is unconditional (indices are clamped instead): with a
     // fixed number of loads in flight the waits the compiler inserts are exact,
-    // so the quantizer only waits for the activations and a block only for its
-    // own chunks.
-    float4 x[FUSED ? kEarlyBlocks : 1];
-    if constexpr (FUSED) {
-        // activations first: their (short) latency must not queue behind the weights
-#pragma unroll
-        for (int b = 0; b < kEarlyBlocks; ++b) {
-            const int clamped = max(min(b, count - 1), 0);
-            x[b] = load_activations<P>(first, second, (begin + clamped) * 256 + lane * 4);
-        }
-    }
-
+    // so a block only waits for its own chunks.
     // Flat stream of (tile, block) pairs this wave processes; the prefetch
     // cursor runs kDepth pairs ahead of the processing cursor and stays on the
     // last pair once the stream is exhausted.
@@ -508,19 +490,6 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     for (int d = 0; d < kDepth; ++d) {
         fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[d]);
         advance_fetch();
-    }
-
-    if constexpr (FUSED) {
-#pragma unroll
-        for (int b = 0; b < kEarlyBlocks; ++b) {
-            if (b < count) quantize_block(x[b], lane, wave_records + b * kActRecord);
-        }
-        // more than kEarlyBlocks blocks per wave: quantize the rest now
-        for (int b = kEarlyBlocks; b < count; ++b) {
-            const float4 v = load_activations<P>(first, second, (begin + b) * 256 + lane * 4);
-            quantize_block(v, lane, wave_records + b * kActRecord);
-        }
-        wave_lds_fence();
     }
 
     // Which A row this lane supplies.
@@ -562,36 +531,22 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                     act.kc = kc;
                     act.keep = a_row.keep;
                     const std::int64_t block = begin + b;
-                    if constexpr (FUSED) {
-                        const std::uint8_t* record = wave_records + b * kActRecord;
-                        act.operand_base = record + a_row.plane * 256;
-                        act.scale[0] = *reinterpret_cast<const float*>(record + kRecordScale);
+                    const int operand_token = a_valid ? a_row.token : 0;
+                    act.operand_base = pass_workspace +
+                        (operand_token * blocks + block) * kActRecord + a_row.plane * 256;
+#pragma unroll
+                    for (int u = 0; u < S; ++u) {
+                        const int token = min(2 * u + kc, pass_tokens - 1);
+                        const std::uint8_t* record =
+                            pass_workspace + (token * blocks + block) * kActRecord;
+                        act.scale[u] = *reinterpret_cast<const float*>(record + kRecordScale);
                         if constexpr (!kQ6) {
                             const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
                             const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
-                            act.sums[0][0] = s0.x; act.sums[0][1] = s0.y;
-                            act.sums[0][2] = s0.z; act.sums[0][3] = s0.w;
-                            act.sums[0][4] = s1.x; act.sums[0][5] = s1.y;
-                            act.sums[0][6] = s1.z; act.sums[0][7] = s1.w;
-                        }
-                    } else {
-                        const int operand_token = a_valid ? a_row.token : 0;
-                        act.operand_base = pass_workspace +
-                            (operand_token * blocks + block) * kActRecord + a_row.plane * 256;
-#pragma unroll
-                        for (int u = 0; u < S; ++u) {
-                            const int token = min(2 * u + kc, pass_tokens - 1);
-                            const std::uint8_t* record =
-                                pass_workspace + (token * blocks + block) * kActRecord;
-                            act.scale[u] = *reinterpret_cast<const float*>(record + kRecordScale);
-                            if constexpr (!kQ6) {
-                                const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
-                                const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
-                                act.sums[u][0] = s0.x; act.sums[u][1] = s0.y;
-                                act.sums[u][2] = s0.z; act.sums[u][3] = s0.w;
-                                act.sums[u][4] = s1.x; act.sums[u][5] = s1.y;
-                                act.sums[u][6] = s1.z; act.sums[u][7] = s1.w;
-                            }
+                            act.sums[u][0] = s0.x; act.sums[u][1] = s0.y;
+                            act.sums[u][2] = s0.z; act.sums[u][3] = s0.w;
+                            act.sums[u][4] = s1.x; act.sums[u][5] = s1.y;
+                            act.sums[u][6] = s1.z; act.sums[u][7] = s1.w;
                         }
                     }
                     if constexpr (ENC == kEncQ4K) {
@@ -646,35 +601,17 @@ __global__ __launch_bounds__(256) void quantize_activations_kernel(
     quantize_block(x, lane, workspace + record * kActRecord);
 }
 
-int compute_units() {
-    static const int count = [] {
-        int device = 0;
-        int value = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-            value <= 0) {
-            return 256;
-        }
-        return value;
-    }();
-    return count;
-}
-
-template <std::uint32_t ENC, int S, bool FUSED, int P>
-void launch_variant(ProjectionSet set, const float* first, const float* second,
-                    const std::uint8_t* workspace, int tokens, int pass_capacity,
-                    hipStream_t stream) {
+template <std::uint32_t ENC, int S>
+void launch_variant(ProjectionSet set, const std::uint8_t* workspace, int tokens,
+                    int pass_capacity, hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
-    const std::int64_t blocks = set.input_dim >> 8;
-    const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
     const std::size_t lds = static_cast<std::size_t>(kWaves) * kTileRows * Format<ENC>::kLdsRow +
-        2u * kWaves * kWave * S * 4 +
-        (FUSED ? static_cast<std::size_t>(kWaves) * max_count * kActRecord : 0);
-    auto kernel = gemv_mfma_kernel<ENC, S, FUSED, P>;
+        2u * kWaves * kWave * S * 4;
+    auto kernel = gemv_mfma_kernel<ENC, S>;
     // More than 64 KB of dynamic LDS has to be allowed once per kernel.
     static const bool raised =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -684,40 +621,22 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
     const std::uint32_t grid = tiles < static_cast<std::uint32_t>(compute_units())
         ? tiles : static_cast<std::uint32_t>(compute_units());
-    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, stream, set, first, second,
-                       workspace, tokens, tiles, pass_capacity);
+    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, stream, set, workspace,
+                       tokens, tiles, pass_capacity);
 }
 
 template <std::uint32_t ENC>
-void launch_encoding(const ProjectionSet& set, const float* first, const float* second,
-                     int prologue, const std::uint8_t* workspace, int tokens,
+void launch_encoding(const ProjectionSet& set, const std::uint8_t* workspace, int tokens,
                      hipStream_t stream) {
     constexpr bool kQ6 = ENC == kEncQ6K;
-    if (tokens == 1) {
-        switch (prologue) {
-            case kGated:
-                launch_variant<ENC, 1, true, kGated>(set, first, second, nullptr, 1, 2, stream);
-                break;
-            case kSwiGlu:
-                launch_variant<ENC, 1, true, kSwiGlu>(set, first, second, nullptr, 1, 2, stream);
-                break;
-            default:
-                launch_variant<ENC, 1, true, kPlain>(set, first, second, nullptr, 1, 2, stream);
-                break;
-        }
-        return;
-    }
     if (tokens <= 2) {
-        launch_variant<ENC, 1, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 2, stream);
+        launch_variant<ENC, 1>(set, workspace, tokens, 2, stream);
     } else if (tokens <= 4) {
-        launch_variant<ENC, 2, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 4, stream);
+        launch_variant<ENC, 2>(set, workspace, tokens, 4, stream);
     } else if (tokens <= 8 || kQ6) {
-        launch_variant<ENC, 4, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 8, stream);
+        launch_variant<ENC, 4>(set, workspace, tokens, 8, stream);
     } else {
-        if constexpr (!kQ6) {
-            launch_variant<ENC, 8, false, kPlain>(set, nullptr, nullptr, workspace, tokens, 16,
-                                                 stream);
-        }
+        if constexpr (!kQ6) launch_variant<ENC, 8>(set, workspace, tokens, 16, stream);
     }
 }
 
@@ -733,8 +652,8 @@ void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second
                       std::int64_t rows, void* workspace, hipStream_t stream) {
     const int tokens = static_cast<int>(rows);
     std::uint8_t* ws = static_cast<std::uint8_t*>(workspace);
-    if (tokens > 1) {
-        // 2..16 tokens: quantize once into the workspace
+    {
+        // quantize the activations once into the workspace
         const std::int64_t records = rows * (set.input_dim >> 8);
         const dim3 grid(static_cast<unsigned>((records + 3) / 4));
         switch (prologue) {
@@ -762,11 +681,11 @@ void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second
         }
         if (group.count == 0) continue;
         if (encoding == kEncQ4K) {
-            launch_encoding<kEncQ4K>(group, first, second, prologue, ws, tokens, stream);
+            launch_encoding<kEncQ4K>(group, ws, tokens, stream);
         } else if (encoding == kEncQ5K) {
-            launch_encoding<kEncQ5K>(group, first, second, prologue, ws, tokens, stream);
+            launch_encoding<kEncQ5K>(group, ws, tokens, stream);
         } else {
-            launch_encoding<kEncQ6K>(group, first, second, prologue, ws, tokens, stream);
+            launch_encoding<kEncQ6K>(group, ws, tokens, stream);
         }
     }
 }

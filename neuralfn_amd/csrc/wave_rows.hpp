@@ -148,20 +148,6 @@ struct PairCursor {
     }
 };
 
-inline int compute_units() {
-    static const int count = [] {
-        int device = 0;
-        int value = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-            value <= 0) {
-            return 256;
-        }
-        return value;
-    }();
-    return count;
-}
-
 // Workgroups of a wave-per-row decode launch.  Small launches are bound by
 // fixed costs: waves start at a limited rate and every workgroup quantizes the
 // whole activation vector, so one workgroup per compute unit (all resident at
