@@ -355,7 +355,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 x int4 dot, f32 accumulate",
+        "dtype": "int8",
         "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K; bf16-rounded N(0,1) activations)",
         "config": {
             "workload": f"decode attention projections Q/K/V (grouped) + O, Q4_K, "

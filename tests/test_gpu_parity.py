@@ -567,7 +567,7 @@ def test_prefill_gemm_reserved_mode_is_refused(cuda):
 
 
 def test_prefill_gemm_full_size_row_subset(cuda, oracle):
-    # BASELINE shape (M=512, 6656 -> 16384): check a slice of output columns.
+    # the benchmark's prefill shape (M=512, 6656 -> 16384): check a slice of output columns.
     rows, out_dim, in_dim = 512, 16384, 6656
     torch = torch_()
     generator = torch.Generator(device="cpu").manual_seed(5)
