@@ -455,6 +455,37 @@ def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
     assert torch_().equal(unfused.max(dim=1).values.cpu(), maxima.cpu())
 
 
+@pytest.mark.parametrize("rows", [1, 4])
+def test_lm_head_full_vocabulary_planted_maxima(cuda, oracle, rows):
+    # The benchmark's lm_head (Q6_K, 6656 -> 202048, 1.1 GB) with random bytes
+    # and planted rows: every token's winner is known, one of them twice (the
+    # lower index must win), one at the last vocabulary row.
+    torch = torch_()
+    out_dim, in_dim = 202048, 6656
+    generator = torch.Generator(device=cuda).manual_seed(11)
+    blocks = torch.randint(0, 256, (out_dim * in_dim // 256, 210), generator=generator,
+                           device=cuda, dtype=torch.uint8)
+    blocks[:, 209] = (blocks[:, 209] & 0x03) | 0x14          # d in [2^-10, 2^-9)
+    packed = blocks.reshape(out_dim, -1)
+    x = kquant.synthetic_activations(95, rows, in_dim, rms_normalize=True)
+    planted = {0: [17, 150000], 1: [202047], 2: [101010], 3: [4096]}
+    expected_index, expected_value = [], []
+    for token in range(rows):
+        strong = (np.sign(x[token]) * 8.0).astype(np.float32).reshape(1, in_dim)
+        row_bytes = kquant.quantize(kquant.Q6_K, strong)
+        for index in planted[token]:
+            packed[index] = to_device(row_bytes, cuda)
+        expected_index.append(min(planted[token]))
+        expected_value.append(oracle.linear(kquant.Q6_K, row_bytes, 1, in_dim, x[token:token + 1])[0, 0])
+    weight = tile_ops.PackedWeight(kquant.Q6_K, out_dim, in_dim, packed.reshape(-1))
+    indices, maxima = tile_ops.lm_head_argmax(weight, to_device(x, cuda))
+    assert indices.cpu().tolist() == expected_index
+    for token in range(rows):
+        # a planted row of one token also scores against the other tokens, but never
+        # as high as that token's own planted row
+        assert abs(maxima.cpu()[token].item() - expected_value[token]) <= TOLERANCE * abs(expected_value[token])
+
+
 # ------------------------------------------------ the benchmark's geometries
 
 def config_layer(seed, encoding=kquant.Q4_K):
