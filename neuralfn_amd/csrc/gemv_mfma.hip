@@ -27,6 +27,7 @@
 //   Q6_K:      y += s*d*sum_16 sc8*dot(q - 32, c)
 #include "common.hpp"
 #include "gemv_mfma.hpp"
+#include "wave_rows.hpp"
 
 #include <type_traits>
 
@@ -40,7 +41,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kTileRows = 32;
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
-constexpr float kCodeRange = 32512.0f;  // 127*256: the high byte stays in [-127, 127]
 constexpr int kActRecord = kActivationRecordBytes;
 // record layout: [0,256) high plane, [256,512) low plane, [512,544) eight int32
 // sums of the codes per 32 values, [544,548) float scale, rest padding
@@ -78,85 +78,23 @@ struct Format<kEncQ6K> {
     static constexpr int kDepth = 3;
 };
 
-template <int CTRL>
-__device__ __forceinline__ int dpp_move(int value) {
-    return __builtin_amdgcn_update_dpp(0, value, CTRL, 0xF, 0xF, true);
-}
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float value) {
-    return __builtin_bit_cast(float, dpp_move<CTRL>(__builtin_bit_cast(int, value)));
-}
-
-constexpr int kQuadXor1 = 0xB1;     // quad_perm [1,0,3,2]
-constexpr int kQuadXor2 = 0x4E;     // quad_perm [2,3,0,1]
-constexpr int kHalfMirror = 0x141;  // lane k <-> 7-k within 8 lanes
-constexpr int kRowMirror = 0x140;   // lane k <-> 15-k within 16 lanes
-
-__device__ __forceinline__ float lane_value(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_move<kQuadXor1>(v));
-    v = fmaxf(v, dpp_move<kQuadXor2>(v));
-    v = fmaxf(v, dpp_move<kHalfMirror>(v));
-    v = fmaxf(v, dpp_move<kRowMirror>(v));
-    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
-                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
-}
-
-__device__ __forceinline__ std::uint32_t perm(std::uint32_t hi, std::uint32_t lo, std::uint32_t sel) {
-    return __builtin_amdgcn_perm(hi, lo, sel);
-}
-
 // Quantize the 256 activations of one block, four per lane, and write the
 // record (planes, per-32 code sums, scale) to `record` (LDS or workspace).
 __device__ __forceinline__ void quantize_block(float4 x, int lane, std::uint8_t* record) {
-    const float local = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
-    const float maximum = wave_max(local);
-    const float inverse = maximum > 1.0e-30f ? kCodeRange * __builtin_amdgcn_rcpf(maximum) : 0.0f;
-    const float scale = maximum * (1.0f / kCodeRange);
-    // 1.5*2^23 + 128: the low 16 bits of the sum's bit pattern are
-    // round-to-nearest-even(x*inverse) + 128 in two's complement.
-    constexpr float kMagic = 12582912.0f + 128.0f;
-    const std::uint32_t u0 = __float_as_uint(fmaf(x.x, inverse, kMagic));
-    const std::uint32_t u1 = __float_as_uint(fmaf(x.y, inverse, kMagic));
-    const std::uint32_t u2 = __float_as_uint(fmaf(x.z, inverse, kMagic));
-    const std::uint32_t u3 = __float_as_uint(fmaf(x.w, inverse, kMagic));
-    // code + 128 = 256*hi + (lo + 128): hi is byte 1, lo is byte 0 with its top bit flipped
-    const std::uint32_t p01 = perm(u1, u0, 0x05010400u);  // [u0.b0, u1.b0, u0.b1, u1.b1]
-    const std::uint32_t p23 = perm(u3, u2, 0x05010400u);
-    const std::uint32_t lo = perm(p23, p01, 0x05040100u) ^ 0x80808080u;
-    const std::uint32_t hi = perm(p23, p01, 0x07060302u);
-    // sum of the four codes, then over the 8 lanes of the 32-value group
-    int sum = (__builtin_amdgcn_sdot4(static_cast<int>(hi), 0x01010101, 0, false) << 8) +
-        __builtin_amdgcn_sdot4(static_cast<int>(lo), 0x01010101, 0, false);
+    const ActivationCodes codes = encode_activations(x);
+    // sum of the codes over the 8 lanes of a 32-value group
+    int sum = codes.sum;
     sum += dpp_move<kQuadXor1>(sum);
     sum += dpp_move<kQuadXor2>(sum);
     sum += dpp_move<kHalfMirror>(sum);
-    *reinterpret_cast<std::uint32_t*>(record + lane * 4) = hi;
-    *reinterpret_cast<std::uint32_t*>(record + 256 + lane * 4) = lo;
+    *reinterpret_cast<std::uint32_t*>(record + lane * 4) = codes.hi;
+    *reinterpret_cast<std::uint32_t*>(record + 256 + lane * 4) = codes.lo;
     if ((lane & 7) == 0) {
         *reinterpret_cast<int*>(record + kRecordSums + (lane >> 3) * 4) = sum;
     }
     if (lane == 0) {
-        *reinterpret_cast<float*>(record + kRecordScale) = scale;
+        *reinterpret_cast<float*>(record + kRecordScale) = codes.maximum * (1.0f / kCodeRange);
     }
-}
-
-template <int P>
-__device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
-                                                   const float* __restrict__ second,
-                                                   std::int64_t column) {
-    float4 x = *reinterpret_cast<const float4*>(first + column);
-    if constexpr (P != kPlain) {
-        const float4 y = *reinterpret_cast<const float4*>(second + column);
-        x.x = apply_prologue<P>(x.x, y.x);
-        x.y = apply_prologue<P>(x.y, y.y);
-        x.z = apply_prologue<P>(x.z, y.z);
-        x.w = apply_prologue<P>(x.w, y.w);
-    }
-    return x;
 }
 
 // Token <-> operand-row bookkeeping of v_mfma_i32_32x32x32_i8.  Output register
@@ -354,7 +292,32 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Where the chunks a lane copies for one tile come from and go to.
+// Projection a tile belongs to.
+__device__ __forceinline__ Projection tile_projection(const ProjectionSet& set, std::uint32_t tile) {
+    int which = 0;
+#pragma unroll
+    for (int index = 1; index < 4; ++index) {
+        if (index < set.count && tile >= set.op[index].first_tile) which = index;
+    }
+    return pick(set, which);
+}
+
+// Where the results of a tile go.
+struct TileOutput {
+    float* output;
+    std::int64_t output_dim;
+    std::int64_t row0;
+    int valid_rows;
+    __device__ __forceinline__ TileOutput(const ProjectionSet& set, std::uint32_t tile) {
+        const Projection op = tile_projection(set, tile);
+        row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
+        valid_rows = static_cast<int>(min(static_cast<std::int64_t>(kTileRows), op.output_dim - row0));
+        output = op.output;
+        output_dim = op.output_dim;
+    }
+};
+
+// Where the chunks a lane copies for one tile come from.
 template <std::uint32_t ENC>
 struct TileSource {
     using F = Format<ENC>;
@@ -363,24 +326,14 @@ struct TileSource {
     const std::uint8_t* base;      // first byte of the tile's first row (uniform)
     const std::uint8_t* data_end;  // end of the tensor (uniform)
     std::uint32_t offset[kLoads];  // byte offset of this lane's chunk i from base
-    float* output;
-    std::int64_t output_dim;
-    std::int64_t row0;
-    int valid_rows;
 
     __device__ __forceinline__ void setup(const ProjectionSet& set, std::uint32_t tile, int lane) {
-        int which = 0;
-#pragma unroll
-        for (int index = 1; index < 4; ++index) {
-            if (index < set.count && tile >= set.op[index].first_tile) which = index;
-        }
-        const Projection& op = set.op[which];
-        row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
-        valid_rows = static_cast<int>(min(static_cast<std::int64_t>(kTileRows), op.output_dim - row0));
+        const Projection op = tile_projection(set, tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
+        const int valid_rows =
+            static_cast<int>(min(static_cast<std::int64_t>(kTileRows), op.output_dim - row0));
         base = op.data + row0 * op.row_stride;
         data_end = op.data + op.output_dim * op.row_stride;
-        output = op.output;
-        output_dim = op.output_dim;
         const std::uint32_t stride = static_cast<std::uint32_t>(op.row_stride);
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
@@ -430,14 +383,42 @@ __device__ __forceinline__ void store_block(const uint4 (&staged)[TileSource<ENC
     }
 }
 
-template <std::uint32_t ENC, int S>
+// Where the int8 activation planes of a launch come from.
+//   kWorkspace: a quantizer launch wrote them to the caller's workspace.
+//   kResident:  every wave quantizes the activations of its own K range once,
+//               at the start, into LDS records it keeps for all its tiles; the
+//               float inputs are loaded before the first packed chunks and are
+//               dead before the main loop starts.  Needs LDS for tokens x blocks
+//               records.
+//   kStream:    every wave quantizes block by block; the float inputs of the
+//               blocks in flight sit in registers next to the packed chunks, so
+//               the prefetch depth is two.  No LDS limit on K.
+constexpr int kWorkspace = 0;
+constexpr int kResident = 1;
+constexpr int kStream = 2;
+constexpr int kEarlyBlocks = 4;  // blocks per wave whose inputs are loaded before the weights
+
+template <std::uint32_t ENC, int MODE>
+constexpr int prefetch_depth() {
+    return MODE == kStream ? 2 : Format<ENC>::kDepth;
+}
+
+// float4 registers one block's inputs take in a lane
+template <int S, int P>
+constexpr int input_registers() {
+    return 2 * S * (P == kPlain ? 1 : 2);
+}
+
+template <std::uint32_t ENC, int S, int MODE, int P>
 __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
-    ProjectionSet set, const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
+    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
+    const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
     int pass_capacity) {
     using F = Format<ENC>;
     using Source = TileSource<ENC>;
     constexpr bool kQ6 = ENC == kEncQ6K;
-    constexpr int kDepth = F::kDepth;
+    constexpr int kTokens = 2 * S;
+    constexpr int kDepth = prefetch_depth<ENC, MODE>();
     constexpr int kTileBytes = kTileRows * F::kLdsRow;
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
 
@@ -450,144 +431,209 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const std::int64_t begin = blocks * wave / kWaves;
     const std::int64_t end = blocks * (wave + 1) / kWaves;
     const int count = static_cast<int>(end - begin);
+    const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
 
-    // LDS: [waves][tile] | [2][waves][lanes][S] partial sums
+    // LDS: [waves][tile] | [2][waves][lanes][S] partial sums | records:
+    // kResident [waves][max_count][tokens], kStream [waves][tokens]
     std::uint8_t* wave_tile = lds + wave * kTileBytes;
     float* partial = reinterpret_cast<float*>(lds + kWaves * kTileBytes);
+    std::uint8_t* wave_records = lds + kWaves * kTileBytes + 2 * kWaves * kWave * S * 4 +
+        wave * (MODE == kResident ? max_count : 1) * kTokens * kActRecord;
 
     const int token0 = blockIdx.y * pass_capacity;
     const int pass_tokens = min(tokens - token0, pass_capacity);
-    const std::uint8_t* pass_workspace =
-        workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord;
+    const std::uint8_t* pass_workspace = MODE == kWorkspace
+        ? workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord : nullptr;
+    const float* pass_first =
+        MODE == kWorkspace ? nullptr : first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_second = MODE == kWorkspace || P == kPlain
+        ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+    // float inputs of block `block` of this wave's range for token slot t
+    auto load_input = [&](int block, int t) {
+        const int token = min(t, pass_tokens - 1);
+        return load_activations<P>(pass_first, pass_second,
+                                   static_cast<std::int64_t>(token) * set.input_dim +
+                                       (begin + block) * 256 + lane * 4);
+    };
 
+    // kResident: the inputs of the first blocks go out before anything else
+    float4 early[MODE == kResident ? kEarlyBlocks : 1][MODE == kResident ? kTokens : 1];
+    if constexpr (MODE == kResident) {
+#pragma unroll
+        for (int b = 0; b < kEarlyBlocks; ++b) {
+#pragma unroll
+            for (int t = 0; t < kTokens; ++t) early[b][t] = load_input(max(min(b, count - 1), 0), t);
+        }
+    }
+
+    // Every wave walks the same flat stream of (tile, step) pairs: its tiles are
+    // blockIdx.x, blockIdx.x + gridDim.x, ..., and a tile takes max_count steps
+    // for every wave (a wave whose K range is one block shorter idles in the
+    // last step), so the waves meet at the end of a tile in uniform control
+    // flow.  Loads run kDepth steps ahead of the arithmetic.  They are all
+    // unconditional (indices are clamped instead) and the loop body is
+    // unrolled over the kDepth register sets, so the compiler knows exactly
+    // how many loads were issued after the one a step needs and a step waits
+    // for nothing but its own chunks and activations.
     const std::uint32_t first_tile = blockIdx.x;
+    const int steps = max_count;
+    const int tile_count = static_cast<int>((total_tiles - first_tile + gridDim.x - 1) / gridDim.x);
+    const int total = tile_count * steps;
 
-    // Every load below is unconditional (indices are clamped instead): with a
-    // fixed number of loads in flight the waits the compiler inserts are exact,
-    // so a block only waits for its own chunks.
-    // Flat stream of (tile, block) pairs this wave processes; the prefetch
-    // cursor runs kDepth pairs ahead of the processing cursor and stays on the
-    // last pair once the stream is exhausted.
     Source fetch_source;
     std::uint32_t fetch_tile = first_tile;
-    int fetch_index = 0;
+    int fetch_step = 0;
     fetch_source.setup(set, fetch_tile, lane);
     uint4 staged[kDepth][Source::kLoads];
-    auto advance_fetch = [&]() {
-        if (fetch_index + 1 < count) {
-            ++fetch_index;
-        } else if (fetch_tile + gridDim.x < total_tiles) {
-            fetch_index = 0;
-            fetch_tile += gridDim.x;
-            fetch_source.setup(set, fetch_tile, lane);
-        } else {
-            // stream exhausted: the remaining (never used) fetches all hit one line
+    float4 inputs[MODE == kStream ? kDepth : 1][MODE == kStream ? kTokens : 1];
+    auto fetch = [&](uint4 (&chunks)[Source::kLoads], float4 (&slot)[MODE == kStream ? kTokens : 1]) {
+        const int block = max(min(fetch_step, count - 1), 0);
+        if constexpr (MODE == kStream) {
+            // the float activations of the block go out ahead of its chunks
 #pragma unroll
-            for (int i = 0; i < Source::kLoads; ++i) fetch_source.offset[i] = 0;
+            for (int t = 0; t < kTokens; ++t) slot[t] = load_input(block, t);
+        }
+        fetch_block<ENC>(fetch_source, begin + block, lane, chunks);
+        if (++fetch_step == steps) {
+            fetch_step = 0;
+            if (fetch_tile + gridDim.x < total_tiles) {
+                fetch_tile += gridDim.x;
+                fetch_source.setup(set, fetch_tile, lane);
+            } else {
+                // stream exhausted: the remaining (never used) fetches all hit one line
+#pragma unroll
+                for (int i = 0; i < Source::kLoads; ++i) fetch_source.offset[i] = 0;
+            }
         }
     };
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-        fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[d]);
-        advance_fetch();
+    for (int d = 0; d < kDepth; ++d) fetch(staged[d], inputs[MODE == kStream ? d : 0]);
+
+    if constexpr (MODE == kResident) {
+#pragma unroll
+        for (int b = 0; b < kEarlyBlocks; ++b) {
+#pragma unroll
+            for (int t = 0; t < kTokens; ++t) {
+                if (b < count && t < pass_tokens) {
+                    quantize_block(early[b][t], lane, wave_records + (b * kTokens + t) * kActRecord);
+                }
+            }
+        }
+        // a longer K range: the rest one block at a time
+        for (int b = kEarlyBlocks; b < count; ++b) {
+#pragma unroll
+            for (int t = 0; t < kTokens; ++t) {
+                const float4 x = load_input(b, t);
+                if (t < pass_tokens) {
+                    quantize_block(x, lane, wave_records + (b * kTokens + t) * kActRecord);
+                }
+            }
+        }
+        wave_lds_fence();
     }
 
     // Which A row this lane supplies.
     const OperandRow<kQ6> a_row(j, kc);
-    const bool a_valid = a_row.token < pass_tokens && a_row.token < 2 * S;
+    const bool a_valid = a_row.token < pass_tokens && a_row.token < kTokens;
+    const int operand_token = a_valid ? a_row.token : 0;
 
-    Source source;
+    std::uint32_t tile = first_tile;
+    int work_step = 0;
     int parity = 0;
-    int slot_base = 0;  // staging slot of the tile's first block, modulo kDepth
-    for (std::uint32_t tile = first_tile; tile < total_tiles; tile += gridDim.x) {
-        source.setup(set, tile, lane);
-        float acc[S];
+    float acc[S];
 #pragma unroll
-        for (int u = 0; u < S; ++u) acc[u] = 0.0f;
+    for (int u = 0; u < S; ++u) acc[u] = 0.0f;
 
-        for (int b = 0; b < count; ++b) {
-            {
-                {
-                    // staging slots rotate with the flat pair index
-                    const int slot = (slot_base + b) % kDepth;
-                    auto rotate = [&](auto slot_constant) {
-                        constexpr int kSlot = decltype(slot_constant)::value;
-                        store_block<ENC>(staged[kSlot], lane, wave_tile);
-                        fetch_block<ENC>(fetch_source, begin + fetch_index, lane, staged[kSlot]);
-                        advance_fetch();
-                    };
-                    if (slot == 0) {
-                        rotate(std::integral_constant<int, 0>{});
-                    } else if (slot == 1) {
-                        rotate(std::integral_constant<int, 1>{});
-                    } else if (slot == 2 || kDepth == 3) {
-                        rotate(std::integral_constant<int, 2>{});
-                    } else {
-                        rotate(std::integral_constant<int, kDepth - 1>{});
-                    }
-                    wave_lds_fence();
-
-                    BlockActivation<S> act;
-                    act.kc = kc;
-                    act.keep = a_row.keep;
-                    const std::int64_t block = begin + b;
-                    const int operand_token = a_valid ? a_row.token : 0;
-                    act.operand_base = pass_workspace +
-                        (operand_token * blocks + block) * kActRecord + a_row.plane * 256;
+    auto step = [&](uint4 (&chunks)[Source::kLoads], float4 (&slot)[MODE == kStream ? kTokens : 1],
+                    int position) {
+        if (position < total) {
+            if (work_step < count) {
+                store_block<ENC>(chunks, lane, wave_tile);
+                if constexpr (MODE == kStream) {
 #pragma unroll
-                    for (int u = 0; u < S; ++u) {
-                        const int token = min(2 * u + kc, pass_tokens - 1);
-                        const std::uint8_t* record =
-                            pass_workspace + (token * blocks + block) * kActRecord;
-                        act.scale[u] = *reinterpret_cast<const float*>(record + kRecordScale);
-                        if constexpr (!kQ6) {
-                            const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
-                            const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
-                            act.sums[u][0] = s0.x; act.sums[u][1] = s0.y;
-                            act.sums[u][2] = s0.z; act.sums[u][3] = s0.w;
-                            act.sums[u][4] = s1.x; act.sums[u][5] = s1.y;
-                            act.sums[u][6] = s1.z; act.sums[u][7] = s1.w;
+                    for (int t = 0; t < kTokens; ++t) {
+                        if (t < pass_tokens) {
+                            quantize_block(slot[t], lane, wave_records + t * kActRecord);
                         }
                     }
-                    if constexpr (ENC == kEncQ4K) {
-                        process_block_q45<S, false>(wave_tile, j, kc, act, acc);
-                    } else if constexpr (ENC == kEncQ5K) {
-                        process_block_q45<S, true>(wave_tile, j, kc, act, acc);
-                    } else {
-                        process_block_q6<S>(wave_tile, j, kc, act, acc);
-                    }
-                    wave_lds_fence();  // the next block's stores stay behind these reads
                 }
-            }
-        }
-        slot_base = (slot_base + count) % kDepth;
+                wave_lds_fence();
 
-        // Cross-wave sum in a fixed order; the two buffers alternate so one
-        // barrier per tile is enough.
-        float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * S;
+                BlockActivation<S> act;
+                act.kc = kc;
+                act.keep = a_row.keep;
+                // records of this block: one per token, in LDS or in the workspace
+                const std::uint8_t* records = MODE == kWorkspace
+                    ? pass_workspace + (begin + work_step) * kActRecord
+                    : wave_records + (MODE == kResident ? work_step * kTokens * kActRecord : 0);
+                const std::int64_t token_stride =
+                    MODE == kWorkspace ? blocks * kActRecord : kActRecord;
+                act.operand_base = records + operand_token * token_stride + a_row.plane * 256;
 #pragma unroll
-        for (int u = 0; u < S; ++u) mine[u] = acc[u];
-        __syncthreads();
-        if (wave == (parity ? kWaves - 1 : 0)) {
-#pragma unroll
-            for (int u = 0; u < S; ++u) {
-                const int token = 2 * u + kc;
-                float total = partial[((parity * kWaves + 0) * kWave + lane) * S + u];
-#pragma unroll
-                for (int w = 1; w < kWaves; ++w) {
-                    total += partial[((parity * kWaves + w) * kWave + lane) * S + u];
+                for (int u = 0; u < S; ++u) {
+                    const int token = min(2 * u + kc, pass_tokens - 1);
+                    const std::uint8_t* record = records + token * token_stride;
+                    act.scale[u] = *reinterpret_cast<const float*>(record + kRecordScale);
+                    if constexpr (!kQ6) {
+                        const int4 s0 = *reinterpret_cast<const int4*>(record + kRecordSums);
+                        const int4 s1 = *reinterpret_cast<const int4*>(record + kRecordSums + 16);
+                        act.sums[u][0] = s0.x; act.sums[u][1] = s0.y;
+                        act.sums[u][2] = s0.z; act.sums[u][3] = s0.w;
+                        act.sums[u][4] = s1.x; act.sums[u][5] = s1.y;
+                        act.sums[u][6] = s1.z; act.sums[u][7] = s1.w;
+                    }
                 }
-                if (token < pass_tokens && j < source.valid_rows) {
-                    source.output[static_cast<std::int64_t>(token0 + token) * source.output_dim +
-                                  source.row0 + j] = total;
+                if constexpr (ENC == kEncQ4K) {
+                    process_block_q45<S, false>(wave_tile, j, kc, act, acc);
+                } else if constexpr (ENC == kEncQ5K) {
+                    process_block_q45<S, true>(wave_tile, j, kc, act, acc);
+                } else {
+                    process_block_q6<S>(wave_tile, j, kc, act, acc);
                 }
+                wave_lds_fence();  // the next block's stores stay behind these reads
+            }
+            if (++work_step == steps) {
+                // Cross-wave sum in a fixed order; the two buffers alternate so
+                // one barrier per tile is enough.
+                float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * S;
+#pragma unroll
+                for (int u = 0; u < S; ++u) mine[u] = acc[u];
+                __syncthreads();
+                if (wave == (parity ? kWaves - 1 : 0)) {
+                    const TileOutput out(set, tile);
+#pragma unroll
+                    for (int u = 0; u < S; ++u) {
+                        const int token = 2 * u + kc;
+                        float sum = partial[((parity * kWaves + 0) * kWave + lane) * S + u];
+#pragma unroll
+                        for (int w = 1; w < kWaves; ++w) {
+                            sum += partial[((parity * kWaves + w) * kWave + lane) * S + u];
+                        }
+                        if (token < pass_tokens && j < out.valid_rows) {
+                            out.output[static_cast<std::int64_t>(token0 + token) * out.output_dim +
+                                       out.row0 + j] = sum;
+                        }
+                    }
+                }
+                parity ^= 1;
+                work_step = 0;
+                tile += gridDim.x;
+#pragma unroll
+                for (int u = 0; u < S; ++u) acc[u] = 0.0f;
             }
         }
-        parity ^= 1;
+        fetch(chunks, slot);
+    };
+
+    for (int position = 0; position < total; position += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            step(staged[d], inputs[MODE == kStream ? d : 0], position + d);
+        }
     }
 }
 
-// ---- activation quantizer for the multi-token passes -----------------------
+// ---- activation quantizer for the passes that do not quantize in the kernel --
 
 template <int P>
 __global__ __launch_bounds__(256) void quantize_activations_kernel(
@@ -601,76 +647,130 @@ __global__ __launch_bounds__(256) void quantize_activations_kernel(
     quantize_block(x, lane, workspace + record * kActRecord);
 }
 
-template <std::uint32_t ENC, int S>
-void launch_variant(ProjectionSet set, const std::uint8_t* workspace, int tokens,
-                    int pass_capacity, hipStream_t stream) {
+void launch_quantizer(const float* first, const float* second, int prologue, std::int64_t records,
+                      std::uint8_t* workspace, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>((records + 3) / 4));
+    switch (prologue) {
+        case kGated:
+            hipLaunchKernelGGL((quantize_activations_kernel<kGated>), grid, dim3(256), 0, stream,
+                               first, second, workspace, records);
+            break;
+        case kSwiGlu:
+            hipLaunchKernelGGL((quantize_activations_kernel<kSwiGlu>), grid, dim3(256), 0, stream,
+                               first, second, workspace, records);
+            break;
+        default:
+            hipLaunchKernelGGL((quantize_activations_kernel<kPlain>), grid, dim3(256), 0, stream,
+                               first, second, workspace, records);
+            break;
+    }
+}
+
+// What one launch needs beyond the projections.
+struct Pass {
+    const float* first;
+    const float* second;
+    int prologue;
+    std::uint8_t* workspace;
+    int tokens;
+    bool* quantized;  // whether the quantizer launch of this call has been enqueued
+    hipStream_t stream;
+};
+
+constexpr std::size_t kLdsBudget = 150 * 1024;
+
+template <std::uint32_t ENC, int S, int MODE>
+std::size_t lds_bytes(std::int64_t blocks) {
+    const std::size_t max_count = static_cast<std::size_t>((blocks + kWaves - 1) / kWaves);
+    const std::size_t records = MODE == kResident ? max_count : MODE == kStream ? 1 : 0;
+    return static_cast<std::size_t>(kWaves) * kTileRows * Format<ENC>::kLdsRow +
+        2u * kWaves * kWave * S * 4 + kWaves * records * 2u * S * kActRecord;
+}
+
+template <std::uint32_t ENC, int S, int MODE, int P>
+void launch_variant(ProjectionSet set, const Pass& pass) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
-    const std::size_t lds = static_cast<std::size_t>(kWaves) * kTileRows * Format<ENC>::kLdsRow +
-        2u * kWaves * kWave * S * 4;
-    auto kernel = gemv_mfma_kernel<ENC, S>;
+    if (MODE == kWorkspace && !*pass.quantized) {
+        launch_quantizer(pass.first, pass.second, pass.prologue,
+                         static_cast<std::int64_t>(pass.tokens) * (set.input_dim >> 8),
+                         pass.workspace, pass.stream);
+        *pass.quantized = true;
+    }
+    auto kernel = gemv_mfma_kernel<ENC, S, MODE, P>;
     // More than 64 KB of dynamic LDS has to be allowed once per kernel.
     static const bool raised =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
-    const int passes = (tokens + pass_capacity - 1) / pass_capacity;
+    const int pass_capacity = 2 * S;
+    const int passes = (pass.tokens + pass_capacity - 1) / pass_capacity;
     // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
     const std::uint32_t grid = tiles < static_cast<std::uint32_t>(compute_units())
         ? tiles : static_cast<std::uint32_t>(compute_units());
-    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, stream, set, workspace,
-                       tokens, tiles, pass_capacity);
+    const std::size_t lds = lds_bytes<ENC, S, MODE>(set.input_dim >> 8);
+    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, pass.stream, set,
+                       pass.first, pass.second, pass.workspace, pass.tokens, tiles, pass_capacity);
+}
+
+// Resident records where LDS holds them and the inputs of the early blocks fit
+// in registers, streamed quantization where only the latter holds, the
+// quantizer launch otherwise.
+template <std::uint32_t ENC, int S, int P>
+void launch_tokens(const ProjectionSet& set, const Pass& pass) {
+    constexpr bool kResidentFits = kEarlyBlocks * input_registers<S, P>() <= 16;
+    constexpr bool kStreamFits = 2 * input_registers<S, P>() <= 16;
+    if constexpr (kResidentFits) {
+        if (lds_bytes<ENC, S, kResident>(set.input_dim >> 8) <= kLdsBudget) {
+            launch_variant<ENC, S, kResident, P>(set, pass);
+            return;
+        }
+    }
+    if constexpr (kStreamFits) {
+        launch_variant<ENC, S, kStream, P>(set, pass);
+    } else {
+        launch_variant<ENC, S, kWorkspace, kPlain>(set, pass);
+    }
+}
+
+template <std::uint32_t ENC, int P>
+void launch_prologue(const ProjectionSet& set, const Pass& pass) {
+    constexpr bool kQ6 = ENC == kEncQ6K;
+    if (pass.tokens <= 2) {
+        launch_tokens<ENC, 1, P>(set, pass);
+    } else if (pass.tokens <= 4) {
+        launch_tokens<ENC, 2, P>(set, pass);
+    } else if (pass.tokens <= 8 || kQ6) {
+        launch_tokens<ENC, 4, P>(set, pass);
+    } else {
+        if constexpr (!kQ6) launch_tokens<ENC, 8, P>(set, pass);
+    }
 }
 
 template <std::uint32_t ENC>
-void launch_encoding(const ProjectionSet& set, const std::uint8_t* workspace, int tokens,
-                     hipStream_t stream) {
-    constexpr bool kQ6 = ENC == kEncQ6K;
-    if (tokens <= 2) {
-        launch_variant<ENC, 1>(set, workspace, tokens, 2, stream);
-    } else if (tokens <= 4) {
-        launch_variant<ENC, 2>(set, workspace, tokens, 4, stream);
-    } else if (tokens <= 8 || kQ6) {
-        launch_variant<ENC, 4>(set, workspace, tokens, 8, stream);
-    } else {
-        if constexpr (!kQ6) launch_variant<ENC, 8>(set, workspace, tokens, 16, stream);
+void launch_encoding(const ProjectionSet& set, const Pass& pass) {
+    switch (pass.prologue) {
+        case kGated: launch_prologue<ENC, kGated>(set, pass); break;
+        case kSwiGlu: launch_prologue<ENC, kSwiGlu>(set, pass); break;
+        default: launch_prologue<ENC, kPlain>(set, pass); break;
     }
 }
 
 }  // namespace
 
 bool gemv_mfma_supports(std::uint32_t encoding, std::int64_t input_dim) {
-    // the activation records of one wave's K range stay in LDS
     return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
         input_dim % 256 == 0 && input_dim <= 65536;
 }
 
 void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second, int prologue,
                       std::int64_t rows, void* workspace, hipStream_t stream) {
-    const int tokens = static_cast<int>(rows);
-    std::uint8_t* ws = static_cast<std::uint8_t*>(workspace);
-    {
-        // quantize the activations once into the workspace
-        const std::int64_t records = rows * (set.input_dim >> 8);
-        const dim3 grid(static_cast<unsigned>((records + 3) / 4));
-        switch (prologue) {
-            case kGated:
-                hipLaunchKernelGGL((quantize_activations_kernel<kGated>), grid, dim3(256), 0,
-                                   stream, first, second, ws, records);
-                break;
-            case kSwiGlu:
-                hipLaunchKernelGGL((quantize_activations_kernel<kSwiGlu>), grid, dim3(256), 0,
-                                   stream, first, second, ws, records);
-                break;
-            default:
-                hipLaunchKernelGGL((quantize_activations_kernel<kPlain>), grid, dim3(256), 0,
-                                   stream, first, second, ws, records);
-                break;
-        }
-    }
+    bool quantized = false;
+    const Pass pass{first, second, prologue, static_cast<std::uint8_t*>(workspace),
+                    static_cast<int>(rows), &quantized, stream};
     // one launch per encoding present
     const std::uint32_t encodings[3] = {kEncQ4K, kEncQ5K, kEncQ6K};
     for (const std::uint32_t encoding : encodings) {
@@ -681,11 +781,11 @@ void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second
         }
         if (group.count == 0) continue;
         if (encoding == kEncQ4K) {
-            launch_encoding<kEncQ4K>(group, ws, tokens, stream);
+            launch_encoding<kEncQ4K>(group, pass);
         } else if (encoding == kEncQ5K) {
-            launch_encoding<kEncQ5K>(group, ws, tokens, stream);
+            launch_encoding<kEncQ5K>(group, pass);
         } else {
-            launch_encoding<kEncQ6K>(group, ws, tokens, stream);
+            launch_encoding<kEncQ6K>(group, pass);
         }
     }
 }

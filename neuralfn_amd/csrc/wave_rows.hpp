@@ -25,13 +25,24 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-    v = fmaxf(v, dpp_move<kQuadXor1>(v));
-    v = fmaxf(v, dpp_move<kQuadXor2>(v));
-    v = fmaxf(v, dpp_move<kHalfMirror>(v));
-    v = fmaxf(v, dpp_move<kRowMirror>(v));
-    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)),
-                 fmaxf(lane_value(v, 32), lane_value(v, 48)));
+// Largest of the wave's values, all of them non-negative: such floats order
+// like their bit patterns, so the reduction runs on unsigned integers (one
+// instruction per step with the lane exchange folded in).  Butterfly within
+// rows of 16 lanes, then row 0 -> 1 and 2 -> 3, then lane 31 -> rows 2 and 3:
+// lane 63 holds the result.
+__device__ __forceinline__ float wave_max(float value) {
+    std::uint32_t v = __float_as_uint(value);
+    v = max(v, static_cast<std::uint32_t>(dpp_move<kQuadXor1>(static_cast<int>(v))));
+    v = max(v, static_cast<std::uint32_t>(dpp_move<kQuadXor2>(static_cast<int>(v))));
+    v = max(v, static_cast<std::uint32_t>(dpp_move<kHalfMirror>(static_cast<int>(v))));
+    v = max(v, static_cast<std::uint32_t>(dpp_move<kRowMirror>(static_cast<int>(v))));
+    constexpr int kRowBroadcast15 = 0x142, kRowBroadcast31 = 0x143;
+    v = max(v, static_cast<std::uint32_t>(__builtin_amdgcn_update_dpp(
+                   static_cast<int>(v), static_cast<int>(v), kRowBroadcast15, 0xA, 0xF, false)));
+    v = max(v, static_cast<std::uint32_t>(__builtin_amdgcn_update_dpp(
+                   static_cast<int>(v), static_cast<int>(v), kRowBroadcast31, 0xC, 0xF, false)));
+    return __uint_as_float(static_cast<std::uint32_t>(
+        __builtin_amdgcn_readlane(static_cast<int>(v), 63)));
 }
 
 // Sum over the wave in a fixed order; the total is returned in every lane.
