@@ -34,6 +34,9 @@ DEVICE_FLAGS = [
     "-ffp-contract=off",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # leading scalar and pointer arguments arrive in registers at wave start
+    # instead of through a first load from the argument block
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall",
     "-Wno-unused-function",
 ]

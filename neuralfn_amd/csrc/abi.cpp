@@ -71,8 +71,8 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
     // One row, and the verifier entry points at any row count: the vector-ALU
-    // kernels.  2..16 rows otherwise: the matrix-core kernel.  Encodings and
-    // widths without either: the float kernel.
+    // kernels.  2..16 rows otherwise: the matrix-core kernel (Q8_0: its dot
+    // kernel).  Encodings and widths without either: the float kernel.
     const bool one_row_arithmetic = rows == 1 || verifier;
     ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, exact{};
     dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = exact.input_dim = input_dim;
@@ -83,8 +83,8 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
             target = &dot;
         } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
             target = &dot6;
-        } else if (one_row_arithmetic && gemv_q8_supports(encoding, input_dim)) {
-            target = &dot8;
+        } else if (gemv_q8_supports(encoding, input_dim)) {
+            target = &dot8;  // Q8_0 has no matrix-core kernel: the dot kernel at any row count
         } else if (rows >= 2 && gemv_mfma_supports(encoding, input_dim)) {
             target = &matrix;
         }

@@ -92,8 +92,8 @@ struct Stage {
 
 template <std::uint32_t ENC, int T, int P>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
-    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows) {
+    const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
+    std::int64_t total_rows, ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
     constexpr int kQuants = kQ5 ? 48 : 16;
@@ -101,14 +101,14 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int blocks = static_cast<int>(set.input_dim >> 8);
+    const int blocks = input_dim >> 8;
     const int units = 4 * blocks;
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
     const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
 
     // rows of this wave: the rows are dealt out evenly over all waves of the grid
     // (counts differ by at most one), each wave a contiguous range
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         const int token = record / blocks;
         const int block = record - token * blocks;
         early[e] = load_activations<P>(pass_first, pass_second,
-                                       static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+                                       static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
     }
 
     // (2) weight loads of the first two (row, iteration) pairs
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,
-            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
     }
     __syncthreads();
@@ -303,7 +303,8 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     (void)raised;
     const int passes = (tokens + T - 1) / T;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kDotWaves)), passes),
-                       dim3(kDotThreads), lds, stream, set, first, second, tokens, rows);
+                       dim3(kDotThreads), lds, stream, first, second, tokens,
+                       static_cast<int>(set.input_dim), rows, set);
 }
 
 template <std::uint32_t ENC, int P>

@@ -411,9 +411,9 @@ constexpr int input_registers() {
 
 template <std::uint32_t ENC, int S, int MODE, int P>
 __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
-    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
+    const float* __restrict__ first, const float* __restrict__ second,
     const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
-    int pass_capacity) {
+    int pass_capacity, int input_dim, ProjectionSet set) {
     using F = Format<ENC>;
     using Source = TileSource<ENC>;
     constexpr bool kQ6 = ENC == kEncQ6K;
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 31;
     const int kc = lane >> 5;
-    const std::int64_t blocks = set.input_dim >> 8;
+    const std::int64_t blocks = input_dim >> 8;
     const std::int64_t begin = blocks * wave / kWaves;
     const std::int64_t end = blocks * (wave + 1) / kWaves;
     const int count = static_cast<int>(end - begin);
@@ -445,14 +445,14 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const std::uint8_t* pass_workspace = MODE == kWorkspace
         ? workspace + static_cast<std::int64_t>(token0) * blocks * kActRecord : nullptr;
     const float* pass_first =
-        MODE == kWorkspace ? nullptr : first + static_cast<std::int64_t>(token0) * set.input_dim;
+        MODE == kWorkspace ? nullptr : first + static_cast<std::int64_t>(token0) * input_dim;
     const float* pass_second = MODE == kWorkspace || P == kPlain
-        ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+        ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
     // float inputs of block `block` of this wave's range for token slot t
     auto load_input = [&](int block, int t) {
         const int token = min(t, pass_tokens - 1);
         return load_activations<P>(pass_first, pass_second,
-                                   static_cast<std::int64_t>(token) * set.input_dim +
+                                   static_cast<std::int64_t>(token) * input_dim +
                                        (begin + block) * 256 + lane * 4);
     };
 
@@ -712,8 +712,9 @@ void launch_variant(ProjectionSet set, const Pass& pass) {
     const std::uint32_t grid = tiles < static_cast<std::uint32_t>(compute_units())
         ? tiles : static_cast<std::uint32_t>(compute_units());
     const std::size_t lds = lds_bytes<ENC, S, MODE>(set.input_dim >> 8);
-    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, pass.stream, set,
-                       pass.first, pass.second, pass.workspace, pass.tokens, tiles, pass_capacity);
+    hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, pass.stream, pass.first,
+                       pass.second, pass.workspace, pass.tokens, tiles, pass_capacity,
+                       static_cast<int>(set.input_dim), set);
 }
 
 // Resident records where LDS holds them and the inputs of the early blocks fit

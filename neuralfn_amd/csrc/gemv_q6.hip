@@ -179,19 +179,19 @@ __device__ __forceinline__ void accumulate_unit(const UnitData& data, std::uint8
 
 template <int T, int P, bool ARGMAX>
 __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
-    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows, LmHeadCandidate* __restrict__ candidates) {
+    const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
+    std::int64_t total_rows, LmHeadCandidate* __restrict__ candidates, ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int blocks = static_cast<int>(set.input_dim >> 8);
+    const int blocks = input_dim >> 8;
     const int units = 4 * blocks;
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
     const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
 
     // rows of this wave: dealt out evenly over all waves of the grid, each wave
     // a contiguous range
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
         const int block = record - token * blocks;
         early[e] = load_activations<P>(
             pass_first, pass_second,
-            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
     }
 
     // (2) weight loads of the first two (row, slice) pairs
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,
-            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
     }
     __syncthreads();
@@ -381,8 +381,8 @@ struct PassLoads {
 // so more tokens per pass want more waves behind each image).
 template <int T, int P, bool ARGMAX, int W>
 __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
-    Projection op, std::int64_t input_dim, const float* __restrict__ first,
-    const float* __restrict__ second, int tokens, int rows_per_wave,
+    Projection op, const float* __restrict__ first, const float* __restrict__ second,
+    std::int64_t input_dim, int tokens, int rows_per_wave,
     LmHeadCandidate* __restrict__ candidates) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -624,7 +624,8 @@ std::int64_t launch_variant(ProjectionSet set, const float* first, const float* 
     const std::int64_t groups = decode_groups(rows, kWaves);
     const int passes = (tokens + T - 1) / T;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
-                       stream, set, first, second, tokens, rows, candidates);
+                       stream, first, second, tokens, static_cast<int>(set.input_dim), rows,
+                       candidates, set);
     return groups;
 }
 
@@ -660,7 +661,7 @@ std::int64_t launch_stream(const ProjectionSet& set, const float* first, const f
     for (int index = 0; index < set.count; ++index) {
         const Geometry g = stream_geometry(set.op[index].output_dim, W);
         hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(W * kWave),
-                           lds, stream, set.op[index], set.input_dim, first, second, tokens,
+                           lds, stream, set.op[index], first, second, set.input_dim, tokens,
                            static_cast<int>(g.rows_per_wave), candidates);
         groups = g.groups;
     }

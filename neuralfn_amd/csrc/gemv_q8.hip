@@ -79,19 +79,19 @@ struct Stage {
 
 template <int T, int P>
 __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
-    ProjectionSet set, const float* __restrict__ first, const float* __restrict__ second,
-    int tokens, std::int64_t total_rows) {
+    const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
+    std::int64_t total_rows, ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int blocks = static_cast<int>(set.input_dim >> 8);
+    const int blocks = input_dim >> 8;
     const int units = 4 * blocks;
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * set.input_dim;
+    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
     const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * set.input_dim;
+        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
 
     // rows of this wave: dealt out evenly over all waves of the grid, each wave
     // a contiguous range
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
         const int block = record - token * blocks;
         early[e] = load_activations<P>(
             pass_first, pass_second,
-            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
     }
 
     // (2) weight loads of the first two (row, slice) pairs
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,
-            static_cast<std::int64_t>(token) * set.input_dim + block * 256 + lane * 4);
+            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
     }
     __syncthreads();
@@ -255,7 +255,8 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     (void)raised;
     const int passes = (tokens + T - 1) / T;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kWaves)), passes),
-                       dim3(kThreads), lds, stream, set, first, second, tokens, rows);
+                       dim3(kThreads), lds, stream, first, second, tokens,
+                       static_cast<int>(set.input_dim), rows, set);
 }
 
 template <int P>
