@@ -93,7 +93,8 @@ struct Stage {
 template <std::uint32_t ENC, int T, int P>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    std::int64_t total_rows, ProjectionSet set) {
+    int total_rows, int rows_per_wave, int longer_waves,
+    ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
     constexpr int kQuants = kQ5 ? 48 : 16;
@@ -111,12 +112,10 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
 
     // rows of this wave: the rows are dealt out evenly over all waves of the grid
-    // (counts differ by at most one), each wave a contiguous range
-    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kDotWaves + wave;
-    const std::int64_t wave_total_count = static_cast<std::int64_t>(gridDim.x) * kDotWaves;
-    const std::int64_t row_begin = wave_index * total_rows / wave_total_count;
-    const int row_count =
-        static_cast<int>((wave_index + 1) * total_rows / wave_total_count - row_begin);
+    // (the first `longer_waves` take one more), each wave a contiguous range
+    const int wave_index = static_cast<int>(blockIdx.x) * kDotWaves + wave;
+    const int row_begin = wave_index * rows_per_wave + min(wave_index, longer_waves);
+    const int row_count = rows_per_wave + (wave_index < longer_waves ? 1 : 0);
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -302,9 +301,12 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
     const int passes = (tokens + T - 1) / T;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kDotWaves)), passes),
-                       dim3(kDotThreads), lds, stream, first, second, tokens,
-                       static_cast<int>(set.input_dim), rows, set);
+    const std::int64_t groups = decode_groups(rows, kDotWaves);
+    const std::int64_t waves = groups * kDotWaves;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
+                       stream, first, second, tokens, static_cast<int>(set.input_dim),
+                       static_cast<int>(rows), static_cast<int>(rows / waves),
+                       static_cast<int>(rows % waves), set);
 }
 
 template <std::uint32_t ENC, int P>

@@ -80,7 +80,8 @@ struct Stage {
 template <int T, int P>
 __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    std::int64_t total_rows, ProjectionSet set) {
+    int total_rows, int rows_per_wave, int longer_waves,
+    ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -95,11 +96,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
 
     // rows of this wave: dealt out evenly over all waves of the grid, each wave
     // a contiguous range
-    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * kWaves + wave;
-    const std::int64_t wave_total_count = static_cast<std::int64_t>(gridDim.x) * kWaves;
-    const std::int64_t row_begin = wave_index * total_rows / wave_total_count;
-    const int row_count =
-        static_cast<int>((wave_index + 1) * total_rows / wave_total_count - row_begin);
+    const int wave_index = static_cast<int>(blockIdx.x) * kWaves + wave;
+    const int row_begin = wave_index * rows_per_wave + min(wave_index, longer_waves);
+    const int row_count = rows_per_wave + (wave_index < longer_waves ? 1 : 0);
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -254,9 +253,12 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
     const int passes = (tokens + T - 1) / T;
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(decode_groups(rows, kWaves)), passes),
-                       dim3(kThreads), lds, stream, first, second, tokens,
-                       static_cast<int>(set.input_dim), rows, set);
+    const std::int64_t groups = decode_groups(rows, kWaves);
+    const std::int64_t waves = groups * kWaves;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
+                       stream, first, second, tokens, static_cast<int>(set.input_dim),
+                       static_cast<int>(rows), static_cast<int>(rows / waves),
+                       static_cast<int>(rows % waves), set);
 }
 
 template <int P>
