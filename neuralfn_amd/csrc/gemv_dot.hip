@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = min(wave + e * kDotWaves, records - 1);
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         early[e] = load_activations<P>(pass_first, pass_second,
                                        static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
@@ -159,13 +159,13 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kDotWaves;
         if (record < records) {
-            const int token = record / blocks;
+            const int token = token_of_record<T>(record, blocks);
             quantize_block(early[e], lane, record - token * blocks, blocks,
                            token_image(lds, token, blocks));
         }
     }
     for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,

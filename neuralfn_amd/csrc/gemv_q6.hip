@@ -210,7 +210,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = min(wave + e * kWaves, records - 1);
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         early[e] = load_activations<P>(
             pass_first, pass_second,
@@ -243,13 +243,13 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kWaves;
         if (record < records) {
-            const int token = record / blocks;
+            const int token = token_of_record<T>(record, blocks);
             quantize_block(early[e], lane, record - token * blocks, blocks,
                            token_image(lds, token, blocks));
         }
     }
     for (int record = wave + kEarly * kWaves; record < records; record += kWaves) {
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = min(wave + e * W, records - 1);
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         early[e] = load_activations<P>(
             pass_first, pass_second,
@@ -452,13 +452,13 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * W;
         if (record < records) {
-            const int token = record / blocks;
+            const int token = token_of_record<T>(record, blocks);
             quantize_block(early[e], lane, record - token * blocks, blocks,
                            token_image(lds, token, blocks));
         }
     }
     for (int record = wave + kEarly * W; record < records; record += W) {
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,

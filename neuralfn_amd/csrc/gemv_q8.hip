@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = min(wave + e * kWaves, records - 1);
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         early[e] = load_activations<P>(
             pass_first, pass_second,
@@ -140,13 +140,13 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kWaves;
         if (record < records) {
-            const int token = record / blocks;
+            const int token = token_of_record<T>(record, blocks);
             quantize_block(early[e], lane, record - token * blocks, blocks,
                            token_image(lds, token, blocks));
         }
     }
     for (int record = wave + kEarly * kWaves; record < records; record += kWaves) {
-        const int token = record / blocks;
+        const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
         const float4 x = load_activations<P>(
             pass_first, pass_second,

@@ -107,6 +107,17 @@ __device__ __forceinline__ float4 load_activations(const float* __restrict__ fir
     return x;
 }
 
+// Token of activation record `record` (records run token by token, `blocks`
+// per token).  One token per pass: no division on the way to the first loads.
+template <int T>
+__device__ __forceinline__ int token_of_record(int record, int blocks) {
+    if constexpr (T == 1) {
+        return 0;
+    } else {
+        return record / blocks;
+    }
+}
+
 // Projection `index` of the set, chosen with scalar selects from fields that
 // were all read with static offsets: a dynamically indexed read of the kernel
 // arguments is a dependent scalar load, and its first touch of a cache line
@@ -134,14 +145,14 @@ struct PairCursor {
     int iteration;            // which 64-unit slice of the row
     const std::uint8_t* row;  // first byte of the row
 
-    __device__ __forceinline__ void start(const ProjectionSet& set, std::int64_t global_row) {
+    __device__ __forceinline__ void start(const ProjectionSet& set, int global_row) {
         op = 0;
 #pragma unroll
         for (int index = 1; index < 4; ++index) {
-            if (index < set.count && global_row >= set.op[index].first_tile) op = index;
+            if (index < set.count && global_row >= static_cast<int>(set.op[index].first_tile)) op = index;
         }
         current = pick(set, op);
-        local_row = global_row - current.first_tile;
+        local_row = global_row - static_cast<int>(current.first_tile);
         iteration = 0;
         row = current.data + local_row * current.row_stride;
     }
