@@ -337,10 +337,10 @@ std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
                                                          std::int64_t output_dim) {
     if (rows < 1 || rows > 8 || output_dim <= 0) return 0;
     // room for either kernel's per-workgroup candidates
-    const std::int64_t f32_groups = lm_head_f32_blocks(output_dim);
-    const std::int64_t q6_groups = lm_head_q6_max_groups(output_dim);
-    const std::int64_t raw = rows * (f32_groups > q6_groups ? f32_groups : q6_groups) *
-        static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+    std::int64_t groups = lm_head_f32_blocks(output_dim);
+    if (lm_head_q6_max_groups(output_dim) > groups) groups = lm_head_q6_max_groups(output_dim);
+    if (lm_head_mfma_tiles(output_dim) > groups) groups = lm_head_mfma_tiles(output_dim);
+    const std::int64_t raw = rows * groups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
     return (raw + 255) & ~std::int64_t(255);
 }
 
@@ -357,7 +357,12 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
     const std::int64_t required =
         nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    if (gemv_q6_supports(normalized.encoding, normalized.input_dim)) {
+    // Two rows and more: the matrix-core kernel (one pass over the weights for
+    // up to four rows).  One row of Q6_K: the streaming dot kernel.
+    if (rows >= 2 && gemv_mfma_supports(normalized.encoding, normalized.input_dim)) {
+        launch_lm_head_mfma(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
+                            output_indices, output_values, as_stream(cuda_stream));
+    } else if (gemv_q6_supports(normalized.encoding, normalized.input_dim)) {
         launch_lm_head_q6(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
                           output_indices, output_values, as_stream(cuda_stream));
     } else {

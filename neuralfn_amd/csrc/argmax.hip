@@ -4,20 +4,13 @@
 // tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1869-1904.
 #include "common.hpp"
 #include "kernels.hpp"
+#include "lm_head.hpp"
 
 namespace nfn {
 
 namespace {
 
 constexpr int kArgmaxThreads = 1024;
-
-__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
-                                       std::int64_t& best_index) {
-    if (value > best_value || (value == best_value && index < best_index)) {
-        best_value = value;
-        best_index = index;
-    }
-}
 
 __global__ __launch_bounds__(kArgmaxThreads) void argmax_rows_kernel(
     const float* __restrict__ values, std::int64_t* __restrict__ indices,

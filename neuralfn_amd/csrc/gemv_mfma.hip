@@ -27,6 +27,7 @@
 //   Q6_K:      y += s*d*sum_16 sc8*dot(q - 32, c)
 #include "common.hpp"
 #include "gemv_mfma.hpp"
+#include "lm_head.hpp"
 #include "wave_rows.hpp"
 
 #include <type_traits>
@@ -409,11 +410,15 @@ constexpr int input_registers() {
     return 2 * S * (P == kPlain ? 1 : 2);
 }
 
-template <std::uint32_t ENC, int S, int MODE, int P>
+// ARGMAX: instead of storing the results the workgroup keeps, per token, the
+// best (value, row) of each tile in `candidates` ([tokens][tiles]); a second
+// launch reduces them, so the logits of an lm_head never reach memory.
+template <std::uint32_t ENC, int S, int MODE, int P, bool ARGMAX>
 __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const float* __restrict__ first, const float* __restrict__ second,
     const std::uint8_t* __restrict__ workspace, int tokens, std::uint32_t total_tiles,
-    int pass_capacity, int input_dim, ProjectionSet set) {
+    int pass_capacity, int input_dim, LmHeadCandidate* __restrict__ candidates,
+    ProjectionSet set) {
     using F = Format<ENC>;
     using Source = TileSource<ENC>;
     constexpr bool kQ6 = ENC == kEncQ6K;
@@ -609,7 +614,25 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                         for (int w = 1; w < kWaves; ++w) {
                             sum += partial[((parity * kWaves + w) * kWave + lane) * S + u];
                         }
-                        if (token < pass_tokens && j < out.valid_rows) {
+                        if constexpr (ARGMAX) {
+                            // best of the tile's 32 rows within each half of the wave
+                            float value = j < out.valid_rows ? sum : -INFINITY;
+                            std::int64_t index = out.row0 + j;
+#pragma unroll
+                            for (int offset = 16; offset > 0; offset >>= 1) {
+                                const float other_value = __shfl_xor(value, offset, 64);
+                                const std::int64_t other_index = __shfl_xor(index, offset, 64);
+                                better(other_value, other_index, value, index);
+                            }
+                            if (j == 0 && token < pass_tokens) {
+                                LmHeadCandidate candidate;
+                                candidate.index = index;
+                                candidate.value = value;
+                                candidate.pad = 0;
+                                candidates[static_cast<std::int64_t>(token0 + token) * total_tiles +
+                                           tile] = candidate;
+                            }
+                        } else if (token < pass_tokens && j < out.valid_rows) {
                             out.output[static_cast<std::int64_t>(token0 + token) * out.output_dim +
                                        out.row0 + j] = sum;
                         }
@@ -674,6 +697,7 @@ struct Pass {
     std::uint8_t* workspace;
     int tokens;
     bool* quantized;  // whether the quantizer launch of this call has been enqueued
+    LmHeadCandidate* candidates;  // lm_head: per-tile candidates instead of outputs
     hipStream_t stream;
 };
 
@@ -687,7 +711,7 @@ std::size_t lds_bytes(std::int64_t blocks) {
         2u * kWaves * kWave * S * 4 + kWaves * records * 2u * S * kActRecord;
 }
 
-template <std::uint32_t ENC, int S, int MODE, int P>
+template <std::uint32_t ENC, int S, int MODE, int P, bool ARGMAX>
 void launch_variant(ProjectionSet set, const Pass& pass) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
@@ -700,7 +724,7 @@ void launch_variant(ProjectionSet set, const Pass& pass) {
                          pass.workspace, pass.stream);
         *pass.quantized = true;
     }
-    auto kernel = gemv_mfma_kernel<ENC, S, MODE, P>;
+    auto kernel = gemv_mfma_kernel<ENC, S, MODE, P, ARGMAX>;
     // More than 64 KB of dynamic LDS has to be allowed once per kernel.
     static const bool raised =
         hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -714,64 +738,57 @@ void launch_variant(ProjectionSet set, const Pass& pass) {
     const std::size_t lds = lds_bytes<ENC, S, MODE>(set.input_dim >> 8);
     hipLaunchKernelGGL(kernel, dim3(grid, passes), dim3(kThreads), lds, pass.stream, pass.first,
                        pass.second, pass.workspace, pass.tokens, tiles, pass_capacity,
-                       static_cast<int>(set.input_dim), set);
+                       static_cast<int>(set.input_dim), pass.candidates, set);
 }
 
 // Resident records where LDS holds them and the inputs of the early blocks fit
 // in registers, streamed quantization where only the latter holds, the
 // quantizer launch otherwise.
-template <std::uint32_t ENC, int S, int P>
+template <std::uint32_t ENC, int S, int P, bool ARGMAX>
 void launch_tokens(const ProjectionSet& set, const Pass& pass) {
     constexpr bool kResidentFits = kEarlyBlocks * input_registers<S, P>() <= 16;
     constexpr bool kStreamFits = 2 * input_registers<S, P>() <= 16;
     if constexpr (kResidentFits) {
         if (lds_bytes<ENC, S, kResident>(set.input_dim >> 8) <= kLdsBudget) {
-            launch_variant<ENC, S, kResident, P>(set, pass);
+            launch_variant<ENC, S, kResident, P, ARGMAX>(set, pass);
             return;
         }
     }
     if constexpr (kStreamFits) {
-        launch_variant<ENC, S, kStream, P>(set, pass);
+        launch_variant<ENC, S, kStream, P, ARGMAX>(set, pass);
     } else {
-        launch_variant<ENC, S, kWorkspace, kPlain>(set, pass);
+        launch_variant<ENC, S, kWorkspace, kPlain, ARGMAX>(set, pass);
     }
 }
 
-template <std::uint32_t ENC, int P>
+template <std::uint32_t ENC, int P, bool ARGMAX>
 void launch_prologue(const ProjectionSet& set, const Pass& pass) {
     constexpr bool kQ6 = ENC == kEncQ6K;
     if (pass.tokens <= 2) {
-        launch_tokens<ENC, 1, P>(set, pass);
+        launch_tokens<ENC, 1, P, ARGMAX>(set, pass);
     } else if (pass.tokens <= 4) {
-        launch_tokens<ENC, 2, P>(set, pass);
+        launch_tokens<ENC, 2, P, ARGMAX>(set, pass);
     } else if (pass.tokens <= 8 || kQ6) {
-        launch_tokens<ENC, 4, P>(set, pass);
+        launch_tokens<ENC, 4, P, ARGMAX>(set, pass);
     } else {
-        if constexpr (!kQ6) launch_tokens<ENC, 8, P>(set, pass);
+        if constexpr (!kQ6 && !ARGMAX) launch_tokens<ENC, 8, P, false>(set, pass);
     }
 }
 
 template <std::uint32_t ENC>
 void launch_encoding(const ProjectionSet& set, const Pass& pass) {
+    if (pass.candidates != nullptr) {
+        launch_prologue<ENC, kPlain, true>(set, pass);
+        return;
+    }
     switch (pass.prologue) {
-        case kGated: launch_prologue<ENC, kGated>(set, pass); break;
-        case kSwiGlu: launch_prologue<ENC, kSwiGlu>(set, pass); break;
-        default: launch_prologue<ENC, kPlain>(set, pass); break;
+        case kGated: launch_prologue<ENC, kGated, false>(set, pass); break;
+        case kSwiGlu: launch_prologue<ENC, kSwiGlu, false>(set, pass); break;
+        default: launch_prologue<ENC, kPlain, false>(set, pass); break;
     }
 }
 
-}  // namespace
-
-bool gemv_mfma_supports(std::uint32_t encoding, std::int64_t input_dim) {
-    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
-        input_dim % 256 == 0 && input_dim <= 65536;
-}
-
-void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second, int prologue,
-                      std::int64_t rows, void* workspace, hipStream_t stream) {
-    bool quantized = false;
-    const Pass pass{first, second, prologue, static_cast<std::uint8_t*>(workspace),
-                    static_cast<int>(rows), &quantized, stream};
+void launch_groups(const ProjectionSet& set, const Pass& pass) {
     // one launch per encoding present
     const std::uint32_t encodings[3] = {kEncQ4K, kEncQ5K, kEncQ6K};
     for (const std::uint32_t encoding : encodings) {
@@ -789,6 +806,44 @@ void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second
             launch_encoding<kEncQ6K>(group, pass);
         }
     }
+}
+
+}  // namespace
+
+bool gemv_mfma_supports(std::uint32_t encoding, std::int64_t input_dim) {
+    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
+        input_dim % 256 == 0 && input_dim <= 65536;
+}
+
+void launch_gemv_mfma(ProjectionSet set, const float* first, const float* second, int prologue,
+                      std::int64_t rows, void* workspace, hipStream_t stream) {
+    bool quantized = false;
+    const Pass pass{first, second, prologue, static_cast<std::uint8_t*>(workspace),
+                    static_cast<int>(rows), &quantized, nullptr, stream};
+    launch_groups(set, pass);
+}
+
+std::int64_t lm_head_mfma_tiles(std::int64_t output_dim) {
+    return (output_dim + kTileRows - 1) / kTileRows;
+}
+
+void launch_lm_head_mfma(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                         LmHeadCandidate* candidates, std::int64_t* indices, float* maxima,
+                         hipStream_t stream) {
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = descriptor.input_dim;
+    set.op[0].data = descriptor.data;
+    set.op[0].output = nullptr;
+    set.op[0].output_dim = descriptor.output_dim;
+    set.op[0].row_stride = descriptor.row_stride_bytes;
+    set.op[0].encoding = descriptor.encoding;
+    bool quantized = false;  // up to eight rows always quantize in the kernel
+    const Pass pass{input, nullptr, kPlain, nullptr, static_cast<int>(rows), &quantized, candidates,
+                    stream};
+    launch_groups(set, pass);
+    launch_lm_head_final(candidates, lm_head_mfma_tiles(descriptor.output_dim), indices, maxima,
+                         rows, stream);
 }
 
 }  // namespace nfn

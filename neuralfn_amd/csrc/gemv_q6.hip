@@ -105,14 +105,6 @@ struct Stage {
     std::uint32_t d_bits;
 };
 
-__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
-                                       std::int64_t& best_index) {
-    if (value > best_value || (value == best_value && index < best_index)) {
-        best_value = value;
-        best_index = index;
-    }
-}
-
 // The packed bytes of one unit: 64 values = positions 16*sixteen .. +15 of the
 // four quarters of one half of a block.
 struct UnitData {

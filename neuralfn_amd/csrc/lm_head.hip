@@ -18,14 +18,6 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 
-__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
-                                       std::int64_t& best_index) {
-    if (value > best_value || (value == best_value && index < best_index)) {
-        best_value = value;
-        best_index = index;
-    }
-}
-
 template <int R>
 __global__ __launch_bounds__(kWavesPerBlock * kWave) void lm_head_partial_kernel(
     Projection op, std::int64_t input_dim, const float* __restrict__ input, std::int64_t rows,

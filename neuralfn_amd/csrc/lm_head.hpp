@@ -13,6 +13,16 @@ struct LmHeadCandidate {
     std::uint32_t pad;
 };
 
+// Keeps the larger value; equal values keep the lower index (the reference's
+// first-maximum rule, neuralfn/csrc/tile_cuda/kernels.cu:1564-1602).
+__device__ __forceinline__ void better(float value, std::int64_t index, float& best_value,
+                                       std::int64_t& best_index) {
+    if (value > best_value || (value == best_value && index < best_index)) {
+        best_value = value;
+        best_index = index;
+    }
+}
+
 // Pass 2: one workgroup per input row reduces `candidate_count` candidates.
 void launch_lm_head_final(const LmHeadCandidate* candidates, std::int64_t candidate_count,
                           std::int64_t* indices, float* maxima, std::int64_t rows,

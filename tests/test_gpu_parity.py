@@ -383,18 +383,21 @@ def test_lm_head_fused_argmax_against_oracle(cuda, oracle, encoding, rows):
             assert logits[row, indices.cpu()[row].item()] >= ordered[0] - 2 * TOLERANCE * scale
 
 
-def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda):
-    # Two identical vocabulary rows far apart: the lower index must win.
+@pytest.mark.parametrize("rows", [1, 2, 5])
+def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda, rows):
+    # Identical vocabulary rows, two in one 32-row tile and one far away: the
+    # lowest index must win for every token (all tokens carry the same input).
     out_dim, in_dim = 3000, 512
     w = kquant.synthetic_weights(5, out_dim, in_dim)
-    x = kquant.synthetic_activations(6, 1, in_dim)
+    x = np.repeat(kquant.synthetic_activations(6, 1, in_dim), rows, axis=0)
     best = w[100] * 0 + np.sign(x[0]) * 0.05
     w[100] = best
+    w[110] = best
     w[2900] = best
     packed = kquant.quantize(kquant.Q6_K, w)
     weight = tile_ops.PackedWeight.from_numpy(kquant.Q6_K, packed, out_dim, in_dim)
     indices, _ = tile_ops.lm_head_argmax(weight, to_device(x, cuda))
-    assert indices.cpu().tolist() == [100]
+    assert indices.cpu().tolist() == [100] * rows
 
 
 @pytest.mark.parametrize("shape", [(130, 256), (515, 6656)])
@@ -451,7 +454,8 @@ def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
             assert indices.cpu()[row].item() == oracle.argmax(logits[row])
     # the fused result equals argmax over the unfused logits of the same kernel
     workspace = tile_ops.small_batch_workspace(rows, in_dim)
-    unfused = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family="mmvq")[0]
+    family = "mmvq" if rows == 1 else "mmq"  # one row: dot kernel; more: matrix cores
+    unfused = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family=family)[0]
     assert torch_().equal(unfused.max(dim=1).values.cpu(), maxima.cpu())
 
 
