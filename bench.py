@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # WRITE_SIZE counters of a `--traffic-probe` run, each calibrated on a plain
 # copy of known size; the figures and commands are in
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_648_540}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_607_181}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
 FFN_DIM = 16384
@@ -220,6 +220,26 @@ def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
     }
 
 
+def decode_batch_extra(layers, device, stream, steps: int, warmup: int, headline_rows: int) -> dict:
+    """The headline workload at the other batch sizes of the same configuration."""
+    import torch
+
+    result = {"workload": "decode attention projections as the headline, other batch sizes, HIP-graph replay"}
+    for rows in (1, 4, 8):
+        if rows == headline_rows:
+            continue
+        step = DecodeStep(layers, rows, device)
+        ms = time_graph(lambda: step.enqueue(int(torch.cuda.current_stream().cuda_stream)),
+                        stream, steps, warmup)
+        traffic = len(layers) * layer_algorithmic_bytes(rows)
+        result[f"rows{rows}"] = {
+            "ms_per_step": round(ms, 5), "GB/s": round(traffic / ms / 1e6, 1),
+            "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(ms * 1e3 / step.launches_per_step, 3),
+            "tokens/s": round(rows / ms * 1e3, 1)}
+    return result
+
+
 def random_packed_on_device(encoding: int, out_dim: int, in_dim: int, device, seed: int):
     """Uniform random quant bytes with small finite scales, made on the GPU.
 
@@ -383,6 +403,8 @@ def main() -> int:
     if not args.no_extras:
         try:
             with torch.cuda.stream(stream):
+                record["decode_batches"] = decode_batch_extra(layers, device, stream, args.steps,
+                                                              args.warmup, args.rows)
                 record["lm_head"] = lm_head_extra(device, stream, args.steps, args.warmup)
                 record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
