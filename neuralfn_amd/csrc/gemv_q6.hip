@@ -372,9 +372,8 @@ struct PassLoads {
 // so more tokens per pass want more waves behind each image).
 template <int T, int P, bool ARGMAX, int W>
 __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
-    Projection op, const float* __restrict__ first, const float* __restrict__ second,
-    std::int64_t input_dim, int tokens, int rows_per_wave,
-    LmHeadCandidate* __restrict__ candidates) {
+    const float* __restrict__ first, const float* __restrict__ second, std::int64_t input_dim,
+    int tokens, int rows_per_wave, LmHeadCandidate* __restrict__ candidates, ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -386,9 +385,17 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
     std::uint8_t* staging = lds + T * token_image_bytes(blocks) + wave * kStagingBytes;
 
-    // rows and blocks of this wave
-    const std::int64_t wave_index = static_cast<std::int64_t>(blockIdx.x) * W + wave;
-    const std::int64_t row_begin = wave_index * rows_per_wave;
+    // rows and blocks of this wave: every projection owns a range of waves
+    // (first_tile is its first wave), a wave a contiguous range of its rows
+    const int wave_index = static_cast<int>(blockIdx.x) * W + wave;
+    int which = 0;
+#pragma unroll
+    for (int index = 1; index < 4; ++index) {
+        if (index < set.count && wave_index >= static_cast<int>(set.op[index].first_tile)) which = index;
+    }
+    const Projection op = pick(set, which);
+    const std::int64_t row_begin =
+        static_cast<std::int64_t>(wave_index - static_cast<int>(op.first_tile)) * rows_per_wave;
     const int row_count = static_cast<int>(max(
         static_cast<std::int64_t>(0),
         min(static_cast<std::int64_t>(rows_per_wave), op.output_dim - row_begin)));
@@ -628,6 +635,12 @@ std::int64_t launch_variant(ProjectionSet set, const float* first, const float* 
 Geometry stream_geometry(std::int64_t rows, int waves_per_group) {
     Geometry g = geometry(rows);
     if (g.rows_per_wave >= 8) g.rows_per_wave &= ~std::int64_t(7);
+    // few rows: up to eight per wave, as many as one workgroup per compute
+    // unit would get, so that a workgroup's quantization of the activations
+    // serves more than a handful of rows
+    const std::int64_t resident = static_cast<std::int64_t>(compute_units()) * waves_per_group;
+    const std::int64_t share = (rows + resident - 1) / resident;
+    if (g.rows_per_wave < 8) g.rows_per_wave = share < 8 ? share : 8;
     g.groups = (rows + g.rows_per_wave * waves_per_group - 1) / (g.rows_per_wave * waves_per_group);
     return g;
 }
@@ -649,15 +662,20 @@ std::int64_t launch_stream(const ProjectionSet& set, const float* first, const f
                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
     (void)raised;
     const int passes = (tokens + T - 1) / T;
-    // one launch per projection: a wave's rows must be contiguous in memory
-    std::int64_t groups = 0;
-    for (int index = 0; index < set.count; ++index) {
-        const Geometry g = stream_geometry(set.op[index].output_dim, W);
-        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(g.groups), passes), dim3(W * kWave),
-                           lds, stream, set.op[index], first, second, set.input_dim, tokens,
-                           static_cast<int>(g.rows_per_wave), candidates);
-        groups = g.groups;
+    // one launch: the projections take consecutive ranges of waves
+    std::int64_t rows = 0;
+    for (int index = 0; index < set.count; ++index) rows += set.op[index].output_dim;
+    const std::int64_t rows_per_wave = stream_geometry(rows, W).rows_per_wave;
+    ProjectionSet placed = set;
+    std::int64_t waves = 0;
+    for (int index = 0; index < placed.count; ++index) {
+        placed.op[index].first_tile = static_cast<std::uint32_t>(waves);
+        waves += (placed.op[index].output_dim + rows_per_wave - 1) / rows_per_wave;
     }
+    const std::int64_t groups = (waves + W - 1) / W;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(W * kWave), lds,
+                       stream, first, second, set.input_dim, tokens, static_cast<int>(rows_per_wave),
+                       candidates, placed);
     return groups;
 }
 
