@@ -306,6 +306,77 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
                         "incl. activation conversion", **result}
 
 
+def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
+    """Four layers of attention and FFN projections with per-tensor formats drawn by seed
+    from {Q4_K, Q5_K, Q6_K, Q8_0} (V, O and down at least Q5_K), at one row (decode)
+    and 1024 rows (prefill): per-format dispatch through the same entry points."""
+    import random
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+
+    draw = random.Random(4)
+    every = [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0]
+    wide = [kquant.Q5_K, kquant.Q6_K, kquant.Q8_0]
+    shapes = {"q": (ATTN_DIM, MODEL_DIM), "k": (KV_DIM, MODEL_DIM), "v": (KV_DIM, MODEL_DIM),
+              "o": (MODEL_DIM, ATTN_DIM), "gate": (FFN_DIM, MODEL_DIM), "up": (FFN_DIM, MODEL_DIM),
+              "down": (MODEL_DIM, FFN_DIM)}
+    layers, formats = [], []
+    for layer in range(4):
+        chosen = {name: draw.choice(wide if name in ("v", "o", "down") else every) for name in shapes}
+        formats.append("/".join(kquant.NAMES[chosen[name]] for name in shapes))
+        layers.append({name: random_packed_on_device(chosen[name], *shapes[name], device,
+                                                     100 + 10 * layer + index)
+                       for index, name in enumerate(shapes)})
+    weight_bytes = sum(weight.nbytes for layer in layers for weight in layer.values())
+    flops_per_row = sum(2.0 * w.input_dim * w.output_dim for layer in layers for w in layer.values())
+    inputs = {MODEL_DIM: kquant.synthetic_activations(41, 1024, MODEL_DIM),
+              ATTN_DIM: kquant.synthetic_activations(42, 1024, ATTN_DIM),
+              FFN_DIM: kquant.synthetic_activations(43, 1024, FFN_DIM)}
+    result = {"workload": "4 layers of Q/K/V (grouped), O, gate+up (grouped), down with seeded per-tensor formats",
+              "formats_q_k_v_o_gate_up_down": formats}
+
+    # decode: one row, the small-batch entry point, grouped where the engine groups
+    x = {dim: torch.from_numpy(values[:1].copy()).to(device) for dim, values in inputs.items()}
+    outs = [{name: torch.empty((1, w.output_dim), dtype=torch.float32, device=device)
+             for name, w in layer.items()} for layer in layers]
+    workspace = tile_ops.small_batch_workspace(1, FFN_DIM)
+
+    def decode():
+        for layer, out in zip(layers, outs):
+            tile_ops.multi_linear([layer["q"], layer["k"], layer["v"]], x[MODEL_DIM], workspace,
+                                  outputs=[out["q"], out["k"], out["v"]])
+            tile_ops.multi_linear([layer["o"]], x[ATTN_DIM], workspace, outputs=[out["o"]])
+            tile_ops.multi_linear([layer["gate"], layer["up"]], x[MODEL_DIM], workspace,
+                                  outputs=[out["gate"], out["up"]])
+            tile_ops.multi_linear([layer["down"]], x[FFN_DIM], workspace, outputs=[out["down"]])
+
+    ms = time_graph(decode, stream, steps, warmup)
+    result["decode_rows1"] = {"ms": round(ms, 4), "GB/s": round(weight_bytes / ms / 1e6, 1),
+                              "frac_hbm": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                              "tokens/s": round(1e3 / ms, 1)}
+
+    # prefill: 1024 rows through the dequant-GEMM, one call per tensor
+    rows = 1024
+    xs = {dim: torch.from_numpy(values).to(device) for dim, values in inputs.items()}
+    big = {name: torch.empty((rows, shape[0]), dtype=torch.float32, device=device)
+           for name, shape in shapes.items()}
+    nbytes = max(tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+        rows, shape[1], shape[0], tile_ops.GEMM_F16) for shape in shapes.values())
+    gemm_workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+    def prefill():
+        for layer in layers:
+            for name, weight in layer.items():
+                tile_ops.gemm(weight, xs[weight.input_dim], tile_ops.GEMM_F16, gemm_workspace, big[name])
+
+    ms = time_graph(prefill, stream, max(5, steps // 2), max(2, warmup // 2))
+    tflops = rows * flops_per_row / ms / 1e9
+    result["prefill_rows1024"] = {"ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
+                                  "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS["f16"], 4),
+                                  "tokens/s": round(rows / ms * 1e3, 1)}
+    return result
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -407,6 +478,7 @@ def main() -> int:
                                                               args.warmup, args.rows)
                 record["lm_head"] = lm_head_extra(device, stream, args.steps, args.warmup)
                 record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
+                record["mixed_profile"] = mixed_profile_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
             record["extras_error"] = repr(error)
     if not args.no_cpu_baseline:
