@@ -80,7 +80,7 @@ struct Stage {
 template <int T, int P>
 __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    int total_rows, int rows_per_wave, int longer_waves,
+    int total_rows, int rows_per_group, int longer_groups,
     ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -94,11 +94,11 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const float* pass_second =
         P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
 
-    // rows of this wave: dealt out evenly over all waves of the grid, each wave
-    // a contiguous range
-    const int wave_index = static_cast<int>(blockIdx.x) * kWaves + wave;
-    const int row_begin = wave_index * rows_per_wave + min(wave_index, longer_waves);
-    const int row_count = rows_per_wave + (wave_index < longer_waves ? 1 : 0);
+    // rows of this wave: dealt out evenly over the workgroups, then over the waves
+    const WaveRows mine =
+        wave_rows<kWaves>(static_cast<int>(blockIdx.x), wave, rows_per_group, longer_groups);
+    const int row_begin = mine.begin;
+    const int row_count = mine.count;
     const int total = row_count * iterations;
 
     // (1) activations of the first records this wave quantizes: loaded first so
@@ -254,11 +254,10 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     (void)raised;
     const int passes = (tokens + T - 1) / T;
     const std::int64_t groups = decode_groups(rows, kWaves);
-    const std::int64_t waves = groups * kWaves;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
                        stream, first, second, tokens, static_cast<int>(set.input_dim),
-                       static_cast<int>(rows), static_cast<int>(rows / waves),
-                       static_cast<int>(rows % waves), set);
+                       static_cast<int>(rows), static_cast<int>(rows / groups),
+                       static_cast<int>(rows % groups), set);
 }
 
 template <int P>

@@ -170,6 +170,29 @@ struct PairCursor {
     }
 };
 
+// The rows of one wave.  The launch deals its rows out evenly twice: over the
+// workgroups (the first `longer_groups` take one more than `rows_per_group`),
+// so that every compute unit streams the same number of bytes, and inside a
+// workgroup over its waves (the first few take one more; they sit on different
+// SIMDs).  Each wave gets a contiguous range.  No division: the quotients come
+// from the host and the wave count is a power of two.
+struct WaveRows {
+    int begin, count;
+};
+template <int WAVES>
+__device__ __forceinline__ WaveRows wave_rows(int group, int wave, int rows_per_group,
+                                              int longer_groups) {
+    static_assert((WAVES & (WAVES - 1)) == 0, "waves per workgroup must be a power of two");
+    const int group_begin = group * rows_per_group + min(group, longer_groups);
+    const int group_rows = rows_per_group + (group < longer_groups ? 1 : 0);
+    const int base = group_rows / WAVES;
+    const int extra = group_rows % WAVES;
+    WaveRows rows;
+    rows.begin = group_begin + wave * base + min(wave, extra);
+    rows.count = base + (wave < extra ? 1 : 0);
+    return rows;
+}
+
 // Workgroups of a wave-per-row decode launch.  Small launches are bound by
 // fixed costs: waves start at a limited rate and every workgroup quantizes the
 // whole activation vector, so one workgroup per compute unit (all resident at
