@@ -70,10 +70,12 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     }
     const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    // One row, and the verifier entry points at any row count: the vector-ALU
-    // kernels.  2..16 rows otherwise: the matrix-core kernel (Q8_0: its dot
-    // kernel).  Encodings and widths without either: the float kernel.
-    const bool one_row_arithmetic = rows == 1 || verifier;
+    // One or two rows, and the verifier entry points at any row count: the
+    // vector-ALU kernels.  3..16 rows otherwise: the matrix-core kernel (Q8_0:
+    // its dot kernel).  Encodings and widths without either: the float kernel.
+    // (two rows are also faster there: the dot kernels walk the token planes
+    // against the same unpacked weights)
+    const bool one_row_arithmetic = rows <= 2 || verifier;
     ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, exact{};
     dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
