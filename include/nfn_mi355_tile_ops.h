@@ -180,6 +180,21 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1(
     void* workspace,
     int64_t workspace_nbytes,
     void* cuda_stream);
+/* Same as the entry point above for an input whose activation records are
+ * already in `workspace`: left there by one of the three
+ * nfn_native_tile_k_quant_mmvq_multi_linear* entry points around this one,
+ * called on that input with the same `rows`, or by the dual-RMS handoff below
+ * (one row).  Skips only the
+ * activation quantization (tile_ops.h:698-709).  Refused when a projection has
+ * no kernel that reads the records. */
+int nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
 int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
     const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
     const float* input,
@@ -207,6 +222,52 @@ int nfn_native_tile_k_quant_mmvq_linear_float32_v1(
     float* output,
     void* workspace,
     int64_t workspace_nbytes,
+    void* cuda_stream);
+
+/* ---- the normalisation step upstream of the decode projections ----------
+ * hidden = residual_input + rms(input, first_weight, first_eps);
+ * residual_output = hidden; normalized_output = rms(hidden, second_weight,
+ * second_eps), with rms(x, w, eps) = x / sqrt(mean(x^2) + eps) * (w or 1, plus
+ * 1 when centered).  A weight is null or a [1, width] F32/BF16 descriptor;
+ * width <= 65536; eps finite and > 0 (tile_ops.h:836-858,
+ * tile_ops.cu:4901-4950). */
+int nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    void* cuda_stream);
+/* One-row variant that also leaves the activation records of
+ * normalized_output in the small-batch workspace, for
+ * nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1
+ * (tile_ops.h:874-894, tile_ops.cu:4952-5010).  rows must be 1, width a
+ * multiple of 256, the workspace at least
+ * nfn_native_tile_k_quant_mmq_workspace_bytes_v1(1, width) bytes. */
+int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    void* mmvq_workspace,
+    int64_t mmvq_workspace_nbytes,
     void* cuda_stream);
 
 /* ---- row argmax, ties to the lowest column (tile_ops.h:757-764) --------- */

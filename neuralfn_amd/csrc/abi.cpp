@@ -12,6 +12,7 @@
 #include "kernels.hpp"
 #include "lm_head.hpp"
 
+#include <cmath>
 #include <limits>
 
 namespace nfn {
@@ -54,7 +55,7 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
                     std::int64_t workspace_nbytes, void* stream) {
     if (descriptors == nullptr || first == nullptr || outputs == nullptr ||
         operation_count < 1 || operation_count > kMaxOperations || workspace == nullptr ||
-        workspace_nbytes <= 0 || (prologue != kPlain && second == nullptr)) {
+        workspace_nbytes <= 0 || ((prologue == kGated || prologue == kSwiGlu) && second == nullptr)) {
         return kInvalid;
     }
     const std::int64_t input_dim = descriptors[0] == nullptr ? 0 : descriptors[0]->input_dim;
@@ -92,14 +93,21 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
         }
         target->op[target->count++] = set.op[index];
     }
+    // Prequantized input: only the dot kernels read activation records.
+    if (prologue == kRecords && (matrix.count > 0 || exact.count > 0)) return kInvalid;
+    // In the verifier family the dot kernels leave their activation records in
+    // the workspace, where a following prequantized call with the same input
+    // finds them (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:3649-3666).
+    std::uint8_t* records =
+        verifier && prologue != kRecords ? static_cast<std::uint8_t*>(workspace) : nullptr;
     if (dot.count > 0) {
-        launch_gemv_dot(dot, first, second, prologue, rows, as_stream(stream));
+        launch_gemv_dot(dot, first, second, records, prologue, rows, as_stream(stream));
     }
     if (dot6.count > 0) {
-        launch_gemv_q6(dot6, first, second, prologue, rows, as_stream(stream));
+        launch_gemv_q6(dot6, first, second, records, prologue, rows, as_stream(stream));
     }
     if (dot8.count > 0) {
-        launch_gemv_q8(dot8, first, second, prologue, rows, as_stream(stream));
+        launch_gemv_q8(dot8, first, second, records, prologue, rows, as_stream(stream));
     }
     if (matrix.count > 0) {
         launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));
@@ -279,6 +287,16 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1(
                            workspace, workspace_nbytes, cuda_stream);
 }
 
+int nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1(
+    const Descriptor* const* descriptors, float* const* outputs, std::int64_t operation_count,
+    std::int64_t rows, void* workspace, std::int64_t workspace_nbytes, void* cuda_stream) {
+    // The workspace holds the activation records of `rows` rows, left there by
+    // a verifier-family call on the same input or by the dual-RMS handoff.
+    return run_small_batch(true, descriptors, static_cast<const float*>(workspace), nullptr,
+                           kRecords, outputs, operation_count, rows, workspace, workspace_nbytes,
+                           cuda_stream);
+}
+
 int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
     const Descriptor* const* descriptors, const float* input, const float* gate,
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
@@ -332,6 +350,72 @@ int nfn_native_tile_swiglu_float32(const float* gate, const float* up, float* ou
                                    std::int64_t n, void* cuda_stream) {
     if (gate == nullptr || up == nullptr || out == nullptr || n <= 0) return kInvalid;
     launch_swiglu(gate, up, out, n, as_stream(cuda_stream));
+    return launch_status();
+}
+
+// Shared argument checks of the two dual-RMS entry points
+// (neuralfn/csrc/native_train/tile_ops.cu:4901-5010): a norm weight is absent
+// or a valid [1, width] descriptor.
+static bool dual_rms_arguments_valid(const float* input, const Descriptor* first_weight,
+                                     const float* residual_input, float* hidden_output,
+                                     const Descriptor* second_weight, float* normalized_output,
+                                     float* residual_output, std::int64_t rows, std::int64_t width,
+                                     float first_eps, float second_eps, Descriptor* first,
+                                     Descriptor* second) {
+    const auto valid_weight = [&](const Descriptor* source, Descriptor* target) {
+        return source == nullptr ||
+            (normalize_descriptor(source, target) && target->output_dim == 1 &&
+             target->input_dim == width);
+    };
+    return input != nullptr && residual_input != nullptr && hidden_output != nullptr &&
+        normalized_output != nullptr && residual_output != nullptr && rows > 0 && width > 0 &&
+        width <= 65536 && std::isfinite(first_eps) && first_eps > 0.0f &&
+        std::isfinite(second_eps) && second_eps > 0.0f && valid_weight(first_weight, first) &&
+        valid_weight(second_weight, second);
+}
+
+int nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t rows, std::int64_t width, float first_eps,
+    bool first_centered, float second_eps, bool second_centered, void* cuda_stream) {
+    Descriptor first{}, second{};
+    if (!dual_rms_arguments_valid(input, first_weight, residual_input, hidden_output,
+                                  second_weight, normalized_output, residual_output, rows, width,
+                                  first_eps, second_eps, &first, &second)) {
+        return kInvalid;
+    }
+    launch_dual_rms_add_capture(input, first_weight != nullptr ? &first : nullptr, first_centered,
+                                residual_input, hidden_output,
+                                second_weight != nullptr ? &second : nullptr, second_centered,
+                                normalized_output, residual_output, rows, width, first_eps,
+                                second_eps, nullptr, as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t rows, std::int64_t width, float first_eps,
+    bool first_centered, float second_eps, bool second_centered, void* mmvq_workspace,
+    std::int64_t mmvq_workspace_nbytes, void* cuda_stream) {
+    Descriptor first{}, second{};
+    // One row only; the records are those of the small-batch workspace, so the
+    // width must be one the small-batch entry points take.
+    const std::int64_t required = rows == 1 ? small_batch_workspace_bytes(1, width) : 0;
+    if (mmvq_workspace == nullptr || rows != 1 || width % 256 != 0 || required == 0 ||
+        mmvq_workspace_nbytes < required ||
+        !dual_rms_arguments_valid(input, first_weight, residual_input, hidden_output,
+                                  second_weight, normalized_output, residual_output, rows, width,
+                                  first_eps, second_eps, &first, &second)) {
+        return kInvalid;
+    }
+    launch_dual_rms_add_capture(input, first_weight != nullptr ? &first : nullptr, first_centered,
+                                residual_input, hidden_output,
+                                second_weight != nullptr ? &second : nullptr, second_centered,
+                                normalized_output, residual_output, rows, width, first_eps,
+                                second_eps, static_cast<std::uint8_t*>(mmvq_workspace),
+                                as_stream(cuda_stream));
     return launch_status();
 }
 

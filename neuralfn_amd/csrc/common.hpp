@@ -94,7 +94,10 @@ struct ProjectionSet {
 };
 
 // Activation prologues of the fused entry points (glimmer_k_mmq.cu:299-317).
-enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2 };
+// kRecords is not a prologue of the floats: the input pointer holds activation
+// records that an earlier launch quantized (the prequantized entry point,
+// neuralfn/csrc/native_train/tile_ops.h:698-709).
+enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2, kRecords = 3 };
 
 #if defined(__HIPCC__)
 

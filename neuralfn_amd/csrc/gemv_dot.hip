@@ -61,10 +61,9 @@ __device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, 
     return image;
 }
 
-// Quantize the 256 activations of block `block`, four per lane.
-__device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
-                                               const TokenImage& image) {
-    const ActivationCodes codes = encode_activations(x);
+// Scatter the codes of block `block`, four values per lane, into the image.
+__device__ __forceinline__ void quantize_block(const ActivationCodes& codes, int lane, int block,
+                                               int blocks, const TokenImage& image) {
     const std::uint32_t hi = codes.hi, lo = codes.lo;
     const float maximum = codes.maximum;
     int sum = codes.sum;
@@ -93,7 +92,7 @@ struct Stage {
 template <std::uint32_t ENC, int T, int P>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    int total_rows, int rows_per_group, int longer_groups,
+    int total_rows, int rows_per_group, int longer_groups, std::uint8_t* __restrict__ records_out,
     ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
@@ -107,9 +106,9 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
-    const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
+    const float* pass_first = pass_input<P>(first, token0, input_dim);
+    const float* pass_second = P == kGated || P == kSwiGlu
+        ? second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
 
     // rows of this wave: dealt out evenly over the workgroups, then over the waves
     const WaveRows mine =
@@ -154,15 +153,24 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     issue(stage0);
     issue(stage1);
 
-    // (3) quantize; one barrier; after it the workgroup never synchronises again
+    // (3) quantize; one barrier; after it the workgroup never synchronises again.
+    // The first workgroup also leaves the records in the caller's workspace
+    // for a later launch that shares this input.
+    const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
+    auto quantize_record = [&](float4 loaded, int record) {
+        const int token = token_of_record<T>(record, blocks);
+        const int block = record - token * blocks;
+        const ActivationCodes codes = activation_codes<P>(loaded);
+        quantize_block(codes, lane, block, blocks, token_image(lds, token, blocks));
+        if (keep_records) {
+            store_record(records_out + (static_cast<std::int64_t>(token0 + token) * blocks + block) *
+                             kActRecord, lane, codes);
+        }
+    };
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kDotWaves;
-        if (record < records) {
-            const int token = token_of_record<T>(record, blocks);
-            quantize_block(early[e], lane, record - token * blocks, blocks,
-                           token_image(lds, token, blocks));
-        }
+        if (record < records) quantize_record(early[e], record);
     }
     for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
         const int token = token_of_record<T>(record, blocks);
@@ -170,7 +178,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         const float4 x = load_activations<P>(
             pass_first, pass_second,
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
-        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+        quantize_record(x, record);
     }
     __syncthreads();
 
@@ -286,7 +294,8 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 }
 
 template <std::uint32_t ENC, int T, int P>
-void launch_variant(ProjectionSet set, const float* first, const float* second, int tokens,
+void launch_variant(ProjectionSet set, const float* first, const float* second,
+        std::uint8_t* records_out, int tokens,
                     hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
@@ -305,11 +314,12 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
                        stream, first, second, tokens, static_cast<int>(set.input_dim),
                        static_cast<int>(rows), static_cast<int>(rows / groups),
-                       static_cast<int>(rows % groups), set);
+                       static_cast<int>(rows % groups), records_out, set);
 }
 
 template <std::uint32_t ENC, int P>
-void launch_tokens(const ProjectionSet& set, const float* first, const float* second, int tokens,
+void launch_tokens(const ProjectionSet& set, const float* first, const float* second,
+        std::uint8_t* records_out, int tokens,
                    hipStream_t stream) {
     // token planes of one pass must fit in LDS: four tokens up to K = 16384
     const std::int64_t image = token_image_bytes_host(set.input_dim >> 8);
@@ -317,23 +327,24 @@ void launch_tokens(const ProjectionSet& set, const float* first, const float* se
     if (capacity > 4) capacity = 4;
     const int per_pass = tokens < capacity ? tokens : capacity;
     if (per_pass <= 1) {
-        launch_variant<ENC, 1, P>(set, first, second, tokens, stream);
+        launch_variant<ENC, 1, P>(set, first, second, records_out, tokens, stream);
     } else if (per_pass == 2) {
-        launch_variant<ENC, 2, P>(set, first, second, tokens, stream);
+        launch_variant<ENC, 2, P>(set, first, second, records_out, tokens, stream);
     } else if (capacity >= 4) {
-        launch_variant<ENC, 4, P>(set, first, second, tokens, stream);
+        launch_variant<ENC, 4, P>(set, first, second, records_out, tokens, stream);
     } else {
-        launch_variant<ENC, 2, P>(set, first, second, tokens, stream);
+        launch_variant<ENC, 2, P>(set, first, second, records_out, tokens, stream);
     }
 }
 
 template <std::uint32_t ENC>
 void launch_prologue(const ProjectionSet& set, const float* first, const float* second,
-                     int prologue, int tokens, hipStream_t stream) {
+        std::uint8_t* records_out, int prologue, int tokens, hipStream_t stream) {
     switch (prologue) {
-        case kGated: launch_tokens<ENC, kGated>(set, first, second, tokens, stream); break;
-        case kSwiGlu: launch_tokens<ENC, kSwiGlu>(set, first, second, tokens, stream); break;
-        default: launch_tokens<ENC, kPlain>(set, first, second, tokens, stream); break;
+        case kGated: launch_tokens<ENC, kGated>(set, first, second, records_out, tokens, stream); break;
+        case kSwiGlu: launch_tokens<ENC, kSwiGlu>(set, first, second, records_out, tokens, stream); break;
+        case kRecords: launch_tokens<ENC, kRecords>(set, first, second, nullptr, tokens, stream); break;
+        default: launch_tokens<ENC, kPlain>(set, first, second, records_out, tokens, stream); break;
     }
 }
 
@@ -345,7 +356,7 @@ bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* second,
-                     int prologue, std::int64_t rows, hipStream_t stream) {
+        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
     const std::uint32_t encodings[2] = {kEncQ4K, kEncQ5K};
     for (const std::uint32_t encoding : encodings) {
         ProjectionSet group{};
@@ -355,9 +366,9 @@ void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* 
         }
         if (group.count == 0) continue;
         if (encoding == kEncQ4K) {
-            launch_prologue<kEncQ4K>(group, first, second, prologue, static_cast<int>(rows), stream);
+            launch_prologue<kEncQ4K>(group, first, second, records_out, prologue, static_cast<int>(rows), stream);
         } else {
-            launch_prologue<kEncQ5K>(group, first, second, prologue, static_cast<int>(rows), stream);
+            launch_prologue<kEncQ5K>(group, first, second, records_out, prologue, static_cast<int>(rows), stream);
         }
     }
 }

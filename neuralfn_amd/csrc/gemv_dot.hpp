@@ -8,8 +8,12 @@ namespace nfn {
 
 bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim);
 
-// rows 1..16; activations are quantized inside the launch, no workspace.
+// rows 1..16; activations are quantized inside the launch.  `records_out`
+// (may be null): where the launch also leaves its activation records
+// (kActRecord bytes per token and 256 values) for a later launch with
+// prologue kRecords, whose `first` is then that pointer.
 void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* second,
-                     int prologue, std::int64_t rows, hipStream_t stream);
+                     std::uint8_t* records_out, int prologue, std::int64_t rows,
+                     hipStream_t stream);
 
 }  // namespace nfn

@@ -42,11 +42,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 constexpr int kTileRows = 32;
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
-constexpr int kActRecord = kActivationRecordBytes;
-// record layout: [0,256) high plane, [256,512) low plane, [512,544) eight int32
-// sums of the codes per 32 values, [544,548) float scale, rest padding
-constexpr int kRecordSums = 512;
-constexpr int kRecordScale = 544;
+static_assert(kActRecord == kActivationRecordBytes, "record size is part of the workspace contract");
 
 struct __attribute__((packed, aligned(2))) Chunk16 {
     std::uint32_t v[4];
@@ -82,20 +78,7 @@ struct Format<kEncQ6K> {
 // Quantize the 256 activations of one block, four per lane, and write the
 // record (planes, per-32 code sums, scale) to `record` (LDS or workspace).
 __device__ __forceinline__ void quantize_block(float4 x, int lane, std::uint8_t* record) {
-    const ActivationCodes codes = encode_activations(x);
-    // sum of the codes over the 8 lanes of a 32-value group
-    int sum = codes.sum;
-    sum += dpp_move<kQuadXor1>(sum);
-    sum += dpp_move<kQuadXor2>(sum);
-    sum += dpp_move<kHalfMirror>(sum);
-    *reinterpret_cast<std::uint32_t*>(record + lane * 4) = codes.hi;
-    *reinterpret_cast<std::uint32_t*>(record + 256 + lane * 4) = codes.lo;
-    if ((lane & 7) == 0) {
-        *reinterpret_cast<int*>(record + kRecordSums + (lane >> 3) * 4) = sum;
-    }
-    if (lane == 0) {
-        *reinterpret_cast<float*>(record + kRecordScale) = codes.maximum * (1.0f / kCodeRange);
-    }
+    store_record(record, lane, encode_activations(x));
 }
 
 // Token <-> operand-row bookkeeping of v_mfma_i32_32x32x32_i8.  Output register

@@ -81,9 +81,8 @@ __device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, 
 
 // Quantize the 256 activations of block `block`, four per lane: lane L holds
 // positions 4L..4L+3 = half L/32, quarter (L/8)%4, sixteen (L/4)%2, bytes 4*(L%4)..
-__device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
-                                               const TokenImage& image) {
-    const ActivationCodes codes = encode_activations(x);
+__device__ __forceinline__ void quantize_block(const ActivationCodes& codes, int lane, int block,
+                                               int blocks, const TokenImage& image) {
     int sum = codes.sum;
     sum += dpp_move<kQuadXor1>(sum);
     sum += dpp_move<kQuadXor2>(sum);
@@ -173,7 +172,8 @@ template <int T, int P, bool ARGMAX>
 __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
     int total_rows, int rows_per_group, int longer_groups,
-    LmHeadCandidate* __restrict__ candidates, ProjectionSet set) {
+    LmHeadCandidate* __restrict__ candidates, std::uint8_t* __restrict__ records_out,
+    ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -182,9 +182,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
-    const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
+    const float* pass_first = pass_input<P>(first, token0, static_cast<int>(input_dim));
+    const float* pass_second = P == kGated || P == kSwiGlu
+        ? second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
 
     // rows of this wave: dealt out evenly over the workgroups, then over the waves
     const WaveRows mine =
@@ -231,14 +231,23 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
     issue(stage1);
 
     // (3) quantize; one barrier
+    // (the first workgroup also leaves the records in the caller's workspace
+    // for a later launch that shares this input)
+    const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
+    auto quantize_record = [&](float4 loaded, int record) {
+        const int token = token_of_record<T>(record, blocks);
+        const int block = record - token * blocks;
+        const ActivationCodes codes = activation_codes<P>(loaded);
+        quantize_block(codes, lane, block, blocks, token_image(lds, token, blocks));
+        if (keep_records) {
+            store_record(records_out + (static_cast<std::int64_t>(token0 + token) * blocks + block) *
+                             kActRecord, lane, codes);
+        }
+    };
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kWaves;
-        if (record < records) {
-            const int token = token_of_record<T>(record, blocks);
-            quantize_block(early[e], lane, record - token * blocks, blocks,
-                           token_image(lds, token, blocks));
-        }
+        if (record < records) quantize_record(early[e], record);
     }
     for (int record = wave + kEarly * kWaves; record < records; record += kWaves) {
         const int token = token_of_record<T>(record, blocks);
@@ -246,7 +255,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
         const float4 x = load_activations<P>(
             pass_first, pass_second,
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
-        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+        quantize_record(x, record);
     }
     __syncthreads();
 
@@ -373,16 +382,17 @@ struct PassLoads {
 template <int T, int P, bool ARGMAX, int W>
 __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
     const float* __restrict__ first, const float* __restrict__ second, std::int64_t input_dim,
-    int tokens, int rows_per_wave, LmHeadCandidate* __restrict__ candidates, ProjectionSet set) {
+    int tokens, int rows_per_wave, LmHeadCandidate* __restrict__ candidates,
+    std::uint8_t* __restrict__ records_out, ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int blocks = static_cast<int>(input_dim >> 8);  // per row, >= 16
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
-    const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
+    const float* pass_first = pass_input<P>(first, token0, static_cast<int>(input_dim));
+    const float* pass_second = P == kGated || P == kSwiGlu
+        ? second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
     std::uint8_t* staging = lds + T * token_image_bytes(blocks) + wave * kStagingBytes;
 
     // rows and blocks of this wave: every projection owns a range of waves
@@ -447,14 +457,23 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
     issue(loads1, min(1, max(passes - 1, 0)));
 
     // (3) quantize; one barrier
+    // (the first workgroup also leaves the records in the caller's workspace
+    // for a later launch that shares this input)
+    const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
+    auto quantize_record = [&](float4 loaded, int record) {
+        const int token = token_of_record<T>(record, blocks);
+        const int block = record - token * blocks;
+        const ActivationCodes codes = activation_codes<P>(loaded);
+        quantize_block(codes, lane, block, blocks, token_image(lds, token, blocks));
+        if (keep_records) {
+            store_record(records_out + (static_cast<std::int64_t>(token0 + token) * blocks + block) *
+                             kActRecord, lane, codes);
+        }
+    };
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * W;
-        if (record < records) {
-            const int token = token_of_record<T>(record, blocks);
-            quantize_block(early[e], lane, record - token * blocks, blocks,
-                           token_image(lds, token, blocks));
-        }
+        if (record < records) quantize_record(early[e], record);
     }
     for (int record = wave + kEarly * W; record < records; record += W) {
         const int token = token_of_record<T>(record, blocks);
@@ -462,7 +481,7 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
         const float4 x = load_activations<P>(
             pass_first, pass_second,
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
-        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+        quantize_record(x, record);
     }
     __syncthreads();
 
@@ -606,7 +625,7 @@ Geometry geometry(std::int64_t rows) {
 // launch: with the argmax fused in, that is the number of candidates per token.
 template <int T, int P, bool ARGMAX>
 std::int64_t launch_variant(ProjectionSet set, const float* first, const float* second,
-                            int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
@@ -624,7 +643,7 @@ std::int64_t launch_variant(ProjectionSet set, const float* first, const float* 
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
                        stream, first, second, tokens, static_cast<int>(set.input_dim),
                        static_cast<int>(rows), static_cast<int>(rows / groups),
-                       static_cast<int>(rows % groups), candidates, set);
+                       static_cast<int>(rows % groups), candidates, records_out, set);
     return groups;
 }
 
@@ -651,7 +670,7 @@ constexpr int stream_waves(int tokens_per_pass) {
 
 template <int T, int P, bool ARGMAX>
 std::int64_t launch_stream(const ProjectionSet& set, const float* first, const float* second,
-                           int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
     constexpr int W = stream_waves(T);
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8) +
         W * kStagingBytes;
@@ -674,7 +693,7 @@ std::int64_t launch_stream(const ProjectionSet& set, const float* first, const f
     const std::int64_t groups = (waves + W - 1) / W;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(W * kWave), lds,
                        stream, first, second, set.input_dim, tokens, static_cast<int>(rows_per_wave),
-                       candidates, placed);
+                       candidates, records_out, placed);
     return groups;
 }
 
@@ -682,7 +701,7 @@ bool streams(std::int64_t input_dim) { return (input_dim >> 8) >= kPassBlocks; }
 
 template <int P, bool ARGMAX>
 std::int64_t launch_tokens(const ProjectionSet& set, const float* first, const float* second,
-                           int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
     // the token images of one pass (and the staging areas) must fit in LDS
     const std::int64_t image = token_image_bytes(set.input_dim >> 8);
     int capacity = static_cast<int>((150 * 1024 - 16 * kStagingBytes) / image);
@@ -690,20 +709,20 @@ std::int64_t launch_tokens(const ProjectionSet& set, const float* first, const f
     const int per_pass = tokens < capacity ? tokens : capacity;
     if (streams(set.input_dim)) {
         if (per_pass <= 1) {
-            return launch_stream<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+            return launch_stream<1, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
         }
         if (per_pass == 2 || capacity < 4) {
-            return launch_stream<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+            return launch_stream<2, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
         }
-        return launch_stream<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+        return launch_stream<4, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
     }
     if (per_pass <= 1) {
-        return launch_variant<1, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+        return launch_variant<1, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
     }
     if (per_pass == 2 || capacity < 4) {
-        return launch_variant<2, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+        return launch_variant<2, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
     }
-    return launch_variant<4, P, ARGMAX>(set, first, second, tokens, candidates, stream);
+    return launch_variant<4, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
 }
 
 }  // namespace
@@ -714,7 +733,7 @@ bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
-                    int prologue, std::int64_t rows, hipStream_t stream) {
+        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
     ProjectionSet group{};
     group.input_dim = set.input_dim;
     for (int index = 0; index < set.count; ++index) {
@@ -724,13 +743,16 @@ void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* s
     const int tokens = static_cast<int>(rows);
     switch (prologue) {
         case kGated:
-            launch_tokens<kGated, false>(group, first, second, tokens, nullptr, stream);
+            launch_tokens<kGated, false>(group, first, second, records_out, tokens, nullptr, stream);
             break;
         case kSwiGlu:
-            launch_tokens<kSwiGlu, false>(group, first, second, tokens, nullptr, stream);
+            launch_tokens<kSwiGlu, false>(group, first, second, records_out, tokens, nullptr, stream);
+            break;
+        case kRecords:
+            launch_tokens<kRecords, false>(group, first, second, nullptr, tokens, nullptr, stream);
             break;
         default:
-            launch_tokens<kPlain, false>(group, first, second, tokens, nullptr, stream);
+            launch_tokens<kPlain, false>(group, first, second, records_out, tokens, nullptr, stream);
             break;
     }
 }
@@ -754,7 +776,8 @@ void launch_lm_head_q6(const Descriptor& descriptor, const float* input, std::in
     set.op[0].row_stride = descriptor.row_stride_bytes;
     set.op[0].encoding = descriptor.encoding;
     const std::int64_t groups =
-        launch_tokens<kPlain, true>(set, input, nullptr, static_cast<int>(rows), candidates, stream);
+        launch_tokens<kPlain, true>(set, input, nullptr, nullptr, static_cast<int>(rows), candidates,
+                                    stream);
     launch_lm_head_final(candidates, groups, indices, maxima, rows, stream);
 }
 

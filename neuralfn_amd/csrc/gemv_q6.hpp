@@ -9,9 +9,10 @@ namespace nfn {
 bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim);
 
 // The Q6_K projections of `set`, rows 1..16; activations are quantized inside
-// the launch, no workspace.
+// the launch.  `records_out` and prologue kRecords as for launch_gemv_dot.
 void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
-                    int prologue, std::int64_t rows, hipStream_t stream);
+                    std::uint8_t* records_out, int prologue, std::int64_t rows,
+                    hipStream_t stream);
 
 // Upper bound of the workgroups of a fused lm_head launch (= candidates per
 // input row) over all input widths and token counts, for sizing the workspace.

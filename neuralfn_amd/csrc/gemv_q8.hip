@@ -60,9 +60,8 @@ __device__ __forceinline__ TokenImage token_image(std::uint8_t* lds, int token, 
 
 // Quantize the 256 activations of block `block`, four per lane: lane L holds
 // values 4L..4L+3 = unit L/16 of the block, sixteen (L/4)%4, bytes 4*(L%4)..
-__device__ __forceinline__ void quantize_block(float4 x, int lane, int block, int blocks,
-                                               const TokenImage& image) {
-    const ActivationCodes codes = encode_activations(x);
+__device__ __forceinline__ void quantize_block(const ActivationCodes& codes, int lane, int block,
+                                               int blocks, const TokenImage& image) {
     const int units = 4 * blocks;
     const int unit = 4 * block + (lane >> 4);
     const int sixteen = (lane >> 2) & 3;
@@ -80,7 +79,7 @@ struct Stage {
 template <int T, int P>
 __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    int total_rows, int rows_per_group, int longer_groups,
+    int total_rows, int rows_per_group, int longer_groups, std::uint8_t* __restrict__ records_out,
     ProjectionSet set) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -90,9 +89,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     const int iterations = (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = min(tokens - token0, T);
-    const float* pass_first = first + static_cast<std::int64_t>(token0) * input_dim;
-    const float* pass_second =
-        P == kPlain ? nullptr : second + static_cast<std::int64_t>(token0) * input_dim;
+    const float* pass_first = pass_input<P>(first, token0, static_cast<int>(input_dim));
+    const float* pass_second = P == kGated || P == kSwiGlu
+        ? second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
 
     // rows of this wave: dealt out evenly over the workgroups, then over the waves
     const WaveRows mine =
@@ -136,14 +135,23 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     issue(stage1);
 
     // (3) quantize; one barrier
+    // (the first workgroup also leaves the records in the caller's workspace
+    // for a later launch that shares this input)
+    const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
+    auto quantize_record = [&](float4 loaded, int record) {
+        const int token = token_of_record<T>(record, blocks);
+        const int block = record - token * blocks;
+        const ActivationCodes codes = activation_codes<P>(loaded);
+        quantize_block(codes, lane, block, blocks, token_image(lds, token, blocks));
+        if (keep_records) {
+            store_record(records_out + (static_cast<std::int64_t>(token0 + token) * blocks + block) *
+                             kActRecord, lane, codes);
+        }
+    };
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
         const int record = wave + e * kWaves;
-        if (record < records) {
-            const int token = token_of_record<T>(record, blocks);
-            quantize_block(early[e], lane, record - token * blocks, blocks,
-                           token_image(lds, token, blocks));
-        }
+        if (record < records) quantize_record(early[e], record);
     }
     for (int record = wave + kEarly * kWaves; record < records; record += kWaves) {
         const int token = token_of_record<T>(record, blocks);
@@ -151,7 +159,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
         const float4 x = load_activations<P>(
             pass_first, pass_second,
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
-        quantize_block(x, lane, block, blocks, token_image(lds, token, blocks));
+        quantize_record(x, record);
     }
     __syncthreads();
 
@@ -239,7 +247,8 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
 }
 
 template <int T, int P>
-void launch_variant(ProjectionSet set, const float* first, const float* second, int tokens,
+void launch_variant(ProjectionSet set, const float* first, const float* second,
+        std::uint8_t* records_out, int tokens,
                     hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
@@ -257,11 +266,12 @@ void launch_variant(ProjectionSet set, const float* first, const float* second, 
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
                        stream, first, second, tokens, static_cast<int>(set.input_dim),
                        static_cast<int>(rows), static_cast<int>(rows / groups),
-                       static_cast<int>(rows % groups), set);
+                       static_cast<int>(rows % groups), records_out, set);
 }
 
 template <int P>
-void launch_tokens(const ProjectionSet& set, const float* first, const float* second, int tokens,
+void launch_tokens(const ProjectionSet& set, const float* first, const float* second,
+        std::uint8_t* records_out, int tokens,
                    hipStream_t stream) {
     // the token images of one pass must fit in LDS
     const std::int64_t image = token_image_bytes(set.input_dim >> 8);
@@ -269,11 +279,11 @@ void launch_tokens(const ProjectionSet& set, const float* first, const float* se
     if (capacity > 4) capacity = 4;
     const int per_pass = tokens < capacity ? tokens : capacity;
     if (per_pass <= 1) {
-        launch_variant<1, P>(set, first, second, tokens, stream);
+        launch_variant<1, P>(set, first, second, records_out, tokens, stream);
     } else if (per_pass == 2 || capacity < 4) {
-        launch_variant<2, P>(set, first, second, tokens, stream);
+        launch_variant<2, P>(set, first, second, records_out, tokens, stream);
     } else {
-        launch_variant<4, P>(set, first, second, tokens, stream);
+        launch_variant<4, P>(set, first, second, records_out, tokens, stream);
     }
 }
 
@@ -285,7 +295,7 @@ bool gemv_q8_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_q8(const ProjectionSet& set, const float* first, const float* second,
-                    int prologue, std::int64_t rows, hipStream_t stream) {
+        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
     ProjectionSet group{};
     group.input_dim = set.input_dim;
     for (int index = 0; index < set.count; ++index) {
@@ -294,9 +304,10 @@ void launch_gemv_q8(const ProjectionSet& set, const float* first, const float* s
     if (group.count == 0) return;
     const int tokens = static_cast<int>(rows);
     switch (prologue) {
-        case kGated: launch_tokens<kGated>(group, first, second, tokens, stream); break;
-        case kSwiGlu: launch_tokens<kSwiGlu>(group, first, second, tokens, stream); break;
-        default: launch_tokens<kPlain>(group, first, second, tokens, stream); break;
+        case kGated: launch_tokens<kGated>(group, first, second, records_out, tokens, stream); break;
+        case kSwiGlu: launch_tokens<kSwiGlu>(group, first, second, records_out, tokens, stream); break;
+        case kRecords: launch_tokens<kRecords>(group, first, second, nullptr, tokens, stream); break;
+        default: launch_tokens<kPlain>(group, first, second, records_out, tokens, stream); break;
     }
 }
 

@@ -29,4 +29,15 @@ void launch_sigmoid_gate(const float* values, const float* gate, float* output,
 void launch_swiglu(const float* gate, const float* up, float* output, std::int64_t count,
                    hipStream_t stream);
 
+// rms.hip — two adjacent RMS normalisations of the decode loop in one launch;
+// `records` (may be null, else one row only): the small-batch workspace that
+// receives the activation records of normalized_output.
+void launch_dual_rms_add_capture(const float* input, const Descriptor* first_weight,
+                                 bool first_centered, const float* residual_input,
+                                 float* hidden_output, const Descriptor* second_weight,
+                                 bool second_centered, float* normalized_output,
+                                 float* residual_output, std::int64_t rows, std::int64_t width,
+                                 float first_eps, float second_eps, std::uint8_t* records,
+                                 hipStream_t stream);
+
 }  // namespace nfn

@@ -1,0 +1,178 @@
+// Two adjacent RMS normalisations of the decode loop in one launch:
+//
+//   hidden            = residual_input + rms(input, first_weight, first_eps)
+//   residual_output   = hidden
+//   normalized_output = rms(hidden, second_weight, second_eps)
+//
+// and, for the one-row handoff, the activation records of normalized_output in
+// the caller's small-batch workspace, so that the projection that follows can
+// skip its own quantization.
+//
+// One workgroup of 256 threads per row.  The float arithmetic follows the
+// reference kernel operation for operation
+// (neuralfn/csrc/tile_cuda/kernels.cu:2155-2243): thread t accumulates the
+// squares of columns t, t+256, ... with fused multiply-adds, the 256 partial
+// sums are added in a halving tree, normalized = (x * inverse_rms) * scale with
+// two roundings, hidden = normalized + residual with one.  The only departure:
+// inverse_rms is 1 / sqrt(mean + eps) with correctly rounded division and
+// square root where the reference calls the device's approximate reciprocal
+// square root, so the two can differ in the last bits of that one factor.
+#include "common.hpp"
+#include "kernels.hpp"
+#include "wave_rows.hpp"
+
+namespace nfn {
+
+namespace {
+
+constexpr int kRmsThreads = 256;
+constexpr int kBatch = 8;  // columns per thread whose loads are issued together
+
+// Affine weight of one normalisation: a [1, width] packed row, or none.
+struct NormWeight {
+    const std::uint8_t* data;
+    std::uint32_t encoding;
+    int present;
+    int centered;  // the stored weight is (scale - 1)
+};
+
+__device__ __forceinline__ float norm_scale(const NormWeight& weight, std::int64_t column) {
+    if (!weight.present) return 1.0f;
+    float scale = weight_value(weight.encoding, weight.data, column);
+    if (weight.centered) scale += 1.0f;
+    return scale;
+}
+
+// 1 / sqrt(mean of squares + eps) of `values[0, width)`, the same number in every thread.
+__device__ __forceinline__ float inverse_rms(const float* values, std::int64_t width, float eps,
+                                             float* partials) {
+    // Same order as a plain strided loop; the loads of a batch go out together
+    // (a column past the end contributes fma(0, 0, sum) = sum).
+    float square_sum = 0.0f;
+    for (std::int64_t base = threadIdx.x; base < width; base += kBatch * kRmsThreads) {
+        float value[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const std::int64_t column = base + i * kRmsThreads;
+            value[i] = column < width ? values[column] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) square_sum = fmaf(value[i], value[i], square_sum);
+    }
+    partials[threadIdx.x] = square_sum;
+    __syncthreads();
+    for (int stride = kRmsThreads / 2; stride > 0; stride /= 2) {
+        if (threadIdx.x < static_cast<unsigned>(stride)) {
+            partials[threadIdx.x] += partials[threadIdx.x + stride];
+        }
+        __syncthreads();
+    }
+    const float result = 1.0f / sqrtf(partials[0] / static_cast<float>(width) + eps);
+    __syncthreads();  // partials are reused by the next reduction
+    return result;
+}
+
+template <bool HANDOFF>
+__global__ __launch_bounds__(kRmsThreads) void dual_rms_add_capture_kernel(
+    const float* __restrict__ input, NormWeight first_weight,
+    const float* __restrict__ residual_input, float* hidden_output, NormWeight second_weight,
+    float* normalized_output, float* __restrict__ residual_output, std::int64_t width,
+    float first_eps, float second_eps, std::uint8_t* __restrict__ records) {
+    __shared__ float partials[kRmsThreads];
+    const std::int64_t row = blockIdx.x;
+    const float* source = input + row * width;
+    const float* residual = residual_input + row * width;
+    float* hidden = hidden_output + row * width;
+    float* captured = residual_output + row * width;
+    float* normalized = normalized_output + row * width;
+
+    const float first_inverse = inverse_rms(source, width, first_eps, partials);
+    for (std::int64_t base = threadIdx.x; base < width; base += kBatch * kRmsThreads) {
+        float value[kBatch], other[kBatch], scale[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const std::int64_t column = min(base + i * kRmsThreads, width - 1);
+            value[i] = source[column];
+            other[i] = residual[column];
+            scale[i] = norm_scale(first_weight, column);
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const std::int64_t column = base + i * kRmsThreads;
+            const float sum =
+                __fadd_rn(__fmul_rn(__fmul_rn(value[i], first_inverse), scale[i]), other[i]);
+            if (column < width) {
+                hidden[column] = sum;
+                captured[column] = sum;
+            }
+        }
+    }
+    __syncthreads();  // every thread reads hidden values other threads wrote
+
+    const float second_inverse = inverse_rms(hidden, width, second_eps, partials);
+    for (std::int64_t base = threadIdx.x; base < width; base += kBatch * kRmsThreads) {
+        float value[kBatch], scale[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const std::int64_t column = min(base + i * kRmsThreads, width - 1);
+            value[i] = hidden[column];
+            scale[i] = norm_scale(second_weight, column);
+        }
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) {
+            const std::int64_t column = base + i * kRmsThreads;
+            if (column < width) {
+                normalized[column] = __fmul_rn(__fmul_rn(value[i], second_inverse), scale[i]);
+            }
+        }
+    }
+
+    if constexpr (HANDOFF) {
+        __syncthreads();
+        // one wave per 256-value block: the quantizer of the decode kernels
+        const int lane = threadIdx.x & 63;
+        const int wave = threadIdx.x >> 6;
+        const int blocks = static_cast<int>(width >> 8);
+        for (int block = wave; block < blocks; block += kRmsThreads / kWave) {
+            const float4 x = *reinterpret_cast<const float4*>(normalized + block * 256 + lane * 4);
+            store_record(records + static_cast<std::int64_t>(block) * kActRecord, lane,
+                         encode_activations(x));
+        }
+    }
+}
+
+NormWeight norm_weight(const Descriptor* descriptor, bool centered) {
+    NormWeight weight{};
+    if (descriptor != nullptr) {
+        weight.data = descriptor->data;
+        weight.encoding = descriptor->encoding;
+        weight.present = 1;
+        weight.centered = centered ? 1 : 0;
+    }
+    return weight;
+}
+
+}  // namespace
+
+void launch_dual_rms_add_capture(const float* input, const Descriptor* first_weight,
+                                 bool first_centered, const float* residual_input,
+                                 float* hidden_output, const Descriptor* second_weight,
+                                 bool second_centered, float* normalized_output,
+                                 float* residual_output, std::int64_t rows, std::int64_t width,
+                                 float first_eps, float second_eps, std::uint8_t* records,
+                                 hipStream_t stream) {
+    const NormWeight first = norm_weight(first_weight, first_centered);
+    const NormWeight second = norm_weight(second_weight, second_centered);
+    const dim3 grid(static_cast<unsigned>(rows));
+    if (records != nullptr) {
+        hipLaunchKernelGGL((dual_rms_add_capture_kernel<true>), grid, dim3(kRmsThreads), 0, stream,
+                           input, first, residual_input, hidden_output, second, normalized_output,
+                           residual_output, width, first_eps, second_eps, records);
+    } else {
+        hipLaunchKernelGGL((dual_rms_add_capture_kernel<false>), grid, dim3(kRmsThreads), 0, stream,
+                           input, first, residual_input, hidden_output, second, normalized_output,
+                           residual_output, width, first_eps, second_eps, records);
+    }
+}
+
+}  // namespace nfn

@@ -92,12 +92,35 @@ __device__ __forceinline__ ActivationCodes encode_activations(float4 x) {
     return codes;
 }
 
+// Activation record of one (token, 256-value block) in a caller's workspace:
+// what a later launch needs to skip the quantization.  [0,256) high plane,
+// [256,512) low plane (value order), [512,544) eight int32 sums of the codes
+// per 32 values, [544] the scale, [548] the block's largest magnitude.
+constexpr int kActRecord = 576;
+constexpr int kRecordSums = 512;
+constexpr int kRecordScale = 544;
+constexpr int kRecordMaximum = 548;
+
+// The four values of lane `column % 256 / 4` of block `column / 256` as the
+// kernels' quantizers take them: floats with the prologue applied, or for
+// kRecords the raw (high word, low word, maximum) of the stored record.
 template <int P>
 __device__ __forceinline__ float4 load_activations(const float* __restrict__ first,
                                                    const float* __restrict__ second,
                                                    std::int64_t column) {
+    if constexpr (P == kRecords) {
+        const std::uint8_t* record =
+            reinterpret_cast<const std::uint8_t*>(first) + (column >> 8) * kActRecord;
+        const int offset = static_cast<int>(column & 255);  // 4 * lane
+        float4 raw;
+        raw.x = *reinterpret_cast<const float*>(record + offset);
+        raw.y = *reinterpret_cast<const float*>(record + 256 + offset);
+        raw.z = *reinterpret_cast<const float*>(record + kRecordMaximum);
+        raw.w = 0.0f;
+        return raw;
+    }
     float4 x = *reinterpret_cast<const float4*>(first + column);
-    if constexpr (P != kPlain) {
+    if constexpr (P == kGated || P == kSwiGlu) {
         const float4 y = *reinterpret_cast<const float4*>(second + column);
         x.x = apply_prologue<P>(x.x, y.x);
         x.y = apply_prologue<P>(x.y, y.y);
@@ -105,6 +128,49 @@ __device__ __forceinline__ float4 load_activations(const float* __restrict__ fir
         x.w = apply_prologue<P>(x.w, y.w);
     }
     return x;
+}
+
+// First input of the pass that starts at token `token0`.
+template <int P>
+__device__ __forceinline__ const float* pass_input(const float* first, int token0, int input_dim) {
+    if constexpr (P == kRecords) {
+        return reinterpret_cast<const float*>(reinterpret_cast<const std::uint8_t*>(first) +
+                                              static_cast<std::int64_t>(token0) * (input_dim >> 8) * kActRecord);
+    } else {
+        return first + static_cast<std::int64_t>(token0) * input_dim;
+    }
+}
+
+// Codes of what load_activations<P> returned.
+template <int P>
+__device__ __forceinline__ ActivationCodes activation_codes(float4 loaded) {
+    if constexpr (P == kRecords) {
+        ActivationCodes codes;
+        codes.hi = __float_as_uint(loaded.x);
+        codes.lo = __float_as_uint(loaded.y);
+        codes.maximum = loaded.z;
+        codes.sum = (__builtin_amdgcn_sdot4(static_cast<int>(codes.hi), 0x01010101, 0, false) << 8) +
+            __builtin_amdgcn_sdot4(static_cast<int>(codes.lo), 0x01010101, 0, false);
+        return codes;
+    } else {
+        return encode_activations(loaded);
+    }
+}
+
+// Writes the record of one block (four values per lane) for a later launch.
+__device__ __forceinline__ void store_record(std::uint8_t* record, int lane,
+                                             const ActivationCodes& codes) {
+    int sum = codes.sum;  // over the 8 lanes of a 32-value group
+    sum += dpp_move<kQuadXor1>(sum);
+    sum += dpp_move<kQuadXor2>(sum);
+    sum += dpp_move<kHalfMirror>(sum);
+    *reinterpret_cast<std::uint32_t*>(record + lane * 4) = codes.hi;
+    *reinterpret_cast<std::uint32_t*>(record + 256 + lane * 4) = codes.lo;
+    if ((lane & 7) == 0) *reinterpret_cast<int*>(record + kRecordSums + (lane >> 3) * 4) = sum;
+    if (lane == 0) {
+        *reinterpret_cast<float*>(record + kRecordScale) = codes.maximum * (1.0f / kCodeRange);
+        *reinterpret_cast<float*>(record + kRecordMaximum) = codes.maximum;
+    }
 }
 
 // Token of activation record `record` (records run token by token, `blocks`

@@ -75,12 +75,20 @@ SIGNATURES = {
         ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_linear_float32_v1": (
         ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P]),
+    "nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
     "nfn_native_tile_argmax_rows_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "nfn_native_tile_glimmer_sigmoid_gate_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
     "nfn_native_tile_swiglu_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
@@ -242,6 +250,54 @@ def multi_linear(weights: Sequence[PackedWeight], x, workspace, second=None, fam
              workspace.numel(), stream]
     check(function(*args), _MULTI[(family, prologue)])
     return outputs
+
+
+def multi_linear_prequantized(weights: Sequence[PackedWeight], rows: int, workspace, outputs=None):
+    """Projections of the input whose activation records a verifier-family call or the
+    dual-RMS handoff left in `workspace`."""
+    import torch
+    stream = _stream_handle()
+    if outputs is None:
+        outputs = [torch.empty((rows, w.output_dim), dtype=torch.float32, device=workspace.device)
+                   for w in weights]
+    descriptors = [w.descriptor(stream) for w in weights]
+    check(load().nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1(
+        _descriptor_array(descriptors), _pointer_array(outputs), len(weights), rows,
+        workspace.data_ptr(), workspace.numel(), stream), "mmvq_multi_linear_prequantized")
+    return outputs
+
+
+def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = None,
+                         first_centered: bool = False,
+                         second_weight: Optional[PackedWeight] = None,
+                         second_centered: bool = False, first_eps: float = 1e-6,
+                         second_eps: float = 1e-6, handoff_workspace=None):
+    """hidden = residual + rms(x, first); normalized = rms(hidden, second).
+
+    Returns (hidden, normalized, residual_output).  With `handoff_workspace` (one row) the
+    activation records of `normalized` are left there for multi_linear_prequantized.
+    """
+    import torch
+    rows, width = x.shape
+    stream = _stream_handle()
+    hidden = torch.empty_like(x)
+    normalized = torch.empty_like(x)
+    captured = torch.empty_like(x)
+    first = first_weight.descriptor(stream) if first_weight is not None else None
+    second = second_weight.descriptor(stream) if second_weight is not None else None
+    arguments = [x.data_ptr(), ctypes.byref(first) if first is not None else None,
+                 residual.data_ptr(), hidden.data_ptr(),
+                 ctypes.byref(second) if second is not None else None, normalized.data_ptr(),
+                 captured.data_ptr(), rows, width, first_eps, first_centered, second_eps,
+                 second_centered]
+    if handoff_workspace is None:
+        check(load().nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(*arguments, stream),
+              "dual_rms_add_capture")
+    else:
+        check(load().nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
+            *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
+            "dual_rms_add_capture_mmvq_q8")
+    return hidden, normalized, captured
 
 
 def mmvq_linear(weight: PackedWeight, x, workspace, out=None):

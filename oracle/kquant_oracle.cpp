@@ -17,6 +17,8 @@
 //   Q8_1 quantize    neuralfn/csrc/tile_cuda/kernels.cu:1527-1562
 //   Q8_1 x K dot     neuralfn/csrc/tile_cuda/kernels.cu:1620-1731
 //   Q8_0 layout      neuralfn/csrc/tile_cuda/vendor/llama_mmq_62bf73d/ggml/src/ggml-common.h:251-256
+//   rms_norm         neuralfn/csrc/native_gpt2/resident_glimmer.cpp:713-745
+//   dual RMS         neuralfn/csrc/tile_cuda/kernels.cu:2155-2243
 //
 // Pinning status (what checks each function besides its own formula):
 //   nfo_fp16_to_float   exhaustive 65,536-value sweep against numpy float16.
@@ -37,6 +39,15 @@
 //                       (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:968-1007).
 //   nfo_linear_q8_1     closed form over reconstructed activations, same rule
 //                       as tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1009-1023.
+//   nfo_rms_norm        equals the compiled reference rms_norm() bit for bit where
+//                       that builds; closed form x / sqrt(mean(x^2) + eps) in numpy.
+//   nfo_dual_rms_add_capture  within the reference probe's 2e-5 of the double
+//                       form (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:243-256)
+//                       composed from nfo_rms_norm; its summation order (256
+//                       strided partial sums, halving tree) against an
+//                       independent numpy statement of the same order.  The
+//                       last bits of the reference device kernel's approximate
+//                       reciprocal square root are parity unpinned.
 //
 // Build: g++ -std=c++17 -O2 -pthread -ffp-contract=off -shared -fPIC.
 // -ffp-contract=off keeps `d*float(sc*q) - dmin*float(m)` as two roundings,
@@ -479,6 +490,85 @@ void nfo_swiglu(const float* gate, const float* up, float* output, std::int64_t 
     for (std::int64_t index = 0; index < count; ++index) {
         const float sigmoid = 1.0f / (1.0f + std::exp(-gate[index]));
         output[index] = (up[index] * gate[index]) * sigmoid;
+    }
+}
+
+// RMS normalisation as the reference's CPU engine computes it
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:713-745): squares summed in
+// double in column order, one double reciprocal square root, one rounding to
+// float per element.  `weight` is null or `width` floats; `centered` adds one.
+void nfo_rms_norm(const float* input, const float* weight, int centered, std::int64_t width,
+                  double epsilon, float* output) {
+    double squares = 0.0;
+    for (std::int64_t index = 0; index < width; ++index) {
+        squares += static_cast<double>(input[index]) * input[index];
+    }
+    const double inverse = 1.0 / std::sqrt(squares / static_cast<double>(width) + epsilon);
+    for (std::int64_t index = 0; index < width; ++index) {
+        double scale = 1.0;
+        if (weight != nullptr) {
+            scale = weight[index];
+            if (centered) scale += 1.0;
+        }
+        output[index] = static_cast<float>(static_cast<double>(input[index]) * inverse * scale);
+    }
+}
+
+// The two adjacent normalisations of the decode loop in the strict float
+// order of the reference's device kernel
+// (neuralfn/csrc/tile_cuda/kernels.cu:2155-2243): 256 strided partial sums of
+// squares built with fused multiply-adds, a halving tree over them,
+// (x * inverse_rms) * scale with two roundings, one rounded add of the residual.
+// inverse_rms is 1 / sqrt(mean + eps) with IEEE division and square root; the
+// device kernel of the reference uses an approximate reciprocal square root
+// there, which this restatement cannot reproduce bit for bit.
+static float nfo_strict_inverse_rms(const float* values, std::int64_t width, float eps) {
+    float partials[256];
+    for (int lane = 0; lane < 256; ++lane) {
+        float square_sum = 0.0f;
+        for (std::int64_t column = lane; column < width; column += 256) {
+            square_sum = std::fmaf(values[column], values[column], square_sum);
+        }
+        partials[lane] = square_sum;
+    }
+    for (int stride = 128; stride > 0; stride /= 2) {
+        for (int lane = 0; lane < stride; ++lane) partials[lane] += partials[lane + stride];
+    }
+    const float mean = partials[0] / static_cast<float>(width);
+    return 1.0f / std::sqrt(mean + eps);
+}
+
+void nfo_dual_rms_add_capture(const float* input, const float* first_weight, int first_centered,
+                              const float* residual_input, float* hidden_output,
+                              const float* second_weight, int second_centered,
+                              float* normalized_output, std::int64_t rows, std::int64_t width,
+                              float first_eps, float second_eps) {
+    for (std::int64_t row = 0; row < rows; ++row) {
+        const float* source = input + row * width;
+        const float* residual = residual_input + row * width;
+        float* hidden = hidden_output + row * width;
+        float* normalized = normalized_output + row * width;
+        const float first_inverse = nfo_strict_inverse_rms(source, width, first_eps);
+        for (std::int64_t column = 0; column < width; ++column) {
+            float scale = 1.0f;
+            if (first_weight != nullptr) {
+                scale = first_weight[column];
+                if (first_centered) scale += 1.0f;
+            }
+            const float scaled = source[column] * first_inverse;
+            const float value = scaled * scale;
+            hidden[column] = value + residual[column];
+        }
+        const float second_inverse = nfo_strict_inverse_rms(hidden, width, second_eps);
+        for (std::int64_t column = 0; column < width; ++column) {
+            float scale = 1.0f;
+            if (second_weight != nullptr) {
+                scale = second_weight[column];
+                if (second_centered) scale += 1.0f;
+            }
+            const float scaled = hidden[column] * second_inverse;
+            normalized[column] = scaled * scale;
+        }
     }
 }
 

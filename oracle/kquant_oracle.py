@@ -64,6 +64,11 @@ def lib() -> ctypes.CDLL:
         o.nfo_sigmoid_gate.restype = None
         o.nfo_swiglu.argtypes = [_P, _P, _P, _I64]
         o.nfo_swiglu.restype = None
+        o.nfo_rms_norm.argtypes = [_P, _P, ctypes.c_int, _I64, ctypes.c_double, _P]
+        o.nfo_rms_norm.restype = None
+        o.nfo_dual_rms_add_capture.argtypes = [_P, _P, ctypes.c_int, _P, _P, _P, ctypes.c_int, _P,
+                                               _I64, _I64, ctypes.c_float, ctypes.c_float]
+        o.nfo_dual_rms_add_capture.restype = None
         _oracle = o
     return _oracle
 
@@ -86,6 +91,8 @@ def ref() -> ctypes.CDLL:
         r.nfr_dequantize.restype = ctypes.c_int
         r.nfr_linear.argtypes = [_U32, _P, _I64, _I64, _P, _I64, _P]
         r.nfr_linear.restype = ctypes.c_int
+        r.nfr_rms_norm.argtypes = [_P, _P, ctypes.c_int, _I64, ctypes.c_double, _P]
+        r.nfr_rms_norm.restype = ctypes.c_int
         r.nfr_argmax.argtypes = [_P, _I64]
         r.nfr_argmax.restype = _I64
         _ref = r
@@ -200,7 +207,53 @@ def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
     return out
 
 
+def _optional(values):
+    if values is None:
+        return None, None
+    array = np.ascontiguousarray(values, dtype=np.float32)
+    return array, array.ctypes.data
+
+
+def rms_norm(x: np.ndarray, weight=None, centered: bool = False, epsilon: float = 1e-6) -> np.ndarray:
+    """One row through the CPU engine's RMSNorm (double accumulation)."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    _keep, pointer = _optional(weight)
+    out = np.empty_like(x)
+    lib().nfo_rms_norm(x.ctypes.data, pointer, int(centered), x.size, float(epsilon), out.ctypes.data)
+    return out
+
+
+def dual_rms_add_capture(x: np.ndarray, residual: np.ndarray, first_weight=None,
+                         first_centered: bool = False, second_weight=None,
+                         second_centered: bool = False, first_eps: float = 1e-6,
+                         second_eps: float = 1e-6):
+    """(hidden, normalized) in the strict float order of the device kernel."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    residual = np.ascontiguousarray(residual, dtype=np.float32)
+    rows, width = x.shape
+    _first, first_pointer = _optional(first_weight)
+    _second, second_pointer = _optional(second_weight)
+    hidden = np.empty_like(x)
+    normalized = np.empty_like(x)
+    lib().nfo_dual_rms_add_capture(x.ctypes.data, first_pointer, int(first_centered),
+                                   residual.ctypes.data, hidden.ctypes.data, second_pointer,
+                                   int(second_centered), normalized.ctypes.data, rows, width,
+                                   first_eps, second_eps)
+    return hidden, normalized
+
+
 # ---- the compiled reference (only where `make ref` has been run) ----------
+
+def ref_rms_norm(x: np.ndarray, weight=None, centered: bool = False, epsilon: float = 1e-6):
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    _keep, pointer = _optional(weight)
+    out = np.empty_like(x)
+    status = ref().nfr_rms_norm(x.ctypes.data, pointer, int(centered), x.size, float(epsilon),
+                                out.ctypes.data)
+    if status:
+        raise ValueError(f"reference rms_norm status {status}")
+    return out
+
 
 def ref_dequantize(encoding: int, packed: np.ndarray, output_dim: int, input_dim: int):
     packed = _bytes(packed)

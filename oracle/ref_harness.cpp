@@ -87,6 +87,28 @@ int nfr_linear(std::uint32_t encoding, const std::uint8_t* data, std::int64_t ou
     return 0;
 }
 
+// The reference's CPU RMSNorm (resident_glimmer.cpp:713-745) with an optional
+// F32 weight row.
+int nfr_rms_norm(const float* input, const float* weight, int centered, std::int64_t width,
+                 double epsilon, float* output) {
+    View view;
+    if (weight != nullptr) {
+        if (!make_view(0, reinterpret_cast<const std::uint8_t*>(weight), 1, width, &view)) return 1;
+        view.centered = centered != 0;
+    }
+    const std::atomic<bool> cancelled{false};
+    try {
+        const std::vector<float> source(input, input + width);
+        std::vector<float> result;
+        neuralfn::resident_glimmer::rms_norm(source, weight != nullptr ? &view : nullptr, epsilon,
+                                            &result, cancelled);
+        std::copy(result.begin(), result.end(), output);
+    } catch (const std::exception&) {
+        return 2;
+    }
+    return 0;
+}
+
 std::int64_t nfr_argmax(const float* values, std::int64_t count) {
     const std::vector<float> logits(values, values + count);
     return neuralfn::resident_glimmer::argmax_token(logits);

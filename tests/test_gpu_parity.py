@@ -490,6 +490,135 @@ def test_lm_head_full_vocabulary_planted_maxima(cuda, oracle, rows):
         assert abs(maxima.cpu()[token].item() - expected_value[token]) <= TOLERANCE * abs(expected_value[token])
 
 
+# ---------------------------- dual RMS normalisation and the prequantized handoff
+
+def norm_weight(values, encoding, device):
+    """A [1, width] norm weight as a packed-weight descriptor (F32 or BF16 row)."""
+    values = np.ascontiguousarray(values, dtype=np.float32)
+    if encoding == kquant.BF16:
+        values = (values.view(np.uint32) & 0xffff0000).view(np.float32)  # exactly representable
+        raw = (values.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+    else:
+        raw = values.view(np.uint8)
+    return values, tile_ops.PackedWeight(encoding, 1, values.size, to_device(raw.copy(), device))
+
+
+def probe_rms_input(rows, width):
+    index = np.arange(rows * width)
+    return (((index % 37) - 18) / 11.0).astype(np.float32).reshape(rows, width)  # probe :222-225
+
+
+@pytest.mark.parametrize("weights", ["none", "f32", "bf16_centered"])
+def test_dual_rms_add_capture_against_oracle(cuda, oracle, weights):
+    rows, width = 3, 6656
+    x = probe_rms_input(rows, width)
+    residual = np.random.default_rng(31).standard_normal((rows, width)).astype(np.float32)
+    first = second = None
+    first_values = second_values = None
+    centered = weights == "bf16_centered"
+    if weights != "none":
+        encoding = kquant.F32 if weights == "f32" else kquant.BF16
+        rng = np.random.default_rng(32)
+        first_values, first = norm_weight(rng.standard_normal(width) * 0.2, encoding, cuda)
+        second_values, second = norm_weight(rng.standard_normal(width) * 0.2 + 1.0, encoding, cuda)
+    hidden, normalized, captured = tile_ops.dual_rms_add_capture(
+        to_device(x, cuda), to_device(residual, cuda), first, centered, second, False, 1e-8, 1e-5)
+    expected_hidden, expected_normalized = oracle.dual_rms_add_capture(
+        x, residual, first_values, centered, second_values, False, 1e-8, 1e-5)
+    assert_bits_equal(hidden, expected_hidden, "hidden")
+    assert_bits_equal(normalized, expected_normalized, "normalized")
+    assert_bits_equal(captured, hidden, "residual capture")
+    # the CPU engine's double form, at the reference probe's tolerance (:243-256)
+    for row in range(rows):
+        reference_hidden = oracle.rms_norm(x[row], first_values, centered, 1e-8) + residual[row]
+        assert np.max(np.abs(hidden.cpu().numpy()[row] - reference_hidden)) <= 2e-5
+        reference_normalized = oracle.rms_norm(reference_hidden, second_values, False, 1e-5)
+        assert np.max(np.abs(normalized.cpu().numpy()[row] - reference_normalized)) <= 2e-5
+
+
+def test_dual_rms_handoff_equals_ordinary_path(cuda, oracle):
+    # probe :1694-1762: the handoff's three outputs and the projection fed from
+    # its records equal the ordinary dual RMS followed by the ordinary one-row call.
+    width = 6656
+    x = probe_rms_input(1, width)
+    residual = np.random.default_rng(33).standard_normal((1, width)).astype(np.float32)
+    specs = [(kquant.Q4_K, 129), (kquant.Q5_K, 33), (kquant.Q6_K, 70), (kquant.Q8_0, 17)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, width, 40 + i), n, width)
+               for i, (e, n) in enumerate(specs)]
+    workspace = tile_ops.small_batch_workspace(1, width)
+    ordinary = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda),
+                                             first_eps=1e-8, second_eps=1e-5)
+    ordinary_out = tile_ops.multi_linear(weights, ordinary[1], workspace)
+    workspace.zero_()
+    handoff = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda),
+                                            first_eps=1e-8, second_eps=1e-5,
+                                            handoff_workspace=workspace)
+    handoff_out = tile_ops.multi_linear_prequantized(weights, 1, workspace)
+    for a, b, label in zip(ordinary, handoff, ("hidden", "normalized", "capture")):
+        assert_bits_equal(a, b, label)
+    for a, b, (encoding, _) in zip(ordinary_out, handoff_out, specs):
+        assert_bits_equal(a, b, kquant.NAMES[encoding])
+    # and the values are right, not just equal
+    normalized = ordinary[1].cpu().numpy()
+    for (encoding, out_dim), weight, y in zip(specs, weights, ordinary_out):
+        exact = oracle.linear(encoding, weight.data.cpu().numpy(), out_dim, width, normalized)
+        assert normalised_error(y.cpu().numpy(), exact) <= TOLERANCE
+
+
+@pytest.mark.parametrize("rows", [1, 5, 16])
+def test_prequantized_reuses_the_records_of_a_verifier_call(cuda, rows):
+    # The engine's verifier quantizes once for Q and feeds K, V and the gate from the
+    # same workspace (resident_glimmer_cuda.cpp:3649-3666).
+    in_dim = 1024
+    x = to_device(kquant.synthetic_activations(51, rows, in_dim), cuda)
+    specs = [(kquant.Q4_K, 64), (kquant.Q6_K, 40), (kquant.Q5_K, 24), (kquant.Q8_0, 48)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, in_dim, 60 + i), n, in_dim)
+               for i, (e, n) in enumerate(specs)]
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    direct = tile_ops.multi_linear(weights[1:], x, workspace, family="mmvq")
+    workspace.zero_()
+    tile_ops.multi_linear(weights[:1], x, workspace, family="mmvq")
+    reused = tile_ops.multi_linear_prequantized(weights[1:], rows, workspace)
+    for a, b, (encoding, _) in zip(direct, reused, specs[1:]):
+        assert_bits_equal(a, b, kquant.NAMES[encoding])
+
+
+def test_handoff_and_prequantized_fail_closed(cuda):
+    width = 512
+    lib = tile_ops.load()
+    x = to_device(probe_rms_input(2, width), cuda)
+    outputs = [torch_().empty_like(x) for _ in range(3)]
+    workspace = tile_ops.small_batch_workspace(2, width)
+    head = [x.data_ptr(), None, x.data_ptr(), outputs[0].data_ptr(), None, outputs[1].data_ptr(),
+            outputs[2].data_ptr()]
+    tail = [1e-8, False, 1e-5, False]
+    handoff = lib.nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1
+    required = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(1, width)
+    assert handoff(*head, 1, width, *tail, workspace.data_ptr(), required, None) == 0
+    assert handoff(*head, 2, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 1, width, *tail, workspace.data_ptr(), required - 1, None) == 1
+    assert handoff(*head, 1, width, *tail, None, required, None) == 1
+    assert handoff(*head, 1, 480, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    plain = lib.nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1
+    assert plain(*head, 2, width, *tail, None) == 0
+    assert plain(*head, 2, width, 0.0, False, 1e-5, False, None) == 1
+    assert plain(*head, 2, 65537, *tail, None) == 1
+    assert plain(*head, 0, width, *tail, None) == 1
+    torch_().cuda.synchronize()
+    weight = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, 8, width, 1),
+                                              8, width)
+    out = torch_().empty((16, 8), dtype=torch_().float32, device=cuda)
+    prequantized = lib.nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1
+    descriptor = weight.descriptor(0)
+    descriptors = tile_ops._descriptor_array([descriptor])
+    pointers = tile_ops._pointer_array([out])
+    big = tile_ops.small_batch_workspace(16, width)
+    assert prequantized(descriptors, pointers, 1, 17, big.data_ptr(), big.numel(), None) == 1
+    assert prequantized(descriptors, pointers, 1, 2, big.data_ptr(), required, None) == 1
+    assert prequantized(descriptors, pointers, 0, 1, big.data_ptr(), big.numel(), None) == 1
+    assert prequantized(descriptors, pointers, 1, 1, None, big.numel(), None) == 1
+
+
 # ------------------------------------------------ the benchmark's geometries
 
 def config_layer(seed, encoding=kquant.Q4_K):

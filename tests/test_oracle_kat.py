@@ -230,3 +230,58 @@ def test_worker_count_follows_reference_cap(oracle):
     assert oracle.worker_count(100) == 1
     assert oracle.worker_count(129, cap=2) == 2
     assert oracle.worker_count(10**6, cap=64) <= 32
+
+
+def test_rms_norm_closed_form(oracle):
+    # x / sqrt(mean(x^2) + eps) * (w or 1, plus 1 when centered), in double
+    # (resident_glimmer.cpp:713-745); one rounding to float per element.
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(1536).astype(np.float32)
+    w = rng.standard_normal(1536).astype(np.float32)
+    inverse = 1.0 / np.sqrt(np.mean(x.astype(np.float64) ** 2) + 1e-6)
+    assert np.array_equal(oracle.rms_norm(x, None, False, 1e-6),
+                          (x.astype(np.float64) * inverse).astype(np.float32))
+    assert np.array_equal(oracle.rms_norm(x, w, False, 1e-6),
+                          (x.astype(np.float64) * inverse * w.astype(np.float64)).astype(np.float32))
+    assert np.array_equal(
+        oracle.rms_norm(x, w, True, 1e-6),
+        (x.astype(np.float64) * inverse * (w.astype(np.float64) + 1.0)).astype(np.float32))
+    # a constant row normalises to +-1 (eps negligible)
+    assert np.allclose(oracle.rms_norm(np.full(512, -3.0, np.float32), None, False, 1e-12), -1.0)
+
+
+def test_dual_rms_strict_order_and_double_form(oracle):
+    # The device order (kernels.cu:2155-2243) restated independently in numpy:
+    # 256 strided float partial sums (products are exact in double, each step
+    # rounds once like a fused multiply-add), a halving tree, float arithmetic after.
+    def inverse_rms(values, eps):
+        partials = np.zeros(256, dtype=np.float32)
+        for start in range(0, values.size, 256):
+            chunk = values[start:start + 256].astype(np.float64)
+            lanes = chunk.size
+            partials[:lanes] = (chunk * chunk + partials[:lanes].astype(np.float64)).astype(np.float32)
+        stride = 128
+        while stride:
+            partials[:stride] = partials[:stride] + partials[stride:2 * stride]
+            stride //= 2
+        mean = np.float32(partials[0] / np.float32(values.size))
+        return np.float32(1.0) / np.sqrt(np.float32(mean + np.float32(eps)), dtype=np.float32)
+
+    rows, width = 2, 6656
+    index = np.arange(rows * width)
+    x = (((index % 37) - 18) / 11.0).astype(np.float32).reshape(rows, width)  # probe :222-225
+    residual = np.random.default_rng(6).standard_normal((rows, width)).astype(np.float32)
+    weight = np.random.default_rng(7).standard_normal(width).astype(np.float32)
+    hidden, normalized = oracle.dual_rms_add_capture(x, residual, weight, True, None, False,
+                                                     1e-8, 1e-5)
+    for row in range(rows):
+        first = inverse_rms(x[row], 1e-8)
+        expected_hidden = (x[row] * first) * (weight + np.float32(1.0)) + residual[row]
+        assert np.array_equal(hidden[row], expected_hidden.astype(np.float32))
+        second = inverse_rms(hidden[row], 1e-5)
+        assert np.array_equal(normalized[row], hidden[row] * second)
+        # the double form of the CPU engine, at the reference probe's tolerance (:243-256)
+        reference_hidden = oracle.rms_norm(x[row], weight, True, 1e-8) + residual[row]
+        assert np.max(np.abs(hidden[row] - reference_hidden)) <= 2e-5
+        assert np.max(np.abs(normalized[row] - oracle.rms_norm(reference_hidden, None, False, 1e-5))) <= 2e-5
+

@@ -87,3 +87,16 @@ def test_linear_matches_committed_reference_vectors(oracle, encoding):
     assert np.array_equal(y.view(np.uint32), data[f"{name}_output"].view(np.uint32))
     w = oracle.dequantize(encoding, packed, out_dim, in_dim, q6_as_written=True)
     assert np.array_equal(w.view(np.uint32), data[f"{name}_weights"].view(np.uint32))
+
+
+@needs_ref
+@pytest.mark.parametrize("centered", [False, True])
+def test_rms_norm_matches_reference_bit_for_bit(oracle, centered):
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal(6656).astype(np.float32)
+    weight = rng.standard_normal(6656).astype(np.float32)
+    assert np.array_equal(oracle.rms_norm(x, weight, centered, 1e-6),
+                          oracle.ref_rms_norm(x, weight, centered, 1e-6))
+    assert np.array_equal(oracle.rms_norm(x, None, False, 1e-8),
+                          oracle.ref_rms_norm(x, None, False, 1e-8))
+
