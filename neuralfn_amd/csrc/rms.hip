@@ -8,7 +8,9 @@
 // the caller's small-batch workspace, so that the projection that follows can
 // skip its own quantization.
 //
-// One workgroup of 256 threads per row.  The float arithmetic follows the
+// One workgroup of 256 threads per row; rows of up to 8192 columns take the
+// register-resident kernel, wider ones the kernel that walks memory in batches.
+// The float arithmetic follows the
 // reference kernel operation for operation
 // (neuralfn/csrc/tile_cuda/kernels.cu:2155-2243): thread t accumulates the
 // squares of columns t, t+256, ... with fused multiply-adds, the 256 partial
@@ -141,6 +143,105 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_add_capture_kernel(
     }
 }
 
+// The halving tree over 256 partial sums with the additions in the same order
+// as the loop above: two steps through LDS, the last six inside the first wave
+// (lane t adds the value of lane t + stride, as the tree does).
+__device__ __forceinline__ float tree_total(float square_sum, float* partials) {
+    partials[threadIdx.x] = square_sum;
+    __syncthreads();
+    if (threadIdx.x < 128) partials[threadIdx.x] += partials[threadIdx.x + 128];
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float value = partials[threadIdx.x] + partials[threadIdx.x + 64];
+#pragma unroll
+        for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
+        if (threadIdx.x == 0) partials[0] = value;
+    }
+    __syncthreads();
+    const float total = partials[0];
+    __syncthreads();  // partials are reused by the next reduction
+    return total;
+}
+
+// Rows of up to 8192 columns: a thread keeps its (at most 32) columns of every
+// operand in registers.  All loads of the kernel go out at its start; the
+// second normalisation needs no second pass over memory because the columns a
+// thread sums in the second reduction are the ones it produced in the first.
+// Same arithmetic, same order, same bits as the kernel above.
+constexpr int kOwned = 32;
+
+template <bool HANDOFF>
+__global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
+    const float* __restrict__ input, NormWeight first_weight,
+    const float* __restrict__ residual_input, float* __restrict__ hidden_output,
+    NormWeight second_weight, float* __restrict__ normalized_output,
+    float* __restrict__ residual_output, int width, float first_eps, float second_eps,
+    std::uint8_t* __restrict__ records) {
+    __shared__ float partials[kRmsThreads];
+    extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF: the normalized row
+    const std::int64_t row = blockIdx.x;
+    const float* source = input + row * width;
+    const float* residual = residual_input + row * width;
+    float* hidden = hidden_output + row * width;
+    float* captured = residual_output + row * width;
+    float* normalized = normalized_output + row * width;
+
+    float value[kOwned], other[kOwned], first_scale[kOwned], second_scale[kOwned];
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) {
+        const int column = threadIdx.x + i * kRmsThreads;
+        const int clamped = min(column, width - 1);
+        value[i] = column < width ? source[clamped] : 0.0f;
+        other[i] = residual[clamped];
+        first_scale[i] = norm_scale(first_weight, clamped);
+        second_scale[i] = norm_scale(second_weight, clamped);
+    }
+
+    float square_sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) square_sum = fmaf(value[i], value[i], square_sum);
+    const float first_inverse =
+        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + first_eps);
+
+    square_sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) {
+        const int column = threadIdx.x + i * kRmsThreads;
+        const float sum =
+            __fadd_rn(__fmul_rn(__fmul_rn(value[i], first_inverse), first_scale[i]), other[i]);
+        value[i] = column < width ? sum : 0.0f;
+        if (column < width) {
+            hidden[column] = sum;
+            captured[column] = sum;
+        }
+        square_sum = fmaf(value[i], value[i], square_sum);
+    }
+    const float second_inverse =
+        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + second_eps);
+
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) {
+        const int column = threadIdx.x + i * kRmsThreads;
+        const float result = __fmul_rn(__fmul_rn(value[i], second_inverse), second_scale[i]);
+        if (column < width) {
+            normalized[column] = result;
+            if constexpr (HANDOFF) staged[column] = result;
+        }
+    }
+
+    if constexpr (HANDOFF) {
+        __syncthreads();
+        // one wave per 256-value block: the quantizer of the decode kernels
+        const int lane = threadIdx.x & 63;
+        const int wave = threadIdx.x >> 6;
+        for (int block = wave; block < (width >> 8); block += kRmsThreads / kWave) {
+            const float4 x = *reinterpret_cast<const float4*>(staged + block * 256 + lane * 4);
+            store_record(records + static_cast<std::int64_t>(block) * kActRecord, lane,
+                         encode_activations(x));
+        }
+    }
+}
+
 NormWeight norm_weight(const Descriptor* descriptor, bool centered) {
     NormWeight weight{};
     if (descriptor != nullptr) {
@@ -164,6 +265,21 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
     const NormWeight first = norm_weight(first_weight, first_centered);
     const NormWeight second = norm_weight(second_weight, second_centered);
     const dim3 grid(static_cast<unsigned>(rows));
+    if (width <= kOwned * kRmsThreads) {
+        const int columns = static_cast<int>(width);
+        if (records != nullptr) {
+            hipLaunchKernelGGL((dual_rms_resident_kernel<true>), grid, dim3(kRmsThreads),
+                               static_cast<std::size_t>(columns) * sizeof(float), stream, input,
+                               first, residual_input, hidden_output, second, normalized_output,
+                               residual_output, columns, first_eps, second_eps, records);
+        } else {
+            hipLaunchKernelGGL((dual_rms_resident_kernel<false>), grid, dim3(kRmsThreads), 0, stream,
+                               input, first, residual_input, hidden_output, second,
+                               normalized_output, residual_output, columns, first_eps, second_eps,
+                               records);
+        }
+        return;
+    }
     if (records != nullptr) {
         hipLaunchKernelGGL((dual_rms_add_capture_kernel<true>), grid, dim3(kRmsThreads), 0, stream,
                            input, first, residual_input, hidden_output, second, normalized_output,

@@ -536,6 +536,22 @@ def test_dual_rms_add_capture_against_oracle(cuda, oracle, weights):
         assert np.max(np.abs(normalized.cpu().numpy()[row] - reference_normalized)) <= 2e-5
 
 
+def test_dual_rms_add_capture_wide_rows(cuda, oracle):
+    # wider than the register-resident kernel takes: the kernel that walks memory in batches
+    rows, width = 2, 12288 + 32
+    rng = np.random.default_rng(34)
+    x = rng.standard_normal((rows, width)).astype(np.float32)
+    residual = rng.standard_normal((rows, width)).astype(np.float32)
+    first_values, first = norm_weight(rng.standard_normal(width) * 0.3, kquant.F32, cuda)
+    hidden, normalized, captured = tile_ops.dual_rms_add_capture(
+        to_device(x, cuda), to_device(residual, cuda), first, True, None, False, 1e-6, 1e-6)
+    expected_hidden, expected_normalized = oracle.dual_rms_add_capture(
+        x, residual, first_values, True, None, False, 1e-6, 1e-6)
+    assert_bits_equal(hidden, expected_hidden, "hidden")
+    assert_bits_equal(normalized, expected_normalized, "normalized")
+    assert_bits_equal(captured, hidden, "residual capture")
+
+
 def test_dual_rms_handoff_equals_ordinary_path(cuda, oracle):
     # probe :1694-1762: the handoff's three outputs and the projection fed from
     # its records equal the ordinary dual RMS followed by the ordinary one-row call.
