@@ -295,8 +295,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 
 template <std::uint32_t ENC, int T, int P>
 void launch_variant(ProjectionSet set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens,
-                    hipStream_t stream) {
+                    std::uint8_t* records_out, int tokens, hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
@@ -319,8 +318,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
 
 template <std::uint32_t ENC, int P>
 void launch_tokens(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens,
-                   hipStream_t stream) {
+                   std::uint8_t* records_out, int tokens, hipStream_t stream) {
     // token planes of one pass must fit in LDS: four tokens up to K = 16384
     const std::int64_t image = token_image_bytes_host(set.input_dim >> 8);
     int capacity = static_cast<int>((150 * 1024) / image);
@@ -339,12 +337,20 @@ void launch_tokens(const ProjectionSet& set, const float* first, const float* se
 
 template <std::uint32_t ENC>
 void launch_prologue(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int prologue, int tokens, hipStream_t stream) {
+                     std::uint8_t* records_out, int prologue, int tokens, hipStream_t stream) {
     switch (prologue) {
-        case kGated: launch_tokens<ENC, kGated>(set, first, second, records_out, tokens, stream); break;
-        case kSwiGlu: launch_tokens<ENC, kSwiGlu>(set, first, second, records_out, tokens, stream); break;
-        case kRecords: launch_tokens<ENC, kRecords>(set, first, second, nullptr, tokens, stream); break;
-        default: launch_tokens<ENC, kPlain>(set, first, second, records_out, tokens, stream); break;
+        case kGated:
+            launch_tokens<ENC, kGated>(set, first, second, records_out, tokens, stream);
+            break;
+        case kSwiGlu:
+            launch_tokens<ENC, kSwiGlu>(set, first, second, records_out, tokens, stream);
+            break;
+        case kRecords:
+            launch_tokens<ENC, kRecords>(set, first, second, nullptr, tokens, stream);
+            break;
+        default:
+            launch_tokens<ENC, kPlain>(set, first, second, records_out, tokens, stream);
+            break;
     }
 }
 
@@ -356,7 +362,8 @@ bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
+                     std::uint8_t* records_out, int prologue, std::int64_t rows,
+                     hipStream_t stream) {
     const std::uint32_t encodings[2] = {kEncQ4K, kEncQ5K};
     for (const std::uint32_t encoding : encodings) {
         ProjectionSet group{};
@@ -366,9 +373,11 @@ void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* 
         }
         if (group.count == 0) continue;
         if (encoding == kEncQ4K) {
-            launch_prologue<kEncQ4K>(group, first, second, records_out, prologue, static_cast<int>(rows), stream);
+            launch_prologue<kEncQ4K>(group, first, second, records_out, prologue,
+                                     static_cast<int>(rows), stream);
         } else {
-            launch_prologue<kEncQ5K>(group, first, second, records_out, prologue, static_cast<int>(rows), stream);
+            launch_prologue<kEncQ5K>(group, first, second, records_out, prologue,
+                                     static_cast<int>(rows), stream);
         }
     }
 }

@@ -625,7 +625,8 @@ Geometry geometry(std::int64_t rows) {
 // launch: with the argmax fused in, that is the number of candidates per token.
 template <int T, int P, bool ARGMAX>
 std::int64_t launch_variant(ProjectionSet set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+                            std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates,
+                            hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
@@ -670,7 +671,8 @@ constexpr int stream_waves(int tokens_per_pass) {
 
 template <int T, int P, bool ARGMAX>
 std::int64_t launch_stream(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+                           std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates,
+                           hipStream_t stream) {
     constexpr int W = stream_waves(T);
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8) +
         W * kStagingBytes;
@@ -701,7 +703,8 @@ bool streams(std::int64_t input_dim) { return (input_dim >> 8) >= kPassBlocks; }
 
 template <int P, bool ARGMAX>
 std::int64_t launch_tokens(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
+                           std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates,
+                           hipStream_t stream) {
     // the token images of one pass (and the staging areas) must fit in LDS
     const std::int64_t image = token_image_bytes(set.input_dim >> 8);
     int capacity = static_cast<int>((150 * 1024 - 16 * kStagingBytes) / image);
@@ -733,7 +736,8 @@ bool gemv_q6_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_q6(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
+                    std::uint8_t* records_out, int prologue, std::int64_t rows,
+                    hipStream_t stream) {
     ProjectionSet group{};
     group.input_dim = set.input_dim;
     for (int index = 0; index < set.count; ++index) {

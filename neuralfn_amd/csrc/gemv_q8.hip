@@ -248,8 +248,7 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
 
 template <int T, int P>
 void launch_variant(ProjectionSet set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens,
-                    hipStream_t stream) {
+                    std::uint8_t* records_out, int tokens, hipStream_t stream) {
     std::int64_t rows = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
@@ -271,8 +270,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
 
 template <int P>
 void launch_tokens(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int tokens,
-                   hipStream_t stream) {
+                   std::uint8_t* records_out, int tokens, hipStream_t stream) {
     // the token images of one pass must fit in LDS
     const std::int64_t image = token_image_bytes(set.input_dim >> 8);
     int capacity = static_cast<int>((150 * 1024) / image);
@@ -295,7 +293,8 @@ bool gemv_q8_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 void launch_gemv_q8(const ProjectionSet& set, const float* first, const float* second,
-        std::uint8_t* records_out, int prologue, std::int64_t rows, hipStream_t stream) {
+                    std::uint8_t* records_out, int prologue, std::int64_t rows,
+                    hipStream_t stream) {
     ProjectionSet group{};
     group.input_dim = set.input_dim;
     for (int index = 0; index < set.count; ++index) {
