@@ -464,7 +464,7 @@ std::int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(std::int64_t rows, std::i
         mode != NFN_MI355_GEMM_F16) {
         return 0;
     }
-    return gemm_f16_workspace_bytes(rows, input_dim);
+    return gemm_f16_workspace_bytes(rows, input_dim, output_dim);
 }
 
 int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float* input,

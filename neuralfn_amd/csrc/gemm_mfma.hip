@@ -53,6 +53,7 @@ constexpr int kBM = 256;
 constexpr int kBN = 128;
 constexpr int kBK = 64;
 constexpr int kThreads = 256;
+constexpr int kMaxShares = 4;  // K shares of a split launch at most
 constexpr int kRowBytes = 144;  // 64 fp16 + 16 bytes of padding
 constexpr int kStageBytes = kBN * kRowBytes;
 constexpr int kFragmentBytes = 1024;  // 32 rows x 16 K values of fp16 in operand order
@@ -521,6 +522,10 @@ __device__ __forceinline__ void k_step(
     }
 }
 
+// bytes of 256 packed values
+template <std::uint32_t ENC>
+constexpr int kBlockBytes = ENC == kEncQ4K ? 144 : ENC == kEncQ5K ? 176 : ENC == kEncQ6K ? 210 : 272;
+
 // Workgroups per compute unit (= waves per SIMD): as many as the registers
 // allow; while one wave waits at the barrier or for LDS, another keeps the
 // matrix pipe busy.  With 256-row tiles the Q6_K decode holds too much live
@@ -535,7 +540,7 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB
     const std::uint8_t* __restrict__ weights, std::int64_t row_stride, std::int64_t output_dim,
     std::int64_t input_dim, const std::uint8_t* __restrict__ activations,
     const float* __restrict__ inverse_scale, float* __restrict__ output, std::int64_t rows,
-    int m_tiles) {
+    int m_tiles, std::int64_t split_stride) {
     extern __shared__ __attribute__((aligned(16))) std::uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -545,18 +550,25 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB
     constexpr int kTileRows = 128 * RB;
     const std::int64_t m0 = static_cast<std::int64_t>(m_tile) * kTileRows;
     const std::int64_t n0 = static_cast<std::int64_t>(n_tile) * kBN;
-    const int steps = static_cast<int>(input_dim / kBK);  // a positive multiple of 4
+    // blockIdx.y: which share of the K dimension (whole 256-value blocks) this
+    // workgroup sums; each share writes its own copy of the output
+    const int total_blocks = static_cast<int>(input_dim >> 8);
+    const int first_block = total_blocks * static_cast<int>(blockIdx.y) / static_cast<int>(gridDim.y);
+    const int end_block = total_blocks * (static_cast<int>(blockIdx.y) + 1) / static_cast<int>(gridDim.y);
+    const int steps = (end_block - first_block) * 4;  // a positive multiple of 4
     const int last = steps - 1;
+    output += blockIdx.y * split_stride;
 
     // activations: fragment (row block, K chunk) is 1 KB, a row block's chunks are consecutive
     const std::int64_t row_block_bytes = (input_dim / 16) * kFragmentBytes;
-    const std::uint8_t* a_global =
-        activations + (m0 / 32 + wave * RB) * row_block_bytes + lane * 16;
+    const std::uint8_t* a_global = activations + (m0 / 32 + wave * RB) * row_block_bytes +
+        static_cast<std::int64_t>(first_block) * 16 * kFragmentBytes + lane * 16;
     constexpr int kStepBytes = (kBK / 16) * kFragmentBytes;
     // weights: thread -> (row, which 16 positions of the two 32-value groups)
     const int b_row = tid >> 1;
     const int b_half = tid & 1;
-    const std::uint8_t* b_global = weights + min(n0 + b_row, output_dim - 1) * row_stride;
+    const std::uint8_t* b_global = weights + min(n0 + b_row, output_dim - 1) * row_stride +
+        static_cast<std::int64_t>(first_block) * kBlockBytes<ENC>;
     const int b_target = b_row * kRowBytes + b_half * 32;
 
     v16f acc[RB][4];
@@ -709,37 +721,100 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB
     }
 }
 
+// Sum of the K shares: output[i] = partial[0][i] + partial[1][i] + ..., in that order.
+__global__ __launch_bounds__(256) void sum_shares_kernel(const float* __restrict__ partials,
+                                                         float* __restrict__ output,
+                                                         std::int64_t count, int shares) {
+    const std::int64_t stride = static_cast<std::int64_t>(gridDim.x) * blockDim.x;
+    for (std::int64_t index = static_cast<std::int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+         index < count; index += stride) {
+        float total = partials[index];
+        for (int share = 1; share < shares; ++share) total += partials[share * count + index];
+        output[index] = total;
+    }
+}
+
+// Tile height and K shares of a launch, from a sweep over both on this chip.
+// 256-row tiles reuse each weight fragment twice as often and win whenever
+// they give every compute unit a workgroup.  A smaller problem splits K over
+// several workgroups per tile (at least twelve 256-value blocks each, at most
+// four shares) until the grid fills the units' two (256-row tiles) or three
+// (128-row tiles) workgroup slots; the shares are summed by a second launch in
+// a fixed order.  256-row tiles stay the better choice as long as two shares or
+// more fit; at most 128 rows, or a K too short to split, take 128-row tiles.
+struct Plan {
+    int row_blocks;  // 32-row blocks per wave: 2 = 256-row tiles, 1 = 128-row tiles
+    int shares;
+};
+
+Plan plan(std::uint32_t encoding, std::int64_t rows, std::int64_t output_dim,
+          std::int64_t input_dim) {
+    const std::int64_t units = compute_units();
+    const std::int64_t n_tiles = (output_dim + kBN - 1) / kBN;
+    const std::int64_t tall_tiles = (rows + 255) / 256 * n_tiles;
+    if (tall_tiles >= units) return Plan{2, 1};
+    std::int64_t longest = (input_dim >> 8) / 12;  // shares that still get twelve blocks each
+    if (longest > kMaxShares) longest = kMaxShares;
+    if (rows > 128) {
+        std::int64_t shares = 2 * units / tall_tiles;
+        if (shares > longest) shares = longest;
+        if (shares >= 2) return Plan{2, static_cast<int>(shares)};
+    }
+    const std::int64_t tiles = (rows + 127) / 128 * n_tiles;
+    std::int64_t shares = units * (encoding == kEncQ6K ? 2 : 3) / tiles;
+    if (shares > longest) shares = longest;
+    if (shares < 1) shares = 1;
+    return Plan{1, static_cast<int>(shares)};
+}
+
 template <std::uint32_t ENC>
 void launch_encoding(const Descriptor& descriptor, const std::uint8_t* activations,
-                     const float* inverse_scale, float* output, std::int64_t rows,
-                     hipStream_t stream) {
+                     const float* inverse_scale, float* output, float* partials,
+                     std::int64_t rows, hipStream_t stream) {
     const std::int64_t n_tiles = (descriptor.output_dim + kBN - 1) / kBN;
-    const std::int64_t tall_tiles = (rows + 255) / 256;
-    // 256-row tiles reuse each weight fragment twice as often and win whenever
-    // they give every compute unit a workgroup; 128-row tiles double the number
-    // of workgroups for the small problems that would leave units empty
-    if (tall_tiles * n_tiles >= compute_units()) {
-        const int m_tiles = static_cast<int>(tall_tiles);
-        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 2>), dim3(static_cast<unsigned>(m_tiles * n_tiles)),
+    const Plan chosen = plan(ENC, rows, descriptor.output_dim, descriptor.input_dim);
+    const std::int64_t count = rows * descriptor.output_dim;
+    float* target = chosen.shares > 1 ? partials : output;
+    const std::int64_t split_stride = chosen.shares > 1 ? count : 0;
+    if (chosen.row_blocks == 2) {
+        const int m_tiles = static_cast<int>((rows + 255) / 256);
+        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 2>),
+                           dim3(static_cast<unsigned>(m_tiles * n_tiles), chosen.shares),
                            dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,
                            descriptor.row_stride_bytes, descriptor.output_dim,
-                           descriptor.input_dim, activations, inverse_scale, output, rows, m_tiles);
+                           descriptor.input_dim, activations, inverse_scale, target, rows, m_tiles,
+                           split_stride);
     } else {
         const int m_tiles = static_cast<int>((rows + 127) / 128);
-        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 1>), dim3(static_cast<unsigned>(m_tiles * n_tiles)),
+        hipLaunchKernelGGL((gemm_f16_kernel<ENC, 1>),
+                           dim3(static_cast<unsigned>(m_tiles * n_tiles), chosen.shares),
                            dim3(kThreads), 2 * kStageBytes, stream, descriptor.data,
                            descriptor.row_stride_bytes, descriptor.output_dim,
-                           descriptor.input_dim, activations, inverse_scale, output, rows, m_tiles);
+                           descriptor.input_dim, activations, inverse_scale, target, rows, m_tiles,
+                           split_stride);
+    }
+    if (chosen.shares > 1) {
+        const std::int64_t blocks = (count + 1023) / 1024;
+        hipLaunchKernelGGL(sum_shares_kernel, dim3(static_cast<unsigned>(blocks < 4096 ? blocks : 4096)),
+                           dim3(256), 0, stream, partials, output, count, chosen.shares);
     }
 }
 
 std::int64_t padded_rows(std::int64_t rows) { return (rows + kBM - 1) / kBM * kBM; }
 
+// fp16 activations in whole 256-row tiles, then a scale and its inverse per row
+std::int64_t activation_bytes(std::int64_t rows, std::int64_t input_dim) {
+    return (padded_rows(rows) * input_dim * 2 + padded_rows(rows) * 8 + 255) & ~std::int64_t(255);
+}
+
 }  // namespace
 
-std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
-    // fp16 activations in whole 256-row tiles, then a scale and its inverse per row
-    return padded_rows(rows) * input_dim * 2 + padded_rows(rows) * 8 + 256;
+std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim,
+                                      std::int64_t output_dim) {
+    // the activations, then one copy of the output per K share of a split
+    // launch (the encoding with the most shares bounds the others)
+    const int shares = plan(kEncQ4K, rows, output_dim, input_dim).shares;
+    return activation_bytes(rows, input_dim) + (shares > 1 ? shares * rows * output_dim * 4 : 0) + 256;
 }
 
 bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
@@ -753,6 +828,8 @@ void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* ou
     float* inverse_scale =
         reinterpret_cast<float*>(activations + padded_rows(rows) * descriptor.input_dim * 2);
     float* scale = inverse_scale + padded_rows(rows);
+    float* partials =
+        reinterpret_cast<float*>(activations + activation_bytes(rows, descriptor.input_dim));
     hipLaunchKernelGGL(row_scale_kernel, dim3(static_cast<unsigned>(padded_rows(rows))), dim3(256),
                        0, stream, input, scale, inverse_scale, rows, descriptor.input_dim);
     hipLaunchKernelGGL(convert_activations_kernel,
@@ -762,16 +839,20 @@ void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* ou
                        descriptor.input_dim);
     switch (descriptor.encoding) {
         case kEncQ4K:
-            launch_encoding<kEncQ4K>(descriptor, activations, inverse_scale, output, rows, stream);
+            launch_encoding<kEncQ4K>(descriptor, activations, inverse_scale, output, partials, rows,
+                                     stream);
             break;
         case kEncQ5K:
-            launch_encoding<kEncQ5K>(descriptor, activations, inverse_scale, output, rows, stream);
+            launch_encoding<kEncQ5K>(descriptor, activations, inverse_scale, output, partials, rows,
+                                     stream);
             break;
         case kEncQ6K:
-            launch_encoding<kEncQ6K>(descriptor, activations, inverse_scale, output, rows, stream);
+            launch_encoding<kEncQ6K>(descriptor, activations, inverse_scale, output, partials, rows,
+                                     stream);
             break;
         default:
-            launch_encoding<kEncQ8_0>(descriptor, activations, inverse_scale, output, rows, stream);
+            launch_encoding<kEncQ8_0>(descriptor, activations, inverse_scale, output, partials, rows,
+                                     stream);
             break;
     }
 }

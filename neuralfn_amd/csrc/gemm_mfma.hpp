@@ -6,8 +6,11 @@
 namespace nfn {
 
 // Bytes of device workspace the fp16 path needs: a row-scaled fp16 copy of the
-// activations in whole 256-row tiles and one inverse scale per row.
-std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim);
+// activations in whole 256-row tiles, one inverse scale per row, and, where a
+// small problem splits K over several workgroups per tile, one copy of the
+// output per share.
+std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim,
+                                      std::int64_t output_dim);
 bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim);
 // output[rows, output_dim] = input[rows, input_dim] * W^T, float accumulation.
 void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,

@@ -725,6 +725,22 @@ def test_prefill_gemm_tall_tiles(cuda, oracle, encoding):
     assert normalised_error(y[picked], expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("in_dim", [4096, 6144])
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_prefill_gemm_split_k(cuda, oracle, encoding, in_dim):
+    # few tiles and a long K: the launch splits K into shares (two at 16 blocks,
+    # three at 24) and a second launch sums them
+    rows, out_dim = 96, 130
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(70 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(71, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda)).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    assert normalised_error(y, expected) <= TOLERANCE
+    again = tile_ops.gemm(weight, to_device(x, cuda)).cpu().numpy()
+    assert np.array_equal(y.view(np.uint32), again.view(np.uint32))  # fixed summation order
+
+
 def test_prefill_gemm_activation_range(cuda, oracle):
     # rows scaled far outside the fp16 range, and a zero row: the per-row power
     # of two keeps every row at the same relative accuracy
