@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # WRITE_SIZE counters of a `--traffic-probe` run, each calibrated on a plain
 # copy of known size; the figures and commands are in
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_607_181}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_643_284}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
 FFN_DIM = 16384
