@@ -181,17 +181,30 @@ __device__ __forceinline__ void process_block_q45(const std::uint8_t* tile, int 
             low[w] = static_cast<int>(lo);
             upper[w] = static_cast<int>(up);
         }
+        // Up to eight tokens both matrix instructions of the group go out before
+        // either result is read: the second runs while the first one's products
+        // are scaled.  Beyond that the second result costs more in registers
+        // than the overlap returns.
+        constexpr int kInFlight = S <= 4 ? 2 : 1;
 #pragma unroll
-        for (int part = 0; part < 2; ++part) {
-            const int sub = 2 * g + part;
-            const v16i dot = mfma32(act.operand(sub), part == 0 ? low : upper);
-            const int sc = byte_of(sub < 4 ? sc_lo : sc_hi, sub & 3);
-            const int mn = byte_of(sub < 4 ? mn_lo : mn_hi, sub & 3);
+        for (int first = 0; first < 2; first += kInFlight) {
+            v16i dots[kInFlight];
 #pragma unroll
-            for (int u = 0; u < S; ++u) {
-                acc_hi[u] += __mul24(sc, dot[2 * u]);
-                acc_lo[u] += __mul24(sc, dot[2 * u + 1]);
-                acc_min[u] += __mul24(mn, act.sums[u][sub]);
+            for (int part = 0; part < kInFlight; ++part) {
+                const int sub = 2 * g + first + part;
+                dots[part] = mfma32(act.operand(sub), (sub & 1) == 0 ? low : upper);
+            }
+#pragma unroll
+            for (int part = 0; part < kInFlight; ++part) {
+                const int sub = 2 * g + first + part;
+                const int sc = byte_of(sub < 4 ? sc_lo : sc_hi, sub & 3);
+                const int mn = byte_of(sub < 4 ? mn_lo : mn_hi, sub & 3);
+#pragma unroll
+                for (int u = 0; u < S; ++u) {
+                    acc_hi[u] += __mul24(sc, dots[part][2 * u]);
+                    acc_lo[u] += __mul24(sc, dots[part][2 * u + 1]);
+                    acc_min[u] += __mul24(mn, act.sums[u][sub]);
+                }
             }
         }
     }
@@ -223,8 +236,8 @@ __device__ __forceinline__ void process_block_q6(const std::uint8_t* tile, int j
         const v4i ql_a = *reinterpret_cast<const v4i*>(row + half * 64 + kc * 16);
         const v4i ql_b = *reinterpret_cast<const v4i*>(row + half * 64 + 32 + kc * 16);
         const v4i qh = *reinterpret_cast<const v4i*>(row + 128 + half * 32 + kc * 16);
-#pragma unroll
-        for (int quarter = 0; quarter < 4; ++quarter) {
+        // the codes of quarter `quarter` as signed bytes
+        auto unpack = [&](int quarter) {
             v4i q;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
@@ -234,20 +247,35 @@ __device__ __forceinline__ void process_block_q6(const std::uint8_t* tile, int j
                 // bits 2q, 2q+1 of the high byte move to bits 4, 5
                 const std::uint32_t top =
                     (quarter < 2 ? bits << (4 - 2 * quarter) : bits >> (2 * quarter - 4)) & 0x30303030u;
-                // q - 32 as signed bytes with no borrow between bytes:
-                // ((q | 0x80) - 0x20) ^ 0x80
+                // q - 32 with no borrow between bytes: ((q | 0x80) - 0x20) ^ 0x80
                 q[w] = static_cast<int>(((nib | top | 0x80808080u) - 0x20202020u) ^ 0x80808080u);
             }
-            const int sub = half * 4 + quarter;
-            const v16i dot = mfma32(act.operand(sub), q);
-            // a lane's k-half is one 16-value group: rows of the first group
-            // carry zeros in k-half 1 and the other way round
-            const int s0 = signed_byte_of(scales[sub >> 1], (2 * sub) & 3);
-            const int s1 = signed_byte_of(scales[sub >> 1], (2 * sub + 1) & 3);
+            return q;
+        };
+        // the matrix instructions go out two at a time: the second runs while
+        // the first one's products are scaled
+        // (up to four tokens; beyond that two results in flight cost more in
+        // registers than the overlap returns)
+        constexpr int kInFlight = S <= 2 ? 2 : 1;
 #pragma unroll
-            for (int u = 0; u < S; ++u) {
-                acc_hi[u] += __mul24(s0, dot[4 * u]) + __mul24(s1, dot[4 * u + 2]);
-                acc_lo[u] += __mul24(s0, dot[4 * u + 1]) + __mul24(s1, dot[4 * u + 3]);
+        for (int first = 0; first < 4; first += kInFlight) {
+            v16i dots[kInFlight];
+#pragma unroll
+            for (int part = 0; part < kInFlight; ++part) {
+                dots[part] = mfma32(act.operand(half * 4 + first + part), unpack(first + part));
+            }
+#pragma unroll
+            for (int part = 0; part < kInFlight; ++part) {
+                const int sub = half * 4 + first + part;
+                // a lane's k-half is one 16-value group: rows of the first group
+                // carry zeros in k-half 1 and the other way round
+                const int s0 = signed_byte_of(scales[sub >> 1], (2 * sub) & 3);
+                const int s1 = signed_byte_of(scales[sub >> 1], (2 * sub + 1) & 3);
+#pragma unroll
+                for (int u = 0; u < S; ++u) {
+                    acc_hi[u] += __mul24(s0, dots[part][4 * u]) + __mul24(s1, dots[part][4 * u + 2]);
+                    acc_lo[u] += __mul24(s0, dots[part][4 * u + 1]) + __mul24(s1, dots[part][4 * u + 3]);
+                }
             }
         }
     }
