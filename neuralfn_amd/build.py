@@ -1,4 +1,4 @@
-"""Build recipe for the HIP library and the host-side quantizer.
+"""Build recipe for the HIP library and the host-side library (quantizer, GGUF tensor table).
 
 `build_all()` compiles every source for gfx950 with hipcc and links
 `neuralfn_amd/lib/libnfn_mi355_tile_ops.so`; hipcc cross-compiles, so this runs
@@ -83,9 +83,9 @@ def build_tile_ops(jobs: int = 8) -> Path:
 
 def build_host() -> Path:
     LIB_DIR.mkdir(exist_ok=True)
-    source = CSRC / "host" / "kquant_quantize.cpp"
-    _run(["g++", "-std=c++17", "-O2", "-pthread", "-fPIC", "-shared", "-o", str(HOST_LIB),
-          str(source)])
+    sources = sorted((CSRC / "host").glob("*.cpp"))
+    _run(["g++", "-std=c++17", "-O2", "-pthread", "-fPIC", "-shared", "-Wall", "-o", str(HOST_LIB),
+          *map(str, sources)])
     return HOST_LIB
 
 
