@@ -21,9 +21,9 @@ namespace {
 
 constexpr std::int64_t kMaxSmallRows = 16;
 constexpr std::int64_t kMaxOperations = 4;
-// Private activation record of the small-batch path: per 32 values two int8
-// planes (high and low byte of a 16-bit fixed-point code), a float scale and
-// the float sum of the 32 inputs.
+// Private activation records of the small-batch path, 576 bytes per token and
+// 256 values (two int8 planes of a 16-bit fixed-point code, group sums, scale,
+// block maximum): 72 bytes per 32 values, the unit the workspace is sized in.
 constexpr std::int64_t kActivationGroupBytes = kActivationRecordBytes / 8;
 
 std::int64_t small_batch_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {

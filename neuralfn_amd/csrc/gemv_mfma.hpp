@@ -5,8 +5,8 @@
 
 namespace nfn {
 
-// Workspace record of one (token, 256-value block): high plane [256], low plane
-// [256], 8 float scales, 8 float sums.
+// Bytes of the workspace record of one (token, 256-value block); its layout is
+// in wave_rows.hpp (kActRecord).  The small-batch workspace query is sized from it.
 constexpr int kActivationRecordBytes = 576;
 
 // True when a projection of this encoding and width has a matrix-core kernel.
