@@ -231,7 +231,71 @@ int nfn_native_tile_k_quant_mmvq_linear_float32_v1(
  * 1 when centered).  A weight is null or a [1, width] F32/BF16 descriptor;
  * width <= 65536; eps finite and > 0 (tile_ops.h:836-858,
  * tile_ops.cu:4901-4950). */
+/* One normalisation, output = rms(input, weight, eps), and its fused forms:
+ * with a copy of the input kept as the residual, with that and the public
+ * Q8_1 form of the output (bit-identical to nfn_native_tile_quantize_q8_1 run
+ * on the output; width a multiple of 32), and with a residual added to the
+ * result (tile_ops.h:786-829, tile_ops.cu:4777-4899). */
+int nfn_native_tile_glimmer_rms_norm_affine_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* weight,
+    float* output,
+    int64_t rows,
+    int64_t width,
+    float eps,
+    bool centered,
+    void* cuda_stream);
+int nfn_native_tile_glimmer_rms_norm_affine_capture_residual_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* weight,
+    float* output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float eps,
+    bool centered,
+    void* cuda_stream);
+int nfn_native_tile_glimmer_rms_norm_affine_capture_residual_q8_1_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* weight,
+    float* output,
+    float* residual_output,
+    int8_t* q8_values,
+    float* q8_scales,
+    float* q8_sums,
+    int64_t rows,
+    int64_t width,
+    float eps,
+    bool centered,
+    void* cuda_stream);
+int nfn_native_tile_glimmer_rms_norm_affine_add_residual_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* weight,
+    const float* residual_input,
+    float* output,
+    int64_t rows,
+    int64_t width,
+    float eps,
+    bool centered,
+    void* cuda_stream);
 int nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    void* cuda_stream);
+/* The reference's multi-row specialization of the entry point above: same
+ * results, F32 norm weights only (tile_ops.h:859-873). */
+int nfn_native_tile_glimmer_dual_rms_add_capture_cooperative_batch_float32_v1(
     const float* input,
     const NfnNativeTilePackedWeightDescriptorV1* first_weight,
     const float* residual_input,

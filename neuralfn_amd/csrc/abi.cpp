@@ -353,6 +353,61 @@ int nfn_native_tile_swiglu_float32(const float* gate, const float* up, float* ou
     return launch_status();
 }
 
+// The four single-normalisation entry points
+// (neuralfn/csrc/native_train/tile_ops.cu:4777-4899) share one body.
+static int run_rms_norm(const float* input, const Descriptor* weight, const float* residual_input,
+                        bool wants_residual_input, float* output, float* residual_output,
+                        bool wants_residual_output, std::int8_t* q8_values, float* q8_scales,
+                        float* q8_sums, bool wants_q8, std::int64_t rows, std::int64_t width,
+                        float eps, bool centered, void* cuda_stream) {
+    Descriptor normalized{};
+    if (input == nullptr || output == nullptr || rows <= 0 || width <= 0 || width > 65536 ||
+        !std::isfinite(eps) || !(eps > 0.0f) ||
+        (wants_residual_input && residual_input == nullptr) ||
+        (wants_residual_output && residual_output == nullptr) ||
+        (wants_q8 && (q8_values == nullptr || q8_scales == nullptr || q8_sums == nullptr ||
+                      width % 32 != 0)) ||
+        (weight != nullptr && (!normalize_descriptor(weight, &normalized) ||
+                               normalized.output_dim != 1 || normalized.input_dim != width))) {
+        return kInvalid;
+    }
+    launch_rms_norm(input, weight != nullptr ? &normalized : nullptr, centered,
+                    wants_residual_input ? residual_input : nullptr, output,
+                    wants_residual_output ? residual_output : nullptr,
+                    wants_q8 ? q8_values : nullptr, q8_scales, q8_sums, rows, width, eps,
+                    as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_rms_norm_affine_float32_v1(
+    const float* input, const Descriptor* weight, float* output, std::int64_t rows,
+    std::int64_t width, float eps, bool centered, void* cuda_stream) {
+    return run_rms_norm(input, weight, nullptr, false, output, nullptr, false, nullptr, nullptr,
+                        nullptr, false, rows, width, eps, centered, cuda_stream);
+}
+
+int nfn_native_tile_glimmer_rms_norm_affine_capture_residual_float32_v1(
+    const float* input, const Descriptor* weight, float* output, float* residual_output,
+    std::int64_t rows, std::int64_t width, float eps, bool centered, void* cuda_stream) {
+    return run_rms_norm(input, weight, nullptr, false, output, residual_output, true, nullptr,
+                        nullptr, nullptr, false, rows, width, eps, centered, cuda_stream);
+}
+
+int nfn_native_tile_glimmer_rms_norm_affine_capture_residual_q8_1_float32_v1(
+    const float* input, const Descriptor* weight, float* output, float* residual_output,
+    std::int8_t* q8_values, float* q8_scales, float* q8_sums, std::int64_t rows,
+    std::int64_t width, float eps, bool centered, void* cuda_stream) {
+    return run_rms_norm(input, weight, nullptr, false, output, residual_output, true, q8_values,
+                        q8_scales, q8_sums, true, rows, width, eps, centered, cuda_stream);
+}
+
+int nfn_native_tile_glimmer_rms_norm_affine_add_residual_float32_v1(
+    const float* input, const Descriptor* weight, const float* residual_input, float* output,
+    std::int64_t rows, std::int64_t width, float eps, bool centered, void* cuda_stream) {
+    return run_rms_norm(input, weight, residual_input, true, output, nullptr, false, nullptr,
+                        nullptr, nullptr, false, rows, width, eps, centered, cuda_stream);
+}
+
 // Shared argument checks of the two dual-RMS entry points
 // (neuralfn/csrc/native_train/tile_ops.cu:4901-5010): a norm weight is absent
 // or a valid [1, width] descriptor.
@@ -391,6 +446,24 @@ int nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
                                 normalized_output, residual_output, rows, width, first_eps,
                                 second_eps, nullptr, as_stream(cuda_stream));
     return launch_status();
+}
+
+int nfn_native_tile_glimmer_dual_rms_add_capture_cooperative_batch_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t rows, std::int64_t width, float first_eps,
+    bool first_centered, float second_eps, bool second_centered, void* cuda_stream) {
+    // The reference's multi-row specialization takes F32 norm weights only
+    // (tile_ops.h:859-862); the arithmetic is the ordinary entry point's, which
+    // here already runs one workgroup per row with all loads in flight at once.
+    if ((first_weight != nullptr && first_weight->encoding != kEncF32) ||
+        (second_weight != nullptr && second_weight->encoding != kEncF32)) {
+        return kInvalid;
+    }
+    return nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
+        input, first_weight, residual_input, hidden_output, second_weight, normalized_output,
+        residual_output, rows, width, first_eps, first_centered, second_eps, second_centered,
+        cuda_stream);
 }
 
 int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(

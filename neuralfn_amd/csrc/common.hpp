@@ -187,6 +187,33 @@ __device__ __forceinline__ float weight_value(std::uint32_t encoding,
                      static_cast<float>(quant));
 }
 
+// One value of a 32-value Q8_1 block held by 32 consecutive lanes
+// (neuralfn/csrc/tile_cuda/kernels.cu:1527-1562): code = round(x * 127 / max)
+// clamped to +-127, scale = 1 / (127 / max), sum = the block's float sum
+// (butterfly order).  Scale and sum are the same in all 32 lanes.
+struct Q8_1Value {
+    std::int8_t code;
+    float scale, sum;
+};
+
+__device__ __forceinline__ Q8_1Value quantize_q8_1_value(float value) {
+    float maximum = fabsf(value);
+    float sum = value;
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) {
+        maximum = fmaxf(maximum, __shfl_xor(maximum, offset, 32));
+        sum += __shfl_xor(sum, offset, 32);
+    }
+    const float inverse = maximum > 0.0f ? 127.0f / maximum : 0.0f;
+    Q8_1Value result;
+    result.scale = inverse > 0.0f ? 1.0f / inverse : 0.0f;
+    int code = inverse > 0.0f ? static_cast<int>(roundf(value * inverse)) : 0;
+    code = max(-127, min(127, code));
+    result.code = static_cast<std::int8_t>(code);
+    result.sum = sum;
+    return result;
+}
+
 __device__ __forceinline__ float wave_sum(float value) {
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {

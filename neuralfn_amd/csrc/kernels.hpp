@@ -40,4 +40,12 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
                                  float first_eps, float second_eps, std::uint8_t* records,
                                  hipStream_t stream);
 
+// One normalisation: output = rms(input, weight, eps) (+ residual_input when
+// given); residual_output (may be null) receives a copy of the input; the
+// q8 pointers (all or none) receive the public Q8_1 form of the output.
+void launch_rms_norm(const float* input, const Descriptor* weight, bool centered,
+                     const float* residual_input, float* output, float* residual_output,
+                     std::int8_t* q8_codes, float* q8_scales, float* q8_sums, std::int64_t rows,
+                     std::int64_t width, float eps, hipStream_t stream);
+
 }  // namespace nfn

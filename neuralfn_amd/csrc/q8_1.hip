@@ -23,22 +23,11 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(
     const std::int64_t index = static_cast<std::int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const std::int64_t block = index >> 5;
     if (block >= block_count) return;
-    const float value = input[index];
-    float maximum = fabsf(value);
-    float sum = value;
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) {
-        maximum = fmaxf(maximum, __shfl_xor(maximum, offset, 32));
-        sum += __shfl_xor(sum, offset, 32);
-    }
-    const float inverse = maximum > 0.0f ? 127.0f / maximum : 0.0f;
-    const float scale = inverse > 0.0f ? 1.0f / inverse : 0.0f;
-    int code = inverse > 0.0f ? static_cast<int>(roundf(value * inverse)) : 0;
-    code = max(-127, min(127, code));
-    codes[index] = static_cast<std::int8_t>(code);
+    const Q8_1Value quantized = quantize_q8_1_value(input[index]);
+    codes[index] = quantized.code;
     if ((threadIdx.x & 31) == 0) {
-        scales[block] = scale;
-        sums[block] = sum;
+        scales[block] = quantized.scale;
+        sums[block] = quantized.sum;
     }
 }
 

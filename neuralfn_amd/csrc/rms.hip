@@ -242,6 +242,98 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
     }
 }
 
+// ---- one normalisation: output = rms(input, weight, eps) [+ residual_input],
+// optionally a copy of the input (the residual the caller keeps) and the
+// public Q8_1 form of the output
+// (neuralfn/csrc/tile_cuda/kernels.cu:2065-2153).  Same reduction order as
+// above; the Q8_1 values are those of the standalone quantizer run on the
+// output, computed in registers: 32 consecutive threads hold 32 consecutive
+// columns, one Q8_1 block.
+
+struct Q8_1Outputs {
+    std::int8_t* codes;
+    float* scales;
+    float* sums;
+};
+
+__device__ __forceinline__ void store_q8_1(const Q8_1Outputs& q8, std::int64_t index, float value,
+                                           bool inside) {
+    // all 32 lanes of a block are inside or outside together (width % 32 == 0)
+    const Q8_1Value quantized = quantize_q8_1_value(inside ? value : 0.0f);
+    if (inside) {
+        q8.codes[index] = quantized.code;
+        if ((threadIdx.x & 31) == 0) {
+            q8.scales[index >> 5] = quantized.scale;
+            q8.sums[index >> 5] = quantized.sum;
+        }
+    }
+}
+
+template <bool ADD, bool Q8>
+__global__ __launch_bounds__(kRmsThreads) void rms_resident_kernel(
+    const float* __restrict__ input, NormWeight weight, const float* __restrict__ residual_input,
+    float* __restrict__ output, float* __restrict__ residual_output, int width, float eps,
+    Q8_1Outputs q8) {
+    __shared__ float partials[kRmsThreads];
+    const std::int64_t row = blockIdx.x;
+    const float* source = input + row * width;
+    float value[kOwned], other[kOwned], scale[kOwned];
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) {
+        const int column = threadIdx.x + i * kRmsThreads;
+        const int clamped = min(column, width - 1);
+        value[i] = column < width ? source[clamped] : 0.0f;
+        other[i] = ADD ? residual_input[row * width + clamped] : 0.0f;
+        scale[i] = norm_scale(weight, clamped);
+    }
+    float square_sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) square_sum = fmaf(value[i], value[i], square_sum);
+    const float inverse =
+        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + eps);
+#pragma unroll
+    for (int i = 0; i < kOwned; ++i) {
+        const int column = threadIdx.x + i * kRmsThreads;
+        const bool inside = column < width;
+        const std::int64_t index = row * width + column;
+        float result = __fmul_rn(__fmul_rn(value[i], inverse), scale[i]);
+        if constexpr (ADD) result = __fadd_rn(result, other[i]);
+        if (inside) {
+            output[index] = result;
+            if (residual_output != nullptr) residual_output[index] = value[i];
+        }
+        if constexpr (Q8) {
+            if (i * kRmsThreads < width) store_q8_1(q8, index, result, inside);
+        }
+    }
+}
+
+template <bool ADD, bool Q8>
+__global__ __launch_bounds__(kRmsThreads) void rms_wide_kernel(
+    const float* __restrict__ input, NormWeight weight, const float* __restrict__ residual_input,
+    float* __restrict__ output, float* __restrict__ residual_output, std::int64_t width, float eps,
+    Q8_1Outputs q8) {
+    __shared__ float partials[kRmsThreads];
+    const std::int64_t row = blockIdx.x;
+    const float* source = input + row * width;
+    const float inverse = inverse_rms(source, width, eps, partials);
+    // the loop runs the same number of times in every thread of a 32-lane block
+    for (std::int64_t base = threadIdx.x & ~31; base < width; base += kRmsThreads) {
+        const std::int64_t column = base + (threadIdx.x & 31);
+        const bool inside = column < width;  // true for the whole block: width % 32 == 0 with Q8
+        const std::int64_t clamped = inside ? column : width - 1;
+        const std::int64_t index = row * width + column;
+        const float loaded = source[clamped];
+        float result = __fmul_rn(__fmul_rn(loaded, inverse), norm_scale(weight, clamped));
+        if constexpr (ADD) result = __fadd_rn(result, residual_input[row * width + clamped]);
+        if (inside) {
+            output[index] = result;
+            if (residual_output != nullptr) residual_output[index] = loaded;
+        }
+        if constexpr (Q8) store_q8_1(q8, index, result, inside);
+    }
+}
+
 NormWeight norm_weight(const Descriptor* descriptor, bool centered) {
     NormWeight weight{};
     if (descriptor != nullptr) {
@@ -288,6 +380,46 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
         hipLaunchKernelGGL((dual_rms_add_capture_kernel<false>), grid, dim3(kRmsThreads), 0, stream,
                            input, first, residual_input, hidden_output, second, normalized_output,
                            residual_output, width, first_eps, second_eps, records);
+    }
+}
+
+template <bool ADD, bool Q8>
+static void launch_rms_variant(const float* input, const NormWeight& weight,
+                               const float* residual_input, float* output, float* residual_output,
+                               std::int64_t rows, std::int64_t width, float eps,
+                               const Q8_1Outputs& q8, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>(rows));
+    if (width <= kOwned * kRmsThreads) {
+        hipLaunchKernelGGL((rms_resident_kernel<ADD, Q8>), grid, dim3(kRmsThreads), 0, stream, input,
+                           weight, residual_input, output, residual_output,
+                           static_cast<int>(width), eps, q8);
+    } else {
+        hipLaunchKernelGGL((rms_wide_kernel<ADD, Q8>), grid, dim3(kRmsThreads), 0, stream, input,
+                           weight, residual_input, output, residual_output, width, eps, q8);
+    }
+}
+
+void launch_rms_norm(const float* input, const Descriptor* weight, bool centered,
+                     const float* residual_input, float* output, float* residual_output,
+                     std::int8_t* q8_codes, float* q8_scales, float* q8_sums, std::int64_t rows,
+                     std::int64_t width, float eps, hipStream_t stream) {
+    const NormWeight scale = norm_weight(weight, centered);
+    const Q8_1Outputs q8{q8_codes, q8_scales, q8_sums};
+    const bool add = residual_input != nullptr;
+    if (q8_codes != nullptr) {
+        if (add) {
+            launch_rms_variant<true, true>(input, scale, residual_input, output, residual_output,
+                                           rows, width, eps, q8, stream);
+        } else {
+            launch_rms_variant<false, true>(input, scale, residual_input, output, residual_output,
+                                            rows, width, eps, q8, stream);
+        }
+    } else if (add) {
+        launch_rms_variant<true, false>(input, scale, residual_input, output, residual_output, rows,
+                                        width, eps, q8, stream);
+    } else {
+        launch_rms_variant<false, false>(input, scale, residual_input, output, residual_output, rows,
+                                         width, eps, q8, stream);
     }
 }
 

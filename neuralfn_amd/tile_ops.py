@@ -83,6 +83,17 @@ SIGNATURES = {
         ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_linear_float32_v1": (
         ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P]),
+    "nfn_native_tile_glimmer_rms_norm_affine_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_rms_norm_affine_capture_residual_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_rms_norm_affine_capture_residual_q8_1_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _P, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_rms_norm_affine_add_residual_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_dual_rms_add_capture_cooperative_batch_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _P]),
     "nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1": (
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P]),
@@ -265,6 +276,42 @@ def multi_linear_prequantized(weights: Sequence[PackedWeight], rows: int, worksp
         _descriptor_array(descriptors), _pointer_array(outputs), len(weights), rows,
         workspace.data_ptr(), workspace.numel(), stream), "mmvq_multi_linear_prequantized")
     return outputs
+
+
+def rms_norm(x, weight: Optional[PackedWeight] = None, centered: bool = False, eps: float = 1e-6,
+             residual=None, capture: bool = False, q8: bool = False):
+    """rms(x, weight, eps) (+ residual).  Returns a dict: "output", and per request "captured"
+    (a copy of x), "codes"/"scales"/"sums" (the public Q8_1 form of the output)."""
+    import torch
+    rows, width = x.shape
+    stream = _stream_handle()
+    descriptor = weight.descriptor(stream) if weight is not None else None
+    pointer = ctypes.byref(descriptor) if descriptor is not None else None
+    result = {"output": torch.empty_like(x)}
+    lib = load()
+    if residual is not None:
+        check(lib.nfn_native_tile_glimmer_rms_norm_affine_add_residual_float32_v1(
+            x.data_ptr(), pointer, residual.data_ptr(), result["output"].data_ptr(), rows, width,
+            eps, centered, stream), "rms_norm_affine_add_residual")
+    elif q8:
+        result["captured"] = torch.empty_like(x)
+        result["codes"] = torch.empty((rows, width), dtype=torch.int8, device=x.device)
+        result["scales"] = torch.empty((rows, width // 32), dtype=torch.float32, device=x.device)
+        result["sums"] = torch.empty_like(result["scales"])
+        check(lib.nfn_native_tile_glimmer_rms_norm_affine_capture_residual_q8_1_float32_v1(
+            x.data_ptr(), pointer, result["output"].data_ptr(), result["captured"].data_ptr(),
+            result["codes"].data_ptr(), result["scales"].data_ptr(), result["sums"].data_ptr(),
+            rows, width, eps, centered, stream), "rms_norm_affine_capture_residual_q8_1")
+    elif capture:
+        result["captured"] = torch.empty_like(x)
+        check(lib.nfn_native_tile_glimmer_rms_norm_affine_capture_residual_float32_v1(
+            x.data_ptr(), pointer, result["output"].data_ptr(), result["captured"].data_ptr(),
+            rows, width, eps, centered, stream), "rms_norm_affine_capture_residual")
+    else:
+        check(lib.nfn_native_tile_glimmer_rms_norm_affine_float32_v1(
+            x.data_ptr(), pointer, result["output"].data_ptr(), rows, width, eps, centered,
+            stream), "rms_norm_affine")
+    return result
 
 
 def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = None,

@@ -41,7 +41,7 @@
 //                       as tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1009-1023.
 //   nfo_rms_norm        equals the compiled reference rms_norm() bit for bit where
 //                       that builds; closed form x / sqrt(mean(x^2) + eps) in numpy.
-//   nfo_dual_rms_add_capture  within the reference probe's 2e-5 of the double
+//   nfo_rms_norm_strict, nfo_dual_rms_add_capture  within the reference probe's 2e-5 of the double
 //                       form (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:243-256)
 //                       composed from nfo_rms_norm; its summation order (256
 //                       strided partial sums, halving tree) against an
@@ -536,6 +536,29 @@ static float nfo_strict_inverse_rms(const float* values, std::int64_t width, flo
     }
     const float mean = partials[0] / static_cast<float>(width);
     return 1.0f / std::sqrt(mean + eps);
+}
+
+// One normalisation in the same strict order
+// (neuralfn/csrc/tile_cuda/kernels.cu:2065-2120): output = (x * inverse_rms) *
+// scale, plus the residual with one rounded add when given.
+void nfo_rms_norm_strict(const float* input, const float* weight, int centered,
+                         const float* residual_input, float* output, std::int64_t rows,
+                         std::int64_t width, float eps) {
+    for (std::int64_t row = 0; row < rows; ++row) {
+        const float* source = input + row * width;
+        const float inverse = nfo_strict_inverse_rms(source, width, eps);
+        for (std::int64_t column = 0; column < width; ++column) {
+            float scale = 1.0f;
+            if (weight != nullptr) {
+                scale = weight[column];
+                if (centered) scale += 1.0f;
+            }
+            const float scaled = source[column] * inverse;
+            float value = scaled * scale;
+            if (residual_input != nullptr) value = value + residual_input[row * width + column];
+            output[row * width + column] = value;
+        }
+    }
 }
 
 void nfo_dual_rms_add_capture(const float* input, const float* first_weight, int first_centered,

@@ -66,6 +66,8 @@ def lib() -> ctypes.CDLL:
         o.nfo_swiglu.restype = None
         o.nfo_rms_norm.argtypes = [_P, _P, ctypes.c_int, _I64, ctypes.c_double, _P]
         o.nfo_rms_norm.restype = None
+        o.nfo_rms_norm_strict.argtypes = [_P, _P, ctypes.c_int, _P, _P, _I64, _I64, ctypes.c_float]
+        o.nfo_rms_norm_strict.restype = None
         o.nfo_dual_rms_add_capture.argtypes = [_P, _P, ctypes.c_int, _P, _P, _P, ctypes.c_int, _P,
                                                _I64, _I64, ctypes.c_float, ctypes.c_float]
         o.nfo_dual_rms_add_capture.restype = None
@@ -220,6 +222,19 @@ def rms_norm(x: np.ndarray, weight=None, centered: bool = False, epsilon: float 
     _keep, pointer = _optional(weight)
     out = np.empty_like(x)
     lib().nfo_rms_norm(x.ctypes.data, pointer, int(centered), x.size, float(epsilon), out.ctypes.data)
+    return out
+
+
+def rms_norm_strict(x: np.ndarray, weight=None, centered: bool = False, eps: float = 1e-6,
+                    residual=None) -> np.ndarray:
+    """rms(x, weight, eps) (+ residual) in the strict float order of the device kernel."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, width = x.shape
+    _weight, weight_pointer = _optional(weight)
+    _residual, residual_pointer = _optional(residual)
+    out = np.empty_like(x)
+    lib().nfo_rms_norm_strict(x.ctypes.data, weight_pointer, int(centered), residual_pointer,
+                              out.ctypes.data, rows, width, eps)
     return out
 
 

@@ -536,6 +536,65 @@ def test_dual_rms_add_capture_against_oracle(cuda, oracle, weights):
         assert np.max(np.abs(normalized.cpu().numpy()[row] - reference_normalized)) <= 2e-5
 
 
+@pytest.mark.parametrize("width", [6656, 12288 + 32])
+@pytest.mark.parametrize("weights", ["none", "f32_centered", "bf16"])
+def test_rms_norm_family_against_oracle(cuda, oracle, weights, width):
+    # the single normalisation and its fused forms (probe :243-330): plain, with the
+    # input kept as the residual, with the Q8_1 form of the output, with a residual added
+    rows = 3
+    rng = np.random.default_rng(35)
+    x = probe_rms_input(rows, width) if width == 6656 else \
+        rng.standard_normal((rows, width)).astype(np.float32)
+    residual = rng.standard_normal((rows, width)).astype(np.float32)
+    values = weight = None
+    centered = weights == "f32_centered"
+    if weights != "none":
+        encoding = kquant.F32 if centered else kquant.BF16
+        values, weight = norm_weight(rng.standard_normal(width) * 0.3, encoding, cuda)
+    device_x = to_device(x, cuda)
+    expected = oracle.rms_norm_strict(x, values, centered, 1e-6)
+    plain = tile_ops.rms_norm(device_x, weight, centered, 1e-6)
+    assert_bits_equal(plain["output"], expected, "plain")
+    for row in range(rows):  # the CPU engine's double form at the probe's tolerance
+        assert np.max(np.abs(expected[row] - oracle.rms_norm(x[row], values, centered, 1e-6))) <= 2e-5
+    captured = tile_ops.rms_norm(device_x, weight, centered, 1e-6, capture=True)
+    assert_bits_equal(captured["output"], expected, "capture output")
+    assert_bits_equal(captured["captured"], x, "captured residual")
+    added = tile_ops.rms_norm(device_x, weight, centered, 1e-6, residual=to_device(residual, cuda))
+    assert_bits_equal(added["output"], oracle.rms_norm_strict(x, values, centered, 1e-6, residual),
+                      "add residual")
+    fused = tile_ops.rms_norm(device_x, weight, centered, 1e-6, q8=True)
+    assert_bits_equal(fused["output"], expected, "q8 output")
+    assert_bits_equal(fused["captured"], x, "q8 captured residual")
+    codes, scales, sums = tile_ops.quantize_q8_1(plain["output"])
+    assert torch_().equal(fused["codes"], codes)
+    assert_bits_equal(fused["scales"], scales.reshape(rows, -1), "q8 scales")
+    assert_bits_equal(fused["sums"], sums.reshape(rows, -1), "q8 sums")
+
+
+def test_cooperative_dual_rms_equals_the_ordinary_entry_point(cuda):
+    rows, width = 4, 6656
+    x = to_device(probe_rms_input(rows, width), cuda)
+    residual = to_device(np.random.default_rng(36).standard_normal((rows, width)).astype(np.float32),
+                         cuda)
+    _, first = norm_weight(np.random.default_rng(37).standard_normal(width), kquant.F32, cuda)
+    _, half = norm_weight(np.random.default_rng(38).standard_normal(width), kquant.BF16, cuda)
+    ordinary = tile_ops.dual_rms_add_capture(x, residual, first, True, None, False, 1e-8, 1e-5)
+    outputs = [torch_().empty_like(x) for _ in range(3)]
+    stream = tile_ops._stream_handle()
+    cooperative = tile_ops.load().nfn_native_tile_glimmer_dual_rms_add_capture_cooperative_batch_float32_v1
+    descriptor = first.descriptor(stream)
+    assert cooperative(x.data_ptr(), ctypes.byref(descriptor), residual.data_ptr(),
+                       outputs[0].data_ptr(), None, outputs[1].data_ptr(), outputs[2].data_ptr(),
+                       rows, width, 1e-8, True, 1e-5, False, stream) == 0
+    for a, b in zip(ordinary, outputs):
+        assert_bits_equal(a, b)
+    bf16 = half.descriptor(stream)
+    assert cooperative(x.data_ptr(), ctypes.byref(bf16), residual.data_ptr(), outputs[0].data_ptr(),
+                       None, outputs[1].data_ptr(), outputs[2].data_ptr(), rows, width, 1e-8, True,
+                       1e-5, False, stream) == 1  # F32 norm weights only
+
+
 def test_dual_rms_add_capture_wide_rows(cuda, oracle):
     # wider than the register-resident kernel takes: the kernel that walks memory in batches
     rows, width = 2, 12288 + 32
