@@ -38,6 +38,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_643_284}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
+CU_COUNT = 256
+F16_FLOP_PER_CYCLE_PER_CU = 4096   # 4 SIMDs x one 32x32x16 fp16 matrix instruction per 32 cycles
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
 FFN_DIM = 16384
 VOCAB = 202048
@@ -157,6 +159,30 @@ def time_replays(run, steps: int, warmup: int) -> float:
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / steps
+
+
+def step_distribution(run, steps: int, warmup: int, per_step: int) -> dict:
+    """Median and 5th / 95th percentile of run()'s duration, one event pair per call.
+
+    Reported in microseconds per launch (`per_step` launches per call).
+    """
+    import torch
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+             for _ in range(steps)]
+    for start, stop in pairs:
+        start.record()
+        run()
+        stop.record()
+    torch.cuda.synchronize()
+    times = sorted(start.elapsed_time(stop) * 1e3 / per_step for start, stop in pairs)
+
+    def at(fraction: float) -> float:
+        return round(times[min(len(times) - 1, int(fraction * len(times)))], 3)
+
+    return {"median": at(0.5), "p05": at(0.05), "p95": at(0.95), "samples": len(times)}
 
 
 def time_graph(run, stream, steps: int, warmup: int) -> float:
@@ -302,6 +328,36 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
                     "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
                     "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS[name], 4),
                     "tokens/s": round(rows / ms * 1e3, 1)}
+    # The shader clock while the largest shape runs, and the matrix-core peak at
+    # that clock: 256 CUs x 4096 fp16 flop per cycle per CU.
+    rows = 2048
+    x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
+    out = torch.empty((rows, FFN_DIM), dtype=torch.float32, device=device)
+    nbytes = tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+        rows, MODEL_DIM, FFN_DIM, tile_ops.GEMM_F16)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    probe = tile_ops.ShaderClockProbe(device)
+    for _ in range(10):  # the clock settles under load before the probe's window
+        tile_ops.gemm(gate, x, tile_ops.GEMM_F16, workspace, out)
+    probe.start(5000)
+    for _ in range(16):
+        tile_ops.gemm(gate, x, tile_ops.GEMM_F16, workspace, out)
+    stream.synchronize()
+    megahertz = probe.megahertz()
+    peak_at_clock = megahertz * 1e6 * CU_COUNT * F16_FLOP_PER_CYCLE_PER_CU / 1e12
+    result["shader_clock_under_gemm_MHz"] = round(megahertz, 1)
+    result["f16_peak_at_that_clock_TFLOP/s"] = round(peak_at_clock, 1)
+    result["f16_peak_published_TFLOP/s"] = MFMA_PEAK_TFLOPS["f16"]
+    # The same shape as a plain fp16 GEMM through the vendor library (no packed
+    # weights, no dequantization): what the matrix cores sustain on this box
+    # with operands of the same statistics.
+    a16 = x.to(torch.float16)
+    w16 = (torch.randn(FFN_DIM, MODEL_DIM, device=device) * 0.02).to(torch.float16)
+    ms = time_replays(lambda: torch.matmul(a16, w16.t()), max(5, steps // 2), max(2, warmup // 2))
+    library = 2.0 * rows * MODEL_DIM * FFN_DIM / ms / 1e9
+    result["library_f16_gemm_same_shape_M2048"] = {
+        "ms": round(ms, 4), "TFLOP/s": round(library, 1),
+        "frac_mfma": round(library / MFMA_PEAK_TFLOPS["f16"], 4)}
     return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}, dequant-GEMM "
                         "incl. activation conversion", **result}
 
@@ -431,6 +487,12 @@ def main() -> int:
                 step.enqueue(int(stream.cuda_stream))
 
         ms_per_step = time_replays(run, args.steps, args.warmup)
+        samples = max(30, args.steps)
+        per_launch = {"unit": "us per launch"}
+        if graph is not None:
+            per_launch["graph_replay"] = step_distribution(run, samples, 5, step.launches_per_step)
+        per_launch["eager"] = step_distribution(
+            lambda: step.enqueue(int(stream.cuda_stream)), samples, 5, step.launches_per_step)
 
     bytes_per_step = args.layers * layer_algorithmic_bytes(args.rows)
     value = bytes_per_step / ms_per_step / 1e6  # GB/s
@@ -471,6 +533,7 @@ def main() -> int:
             "us_per_launch": round(ms_per_step * 1e3 / launches, 3),
         },
     }
+    record["per_launch_distribution"] = per_launch
     if not args.no_extras:
         try:
             with torch.cuda.stream(stream):

@@ -400,6 +400,19 @@ int nfn_mi355_k_quant_gemm_float32_v1(
     int mode,
     void* cuda_stream);
 
+/* Shader clock under load, a measurement aid (no counterpart in the reference;
+ * for benchmarks that price a kernel against the matrix-core peak at the clock
+ * the chip really ran at).  Enqueues one wave that waits about `microseconds`
+ * (1..100000) on `cuda_stream` and then writes three uint64 to
+ * `cycles_and_ticks` (device memory, 24 bytes): shader cycles, ticks of the
+ * constant device clock, and that clock's ticks per second
+ * (hipDeviceAttributeWallClockRate).  Launch it on a side stream while the work
+ * under test runs on another. */
+int nfn_mi355_shader_clock_probe_v1(
+    uint64_t* cycles_and_ticks,
+    int64_t microseconds,
+    void* cuda_stream);
+
 #ifdef __cplusplus
 }
 #endif

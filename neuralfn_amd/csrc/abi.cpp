@@ -573,4 +573,21 @@ int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float*
     return launch_status();
 }
 
+int nfn_mi355_shader_clock_probe_v1(std::uint64_t* cycles_and_ticks, std::int64_t microseconds,
+                                    void* cuda_stream) {
+    if (cycles_and_ticks == nullptr || microseconds < 1 || microseconds > 100000) return kInvalid;
+    int ticks_per_millisecond = 0;  // the attribute is in kHz
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&ticks_per_millisecond, hipDeviceAttributeWallClockRate, device) !=
+            hipSuccess ||
+        ticks_per_millisecond <= 0) {
+        return static_cast<int>(hipErrorNotSupported);
+    }
+    launch_clock_probe(cycles_and_ticks, microseconds * ticks_per_millisecond / 1000,
+                       static_cast<std::uint64_t>(ticks_per_millisecond) * 1000,
+                       as_stream(cuda_stream));
+    return launch_status();
+}
+
 }  // extern "C"

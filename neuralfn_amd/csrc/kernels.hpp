@@ -48,4 +48,9 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
                      std::int8_t* q8_codes, float* q8_scales, float* q8_sums, std::int64_t rows,
                      std::int64_t width, float eps, hipStream_t stream);
 
+// clock_probe.hip — out[0] = shader cycles, out[1] = ticks of the constant
+// clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.
+void launch_clock_probe(std::uint64_t* out, std::int64_t ticks, std::uint64_t ticks_per_second,
+                        hipStream_t stream);
+
 }  // namespace nfn

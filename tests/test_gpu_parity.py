@@ -847,3 +847,20 @@ def test_decode_gemv_is_deterministic(cuda):
     first = tile_ops.mmvq_linear(weight, x, workspace).cpu().numpy()
     for _ in range(20):
         assert_bits_equal(tile_ops.mmvq_linear(weight, x, workspace), first)
+
+
+@pytest.mark.gpu
+def test_shader_clock_probe_reports_a_plausible_clock():
+    """nfn_mi355_shader_clock_probe_v1: cycles per tick of the constant clock, and its argument checks."""
+    import torch
+    device = torch.device("cuda:0")
+    probe = tile_ops.ShaderClockProbe(device)
+    probe.start(200)
+    megahertz = probe.megahertz()
+    assert 100.0 < megahertz < 4000.0
+    cycles, ticks, per_second = (int(v) for v in probe.result.tolist())
+    assert per_second > 0 and ticks >= 200 * per_second // 1_000_000
+    lib = tile_ops.load()
+    assert lib.nfn_mi355_shader_clock_probe_v1(None, 100, None) == 1
+    assert lib.nfn_mi355_shader_clock_probe_v1(probe.result.data_ptr(), 0, None) == 1
+    assert lib.nfn_mi355_shader_clock_probe_v1(probe.result.data_ptr(), 100001, None) == 1
