@@ -358,6 +358,188 @@ int nfn_native_tile_swiglu_float32(
     int64_t n,
     void* cuda_stream);
 
+/* ==== the decode loop's remaining operators ===============================
+ * The operators the reference's resident engine requires from the sidecar
+ * besides the packed linears (resident_glimmer_cuda.cpp:431-495): token
+ * embedding, rotary position embedding, one-token and block attention over a
+ * bf16 cache, the cache commit, the logit transform, add and scale.
+ * Arithmetic: the CPU engine's (resident_glimmer.cpp:773-800, 1716-1800,
+ * 1895-1903), computed in float except where a comment says double. */
+
+enum {
+    NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 = 1,      /* tile_ops.h:34 */
+    NFN_NATIVE_TILE_GLIMMER_ROPE_HALF_SPLIT = 0,   /* tile_ops.h:35 */
+    NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED = 1,  /* tile_ops.h:36 */
+    NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL = 1     /* tile_ops.h:37 */
+};
+
+/* Row `token_id` of a packed [vocabulary, width] matrix, dequantized to
+ * output[width] (tile_ops.h:770-785; bit-exact with ...dequantize_float32_v1).
+ * The stream is descriptor->cuda_stream.  The first form checks the token on
+ * the host; the device forms write zeros for a token outside the vocabulary. */
+int nfn_native_tile_glimmer_embedding_gather_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    int64_t token_id,
+    float* output);
+int nfn_native_tile_glimmer_embedding_gather_device_i64_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const int64_t* token_id, /* device */
+    float* output);
+int nfn_native_tile_glimmer_embedding_batch_i32_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const int32_t* token_ids, /* device, [rows] */
+    float* output,            /* [rows, width] */
+    int64_t rows);
+
+/* Rotary position embedding in place (tile_ops.h:895-904, 1016-1027):
+ * query [rows, query_heads, head_dim], key [rows, kv_heads, head_dim]; row r
+ * is at position start_position + r; pair i of a head is elements (i,
+ * i + head_dim/2) for HALF_SPLIT and (2i, 2i+1) for INTERLEAVED; angle =
+ * position / theta^(2i/head_dim), computed in double as the CPU engine does
+ * (resident_glimmer.cpp:773-800); `inverse` rotates by the negative angle.
+ * head_dim even, at most 256. */
+int nfn_native_tile_glimmer_positioned_rope_float32_v1(
+    float* query,
+    float* key,
+    int64_t query_heads,
+    int64_t kv_heads,
+    int64_t head_dim,
+    int64_t position,
+    float theta,
+    uint32_t layout,
+    void* cuda_stream);
+int nfn_native_tile_glimmer_positioned_rope_batch_float32_v1(
+    float* query,
+    float* key,
+    int64_t rows,
+    int64_t query_heads,
+    int64_t kv_heads,
+    int64_t head_dim,
+    int64_t start_position,
+    float theta,
+    uint32_t layout,
+    bool inverse,
+    void* cuda_stream);
+
+/* One-token causal attention of query_heads heads over kv_heads cached heads
+ * (tile_ops.h:308-339, 944-945).  Keys first_key_position .. position-1 are
+ * rows (p % cache_capacity) of the bf16 caches, key `position` is
+ * current_key/current_value in float and not yet in the cache.  Query head h
+ * uses cached head h*kv_heads/query_heads.  output[query_heads, head_dim] =
+ * softmax(scale * q.k) . v.  Read-only on the caches. */
+typedef struct NfnNativeTileGlimmerGqaDecodeDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version; /* NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 */
+    uint32_t flags;   /* 0 */
+    uint32_t reserved0;
+    const float* query;
+    const float* current_key;
+    const float* current_value;
+    const uint16_t* key_cache_bf16;
+    const uint16_t* value_cache_bf16;
+    float* output;
+    int64_t query_heads;
+    int64_t kv_heads;
+    int64_t head_dim; /* 1..256 */
+    int64_t position;
+    int64_t first_key_position; /* 0..position */
+    int64_t cache_capacity;
+    int64_t cache_row_stride; /* elements, >= kv_heads*head_dim */
+    float scale;              /* finite, > 0 */
+    uint32_t reserved1;
+    void* cuda_stream;
+} NfnNativeTileGlimmerGqaDecodeDescriptorV1;
+int nfn_native_tile_glimmer_gqa_decode_float32_v1(
+    const NfnNativeTileGlimmerGqaDecodeDescriptorV1* descriptor);
+
+/* Writes current_key/current_value [kv_heads*head_dim] (rows of them for the
+ * second form, 1..64, row r at position + r) into row (position %
+ * cache_capacity) of the bf16 caches, rounding to nearest even
+ * (tile_ops.h:341-359, 955-959). */
+typedef struct NfnNativeTileGlimmerCacheCommitDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version;
+    uint32_t flags;
+    uint32_t reserved0;
+    const float* current_key;
+    const float* current_value;
+    uint16_t* key_cache_bf16;
+    uint16_t* value_cache_bf16;
+    int64_t kv_heads;
+    int64_t head_dim;
+    int64_t position;
+    int64_t cache_capacity;
+    int64_t cache_row_stride;
+    uint32_t reserved1;
+    uint32_t reserved2;
+    void* cuda_stream;
+} NfnNativeTileGlimmerCacheCommitDescriptorV1;
+int nfn_native_tile_glimmer_cache_commit_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitDescriptorV1* descriptor);
+int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitDescriptorV1* descriptor,
+    int64_t rows);
+
+/* Attention of a block of query_rows rows (positions context_length + r) over
+ * the cached context and the block's own block_rows keys (tile_ops.h:445-486,
+ * 974-975).  Causal (flags = NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL): keys
+ * max(0, p - sliding_window + 1) .. p; block rows before the query's own are
+ * rounded to bf16 on read, as a token-at-a-time decode would have cached them,
+ * the query's own row stays float.  Not causal: keys max(0, p - sliding_window)
+ * .. min(context_length + block_rows - 1, p + sliding_window), block rows in
+ * float.  block_key/block_value: [block_rows, kv_heads, head_dim] float;
+ * query, output: [query_rows, query_heads, head_dim].  block_rows <= 64. */
+typedef struct NfnNativeTileDFlashBlockAttentionDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version;
+    uint32_t flags;
+    uint32_t reserved0;
+    const float* query;
+    const float* block_key;
+    const float* block_value;
+    const uint16_t* key_cache_bf16;
+    const uint16_t* value_cache_bf16;
+    float* output;
+    int64_t query_rows;
+    int64_t block_rows;
+    int64_t query_heads;
+    int64_t kv_heads;
+    int64_t head_dim;
+    int64_t context_length;
+    int64_t sliding_window;
+    int64_t cache_capacity; /* >= sliding_window */
+    int64_t cache_row_stride;
+    float scale;
+    uint32_t reserved1;
+    void* cuda_stream;
+} NfnNativeTileDFlashBlockAttentionDescriptorV1;
+int nfn_native_tile_dflash_block_attention_float32_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* descriptor);
+
+/* logits[i] = softcap * tanh(multiplier * logits[i] / softcap), in place, in
+ * double as the CPU engine computes it (tile_ops.h:1004-1009;
+ * resident_glimmer.cpp:1895-1903).  multiplier, softcap finite and > 0. */
+int nfn_native_tile_glimmer_logit_transform_float32_v1(
+    float* logits,
+    int64_t count,
+    float multiplier,
+    float softcap,
+    void* cuda_stream);
+
+/* out[i] = lhs[i] + rhs[i] (tile_ops.h:1262-1267); values[i] *= scale
+ * (tile_ops.h:1818-1822). */
+int nfn_native_tile_add_float32(
+    const float* lhs,
+    const float* rhs,
+    float* out,
+    int64_t n,
+    void* cuda_stream);
+int nfn_native_tile_scale_inplace_float32(
+    float* values,
+    int64_t n,
+    float scale,
+    void* cuda_stream);
+
 /* ==== additions: no counterpart in the reference ========================= */
 
 int nfn_mi355_abi_version(void);

@@ -1,0 +1,212 @@
+// extern "C" surface of the decode loop's operators around the packed linears:
+// argument checks as the reference's wrappers make them
+// (neuralfn/csrc/native_train/tile_ops.cu:3601-3800, 4734-4775, 5013-5030,
+// 5150-5260, 5348-5362, 5421-5445, 6377-6388, 6944-6951), then one launch.
+#include "common.hpp"
+#include "kernels.hpp"
+
+#include <cmath>
+#include <limits>
+
+namespace nfn {
+
+namespace {
+
+constexpr std::int64_t kMaxHeadDim = 256;
+constexpr std::int64_t kMaxBlockRows = 64;
+constexpr std::int64_t kLimit = std::numeric_limits<std::int64_t>::max();
+
+bool positive_finite(float value) { return std::isfinite(value) && value > 0.0f; }
+
+// kv_heads * head_dim, both positive, fits and does not exceed the row stride
+bool cache_rows_fit(std::int64_t kv_heads, std::int64_t head_dim, std::int64_t row_stride) {
+    return kv_heads <= kLimit / head_dim && kv_heads * head_dim <= row_stride;
+}
+
+bool rope_arguments_valid(const float* query, const float* key, std::int64_t rows,
+                          std::int64_t query_heads, std::int64_t kv_heads, std::int64_t head_dim,
+                          std::int64_t position, float theta, std::uint32_t layout) {
+    return query != nullptr && key != nullptr && rows > 0 && query_heads > 0 && kv_heads > 0 &&
+        query_heads % kv_heads == 0 && head_dim > 0 && head_dim <= kMaxHeadDim &&
+        head_dim % 2 == 0 && position >= 0 && position <= kLimit - rows &&
+        positive_finite(theta) &&
+        (layout == NFN_NATIVE_TILE_GLIMMER_ROPE_HALF_SPLIT ||
+         layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED) &&
+        rows <= kLimit / ((query_heads + kv_heads) * (head_dim / 2));
+}
+
+bool commit_descriptor_valid(const NfnNativeTileGlimmerCacheCommitDescriptorV1* d) {
+    return d != nullptr && d->struct_size >= sizeof(*d) &&
+        d->version == NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 && d->flags == 0 &&
+        d->reserved0 == 0 && d->reserved1 == 0 && d->reserved2 == 0 &&
+        d->current_key != nullptr && d->current_value != nullptr &&
+        d->key_cache_bf16 != nullptr && d->value_cache_bf16 != nullptr && d->kv_heads > 0 &&
+        d->head_dim > 0 && d->head_dim <= kMaxHeadDim && d->position >= 0 &&
+        d->cache_capacity > 0 && d->cache_row_stride > 0 &&
+        cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride);
+}
+
+}  // namespace
+
+}  // namespace nfn
+
+using namespace nfn;
+
+extern "C" {
+
+int nfn_native_tile_glimmer_embedding_gather_float32_v1(const Descriptor* descriptor,
+                                                        std::int64_t token_id, float* output) {
+    Descriptor table{};
+    if (!normalize_descriptor(descriptor, &table) || token_id < 0 ||
+        token_id >= table.output_dim || output == nullptr) {
+        return kInvalid;
+    }
+    launch_embedding(table, 0, token_id, nullptr, output, 1, as_stream(table.cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_embedding_gather_device_i64_float32_v1(const Descriptor* descriptor,
+                                                                   const std::int64_t* token_id,
+                                                                   float* output) {
+    Descriptor table{};
+    if (!normalize_descriptor(descriptor, &table) || token_id == nullptr || output == nullptr) {
+        return kInvalid;
+    }
+    launch_embedding(table, 1, 0, token_id, output, 1, as_stream(table.cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_embedding_batch_i32_float32_v1(const Descriptor* descriptor,
+                                                           const std::int32_t* token_ids,
+                                                           float* output, std::int64_t rows) {
+    Descriptor table{};
+    if (!normalize_descriptor(descriptor, &table) || token_ids == nullptr || output == nullptr ||
+        rows <= 0 || rows > kLimit / table.input_dim) {
+        return kInvalid;
+    }
+    launch_embedding(table, 2, 0, token_ids, output, rows, as_stream(table.cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_positioned_rope_float32_v1(float* query, float* key,
+                                                       std::int64_t query_heads,
+                                                       std::int64_t kv_heads,
+                                                       std::int64_t head_dim,
+                                                       std::int64_t position, float theta,
+                                                       std::uint32_t layout, void* cuda_stream) {
+    if (!rope_arguments_valid(query, key, 1, query_heads, kv_heads, head_dim, position, theta,
+                              layout)) {
+        return kInvalid;
+    }
+    launch_rope(query, key, 1, query_heads, kv_heads, head_dim, position, theta,
+                layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, false, as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_positioned_rope_batch_float32_v1(
+    float* query, float* key, std::int64_t rows, std::int64_t query_heads, std::int64_t kv_heads,
+    std::int64_t head_dim, std::int64_t start_position, float theta, std::uint32_t layout,
+    bool inverse, void* cuda_stream) {
+    if (!rope_arguments_valid(query, key, rows, query_heads, kv_heads, head_dim, start_position,
+                              theta, layout)) {
+        return kInvalid;
+    }
+    launch_rope(query, key, rows, query_heads, kv_heads, head_dim, start_position, theta,
+                layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, inverse,
+                as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_gqa_decode_float32_v1(
+    const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
+    if (d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->query == nullptr ||
+        d->current_key == nullptr || d->current_value == nullptr ||
+        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
+        d->query_heads <= 0 || d->kv_heads <= 0 || d->query_heads % d->kv_heads != 0 ||
+        d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->position < 0 ||
+        d->position == kLimit || d->first_key_position < 0 ||
+        d->first_key_position > d->position || d->cache_capacity <= 0 ||
+        d->cache_row_stride <= 0 || !positive_finite(d->scale) ||
+        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
+        d->query_heads > std::numeric_limits<std::int32_t>::max()) {
+        return kInvalid;
+    }
+    launch_gqa_decode(*d, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_cache_commit_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitDescriptorV1* d) {
+    if (!commit_descriptor_valid(d)) return kInvalid;
+    launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
+                        d->kv_heads * d->head_dim, 1, d->position, d->cache_capacity,
+                        d->cache_row_stride, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitDescriptorV1* d, std::int64_t rows) {
+    if (!commit_descriptor_valid(d) || rows <= 0 || rows > kMaxBlockRows ||
+        d->position > kLimit - rows || d->kv_heads * d->head_dim > kLimit / rows) {
+        return kInvalid;
+    }
+    launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
+                        d->kv_heads * d->head_dim, rows, d->position, d->cache_capacity,
+                        d->cache_row_stride, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_dflash_block_attention_float32_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* d) {
+    if (d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 ||
+        (d->flags & ~static_cast<std::uint32_t>(NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL)) != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->query == nullptr ||
+        d->block_key == nullptr || d->block_value == nullptr || d->key_cache_bf16 == nullptr ||
+        d->value_cache_bf16 == nullptr || d->output == nullptr || d->query_rows <= 0 ||
+        d->block_rows <= 0 || d->query_rows > d->block_rows || d->block_rows > kMaxBlockRows ||
+        d->query_heads <= 0 || d->kv_heads <= 0 || d->query_heads % d->kv_heads != 0 ||
+        d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->context_length < 0 ||
+        d->context_length > kLimit - kMaxBlockRows || d->sliding_window <= 0 ||
+        d->cache_capacity < d->sliding_window || d->cache_row_stride <= 0 ||
+        !positive_finite(d->scale) ||
+        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
+        d->query_heads > std::numeric_limits<std::int32_t>::max() / kMaxBlockRows) {
+        return kInvalid;
+    }
+    launch_block_attention(*d, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_logit_transform_float32_v1(float* logits, std::int64_t count,
+                                                       float multiplier, float softcap,
+                                                       void* cuda_stream) {
+    if (logits == nullptr || count <= 0 || !positive_finite(multiplier) ||
+        !positive_finite(softcap)) {
+        return kInvalid;
+    }
+    launch_logit_transform(logits, count, multiplier, softcap, as_stream(cuda_stream));
+    return launch_status();
+}
+
+// The reference checks only the count here (tile_ops.cu:6377-6388); null
+// pointers would fault in its kernel, this build refuses them.
+int nfn_native_tile_add_float32(const float* lhs, const float* rhs, float* out, std::int64_t n,
+                                void* cuda_stream) {
+    if (n <= 0 || lhs == nullptr || rhs == nullptr || out == nullptr) return kInvalid;
+    launch_add(lhs, rhs, out, n, as_stream(cuda_stream));
+    return launch_status();
+}
+
+// The reference launches whatever it is given (tile_ops.cu:6944-6951); an
+// empty or null array is refused here, anything else is scaled.
+int nfn_native_tile_scale_inplace_float32(float* values, std::int64_t n, float scale,
+                                          void* cuda_stream) {
+    if (values == nullptr || n <= 0) return kInvalid;
+    launch_scale(values, n, scale, as_stream(cuda_stream));
+    return launch_status();
+}
+
+}  // extern "C"

@@ -109,6 +109,20 @@ __device__ __forceinline__ float load_half(const std::uint8_t* p) {
     return half_bits_to_float(static_cast<std::uint32_t>(p[0]) | (static_cast<std::uint32_t>(p[1]) << 8));
 }
 
+// float -> bf16 bits, round to nearest even; a NaN stays a NaN.
+__device__ __forceinline__ std::uint16_t to_bf16(float value) {
+    const std::uint32_t bits = __float_as_uint(value);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) {
+        return static_cast<std::uint16_t>((bits >> 16) | 0x40u);
+    }
+    const std::uint32_t rounding = 0x7fffu + ((bits >> 16) & 1u);
+    return static_cast<std::uint16_t>((bits + rounding) >> 16);
+}
+
+__device__ __forceinline__ float bf16_to_float(std::uint32_t bits) {
+    return __uint_as_float(bits << 16);
+}
+
 // 6-bit scale and minimum of sub-block `index` (resident_glimmer.cpp:178-186).
 __device__ __forceinline__ void k_scale_min(const std::uint8_t* scales, int index,
                                             int* scale, int* minimum) {

@@ -48,6 +48,30 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
                      std::int8_t* q8_codes, float* q8_scales, float* q8_sums, std::int64_t rows,
                      std::int64_t width, float eps, hipStream_t stream);
 
+// engine_ops.hip — the small operators around the packed linears.
+// token_source: 0 = host_token, 1 = one int64 in device memory, 2 = int32 per row.
+void launch_embedding(const Descriptor& table, int token_source, std::int64_t host_token,
+                      const void* device_tokens, float* output, std::int64_t rows,
+                      hipStream_t stream);
+void launch_rope(float* query, float* key, std::int64_t rows, std::int64_t query_heads,
+                 std::int64_t kv_heads, std::int64_t head_dim, std::int64_t start_position,
+                 float theta, bool interleaved, bool inverse, hipStream_t stream);
+void launch_cache_commit(const float* keys, const float* values, std::uint16_t* key_cache,
+                         std::uint16_t* value_cache, std::int64_t width, std::int64_t rows,
+                         std::int64_t position, std::int64_t capacity, std::int64_t row_stride,
+                         hipStream_t stream);
+void launch_logit_transform(float* logits, std::int64_t count, float multiplier, float softcap,
+                            hipStream_t stream);
+void launch_add(const float* lhs, const float* rhs, float* out, std::int64_t count,
+                hipStream_t stream);
+void launch_scale(float* values, std::int64_t count, float scale, hipStream_t stream);
+
+// attention.hip — descriptors already checked.
+void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
+                       hipStream_t stream);
+void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& descriptor,
+                            hipStream_t stream);
+
 // clock_probe.hip — out[0] = shader cycles, out[1] = ticks of the constant
 // clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.
 void launch_clock_probe(std::uint64_t* out, std::int64_t ticks, std::uint64_t ticks_per_second,

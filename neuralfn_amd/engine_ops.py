@@ -1,0 +1,149 @@
+"""torch-tensor front end of the decode loop's operators around the packed linears.
+
+Embedding, rotary position embedding, one-token and block attention over a bf16
+cache, the cache commit, the logit transform, add and scale: the operators the
+reference's resident engine requires from its sidecar besides the linears
+(neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:431-495).  Everything goes
+through the C ABI of libnfn_mi355_tile_ops.so; torch only owns the memory.
+"""
+from __future__ import annotations
+
+import ctypes
+
+from . import tile_ops
+from .tile_ops import (BlockAttentionDescriptor, CacheCommitDescriptor, GqaDecodeDescriptor,
+                       PackedWeight, check, load)
+
+ROPE_HALF_SPLIT = 0
+ROPE_INTERLEAVED = 1
+BLOCK_ATTENTION_CAUSAL = 1
+
+
+def _stream() -> int:
+    return tile_ops._stream_handle()
+
+
+def embedding(table: PackedWeight, tokens):
+    """Rows of the table: `tokens` is an int (host), an int64 tensor of one element, or an int32 tensor."""
+    import torch
+    stream = _stream()
+    descriptor = table.descriptor(stream)
+    device = table.data.device
+    if isinstance(tokens, int):
+        out = torch.empty(table.input_dim, dtype=torch.float32, device=device)
+        check(load().nfn_native_tile_glimmer_embedding_gather_float32_v1(
+            ctypes.byref(descriptor), tokens, out.data_ptr()), "embedding_gather")
+        return out
+    if tokens.dtype == torch.int64:
+        out = torch.empty(table.input_dim, dtype=torch.float32, device=device)
+        check(load().nfn_native_tile_glimmer_embedding_gather_device_i64_float32_v1(
+            ctypes.byref(descriptor), tokens.data_ptr(), out.data_ptr()),
+            "embedding_gather_device_i64")
+        return out
+    rows = tokens.numel()
+    out = torch.empty((rows, table.input_dim), dtype=torch.float32, device=device)
+    check(load().nfn_native_tile_glimmer_embedding_batch_i32_float32_v1(
+        ctypes.byref(descriptor), tokens.data_ptr(), out.data_ptr(), rows), "embedding_batch_i32")
+    return out
+
+
+def rope(query, key, position: int, theta: float, layout: int = ROPE_HALF_SPLIT,
+         inverse: bool = False, batch: bool = False) -> None:
+    """In place.  query [rows, query_heads, head_dim] / key [rows, kv_heads, head_dim] with
+    `batch`, else [query_heads, head_dim] / [kv_heads, head_dim] at one position."""
+    if batch:
+        rows, query_heads, head_dim = query.shape
+        check(load().nfn_native_tile_glimmer_positioned_rope_batch_float32_v1(
+            query.data_ptr(), key.data_ptr(), rows, query_heads, key.shape[1], head_dim,
+            position, theta, layout, inverse, _stream()), "positioned_rope_batch")
+        return
+    query_heads, head_dim = query.shape
+    check(load().nfn_native_tile_glimmer_positioned_rope_float32_v1(
+        query.data_ptr(), key.data_ptr(), query_heads, key.shape[0], head_dim, position, theta,
+        layout, _stream()), "positioned_rope")
+
+
+def gqa_decode(query, current_key, current_value, key_cache, value_cache, position: int,
+               first_key_position: int, scale: float, out=None):
+    """query [query_heads, head_dim]; current_key/value [kv_heads, head_dim]; caches uint16
+    (or bfloat16) [capacity, row_stride]."""
+    import torch
+    if out is None:
+        out = torch.empty_like(query)
+    d = GqaDecodeDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.query, d.current_key, d.current_value = (query.data_ptr(), current_key.data_ptr(),
+                                               current_value.data_ptr())
+    d.key_cache_bf16, d.value_cache_bf16 = key_cache.data_ptr(), value_cache.data_ptr()
+    d.output = out.data_ptr()
+    d.query_heads, d.head_dim = query.shape
+    d.kv_heads = current_key.shape[0]
+    d.position, d.first_key_position = position, first_key_position
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.scale = scale
+    d.cuda_stream = _stream()
+    check(load().nfn_native_tile_glimmer_gqa_decode_float32_v1(ctypes.byref(d)), "gqa_decode")
+    return out
+
+
+def cache_commit(keys, values, key_cache, value_cache, position: int, rows: int = 0) -> None:
+    """keys/values [kv_heads, head_dim] (rows == 0) or [rows, kv_heads, head_dim]."""
+    d = CacheCommitDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.current_key, d.current_value = keys.data_ptr(), values.data_ptr()
+    d.key_cache_bf16, d.value_cache_bf16 = key_cache.data_ptr(), value_cache.data_ptr()
+    d.kv_heads, d.head_dim = keys.shape[-2], keys.shape[-1]
+    d.position = position
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.cuda_stream = _stream()
+    if rows:
+        check(load().nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(ctypes.byref(d), rows),
+              "cache_commit_rows")
+    else:
+        check(load().nfn_native_tile_glimmer_cache_commit_bf16_v1(ctypes.byref(d)), "cache_commit")
+
+
+def block_attention(query, block_key, block_value, key_cache, value_cache, context_length: int,
+                    sliding_window: int, scale: float, causal: bool, out=None):
+    """query [query_rows, query_heads, head_dim]; block_key/value [block_rows, kv_heads, head_dim]."""
+    import torch
+    if out is None:
+        out = torch.empty_like(query)
+    d = BlockAttentionDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.flags = BLOCK_ATTENTION_CAUSAL if causal else 0
+    d.query, d.block_key, d.block_value = (query.data_ptr(), block_key.data_ptr(),
+                                           block_value.data_ptr())
+    d.key_cache_bf16, d.value_cache_bf16 = key_cache.data_ptr(), value_cache.data_ptr()
+    d.output = out.data_ptr()
+    d.query_rows, d.query_heads, d.head_dim = query.shape
+    d.block_rows, d.kv_heads = block_key.shape[0], block_key.shape[1]
+    d.context_length, d.sliding_window = context_length, sliding_window
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.scale = scale
+    d.cuda_stream = _stream()
+    check(load().nfn_native_tile_dflash_block_attention_float32_v1(ctypes.byref(d)),
+          "block_attention")
+    return out
+
+
+def logit_transform(logits, multiplier: float, softcap: float) -> None:
+    check(load().nfn_native_tile_glimmer_logit_transform_float32_v1(
+        logits.data_ptr(), logits.numel(), multiplier, softcap, _stream()), "logit_transform")
+
+
+def add(lhs, rhs, out=None):
+    import torch
+    if out is None:
+        out = torch.empty_like(lhs)
+    check(load().nfn_native_tile_add_float32(lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(),
+                                             lhs.numel(), _stream()), "add")
+    return out
+
+
+def scale_inplace(values, scale: float) -> None:
+    check(load().nfn_native_tile_scale_inplace_float32(values.data_ptr(), values.numel(), scale,
+                                                       _stream()), "scale_inplace")

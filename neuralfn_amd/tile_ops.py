@@ -44,6 +44,49 @@ class PackedWeightDescriptor(ctypes.Structure):
 
 _P = ctypes.c_void_p
 _I64 = ctypes.c_int64
+_U32 = ctypes.c_uint32
+_F32 = ctypes.c_float
+
+
+class GqaDecodeDescriptor(ctypes.Structure):
+    """NfnNativeTileGlimmerGqaDecodeDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:316-339)."""
+
+    _fields_ = [
+        ("struct_size", _U32), ("version", _U32), ("flags", _U32), ("reserved0", _U32),
+        ("query", _P), ("current_key", _P), ("current_value", _P),
+        ("key_cache_bf16", _P), ("value_cache_bf16", _P), ("output", _P),
+        ("query_heads", _I64), ("kv_heads", _I64), ("head_dim", _I64), ("position", _I64),
+        ("first_key_position", _I64), ("cache_capacity", _I64), ("cache_row_stride", _I64),
+        ("scale", _F32), ("reserved1", _U32), ("cuda_stream", _P),
+    ]
+
+
+class CacheCommitDescriptor(ctypes.Structure):
+    """NfnNativeTileGlimmerCacheCommitDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:341-359)."""
+
+    _fields_ = [
+        ("struct_size", _U32), ("version", _U32), ("flags", _U32), ("reserved0", _U32),
+        ("current_key", _P), ("current_value", _P), ("key_cache_bf16", _P),
+        ("value_cache_bf16", _P),
+        ("kv_heads", _I64), ("head_dim", _I64), ("position", _I64), ("cache_capacity", _I64),
+        ("cache_row_stride", _I64), ("reserved1", _U32), ("reserved2", _U32), ("cuda_stream", _P),
+    ]
+
+
+class BlockAttentionDescriptor(ctypes.Structure):
+    """NfnNativeTileDFlashBlockAttentionDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:461-486)."""
+
+    _fields_ = [
+        ("struct_size", _U32), ("version", _U32), ("flags", _U32), ("reserved0", _U32),
+        ("query", _P), ("block_key", _P), ("block_value", _P),
+        ("key_cache_bf16", _P), ("value_cache_bf16", _P), ("output", _P),
+        ("query_rows", _I64), ("block_rows", _I64), ("query_heads", _I64), ("kv_heads", _I64),
+        ("head_dim", _I64), ("context_length", _I64), ("sliding_window", _I64),
+        ("cache_capacity", _I64), ("cache_row_stride", _I64),
+        ("scale", _F32), ("reserved1", _U32), ("cuda_stream", _P),
+    ]
+
+
 _DESC = ctypes.POINTER(PackedWeightDescriptor)
 _DESC_ARRAY = ctypes.POINTER(_DESC)
 _PTR_ARRAY = ctypes.POINTER(ctypes.c_void_p)
@@ -109,6 +152,24 @@ SIGNATURES = {
     "nfn_mi355_k_quant_gemm_float32_v1": (
         ctypes.c_int, [_DESC, _P, _P, _I64, _P, _I64, ctypes.c_int, _P]),
     "nfn_mi355_shader_clock_probe_v1": (ctypes.c_int, [_P, _I64, _P]),
+    "nfn_native_tile_glimmer_embedding_gather_float32_v1": (ctypes.c_int, [_DESC, _I64, _P]),
+    "nfn_native_tile_glimmer_embedding_gather_device_i64_float32_v1": (ctypes.c_int, [_DESC, _P, _P]),
+    "nfn_native_tile_glimmer_embedding_batch_i32_float32_v1": (ctypes.c_int, [_DESC, _P, _P, _I64]),
+    "nfn_native_tile_glimmer_positioned_rope_float32_v1": (
+        ctypes.c_int, [_P, _P, _I64, _I64, _I64, _I64, _F32, _U32, _P]),
+    "nfn_native_tile_glimmer_positioned_rope_batch_float32_v1": (
+        ctypes.c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _F32, _U32, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_gqa_decode_float32_v1": (
+        ctypes.c_int, [ctypes.POINTER(GqaDecodeDescriptor)]),
+    "nfn_native_tile_glimmer_cache_commit_bf16_v1": (
+        ctypes.c_int, [ctypes.POINTER(CacheCommitDescriptor)]),
+    "nfn_native_tile_glimmer_cache_commit_rows_bf16_v1": (
+        ctypes.c_int, [ctypes.POINTER(CacheCommitDescriptor), _I64]),
+    "nfn_native_tile_dflash_block_attention_float32_v1": (
+        ctypes.c_int, [ctypes.POINTER(BlockAttentionDescriptor)]),
+    "nfn_native_tile_glimmer_logit_transform_float32_v1": (ctypes.c_int, [_P, _I64, _F32, _F32, _P]),
+    "nfn_native_tile_add_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
+    "nfn_native_tile_scale_inplace_float32": (ctypes.c_int, [_P, _I64, _F32, _P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -595,4 +595,133 @@ void nfo_dual_rms_add_capture(const float* input, const float* first_weight, int
     }
 }
 
+// ---- the decode loop's operators around the packed linears -----------------
+
+// Rotary position embedding of `heads` heads at one position, in double
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:773-800): pair i is elements
+// (i, i + head_dim/2), or (2i, 2i+1) when interleaved; angle = position /
+// theta^(2i/head_dim); [a, b] -> [a cos - b sin, b cos + a sin].  `inverse`
+// rotates by the negative angle (neuralfn/csrc/tile_cuda/kernels.cu:3545-3553).
+// Pinned by the compiled reference's apply_rope and by rotation invariants
+// (norm preserved, position 0 is the identity, inverse undoes).
+void nfo_rope(float* values, std::int64_t heads, std::int64_t head_dim, std::int64_t position,
+              double theta, int interleaved, int inverse) {
+    const std::int64_t half = head_dim / 2;
+    for (std::int64_t head = 0; head < heads; ++head) {
+        float* row = values + head * head_dim;
+        for (std::int64_t index = 0; index < half; ++index) {
+            const double inverse_frequency = 1.0 / std::pow(
+                theta, static_cast<double>(2 * index) / static_cast<double>(head_dim));
+            double angle = static_cast<double>(position) * inverse_frequency;
+            if (inverse) angle = -angle;
+            const double cosine = std::cos(angle);
+            const double sine = std::sin(angle);
+            const std::int64_t first_index = interleaved ? 2 * index : index;
+            const std::int64_t second_index = interleaved ? 2 * index + 1 : index + half;
+            const float first = row[first_index];
+            const float second = row[second_index];
+            row[first_index] = static_cast<float>(first * cosine - second * sine);
+            row[second_index] = static_cast<float>(second * cosine + first * sine);
+        }
+    }
+}
+
+// float -> bf16 bits, round to nearest even (the cache commit,
+// neuralfn/csrc/tile_cuda/kernels.cu:2826-2840; the reference's probe states the
+// same rule on the host, tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:2484-2512).
+// Pinned by closed forms: exact values stay, ties go to even, 65,536 patterns
+// round-trip.
+std::uint16_t nfo_to_bf16(float value) {
+    std::uint32_t bits;
+    std::memcpy(&bits, &value, 4);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) return static_cast<std::uint16_t>((bits >> 16) | 0x40u);
+    const std::uint32_t rounding = 0x7fffu + ((bits >> 16) & 1u);
+    return static_cast<std::uint16_t>((bits + rounding) >> 16);
+}
+
+float nfo_bf16_to_float(std::uint16_t bits) {
+    const std::uint32_t wide = static_cast<std::uint32_t>(bits) << 16;
+    float value;
+    std::memcpy(&value, &wide, 4);
+    return value;
+}
+
+// Block attention over a bf16 cache in double: the expected values of the
+// reference's probe (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:2446-2482)
+// with the key ranges and the causal rounding rule of the device kernel
+// (neuralfn/csrc/tile_cuda/kernels.cu:2943-2990).  Query row r is at position
+// context_length + r.  Causal: keys max(0, p - window + 1) .. p, block rows
+// before r rounded to bf16.  Otherwise: keys max(0, p - window) ..
+// min(context_length + block_rows - 1, p + window).  The one-token form is
+// query_rows = block_rows = 1, causal, window = position - first_key + 1.
+// Pinned by the reference's CPU sidecar compiled from its source and by closed
+// forms (one key, equal scores, a dominating key).
+void nfo_block_attention(const float* query, const float* block_key, const float* block_value,
+                         const std::uint16_t* key_cache, const std::uint16_t* value_cache,
+                         float* output, std::int64_t query_rows, std::int64_t block_rows,
+                         std::int64_t query_heads, std::int64_t kv_heads, std::int64_t head_dim,
+                         std::int64_t context_length, std::int64_t sliding_window,
+                         std::int64_t cache_capacity, std::int64_t cache_row_stride, float scale,
+                         int causal) {
+    std::vector<double> scores;
+    for (std::int64_t row = 0; row < query_rows; ++row) {
+        const std::int64_t position = context_length + row;
+        const std::int64_t first =
+            std::max<std::int64_t>(0, position - sliding_window + (causal ? 1 : 0));
+        const std::int64_t last = causal
+            ? position
+            : std::min<std::int64_t>(context_length + block_rows - 1, position + sliding_window);
+        for (std::int64_t head = 0; head < query_heads; ++head) {
+            const std::int64_t kv_head = head * kv_heads / query_heads;
+            const float* q = query + (row * query_heads + head) * head_dim;
+            const auto key_at = [&](std::int64_t key_position, std::int64_t dim,
+                                    const float* block, const std::uint16_t* cache) -> float {
+                if (key_position >= context_length) {
+                    const std::int64_t block_row = key_position - context_length;
+                    float value = block[(block_row * kv_heads + kv_head) * head_dim + dim];
+                    if (causal && block_row < row) value = nfo_bf16_to_float(nfo_to_bf16(value));
+                    return value;
+                }
+                return nfo_bf16_to_float(cache[(key_position % cache_capacity) * cache_row_stride +
+                                               kv_head * head_dim + dim]);
+            };
+            scores.assign(static_cast<std::size_t>(last - first + 1), 0.0);
+            double maximum = -std::numeric_limits<double>::infinity();
+            for (std::int64_t key_position = first; key_position <= last; ++key_position) {
+                double dot = 0.0;
+                for (std::int64_t dim = 0; dim < head_dim; ++dim) {
+                    dot += static_cast<double>(q[dim]) *
+                        key_at(key_position, dim, block_key, key_cache);
+                }
+                scores[static_cast<std::size_t>(key_position - first)] = dot * scale;
+                maximum = std::max(maximum, dot * scale);
+            }
+            double denominator = 0.0;
+            for (double& score : scores) {
+                score = std::exp(score - maximum);
+                denominator += score;
+            }
+            for (std::int64_t dim = 0; dim < head_dim; ++dim) {
+                double sum = 0.0;
+                for (std::int64_t key_position = first; key_position <= last; ++key_position) {
+                    sum += scores[static_cast<std::size_t>(key_position - first)] *
+                        key_at(key_position, dim, block_value, value_cache);
+                }
+                output[(row * query_heads + head) * head_dim + dim] =
+                    static_cast<float>(sum / denominator);
+            }
+        }
+    }
+}
+
+// softcap * tanh(multiplier * x / softcap) in double
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:1895-1903).  Pinned by closed
+// forms: odd, bounded by softcap, slope `multiplier` at 0, tanh(1) at x = softcap/multiplier.
+void nfo_logit_transform(float* logits, std::int64_t count, double multiplier, double softcap) {
+    for (std::int64_t index = 0; index < count; ++index) {
+        logits[index] = static_cast<float>(
+            softcap * std::tanh((multiplier * static_cast<double>(logits[index])) / softcap));
+    }
+}
+
 }  // extern "C"

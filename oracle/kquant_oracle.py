@@ -16,6 +16,7 @@ import numpy as np
 HERE = Path(__file__).resolve().parent
 ORACLE_LIB = HERE / "libnfn_kquant_oracle.so"
 REF_LIB = HERE / "_ref" / "libnfn_kquant_ref.so"
+SIDECAR_REF_LIB = HERE / "_ref" / "libnfn_cpu_sidecar_ref.so"
 REFERENCE_ROOT = Path("/root/reference")
 
 _P = ctypes.c_void_p
@@ -71,6 +72,15 @@ def lib() -> ctypes.CDLL:
         o.nfo_dual_rms_add_capture.argtypes = [_P, _P, ctypes.c_int, _P, _P, _P, ctypes.c_int, _P,
                                                _I64, _I64, ctypes.c_float, ctypes.c_float]
         o.nfo_dual_rms_add_capture.restype = None
+        o.nfo_rope.argtypes = [_P, _I64, _I64, _I64, ctypes.c_double, ctypes.c_int, ctypes.c_int]
+        o.nfo_rope.restype = None
+        o.nfo_to_bf16.argtypes = [ctypes.c_float]
+        o.nfo_to_bf16.restype = ctypes.c_uint16
+        o.nfo_block_attention.argtypes = [_P, _P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64,
+                                          _I64, _I64, _I64, _I64, ctypes.c_float, ctypes.c_int]
+        o.nfo_block_attention.restype = None
+        o.nfo_logit_transform.argtypes = [_P, _I64, ctypes.c_double, ctypes.c_double]
+        o.nfo_logit_transform.restype = None
         _oracle = o
     return _oracle
 
@@ -97,6 +107,8 @@ def ref() -> ctypes.CDLL:
         r.nfr_rms_norm.restype = ctypes.c_int
         r.nfr_argmax.argtypes = [_P, _I64]
         r.nfr_argmax.restype = _I64
+        r.nfr_apply_rope.argtypes = [_P, _I64, _I64, _I64, ctypes.c_double, ctypes.c_int]
+        r.nfr_apply_rope.restype = ctypes.c_int
         _ref = r
     return _ref
 
@@ -257,6 +269,73 @@ def dual_rms_add_capture(x: np.ndarray, residual: np.ndarray, first_weight=None,
     return hidden, normalized
 
 
+# ---- the decode loop's operators around the packed linears ----------------
+
+def rope(values: np.ndarray, position: int, theta: float, interleaved: bool = False,
+         inverse: bool = False) -> np.ndarray:
+    """values [heads, head_dim] rotated at `position`; returns a new array."""
+    out = np.array(values, dtype=np.float32, order="C", copy=True)
+    heads, head_dim = out.shape
+    lib().nfo_rope(out.ctypes.data, heads, head_dim, int(position), float(theta), int(interleaved),
+                   int(inverse))
+    return out
+
+
+def to_bf16(values: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bits (uint16), round to nearest even, vectorised restatement of nfo_to_bf16."""
+    bits = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32)
+    rounding = np.uint32(0x7FFF) + ((bits >> np.uint32(16)) & np.uint32(1))
+    rounded = ((bits + rounding) >> np.uint32(16)).astype(np.uint16)
+    nan = (bits & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    return np.where(nan, ((bits >> np.uint32(16)) | np.uint32(0x40)).astype(np.uint16), rounded)
+
+
+def to_bf16_scalar(value: float) -> int:
+    return int(lib().nfo_to_bf16(float(value)))
+
+
+def bf16_to_float(bits: np.ndarray) -> np.ndarray:
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(
+        np.float32)
+
+
+def block_attention(query, block_key, block_value, key_cache, value_cache, context_length: int,
+                    sliding_window: int, scale: float, causal: bool, cache_row_stride=None):
+    """query [rows, query_heads, head_dim]; block_key/value [block_rows, kv_heads, head_dim];
+    caches uint16 [capacity, row_stride]."""
+    query = np.ascontiguousarray(query, dtype=np.float32)
+    block_key = np.ascontiguousarray(block_key, dtype=np.float32)
+    block_value = np.ascontiguousarray(block_value, dtype=np.float32)
+    key_cache = np.ascontiguousarray(key_cache, dtype=np.uint16)
+    value_cache = np.ascontiguousarray(value_cache, dtype=np.uint16)
+    rows, query_heads, head_dim = query.shape
+    block_rows, kv_heads, _ = block_key.shape
+    capacity, stride = key_cache.shape
+    out = np.empty_like(query)
+    lib().nfo_block_attention(query.ctypes.data, block_key.ctypes.data, block_value.ctypes.data,
+                              key_cache.ctypes.data, value_cache.ctypes.data, out.ctypes.data,
+                              rows, block_rows, query_heads, kv_heads, head_dim,
+                              int(context_length), int(sliding_window), capacity,
+                              stride if cache_row_stride is None else cache_row_stride,
+                              float(scale), int(causal))
+    return out
+
+
+def gqa_decode(query, current_key, current_value, key_cache, value_cache, position: int,
+               first_key_position: int, scale: float):
+    """One-token attention: query [query_heads, head_dim], current_key/value [kv_heads, head_dim]."""
+    out = block_attention(np.asarray(query)[None], np.asarray(current_key)[None],
+                          np.asarray(current_value)[None], key_cache, value_cache, position,
+                          position - first_key_position + 1, scale, True)
+    return out[0]
+
+
+def logit_transform(logits: np.ndarray, multiplier: float, softcap: float) -> np.ndarray:
+    out = np.array(logits, dtype=np.float32, order="C", copy=True)
+    lib().nfo_logit_transform(out.ctypes.data, out.size, float(multiplier), float(softcap))
+    return out
+
+
 # ---- the compiled reference (only where `make ref` has been run) ----------
 
 def ref_rms_norm(x: np.ndarray, weight=None, centered: bool = False, epsilon: float = 1e-6):
@@ -289,4 +368,108 @@ def ref_linear(encoding: int, packed: np.ndarray, output_dim: int, input_dim: in
                               x.ctypes.data, x.shape[0], out.ctypes.data)
     if status:
         raise ValueError(f"reference linear status {status}")
+    return out
+
+
+def ref_apply_rope(values: np.ndarray, position: int, theta: float, interleaved: bool = False):
+    out = np.array(values, dtype=np.float32, order="C", copy=True)
+    heads, head_dim = out.shape
+    status = ref().nfr_apply_rope(out.ctypes.data, heads, head_dim, int(position), float(theta),
+                                  int(interleaved))
+    if status:
+        raise ValueError(f"reference apply_rope status {status}")
+    return out
+
+
+# The reference's CPU stand-in for its sidecar (tests/cpp/fake_glimmer_tile_ops.cpp),
+# compiled by `make ref`: same C ABI as the GPU library, host pointers.
+
+class GqaDecodeDescriptor(ctypes.Structure):
+    _fields_ = [("struct_size", ctypes.c_uint32), ("version", ctypes.c_uint32),
+                ("flags", ctypes.c_uint32), ("reserved0", ctypes.c_uint32),
+                ("query", _P), ("current_key", _P), ("current_value", _P),
+                ("key_cache_bf16", _P), ("value_cache_bf16", _P), ("output", _P),
+                ("query_heads", _I64), ("kv_heads", _I64), ("head_dim", _I64),
+                ("position", _I64), ("first_key_position", _I64), ("cache_capacity", _I64),
+                ("cache_row_stride", _I64), ("scale", ctypes.c_float),
+                ("reserved1", ctypes.c_uint32), ("cuda_stream", _P)]
+
+
+class BlockAttentionDescriptor(ctypes.Structure):
+    _fields_ = [("struct_size", ctypes.c_uint32), ("version", ctypes.c_uint32),
+                ("flags", ctypes.c_uint32), ("reserved0", ctypes.c_uint32),
+                ("query", _P), ("block_key", _P), ("block_value", _P),
+                ("key_cache_bf16", _P), ("value_cache_bf16", _P), ("output", _P),
+                ("query_rows", _I64), ("block_rows", _I64), ("query_heads", _I64),
+                ("kv_heads", _I64), ("head_dim", _I64), ("context_length", _I64),
+                ("sliding_window", _I64), ("cache_capacity", _I64), ("cache_row_stride", _I64),
+                ("scale", ctypes.c_float), ("reserved1", ctypes.c_uint32), ("cuda_stream", _P)]
+
+
+_sidecar_ref: Optional[ctypes.CDLL] = None
+
+
+def sidecar_reference_available() -> bool:
+    return SIDECAR_REF_LIB.exists()
+
+
+def sidecar_ref() -> ctypes.CDLL:
+    global _sidecar_ref
+    if _sidecar_ref is None:
+        s = ctypes.CDLL(str(SIDECAR_REF_LIB), mode=ctypes.RTLD_LOCAL)
+        s.nfn_native_tile_glimmer_gqa_decode_float32_v1.argtypes = [_P]
+        s.nfn_native_tile_dflash_block_attention_float32_v1.argtypes = [_P]
+        s.nfn_native_tile_glimmer_positioned_rope_float32_v1.argtypes = [
+            _P, _P, _I64, _I64, _I64, _I64, ctypes.c_float, _U32, _P]
+        _sidecar_ref = s
+    return _sidecar_ref
+
+
+def ref_sidecar_block_attention(query, block_key, block_value, key_cache, value_cache,
+                                context_length: int, sliding_window: int, scale: float,
+                                causal: bool):
+    query = np.ascontiguousarray(query, dtype=np.float32)
+    block_key = np.ascontiguousarray(block_key, dtype=np.float32)
+    block_value = np.ascontiguousarray(block_value, dtype=np.float32)
+    key_cache = np.ascontiguousarray(key_cache, dtype=np.uint16)
+    value_cache = np.ascontiguousarray(value_cache, dtype=np.uint16)
+    out = np.empty_like(query)
+    d = BlockAttentionDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.flags = 1 if causal else 0
+    d.query, d.block_key, d.block_value = query.ctypes.data, block_key.ctypes.data, block_value.ctypes.data
+    d.key_cache_bf16, d.value_cache_bf16, d.output = key_cache.ctypes.data, value_cache.ctypes.data, out.ctypes.data
+    d.query_rows, d.query_heads, d.head_dim = query.shape
+    d.block_rows, d.kv_heads = block_key.shape[0], block_key.shape[1]
+    d.context_length, d.sliding_window = int(context_length), int(sliding_window)
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.scale = float(scale)
+    status = sidecar_ref().nfn_native_tile_dflash_block_attention_float32_v1(ctypes.byref(d))
+    if status:
+        raise ValueError(f"reference sidecar block attention status {status}")
+    return out
+
+
+def ref_sidecar_gqa_decode(query, current_key, current_value, key_cache, value_cache,
+                           position: int, first_key_position: int, scale: float):
+    query = np.ascontiguousarray(query, dtype=np.float32)
+    current_key = np.ascontiguousarray(current_key, dtype=np.float32)
+    current_value = np.ascontiguousarray(current_value, dtype=np.float32)
+    key_cache = np.ascontiguousarray(key_cache, dtype=np.uint16)
+    value_cache = np.ascontiguousarray(value_cache, dtype=np.uint16)
+    out = np.empty_like(query)
+    d = GqaDecodeDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.query, d.current_key, d.current_value = query.ctypes.data, current_key.ctypes.data, current_value.ctypes.data
+    d.key_cache_bf16, d.value_cache_bf16, d.output = key_cache.ctypes.data, value_cache.ctypes.data, out.ctypes.data
+    d.query_heads, d.head_dim = query.shape
+    d.kv_heads = current_key.shape[0]
+    d.position, d.first_key_position = int(position), int(first_key_position)
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.scale = float(scale)
+    status = sidecar_ref().nfn_native_tile_glimmer_gqa_decode_float32_v1(ctypes.byref(d))
+    if status:
+        raise ValueError(f"reference sidecar gqa decode status {status}")
     return out

@@ -114,4 +114,20 @@ std::int64_t nfr_argmax(const float* values, std::int64_t count) {
     return neuralfn::resident_glimmer::argmax_token(logits);
 }
 
+// The reference's CPU rotary position embedding (resident_glimmer.cpp:773-800),
+// in place on `heads` heads of one position.
+int nfr_apply_rope(float* values, std::int64_t heads, std::int64_t head_dim, std::int64_t position,
+                   double theta, int interleaved) {
+    const std::atomic<bool> cancelled{false};
+    try {
+        std::vector<float> buffer(values, values + heads * head_dim);
+        neuralfn::resident_glimmer::apply_rope(&buffer, heads, head_dim, position, theta,
+                                               interleaved != 0, cancelled);
+        std::copy(buffer.begin(), buffer.end(), values);
+    } catch (const std::exception&) {
+        return 2;
+    }
+    return 0;
+}
+
 }  // extern "C"
