@@ -3,16 +3,14 @@
 // model (semantics: neuralfn/csrc/native_train/tile_ops.h:308-339, 445-486;
 // reference kernels: neuralfn/csrc/tile_cuda/kernels.cu:2475-2824, 2924-3075).
 //
-// One workgroup per (query row, query head), up to sixteen waves.  A wave takes
-// every waves-th tile of 64 keys.  Inside a tile a lane owns one key for the
-// scores (it walks the key's head_dim values in 16-byte pieces against the
-// query, which sits in LDS and is read as a broadcast), the wave reduces the
-// tile's maximum and sum once, and for the weighted sum of the values a lane
-// owns the output dimensions lane, lane + 64, ...: the weight of key k comes
-// from lane k by a lane read, the value row is read coalesced.  Every wave
-// keeps a running (maximum, denominator, accumulator) and the workgroup
-// merges them through LDS at the end.  The one-token form is the block form
-// with one query row whose own key is the only block row.
+// One workgroup per (query row, query head), up to eight waves.  A wave takes
+// every active-th tile of 64 keys, keeps a running (maximum, denominator,
+// accumulator), and the workgroup merges the waves through LDS at the end.
+// The query sits in LDS and is read as a broadcast.  Two kernels: a vector
+// form for head sizes that are multiples of 32 (everything in 16-byte pieces,
+// all loads of a phase in flight together) and a generic element-wise form.
+// The one-token form is the block form with one query row whose own key is
+// the only block row.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -20,7 +18,7 @@ namespace nfn {
 
 namespace {
 
-constexpr int kMaxWaves = 16;
+constexpr int kMaxWaves = 8;   // 512 threads: 256 vector registers per lane
 constexpr int kMaxHeadDim = 256;
 constexpr int kOwned = kMaxHeadDim / kWave;  // output dimensions per lane
 
@@ -34,6 +32,7 @@ struct AttentionArguments {
     std::int64_t query_heads;
     std::int64_t kv_heads;
     std::int64_t head_dim;
+    std::uint32_t heads_per_kv;  // query_heads / kv_heads
     std::int64_t context_length;
     std::int64_t block_rows;
     std::int64_t sliding_window;
@@ -59,63 +58,57 @@ __device__ __forceinline__ float wave_sum_f(float value) {
     return value;
 }
 
-// q . k for one key held by this lane.  VEC: head_dim is a multiple of 8 and
-// every row starts 16-byte aligned.
-template <bool VEC>
+// ---------------------------------------------------------------------------
+// Generic form: any head_dim, any alignment; element-wise loads.  A lane owns
+// one key for the scores and the output dimensions lane, lane + 64, ... for
+// the weighted sum.
+// ---------------------------------------------------------------------------
 __device__ __forceinline__ float score_cache_key(const float* q, const std::uint16_t* key,
                                                  int head_dim) {
     float dot = 0.0f;
-    if constexpr (VEC) {
-        for (int d = 0; d < head_dim; d += 8) {
-            const uint4 packed = *reinterpret_cast<const uint4*>(key + d);
-            const float4 q0 = *reinterpret_cast<const float4*>(q + d);
-            const float4 q1 = *reinterpret_cast<const float4*>(q + d + 4);
-            dot = fmaf(q0.x, __uint_as_float(packed.x << 16), dot);
-            dot = fmaf(q0.y, __uint_as_float(packed.x & 0xffff0000u), dot);
-            dot = fmaf(q0.z, __uint_as_float(packed.y << 16), dot);
-            dot = fmaf(q0.w, __uint_as_float(packed.y & 0xffff0000u), dot);
-            dot = fmaf(q1.x, __uint_as_float(packed.z << 16), dot);
-            dot = fmaf(q1.y, __uint_as_float(packed.z & 0xffff0000u), dot);
-            dot = fmaf(q1.z, __uint_as_float(packed.w << 16), dot);
-            dot = fmaf(q1.w, __uint_as_float(packed.w & 0xffff0000u), dot);
-        }
-    } else {
-        for (int d = 0; d < head_dim; ++d) dot = fmaf(q[d], bf16_to_float(key[d]), dot);
-    }
+    for (int d = 0; d < head_dim; ++d) dot = fmaf(q[d], bf16_to_float(key[d]), dot);
     return dot;
 }
 
-template <bool VEC>
 __device__ __forceinline__ float score_block_key(const float* q, const float* key, int head_dim,
                                                  bool as_cached) {
     float dot = 0.0f;
-    if constexpr (VEC) {
-        for (int d = 0; d < head_dim; d += 4) {
-            float4 k = *reinterpret_cast<const float4*>(key + d);
-            const float4 qv = *reinterpret_cast<const float4*>(q + d);
-            if (as_cached) {
-                k.x = bf16_to_float(to_bf16(k.x));
-                k.y = bf16_to_float(to_bf16(k.y));
-                k.z = bf16_to_float(to_bf16(k.z));
-                k.w = bf16_to_float(to_bf16(k.w));
-            }
-            dot = fmaf(qv.x, k.x, dot);
-            dot = fmaf(qv.y, k.y, dot);
-            dot = fmaf(qv.z, k.z, dot);
-            dot = fmaf(qv.w, k.w, dot);
-        }
-    } else {
-        for (int d = 0; d < head_dim; ++d) {
-            float k = key[d];
-            if (as_cached) k = bf16_to_float(to_bf16(k));
-            dot = fmaf(q[d], k, dot);
-        }
+    for (int d = 0; d < head_dim; ++d) {
+        float k = key[d];
+        if (as_cached) k = bf16_to_float(to_bf16(k));
+        dot = fmaf(q[d], k, dot);
     }
     return dot;
 }
 
-template <bool VEC>
-__global__ __launch_bounds__(kMaxWaves * kWave) void attention_kernel(AttentionArguments a) {
+// The key range of one query row, and how many waves share it.  The split
+// depends on the row's key count only, not on the launch: a row of a causal
+// block then sums in the same order as the one-token call at the same
+// position, and gives the same bits.
+struct KeyRange {
+    std::int64_t first, last;
+    int active;
+};
+
+__device__ __forceinline__ KeyRange key_range(const AttentionArguments& a, std::int64_t query_row,
+                                              int waves) {
+    const std::int64_t query_position = a.context_length + query_row;
+    const bool causal = a.causal != 0;
+    KeyRange range;
+    range.first = query_position - a.sliding_window + (causal ? 1 : 0);
+    if (range.first < 0) range.first = 0;
+    range.last = query_position;
+    if (!causal) {
+        const std::int64_t end = a.context_length + a.block_rows - 1;
+        range.last =
+            a.sliding_window < end - query_position ? query_position + a.sliding_window : end;
+    }
+    const std::int64_t tiles = (range.last - range.first) / kWave + 1;
+    range.active = static_cast<int>(tiles < waves ? tiles : waves);
+    return range;
+}
+
+__global__ __launch_bounds__(kMaxWaves * kWave) void attention_generic_kernel(AttentionArguments a) {
     __shared__ __attribute__((aligned(16))) float q[kMaxHeadDim];
     __shared__ float wave_maximum[kMaxWaves];
     __shared__ float wave_denominator[kMaxWaves];
@@ -126,18 +119,15 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_kernel(AttentionA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int waves = static_cast<int>(blockDim.x >> 6);
     const int head_dim = static_cast<int>(a.head_dim);
-    const std::int64_t query_row = blockIdx.x / a.query_heads;
-    const std::int64_t query_head = blockIdx.x - query_row * a.query_heads;
-    const std::int64_t kv_head = query_head * a.kv_heads / a.query_heads;
-    const std::int64_t query_position = a.context_length + query_row;
+    // query_heads and the grid fit 32 bits (checked by the caller): no 64-bit division
+    const std::uint32_t heads = static_cast<std::uint32_t>(a.query_heads);
+    const std::int64_t query_row = blockIdx.x / heads;
+    const std::int64_t query_head = blockIdx.x % heads;
+    const std::int64_t kv_head = static_cast<std::uint32_t>(query_head) / a.heads_per_kv;
     const bool causal = a.causal != 0;
-    std::int64_t first = query_position - a.sliding_window + (causal ? 1 : 0);
-    if (first < 0) first = 0;
-    std::int64_t last = query_position;
-    if (!causal) {
-        const std::int64_t end = a.context_length + a.block_rows - 1;
-        last = a.sliding_window < end - query_position ? query_position + a.sliding_window : end;
-    }
+    const KeyRange range = key_range(a, query_row, waves);
+    const std::int64_t last = range.last;
+    const int active = range.active;
 
     const float* query = a.query + (query_row * a.query_heads + query_head) * a.head_dim;
     for (int d = tid; d < head_dim; d += blockDim.x) q[d] = query[d];
@@ -149,12 +139,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_kernel(AttentionA
 #pragma unroll
     for (int j = 0; j < kOwned; ++j) accumulator[j] = 0.0f;
 
-    // How many waves share the keys depends on this row's key count only, not
-    // on the launch: a row of a causal block then sums in the same order as
-    // the one-token call at the same position, and gives the same bits.
-    const std::int64_t tiles = (last - first) / kWave + 1;
-    const int active = static_cast<int>(tiles < waves ? tiles : waves);
-    for (std::int64_t tile = first + static_cast<std::int64_t>(wave) * kWave;
+    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
          wave < active && tile <= last; tile += static_cast<std::int64_t>(active) * kWave) {
         const std::int64_t key_position = tile + lane;
         const bool live = key_position <= last;
@@ -163,11 +148,11 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_kernel(AttentionA
             if (key_position >= a.context_length) {
                 const std::int64_t block_row = key_position - a.context_length;
                 const float* key = a.block_key + (block_row * a.kv_heads + kv_head) * a.head_dim;
-                score = score_block_key<VEC>(q, key, head_dim, causal && block_row < query_row);
+                score = score_block_key(q, key, head_dim, causal && block_row < query_row);
             } else {
                 const std::uint16_t* key = a.key_cache +
                     (key_position % a.cache_capacity) * a.cache_row_stride + kv_head * a.head_dim;
-                score = score_cache_key<VEC>(q, key, head_dim);
+                score = score_cache_key(q, key, head_dim);
             }
             score *= a.scale;
         }
@@ -242,6 +227,304 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_kernel(AttentionA
     }
 }
 
+// ---------------------------------------------------------------------------
+// Vector form: head_dim 32, 64, 128 or 256, rows 16-byte aligned, a ring of at
+// least 64 rows.  Everything moves in 16-byte pieces.  Scores: a lane owns one
+// key and reads its head_dim / 8 pieces.  Weighted sum: LANES_PER_KEY =
+// head_dim / 8 lanes share a value row; lane (g, i) = (lane / LANES_PER_KEY,
+// lane % LANES_PER_KEY) owns dimensions 8i .. 8i+7 of the keys g, g + G,
+// g + 2G ... of the tile (G = 64 / LANES_PER_KEY keys per load instruction),
+// so a tile's values arrive with LANES_PER_KEY load instructions; the G
+// partial sums of a dimension meet in a butterfly once, after the last tile.
+// A tile that lies wholly in the cache (all but the last one or two of a row)
+// runs straight-line code with up to sixteen loads per lane in flight; a tile
+// that holds block rows takes the same sums in the same order through a
+// slower path that can fetch either kind of row.
+// ---------------------------------------------------------------------------
+struct Piece {
+    float v[8];
+};
+
+__device__ __forceinline__ Piece unpack_bf16(uint4 packed) {
+    Piece p;
+    p.v[0] = __uint_as_float(packed.x << 16);
+    p.v[1] = __uint_as_float(packed.x & 0xffff0000u);
+    p.v[2] = __uint_as_float(packed.y << 16);
+    p.v[3] = __uint_as_float(packed.y & 0xffff0000u);
+    p.v[4] = __uint_as_float(packed.z << 16);
+    p.v[5] = __uint_as_float(packed.z & 0xffff0000u);
+    p.v[6] = __uint_as_float(packed.w << 16);
+    p.v[7] = __uint_as_float(packed.w & 0xffff0000u);
+    return p;
+}
+
+__device__ __forceinline__ Piece from_floats(float4 low, float4 high, bool as_cached) {
+    Piece p = {{low.x, low.y, low.z, low.w, high.x, high.y, high.z, high.w}};
+    if (as_cached) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p.v[e] = bf16_to_float(to_bf16(p.v[e]));
+    }
+    return p;
+}
+
+__device__ __forceinline__ float dot_piece(const float* q, const Piece& p, float dot) {
+    const float4 q0 = *reinterpret_cast<const float4*>(q);
+    const float4 q1 = *reinterpret_cast<const float4*>(q + 4);
+    dot = fmaf(q0.x, p.v[0], dot);
+    dot = fmaf(q0.y, p.v[1], dot);
+    dot = fmaf(q0.z, p.v[2], dot);
+    dot = fmaf(q0.w, p.v[3], dot);
+    dot = fmaf(q1.x, p.v[4], dot);
+    dot = fmaf(q1.y, p.v[5], dot);
+    dot = fmaf(q1.z, p.v[6], dot);
+    dot = fmaf(q1.w, p.v[7], dot);
+    return dot;
+}
+
+template <int LANES_PER_KEY>
+__global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(AttentionArguments a) {
+    constexpr int kPieces = LANES_PER_KEY;             // head_dim / 8
+    constexpr int kKeysPerLoad = kWave / LANES_PER_KEY;
+    __shared__ __attribute__((aligned(16))) float q[kMaxHeadDim];
+    __shared__ float wave_maximum[kMaxWaves];
+    __shared__ float wave_denominator[kMaxWaves];
+    __shared__ __attribute__((aligned(16))) float wave_accumulator[kMaxWaves][kMaxHeadDim];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
+    constexpr int head_dim = kPieces * 8;
+    // query_heads and the grid fit 32 bits (checked by the caller): no 64-bit division
+    const std::uint32_t heads = static_cast<std::uint32_t>(a.query_heads);
+    const std::int64_t query_row = blockIdx.x / heads;
+    const std::int64_t query_head = blockIdx.x % heads;
+    const std::int64_t kv_head = static_cast<std::uint32_t>(query_head) / a.heads_per_kv;
+    const bool causal = a.causal != 0;
+    const KeyRange range = key_range(a, query_row, waves);
+    const std::int64_t last = range.last;
+    const int active = range.active;
+    const std::int64_t head_offset = kv_head * head_dim;
+    const std::int64_t block_stride = a.kv_heads * head_dim;
+
+    const float* query = a.query + (query_row * a.query_heads + query_head) * head_dim;
+    for (int d = tid; d < head_dim; d += blockDim.x) q[d] = query[d];
+    __syncthreads();
+
+    // Ring rows without a division per key: the slot of a wave's first tile and
+    // of its tile-to-tile step are computed once, the rest is compare-and-subtract
+    // (the ring has at least 64 rows here).
+    const std::int64_t capacity = a.cache_capacity;
+    const std::int64_t tile_step = static_cast<std::int64_t>(active) * kWave;
+    const std::int64_t slot_step = tile_step % capacity;
+    std::int64_t tile_slot = (range.first + static_cast<std::int64_t>(wave) * kWave) % capacity;
+    const auto ring_row = [capacity](std::int64_t slot) {  // slot < 2 * capacity
+        return slot >= capacity ? slot - capacity : slot;
+    };
+
+    const int group = lane / LANES_PER_KEY;  // which key of a load instruction
+    const int piece = lane % LANES_PER_KEY;  // which 8 dimensions
+
+    float maximum = -INFINITY;
+    float denominator = 0.0f;
+    float accumulator[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) accumulator[e] = 0.0f;
+
+    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
+         wave < active && tile <= last;
+         tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
+        // Keys past the range repeat the last key of the tile with weight 0.
+        const int in_tile = static_cast<int>(last - tile < kWave - 1 ? last - tile : kWave - 1);
+        const bool live = lane <= in_tile;
+        const int my_key = live ? lane : in_tile;
+        const bool cache_only = tile + kWave - 1 < a.context_length;  // wave-uniform
+
+        // running maximum, denominator and accumulator take in the tile's scores;
+        // returns this lane's weight exp(score - maximum)
+        const auto fold = [&](float raw_score) {
+            const float score = live ? raw_score * a.scale : -INFINITY;
+            const float next_maximum = fmaxf(maximum, wave_max_f(score));
+            const float keep = expf(maximum - next_maximum);  // 0 on the first tile
+            const float weight = live ? expf(score - next_maximum) : 0.0f;
+            denominator = denominator * keep + wave_sum_f(weight);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) accumulator[e] *= keep;
+            maximum = next_maximum;
+            return weight;
+        };
+        // value row of key k of the tile (keys past the range repeat the last one)
+        const auto cached_value_piece = [&](int k) {
+            const int clamped = k < in_tile ? k : in_tile;
+            return reinterpret_cast<const uint4*>(
+                a.value_cache + ring_row(tile_slot + clamped) * a.cache_row_stride +
+                head_offset)[piece];
+        };
+
+        // Scores: lane = key.  Weighted sum: lane = (key of the load, 8 dimensions);
+        // every form adds the keys of the tile in the same order, key g, g + G, ...
+        if (cache_only) {
+            const uint4* key = reinterpret_cast<const uint4*>(
+                a.key_cache + ring_row(tile_slot + my_key) * a.cache_row_stride + head_offset);
+            if constexpr (kPieces <= 16) {
+                // the whole tile's keys and values are requested before anything is used
+                uint4 key_raw[kPieces], value_raw[kPieces];
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) key_raw[u] = key[u];
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    value_raw[u] = cached_value_piece(u * kKeysPerLoad + group);
+                }
+                float score = 0.0f;
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    score = dot_piece(q + u * 8, unpack_bf16(key_raw[u]), score);
+                }
+                const float weight = fold(score);
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    const float weight_k = __shfl(weight, u * kKeysPerLoad + group);
+                    const Piece value = unpack_bf16(value_raw[u]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        accumulator[e] = fmaf(weight_k, value.v[e], accumulator[e]);
+                    }
+                }
+            } else {
+                float score = 0.0f;
+#pragma unroll
+                for (int c = 0; c < kPieces; c += 16) {
+                    uint4 raw[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) raw[u] = key[c + u];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        score = dot_piece(q + (c + u) * 8, unpack_bf16(raw[u]), score);
+                    }
+                }
+                const float weight = fold(score);
+#pragma unroll
+                for (int t0 = 0; t0 < kPieces; t0 += 16) {
+                    uint4 raw[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        raw[u] = cached_value_piece((t0 + u) * kKeysPerLoad + group);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        const float weight_k = __shfl(weight, (t0 + u) * kKeysPerLoad + group);
+                        const Piece value = unpack_bf16(raw[u]);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            accumulator[e] = fmaf(weight_k, value.v[e], accumulator[e]);
+                        }
+                    }
+                }
+            }
+        } else {
+            float score = 0.0f;
+            const std::int64_t key_position = tile + my_key;
+            if (key_position >= a.context_length) {
+                const std::int64_t block_row = key_position - a.context_length;
+                const float4* key = reinterpret_cast<const float4*>(
+                    a.block_key + block_row * block_stride + head_offset);
+                const bool as_cached = causal && block_row < query_row;
+                for (int c = 0; c < kPieces; c += 4) {
+                    float4 raw[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) raw[u] = key[2 * c + u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        score = dot_piece(q + (c + u) * 8,
+                                          from_floats(raw[2 * u], raw[2 * u + 1], as_cached), score);
+                    }
+                }
+            } else {
+                const uint4* key = reinterpret_cast<const uint4*>(
+                    a.key_cache + ring_row(tile_slot + my_key) * a.cache_row_stride + head_offset);
+                for (int c = 0; c < kPieces; c += 4) {
+                    uint4 raw[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) raw[u] = key[c + u];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        score = dot_piece(q + (c + u) * 8, unpack_bf16(raw[u]), score);
+                    }
+                }
+            }
+            const float weight = fold(score);
+            for (int t0 = 0; t0 < kPieces; t0 += 4) {
+                if (t0 * kKeysPerLoad > in_tile) break;  // wave-uniform: only dead keys left
+                uint4 cached[4];
+                float4 low[4], high[4];
+                float weights[4];
+                bool from_block[4], as_cached[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int k = (t0 + u) * kKeysPerLoad + group;
+                    const int clamped = k < in_tile ? k : in_tile;
+                    const std::int64_t position = tile + clamped;
+                    weights[u] = __shfl(weight, k);
+                    from_block[u] = position >= a.context_length;
+                    const std::int64_t block_row = from_block[u] ? position - a.context_length : 0;
+                    as_cached[u] = causal && block_row < query_row;
+                    const std::int64_t slot = from_block[u] ? 0 : ring_row(tile_slot + clamped);
+                    cached[u] = reinterpret_cast<const uint4*>(
+                        a.value_cache + slot * a.cache_row_stride + head_offset)[piece];
+                    const float4* row = reinterpret_cast<const float4*>(
+                        a.block_value + block_row * block_stride + head_offset);
+                    low[u] = row[2 * piece];
+                    high[u] = row[2 * piece + 1];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const Piece from_cache = unpack_bf16(cached[u]);
+                    const Piece block = from_floats(low[u], high[u], as_cached[u]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float value = from_block[u] ? block.v[e] : from_cache.v[e];
+                        accumulator[e] = fmaf(weights[u], value, accumulator[e]);
+                    }
+                }
+            }
+        }
+    }
+
+    // the partial sums of the key groups meet; group 0 ends up with the totals
+#pragma unroll
+    for (int offset = LANES_PER_KEY; offset < kWave; offset <<= 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) accumulator[e] += __shfl_xor(accumulator[e], offset);
+    }
+    if (lane == 0) {
+        wave_maximum[wave] = maximum;
+        wave_denominator[wave] = denominator;
+    }
+    if (group == 0) {
+        float* target = &wave_accumulator[wave][piece * 8];
+        *reinterpret_cast<float4*>(target) =
+            make_float4(accumulator[0], accumulator[1], accumulator[2], accumulator[3]);
+        *reinterpret_cast<float4*>(target + 4) =
+            make_float4(accumulator[4], accumulator[5], accumulator[6], accumulator[7]);
+    }
+    __syncthreads();
+
+    float overall = wave_maximum[0];
+    for (int w = 1; w < active; ++w) overall = fmaxf(overall, wave_maximum[w]);
+    float total = 0.0f;
+    for (int w = 0; w < active; ++w) {
+        total = fmaf(wave_denominator[w], expf(wave_maximum[w] - overall), total);
+    }
+    float* output = a.output + (query_row * a.query_heads + query_head) * head_dim;
+    for (int d = tid; d < head_dim; d += blockDim.x) {
+        float sum = 0.0f;
+        for (int w = 0; w < active; ++w) {
+            sum = fmaf(wave_accumulator[w][d], expf(wave_maximum[w] - overall), sum);
+        }
+        output[d] = sum / total;
+    }
+}
+
 void launch_attention(const AttentionArguments& arguments, std::int64_t query_rows,
                       std::int64_t longest_key_range, hipStream_t stream) {
     std::int64_t waves = (longest_key_range + kWave - 1) / kWave;
@@ -250,14 +533,24 @@ void launch_attention(const AttentionArguments& arguments, std::int64_t query_ro
     const auto aligned = [](const void* pointer) {
         return reinterpret_cast<std::uintptr_t>(pointer) % 16 == 0;
     };
-    const bool vectors = arguments.head_dim % 8 == 0 && arguments.cache_row_stride % 8 == 0 &&
-        aligned(arguments.key_cache) && aligned(arguments.block_key);
+    const std::int64_t head_dim = arguments.head_dim;
+    const bool vectors =
+        (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
+        arguments.cache_row_stride % 8 == 0 && arguments.cache_capacity >= kWave &&
+        aligned(arguments.key_cache) && aligned(arguments.value_cache) &&
+        aligned(arguments.block_key) && aligned(arguments.block_value);
     const dim3 grid(static_cast<unsigned>(query_rows * arguments.query_heads));
     const dim3 block(static_cast<unsigned>(waves * kWave));
-    if (vectors) {
-        hipLaunchKernelGGL(attention_kernel<true>, grid, block, 0, stream, arguments);
+    if (!vectors) {
+        hipLaunchKernelGGL(attention_generic_kernel, grid, block, 0, stream, arguments);
+    } else if (head_dim == 32) {
+        hipLaunchKernelGGL(attention_vector_kernel<4>, grid, block, 0, stream, arguments);
+    } else if (head_dim == 64) {
+        hipLaunchKernelGGL(attention_vector_kernel<8>, grid, block, 0, stream, arguments);
+    } else if (head_dim == 128) {
+        hipLaunchKernelGGL(attention_vector_kernel<16>, grid, block, 0, stream, arguments);
     } else {
-        hipLaunchKernelGGL(attention_kernel<false>, grid, block, 0, stream, arguments);
+        hipLaunchKernelGGL(attention_vector_kernel<32>, grid, block, 0, stream, arguments);
     }
 }
 
@@ -274,6 +567,7 @@ void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, hipSt
     a.query_heads = d.query_heads;
     a.kv_heads = d.kv_heads;
     a.head_dim = d.head_dim;
+    a.heads_per_kv = static_cast<std::uint32_t>(d.query_heads / d.kv_heads);
     a.context_length = d.position;
     a.block_rows = 1;
     a.sliding_window = d.position - d.first_key_position + 1;
@@ -296,6 +590,7 @@ void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1&
     a.query_heads = d.query_heads;
     a.kv_heads = d.kv_heads;
     a.head_dim = d.head_dim;
+    a.heads_per_kv = static_cast<std::uint32_t>(d.query_heads / d.kv_heads);
     a.context_length = d.context_length;
     a.block_rows = d.block_rows;
     a.sliding_window = d.sliding_window;

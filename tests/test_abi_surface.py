@@ -49,6 +49,54 @@ def test_descriptor_is_72_bytes():
     assert tile_ops.PackedWeightDescriptor.cuda_stream.offset == 64
 
 
+def test_attention_and_cache_descriptors_have_the_reference_layout():
+    # sizeof / offsetof of the structs in the reference's tile_ops.h:316-339, 341-359, 461-486,
+    # as its own header compiles with g++ on x86-64
+    for struct, size, field, offset, stream in (
+            (tile_ops.GqaDecodeDescriptor, 136, "scale", 120, 128),
+            (tile_ops.CacheCommitDescriptor, 104, "cache_row_stride", 80, 96),
+            (tile_ops.BlockAttentionDescriptor, 152, "scale", 136, 144)):
+        assert ctypes.sizeof(struct) == size
+        assert getattr(struct, field).offset == offset
+        assert struct.cuda_stream.offset == stream
+
+
+def test_every_symbol_the_reference_engine_requires_is_exported(lib):
+    """tests/golden/engine_sidecar_symbols.json lists what the reference's resident engine
+    binds from its sidecar (resident_glimmer_cuda.cpp:336-495): everything it requires for
+    text decoding must be here, and optional groups must be whole where the engine insists
+    (resident_glimmer_cuda.cpp:356-359, 385-428, 453-461)."""
+    import json
+    symbols = json.loads((ROOT / "tests" / "golden" / "engine_sidecar_symbols.json").read_text())
+    assert len(symbols["required"]) == 20
+    missing = [name for name in symbols["required"] if not hasattr(lib, name)]
+    assert not missing, missing
+    exported = {name for name in symbols["optional"] if hasattr(lib, name)}
+    assert set(symbols["optional"]) - exported == {
+        "nfn_native_tile_dflash_block_attention_short_split_float32_v1",
+        "nfn_native_tile_glimmer_cache_commit_layers_bf16_v1",
+        "nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1",
+        "nfn_native_tile_glimmer_fused_decode_attention_float32_v1",
+        "nfn_native_tile_glimmer_pack_target_taps_float32_v1",
+        "nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1",
+        "nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1",
+    }
+
+    def together(*names):
+        present = [("nfn_native_tile_" + name) in exported for name in names]
+        assert all(present) or not any(present), names
+
+    together("quantize_q8_1_float32_v1", "linear_packed_weight_q8_1_float32_v1")
+    together("k_quant_mmq_abi_version", "k_quant_mmq_workspace_bytes_v1",
+             "k_quant_mmq_multi_linear_float32_v1")
+    together("k_quant_mmvq_multi_linear_float32_v1", "k_quant_mmvq_multi_linear_gated_float32_v1",
+             "k_quant_mmvq_multi_linear_swiglu_float32_v1")
+    together("glimmer_rms_norm_affine_capture_residual_float32_v1",
+             "glimmer_rms_norm_affine_add_residual_float32_v1")
+    together("glimmer_dual_rms_add_capture_mmvq_q8_float32_v1",
+             "k_quant_mmvq_multi_linear_prequantized_float32_v1")
+
+
 def _descriptor(encoding=kquant.Q4_K, out_dim=5, in_dim=512):
     return tile_ops.make_descriptor(encoding, 0x1000, out_dim, in_dim)
 
