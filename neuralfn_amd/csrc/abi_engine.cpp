@@ -23,16 +23,25 @@ bool cache_rows_fit(std::int64_t kv_heads, std::int64_t head_dim, std::int64_t r
     return kv_heads <= kLimit / head_dim && kv_heads * head_dim <= row_stride;
 }
 
+// One thread per element (or pair) and no grid-stride loop in these kernels:
+// the count must fit a grid of 256-thread workgroups.
+constexpr std::int64_t kMaxThreads = std::int64_t(0x7fffffff) * 256;
+
 bool rope_arguments_valid(const float* query, const float* key, std::int64_t rows,
                           std::int64_t query_heads, std::int64_t kv_heads, std::int64_t head_dim,
                           std::int64_t position, float theta, std::uint32_t layout) {
-    return query != nullptr && key != nullptr && rows > 0 && query_heads > 0 && kv_heads > 0 &&
-        query_heads % kv_heads == 0 && head_dim > 0 && head_dim <= kMaxHeadDim &&
-        head_dim % 2 == 0 && position >= 0 && position <= kLimit - rows &&
-        positive_finite(theta) &&
-        (layout == NFN_NATIVE_TILE_GLIMMER_ROPE_HALF_SPLIT ||
-         layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED) &&
-        rows <= kLimit / ((query_heads + kv_heads) * (head_dim / 2));
+    if (query == nullptr || key == nullptr || rows <= 0 || query_heads <= 0 || kv_heads <= 0 ||
+        query_heads % kv_heads != 0 || head_dim <= 0 || head_dim > kMaxHeadDim ||
+        head_dim % 2 != 0 || position < 0 || position > kLimit - rows || !positive_finite(theta) ||
+        (layout != NFN_NATIVE_TILE_GLIMMER_ROPE_HALF_SPLIT &&
+         layout != NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED)) {
+        return false;
+    }
+    // rows * (query_heads + kv_heads) * head_dim / 2 pairs, without overflow on the way
+    const std::int64_t half = head_dim / 2;
+    if (query_heads > kMaxThreads / half || kv_heads > query_heads) return false;
+    const std::int64_t pairs_per_row = (query_heads + kv_heads) * half;
+    return rows <= kMaxThreads / pairs_per_row;
 }
 
 bool commit_descriptor_valid(const NfnNativeTileGlimmerCacheCommitDescriptorV1* d) {
@@ -139,7 +148,7 @@ int nfn_native_tile_glimmer_gqa_decode_float32_v1(
 
 int nfn_native_tile_glimmer_cache_commit_bf16_v1(
     const NfnNativeTileGlimmerCacheCommitDescriptorV1* d) {
-    if (!commit_descriptor_valid(d)) return kInvalid;
+    if (!commit_descriptor_valid(d) || d->kv_heads * d->head_dim > kMaxThreads) return kInvalid;
     launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
                         d->kv_heads * d->head_dim, 1, d->position, d->cache_capacity,
                         d->cache_row_stride, as_stream(d->cuda_stream));
@@ -149,7 +158,7 @@ int nfn_native_tile_glimmer_cache_commit_bf16_v1(
 int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
     const NfnNativeTileGlimmerCacheCommitDescriptorV1* d, std::int64_t rows) {
     if (!commit_descriptor_valid(d) || rows <= 0 || rows > kMaxBlockRows ||
-        d->position > kLimit - rows || d->kv_heads * d->head_dim > kLimit / rows) {
+        d->position > kLimit - rows || d->kv_heads * d->head_dim > kMaxThreads / rows) {
         return kInvalid;
     }
     launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
