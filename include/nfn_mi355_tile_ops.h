@@ -87,9 +87,10 @@ int nfn_native_tile_packed_weight_dequantize_float32_v1(
     const NfnNativeTilePackedWeightDescriptorV1* descriptor,
     float* output);
 
-/* ---- generic float-activation linear, any row count (tile_ops.h:614-620).
- *      rows <= 16 run a float GEMV; larger row counts with a K-quant weight
- *      run the MFMA dequant-GEMM. ------------------------------------------ */
+/* ---- generic float-activation linear, any row count (tile_ops.h:614-620):
+ *      float weights times float activations, no quantization of the input.
+ *      It has no workspace argument, so large row counts take the same float
+ *      kernel; nfn_mi355_k_quant_gemm_float32_v1 is the matrix-core route. -- */
 int nfn_native_tile_linear_packed_weight_float32_v1(
     const NfnNativeTilePackedWeightDescriptorV1* descriptor,
     const float* input,
