@@ -362,6 +362,64 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
                         "incl. activation conversion", **result}
 
 
+def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
+    """Whole decode layers at the workload's geometry, every operator through the C ABI in the
+    engine's order (neuralfn_amd/decode_layer.py): what a token costs beyond the projections."""
+    import torch
+    from neuralfn_amd import decode_layer as dl, kquant, tile_ops
+    layers, position = 8, 5000
+    g = dl.LayerGeometry(model_dim=MODEL_DIM, query_heads=ATTN_DIM // 128, kv_heads=KV_DIM // 128,
+                         head_dim=128, ffn_dim=FFN_DIM, sliding_window=2048)
+    ones = {width: tile_ops.PackedWeight(
+        kquant.F32, 1, width, torch.ones(width, dtype=torch.float32, device=device).view(torch.uint8))
+        for width in (MODEL_DIM, 128)}
+    shapes = dict(q=(ATTN_DIM, MODEL_DIM), k=(KV_DIM, MODEL_DIM), v=(KV_DIM, MODEL_DIM),
+                  attention_gate=(ATTN_DIM, MODEL_DIM), output=(MODEL_DIM, ATTN_DIM),
+                  mlp_gate=(FFN_DIM, MODEL_DIM), mlp_up=(FFN_DIM, MODEL_DIM),
+                  mlp_down=(MODEL_DIM, FFN_DIM))
+    stack = []
+    for layer in range(layers):
+        packed = {name: random_packed_on_device(kquant.Q4_K, out_dim, in_dim, device,
+                                                1000 + 10 * layer + index)
+                  for index, (name, (out_dim, in_dim)) in enumerate(shapes.items())}
+        weights = dl.LayerWeights(
+            **packed, input_norm=ones[MODEL_DIM], q_norm=ones[128], k_norm=ones[128],
+            post_attention_norm=ones[MODEL_DIM], pre_feedforward_norm=ones[MODEL_DIM],
+            post_feedforward_norm=ones[MODEL_DIM])
+        cache = dl.LayerCache(g, device)
+        cache.keys.copy_(torch.randn(cache.keys.shape, device=device).to(torch.bfloat16).view(torch.int16))
+        cache.values.copy_(torch.randn(cache.values.shape, device=device).to(torch.bfloat16).view(torch.int16))
+        stack.append((weights, cache))
+    workspace = tile_ops.small_batch_workspace(1, FFN_DIM, device)
+    embedding = torch.from_numpy(kquant.synthetic_activations(41, 1, MODEL_DIM)).to(device)
+    zeros = torch.zeros_like(embedding)
+    last = {}
+
+    def token():
+        pending, residual, pending_norm = embedding, zeros, None
+        for weights, cache in stack:
+            pending, residual = dl.decode_layer(g, weights, cache, pending, residual, pending_norm,
+                                                position, workspace)
+            pending_norm = weights.post_feedforward_norm
+        last["hidden"] = residual
+
+    ms = time_graph(token, stream, max(5, steps // 2), max(2, warmup // 2))
+    if not bool(torch.isfinite(last["hidden"]).all()):
+        raise RuntimeError("the decode-layer chain produced a non-finite hidden state")
+    weight_bytes = sum(weights.packed_bytes() for weights, _ in stack)
+    cache_bytes = layers * 2 * g.sliding_window * g.kv_dim * 2
+    per_layer_us = ms * 1e3 / layers
+    return {
+        "workload": f"{layers} whole decode layers (Q4_K projections incl. attention gate and FFN "
+                    f"{MODEL_DIM}<->{FFN_DIM}, 2048-key local attention), one token, HIP-graph replay",
+        "us_per_layer": round(per_layer_us, 2),
+        "launches_per_layer": dl.LAUNCHES_PER_LAYER,
+        "weight_GB/s": round(weight_bytes / ms / 1e6, 1),
+        "frac_hbm": round((weight_bytes + cache_bytes) / ms / 1e6 / HBM_PEAK_GBS, 4),
+        "tokens/s_at_48_layers_without_lm_head": round(1e6 / (48 * per_layer_us), 1),
+    }
+
+
 def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
     """Four layers of attention and FFN projections with per-tensor formats drawn by seed
     from {Q4_K, Q5_K, Q6_K, Q8_0} (V, O and down at least Q5_K), at one row (decode)
@@ -542,6 +600,7 @@ def main() -> int:
                 record["lm_head"] = lm_head_extra(device, stream, args.steps, args.warmup)
                 record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
                 record["mixed_profile"] = mixed_profile_extra(device, stream, args.steps, args.warmup)
+                record["decode_layer"] = decode_layer_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
             record["extras_error"] = repr(error)
     if not args.no_cpu_baseline:

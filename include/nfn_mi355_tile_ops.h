@@ -422,6 +422,49 @@ int nfn_native_tile_glimmer_positioned_rope_batch_float32_v1(
     bool inverse,
     void* cuda_stream);
 
+/* Per-head RMS normalisation of query and key (optional [1, head_dim] weights),
+ * query *= query_scale, then the rotary embedding when apply_rope, in place, in
+ * one launch (tile_ops.h:905-943).  Equal bit for bit to
+ * rms_norm_affine(rows = heads, width = head_dim) on query and on key,
+ * scale_inplace on query and positioned_rope, which is the reference probe's rule
+ * (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:461-610).  The batch form
+ * handles rows 1..64, row r at position + r. */
+int nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1(
+    float* query,
+    float* key,
+    const NfnNativeTilePackedWeightDescriptorV1* query_norm_weight,
+    const NfnNativeTilePackedWeightDescriptorV1* key_norm_weight,
+    int64_t query_heads,
+    int64_t kv_heads,
+    int64_t head_dim,
+    float eps,
+    bool query_norm_centered,
+    bool key_norm_centered,
+    float query_scale,
+    int64_t position,
+    float theta,
+    uint32_t layout,
+    bool apply_rope,
+    void* cuda_stream);
+int nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
+    float* query,
+    float* key,
+    const NfnNativeTilePackedWeightDescriptorV1* query_norm_weight,
+    const NfnNativeTilePackedWeightDescriptorV1* key_norm_weight,
+    int64_t rows,
+    int64_t query_heads,
+    int64_t kv_heads,
+    int64_t head_dim,
+    float eps,
+    bool query_norm_centered,
+    bool key_norm_centered,
+    float query_scale,
+    int64_t position,
+    float theta,
+    uint32_t layout,
+    bool apply_rope,
+    void* cuda_stream);
+
 /* One-token causal attention of query_heads heads over kv_heads cached heads
  * (tile_ops.h:308-339, 944-945).  Keys first_key_position .. position-1 are
  * rows (p % cache_capacity) of the bf16 caches, key `position` is
@@ -480,6 +523,49 @@ int nfn_native_tile_glimmer_cache_commit_bf16_v1(
 int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
     const NfnNativeTileGlimmerCacheCommitDescriptorV1* descriptor,
     int64_t rows);
+
+/* The three dependent per-layer decode steps in one call (tile_ops.h:361-405,
+ * 946-947): qk_norm_scale_rope on query/key (in place), gqa_decode with key as
+ * the current key, and the bf16 cache commit of key/current_value at
+ * `position`.  The norm weights are embedded by value; has_*_norm_weight == 0
+ * makes the corresponding descriptor inert.  Here it is those three launches
+ * in sequence on the descriptor's stream, so it equals the separate calls bit
+ * for bit. */
+typedef struct NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version;
+    uint32_t flags;
+    uint32_t reserved0;
+    float* query;
+    float* key;
+    const float* current_value;
+    uint16_t* key_cache_bf16;
+    uint16_t* value_cache_bf16;
+    float* output;
+    NfnNativeTilePackedWeightDescriptorV1 query_norm_weight;
+    NfnNativeTilePackedWeightDescriptorV1 key_norm_weight;
+    int64_t query_heads; /* at most 256 */
+    int64_t kv_heads;
+    int64_t head_dim;
+    int64_t position;
+    int64_t first_key_position;
+    int64_t cache_capacity;
+    int64_t cache_row_stride;
+    float norm_eps;
+    float query_scale;
+    float rope_theta;
+    float attention_scale;
+    uint32_t rope_layout;
+    uint32_t has_query_norm_weight;
+    uint32_t has_key_norm_weight;
+    uint32_t query_norm_centered;
+    uint32_t key_norm_centered;
+    uint32_t apply_rope;
+    uint32_t reserved1;
+    void* cuda_stream;
+} NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1;
+int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor);
 
 /* Attention of a block of query_rows rows (positions context_length + r) over
  * the cached context and the block's own block_rows keys (tile_ops.h:445-486,

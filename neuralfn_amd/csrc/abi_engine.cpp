@@ -55,6 +55,29 @@ bool commit_descriptor_valid(const NfnNativeTileGlimmerCacheCommitDescriptorV1* 
         cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride);
 }
 
+// Shared checks of the two qk_norm_scale_rope forms and of the fused decode step.
+// `normalized_*` receive the checked weight descriptors; a null weight leaves
+// its output untouched and reports "no weight" through the returned pointers.
+bool qk_norm_arguments_valid(const float* query, const float* key, const Descriptor* query_weight,
+                             const Descriptor* key_weight, std::int64_t rows,
+                             std::int64_t query_heads, std::int64_t kv_heads,
+                             std::int64_t head_dim, float eps, float query_scale,
+                             std::int64_t position, float theta, std::uint32_t layout,
+                             Descriptor* normalized_query, Descriptor* normalized_key) {
+    if (rows > kMaxBlockRows || !positive_finite(eps) || !positive_finite(query_scale) ||
+        !rope_arguments_valid(query, key, rows, query_heads, kv_heads, head_dim, position, theta,
+                              layout) ||
+        query_heads + kv_heads > std::numeric_limits<std::int32_t>::max() / kMaxBlockRows) {
+        return false;
+    }
+    const auto weight_valid = [head_dim](const Descriptor* weight, Descriptor* normalized) {
+        return weight == nullptr ||
+            (normalize_descriptor(weight, normalized) && normalized->output_dim == 1 &&
+             normalized->input_dim == head_dim);
+    };
+    return weight_valid(query_weight, normalized_query) && weight_valid(key_weight, normalized_key);
+}
+
 }  // namespace
 
 }  // namespace nfn
@@ -123,6 +146,93 @@ int nfn_native_tile_glimmer_positioned_rope_batch_float32_v1(
     launch_rope(query, key, rows, query_heads, kv_heads, head_dim, start_position, theta,
                 layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, inverse,
                 as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
+    float* query, float* key, const Descriptor* query_norm_weight,
+    const Descriptor* key_norm_weight, std::int64_t rows, std::int64_t query_heads,
+    std::int64_t kv_heads, std::int64_t head_dim, float eps, bool query_norm_centered,
+    bool key_norm_centered, float query_scale, std::int64_t position, float theta,
+    std::uint32_t layout, bool apply_rope, void* cuda_stream) {
+    Descriptor query_weight{}, key_weight{};
+    if (!qk_norm_arguments_valid(query, key, query_norm_weight, key_norm_weight, rows, query_heads,
+                                 kv_heads, head_dim, eps, query_scale, position, theta, layout,
+                                 &query_weight, &key_weight)) {
+        return kInvalid;
+    }
+    launch_qk_norm_scale_rope(query, key, query_norm_weight != nullptr ? &query_weight : nullptr,
+                              query_norm_centered,
+                              key_norm_weight != nullptr ? &key_weight : nullptr,
+                              key_norm_centered, rows, query_heads, kv_heads, head_dim, eps,
+                              query_scale, position, theta,
+                              layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, apply_rope,
+                              as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1(
+    float* query, float* key, const Descriptor* query_norm_weight,
+    const Descriptor* key_norm_weight, std::int64_t query_heads, std::int64_t kv_heads,
+    std::int64_t head_dim, float eps, bool query_norm_centered, bool key_norm_centered,
+    float query_scale, std::int64_t position, float theta, std::uint32_t layout, bool apply_rope,
+    void* cuda_stream) {
+    return nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
+        query, key, query_norm_weight, key_norm_weight, 1, query_heads, kv_heads, head_dim, eps,
+        query_norm_centered, key_norm_centered, query_scale, position, theta, layout, apply_rope,
+        cuda_stream);
+}
+
+int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d) {
+    if (d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->current_value == nullptr ||
+        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
+        d->query_heads > 256 || d->position == kLimit || d->first_key_position < 0 ||
+        d->first_key_position > d->position || d->cache_capacity <= 0 ||
+        d->cache_row_stride <= 0 || !positive_finite(d->attention_scale) ||
+        d->has_query_norm_weight > 1 || d->has_key_norm_weight > 1 ||
+        d->query_norm_centered > 1 || d->key_norm_centered > 1 || d->apply_rope > 1) {
+        return kInvalid;
+    }
+    Descriptor query_weight{}, key_weight{};
+    const Descriptor* query_source = d->has_query_norm_weight != 0 ? &d->query_norm_weight : nullptr;
+    const Descriptor* key_source = d->has_key_norm_weight != 0 ? &d->key_norm_weight : nullptr;
+    if (!qk_norm_arguments_valid(d->query, d->key, query_source, key_source, 1, d->query_heads,
+                                 d->kv_heads, d->head_dim, d->norm_eps, d->query_scale,
+                                 d->position, d->rope_theta, d->rope_layout, &query_weight,
+                                 &key_weight) ||
+        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride)) {
+        return kInvalid;
+    }
+    const hipStream_t stream = as_stream(d->cuda_stream);
+    launch_qk_norm_scale_rope(d->query, d->key, query_source != nullptr ? &query_weight : nullptr,
+                              d->query_norm_centered != 0,
+                              key_source != nullptr ? &key_weight : nullptr,
+                              d->key_norm_centered != 0, 1, d->query_heads, d->kv_heads,
+                              d->head_dim, d->norm_eps, d->query_scale, d->position, d->rope_theta,
+                              d->rope_layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED,
+                              d->apply_rope != 0, stream);
+    NfnNativeTileGlimmerGqaDecodeDescriptorV1 attention{};
+    attention.query = d->query;
+    attention.current_key = d->key;
+    attention.current_value = d->current_value;
+    attention.key_cache_bf16 = d->key_cache_bf16;
+    attention.value_cache_bf16 = d->value_cache_bf16;
+    attention.output = d->output;
+    attention.query_heads = d->query_heads;
+    attention.kv_heads = d->kv_heads;
+    attention.head_dim = d->head_dim;
+    attention.position = d->position;
+    attention.first_key_position = d->first_key_position;
+    attention.cache_capacity = d->cache_capacity;
+    attention.cache_row_stride = d->cache_row_stride;
+    attention.scale = d->attention_scale;
+    launch_gqa_decode(attention, stream);
+    launch_cache_commit(d->key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
+                        d->kv_heads * d->head_dim, 1, d->position, d->cache_capacity,
+                        d->cache_row_stride, stream);
     return launch_status();
 }
 

@@ -123,6 +123,24 @@ __device__ __forceinline__ float bf16_to_float(std::uint32_t bits) {
     return __uint_as_float(bits << 16);
 }
 
+// One rotary pair at `position`: angle = position / theta^(2*pair/head_dim) in
+// double, [a, b] -> [a cos - b sin, b cos + a sin]
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:773-800).
+__device__ __forceinline__ void rope_rotate(float& first, float& second, std::int64_t position,
+                                            std::int64_t pair, std::int64_t head_dim, double theta,
+                                            bool inverse) {
+    const double inverse_frequency =
+        1.0 / pow(theta, static_cast<double>(2 * pair) / static_cast<double>(head_dim));
+    double angle = static_cast<double>(position) * inverse_frequency;
+    if (inverse) angle = -angle;
+    double sine, cosine;
+    sincos(angle, &sine, &cosine);
+    const float lhs = first;
+    const float rhs = second;
+    first = static_cast<float>(lhs * cosine - rhs * sine);
+    second = static_cast<float>(rhs * cosine + lhs * sine);
+}
+
 // 6-bit scale and minimum of sub-block `index` (resident_glimmer.cpp:178-186).
 __device__ __forceinline__ void k_scale_min(const std::uint8_t* scales, int index,
                                             int* scale, int* minimum) {

@@ -64,16 +64,7 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(
         : key + (row * kv_heads + head - query_heads) * head_dim;
     const std::int64_t first = interleaved ? 2 * pair : pair;
     const std::int64_t second = interleaved ? 2 * pair + 1 : pair + half;
-    const double inverse_frequency =
-        1.0 / pow(theta, static_cast<double>(2 * pair) / static_cast<double>(head_dim));
-    double angle = static_cast<double>(start_position + row) * inverse_frequency;
-    if (inverse) angle = -angle;
-    double sine, cosine;
-    sincos(angle, &sine, &cosine);
-    const float lhs = values[first];
-    const float rhs = values[second];
-    values[first] = static_cast<float>(lhs * cosine - rhs * sine);
-    values[second] = static_cast<float>(rhs * cosine + lhs * sine);
+    rope_rotate(values[first], values[second], start_position + row, pair, head_dim, theta, inverse);
 }
 
 // ---- cache commit -----------------------------------------------------------

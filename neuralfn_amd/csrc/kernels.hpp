@@ -48,6 +48,15 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
                      std::int8_t* q8_codes, float* q8_scales, float* q8_sums, std::int64_t rows,
                      std::int64_t width, float eps, hipStream_t stream);
 
+// rms.hip — per-head Q/K normalisation, query scale and rotary embedding of
+// `rows` rows in one launch; row r is at position + r.
+void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query_weight,
+                               bool query_centered, const Descriptor* key_weight,
+                               bool key_centered, std::int64_t rows, std::int64_t query_heads,
+                               std::int64_t kv_heads, std::int64_t head_dim, float eps,
+                               float query_scale, std::int64_t position, float theta,
+                               bool interleaved, bool apply_rope, hipStream_t stream);
+
 // engine_ops.hip — the small operators around the packed linears.
 // token_source: 0 = host_token, 1 = one int64 in device memory, 2 = int32 per row.
 void launch_embedding(const Descriptor& table, int token_source, std::int64_t host_token,

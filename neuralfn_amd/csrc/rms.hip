@@ -45,6 +45,36 @@ __device__ __forceinline__ float norm_scale(const NormWeight& weight, std::int64
     return scale;
 }
 
+// The scales of N columns at once.  The encoding is looked at once, outside the
+// loop, so that for float and bf16 rows (what norm weights are) the N loads are
+// plain and independent and go out together instead of one behind the other's
+// branch.
+template <int N, typename Index>
+__device__ __forceinline__ void norm_scales(const NormWeight& weight, const Index (&columns)[N],
+                                            float (&scale)[N]) {
+    if (!weight.present) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) scale[i] = 1.0f;
+        return;
+    }
+    if (weight.encoding == kEncF32) {
+        const float* values = reinterpret_cast<const float*>(weight.data);
+#pragma unroll
+        for (int i = 0; i < N; ++i) scale[i] = values[columns[i]];
+    } else if (weight.encoding == kEncBF16) {
+        const std::uint16_t* values = reinterpret_cast<const std::uint16_t*>(weight.data);
+#pragma unroll
+        for (int i = 0; i < N; ++i) scale[i] = bf16_to_float(values[columns[i]]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) scale[i] = weight_value(weight.encoding, weight.data, columns[i]);
+    }
+    if (weight.centered) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) scale[i] += 1.0f;
+    }
+}
+
 // 1 / sqrt(mean of squares + eps) of `values[0, width)`, the same number in every thread.
 __device__ __forceinline__ float inverse_rms(const float* values, std::int64_t width, float eps,
                                              float* partials) {
@@ -91,13 +121,14 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_add_capture_kernel(
     const float first_inverse = inverse_rms(source, width, first_eps, partials);
     for (std::int64_t base = threadIdx.x; base < width; base += kBatch * kRmsThreads) {
         float value[kBatch], other[kBatch], scale[kBatch];
+        std::int64_t columns[kBatch];
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const std::int64_t column = min(base + i * kRmsThreads, width - 1);
-            value[i] = source[column];
-            other[i] = residual[column];
-            scale[i] = norm_scale(first_weight, column);
+            columns[i] = min(base + i * kRmsThreads, width - 1);
+            value[i] = source[columns[i]];
+            other[i] = residual[columns[i]];
         }
+        norm_scales(first_weight, columns, scale);
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const std::int64_t column = base + i * kRmsThreads;
@@ -114,12 +145,13 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_add_capture_kernel(
     const float second_inverse = inverse_rms(hidden, width, second_eps, partials);
     for (std::int64_t base = threadIdx.x; base < width; base += kBatch * kRmsThreads) {
         float value[kBatch], scale[kBatch];
+        std::int64_t columns[kBatch];
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
-            const std::int64_t column = min(base + i * kRmsThreads, width - 1);
-            value[i] = hidden[column];
-            scale[i] = norm_scale(second_weight, column);
+            columns[i] = min(base + i * kRmsThreads, width - 1);
+            value[i] = hidden[columns[i]];
         }
+        norm_scales(second_weight, columns, scale);
 #pragma unroll
         for (int i = 0; i < kBatch; ++i) {
             const std::int64_t column = base + i * kRmsThreads;
@@ -187,15 +219,16 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
     float* normalized = normalized_output + row * width;
 
     float value[kOwned], other[kOwned], first_scale[kOwned], second_scale[kOwned];
+    int clamped[kOwned];
 #pragma unroll
     for (int i = 0; i < kOwned; ++i) {
         const int column = threadIdx.x + i * kRmsThreads;
-        const int clamped = min(column, width - 1);
-        value[i] = column < width ? source[clamped] : 0.0f;
-        other[i] = residual[clamped];
-        first_scale[i] = norm_scale(first_weight, clamped);
-        second_scale[i] = norm_scale(second_weight, clamped);
+        clamped[i] = min(column, width - 1);
+        value[i] = column < width ? source[clamped[i]] : 0.0f;
+        other[i] = residual[clamped[i]];
     }
+    norm_scales(first_weight, clamped, first_scale);
+    norm_scales(second_weight, clamped, second_scale);
 
     float square_sum = 0.0f;
 #pragma unroll
@@ -278,14 +311,15 @@ __global__ __launch_bounds__(kRmsThreads) void rms_resident_kernel(
     const std::int64_t row = blockIdx.x;
     const float* source = input + row * width;
     float value[kOwned], other[kOwned], scale[kOwned];
+    int clamped[kOwned];
 #pragma unroll
     for (int i = 0; i < kOwned; ++i) {
         const int column = threadIdx.x + i * kRmsThreads;
-        const int clamped = min(column, width - 1);
-        value[i] = column < width ? source[clamped] : 0.0f;
-        other[i] = ADD ? residual_input[row * width + clamped] : 0.0f;
-        scale[i] = norm_scale(weight, clamped);
+        clamped[i] = min(column, width - 1);
+        value[i] = column < width ? source[clamped[i]] : 0.0f;
+        other[i] = ADD ? residual_input[row * width + clamped[i]] : 0.0f;
     }
+    norm_scales(weight, clamped, scale);
     float square_sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < kOwned; ++i) square_sum = fmaf(value[i], value[i], square_sum);
@@ -331,6 +365,53 @@ __global__ __launch_bounds__(kRmsThreads) void rms_wide_kernel(
             if (residual_output != nullptr) residual_output[index] = loaded;
         }
         if constexpr (Q8) store_q8_1(q8, index, result, inside);
+    }
+}
+
+// ---- per-head Q/K normalisation, query scale and rotary embedding in one launch
+// (neuralfn/csrc/native_train/tile_ops.h:905-943; reference kernel
+// neuralfn/csrc/tile_cuda/kernels.cu:2381-2473).  One workgroup per (row, head);
+// a thread owns one column.  Each step is the arithmetic of the separate
+// operator it replaces, in the same order (rms_resident_kernel at width =
+// head_dim, the in-place scale, the rotary kernel), so the result equals the
+// three calls bit for bit.
+__global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
+    float* __restrict__ query, float* __restrict__ key, NormWeight query_weight,
+    NormWeight key_weight, int query_heads, int kv_heads, int head_dim, float eps,
+    float query_scale, std::int64_t position, double theta, bool interleaved, bool apply_rope) {
+    __shared__ float partials[kRmsThreads];
+    __shared__ float normalized[kRmsThreads];
+    const int heads_per_row = query_heads + kv_heads;
+    const int row = blockIdx.x / heads_per_row;
+    const int combined = blockIdx.x - row * heads_per_row;
+    const bool is_query = combined < query_heads;
+    float* values = is_query
+        ? query + (static_cast<std::int64_t>(row) * query_heads + combined) * head_dim
+        : key + (static_cast<std::int64_t>(row) * kv_heads + combined - query_heads) * head_dim;
+    const int column = threadIdx.x;
+    const bool inside = column < head_dim;
+    const int clamped[1] = {inside ? column : head_dim - 1};
+    const float value = inside ? values[clamped[0]] : 0.0f;
+    float scale[1];
+    norm_scales(is_query ? query_weight : key_weight, clamped, scale);
+    const float inverse = 1.0f / sqrtf(tree_total(fmaf(value, value, 0.0f), partials) /
+                                           static_cast<float>(head_dim) + eps);
+    float result = __fmul_rn(__fmul_rn(value, inverse), scale[0]);
+    if (is_query) result = __fmul_rn(result, query_scale);
+    if (!apply_rope) {
+        if (inside) values[column] = result;
+        return;
+    }
+    normalized[column] = result;
+    __syncthreads();
+    const int half = head_dim / 2;
+    if (column < half) {
+        const int first = interleaved ? 2 * column : column;
+        const int second = interleaved ? 2 * column + 1 : column + half;
+        float a = normalized[first], b = normalized[second];
+        rope_rotate(a, b, position + row, column, head_dim, theta, false);
+        values[first] = a;
+        values[second] = b;
     }
 }
 
@@ -421,6 +502,21 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
         launch_rms_variant<false, false>(input, scale, residual_input, output, residual_output, rows,
                                          width, eps, q8, stream);
     }
+}
+
+void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query_weight,
+                               bool query_centered, const Descriptor* key_weight,
+                               bool key_centered, std::int64_t rows, std::int64_t query_heads,
+                               std::int64_t kv_heads, std::int64_t head_dim, float eps,
+                               float query_scale, std::int64_t position, float theta,
+                               bool interleaved, bool apply_rope, hipStream_t stream) {
+    hipLaunchKernelGGL(qk_norm_scale_rope_kernel,
+                       dim3(static_cast<unsigned>(rows * (query_heads + kv_heads))),
+                       dim3(kRmsThreads), 0, stream, query, key,
+                       norm_weight(query_weight, query_centered),
+                       norm_weight(key_weight, key_centered), static_cast<int>(query_heads),
+                       static_cast<int>(kv_heads), static_cast<int>(head_dim), eps, query_scale,
+                       position, static_cast<double>(theta), interleaved, apply_rope);
 }
 
 }  // namespace nfn

@@ -1,0 +1,119 @@
+"""One decode step of one transformer layer as the reference's resident engine sequences it,
+every operator through the C ABI of libnfn_mi355_tile_ops.so.
+
+The arithmetic of a layer is the CPU engine's
+(neuralfn/csrc/native_gpt2/resident_glimmer.cpp:1719-1830): input norm; Q, K, V and attention-gate
+projections; per-head Q/K norm; rope; attention over the bf16 cache; sigmoid gate; output
+projection; post-attention norm + residual; pre-feed-forward norm; gate/up projections; SwiGLU;
+down projection; post-feed-forward norm + residual.  The grouping into calls is the device
+engine's: one grouped small-batch call per shared input, the sigmoid gate and SwiGLU as prologues
+of the projection that consumes them, two adjacent norms in one dual-RMS call
+(neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:2233-2585, 2913-2960), and the Q/K norms,
+rope, attention and cache commit in its fused decode-attention call (three launches here).
+Nine launches per layer and token.
+
+This is host-side sequencing for tests and benchmarks, not an engine: no sampling, no prompt
+handling, one token per step.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+from . import engine_ops, tile_ops
+from .tile_ops import PackedWeight
+
+
+@dataclass
+class LayerGeometry:
+    model_dim: int
+    query_heads: int
+    kv_heads: int
+    head_dim: int
+    ffn_dim: int
+    sliding_window: int      # keys a local layer attends to, cache capacity of the layer
+    rope_theta: float = 500000.0
+    norm_eps: float = 1e-5
+    post_norm_eps: float = 1e-5
+    interleaved_rope: bool = True  # the GGUF container's layout (resident_glimmer.cpp:1736-1743)
+
+    @property
+    def attention_dim(self) -> int:
+        return self.query_heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.kv_heads * self.head_dim
+
+
+@dataclass
+class LayerWeights:
+    """Packed projections and float norm rows (PackedWeight with encoding F32 or BF16, [1, width])."""
+    q: PackedWeight
+    k: PackedWeight
+    v: PackedWeight
+    attention_gate: PackedWeight
+    output: PackedWeight
+    mlp_gate: PackedWeight
+    mlp_up: PackedWeight
+    mlp_down: PackedWeight
+    input_norm: Optional[PackedWeight] = None
+    q_norm: Optional[PackedWeight] = None
+    k_norm: Optional[PackedWeight] = None
+    post_attention_norm: Optional[PackedWeight] = None
+    pre_feedforward_norm: Optional[PackedWeight] = None
+    post_feedforward_norm: Optional[PackedWeight] = None
+
+    def packed_bytes(self) -> int:
+        return sum(w.nbytes for w in (self.q, self.k, self.v, self.attention_gate, self.output,
+                                      self.mlp_gate, self.mlp_up, self.mlp_down))
+
+
+class LayerCache:
+    """bf16 key/value ring of one layer: [capacity, kv_heads * head_dim] each."""
+
+    def __init__(self, geometry: LayerGeometry, device):
+        import torch
+        shape = (geometry.sliding_window, geometry.kv_dim)
+        self.keys = torch.zeros(shape, dtype=torch.int16, device=device)
+        self.values = torch.zeros(shape, dtype=torch.int16, device=device)
+
+
+def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
+                 pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True):
+    """One token through one layer.
+
+    `pending` is the previous layer's down-projection output whose post-feed-forward norm and
+    residual add are still owed (for the first layer: the embedding row with `pending_norm` None
+    and `residual` zeros gives hidden = rms(embedding), the engine's embedding norm,
+    resident_glimmer.cpp:1700-1701).  Returns (down, hidden): this layer's owed pair.
+    """
+    g = geometry
+    # hidden = residual + rms(pending); normalized = rms(hidden, input_norm)
+    hidden, normalized, _ = tile_ops.dual_rms_add_capture(
+        pending, residual, pending_norm, False, weights.input_norm, False,
+        g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps)
+    query, key, value, gate = tile_ops.multi_linear(
+        [weights.q, weights.k, weights.v, weights.attention_gate], normalized, workspace)
+    # per-head norms, rope on local layers, attention and the cache commit: one call
+    query = query.view(g.query_heads, g.head_dim)
+    key = key.view(g.kv_heads, g.head_dim)
+    first = max(0, position - g.sliding_window + 1) if local else 0
+    attention = engine_ops.fused_decode_attention(
+        query, key, value.view(g.kv_heads, g.head_dim), cache.keys, cache.values, position, first,
+        g.head_dim ** -0.5, weights.q_norm, weights.k_norm, g.norm_eps, 1.0, g.rope_theta,
+        engine_ops.ROPE_INTERLEAVED if g.interleaved_rope else engine_ops.ROPE_HALF_SPLIT, local)
+    # output projection of attention * sigmoid(gate), the gate as the call's prologue
+    (projected,) = tile_ops.multi_linear([weights.output], attention.view(1, g.attention_dim),
+                                         workspace, second=gate, prologue="gated")
+    hidden, normalized, _ = tile_ops.dual_rms_add_capture(
+        projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
+        g.post_norm_eps, g.norm_eps)
+    mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
+                                             workspace)
+    (down,) = tile_ops.multi_linear([weights.mlp_down], mlp_gate, workspace, second=mlp_up,
+                                    prologue="swiglu")
+    return down, hidden
+
+
+LAUNCHES_PER_LAYER = 9

@@ -11,8 +11,9 @@ from __future__ import annotations
 import ctypes
 
 from . import tile_ops
-from .tile_ops import (BlockAttentionDescriptor, CacheCommitDescriptor, GqaDecodeDescriptor,
-                       PackedWeight, check, load)
+from .tile_ops import (BlockAttentionDescriptor, CacheCommitDescriptor,
+                       FusedDecodeAttentionDescriptor, GqaDecodeDescriptor, PackedWeight, check,
+                       load)
 
 ROPE_HALF_SPLIT = 0
 ROPE_INTERLEAVED = 1
@@ -61,6 +62,67 @@ def rope(query, key, position: int, theta: float, layout: int = ROPE_HALF_SPLIT,
     check(load().nfn_native_tile_glimmer_positioned_rope_float32_v1(
         query.data_ptr(), key.data_ptr(), query_heads, key.shape[0], head_dim, position, theta,
         layout, _stream()), "positioned_rope")
+
+
+def qk_norm_scale_rope(query, key, query_weight=None, key_weight=None, eps: float = 1e-5,
+                       query_scale: float = 1.0, position: int = 0, theta: float = 500000.0,
+                       layout: int = ROPE_HALF_SPLIT, apply_rope: bool = True,
+                       query_centered: bool = False, key_centered: bool = False) -> None:
+    """In place: per-head RMS norm, query scale, rope.  query [heads, head_dim] or
+    [rows, heads, head_dim] (then key [rows, kv_heads, head_dim], row r at position + r)."""
+    stream = _stream()
+    q_descriptor = query_weight.descriptor(stream) if query_weight is not None else None
+    k_descriptor = key_weight.descriptor(stream) if key_weight is not None else None
+    q_pointer = ctypes.byref(q_descriptor) if q_descriptor is not None else None
+    k_pointer = ctypes.byref(k_descriptor) if k_descriptor is not None else None
+    if query.dim() == 3:
+        rows, query_heads, head_dim = query.shape
+        check(load().nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
+            query.data_ptr(), key.data_ptr(), q_pointer, k_pointer, rows, query_heads,
+            key.shape[1], head_dim, eps, query_centered, key_centered, query_scale, position,
+            theta, layout, apply_rope, stream), "qk_norm_scale_rope_batch")
+        return
+    query_heads, head_dim = query.shape
+    check(load().nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1(
+        query.data_ptr(), key.data_ptr(), q_pointer, k_pointer, query_heads, key.shape[0],
+        head_dim, eps, query_centered, key_centered, query_scale, position, theta, layout,
+        apply_rope, stream), "qk_norm_scale_rope")
+
+
+def fused_decode_attention(query, key, value, key_cache, value_cache, position: int,
+                           first_key_position: int, attention_scale: float, query_weight=None,
+                           key_weight=None, eps: float = 1e-5, query_scale: float = 1.0,
+                           theta: float = 500000.0, layout: int = ROPE_HALF_SPLIT,
+                           apply_rope: bool = True, out=None):
+    """qk_norm_scale_rope (in place on query/key), one-token attention, cache commit."""
+    import torch
+    if out is None:
+        out = torch.empty_like(query)
+    stream = _stream()
+    d = FusedDecodeAttentionDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.query, d.key, d.current_value = query.data_ptr(), key.data_ptr(), value.data_ptr()
+    d.key_cache_bf16, d.value_cache_bf16 = key_cache.data_ptr(), value_cache.data_ptr()
+    d.output = out.data_ptr()
+    if query_weight is not None:
+        d.query_norm_weight = query_weight.descriptor(stream)
+        d.has_query_norm_weight = 1
+    if key_weight is not None:
+        d.key_norm_weight = key_weight.descriptor(stream)
+        d.has_key_norm_weight = 1
+    d.query_heads, d.head_dim = query.shape
+    d.kv_heads = key.shape[0]
+    d.position, d.first_key_position = position, first_key_position
+    d.cache_capacity, d.cache_row_stride = key_cache.shape
+    d.norm_eps, d.query_scale, d.rope_theta = eps, query_scale, theta
+    d.attention_scale = attention_scale
+    d.rope_layout = layout
+    d.apply_rope = 1 if apply_rope else 0
+    d.cuda_stream = stream
+    check(load().nfn_native_tile_glimmer_fused_decode_attention_float32_v1(ctypes.byref(d)),
+          "fused_decode_attention")
+    return out
 
 
 def gqa_decode(query, current_key, current_value, key_cache, value_cache, position: int,

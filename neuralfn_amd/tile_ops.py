@@ -87,6 +87,23 @@ class BlockAttentionDescriptor(ctypes.Structure):
     ]
 
 
+class FusedDecodeAttentionDescriptor(ctypes.Structure):
+    """NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:373-405)."""
+
+    _fields_ = [
+        ("struct_size", _U32), ("version", _U32), ("flags", _U32), ("reserved0", _U32),
+        ("query", _P), ("key", _P), ("current_value", _P),
+        ("key_cache_bf16", _P), ("value_cache_bf16", _P), ("output", _P),
+        ("query_norm_weight", PackedWeightDescriptor), ("key_norm_weight", PackedWeightDescriptor),
+        ("query_heads", _I64), ("kv_heads", _I64), ("head_dim", _I64), ("position", _I64),
+        ("first_key_position", _I64), ("cache_capacity", _I64), ("cache_row_stride", _I64),
+        ("norm_eps", _F32), ("query_scale", _F32), ("rope_theta", _F32), ("attention_scale", _F32),
+        ("rope_layout", _U32), ("has_query_norm_weight", _U32), ("has_key_norm_weight", _U32),
+        ("query_norm_centered", _U32), ("key_norm_centered", _U32), ("apply_rope", _U32),
+        ("reserved1", _U32), ("cuda_stream", _P),
+    ]
+
+
 _DESC = ctypes.POINTER(PackedWeightDescriptor)
 _DESC_ARRAY = ctypes.POINTER(_DESC)
 _PTR_ARRAY = ctypes.POINTER(ctypes.c_void_p)
@@ -159,6 +176,14 @@ SIGNATURES = {
         ctypes.c_int, [_P, _P, _I64, _I64, _I64, _I64, _F32, _U32, _P]),
     "nfn_native_tile_glimmer_positioned_rope_batch_float32_v1": (
         ctypes.c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _F32, _U32, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1": (
+        ctypes.c_int, [_P, _P, _DESC, _DESC, _I64, _I64, _I64, _F32, ctypes.c_bool, ctypes.c_bool,
+                       _F32, _I64, _F32, _U32, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1": (
+        ctypes.c_int, [_P, _P, _DESC, _DESC, _I64, _I64, _I64, _I64, _F32, ctypes.c_bool,
+                       ctypes.c_bool, _F32, _I64, _F32, _U32, ctypes.c_bool, _P]),
+    "nfn_native_tile_glimmer_fused_decode_attention_float32_v1": (
+        ctypes.c_int, [ctypes.POINTER(FusedDecodeAttentionDescriptor)]),
     "nfn_native_tile_glimmer_gqa_decode_float32_v1": (
         ctypes.c_int, [ctypes.POINTER(GqaDecodeDescriptor)]),
     "nfn_native_tile_glimmer_cache_commit_bf16_v1": (

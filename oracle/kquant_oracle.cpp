@@ -724,4 +724,25 @@ void nfo_logit_transform(float* logits, std::int64_t count, double multiplier, d
     }
 }
 
+// Per-head Q/K normalisation in double
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:746-771): every head of
+// `values` [heads, head_dim] is divided by its root mean square and multiplied
+// by the learned row (or 1) and by `scalar`, one rounding at the end.  Pinned by
+// the compiled reference's qk_norm_in_place.
+void nfo_qk_norm(float* values, std::int64_t heads, std::int64_t head_dim, const float* weight,
+                 double epsilon, double scalar) {
+    for (std::int64_t head = 0; head < heads; ++head) {
+        float* row = values + head * head_dim;
+        double squares = 0.0;
+        for (std::int64_t dim = 0; dim < head_dim; ++dim) {
+            squares += static_cast<double>(row[dim]) * row[dim];
+        }
+        const double inverse = 1.0 / std::sqrt(squares / static_cast<double>(head_dim) + epsilon);
+        for (std::int64_t dim = 0; dim < head_dim; ++dim) {
+            const double learned = weight == nullptr ? 1.0 : weight[dim];
+            row[dim] = static_cast<float>(static_cast<double>(row[dim]) * inverse * learned * scalar);
+        }
+    }
+}
+
 }  // extern "C"

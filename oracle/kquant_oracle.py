@@ -81,6 +81,8 @@ def lib() -> ctypes.CDLL:
         o.nfo_block_attention.restype = None
         o.nfo_logit_transform.argtypes = [_P, _I64, ctypes.c_double, ctypes.c_double]
         o.nfo_logit_transform.restype = None
+        o.nfo_qk_norm.argtypes = [_P, _I64, _I64, _P, ctypes.c_double, ctypes.c_double]
+        o.nfo_qk_norm.restype = None
         _oracle = o
     return _oracle
 
@@ -109,6 +111,8 @@ def ref() -> ctypes.CDLL:
         r.nfr_argmax.restype = _I64
         r.nfr_apply_rope.argtypes = [_P, _I64, _I64, _I64, ctypes.c_double, ctypes.c_int]
         r.nfr_apply_rope.restype = ctypes.c_int
+        r.nfr_qk_norm.argtypes = [_P, _I64, _I64, _P, ctypes.c_double, ctypes.c_double]
+        r.nfr_qk_norm.restype = ctypes.c_int
         _ref = r
     return _ref
 
@@ -281,6 +285,15 @@ def rope(values: np.ndarray, position: int, theta: float, interleaved: bool = Fa
     return out
 
 
+def qk_norm(values: np.ndarray, weight=None, epsilon: float = 1e-5, scalar: float = 1.0):
+    """values [heads, head_dim], each head RMS-normalised, times the weight row and `scalar`."""
+    out = np.array(values, dtype=np.float32, order="C", copy=True)
+    heads, head_dim = out.shape
+    _keep, pointer = _optional(weight)
+    lib().nfo_qk_norm(out.ctypes.data, heads, head_dim, pointer, float(epsilon), float(scalar))
+    return out
+
+
 def to_bf16(values: np.ndarray) -> np.ndarray:
     """float32 -> bf16 bits (uint16), round to nearest even, vectorised restatement of nfo_to_bf16."""
     bits = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32)
@@ -368,6 +381,17 @@ def ref_linear(encoding: int, packed: np.ndarray, output_dim: int, input_dim: in
                               x.ctypes.data, x.shape[0], out.ctypes.data)
     if status:
         raise ValueError(f"reference linear status {status}")
+    return out
+
+
+def ref_qk_norm(values: np.ndarray, weight=None, epsilon: float = 1e-5, scalar: float = 1.0):
+    out = np.array(values, dtype=np.float32, order="C", copy=True)
+    heads, head_dim = out.shape
+    _keep, pointer = _optional(weight)
+    status = ref().nfr_qk_norm(out.ctypes.data, heads, head_dim, pointer, float(epsilon),
+                               float(scalar))
+    if status:
+        raise ValueError(f"reference qk_norm status {status}")
     return out
 
 

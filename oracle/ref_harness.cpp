@@ -130,4 +130,26 @@ int nfr_apply_rope(float* values, std::int64_t heads, std::int64_t head_dim, std
     return 0;
 }
 
+// The reference's CPU per-head norm (resident_glimmer.cpp:746-771) with an
+// optional F32 weight row.
+int nfr_qk_norm(float* values, std::int64_t heads, std::int64_t head_dim, const float* weight,
+                double epsilon, double scalar) {
+    View view;
+    if (weight != nullptr &&
+        !make_view(0, reinterpret_cast<const std::uint8_t*>(weight), 1, head_dim, &view)) {
+        return 1;
+    }
+    const std::atomic<bool> cancelled{false};
+    try {
+        std::vector<float> buffer(values, values + heads * head_dim);
+        neuralfn::resident_glimmer::qk_norm_in_place(&buffer, heads, head_dim,
+                                                     weight != nullptr ? &view : nullptr, epsilon,
+                                                     scalar, cancelled);
+        std::copy(buffer.begin(), buffer.end(), values);
+    } catch (const std::exception&) {
+        return 2;
+    }
+    return 0;
+}
+
 }  // extern "C"

@@ -50,12 +50,13 @@ def test_descriptor_is_72_bytes():
 
 
 def test_attention_and_cache_descriptors_have_the_reference_layout():
-    # sizeof / offsetof of the structs in the reference's tile_ops.h:316-339, 341-359, 461-486,
+    # sizeof / offsetof of the structs in the reference's tile_ops.h:316-339, 341-359, 373-405, 461-486,
     # as its own header compiles with g++ on x86-64
     for struct, size, field, offset, stream in (
             (tile_ops.GqaDecodeDescriptor, 136, "scale", 120, 128),
             (tile_ops.CacheCommitDescriptor, 104, "cache_row_stride", 80, 96),
-            (tile_ops.BlockAttentionDescriptor, 152, "scale", 136, 144)):
+            (tile_ops.BlockAttentionDescriptor, 152, "scale", 136, 144),
+            (tile_ops.FusedDecodeAttentionDescriptor, 320, "query_heads", 208, 312)):
         assert ctypes.sizeof(struct) == size
         assert getattr(struct, field).offset == offset
         assert struct.cuda_stream.offset == stream
@@ -76,10 +77,7 @@ def test_every_symbol_the_reference_engine_requires_is_exported(lib):
         "nfn_native_tile_dflash_block_attention_short_split_float32_v1",
         "nfn_native_tile_glimmer_cache_commit_layers_bf16_v1",
         "nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1",
-        "nfn_native_tile_glimmer_fused_decode_attention_float32_v1",
         "nfn_native_tile_glimmer_pack_target_taps_float32_v1",
-        "nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1",
-        "nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1",
     }
 
     def together(*names):

@@ -407,3 +407,218 @@ def test_logit_transform_add_scale(cuda, oracle):
     assert lib.nfn_native_tile_glimmer_logit_transform_float32_v1(values.data_ptr(), 4, 1.0, float("inf"), None) == 1
     assert lib.nfn_native_tile_add_float32(values.data_ptr(), values.data_ptr(), values.data_ptr(), 0, None) == 1
     assert lib.nfn_native_tile_scale_inplace_float32(None, 4, 1.0, None) == 1
+
+
+# ---- fused per-head norm + scale + rope, fused decode attention ---------------------------------------
+
+def _norm_row(values):
+    return tile_ops.PackedWeight.from_numpy(kquant.F32, values.view(np.uint8).copy(), 1, values.size)
+
+
+@pytest.mark.parametrize("apply_rope", [False, True])
+@pytest.mark.parametrize("weights", ["none", "f32", "f32_centered"])
+def test_qk_norm_scale_rope_equals_the_three_separate_calls(cuda, oracle, weights, apply_rope):
+    # probe :461-610: the fused result is the unfused composition bit for bit
+    query_heads, kv_heads, head_dim = 32, 2, 128
+    eps, query_scale, position, theta = 1e-5, 3.87, 2051, 500000.0
+    query = (((np.arange(query_heads * head_dim) * 31 + 11) % 257 - 128) / np.float32(73.0)).astype(np.float32)
+    key = (((np.arange(kv_heads * head_dim) * 23 + 5) % 193 - 96) / np.float32(61.0)).astype(np.float32)
+    query, key = query.reshape(query_heads, head_dim), key.reshape(kv_heads, head_dim)
+    rng = np.random.default_rng(31)
+    q_row = (0.1 * rng.standard_normal(head_dim)).astype(np.float32) + (0 if weights == "f32_centered" else 1)
+    k_row = (0.1 * rng.standard_normal(head_dim)).astype(np.float32) + (0 if weights == "f32_centered" else 1)
+    q_weight = None if weights == "none" else _norm_row(q_row.astype(np.float32))
+    k_weight = None if weights == "none" else _norm_row(k_row.astype(np.float32))
+    centered = weights == "f32_centered"
+
+    baseline_q = tile_ops.rms_norm(to_device(query, cuda), q_weight, centered, eps)["output"]
+    baseline_k = tile_ops.rms_norm(to_device(key, cuda), k_weight, centered, eps)["output"]
+    engine_ops.scale_inplace(baseline_q, query_scale)
+    if apply_rope:
+        engine_ops.rope(baseline_q, baseline_k, position, theta)
+    fused_q, fused_k = to_device(query, cuda), to_device(key, cuda)
+    engine_ops.qk_norm_scale_rope(fused_q, fused_k, q_weight, k_weight, eps, query_scale, position,
+                                  theta, engine_ops.ROPE_HALF_SPLIT, apply_rope, centered, centered)
+    assert_bits_equal(fused_q, baseline_q, "query")
+    assert_bits_equal(fused_k, baseline_k, "key")
+
+    # and the CPU engine's double-precision statement of the same thing
+    scale_q = None if weights == "none" else (q_row + 1 if centered else q_row).astype(np.float32)
+    scale_k = None if weights == "none" else (k_row + 1 if centered else k_row).astype(np.float32)
+    expected_q = oracle.qk_norm(query, scale_q, eps, query_scale)
+    expected_k = oracle.qk_norm(key, scale_k, eps, 1.0)
+    if apply_rope:
+        expected_q = oracle.rope(expected_q, position, theta)
+        expected_k = oracle.rope(expected_k, position, theta)
+    assert np.abs(fused_q.cpu().numpy() - expected_q).max() <= 4e-6 * np.abs(expected_q).max()
+    assert np.abs(fused_k.cpu().numpy() - expected_k).max() <= 4e-6 * np.abs(expected_k).max()
+
+
+def test_qk_norm_scale_rope_batch_rows_and_fail_closed(cuda):
+    rng = np.random.default_rng(32)
+    rows, query_heads, kv_heads, head_dim = 5, 6, 3, 64
+    query = rng.standard_normal((rows, query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((rows, kv_heads, head_dim)).astype(np.float32)
+    q, k = to_device(query, cuda), to_device(key, cuda)
+    engine_ops.qk_norm_scale_rope(q, k, None, None, 1e-6, 0.5, 700, 10000.0,
+                                  engine_ops.ROPE_INTERLEAVED, True)
+    for row in range(rows):
+        q1, k1 = to_device(query[row], cuda), to_device(key[row], cuda)
+        engine_ops.qk_norm_scale_rope(q1, k1, None, None, 1e-6, 0.5, 700 + row, 10000.0,
+                                      engine_ops.ROPE_INTERLEAVED, True)
+        assert_bits_equal(q[row], q1, f"query row {row}")
+        assert_bits_equal(k[row], k1, f"key row {row}")
+    lib = tile_ops.load()
+    good = [q.data_ptr(), k.data_ptr(), None, None, rows, query_heads, kv_heads, head_dim, 1e-6, False,
+            False, 0.5, 700, 10000.0, 0, True, None]
+    call = lib.nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1
+    assert call(*good) == 0
+    for index, bad in ((0, None), (1, None), (4, 0), (4, 65), (5, 4), (7, 63), (7, 258), (8, 0.0),
+                       (11, 0.0), (11, float("inf")), (12, -1), (13, float("nan")), (14, 2)):
+        arguments = list(good)
+        arguments[index] = bad
+        assert call(*arguments) == 1, (index, bad)
+    wrong_width = _norm_row(np.ones(32, dtype=np.float32)).descriptor(0)
+    arguments = list(good)
+    arguments[2] = ctypes.byref(wrong_width)
+    assert call(*arguments) == 1
+    torch_().cuda.synchronize()
+
+
+@pytest.mark.parametrize("apply_rope", [False, True])
+def test_fused_decode_attention_equals_the_separate_calls(cuda, oracle, apply_rope):
+    rng = np.random.default_rng(33)
+    query_heads, kv_heads, head_dim, capacity, position = 32, 2, 128, 2048, 4100
+    first = position - capacity + 1 if apply_rope else 2500
+    stride = kv_heads * head_dim
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    keys = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    values = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    q_weight = _norm_row((1.0 + 0.1 * rng.standard_normal(head_dim)).astype(np.float32))
+    k_weight = _norm_row((1.0 + 0.1 * rng.standard_normal(head_dim)).astype(np.float32))
+    scale = head_dim ** -0.5
+
+    q1, k1, v1 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc1, vc1 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    engine_ops.qk_norm_scale_rope(q1, k1, q_weight, k_weight, 1e-5, 1.0, position, 500000.0,
+                                  engine_ops.ROPE_INTERLEAVED, apply_rope)
+    separate = engine_ops.gqa_decode(q1, k1, v1, kc1, vc1, position, first, scale)
+    engine_ops.cache_commit(k1, v1, kc1, vc1, position)
+
+    q2, k2, v2 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc2, vc2 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    fused = engine_ops.fused_decode_attention(q2, k2, v2, kc2, vc2, position, first, scale, q_weight,
+                                              k_weight, 1e-5, 1.0, 500000.0,
+                                              engine_ops.ROPE_INTERLEAVED, apply_rope)
+    assert_bits_equal(fused, separate, "attention output")
+    assert_bits_equal(q2, q1, "query in place")
+    assert_bits_equal(k2, k1, "key in place")
+    assert np.array_equal(bits_of(kc2), bits_of(kc1)) and np.array_equal(bits_of(vc2), bits_of(vc1))
+    assert np.array_equal(bits_of(kc2)[position % capacity], oracle.to_bf16(k1.cpu().numpy().reshape(-1)))
+    lib = tile_ops.load()
+    assert lib.nfn_native_tile_glimmer_fused_decode_attention_float32_v1(None) == 1
+    empty = tile_ops.FusedDecodeAttentionDescriptor()
+    assert lib.nfn_native_tile_glimmer_fused_decode_attention_float32_v1(ctypes.byref(empty)) == 1
+
+
+# ---- a whole decode layer ---------------------------------------------------------------------------
+
+def test_two_decode_layers_against_the_cpu_engine_arithmetic(cuda, oracle):
+    """neuralfn_amd/decode_layer.py sequences every operator of a layer through the C ABI; the
+    same layer in the oracle's double-precision operators (resident_glimmer.cpp:1719-1830) must
+    agree at the linear path's tolerance."""
+    from neuralfn_amd import decode_layer as dl
+    rng = np.random.default_rng(21)
+    g = dl.LayerGeometry(model_dim=512, query_heads=4, kv_heads=2, head_dim=64, ffn_dim=768,
+                         sliding_window=128)
+    position = 200  # the ring has wrapped
+    formats = dict(q=kquant.Q4_K, k=kquant.Q5_K, v=kquant.Q6_K, attention_gate=kquant.Q4_K,
+                   output=kquant.Q5_K, mlp_gate=kquant.Q4_K, mlp_up=kquant.Q8_0, mlp_down=kquant.Q6_K)
+    shapes = dict(q=(g.attention_dim, g.model_dim), k=(g.kv_dim, g.model_dim),
+                  v=(g.kv_dim, g.model_dim), attention_gate=(g.attention_dim, g.model_dim),
+                  output=(g.model_dim, g.attention_dim), mlp_gate=(g.ffn_dim, g.model_dim),
+                  mlp_up=(g.ffn_dim, g.model_dim), mlp_down=(g.model_dim, g.ffn_dim))
+    norms = dict(input_norm=g.model_dim, q_norm=g.head_dim, k_norm=g.head_dim,
+                 post_attention_norm=g.model_dim, pre_feedforward_norm=g.model_dim,
+                 post_feedforward_norm=g.model_dim)
+
+    host_layers, device_layers, host_caches, device_caches = [], [], [], []
+    for _ in range(2):
+        host, device = {}, {}
+        for name, (out_dim, in_dim) in shapes.items():
+            packed = kquant.quantize(formats[name],
+                                     (rng.standard_normal((out_dim, in_dim)) * 0.05).astype(np.float32))
+            host[name] = (formats[name], packed, out_dim, in_dim)
+            device[name] = tile_ops.PackedWeight.from_numpy(formats[name], packed, out_dim, in_dim)
+        for name, width in norms.items():
+            row = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+            host[name] = row
+            device[name] = tile_ops.PackedWeight.from_numpy(kquant.F32, row.view(np.uint8).copy(), 1, width)
+        host_layers.append(host)
+        device_layers.append(dl.LayerWeights(**device))
+        keys = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+        values = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+        host_caches.append((keys.copy(), values.copy()))
+        cache = dl.LayerCache(g, cuda)
+        cache.keys.copy_(bf16_tensor(keys, cuda))
+        cache.values.copy_(bf16_tensor(values, cuda))
+        device_caches.append(cache)
+
+    embedding = rng.standard_normal((1, g.model_dim)).astype(np.float32)
+
+    # ---- the library ----
+    workspace = tile_ops.small_batch_workspace(1, max(g.model_dim, g.ffn_dim))
+    pending, residual, pending_norm = to_device(embedding, cuda), to_device(np.zeros_like(embedding), cuda), None
+    for weights, cache in zip(device_layers, device_caches):
+        pending, residual = dl.decode_layer(g, weights, cache, pending, residual, pending_norm,
+                                            position, workspace)
+        pending_norm = weights.post_feedforward_norm
+    actual_down, actual_hidden = pending.cpu().numpy(), residual.cpu().numpy()
+
+    # ---- the oracle ----
+    def linear(entry, x):
+        encoding, packed, out_dim, in_dim = entry
+        return oracle.linear(encoding, packed, out_dim, in_dim, x.reshape(1, in_dim))[0]
+
+    owed, hidden_before, owed_norm = embedding[0], np.zeros(g.model_dim, dtype=np.float32), None
+    for host, (keys, values) in zip(host_layers, host_caches):
+        eps = g.post_norm_eps if owed_norm is not None else g.norm_eps
+        hidden = hidden_before + oracle.rms_norm(owed, owed_norm, False, eps)
+        normalized = oracle.rms_norm(hidden, host["input_norm"], False, g.norm_eps)
+        query = linear(host["q"], normalized).reshape(g.query_heads, g.head_dim)
+        key = linear(host["k"], normalized).reshape(g.kv_heads, g.head_dim)
+        value = linear(host["v"], normalized).reshape(g.kv_heads, g.head_dim)
+        gate = linear(host["attention_gate"], normalized)
+        query = np.stack([oracle.rms_norm(row, host["q_norm"], False, g.norm_eps) for row in query])
+        key = np.stack([oracle.rms_norm(row, host["k_norm"], False, g.norm_eps) for row in key])
+        query = oracle.rope(query, position, g.rope_theta, True)
+        key = oracle.rope(key, position, g.rope_theta, True)
+        attention = oracle.gqa_decode(query, key, value, keys, values, position,
+                                      position - g.sliding_window + 1, g.head_dim ** -0.5)
+        gated = oracle.sigmoid_gate(attention.reshape(-1), gate)
+        projected = linear(host["output"], gated)
+        hidden = hidden + oracle.rms_norm(projected, host["post_attention_norm"], False, g.post_norm_eps)
+        normalized = oracle.rms_norm(hidden, host["pre_feedforward_norm"], False, g.norm_eps)
+        activated = oracle.swiglu(linear(host["mlp_gate"], normalized), linear(host["mlp_up"], normalized))
+        owed, hidden_before, owed_norm = linear(host["mlp_down"], activated), hidden, host["post_feedforward_norm"]
+        # what the commit must have left in the ring
+        keys[position % g.sliding_window] = oracle.to_bf16(key.reshape(-1))
+        values[position % g.sliding_window] = oracle.to_bf16(value.reshape(-1))
+
+    def error(actual, expected):
+        return float(np.max(np.abs(actual.reshape(-1) - expected)) / np.max(np.abs(expected)))
+
+    assert error(actual_hidden, hidden_before) <= 2e-3
+    assert error(actual_down, owed) <= 4e-3  # two layers of 2e-3 operators in sequence
+    # The committed rows: bf16 of values that carry the projections' error, so a rounding step
+    # (2^-8 relative) apart at most, and exact for most entries.
+    for cache, (keys, values) in zip(device_caches, host_caches):
+        slot = position % g.sliding_window
+        for device_rows, host_rows in ((cache.keys, keys), (cache.values, values)):
+            committed = oracle.bf16_to_float(bits_of(device_rows)[slot])
+            expected = oracle.bf16_to_float(host_rows[slot])
+            assert np.max(np.abs(committed - expected)) <= 2e-3 * np.max(np.abs(expected)) + 2.0 ** -8 * np.max(np.abs(expected))
+        untouched = np.delete(np.arange(g.sliding_window), slot)
+        assert np.array_equal(bits_of(cache.keys)[untouched], keys[untouched])

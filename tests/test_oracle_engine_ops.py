@@ -33,6 +33,31 @@ def test_rope_equals_the_compiled_reference(oracle, interleaved):
                               oracle.ref_apply_rope(x, position, theta, interleaved))
 
 
+@needs_ref
+def test_qk_norm_equals_the_compiled_reference(oracle):
+    rng = np.random.default_rng(10)
+    for heads, head_dim in ((32, 128), (2, 128), (5, 64), (3, 6)):
+        x = (rng.standard_normal((heads, head_dim)) * 3.0).astype(np.float32)
+        weight = (1.0 + 0.2 * rng.standard_normal(head_dim)).astype(np.float32)
+        assert np.array_equal(oracle.qk_norm(x, None, 1e-5, 1.0), oracle.ref_qk_norm(x, None, 1e-5, 1.0))
+        assert np.array_equal(oracle.qk_norm(x, weight, 1e-6, 3.87),
+                              oracle.ref_qk_norm(x, weight, 1e-6, 3.87))
+
+
+def test_qk_norm_closed_forms(oracle):
+    # a head of equal values v normalises to sign(v) / sqrt(1 + eps / v^2); scaling the input changes nothing
+    x = np.full((2, 64), 3.0, dtype=np.float32)
+    x[1] = -0.5
+    y = oracle.qk_norm(x, None, 1e-5, 2.0)
+    assert np.allclose(y[0], 2.0 / np.sqrt(1.0 + 1e-5 / 9.0), rtol=1e-7)
+    assert np.allclose(y[1], -2.0 / np.sqrt(1.0 + 1e-5 / 0.25), rtol=1e-7)
+    rng = np.random.default_rng(11)
+    z = rng.standard_normal((3, 128)).astype(np.float32)
+    unit = oracle.qk_norm(z, None, 1e-12, 1.0)
+    assert np.allclose((unit.astype(np.float64) ** 2).mean(axis=1), 1.0, rtol=1e-6)
+    assert np.allclose(oracle.qk_norm(z * 8.0, None, 1e-12, 1.0), unit, rtol=1e-6)
+
+
 def test_rope_is_a_rotation(oracle):
     rng = np.random.default_rng(4)
     x = rng.standard_normal((4, 128)).astype(np.float32)
