@@ -395,29 +395,36 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
     zeros = torch.zeros_like(embedding)
     last = {}
 
-    def token():
-        pending, residual, pending_norm = embedding, zeros, None
-        for weights, cache in stack:
-            pending, residual = dl.decode_layer(g, weights, cache, pending, residual, pending_norm,
-                                                position, workspace)
-            pending_norm = weights.post_feedforward_norm
-        last["hidden"] = residual
-
-    ms = time_graph(token, stream, max(5, steps // 2), max(2, warmup // 2))
-    if not bool(torch.isfinite(last["hidden"]).all()):
-        raise RuntimeError("the decode-layer chain produced a non-finite hidden state")
     weight_bytes = sum(weights.packed_bytes() for weights, _ in stack)
     cache_bytes = layers * 2 * g.sliding_window * g.kv_dim * 2
-    per_layer_us = ms * 1e3 / layers
-    return {
+    result = {
         "workload": f"{layers} whole decode layers (Q4_K projections incl. attention gate and FFN "
-                    f"{MODEL_DIM}<->{FFN_DIM}, 2048-key local attention), one token, HIP-graph replay",
-        "us_per_layer": round(per_layer_us, 2),
-        "launches_per_layer": dl.LAUNCHES_PER_LAYER,
-        "weight_GB/s": round(weight_bytes / ms / 1e6, 1),
-        "frac_hbm": round((weight_bytes + cache_bytes) / ms / 1e6 / HBM_PEAK_GBS, 4),
-        "tokens/s_at_48_layers_without_lm_head": round(1e6 / (48 * per_layer_us), 1),
-    }
+                    f"{MODEL_DIM}<->{FFN_DIM}, 2048-key local attention), one token, HIP-graph replay"}
+    from neuralfn_amd import engine_ops
+    forms = (("reference_fused_attention", None, dl.LAUNCHES_PER_LAYER),
+             ("split_attention", engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim, device),
+              dl.LAUNCHES_PER_LAYER_SPLIT))
+    for name, attention_workspace, launches in forms:
+        def token():
+            pending, residual, pending_norm = embedding, zeros, None
+            for weights, cache in stack:
+                pending, residual = dl.decode_layer(g, weights, cache, pending, residual,
+                                                    pending_norm, position, workspace, True,
+                                                    attention_workspace)
+                pending_norm = weights.post_feedforward_norm
+            last["hidden"] = residual
+
+        ms = time_graph(token, stream, max(5, steps // 2), max(2, warmup // 2))
+        if not bool(torch.isfinite(last["hidden"]).all()):
+            raise RuntimeError("the decode-layer chain produced a non-finite hidden state")
+        per_layer_us = ms * 1e3 / layers
+        result[name] = {
+            "us_per_layer": round(per_layer_us, 2),
+            "launches_per_layer": launches,
+            "weight_GB/s": round(weight_bytes / ms / 1e6, 1),
+            "frac_hbm": round((weight_bytes + cache_bytes) / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "tokens/s_at_48_layers_without_lm_head": round(1e6 / (48 * per_layer_us), 1)}
+    return result
 
 
 def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:

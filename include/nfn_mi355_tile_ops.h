@@ -669,6 +669,22 @@ int nfn_mi355_k_quant_gemm_float32_v1(
     int mode,
     void* cuda_stream);
 
+/* One-token attention with a workspace: nfn_native_tile_glimmer_gqa_decode_float32_v1
+ * runs one workgroup per query head because it has nowhere to put partial
+ * results; with a workspace the keys of every head are dealt over up to 32
+ * workgroups and a second launch merges their partial sums.  Same descriptor,
+ * same semantics, same tolerance against the double-precision formula; the
+ * summation order differs, so the bits can differ from the ordinary entry
+ * point (and the causal-block equality rule is stated for that one).  The
+ * workspace is 16-byte aligned device memory of
+ * nfn_mi355_gqa_decode_split_workspace_bytes_v1(query_heads, head_dim) bytes
+ * (0 = unsupported geometry), private to one call at a time. */
+int64_t nfn_mi355_gqa_decode_split_workspace_bytes_v1(int64_t query_heads, int64_t head_dim);
+int nfn_mi355_gqa_decode_split_v1(
+    const NfnNativeTileGlimmerGqaDecodeDescriptorV1* descriptor,
+    void* workspace,
+    int64_t workspace_nbytes);
+
 /* Shader clock under load, a measurement aid (no counterpart in the reference;
  * for benchmarks that price a kernel against the matrix-core peak at the clock
  * the chip really ran at).  Enqueues one wave that waits about `microseconds`

@@ -78,6 +78,21 @@ bool qk_norm_arguments_valid(const float* query, const float* key, const Descrip
     return weight_valid(query_weight, normalized_query) && weight_valid(key_weight, normalized_key);
 }
 
+bool gqa_descriptor_valid(const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
+    return !(d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->query == nullptr ||
+        d->current_key == nullptr || d->current_value == nullptr ||
+        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
+        d->query_heads <= 0 || d->kv_heads <= 0 || d->query_heads % d->kv_heads != 0 ||
+        d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->position < 0 ||
+        d->position == kLimit || d->first_key_position < 0 ||
+        d->first_key_position > d->position || d->cache_capacity <= 0 ||
+        d->cache_row_stride <= 0 || !positive_finite(d->scale) ||
+        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
+        d->query_heads > std::numeric_limits<std::int32_t>::max());
+}
+
 }  // namespace
 
 }  // namespace nfn
@@ -238,21 +253,30 @@ int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
 
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(
     const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
-    if (d == nullptr || d->struct_size < sizeof(*d) ||
-        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
-        d->reserved0 != 0 || d->reserved1 != 0 || d->query == nullptr ||
-        d->current_key == nullptr || d->current_value == nullptr ||
-        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
-        d->query_heads <= 0 || d->kv_heads <= 0 || d->query_heads % d->kv_heads != 0 ||
-        d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->position < 0 ||
-        d->position == kLimit || d->first_key_position < 0 ||
-        d->first_key_position > d->position || d->cache_capacity <= 0 ||
-        d->cache_row_stride <= 0 || !positive_finite(d->scale) ||
-        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
-        d->query_heads > std::numeric_limits<std::int32_t>::max()) {
+    if (!gqa_descriptor_valid(d)) return kInvalid;
+    launch_gqa_decode(*d, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+std::int64_t nfn_mi355_gqa_decode_split_workspace_bytes_v1(std::int64_t query_heads,
+                                                           std::int64_t head_dim) {
+    if (query_heads <= 0 || query_heads > std::numeric_limits<std::int32_t>::max() ||
+        head_dim <= 0 || head_dim > kMaxHeadDim) {
+        return 0;
+    }
+    return (gqa_decode_split_workspace_bytes(query_heads, head_dim) + 255) & ~std::int64_t(255);
+}
+
+int nfn_mi355_gqa_decode_split_v1(const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d,
+                                  void* workspace, std::int64_t workspace_nbytes) {
+    if (!gqa_descriptor_valid(d) || workspace == nullptr ||
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
         return kInvalid;
     }
-    launch_gqa_decode(*d, as_stream(d->cuda_stream));
+    const std::int64_t required =
+        nfn_mi355_gqa_decode_split_workspace_bytes_v1(d->query_heads, d->head_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    launch_gqa_decode_split(*d, static_cast<float*>(workspace), as_stream(d->cuda_stream));
     return launch_status();
 }
 

@@ -20,6 +20,7 @@ namespace {
 
 constexpr int kMaxWaves = 8;   // 512 threads: 256 vector registers per lane
 constexpr int kMaxHeadDim = 256;
+constexpr int kMaxSplits = 32;  // most shares of one head's keys in the split form
 constexpr int kOwned = kMaxHeadDim / kWave;  // output dimensions per lane
 
 struct AttentionArguments {
@@ -40,7 +41,17 @@ struct AttentionArguments {
     std::int64_t cache_row_stride;
     float scale;
     int causal;
+    // Split form: workgroup (x, y) takes the y-th of `splits` shares of the row's
+    // tiles and leaves (maximum, denominator, accumulator) in `partials`
+    // instead of an output row; null for the ordinary form.
+    float* partials;
+    int splits;
 };
+
+// floats per (query row, query head, split) in the partial buffer
+__host__ __device__ constexpr std::int64_t partial_floats(std::int64_t head_dim) {
+    return head_dim + 2;
+}
 
 __device__ __forceinline__ float wave_max_f(float value) {
 #pragma unroll
@@ -103,7 +114,17 @@ __device__ __forceinline__ KeyRange key_range(const AttentionArguments& a, std::
         range.last =
             a.sliding_window < end - query_position ? query_position + a.sliding_window : end;
     }
-    const std::int64_t tiles = (range.last - range.first) / kWave + 1;
+    std::int64_t tiles = (range.last - range.first) / kWave + 1;
+    if (a.partials != nullptr) {
+        // this workgroup's share: whole tiles, contiguous; an empty share has last < first
+        const std::int64_t share = (tiles + a.splits - 1) / a.splits;
+        const std::int64_t begin = static_cast<std::int64_t>(blockIdx.y) * share;
+        const std::int64_t end = begin + share < tiles ? begin + share : tiles;
+        const std::int64_t share_last = range.first + end * kWave - 1;
+        range.first += begin * kWave;
+        if (share_last < range.last) range.last = share_last;
+        tiles = end > begin ? end - begin : 0;
+    }
     range.active = static_cast<int>(tiles < waves ? tiles : waves);
     return range;
 }
@@ -509,11 +530,29 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
     }
     __syncthreads();
 
-    float overall = wave_maximum[0];
+    float overall = active > 0 ? wave_maximum[0] : -INFINITY;
     for (int w = 1; w < active; ++w) overall = fmaxf(overall, wave_maximum[w]);
     float total = 0.0f;
     for (int w = 0; w < active; ++w) {
         total = fmaf(wave_denominator[w], expf(wave_maximum[w] - overall), total);
+    }
+    if (a.partials != nullptr) {
+        // unnormalised, relative to this share's maximum; an empty share says (-inf, 0, 0)
+        float* partial = a.partials +
+            ((query_row * a.query_heads + query_head) * a.splits + blockIdx.y) *
+                partial_floats(head_dim);
+        if (tid == 0) {
+            partial[0] = overall;
+            partial[1] = total;
+        }
+        for (int d = tid; d < head_dim; d += blockDim.x) {
+            float sum = 0.0f;
+            for (int w = 0; w < active; ++w) {
+                sum = fmaf(wave_accumulator[w][d], expf(wave_maximum[w] - overall), sum);
+            }
+            partial[2 + d] = sum;
+        }
+        return;
     }
     float* output = a.output + (query_row * a.query_heads + query_head) * head_dim;
     for (int d = tid; d < head_dim; d += blockDim.x) {
@@ -525,23 +564,48 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
     }
 }
 
-void launch_attention(const AttentionArguments& arguments, std::int64_t query_rows,
-                      std::int64_t longest_key_range, hipStream_t stream) {
-    std::int64_t waves = (longest_key_range + kWave - 1) / kWave;
-    if (waves < 1) waves = 1;
-    if (waves > kMaxWaves) waves = kMaxWaves;
+// Split form, second launch: one workgroup per (query row, query head) merges
+// the shares in order.
+__global__ __launch_bounds__(kMaxHeadDim) void attention_merge_kernel(
+    const float* __restrict__ partials, float* __restrict__ output, int splits, int head_dim) {
+    const float* mine = partials + static_cast<std::int64_t>(blockIdx.x) * splits *
+        partial_floats(head_dim);
+    float overall = -INFINITY;
+    for (int s = 0; s < splits; ++s) overall = fmaxf(overall, mine[s * partial_floats(head_dim)]);
+    float total = 0.0f;
+    float sum = 0.0f;
+    const int d = threadIdx.x;
+    for (int s = 0; s < splits; ++s) {
+        const float* share = mine + s * partial_floats(head_dim);
+        const float factor = expf(share[0] - overall);  // 0 for an empty share
+        total = fmaf(share[1], factor, total);
+        if (d < head_dim) sum = fmaf(share[2 + d], factor, sum);
+    }
+    if (d < head_dim) output[static_cast<std::int64_t>(blockIdx.x) * head_dim + d] = sum / total;
+}
+
+bool vector_form_fits(const AttentionArguments& arguments) {
     const auto aligned = [](const void* pointer) {
         return reinterpret_cast<std::uintptr_t>(pointer) % 16 == 0;
     };
     const std::int64_t head_dim = arguments.head_dim;
-    const bool vectors =
-        (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
+    return (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
         arguments.cache_row_stride % 8 == 0 && arguments.cache_capacity >= kWave &&
         aligned(arguments.key_cache) && aligned(arguments.value_cache) &&
         aligned(arguments.block_key) && aligned(arguments.block_value);
-    const dim3 grid(static_cast<unsigned>(query_rows * arguments.query_heads));
+}
+
+// `tiles_per_group`: the most 64-key tiles one workgroup has to cover.
+void launch_attention(const AttentionArguments& arguments, std::int64_t query_rows,
+                      std::int64_t tiles_per_group, hipStream_t stream) {
+    std::int64_t waves = tiles_per_group;
+    if (waves < 1) waves = 1;
+    if (waves > kMaxWaves) waves = kMaxWaves;
+    const std::int64_t head_dim = arguments.head_dim;
+    const unsigned splits = arguments.partials != nullptr ? arguments.splits : 1;
+    const dim3 grid(static_cast<unsigned>(query_rows * arguments.query_heads), splits);
     const dim3 block(static_cast<unsigned>(waves * kWave));
-    if (!vectors) {
+    if (!vector_form_fits(arguments)) {
         hipLaunchKernelGGL(attention_generic_kernel, grid, block, 0, stream, arguments);
     } else if (head_dim == 32) {
         hipLaunchKernelGGL(attention_vector_kernel<4>, grid, block, 0, stream, arguments);
@@ -554,9 +618,7 @@ void launch_attention(const AttentionArguments& arguments, std::int64_t query_ro
     }
 }
 
-}  // namespace
-
-void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, hipStream_t stream) {
+AttentionArguments decode_arguments(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d) {
     AttentionArguments a{};
     a.query = d.query;
     a.block_key = d.current_key;
@@ -575,7 +637,44 @@ void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, hipSt
     a.cache_row_stride = d.cache_row_stride;
     a.scale = d.scale;
     a.causal = 1;
-    launch_attention(a, 1, a.sliding_window, stream);
+    return a;
+}
+
+std::int64_t tiles_of(std::int64_t keys) { return (keys + kWave - 1) / kWave; }
+
+}  // namespace
+
+void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, hipStream_t stream) {
+    const AttentionArguments a = decode_arguments(d);
+    launch_attention(a, 1, tiles_of(a.sliding_window), stream);
+}
+
+std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int64_t head_dim) {
+    return query_heads * kMaxSplits * partial_floats(head_dim) * 4;
+}
+
+void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, float* partials,
+                             hipStream_t stream) {
+    AttentionArguments a = decode_arguments(d);
+    const std::int64_t tiles = tiles_of(a.sliding_window);
+    if (!vector_form_fits(a) || tiles < 2) {
+        launch_attention(a, 1, tiles, stream);  // nothing to split, or no vector form: one launch
+        return;
+    }
+    a.partials = partials;
+    // About one workgroup of up to eight waves per compute unit: fewer, fatter
+    // shares beat many small ones (every workgroup pays for the query load, the
+    // ring arithmetic and a partial row).
+    std::int64_t splits = compute_units() / d.query_heads;
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits > tiles) splits = tiles;
+    if (splits < 2) splits = 2;
+    a.splits = static_cast<int>(splits);
+    launch_attention(a, 1, (tiles + a.splits - 1) / a.splits, stream);
+    const int threads = static_cast<int>((d.head_dim + kWave - 1) / kWave * kWave);
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(static_cast<unsigned>(d.query_heads)),
+                       dim3(threads), 0, stream, partials, d.output, a.splits,
+                       static_cast<int>(d.head_dim));
 }
 
 void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& d,
@@ -603,7 +702,7 @@ void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1&
         const std::int64_t window = a.causal ? d.sliding_window : 2 * d.sliding_window + 1;
         if (window < longest) longest = window;
     }
-    launch_attention(a, d.query_rows, longest, stream);
+    launch_attention(a, d.query_rows, tiles_of(longest), stream);
 }
 
 }  // namespace nfn

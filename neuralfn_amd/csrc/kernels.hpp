@@ -80,6 +80,11 @@ void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descript
                        hipStream_t stream);
 void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& descriptor,
                             hipStream_t stream);
+// One-token attention with the keys of every head dealt over several
+// workgroups; `partials` holds gqa_decode_split_workspace_bytes() bytes.
+std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int64_t head_dim);
+void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
+                             float* partials, hipStream_t stream);
 
 // clock_probe.hip — out[0] = shader cycles, out[1] = ticks of the constant
 // clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.

@@ -80,13 +80,15 @@ class LayerCache:
 
 
 def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
-                 pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True):
+                 pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
+                 attention_workspace=None):
     """One token through one layer.
 
     `pending` is the previous layer's down-projection output whose post-feed-forward norm and
     residual add are still owed (for the first layer: the embedding row with `pending_norm` None
     and `residual` zeros gives hidden = rms(embedding), the engine's embedding norm,
     resident_glimmer.cpp:1700-1701).  Returns (down, hidden): this layer's owed pair.
+    `attention_workspace` (engine_ops.gqa_decode_workspace) selects the split attention form.
     """
     g = geometry
     # hidden = residual + rms(pending); normalized = rms(hidden, input_norm)
@@ -95,14 +97,24 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
         g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps)
     query, key, value, gate = tile_ops.multi_linear(
         [weights.q, weights.k, weights.v, weights.attention_gate], normalized, workspace)
-    # per-head norms, rope on local layers, attention and the cache commit: one call
+    # per-head norms and rope in one launch, attention, the cache commit
     query = query.view(g.query_heads, g.head_dim)
     key = key.view(g.kv_heads, g.head_dim)
+    value = value.view(g.kv_heads, g.head_dim)
     first = max(0, position - g.sliding_window + 1) if local else 0
-    attention = engine_ops.fused_decode_attention(
-        query, key, value.view(g.kv_heads, g.head_dim), cache.keys, cache.values, position, first,
-        g.head_dim ** -0.5, weights.q_norm, weights.k_norm, g.norm_eps, 1.0, g.rope_theta,
-        engine_ops.ROPE_INTERLEAVED if g.interleaved_rope else engine_ops.ROPE_HALF_SPLIT, local)
+    layout = engine_ops.ROPE_INTERLEAVED if g.interleaved_rope else engine_ops.ROPE_HALF_SPLIT
+    if attention_workspace is None:
+        # the reference's fused call: no workspace, one workgroup per query head
+        attention = engine_ops.fused_decode_attention(
+            query, key, value, cache.keys, cache.values, position, first, g.head_dim ** -0.5,
+            weights.q_norm, weights.k_norm, g.norm_eps, 1.0, g.rope_theta, layout, local)
+    else:
+        # this library's split form: the keys of a head over several workgroups
+        engine_ops.qk_norm_scale_rope(query, key, weights.q_norm, weights.k_norm, g.norm_eps, 1.0,
+                                      position, g.rope_theta, layout, local)
+        attention = engine_ops.gqa_decode(query, key, value, cache.keys, cache.values, position,
+                                          first, g.head_dim ** -0.5, workspace=attention_workspace)
+        engine_ops.cache_commit(key, value, cache.keys, cache.values, position)
     # output projection of attention * sigmoid(gate), the gate as the call's prologue
     (projected,) = tile_ops.multi_linear([weights.output], attention.view(1, g.attention_dim),
                                          workspace, second=gate, prologue="gated")
@@ -116,4 +128,5 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     return down, hidden
 
 
-LAUNCHES_PER_LAYER = 9
+LAUNCHES_PER_LAYER = 9           # with the reference's fused attention call
+LAUNCHES_PER_LAYER_SPLIT = 10    # with the split attention form (one more: the merge)

@@ -125,10 +125,19 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     return out
 
 
+def gqa_decode_workspace(query_heads: int, head_dim: int, device="cuda:0"):
+    """Workspace of the split form of gqa_decode (nfn_mi355_gqa_decode_split_v1)."""
+    import torch
+    nbytes = load().nfn_mi355_gqa_decode_split_workspace_bytes_v1(query_heads, head_dim)
+    if nbytes <= 0:
+        raise ValueError("no split-attention workspace for this geometry")
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def gqa_decode(query, current_key, current_value, key_cache, value_cache, position: int,
-               first_key_position: int, scale: float, out=None):
+               first_key_position: int, scale: float, out=None, workspace=None):
     """query [query_heads, head_dim]; current_key/value [kv_heads, head_dim]; caches uint16
-    (or bfloat16) [capacity, row_stride]."""
+    (or bfloat16) [capacity, row_stride].  With `workspace` the split form runs."""
     import torch
     if out is None:
         out = torch.empty_like(query)
@@ -145,7 +154,11 @@ def gqa_decode(query, current_key, current_value, key_cache, value_cache, positi
     d.cache_capacity, d.cache_row_stride = key_cache.shape
     d.scale = scale
     d.cuda_stream = _stream()
-    check(load().nfn_native_tile_glimmer_gqa_decode_float32_v1(ctypes.byref(d)), "gqa_decode")
+    if workspace is not None:
+        check(load().nfn_mi355_gqa_decode_split_v1(ctypes.byref(d), workspace.data_ptr(),
+                                                   workspace.numel()), "gqa_decode_split")
+    else:
+        check(load().nfn_native_tile_glimmer_gqa_decode_float32_v1(ctypes.byref(d)), "gqa_decode")
     return out
 
 

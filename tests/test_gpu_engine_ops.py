@@ -243,6 +243,39 @@ def test_gqa_against_oracle(cuda, oracle, query_heads, kv_heads, head_dim, posit
     assert np.abs(out.cpu().numpy() - expected).max() <= 4e-6
 
 
+@pytest.mark.parametrize("query_heads,kv_heads,head_dim,position,first,capacity", [
+    (32, 2, 128, 5000, 2953, 2048),   # a full local window: 32 tiles in eight shares
+    (32, 2, 128, 9000, 0, 16384),     # 141 tiles, shares of 18
+    (8, 8, 64, 200, 0, 256),          # four tiles in four shares, the last one holds the current key
+    (4, 1, 256, 130, 2, 2048),        # three tiles
+    (6, 3, 128, 70, 7, 64),           # one tile: nothing to split
+    (6, 3, 50, 300, 100, 256),        # no vector form: the ordinary kernel
+])
+def test_gqa_split_form_against_oracle(cuda, oracle, query_heads, kv_heads, head_dim, position, first,
+                                       capacity):
+    rng = np.random.default_rng(position + head_dim + 1)
+    stride = kv_heads * head_dim + (6 if head_dim == 50 else 0)
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    key_cache = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    value_cache = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    scale = 1.0 / np.sqrt(head_dim)
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+    workspace.fill_(0xFF)  # the workspace comes uninitialised: NaN patterns must not leak
+    arguments = (to_device(query, cuda), to_device(key, cuda), to_device(value, cuda),
+                 bf16_tensor(key_cache, cuda), bf16_tensor(value_cache, cuda), position, first, scale)
+    out = engine_ops.gqa_decode(*arguments, workspace=workspace)
+    expected = oracle.gqa_decode(query, key, value, key_cache, value_cache, position, first, scale)
+    assert np.abs(out.cpu().numpy() - expected).max() <= 4e-6
+    again = engine_ops.gqa_decode(*arguments, workspace=workspace)
+    assert_bits_equal(out, again, "repeatable")
+    lib = tile_ops.load()
+    assert lib.nfn_mi355_gqa_decode_split_workspace_bytes_v1(0, 128) == 0
+    assert lib.nfn_mi355_gqa_decode_split_workspace_bytes_v1(32, 257) == 0
+    assert lib.nfn_mi355_gqa_decode_split_v1(None, workspace.data_ptr(), workspace.numel()) == 1
+
+
 def test_gqa_fails_closed(cuda):
     lib = tile_ops.load()
     x = torch_().zeros(4096, dtype=torch_().float32, device=cuda)
