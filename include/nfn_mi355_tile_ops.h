@@ -567,6 +567,60 @@ typedef struct NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1 {
 int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
     const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor);
 
+/* The same with the position in device memory (tile_ops.h:948-954): `position`
+ * and `first_key_position` of the descriptor are ignored, the kernels read
+ * *device_position when they run, so one captured graph serves every token.
+ * With apply_rope (a local layer) the keys are the last `sliding_window` ones,
+ * otherwise all from key 0.  1 <= sliding_window <= cache_capacity. */
+int nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor,
+    const int64_t* device_position,
+    int64_t sliding_window);
+
+/* Rows 0..rows-1 of a staged verification block, laid out [layer, source_rows,
+ * kv_heads*head_dim] float, into the bf16 rings of up to 64 layers in one
+ * launch (tile_ops.h:416-453, 960-961).  `layers` is a host array read during
+ * the call; the cache pointers inside it are device pointers. */
+typedef struct NfnNativeTileGlimmerCacheLayerV1 {
+    uint16_t* key_cache_bf16;
+    uint16_t* value_cache_bf16;
+    int64_t cache_capacity;
+    int64_t cache_row_stride;
+} NfnNativeTileGlimmerCacheLayerV1;
+typedef struct NfnNativeTileGlimmerCacheCommitLayersDescriptorV1 {
+    uint32_t struct_size;
+    uint32_t version;
+    uint32_t flags;
+    uint32_t reserved0;
+    const float* staged_keys;
+    const float* staged_values;
+    const NfnNativeTileGlimmerCacheLayerV1* layers;
+    int64_t layer_count; /* 1..64 */
+    int64_t source_rows; /* 1..64 */
+    int64_t rows;        /* 1..source_rows */
+    int64_t kv_heads;
+    int64_t head_dim;
+    int64_t position;
+    int64_t source_layer_stride; /* elements, >= source_rows*kv_heads*head_dim */
+    uint32_t reserved1;
+    uint32_t reserved2;
+    void* cuda_stream;
+} NfnNativeTileGlimmerCacheCommitLayersDescriptorV1;
+int nfn_native_tile_glimmer_cache_commit_layers_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitLayersDescriptorV1* descriptor);
+
+/* [tap, source_row, hidden] -> [row, tap, hidden] for source rows
+ * source_row_offset .. source_row_offset + rows - 1 (tile_ops.h:962-973). */
+int nfn_native_tile_glimmer_pack_target_taps_float32_v1(
+    const float* tap_major,
+    float* row_major,
+    int64_t source_rows,
+    int64_t source_row_offset,
+    int64_t rows,
+    int64_t tap_count,
+    int64_t hidden_width,
+    void* cuda_stream);
+
 /* Attention of a block of query_rows rows (positions context_length + r) over
  * the cached context and the block's own block_rows keys (tile_ops.h:445-486,
  * 974-975).  Causal (flags = NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL): keys
@@ -602,6 +656,18 @@ typedef struct NfnNativeTileDFlashBlockAttentionDescriptorV1 {
 } NfnNativeTileDFlashBlockAttentionDescriptorV1;
 int nfn_native_tile_dflash_block_attention_float32_v1(
     const NfnNativeTileDFlashBlockAttentionDescriptorV1* descriptor);
+
+/* The reference's short-context specialisation of the block attention
+ * (tile_ops.h:976-982): same descriptor and result, a caller-supplied score
+ * workspace, and a narrow geometry (32 query heads, head size 128, at most 16
+ * query rows, at most 128 keys, a non-null stream) outside of which it fails
+ * closed so that the caller keeps the general entry point.  Here the general
+ * kernel serves it and the workspace stays untouched; the checks, including
+ * the workspace size, are the reference's (glimmer_k_mmq.cu:2432-2472). */
+int nfn_native_tile_dflash_block_attention_short_split_float32_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* descriptor,
+    float* score_workspace,
+    int64_t score_workspace_nbytes);
 
 /* logits[i] = softcap * tanh(multiplier * logits[i] / softcap), in place, in
  * double as the CPU engine computes it (tile_ops.h:1004-1009;

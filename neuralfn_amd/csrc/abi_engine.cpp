@@ -93,6 +93,70 @@ bool gqa_descriptor_valid(const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
         d->query_heads > std::numeric_limits<std::int32_t>::max());
 }
 
+// Shared body of the two fused decode entry points; device_position null = the
+// position and first key of the descriptor.
+int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d,
+                            const std::int64_t* device_position, std::int64_t sliding_window) {
+    const bool on_device = device_position != nullptr;
+    if (d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->current_value == nullptr ||
+        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
+        d->query_heads > 256 || d->position == kLimit || d->first_key_position < 0 ||
+        d->first_key_position > d->position || d->cache_capacity <= 0 ||
+        d->cache_row_stride <= 0 || !positive_finite(d->attention_scale) ||
+        d->has_query_norm_weight > 1 || d->has_key_norm_weight > 1 ||
+        d->query_norm_centered > 1 || d->key_norm_centered > 1 || d->apply_rope > 1 ||
+        (on_device && (sliding_window <= 0 || sliding_window > d->cache_capacity))) {
+        return kInvalid;
+    }
+    Descriptor query_weight{}, key_weight{};
+    const Descriptor* query_source = d->has_query_norm_weight != 0 ? &d->query_norm_weight : nullptr;
+    const Descriptor* key_source = d->has_key_norm_weight != 0 ? &d->key_norm_weight : nullptr;
+    if (!qk_norm_arguments_valid(d->query, d->key, query_source, key_source, 1, d->query_heads,
+                                 d->kv_heads, d->head_dim, d->norm_eps, d->query_scale,
+                                 d->position, d->rope_theta, d->rope_layout, &query_weight,
+                                 &key_weight) ||
+        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride)) {
+        return kInvalid;
+    }
+    const hipStream_t stream = as_stream(d->cuda_stream);
+    launch_qk_norm_scale_rope(d->query, d->key, query_source != nullptr ? &query_weight : nullptr,
+                              d->query_norm_centered != 0,
+                              key_source != nullptr ? &key_weight : nullptr,
+                              d->key_norm_centered != 0, 1, d->query_heads, d->kv_heads,
+                              d->head_dim, d->norm_eps, d->query_scale, d->position,
+                              device_position, d->rope_theta,
+                              d->rope_layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED,
+                              d->apply_rope != 0, stream);
+    NfnNativeTileGlimmerGqaDecodeDescriptorV1 attention{};
+    attention.query = d->query;
+    attention.current_key = d->key;
+    attention.current_value = d->current_value;
+    attention.key_cache_bf16 = d->key_cache_bf16;
+    attention.value_cache_bf16 = d->value_cache_bf16;
+    attention.output = d->output;
+    attention.query_heads = d->query_heads;
+    attention.kv_heads = d->kv_heads;
+    attention.head_dim = d->head_dim;
+    attention.position = d->position;
+    attention.first_key_position = d->first_key_position;
+    attention.cache_capacity = d->cache_capacity;
+    attention.cache_row_stride = d->cache_row_stride;
+    attention.scale = d->attention_scale;
+    if (on_device) {
+        // a local layer (rope applied) sees its window, a global one everything
+        launch_gqa_decode_device_position(attention, device_position, sliding_window,
+                                          d->apply_rope == 0, stream);
+    } else {
+        launch_gqa_decode(attention, stream);
+    }
+    launch_cache_commit(d->key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
+                        d->kv_heads * d->head_dim, 1, d->position, device_position,
+                        d->cache_capacity, d->cache_row_stride, stream);
+    return launch_status();
+}
+
 }  // namespace
 
 }  // namespace nfn
@@ -180,7 +244,7 @@ int nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
                               query_norm_centered,
                               key_norm_weight != nullptr ? &key_weight : nullptr,
                               key_norm_centered, rows, query_heads, kv_heads, head_dim, eps,
-                              query_scale, position, theta,
+                              query_scale, position, nullptr, theta,
                               layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, apply_rope,
                               as_stream(cuda_stream));
     return launch_status();
@@ -200,55 +264,14 @@ int nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1(
 
 int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
     const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d) {
-    if (d == nullptr || d->struct_size < sizeof(*d) ||
-        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
-        d->reserved0 != 0 || d->reserved1 != 0 || d->current_value == nullptr ||
-        d->key_cache_bf16 == nullptr || d->value_cache_bf16 == nullptr || d->output == nullptr ||
-        d->query_heads > 256 || d->position == kLimit || d->first_key_position < 0 ||
-        d->first_key_position > d->position || d->cache_capacity <= 0 ||
-        d->cache_row_stride <= 0 || !positive_finite(d->attention_scale) ||
-        d->has_query_norm_weight > 1 || d->has_key_norm_weight > 1 ||
-        d->query_norm_centered > 1 || d->key_norm_centered > 1 || d->apply_rope > 1) {
-        return kInvalid;
-    }
-    Descriptor query_weight{}, key_weight{};
-    const Descriptor* query_source = d->has_query_norm_weight != 0 ? &d->query_norm_weight : nullptr;
-    const Descriptor* key_source = d->has_key_norm_weight != 0 ? &d->key_norm_weight : nullptr;
-    if (!qk_norm_arguments_valid(d->query, d->key, query_source, key_source, 1, d->query_heads,
-                                 d->kv_heads, d->head_dim, d->norm_eps, d->query_scale,
-                                 d->position, d->rope_theta, d->rope_layout, &query_weight,
-                                 &key_weight) ||
-        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride)) {
-        return kInvalid;
-    }
-    const hipStream_t stream = as_stream(d->cuda_stream);
-    launch_qk_norm_scale_rope(d->query, d->key, query_source != nullptr ? &query_weight : nullptr,
-                              d->query_norm_centered != 0,
-                              key_source != nullptr ? &key_weight : nullptr,
-                              d->key_norm_centered != 0, 1, d->query_heads, d->kv_heads,
-                              d->head_dim, d->norm_eps, d->query_scale, d->position, d->rope_theta,
-                              d->rope_layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED,
-                              d->apply_rope != 0, stream);
-    NfnNativeTileGlimmerGqaDecodeDescriptorV1 attention{};
-    attention.query = d->query;
-    attention.current_key = d->key;
-    attention.current_value = d->current_value;
-    attention.key_cache_bf16 = d->key_cache_bf16;
-    attention.value_cache_bf16 = d->value_cache_bf16;
-    attention.output = d->output;
-    attention.query_heads = d->query_heads;
-    attention.kv_heads = d->kv_heads;
-    attention.head_dim = d->head_dim;
-    attention.position = d->position;
-    attention.first_key_position = d->first_key_position;
-    attention.cache_capacity = d->cache_capacity;
-    attention.cache_row_stride = d->cache_row_stride;
-    attention.scale = d->attention_scale;
-    launch_gqa_decode(attention, stream);
-    launch_cache_commit(d->key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
-                        d->kv_heads * d->head_dim, 1, d->position, d->cache_capacity,
-                        d->cache_row_stride, stream);
-    return launch_status();
+    return run_fused_decode(d, nullptr, 0);
+}
+
+int nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d,
+    const std::int64_t* device_position, std::int64_t sliding_window) {
+    if (device_position == nullptr) return kInvalid;
+    return run_fused_decode(d, device_position, sliding_window);
 }
 
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(
@@ -284,7 +307,7 @@ int nfn_native_tile_glimmer_cache_commit_bf16_v1(
     const NfnNativeTileGlimmerCacheCommitDescriptorV1* d) {
     if (!commit_descriptor_valid(d) || d->kv_heads * d->head_dim > kMaxThreads) return kInvalid;
     launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
-                        d->kv_heads * d->head_dim, 1, d->position, d->cache_capacity,
+                        d->kv_heads * d->head_dim, 1, d->position, nullptr, d->cache_capacity,
                         d->cache_row_stride, as_stream(d->cuda_stream));
     return launch_status();
 }
@@ -296,7 +319,7 @@ int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
         return kInvalid;
     }
     launch_cache_commit(d->current_key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
-                        d->kv_heads * d->head_dim, rows, d->position, d->cache_capacity,
+                        d->kv_heads * d->head_dim, rows, d->position, nullptr, d->cache_capacity,
                         d->cache_row_stride, as_stream(d->cuda_stream));
     return launch_status();
 }
@@ -321,6 +344,74 @@ int nfn_native_tile_dflash_block_attention_float32_v1(
     }
     launch_block_attention(*d, as_stream(d->cuda_stream));
     return launch_status();
+}
+
+int nfn_native_tile_glimmer_cache_commit_layers_bf16_v1(
+    const NfnNativeTileGlimmerCacheCommitLayersDescriptorV1* d) {
+    if (d == nullptr || d->struct_size < sizeof(*d) ||
+        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
+        d->reserved0 != 0 || d->reserved1 != 0 || d->reserved2 != 0 ||
+        d->staged_keys == nullptr || d->staged_values == nullptr || d->layers == nullptr ||
+        d->layer_count <= 0 || d->layer_count > 64 || d->source_rows <= 0 ||
+        d->source_rows > kMaxBlockRows || d->rows <= 0 || d->rows > d->source_rows ||
+        d->kv_heads <= 0 || d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->position < 0 ||
+        d->position > kLimit - d->rows || d->source_layer_stride <= 0 ||
+        d->kv_heads > kMaxThreads / d->head_dim) {
+        return kInvalid;
+    }
+    const std::int64_t width = d->kv_heads * d->head_dim;
+    if (width > kLimit / d->source_rows || d->source_layer_stride < d->source_rows * width ||
+        d->source_layer_stride > kLimit / d->layer_count) {
+        return kInvalid;
+    }
+    for (std::int64_t index = 0; index < d->layer_count; ++index) {
+        const NfnNativeTileGlimmerCacheLayerV1& layer = d->layers[index];
+        if (layer.key_cache_bf16 == nullptr || layer.value_cache_bf16 == nullptr ||
+            layer.cache_capacity <= 0 || layer.cache_row_stride < width) {
+            return kInvalid;
+        }
+    }
+    launch_cache_commit_layers(*d, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_glimmer_pack_target_taps_float32_v1(const float* tap_major, float* row_major,
+                                                        std::int64_t source_rows,
+                                                        std::int64_t source_row_offset,
+                                                        std::int64_t rows, std::int64_t tap_count,
+                                                        std::int64_t hidden_width,
+                                                        void* cuda_stream) {
+    if (tap_major == nullptr || row_major == nullptr || source_rows <= 0 ||
+        source_rows > kMaxBlockRows || source_row_offset < 0 || rows <= 0 ||
+        rows > kMaxBlockRows || source_row_offset + rows > source_rows || tap_count <= 0 ||
+        tap_count > 64 || hidden_width <= 0 || hidden_width > 65536) {
+        return kInvalid;
+    }
+    launch_pack_target_taps(tap_major, row_major, source_rows, source_row_offset, rows, tap_count,
+                            hidden_width, as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_native_tile_dflash_block_attention_short_split_float32_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* d, float* score_workspace,
+    std::int64_t score_workspace_nbytes) {
+    // the reference's geometry (glimmer_k_mmq.cu:1928-1929, 2432-2472): tiles of 8 keys, 128 keys at most
+    constexpr std::int64_t kKeysPerScoreTile = 8;
+    constexpr std::int64_t kMaxKeys = 128;
+    if (d == nullptr || score_workspace == nullptr || d->query_rows <= 0 || d->query_rows > 16 ||
+        d->query_heads != 32 || d->head_dim != 128 || d->cuda_stream == nullptr ||
+        d->block_rows <= 0 || d->context_length < 0 || d->sliding_window <= 0 ||
+        d->context_length > kLimit - kMaxBlockRows) {
+        return kInvalid;
+    }
+    const std::int64_t available = d->context_length + d->block_rows;
+    const std::int64_t maximum_keys = d->sliding_window < available ? d->sliding_window : available;
+    if (maximum_keys > kMaxKeys) return kInvalid;
+    const std::int64_t score_tiles = (maximum_keys + kKeysPerScoreTile - 1) / kKeysPerScoreTile;
+    const std::int64_t score_count = d->query_rows * d->query_heads * score_tiles * kKeysPerScoreTile;
+    if (score_workspace_nbytes < score_count * 4) return kInvalid;
+    // everything else is the general entry point's business, checks included
+    return nfn_native_tile_dflash_block_attention_float32_v1(d);
 }
 
 int nfn_native_tile_glimmer_logit_transform_float32_v1(float* logits, std::int64_t count,

@@ -46,7 +46,21 @@ struct AttentionArguments {
     // instead of an output row; null for the ordinary form.
     float* partials;
     int splits;
+    // One-token form with the position in device memory (read when the kernel
+    // runs, so that one captured graph serves every token): context_length is
+    // *device_position and the window is `sliding_window` keys, or everything
+    // from key 0 when `whole_context`.  Null for a position known at launch.
+    const std::int64_t* device_position;
+    int whole_context;
 };
+
+// Resolves a device-side position into the fields the kernels work with.
+__device__ __forceinline__ void resolve_position(AttentionArguments& a) {
+    if (a.device_position == nullptr) return;
+    const std::int64_t position = a.device_position[0];
+    a.context_length = position;
+    if (a.whole_context) a.sliding_window = position + 1;
+}
 
 // floats per (query row, query head, split) in the partial buffer
 __host__ __device__ constexpr std::int64_t partial_floats(std::int64_t head_dim) {
@@ -135,6 +149,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_generic_kernel(At
     __shared__ float wave_denominator[kMaxWaves];
     __shared__ float wave_accumulator[kMaxWaves][kMaxHeadDim];
 
+    resolve_position(a);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -311,6 +326,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
     __shared__ float wave_denominator[kMaxWaves];
     __shared__ __attribute__((aligned(16))) float wave_accumulator[kMaxWaves][kMaxHeadDim];
 
+    resolve_position(a);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -647,6 +663,19 @@ std::int64_t tiles_of(std::int64_t keys) { return (keys + kWave - 1) / kWave; }
 void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, hipStream_t stream) {
     const AttentionArguments a = decode_arguments(d);
     launch_attention(a, 1, tiles_of(a.sliding_window), stream);
+}
+
+void launch_gqa_decode_device_position(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d,
+                                       const std::int64_t* device_position,
+                                       std::int64_t sliding_window, bool whole_context,
+                                       hipStream_t stream) {
+    AttentionArguments a = decode_arguments(d);
+    a.device_position = device_position;
+    a.sliding_window = sliding_window;
+    a.whole_context = whole_context ? 1 : 0;
+    // the key count is not known here: the largest workgroup, of which as many
+    // waves work as the row has tiles
+    launch_attention(a, 1, kMaxWaves, stream);
 }
 
 std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int64_t head_dim) {

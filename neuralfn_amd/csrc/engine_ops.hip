@@ -71,15 +71,52 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(
 __global__ __launch_bounds__(kThreads) void cache_commit_kernel(
     const float* __restrict__ keys, const float* __restrict__ values,
     std::uint16_t* __restrict__ key_cache, std::uint16_t* __restrict__ value_cache,
-    std::int64_t width, std::int64_t rows, std::int64_t position, std::int64_t capacity,
+    std::int64_t width, std::int64_t rows, std::int64_t position,
+    const std::int64_t* __restrict__ device_position, std::int64_t capacity,
     std::int64_t row_stride) {
     const std::int64_t index = static_cast<std::int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (index >= rows * width) return;
+    if (device_position != nullptr) position = device_position[0];
     const std::int64_t row = index / width;
     const std::int64_t column = index - row * width;
     const std::int64_t target = ((position + row) % capacity) * row_stride + column;
     key_cache[target] = to_bf16(keys[index]);
     value_cache[target] = to_bf16(values[index]);
+}
+
+// Rows 0..rows-1 of a staged block into the rings of up to 64 layers, one launch
+// (neuralfn/csrc/tile_cuda/kernels.cu:2862-2901).  blockIdx = (columns, row, layer).
+struct CacheLayers {
+    NfnNativeTileGlimmerCacheLayerV1 layer[64];
+};
+
+__global__ __launch_bounds__(kThreads) void cache_commit_layers_kernel(
+    const float* __restrict__ keys, const float* __restrict__ values, std::int64_t width,
+    std::int64_t position, std::int64_t layer_stride, CacheLayers layers) {
+    const std::int64_t column = static_cast<std::int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (column >= width) return;
+    const std::int64_t row = blockIdx.y;
+    const NfnNativeTileGlimmerCacheLayerV1& layer = layers.layer[blockIdx.z];
+    const std::int64_t source = blockIdx.z * layer_stride + row * width + column;
+    const std::int64_t target =
+        ((position + row) % layer.cache_capacity) * layer.cache_row_stride + column;
+    layer.key_cache_bf16[target] = to_bf16(keys[source]);
+    layer.value_cache_bf16[target] = to_bf16(values[source]);
+}
+
+// [tap, source_row, hidden] -> [row, tap, hidden] for rows source_row_offset .. +rows-1
+// (neuralfn/csrc/tile_cuda/kernels.cu:2903-2922).
+__global__ __launch_bounds__(kThreads) void pack_target_taps_kernel(
+    const float* __restrict__ tap_major, float* __restrict__ row_major, std::int64_t source_rows,
+    std::int64_t source_row_offset, std::int64_t tap_count, std::int64_t hidden_width,
+    std::int64_t count) {
+    const std::int64_t index = static_cast<std::int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= count) return;
+    const std::int64_t hidden = index % hidden_width;
+    const std::int64_t row_tap = index / hidden_width;
+    const std::int64_t tap = row_tap % tap_count;
+    const std::int64_t row = row_tap / tap_count;
+    row_major[index] = tap_major[(tap * source_rows + source_row_offset + row) * hidden_width + hidden];
 }
 
 // ---- element-wise -------------------------------------------------------------
@@ -148,12 +185,34 @@ void launch_rope(float* query, float* key, std::int64_t rows, std::int64_t query
 
 void launch_cache_commit(const float* keys, const float* values, std::uint16_t* key_cache,
                          std::uint16_t* value_cache, std::int64_t width, std::int64_t rows,
-                         std::int64_t position, std::int64_t capacity, std::int64_t row_stride,
-                         hipStream_t stream) {
+                         std::int64_t position, const std::int64_t* device_position,
+                         std::int64_t capacity, std::int64_t row_stride, hipStream_t stream) {
     hipLaunchKernelGGL(cache_commit_kernel,
                        dim3(blocks_for(rows * width, std::int64_t(1) << 31)), dim3(kThreads), 0,
                        stream, keys, values, key_cache, value_cache, width, rows, position,
-                       capacity, row_stride);
+                       device_position, capacity, row_stride);
+}
+
+void launch_cache_commit_layers(const NfnNativeTileGlimmerCacheCommitLayersDescriptorV1& d,
+                                hipStream_t stream) {
+    CacheLayers layers{};
+    for (std::int64_t index = 0; index < d.layer_count; ++index) layers.layer[index] = d.layers[index];
+    const std::int64_t width = d.kv_heads * d.head_dim;
+    hipLaunchKernelGGL(cache_commit_layers_kernel,
+                       dim3(blocks_for(width), static_cast<unsigned>(d.rows),
+                            static_cast<unsigned>(d.layer_count)),
+                       dim3(kThreads), 0, stream, d.staged_keys, d.staged_values, width, d.position,
+                       d.source_layer_stride, layers);
+}
+
+void launch_pack_target_taps(const float* tap_major, float* row_major, std::int64_t source_rows,
+                             std::int64_t source_row_offset, std::int64_t rows,
+                             std::int64_t tap_count, std::int64_t hidden_width,
+                             hipStream_t stream) {
+    const std::int64_t count = rows * tap_count * hidden_width;
+    hipLaunchKernelGGL(pack_target_taps_kernel, dim3(blocks_for(count, std::int64_t(1) << 31)),
+                       dim3(kThreads), 0, stream, tap_major, row_major, source_rows,
+                       source_row_offset, tap_count, hidden_width, count);
 }
 
 void launch_logit_transform(float* logits, std::int64_t count, float multiplier, float softcap,

@@ -49,12 +49,14 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
                      std::int64_t width, float eps, hipStream_t stream);
 
 // rms.hip — per-head Q/K normalisation, query scale and rotary embedding of
-// `rows` rows in one launch; row r is at position + r.
+// `rows` rows in one launch; row r is at position + r.  A non-null
+// device_position replaces `position` when the kernel runs.
 void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query_weight,
                                bool query_centered, const Descriptor* key_weight,
                                bool key_centered, std::int64_t rows, std::int64_t query_heads,
                                std::int64_t kv_heads, std::int64_t head_dim, float eps,
-                               float query_scale, std::int64_t position, float theta,
+                               float query_scale, std::int64_t position,
+                               const std::int64_t* device_position, float theta,
                                bool interleaved, bool apply_rope, hipStream_t stream);
 
 // engine_ops.hip — the small operators around the packed linears.
@@ -67,8 +69,14 @@ void launch_rope(float* query, float* key, std::int64_t rows, std::int64_t query
                  float theta, bool interleaved, bool inverse, hipStream_t stream);
 void launch_cache_commit(const float* keys, const float* values, std::uint16_t* key_cache,
                          std::uint16_t* value_cache, std::int64_t width, std::int64_t rows,
-                         std::int64_t position, std::int64_t capacity, std::int64_t row_stride,
-                         hipStream_t stream);
+                         std::int64_t position, const std::int64_t* device_position,
+                         std::int64_t capacity, std::int64_t row_stride, hipStream_t stream);
+void launch_cache_commit_layers(const NfnNativeTileGlimmerCacheCommitLayersDescriptorV1& descriptor,
+                                hipStream_t stream);
+void launch_pack_target_taps(const float* tap_major, float* row_major, std::int64_t source_rows,
+                             std::int64_t source_row_offset, std::int64_t rows,
+                             std::int64_t tap_count, std::int64_t hidden_width,
+                             hipStream_t stream);
 void launch_logit_transform(float* logits, std::int64_t count, float multiplier, float softcap,
                             hipStream_t stream);
 void launch_add(const float* lhs, const float* rhs, float* out, std::int64_t count,
@@ -82,6 +90,12 @@ void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1&
                             hipStream_t stream);
 // One-token attention with the keys of every head dealt over several
 // workgroups; `partials` holds gqa_decode_split_workspace_bytes() bytes.
+// One-token attention whose position is read from device memory when the kernel
+// runs; the keys are the last `sliding_window` ones, or all when whole_context.
+void launch_gqa_decode_device_position(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
+                                       const std::int64_t* device_position,
+                                       std::int64_t sliding_window, bool whole_context,
+                                       hipStream_t stream);
 std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int64_t head_dim);
 void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
                              float* partials, hipStream_t stream);

@@ -378,9 +378,11 @@ __global__ __launch_bounds__(kRmsThreads) void rms_wide_kernel(
 __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
     float* __restrict__ query, float* __restrict__ key, NormWeight query_weight,
     NormWeight key_weight, int query_heads, int kv_heads, int head_dim, float eps,
-    float query_scale, std::int64_t position, double theta, bool interleaved, bool apply_rope) {
+    float query_scale, std::int64_t position, const std::int64_t* __restrict__ device_position,
+    double theta, bool interleaved, bool apply_rope) {
     __shared__ float partials[kRmsThreads];
     __shared__ float normalized[kRmsThreads];
+    if (device_position != nullptr) position = device_position[0];
     const int heads_per_row = query_heads + kv_heads;
     const int row = blockIdx.x / heads_per_row;
     const int combined = blockIdx.x - row * heads_per_row;
@@ -508,7 +510,8 @@ void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query
                                bool query_centered, const Descriptor* key_weight,
                                bool key_centered, std::int64_t rows, std::int64_t query_heads,
                                std::int64_t kv_heads, std::int64_t head_dim, float eps,
-                               float query_scale, std::int64_t position, float theta,
+                               float query_scale, std::int64_t position,
+                               const std::int64_t* device_position, float theta,
                                bool interleaved, bool apply_rope, hipStream_t stream) {
     hipLaunchKernelGGL(qk_norm_scale_rope_kernel,
                        dim3(static_cast<unsigned>(rows * (query_heads + kv_heads))),
@@ -516,7 +519,8 @@ void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query
                        norm_weight(query_weight, query_centered),
                        norm_weight(key_weight, key_centered), static_cast<int>(query_heads),
                        static_cast<int>(kv_heads), static_cast<int>(head_dim), eps, query_scale,
-                       position, static_cast<double>(theta), interleaved, apply_rope);
+                       position, device_position, static_cast<double>(theta), interleaved,
+                       apply_rope);
 }
 
 }  // namespace nfn

@@ -93,8 +93,13 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
                            first_key_position: int, attention_scale: float, query_weight=None,
                            key_weight=None, eps: float = 1e-5, query_scale: float = 1.0,
                            theta: float = 500000.0, layout: int = ROPE_HALF_SPLIT,
-                           apply_rope: bool = True, out=None):
-    """qk_norm_scale_rope (in place on query/key), one-token attention, cache commit."""
+                           apply_rope: bool = True, out=None, device_position=None,
+                           sliding_window: int = 0):
+    """qk_norm_scale_rope (in place on query/key), one-token attention, cache commit.
+
+    With `device_position` (an int64 tensor of one element) the kernels read the position when
+    they run and `position` / `first_key_position` are ignored; `sliding_window` then bounds a
+    local layer's keys."""
     import torch
     if out is None:
         out = torch.empty_like(query)
@@ -120,8 +125,13 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     d.rope_layout = layout
     d.apply_rope = 1 if apply_rope else 0
     d.cuda_stream = stream
-    check(load().nfn_native_tile_glimmer_fused_decode_attention_float32_v1(ctypes.byref(d)),
-          "fused_decode_attention")
+    if device_position is not None:
+        check(load().nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1(
+            ctypes.byref(d), device_position.data_ptr(), sliding_window),
+            "fused_decode_attention_device_position")
+    else:
+        check(load().nfn_native_tile_glimmer_fused_decode_attention_float32_v1(ctypes.byref(d)),
+              "fused_decode_attention")
     return out
 
 
@@ -222,3 +232,35 @@ def add(lhs, rhs, out=None):
 def scale_inplace(values, scale: float) -> None:
     check(load().nfn_native_tile_scale_inplace_float32(values.data_ptr(), values.numel(), scale,
                                                        _stream()), "scale_inplace")
+
+
+def cache_commit_layers(staged_keys, staged_values, caches, rows: int, position: int) -> None:
+    """staged_keys/values [layers, source_rows, kv_heads, head_dim]; caches: a (key_cache,
+    value_cache) pair per layer.  Rows 0..rows-1 go to positions position .. position+rows-1."""
+    layers, source_rows, kv_heads, head_dim = staged_keys.shape
+    table = (tile_ops.CacheLayer * layers)()
+    for entry, (key_cache, value_cache) in zip(table, caches):
+        entry.key_cache_bf16, entry.value_cache_bf16 = key_cache.data_ptr(), value_cache.data_ptr()
+        entry.cache_capacity, entry.cache_row_stride = key_cache.shape
+    d = tile_ops.CacheCommitLayersDescriptor()
+    d.struct_size = ctypes.sizeof(d)
+    d.version = 1
+    d.staged_keys, d.staged_values = staged_keys.data_ptr(), staged_values.data_ptr()
+    d.layers = table
+    d.layer_count, d.source_rows, d.rows = layers, source_rows, rows
+    d.kv_heads, d.head_dim, d.position = kv_heads, head_dim, position
+    d.source_layer_stride = source_rows * kv_heads * head_dim
+    d.cuda_stream = _stream()
+    check(load().nfn_native_tile_glimmer_cache_commit_layers_bf16_v1(ctypes.byref(d)),
+          "cache_commit_layers")
+
+
+def pack_target_taps(tap_major, source_row_offset: int, rows: int):
+    """[taps, source_rows, hidden] -> [rows, taps, hidden]."""
+    import torch
+    taps, source_rows, hidden = tap_major.shape
+    out = torch.empty((rows, taps, hidden), dtype=torch.float32, device=tap_major.device)
+    check(load().nfn_native_tile_glimmer_pack_target_taps_float32_v1(
+        tap_major.data_ptr(), out.data_ptr(), source_rows, source_row_offset, rows, taps, hidden,
+        _stream()), "pack_target_taps")
+    return out

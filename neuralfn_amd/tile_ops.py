@@ -104,6 +104,25 @@ class FusedDecodeAttentionDescriptor(ctypes.Structure):
     ]
 
 
+class CacheLayer(ctypes.Structure):
+    """NfnNativeTileGlimmerCacheLayerV1 (neuralfn/csrc/native_train/tile_ops.h:416-421)."""
+
+    _fields_ = [("key_cache_bf16", _P), ("value_cache_bf16", _P), ("cache_capacity", _I64),
+                ("cache_row_stride", _I64)]
+
+
+class CacheCommitLayersDescriptor(ctypes.Structure):
+    """NfnNativeTileGlimmerCacheCommitLayersDescriptorV1 (neuralfn/csrc/native_train/tile_ops.h:430-453)."""
+
+    _fields_ = [
+        ("struct_size", _U32), ("version", _U32), ("flags", _U32), ("reserved0", _U32),
+        ("staged_keys", _P), ("staged_values", _P), ("layers", ctypes.POINTER(CacheLayer)),
+        ("layer_count", _I64), ("source_rows", _I64), ("rows", _I64), ("kv_heads", _I64),
+        ("head_dim", _I64), ("position", _I64), ("source_layer_stride", _I64),
+        ("reserved1", _U32), ("reserved2", _U32), ("cuda_stream", _P),
+    ]
+
+
 _DESC = ctypes.POINTER(PackedWeightDescriptor)
 _DESC_ARRAY = ctypes.POINTER(_DESC)
 _PTR_ARRAY = ctypes.POINTER(ctypes.c_void_p)
@@ -186,6 +205,14 @@ SIGNATURES = {
                        ctypes.c_bool, _F32, _I64, _F32, _U32, ctypes.c_bool, _P]),
     "nfn_native_tile_glimmer_fused_decode_attention_float32_v1": (
         ctypes.c_int, [ctypes.POINTER(FusedDecodeAttentionDescriptor)]),
+    "nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1": (
+        ctypes.c_int, [ctypes.POINTER(FusedDecodeAttentionDescriptor), _P, _I64]),
+    "nfn_native_tile_glimmer_cache_commit_layers_bf16_v1": (
+        ctypes.c_int, [ctypes.POINTER(CacheCommitLayersDescriptor)]),
+    "nfn_native_tile_glimmer_pack_target_taps_float32_v1": (
+        ctypes.c_int, [_P, _P, _I64, _I64, _I64, _I64, _I64, _P]),
+    "nfn_native_tile_dflash_block_attention_short_split_float32_v1": (
+        ctypes.c_int, [ctypes.POINTER(BlockAttentionDescriptor), _P, _I64]),
     "nfn_native_tile_glimmer_gqa_decode_float32_v1": (
         ctypes.c_int, [ctypes.POINTER(GqaDecodeDescriptor)]),
     "nfn_native_tile_glimmer_cache_commit_bf16_v1": (

@@ -556,6 +556,125 @@ def test_fused_decode_attention_equals_the_separate_calls(cuda, oracle, apply_ro
     assert lib.nfn_native_tile_glimmer_fused_decode_attention_float32_v1(ctypes.byref(empty)) == 1
 
 
+@pytest.mark.parametrize("apply_rope,position", [(True, 4100), (True, 70), (False, 1500), (False, 0)])
+def test_fused_decode_attention_with_the_position_on_the_device(cuda, oracle, apply_rope, position):
+    """The graph form reads the position when the kernels run: same bits as the host form at
+    that position, with the window rule of the reference (kernels.cu:2604-2611): a layer with
+    rope sees its last `sliding_window` keys, one without sees everything."""
+    rng = np.random.default_rng(34 + position)
+    query_heads, kv_heads, head_dim, window = 32, 2, 128, 2048
+    capacity = window if apply_rope else 4096
+    stride = kv_heads * head_dim
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    keys = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    values = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    weight = _norm_row((1.0 + 0.1 * rng.standard_normal(head_dim)).astype(np.float32))
+    first = max(0, position - window + 1) if apply_rope else 0
+    common = dict(query_weight=weight, key_weight=weight, eps=1e-5, query_scale=1.0, theta=500000.0,
+                  layout=engine_ops.ROPE_INTERLEAVED, apply_rope=apply_rope)
+
+    q1, k1, v1 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc1, vc1 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    host = engine_ops.fused_decode_attention(q1, k1, v1, kc1, vc1, position, first,
+                                             head_dim ** -0.5, **common)
+    q2, k2, v2 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc2, vc2 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    device_position = to_device(np.array([position], dtype=np.int64), cuda)
+    # the descriptor's own position fields are ignored in this form: give it other ones
+    device = engine_ops.fused_decode_attention(q2, k2, v2, kc2, vc2, 7, 3, head_dim ** -0.5,
+                                               device_position=device_position,
+                                               sliding_window=window, **common)
+    assert_bits_equal(device, host, "attention output")
+    assert_bits_equal(q2, q1, "query")
+    assert_bits_equal(k2, k1, "key")
+    assert np.array_equal(bits_of(kc2), bits_of(kc1)) and np.array_equal(bits_of(vc2), bits_of(vc1))
+    lib = tile_ops.load()
+    call = lib.nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1
+    assert call(None, device_position.data_ptr(), window) == 1
+
+
+def test_cache_commit_layers_and_pack_target_taps(cuda, oracle):
+    rng = np.random.default_rng(35)
+    layers, source_rows, rows, kv_heads, head_dim, position = 5, 9, 6, 2, 64, 1021
+    width = kv_heads * head_dim
+    capacities = [1024, 2048, 64, 1024, 4096]  # rows wrap in some rings and not in others
+    staged_keys = rng.standard_normal((layers, source_rows, kv_heads, head_dim)).astype(np.float32)
+    staged_values = rng.standard_normal((layers, source_rows, kv_heads, head_dim)).astype(np.float32)
+    before = [rng.integers(0, 65536, (capacity, width + 8), dtype=np.uint16) for capacity in capacities]
+    caches = [(bf16_tensor(b, cuda), bf16_tensor(b, cuda)) for b in before]
+    engine_ops.cache_commit_layers(to_device(staged_keys, cuda), to_device(staged_values, cuda), caches,
+                                   rows, position)
+    for layer, (capacity, start) in enumerate(zip(capacities, before)):
+        expected_keys, expected_values = start.copy(), start.copy()
+        for row in range(rows):
+            slot = (position + row) % capacity
+            expected_keys[slot, :width] = oracle.to_bf16(staged_keys[layer, row].reshape(-1))
+            expected_values[slot, :width] = oracle.to_bf16(staged_values[layer, row].reshape(-1))
+        assert np.array_equal(bits_of(caches[layer][0]), expected_keys), f"layer {layer} keys"
+        assert np.array_equal(bits_of(caches[layer][1]), expected_values), f"layer {layer} values"
+    lib = tile_ops.load()
+    assert lib.nfn_native_tile_glimmer_cache_commit_layers_bf16_v1(None) == 1
+    empty = tile_ops.CacheCommitLayersDescriptor()
+    assert lib.nfn_native_tile_glimmer_cache_commit_layers_bf16_v1(ctypes.byref(empty)) == 1
+
+    taps, hidden = 4, 6656
+    tap_major = rng.standard_normal((taps, source_rows, hidden)).astype(np.float32)
+    packed = engine_ops.pack_target_taps(to_device(tap_major, cuda), 2, 5).cpu().numpy()
+    assert np.array_equal(packed, np.transpose(tap_major[:, 2:7], (1, 0, 2)))
+    x = to_device(tap_major, cuda)
+    call = lib.nfn_native_tile_glimmer_pack_target_taps_float32_v1
+    assert call(x.data_ptr(), x.data_ptr(), source_rows, 5, 5, taps, hidden, None) == 1  # 5 + 5 > 9
+    assert call(None, x.data_ptr(), source_rows, 0, 5, taps, hidden, None) == 1
+    assert call(x.data_ptr(), x.data_ptr(), 65, 0, 5, taps, hidden, None) == 1
+    assert call(x.data_ptr(), x.data_ptr(), source_rows, 0, 5, taps, 65537, None) == 1
+
+
+def test_short_split_block_attention_is_the_general_one_inside_its_geometry(cuda, oracle):
+    # probe :2666-2682: the short-split output within 5e-4 of the general one; here the same bits
+    query, block_key, block_value, key_cache, value_cache, context, window, scale = \
+        _probe_block_case(oracle)
+    import torch
+    arguments = (to_device(query, cuda), to_device(block_key, cuda), to_device(block_value, cuda),
+                 bf16_tensor(key_cache, cuda), bf16_tensor(value_cache, cuda))
+    general = engine_ops.block_attention(*arguments, context, window, scale, False)
+    lib = tile_ops.load()
+    call = lib.nfn_native_tile_dflash_block_attention_short_split_float32_v1
+    stream = torch.cuda.Stream()
+
+    def descriptor(out, **changes):
+        d = tile_ops.BlockAttentionDescriptor()
+        d.struct_size, d.version = ctypes.sizeof(d), 1
+        d.query, d.block_key, d.block_value = (t.data_ptr() for t in arguments[:3])
+        d.key_cache_bf16, d.value_cache_bf16, d.output = (arguments[3].data_ptr(),
+                                                          arguments[4].data_ptr(), out.data_ptr())
+        d.query_rows, d.query_heads, d.head_dim = query.shape
+        d.block_rows, d.kv_heads = block_key.shape[0], block_key.shape[1]
+        d.context_length, d.sliding_window = context, window
+        d.cache_capacity, d.cache_row_stride = key_cache.shape
+        d.scale = scale
+        d.cuda_stream = int(stream.cuda_stream)
+        for name, value in changes.items():
+            setattr(d, name, value)
+        return d
+
+    score_count = 16 * 32 * 6 * 8  # rows x heads x ceil(48 keys / 8) x 8, the probe's workspace
+    scores = torch.empty(score_count, dtype=torch.float32, device=cuda)
+    out = torch.zeros_like(general)
+    torch.cuda.synchronize()
+    assert call(ctypes.byref(descriptor(out)), scores.data_ptr(), score_count * 4) == 0
+    stream.synchronize()
+    assert_bits_equal(out, general)
+    # outside the geometry, or with too small a workspace, it fails closed
+    assert call(ctypes.byref(descriptor(out)), scores.data_ptr(), score_count * 4 - 1) == 1
+    assert call(ctypes.byref(descriptor(out)), None, score_count * 4) == 1
+    assert call(ctypes.byref(descriptor(out, cuda_stream=None)), scores.data_ptr(), score_count * 4) == 1
+    assert call(ctypes.byref(descriptor(out, sliding_window=4096, context_length=500)),
+                scores.data_ptr(), 1 << 30) == 1  # more than 128 keys
+    assert call(ctypes.byref(descriptor(out, query_heads=16)), scores.data_ptr(), score_count * 4) == 1
+
+
 # ---- a whole decode layer ---------------------------------------------------------------------------
 
 def test_two_decode_layers_against_the_cpu_engine_arithmetic(cuda, oracle):
