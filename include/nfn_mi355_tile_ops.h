@@ -528,9 +528,11 @@ int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
  * 946-947): qk_norm_scale_rope on query/key (in place), gqa_decode with key as
  * the current key, and the bf16 cache commit of key/current_value at
  * `position`.  The norm weights are embedded by value; has_*_norm_weight == 0
- * makes the corresponding descriptor inert.  Here it is those three launches
- * in sequence on the descriptor's stream, so it equals the separate calls bit
- * for bit. */
+ * makes the corresponding descriptor inert.  Here it is two launches on the
+ * descriptor's stream (the norm/rope kernel also writes the cache row, which a
+ * one-token attention at this position does not read; a key range as long as
+ * the ring gets the commit as a third launch, after the attention), with the
+ * arithmetic of the separate calls, so it equals them bit for bit. */
 typedef struct NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1 {
     uint32_t struct_size;
     uint32_t version;
@@ -748,6 +750,14 @@ int nfn_mi355_k_quant_gemm_float32_v1(
 int64_t nfn_mi355_gqa_decode_split_workspace_bytes_v1(int64_t query_heads, int64_t head_dim);
 int nfn_mi355_gqa_decode_split_v1(
     const NfnNativeTileGlimmerGqaDecodeDescriptorV1* descriptor,
+    void* workspace,
+    int64_t workspace_nbytes);
+
+/* nfn_native_tile_glimmer_fused_decode_attention_float32_v1 with the split
+ * attention form above: three launches (norm/rope/commit, attention shares,
+ * merge).  Same descriptor, same workspace as nfn_mi355_gqa_decode_split_v1. */
+int nfn_mi355_fused_decode_attention_split_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor,
     void* workspace,
     int64_t workspace_nbytes);
 

@@ -93,10 +93,12 @@ bool gqa_descriptor_valid(const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
         d->query_heads > std::numeric_limits<std::int32_t>::max());
 }
 
-// Shared body of the two fused decode entry points; device_position null = the
-// position and first key of the descriptor.
+// Shared body of the fused decode entry points; device_position null = the
+// position and first key of the descriptor; split_partials non-null = the
+// split attention form with that workspace.
 int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d,
-                            const std::int64_t* device_position, std::int64_t sliding_window) {
+                     const std::int64_t* device_position, std::int64_t sliding_window,
+                     float* split_partials) {
     const bool on_device = device_position != nullptr;
     if (d == nullptr || d->struct_size < sizeof(*d) ||
         d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 || d->flags != 0 ||
@@ -121,6 +123,11 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
         return kInvalid;
     }
     const hipStream_t stream = as_stream(d->cuda_stream);
+    // The new cache row is written by the first launch, before the attention
+    // runs: right as long as the attention does not read that ring row, which
+    // holds for every key range shorter than the ring (and for the device
+    // form, whose window is at most the ring).  Otherwise the commit follows.
+    const bool commit_first = on_device || d->position - d->first_key_position < d->cache_capacity;
     launch_qk_norm_scale_rope(d->query, d->key, query_source != nullptr ? &query_weight : nullptr,
                               d->query_norm_centered != 0,
                               key_source != nullptr ? &key_weight : nullptr,
@@ -128,7 +135,9 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
                               d->head_dim, d->norm_eps, d->query_scale, d->position,
                               device_position, d->rope_theta,
                               d->rope_layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED,
-                              d->apply_rope != 0, stream);
+                              d->apply_rope != 0, commit_first ? d->key_cache_bf16 : nullptr,
+                              d->value_cache_bf16, d->current_value, d->cache_capacity,
+                              d->cache_row_stride, stream);
     NfnNativeTileGlimmerGqaDecodeDescriptorV1 attention{};
     attention.query = d->query;
     attention.current_key = d->key;
@@ -148,12 +157,16 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
         // a local layer (rope applied) sees its window, a global one everything
         launch_gqa_decode_device_position(attention, device_position, sliding_window,
                                           d->apply_rope == 0, stream);
+    } else if (split_partials != nullptr) {
+        launch_gqa_decode_split(attention, split_partials, stream);
     } else {
         launch_gqa_decode(attention, stream);
     }
-    launch_cache_commit(d->key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
-                        d->kv_heads * d->head_dim, 1, d->position, device_position,
-                        d->cache_capacity, d->cache_row_stride, stream);
+    if (!commit_first) {
+        launch_cache_commit(d->key, d->current_value, d->key_cache_bf16, d->value_cache_bf16,
+                            d->kv_heads * d->head_dim, 1, d->position, nullptr, d->cache_capacity,
+                            d->cache_row_stride, stream);
+    }
     return launch_status();
 }
 
@@ -246,7 +259,7 @@ int nfn_native_tile_glimmer_qk_norm_scale_rope_batch_float32_v1(
                               key_norm_centered, rows, query_heads, kv_heads, head_dim, eps,
                               query_scale, position, nullptr, theta,
                               layout == NFN_NATIVE_TILE_GLIMMER_ROPE_INTERLEAVED, apply_rope,
-                              as_stream(cuda_stream));
+                              nullptr, nullptr, nullptr, 0, 0, as_stream(cuda_stream));
     return launch_status();
 }
 
@@ -264,14 +277,27 @@ int nfn_native_tile_glimmer_qk_norm_scale_rope_float32_v1(
 
 int nfn_native_tile_glimmer_fused_decode_attention_float32_v1(
     const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d) {
-    return run_fused_decode(d, nullptr, 0);
+    return run_fused_decode(d, nullptr, 0, nullptr);
 }
 
 int nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1(
     const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d,
     const std::int64_t* device_position, std::int64_t sliding_window) {
     if (device_position == nullptr) return kInvalid;
-    return run_fused_decode(d, device_position, sliding_window);
+    return run_fused_decode(d, device_position, sliding_window, nullptr);
+}
+
+int nfn_mi355_fused_decode_attention_split_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d, void* workspace,
+    std::int64_t workspace_nbytes) {
+    if (d == nullptr || workspace == nullptr ||
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
+        return kInvalid;
+    }
+    const std::int64_t required =
+        nfn_mi355_gqa_decode_split_workspace_bytes_v1(d->query_heads, d->head_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    return run_fused_decode(d, nullptr, 0, static_cast<float*>(workspace));
 }
 
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(

@@ -50,14 +50,19 @@ void launch_rms_norm(const float* input, const Descriptor* weight, bool centered
 
 // rms.hip — per-head Q/K normalisation, query scale and rotary embedding of
 // `rows` rows in one launch; row r is at position + r.  A non-null
-// device_position replaces `position` when the kernel runs.
+// device_position replaces `position` when the kernel runs.  With key_cache
+// non-null (rows == 1) the new key and current_value rows also go to the bf16
+// rings at `position`.
 void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query_weight,
                                bool query_centered, const Descriptor* key_weight,
                                bool key_centered, std::int64_t rows, std::int64_t query_heads,
                                std::int64_t kv_heads, std::int64_t head_dim, float eps,
                                float query_scale, std::int64_t position,
                                const std::int64_t* device_position, float theta,
-                               bool interleaved, bool apply_rope, hipStream_t stream);
+                               bool interleaved, bool apply_rope, std::uint16_t* key_cache,
+                               std::uint16_t* value_cache, const float* current_value,
+                               std::int64_t cache_capacity, std::int64_t cache_row_stride,
+                               hipStream_t stream);
 
 // engine_ops.hip — the small operators around the packed linears.
 // token_source: 0 = host_token, 1 = one int64 in device memory, 2 = int32 per row.

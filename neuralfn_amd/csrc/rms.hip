@@ -368,18 +368,30 @@ __global__ __launch_bounds__(kRmsThreads) void rms_wide_kernel(
     }
 }
 
+// Where the fused decode step also leaves the new key and value row (bf16 ring
+// caches); key_cache null = no commit.
+struct CacheRow {
+    std::uint16_t* key_cache;
+    std::uint16_t* value_cache;
+    const float* values;  // [kv_heads, head_dim], the current value row
+    std::int64_t capacity;
+    std::int64_t row_stride;
+};
+
 // ---- per-head Q/K normalisation, query scale and rotary embedding in one launch
 // (neuralfn/csrc/native_train/tile_ops.h:905-943; reference kernel
 // neuralfn/csrc/tile_cuda/kernels.cu:2381-2473).  One workgroup per (row, head);
 // a thread owns one column.  Each step is the arithmetic of the separate
 // operator it replaces, in the same order (rms_resident_kernel at width =
 // head_dim, the in-place scale, the rotary kernel), so the result equals the
-// three calls bit for bit.
+// three calls bit for bit.  For the fused decode step the key heads' workgroups
+// also write the bf16 cache row of the new key and value (the row a one-token
+// attention at this position never reads).
 __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
     float* __restrict__ query, float* __restrict__ key, NormWeight query_weight,
     NormWeight key_weight, int query_heads, int kv_heads, int head_dim, float eps,
     float query_scale, std::int64_t position, const std::int64_t* __restrict__ device_position,
-    double theta, bool interleaved, bool apply_rope) {
+    double theta, bool interleaved, bool apply_rope, CacheRow commit) {
     __shared__ float partials[kRmsThreads];
     __shared__ float normalized[kRmsThreads];
     if (device_position != nullptr) position = device_position[0];
@@ -400,8 +412,21 @@ __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
                                            static_cast<float>(head_dim) + eps);
     float result = __fmul_rn(__fmul_rn(value, inverse), scale[0]);
     if (is_query) result = __fmul_rn(result, query_scale);
+    // a key head also goes to the cache (one row only), with its value head
+    const bool commits = !is_query && commit.key_cache != nullptr;
+    const std::int64_t cache_index = commits
+        ? (position % commit.capacity) * commit.row_stride +
+            static_cast<std::int64_t>(combined - query_heads) * head_dim
+        : 0;
+    if (commits && inside) {
+        commit.value_cache[cache_index + column] =
+            to_bf16(commit.values[static_cast<std::int64_t>(combined - query_heads) * head_dim + column]);
+    }
     if (!apply_rope) {
-        if (inside) values[column] = result;
+        if (inside) {
+            values[column] = result;
+            if (commits) commit.key_cache[cache_index + column] = to_bf16(result);
+        }
         return;
     }
     normalized[column] = result;
@@ -414,6 +439,10 @@ __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
         rope_rotate(a, b, position + row, column, head_dim, theta, false);
         values[first] = a;
         values[second] = b;
+        if (commits) {
+            commit.key_cache[cache_index + first] = to_bf16(a);
+            commit.key_cache[cache_index + second] = to_bf16(b);
+        }
     }
 }
 
@@ -512,7 +541,11 @@ void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query
                                std::int64_t kv_heads, std::int64_t head_dim, float eps,
                                float query_scale, std::int64_t position,
                                const std::int64_t* device_position, float theta,
-                               bool interleaved, bool apply_rope, hipStream_t stream) {
+                               bool interleaved, bool apply_rope, std::uint16_t* key_cache,
+                               std::uint16_t* value_cache, const float* current_value,
+                               std::int64_t cache_capacity, std::int64_t cache_row_stride,
+                               hipStream_t stream) {
+    const CacheRow commit{key_cache, value_cache, current_value, cache_capacity, cache_row_stride};
     hipLaunchKernelGGL(qk_norm_scale_rope_kernel,
                        dim3(static_cast<unsigned>(rows * (query_heads + kv_heads))),
                        dim3(kRmsThreads), 0, stream, query, key,
@@ -520,7 +553,7 @@ void launch_qk_norm_scale_rope(float* query, float* key, const Descriptor* query
                        norm_weight(key_weight, key_centered), static_cast<int>(query_heads),
                        static_cast<int>(kv_heads), static_cast<int>(head_dim), eps, query_scale,
                        position, device_position, static_cast<double>(theta), interleaved,
-                       apply_rope);
+                       apply_rope, commit);
 }
 
 }  // namespace nfn

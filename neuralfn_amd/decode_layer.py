@@ -9,8 +9,8 @@ down projection; post-feed-forward norm + residual.  The grouping into calls is 
 engine's: one grouped small-batch call per shared input, the sigmoid gate and SwiGLU as prologues
 of the projection that consumes them, two adjacent norms in one dual-RMS call
 (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:2233-2585, 2913-2960), and the Q/K norms,
-rope, attention and cache commit in its fused decode-attention call (three launches here).
-Nine launches per layer and token.
+rope, attention and cache commit in its fused decode-attention call (two launches here).
+Eight launches per layer and token.
 
 This is host-side sequencing for tests and benchmarks, not an engine: no sampling, no prompt
 handling, one token per step.
@@ -103,18 +103,12 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     value = value.view(g.kv_heads, g.head_dim)
     first = max(0, position - g.sliding_window + 1) if local else 0
     layout = engine_ops.ROPE_INTERLEAVED if g.interleaved_rope else engine_ops.ROPE_HALF_SPLIT
-    if attention_workspace is None:
-        # the reference's fused call: no workspace, one workgroup per query head
-        attention = engine_ops.fused_decode_attention(
-            query, key, value, cache.keys, cache.values, position, first, g.head_dim ** -0.5,
-            weights.q_norm, weights.k_norm, g.norm_eps, 1.0, g.rope_theta, layout, local)
-    else:
-        # this library's split form: the keys of a head over several workgroups
-        engine_ops.qk_norm_scale_rope(query, key, weights.q_norm, weights.k_norm, g.norm_eps, 1.0,
-                                      position, g.rope_theta, layout, local)
-        attention = engine_ops.gqa_decode(query, key, value, cache.keys, cache.values, position,
-                                          first, g.head_dim ** -0.5, workspace=attention_workspace)
-        engine_ops.cache_commit(key, value, cache.keys, cache.values, position)
+    # the reference's fused call (one workgroup per query head), or with a workspace this
+    # library's split form of it (the keys of a head over several workgroups)
+    attention = engine_ops.fused_decode_attention(
+        query, key, value, cache.keys, cache.values, position, first, g.head_dim ** -0.5,
+        weights.q_norm, weights.k_norm, g.norm_eps, 1.0, g.rope_theta, layout, local,
+        workspace=attention_workspace)
     # output projection of attention * sigmoid(gate), the gate as the call's prologue
     (projected,) = tile_ops.multi_linear([weights.output], attention.view(1, g.attention_dim),
                                          workspace, second=gate, prologue="gated")
@@ -128,5 +122,5 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     return down, hidden
 
 
-LAUNCHES_PER_LAYER = 9           # with the reference's fused attention call
-LAUNCHES_PER_LAYER_SPLIT = 10    # with the split attention form (one more: the merge)
+LAUNCHES_PER_LAYER = 8           # with the reference's fused attention call
+LAUNCHES_PER_LAYER_SPLIT = 9     # with the split attention form (one more: the merge)

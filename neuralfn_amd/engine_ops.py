@@ -94,12 +94,12 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
                            key_weight=None, eps: float = 1e-5, query_scale: float = 1.0,
                            theta: float = 500000.0, layout: int = ROPE_HALF_SPLIT,
                            apply_rope: bool = True, out=None, device_position=None,
-                           sliding_window: int = 0):
+                           sliding_window: int = 0, workspace=None):
     """qk_norm_scale_rope (in place on query/key), one-token attention, cache commit.
 
     With `device_position` (an int64 tensor of one element) the kernels read the position when
     they run and `position` / `first_key_position` are ignored; `sliding_window` then bounds a
-    local layer's keys."""
+    local layer's keys.  With `workspace` (gqa_decode_workspace) the attention is the split form."""
     import torch
     if out is None:
         out = torch.empty_like(query)
@@ -125,7 +125,10 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     d.rope_layout = layout
     d.apply_rope = 1 if apply_rope else 0
     d.cuda_stream = stream
-    if device_position is not None:
+    if workspace is not None:
+        check(load().nfn_mi355_fused_decode_attention_split_v1(
+            ctypes.byref(d), workspace.data_ptr(), workspace.numel()), "fused_decode_attention_split")
+    elif device_position is not None:
         check(load().nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1(
             ctypes.byref(d), device_position.data_ptr(), sliding_window),
             "fused_decode_attention_device_position")

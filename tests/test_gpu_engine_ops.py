@@ -518,11 +518,12 @@ def test_qk_norm_scale_rope_batch_rows_and_fail_closed(cuda):
     torch_().cuda.synchronize()
 
 
-@pytest.mark.parametrize("apply_rope", [False, True])
-def test_fused_decode_attention_equals_the_separate_calls(cuda, oracle, apply_rope):
+@pytest.mark.parametrize("apply_rope,first", [(False, 2500), (True, 4100 - 2048 + 1), (True, 4100 - 2048)])
+def test_fused_decode_attention_equals_the_separate_calls(cuda, oracle, apply_rope, first):
+    # the last case reads as many keys as the ring has rows: the oldest one sits in the row
+    # the commit overwrites, so the commit has to come after the attention, as in the separate calls
     rng = np.random.default_rng(33)
     query_heads, kv_heads, head_dim, capacity, position = 32, 2, 128, 2048, 4100
-    first = position - capacity + 1 if apply_rope else 2500
     stride = kv_heads * head_dim
     query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
     key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
@@ -550,6 +551,16 @@ def test_fused_decode_attention_equals_the_separate_calls(cuda, oracle, apply_ro
     assert_bits_equal(k2, k1, "key in place")
     assert np.array_equal(bits_of(kc2), bits_of(kc1)) and np.array_equal(bits_of(vc2), bits_of(vc1))
     assert np.array_equal(bits_of(kc2)[position % capacity], oracle.to_bf16(k1.cpu().numpy().reshape(-1)))
+    # the split form of the fused call: same in-place results and cache, attention within tolerance
+    q3, k3, v3 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc3, vc3 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    split = engine_ops.fused_decode_attention(q3, k3, v3, kc3, vc3, position, first, scale, q_weight,
+                                              k_weight, 1e-5, 1.0, 500000.0,
+                                              engine_ops.ROPE_INTERLEAVED, apply_rope,
+                                              workspace=engine_ops.gqa_decode_workspace(query_heads, head_dim))
+    assert_bits_equal(q3, q1, "query, split form")
+    assert np.array_equal(bits_of(kc3), bits_of(kc1)) and np.array_equal(bits_of(vc3), bits_of(vc1))
+    assert np.abs(split.cpu().numpy() - separate.cpu().numpy()).max() <= 4e-6
     lib = tile_ops.load()
     assert lib.nfn_native_tile_glimmer_fused_decode_attention_float32_v1(None) == 1
     empty = tile_ops.FusedDecodeAttentionDescriptor()
