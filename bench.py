@@ -476,7 +476,7 @@ def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
                               "frac_hbm": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                               "tokens/s": round(1e3 / ms, 1)}
 
-    # prefill: 1024 rows through the dequant-GEMM, one call per tensor
+    # prefill: 1024 rows through the dequant-GEMM
     rows = 1024
     xs = {dim: torch.from_numpy(values).to(device) for dim, values in inputs.items()}
     big = {name: torch.empty((rows, shape[0]), dtype=torch.float32, device=device)
@@ -486,9 +486,14 @@ def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
     gemm_workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
 
     def prefill():
+        # grouped where the engine groups: projections of one input convert it once
         for layer in layers:
-            for name, weight in layer.items():
-                tile_ops.gemm(weight, xs[weight.input_dim], tile_ops.GEMM_F16, gemm_workspace, big[name])
+            tile_ops.gemm_multi([layer["q"], layer["k"], layer["v"]], xs[MODEL_DIM], tile_ops.GEMM_F16,
+                                gemm_workspace, [big["q"], big["k"], big["v"]])
+            tile_ops.gemm(layer["o"], xs[ATTN_DIM], tile_ops.GEMM_F16, gemm_workspace, big["o"])
+            tile_ops.gemm_multi([layer["gate"], layer["up"]], xs[MODEL_DIM], tile_ops.GEMM_F16,
+                                gemm_workspace, [big["gate"], big["up"]])
+            tile_ops.gemm(layer["down"], xs[FFN_DIM], tile_ops.GEMM_F16, gemm_workspace, big["down"])
 
     ms = time_graph(prefill, stream, max(5, steps // 2), max(2, warmup // 2))
     tflops = rows * flops_per_row / ms / 1e9

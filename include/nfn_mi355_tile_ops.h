@@ -737,6 +737,23 @@ int nfn_mi355_k_quant_gemm_float32_v1(
     int mode,
     void* cuda_stream);
 
+/* The same for 1..4 projections of one input (Q/K/V, gate/up), the way the
+ * small-batch entry points group them: the activations are converted once and
+ * every projection runs from that copy.  All descriptors share input_dim (a
+ * multiple of 256) and are Q4_K, Q5_K, Q6_K or Q8_0.  The workspace is the
+ * largest of the single-projection sizes (the query above with each
+ * output_dim).  Results are those of the single-projection call, bit for bit. */
+int nfn_mi355_k_quant_gemm_multi_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    const float* input,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    int mode,
+    void* cuda_stream);
+
 /* One-token attention with a workspace: nfn_native_tile_glimmer_gqa_decode_float32_v1
  * runs one workgroup per query head because it has nowhere to put partial
  * results; with a workspace the keys of every head are dealt over up to 32

@@ -573,6 +573,41 @@ int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float*
     return launch_status();
 }
 
+int nfn_mi355_k_quant_gemm_multi_float32_v1(const Descriptor* const* descriptors, const float* input,
+                                            float* const* outputs, std::int64_t operation_count,
+                                            std::int64_t rows, void* workspace,
+                                            std::int64_t workspace_nbytes, int mode,
+                                            void* cuda_stream) {
+    if (descriptors == nullptr || input == nullptr || outputs == nullptr || workspace == nullptr ||
+        operation_count < 1 || operation_count > kMaxOperations || rows <= 0 ||
+        mode != NFN_MI355_GEMM_F16 || reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
+        return kInvalid;
+    }
+    Descriptor normalized[kMaxOperations];
+    std::int64_t required = 0;
+    for (std::int64_t index = 0; index < operation_count; ++index) {
+        const Descriptor* descriptor = descriptors[index];
+        if (outputs[index] == nullptr ||
+            !validate_k_descriptor(descriptor, descriptors[0] == nullptr ? 0 : descriptors[0]->input_dim,
+                                   cuda_stream, true) ||
+            !normalize_descriptor(descriptor, &normalized[index]) ||
+            !gemm_f16_supports(normalized[index].encoding, normalized[index].input_dim)) {
+            return kInvalid;
+        }
+        const std::int64_t bytes = nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+            rows, normalized[index].input_dim, normalized[index].output_dim, mode);
+        if (bytes == 0) return kInvalid;
+        if (bytes > required) required = bytes;
+    }
+    if (workspace_nbytes < required) return kInvalid;
+    const hipStream_t stream = as_stream(cuda_stream);
+    convert_gemm_activations(input, rows, normalized[0].input_dim, workspace, stream);
+    for (std::int64_t index = 0; index < operation_count; ++index) {
+        launch_gemm_f16_converted(normalized[index], outputs[index], rows, workspace, stream);
+    }
+    return launch_status();
+}
+
 int nfn_mi355_shader_clock_probe_v1(std::uint64_t* cycles_and_ticks, std::int64_t microseconds,
                                     void* cuda_stream) {
     if (cycles_and_ticks == nullptr || microseconds < 1 || microseconds > 100000) return kInvalid;

@@ -822,21 +822,32 @@ bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
             encoding == kEncQ8_0) && input_dim % 256 == 0;
 }
 
+void convert_gemm_activations(const float* input, std::int64_t rows, std::int64_t input_dim,
+                              void* workspace, hipStream_t stream) {
+    std::uint8_t* activations = static_cast<std::uint8_t*>(workspace);
+    float* inverse_scale = reinterpret_cast<float*>(activations + padded_rows(rows) * input_dim * 2);
+    float* scale = inverse_scale + padded_rows(rows);
+    hipLaunchKernelGGL(row_scale_kernel, dim3(static_cast<unsigned>(padded_rows(rows))), dim3(256),
+                       0, stream, input, scale, inverse_scale, rows, input_dim);
+    hipLaunchKernelGGL(convert_activations_kernel,
+                       dim3(static_cast<unsigned>(padded_rows(rows) / 32),
+                            static_cast<unsigned>((input_dim + 511) / 512)),
+                       dim3(256), 0, stream, input, scale, activations, rows, input_dim);
+}
+
 void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,
                      std::int64_t rows, void* workspace, hipStream_t stream) {
+    convert_gemm_activations(input, rows, descriptor.input_dim, workspace, stream);
+    launch_gemm_f16_converted(descriptor, output, rows, workspace, stream);
+}
+
+void launch_gemm_f16_converted(const Descriptor& descriptor, float* output, std::int64_t rows,
+                               void* workspace, hipStream_t stream) {
     std::uint8_t* activations = static_cast<std::uint8_t*>(workspace);
     float* inverse_scale =
         reinterpret_cast<float*>(activations + padded_rows(rows) * descriptor.input_dim * 2);
-    float* scale = inverse_scale + padded_rows(rows);
     float* partials =
         reinterpret_cast<float*>(activations + activation_bytes(rows, descriptor.input_dim));
-    hipLaunchKernelGGL(row_scale_kernel, dim3(static_cast<unsigned>(padded_rows(rows))), dim3(256),
-                       0, stream, input, scale, inverse_scale, rows, descriptor.input_dim);
-    hipLaunchKernelGGL(convert_activations_kernel,
-                       dim3(static_cast<unsigned>(padded_rows(rows) / 32),
-                            static_cast<unsigned>((descriptor.input_dim + 511) / 512)),
-                       dim3(256), 0, stream, input, scale, activations, rows,
-                       descriptor.input_dim);
     switch (descriptor.encoding) {
         case kEncQ4K:
             launch_encoding<kEncQ4K>(descriptor, activations, inverse_scale, output, partials, rows,

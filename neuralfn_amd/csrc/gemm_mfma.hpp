@@ -15,5 +15,12 @@ bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim);
 // output[rows, output_dim] = input[rows, input_dim] * W^T, float accumulation.
 void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,
                       std::int64_t rows, void* workspace, hipStream_t stream);
+// The same in two steps, for several projections of one input: the activations
+// go to the workspace once, then each projection runs from there (the split-K
+// partial buffer behind them is reused; the launches are stream-ordered).
+void convert_gemm_activations(const float* input, std::int64_t rows, std::int64_t input_dim,
+                              void* workspace, hipStream_t stream);
+void launch_gemm_f16_converted(const Descriptor& descriptor, float* output, std::int64_t rows,
+                               void* workspace, hipStream_t stream);
 
 }  // namespace nfn

@@ -187,6 +187,8 @@ SIGNATURES = {
     "nfn_mi355_k_quant_gemm_workspace_bytes_v1": (_I64, [_I64, _I64, _I64, ctypes.c_int]),
     "nfn_mi355_k_quant_gemm_float32_v1": (
         ctypes.c_int, [_DESC, _P, _P, _I64, _P, _I64, ctypes.c_int, _P]),
+    "nfn_mi355_k_quant_gemm_multi_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, ctypes.c_int, _P]),
     "nfn_mi355_shader_clock_probe_v1": (ctypes.c_int, [_P, _I64, _P]),
     "nfn_mi355_gqa_decode_split_workspace_bytes_v1": (_I64, [_I64, _I64]),
     "nfn_mi355_gqa_decode_split_v1": (ctypes.c_int, [ctypes.POINTER(GqaDecodeDescriptor), _P, _I64]),
@@ -583,6 +585,28 @@ def gemm(weight: PackedWeight, x, mode: int = GEMM_F16, workspace=None, out=None
         ctypes.byref(descriptor), x.data_ptr(), out.data_ptr(), rows, workspace.data_ptr(),
         workspace.numel(), mode, stream), "k_quant_gemm")
     return out
+
+
+def gemm_multi(weights: Sequence[PackedWeight], x, mode: int = GEMM_F16, workspace=None,
+               outputs=None):
+    """nfn_mi355_k_quant_gemm_multi_float32_v1: 1..4 projections of one input, converted once."""
+    import torch
+    rows = x.shape[0]
+    stream = _stream_handle()
+    if workspace is None:
+        nbytes = max(load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+            rows, w.input_dim, w.output_dim, mode) for w in weights)
+        if nbytes <= 0:
+            raise ValueError("unsupported GEMM geometry or mode")
+        workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    if outputs is None:
+        outputs = [torch.empty((rows, w.output_dim), dtype=torch.float32, device=x.device)
+                   for w in weights]
+    descriptors = [w.descriptor(stream) for w in weights]
+    check(load().nfn_mi355_k_quant_gemm_multi_float32_v1(
+        _descriptor_array(descriptors), x.data_ptr(), _pointer_array(outputs), len(weights), rows,
+        workspace.data_ptr(), workspace.numel(), mode, stream), "k_quant_gemm_multi")
+    return outputs
 
 
 class ShaderClockProbe:

@@ -800,6 +800,36 @@ def test_prefill_gemm_split_k(cuda, oracle, encoding, in_dim):
     assert np.array_equal(y.view(np.uint32), again.view(np.uint32))  # fixed summation order
 
 
+def test_prefill_gemm_multi_equals_single_calls(cuda, oracle):
+    """nfn_mi355_k_quant_gemm_multi_float32_v1: one conversion of the input, the single call's bits."""
+    rows, in_dim = 300, 1024
+    specs = [(kquant.Q4_K, 384), (kquant.Q6_K, 130), (kquant.Q8_0, 17), (kquant.Q5_K, 256)]
+    weights = [tile_ops.PackedWeight.from_numpy(
+        e, kquant.quantize(e, kquant.synthetic_weights(70 + i, n, in_dim)), n, in_dim)
+        for i, (e, n) in enumerate(specs)]
+    x = to_device(kquant.synthetic_activations(71, rows, in_dim), cuda)
+    grouped = tile_ops.gemm_multi(weights, x)
+    for weight, y in zip(weights, grouped):
+        assert_bits_equal(y, tile_ops.gemm(weight, x), kquant.NAMES[weight.encoding])
+    lib = tile_ops.load()
+    descriptors = [w.descriptor(0) for w in weights]
+    outputs = [torch_().empty((rows, w.output_dim), dtype=torch_().float32, device=cuda) for w in weights]
+    workspace = torch_().empty(1 << 24, dtype=torch_().uint8, device=cuda)
+
+    def call(count=4, rows=rows, nbytes=workspace.numel(), mode=tile_ops.GEMM_F16, descs=descriptors):
+        return lib.nfn_mi355_k_quant_gemm_multi_float32_v1(
+            tile_ops._descriptor_array(descs), x.data_ptr(), tile_ops._pointer_array(outputs), count,
+            rows, workspace.data_ptr(), nbytes, mode, None)
+
+    assert call() == 0
+    assert call(count=0) == 1 and call(count=5) == 1 and call(rows=0) == 1
+    assert call(nbytes=1024) == 1 and call(mode=tile_ops.GEMM_INT8) == 1
+    other = tile_ops.PackedWeight.from_numpy(
+        kquant.Q4_K, kquant.quantize(kquant.Q4_K, kquant.synthetic_weights(72, 64, 512)), 64, 512)
+    assert call(descs=descriptors[:3] + [other.descriptor(0)]) == 1  # another input width
+    torch_().cuda.synchronize()
+
+
 def test_prefill_gemm_activation_range(cuda, oracle):
     # rows scaled far outside the fp16 range, and a zero row: the per-row power
     # of two keeps every row at the same relative accuracy
