@@ -111,3 +111,63 @@ def test_gemm_random_case(cuda, oracle, seed):
     z = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
     for row in range(0, rows, 7):
         assert normalised_error(z[row], expected[row]) <= 1e-5, f"{label} row {row} (generic linear)"
+
+
+# ---- attention ---------------------------------------------------------------------------------------
+
+def _bf16(oracle, rng, shape):
+    return oracle.to_bf16(rng.standard_normal(shape).astype(np.float32))
+
+
+def _bf16_tensor(bits_, device):
+    return to_device(np.ascontiguousarray(bits_, dtype=np.uint16).view(np.int16), device)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_attention_random_case(cuda, oracle, seed):
+    """One-token attention (both forms) and block attention (both modes) on drawn geometries: head sizes
+    on and off the vector kernel, padded cache rows, rings smaller than a tile, windows that cut the
+    context or exceed it, positions before and after the ring wraps."""
+    from neuralfn_amd import engine_ops
+    rng = np.random.default_rng(3000 + seed)
+    head_dim = int(rng.choice([8, 32, 50, 64, 96, 128, 128, 256]))
+    kv_heads = int(rng.choice([1, 2, 4]))
+    query_heads = kv_heads * int(rng.choice([1, 2, 4, 16]))
+    capacity = int(rng.choice([16, 63, 64, 100, 512, 2048]))
+    padding = int(rng.choice([0, 0, 8, 6]))
+    stride = kv_heads * head_dim + padding
+    position = int(rng.integers(0, 3 * capacity))
+    window = int(rng.integers(1, capacity + 1))
+    first = max(0, position - window + 1)
+    scale = float(head_dim ** -0.5)
+    key_cache, value_cache = _bf16(oracle, rng, (capacity, stride)), _bf16(oracle, rng, (capacity, stride))
+    device_keys, device_values = _bf16_tensor(key_cache, cuda), _bf16_tensor(value_cache, cuda)
+    label = (f"heads {query_heads}/{kv_heads} x {head_dim}, ring {capacity} x {stride}, position {position}, "
+             f"window {window}")
+
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    expected = oracle.gqa_decode(query, key, value, key_cache, value_cache, position, first, scale)
+    arguments = (to_device(query, cuda), to_device(key, cuda), to_device(value, cuda), device_keys,
+                 device_values, position, first, scale)
+    plain = engine_ops.gqa_decode(*arguments).cpu().numpy()
+    assert np.abs(plain - expected).max() <= 4e-6, label
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+    workspace.fill_(0xFF)
+    split = engine_ops.gqa_decode(*arguments, workspace=workspace).cpu().numpy()
+    assert np.abs(split - expected).max() <= 4e-6, label + " (split form)"
+
+    rows = int(rng.integers(1, 9))
+    block_rows = rows + int(rng.integers(0, 5))
+    context = position
+    block_query = rng.standard_normal((rows, query_heads, head_dim)).astype(np.float32)
+    block_key = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    block_value = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    for causal in (True, False):
+        expected = oracle.block_attention(block_query, block_key, block_value, key_cache, value_cache,
+                                          context, window, scale, causal)
+        actual = engine_ops.block_attention(
+            to_device(block_query, cuda), to_device(block_key, cuda), to_device(block_value, cuda),
+            device_keys, device_values, context, window, scale, causal).cpu().numpy()
+        assert np.abs(actual - expected).max() <= 4e-6, f"{label}, block {rows}/{block_rows}, causal {causal}"
