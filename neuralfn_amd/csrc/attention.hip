@@ -317,6 +317,15 @@ __device__ __forceinline__ float dot_piece(const float* q, const Piece& p, float
     return dot;
 }
 
+// Ties two values together for the compiler: whatever is computed from either after this
+// point cannot be scheduled before both have their values here.  (Used to bound how many
+// registers a long unrolled stretch holds at once.)
+template <typename A, typename B>
+__device__ __forceinline__ void tie(A& first, B& second) {
+    asm volatile("" : "+v"(first), "+v"(second));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int LANES_PER_KEY>
 __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(AttentionArguments a) {
     constexpr int kPieces = LANES_PER_KEY;             // head_dim / 8
@@ -368,8 +377,119 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
 #pragma unroll
     for (int e = 0; e < 8; ++e) accumulator[e] = 0.0f;
 
-    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
-         wave < active && tile <= last;
+    // running maximum, denominator and accumulator take in a tile's scores;
+    // returns this lane's weight exp(score - maximum)
+    const auto fold = [&](float raw_score, bool live) {
+        const float score = live ? raw_score * a.scale : -INFINITY;
+        const float next_maximum = fmaxf(maximum, wave_max_f(score));
+        const float keep = expf(maximum - next_maximum);  // 0 on the first tile
+        const float weight = live ? expf(score - next_maximum) : 0.0f;
+        denominator = denominator * keep + wave_sum_f(weight);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) accumulator[e] *= keep;
+        maximum = next_maximum;
+        return weight;
+    };
+    // this lane's 8 dimensions of the cached value row of key k of the tile whose first
+    // row is ring slot `slot` (keys past the range repeat the last one)
+    const auto cached_value_piece = [&](std::int64_t slot, int k, int in_tile) {
+        const int clamped = k < in_tile ? k : in_tile;
+        return reinterpret_cast<const uint4*>(
+            a.value_cache + ring_row(slot + clamped) * a.cache_row_stride + head_offset)[piece];
+    };
+
+    // Scores: lane = key.  Weighted sum: lane = (key of the load, 8 dimensions);
+    // every form adds the keys of the tile in the same order, key g, g + G, ...
+    std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
+
+    // A wave's tiles that lie wholly in the cache come first.  Keys and values of such a
+    // tile are requested before anything of it is used, and the keys of the next such
+    // tile (if it is a full one) while the weighted sum of the current one runs.
+    if constexpr (kPieces <= 16) {
+        uint4 key_raw[kPieces];
+        bool requested_ahead = false;  // wave-uniform
+        // bytes from a load's first value row to this lane's 8 dimensions (fits 32 bits:
+        // the launcher bounds the row stride)
+        const std::uint32_t value_lane_offset =
+            static_cast<std::uint32_t>(group) * static_cast<std::uint32_t>(a.cache_row_stride) * 2u +
+            static_cast<std::uint32_t>(piece) * 16u;
+        for (; wave < active && tile <= last && tile + kWave - 1 < a.context_length;
+             tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
+            const int in_tile = static_cast<int>(last - tile < kWave - 1 ? last - tile : kWave - 1);
+            const bool live = lane <= in_tile;
+            const int my_key = live ? lane : in_tile;
+            uint4 value_raw[kPieces];
+            if (!requested_ahead) {
+                const uint4* key = reinterpret_cast<const uint4*>(
+                    a.key_cache + ring_row(tile_slot + my_key) * a.cache_row_stride + head_offset);
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) key_raw[u] = key[u];
+            }
+            if (in_tile == kWave - 1 && tile_slot + kWave <= capacity) {
+                // a full tile that does not wrap: one wave-uniform row address per load
+                // and the same 32-bit lane offset for all of them
+                const char* rows = reinterpret_cast<const char*>(
+                    a.value_cache + tile_slot * a.cache_row_stride + head_offset);
+                const std::int64_t load_stride = kKeysPerLoad * a.cache_row_stride * 2;
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    value_raw[u] = *reinterpret_cast<const uint4*>(rows + u * load_stride +
+                                                                   value_lane_offset);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) {
+                    value_raw[u] = cached_value_piece(tile_slot, u * kKeysPerLoad + group, in_tile);
+                }
+            }
+            // the query comes out of shared memory a few pieces at a time (all of it at
+            // once would take as many registers as the tile's keys and values together)
+            // (four pieces at a time; the offset, tied to the running score, keeps the
+            // compiler from holding the whole query in registers)
+            int query_offset = 0;
+            float score = 0.0f;
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) {
+                if (u % 4 == 0) tie(query_offset, score);
+                score = dot_piece(q + query_offset + u * 8, unpack_bf16(key_raw[u]), score);
+            }
+            const std::int64_t next_end = tile + tile_step + kWave - 1;
+            requested_ahead = next_end <= last && next_end < a.context_length;
+            // the next keys go into the registers the scores have just freed: their loads
+            // must come after the last use of the current keys
+            int next_lane = lane;
+            tie(next_lane, score);
+            if (requested_ahead) {
+                const uint4* next_key = reinterpret_cast<const uint4*>(
+                    a.key_cache +
+                    ring_row(ring_row(tile_slot + slot_step) + next_lane) * a.cache_row_stride +
+                    head_offset);
+#pragma unroll
+                for (int u = 0; u < kPieces; ++u) key_raw[u] = next_key[u];
+            }
+            const float weight = fold(score, live);
+            float weight_of[kPieces];
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) {
+                weight_of[u] = __shfl(weight, u * kKeysPerLoad + group);
+            }
+            // values are unpacked a few loads at a time: unpacking all of them at once
+            // would not fit the registers beside the keys requested ahead
+#pragma unroll
+            for (int u = 0; u < kPieces; ++u) {
+                if (u % 2 == 0) tie(value_raw[u].x, accumulator[0]);
+                const Piece value = unpack_bf16(value_raw[u]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    accumulator[e] = fmaf(weight_of[u], value.v[e], accumulator[e]);
+                }
+            }
+        }
+    }
+
+    // The remaining tiles: those that hold rows of the block, and with more than 128
+    // dimensions a head also the cached ones (16 loads in flight at a time).
+    for (; wave < active && tile <= last;
          tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
         // Keys past the range repeat the last key of the tile with weight 0.
         const int in_tile = static_cast<int>(last - tile < kWave - 1 ? last - tile : kWave - 1);
@@ -377,89 +497,43 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
         const int my_key = live ? lane : in_tile;
         const bool cache_only = tile + kWave - 1 < a.context_length;  // wave-uniform
 
-        // running maximum, denominator and accumulator take in the tile's scores;
-        // returns this lane's weight exp(score - maximum)
-        const auto fold = [&](float raw_score) {
-            const float score = live ? raw_score * a.scale : -INFINITY;
-            const float next_maximum = fmaxf(maximum, wave_max_f(score));
-            const float keep = expf(maximum - next_maximum);  // 0 on the first tile
-            const float weight = live ? expf(score - next_maximum) : 0.0f;
-            denominator = denominator * keep + wave_sum_f(weight);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) accumulator[e] *= keep;
-            maximum = next_maximum;
-            return weight;
-        };
-        // value row of key k of the tile (keys past the range repeat the last one)
-        const auto cached_value_piece = [&](int k) {
-            const int clamped = k < in_tile ? k : in_tile;
-            return reinterpret_cast<const uint4*>(
-                a.value_cache + ring_row(tile_slot + clamped) * a.cache_row_stride +
-                head_offset)[piece];
-        };
-
-        // Scores: lane = key.  Weighted sum: lane = (key of the load, 8 dimensions);
-        // every form adds the keys of the tile in the same order, key g, g + G, ...
-        if (cache_only) {
+        if (kPieces > 16 && cache_only) {
             const uint4* key = reinterpret_cast<const uint4*>(
                 a.key_cache + ring_row(tile_slot + my_key) * a.cache_row_stride + head_offset);
-            if constexpr (kPieces <= 16) {
-                // the whole tile's keys and values are requested before anything is used
-                uint4 key_raw[kPieces], value_raw[kPieces];
+            float score = 0.0f;
+            int query_offset = 0;
 #pragma unroll
-                for (int u = 0; u < kPieces; ++u) key_raw[u] = key[u];
+            for (int c = 0; c < kPieces; c += 16) {
+                uint4 raw[16];
 #pragma unroll
-                for (int u = 0; u < kPieces; ++u) {
-                    value_raw[u] = cached_value_piece(u * kKeysPerLoad + group);
+                for (int u = 0; u < 16; ++u) raw[u] = key[c + u];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    if (u % 4 == 0) tie(query_offset, score);
+                    score = dot_piece(q + query_offset + (c + u) * 8, unpack_bf16(raw[u]), score);
                 }
-                float score = 0.0f;
+            }
+            const float weight = fold(score, live);
 #pragma unroll
-                for (int u = 0; u < kPieces; ++u) {
-                    score = dot_piece(q + u * 8, unpack_bf16(key_raw[u]), score);
+            for (int t0 = 0; t0 < kPieces; t0 += 16) {
+                uint4 raw[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    raw[u] = cached_value_piece(tile_slot, (t0 + u) * kKeysPerLoad + group, in_tile);
                 }
-                const float weight = fold(score);
 #pragma unroll
-                for (int u = 0; u < kPieces; ++u) {
-                    const float weight_k = __shfl(weight, u * kKeysPerLoad + group);
-                    const Piece value = unpack_bf16(value_raw[u]);
+                for (int u = 0; u < 16; ++u) {
+                    const float weight_k = __shfl(weight, (t0 + u) * kKeysPerLoad + group);
+                    const Piece value = unpack_bf16(raw[u]);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         accumulator[e] = fmaf(weight_k, value.v[e], accumulator[e]);
                     }
                 }
-            } else {
-                float score = 0.0f;
-#pragma unroll
-                for (int c = 0; c < kPieces; c += 16) {
-                    uint4 raw[16];
-#pragma unroll
-                    for (int u = 0; u < 16; ++u) raw[u] = key[c + u];
-#pragma unroll
-                    for (int u = 0; u < 16; ++u) {
-                        score = dot_piece(q + (c + u) * 8, unpack_bf16(raw[u]), score);
-                    }
-                }
-                const float weight = fold(score);
-#pragma unroll
-                for (int t0 = 0; t0 < kPieces; t0 += 16) {
-                    uint4 raw[16];
-#pragma unroll
-                    for (int u = 0; u < 16; ++u) {
-                        raw[u] = cached_value_piece((t0 + u) * kKeysPerLoad + group);
-                    }
-#pragma unroll
-                    for (int u = 0; u < 16; ++u) {
-                        const float weight_k = __shfl(weight, (t0 + u) * kKeysPerLoad + group);
-                        const Piece value = unpack_bf16(raw[u]);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            accumulator[e] = fmaf(weight_k, value.v[e], accumulator[e]);
-                        }
-                    }
-                }
             }
         } else {
             float score = 0.0f;
+            int query_offset = 0;
             const std::int64_t key_position = tile + my_key;
             if (key_position >= a.context_length) {
                 const std::int64_t block_row = key_position - a.context_length;
@@ -470,9 +544,10 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
                     float4 raw[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) raw[u] = key[2 * c + u];
+                    tie(query_offset, score);
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        score = dot_piece(q + (c + u) * 8,
+                        score = dot_piece(q + query_offset + (c + u) * 8,
                                           from_floats(raw[2 * u], raw[2 * u + 1], as_cached), score);
                     }
                 }
@@ -483,13 +558,14 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
                     uint4 raw[4];
 #pragma unroll
                     for (int u = 0; u < 4; ++u) raw[u] = key[c + u];
+                    tie(query_offset, score);
 #pragma unroll
                     for (int u = 0; u < 4; ++u) {
-                        score = dot_piece(q + (c + u) * 8, unpack_bf16(raw[u]), score);
+                        score = dot_piece(q + query_offset + (c + u) * 8, unpack_bf16(raw[u]), score);
                     }
                 }
             }
-            const float weight = fold(score);
+            const float weight = fold(score, live);
             for (int t0 = 0; t0 < kPieces; t0 += 4) {
                 if (t0 * kKeysPerLoad > in_tile) break;  // wave-uniform: only dead keys left
                 uint4 cached[4];
@@ -606,7 +682,8 @@ bool vector_form_fits(const AttentionArguments& arguments) {
     };
     const std::int64_t head_dim = arguments.head_dim;
     return (head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
-        arguments.cache_row_stride % 8 == 0 && arguments.cache_capacity >= kWave &&
+        arguments.cache_row_stride % 8 == 0 && arguments.cache_row_stride < (1 << 24) &&
+        arguments.cache_capacity >= kWave &&
         aligned(arguments.key_cache) && aligned(arguments.value_cache) &&
         aligned(arguments.block_key) && aligned(arguments.block_value);
 }
