@@ -756,8 +756,11 @@ int nfn_mi355_k_quant_gemm_multi_float32_v1(
 
 /* One-token attention with a workspace: nfn_native_tile_glimmer_gqa_decode_float32_v1
  * runs one workgroup per query head because it has nowhere to put partial
- * results; with a workspace the keys of every head are dealt over up to 32
- * workgroups and a second launch merges their partial sums.  Same descriptor,
+ * results; with a workspace the keys of every head are dealt over many
+ * workgroups (up to 128 shares) and a second launch merges their partial sums.
+ * With head_dim 128 and four or more query heads per key/value head a
+ * workgroup serves up to 16 query heads of one key/value head on the matrix
+ * cores, so a cache row is read once for all of them.  Same descriptor,
  * same semantics, same tolerance against the double-precision formula; the
  * summation order differs, so the bits can differ from the ordinary entry
  * point (and the causal-block equality rule is stated for that one).  The
@@ -775,6 +778,18 @@ int nfn_mi355_gqa_decode_split_v1(
  * merge).  Same descriptor, same workspace as nfn_mi355_gqa_decode_split_v1. */
 int nfn_mi355_fused_decode_attention_split_v1(
     const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor,
+    void* workspace,
+    int64_t workspace_nbytes);
+
+/* nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1
+ * (position read from device memory when the kernels run, so one captured
+ * graph serves every token) with the split attention form: the shares are cut
+ * from the row's real key count on the device.  Arguments as in the two entry
+ * points it combines. */
+int nfn_mi355_fused_decode_attention_split_device_position_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* descriptor,
+    const int64_t* device_position,
+    int64_t sliding_window,
     void* workspace,
     int64_t workspace_nbytes);
 

@@ -153,7 +153,10 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
     attention.cache_capacity = d->cache_capacity;
     attention.cache_row_stride = d->cache_row_stride;
     attention.scale = d->attention_scale;
-    if (on_device) {
+    if (on_device && split_partials != nullptr) {
+        launch_gqa_decode_split_device_position(attention, device_position, sliding_window,
+                                                d->apply_rope == 0, split_partials, stream);
+    } else if (on_device) {
         // a local layer (rope applied) sees its window, a global one everything
         launch_gqa_decode_device_position(attention, device_position, sliding_window,
                                           d->apply_rope == 0, stream);
@@ -298,6 +301,20 @@ int nfn_mi355_fused_decode_attention_split_v1(
         nfn_mi355_gqa_decode_split_workspace_bytes_v1(d->query_heads, d->head_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
     return run_fused_decode(d, nullptr, 0, static_cast<float*>(workspace));
+}
+
+int nfn_mi355_fused_decode_attention_split_device_position_v1(
+    const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1* d,
+    const std::int64_t* device_position, std::int64_t sliding_window, void* workspace,
+    std::int64_t workspace_nbytes) {
+    if (d == nullptr || device_position == nullptr || workspace == nullptr ||
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
+        return kInvalid;
+    }
+    const std::int64_t required =
+        nfn_mi355_gqa_decode_split_workspace_bytes_v1(d->query_heads, d->head_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    return run_fused_decode(d, device_position, sliding_window, static_cast<float*>(workspace));
 }
 
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(

@@ -20,7 +20,8 @@ namespace {
 
 constexpr int kMaxWaves = 8;   // 512 threads: 256 vector registers per lane
 constexpr int kMaxHeadDim = 256;
-constexpr int kMaxSplits = 32;  // most shares of one head's keys in the split form
+constexpr int kMaxSplits = 128;    // most shares of one head's keys in the split form
+constexpr int kVectorSplits = 32;  // ... when every query head has workgroups of its own
 constexpr int kOwned = kMaxHeadDim / kWave;  // output dimensions per lane
 
 struct AttentionArguments {
@@ -657,23 +658,368 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_vector_kernel(Att
 }
 
 // Split form, second launch: one workgroup per (query row, query head) merges
-// the shares in order.
-__global__ __launch_bounds__(kMaxHeadDim) void attention_merge_kernel(
+// the shares.  Four threads share an output dimension and take every fourth
+// share each, so that the loads of many shares are in flight together (read
+// one after the other, 32 shares cost more than the attention itself).
+constexpr int kMergeLanes = 4;
+
+__global__ __launch_bounds__(kMaxHeadDim * kMergeLanes) void attention_merge_kernel(
     const float* __restrict__ partials, float* __restrict__ output, int splits, int head_dim) {
-    const float* mine = partials + static_cast<std::int64_t>(blockIdx.x) * splits *
-        partial_floats(head_dim);
-    float overall = -INFINITY;
-    for (int s = 0; s < splits; ++s) overall = fmaxf(overall, mine[s * partial_floats(head_dim)]);
-    float total = 0.0f;
+    __shared__ float factor[kMaxSplits];
+    __shared__ float wave_part[2][kMaxHeadDim * kMergeLanes / kWave];
+    __shared__ float lane_sum[kMergeLanes][kMaxHeadDim];
+    const std::int64_t stride = partial_floats(head_dim);
+    const float* mine = partials + static_cast<std::int64_t>(blockIdx.x) * splits * stride;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int dims = static_cast<int>(blockDim.x) / kMergeLanes;  // head_dim rounded up to waves
+
+    // thread s holds share s (at most 128 shares, at least 256 threads)
+    const float maximum = tid < splits ? mine[tid * stride] : -INFINITY;
+    const float denominator = tid < splits ? mine[tid * stride + 1] : 0.0f;
+    const float wave_maximum = wave_max_f(maximum);
+    if (lane == 0) wave_part[0][wave] = wave_maximum;
+    __syncthreads();
+    const float overall = fmaxf(wave_part[0][0], wave_part[0][1]);
+    const float mine_factor = expf(maximum - overall);  // 0 for an empty share
+    if (tid < splits) factor[tid] = mine_factor;
+    const float wave_total = wave_sum_f(denominator * mine_factor);
+    if (lane == 0) wave_part[1][wave] = wave_total;
+    __syncthreads();
+    const float total = wave_part[1][0] + wave_part[1][1];
+
+    const int d = tid % dims;
+    const int share_lane = tid / dims;
     float sum = 0.0f;
-    const int d = threadIdx.x;
-    for (int s = 0; s < splits; ++s) {
-        const float* share = mine + s * partial_floats(head_dim);
-        const float factor = expf(share[0] - overall);  // 0 for an empty share
-        total = fmaf(share[1], factor, total);
-        if (d < head_dim) sum = fmaf(share[2 + d], factor, sum);
+    if (d < head_dim) {
+#pragma unroll 4
+        for (int s = share_lane; s < splits; s += kMergeLanes) {
+            sum = fmaf(mine[s * stride + 2 + d], factor[s], sum);
+        }
     }
-    if (d < head_dim) output[static_cast<std::int64_t>(blockIdx.x) * head_dim + d] = sum / total;
+    lane_sum[share_lane][d] = sum;
+    __syncthreads();
+    if (share_lane == 0 && d < head_dim) {
+        const float all = (lane_sum[0][d] + lane_sum[1][d]) + (lane_sum[2][d] + lane_sum[3][d]);
+        output[static_cast<std::int64_t>(blockIdx.x) * head_dim + d] = all / total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Grouped one-token form on the matrix cores (split form only, head_dim 128):
+// one workgroup per (key/value head, group of up to 16 of its query heads,
+// share of the keys).  All query heads of a group read a key/value row once.
+//
+// Lane = (j, i) = (lane / 16, lane % 16).  Scores of 16 keys x 16 heads are one
+// accumulator of v_mfma_f32_16x16x32_bf16 per 32 dimensions: operand A is the
+// cached key as it lies in memory (lane (j, i): key i, dimensions 8j..8j+7 of
+// the 32), operand B the query of head i cut into three bf16 terms whose sum is
+// the float, so that every product is exact.  The result leaves lane (j, i)
+// with keys 4j..4j+3 of head i -- which is operand A of v_mfma_f32_16x16x4_f32
+// (head i, k = j) for the weighted sum if the instruction's k index is read as
+// "key 4j + r"; operand B is then lane (j, i)'s own load of value row 4j + r,
+// dimensions 8i..8i+7, one instruction per dimension e of the eight with
+// column i standing for dimension 8i + e.  Values and weights stay floats.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kGroupWaves = 4;
+constexpr int kGroupHeads = 16;
+constexpr int kGroupHeadDim = 128;
+constexpr int kGroupRowPad = 4;  // floats between the rows of a wave's result in LDS
+constexpr int kGroupMinHeads = 4;  // fewer query heads per key/value head: the vector form
+
+struct QueryTerms {
+    bf16x8 high, middle, low;
+};
+
+// x = high + middle + low exactly, every term a bf16: each term takes the next eight
+// significant bits of what is left (truncation, so the remainders are exact)
+__device__ __forceinline__ QueryTerms split_query(const float (&x)[8]) {
+    std::uint32_t words[3][4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        std::uint32_t term[3][2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            float rest = x[2 * w + half];
+#pragma unroll
+            for (int t = 0; t < 3; ++t) {
+                term[t][half] = __float_as_uint(rest) & 0xffff0000u;
+                rest -= __uint_as_float(term[t][half]);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 3; ++t) words[t][w] = (term[t][0] >> 16) | term[t][1];
+    }
+    QueryTerms terms;
+    terms.high = __builtin_bit_cast(bf16x8, make_uint4(words[0][0], words[0][1], words[0][2], words[0][3]));
+    terms.middle = __builtin_bit_cast(bf16x8, make_uint4(words[1][0], words[1][1], words[1][2], words[1][3]));
+    terms.low = __builtin_bit_cast(bf16x8, make_uint4(words[2][0], words[2][1], words[2][2], words[2][3]));
+    return terms;
+}
+
+__global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(AttentionArguments a) {
+    __shared__ float wave_maximum[kGroupWaves][kGroupHeads];
+    __shared__ float wave_denominator[kGroupWaves][kGroupHeads];
+    __shared__ __attribute__((aligned(16))) float
+        wave_accumulator[kGroupWaves][kGroupHeads][kGroupHeadDim + kGroupRowPad];
+
+    resolve_position(a);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = static_cast<int>(blockDim.x >> 6);
+    const int j = lane >> 4;
+    const int i = lane & 15;
+    const std::uint32_t groups_per_kv = (a.heads_per_kv + kGroupHeads - 1) / kGroupHeads;
+    const std::uint32_t kv_head = blockIdx.x / groups_per_kv;
+    const std::uint32_t head_group = blockIdx.x % groups_per_kv;
+    const int heads_here = static_cast<int>(
+        a.heads_per_kv - head_group * kGroupHeads < kGroupHeads
+            ? a.heads_per_kv - head_group * kGroupHeads : kGroupHeads);
+    const std::int64_t first_head =
+        static_cast<std::int64_t>(kv_head) * a.heads_per_kv + head_group * kGroupHeads;
+    const KeyRange range = key_range(a, 0, waves);
+    const int active = range.active;
+    // the row's own key is the block row, everything before it is in the cache
+    const bool has_current = active > 0 && range.last >= a.context_length;
+    const std::int64_t cached_last = has_current ? a.context_length - 1 : range.last;
+    const std::int64_t head_offset = static_cast<std::int64_t>(kv_head) * kGroupHeadDim;
+
+    // query of head i, dimensions 32s + 8j .. + 7 (zeros for the heads a group lacks)
+    const float* query = a.query + (first_head + i) * kGroupHeadDim + 8 * j;
+    QueryTerms q[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        float x[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (i < heads_here) {
+            const float4 low = *reinterpret_cast<const float4*>(query + 32 * s);
+            const float4 high = *reinterpret_cast<const float4*>(query + 32 * s + 4);
+            x[0] = low.x, x[1] = low.y, x[2] = low.z, x[3] = low.w;
+            x[4] = high.x, x[5] = high.y, x[6] = high.z, x[7] = high.w;
+        }
+        q[s] = split_query(x);
+    }
+
+    const std::int64_t capacity = a.cache_capacity;
+    const std::int64_t tile_step = static_cast<std::int64_t>(active) * kWave;
+    const std::int64_t slot_step = tile_step % capacity;
+    std::int64_t tile_slot = (range.first + static_cast<std::int64_t>(wave) * kWave) % capacity;
+    const auto ring_row = [capacity](std::int64_t slot) {  // slot < 2 * capacity
+        return slot >= capacity ? slot - capacity : slot;
+    };
+
+    float maximum = -INFINITY;  // of head i; the same in the four lanes (., i)
+    float denominator = 0.0f;
+    f32x4 accumulator[8];  // [e][r]: head 4j + r, dimension 8i + e
+#pragma unroll
+    for (int e = 0; e < 8; ++e) accumulator[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // running state of head i takes in `tile_maximum` and the weights' sum; the
+    // accumulator rows (heads 4j + r) are scaled by their heads' factors
+    const auto rescale = [&](float keep) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float keep_r = __shfl(keep, 4 * j + r);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) accumulator[e][r] *= keep_r;
+        }
+    };
+    const auto across_j_max = [](float value) {
+        value = fmaxf(value, __shfl_xor(value, 16));
+        return fmaxf(value, __shfl_xor(value, 32));
+    };
+    const auto across_j_sum = [](float value) {
+        value += __shfl_xor(value, 16);
+        return value + __shfl_xor(value, 32);
+    };
+
+    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
+         wave < active && tile <= cached_last;
+         tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
+        // keys past the range repeat the last key of the tile with weight 0
+        const int in_tile =
+            static_cast<int>(cached_last - tile < kWave - 1 ? cached_last - tile : kWave - 1);
+        uint4 key_raw[4][4], value_raw[4][4];
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+            const int key = block * 16 + i < in_tile ? block * 16 + i : in_tile;
+            const std::uint16_t* row = a.key_cache +
+                ring_row(tile_slot + key) * a.cache_row_stride + head_offset + 8 * j;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                key_raw[block][s] = *reinterpret_cast<const uint4*>(row + 32 * s);
+            }
+        }
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int wanted = block * 16 + 4 * j + r;
+                const int key = wanted < in_tile ? wanted : in_tile;
+                value_raw[block][r] = *reinterpret_cast<const uint4*>(
+                    a.value_cache + ring_row(tile_slot + key) * a.cache_row_stride + head_offset +
+                    8 * i);
+            }
+        }
+
+        // scores: the small terms of the query first
+        f32x4 score[4];
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+            f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].low, sum, 0, 0, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].middle, sum, 0, 0, 0);
+            }
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].high, sum, 0, 0, 0);
+            }
+            score[block] = sum;
+        }
+
+        float tile_maximum = -INFINITY;
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool live = block * 16 + 4 * j + r <= in_tile;
+                score[block][r] = live ? score[block][r] * a.scale : -INFINITY;
+                tile_maximum = fmaxf(tile_maximum, score[block][r]);
+            }
+        }
+        const float next_maximum = fmaxf(maximum, across_j_max(tile_maximum));
+        const float keep = expf(maximum - next_maximum);  // 0 on the first tile
+        float weights = 0.0f;
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                score[block][r] = expf(score[block][r] - next_maximum);  // 0 for a dead key
+                weights += score[block][r];
+            }
+        }
+        denominator = denominator * keep + across_j_sum(weights);
+        maximum = next_maximum;
+        rescale(keep);
+
+#pragma unroll
+        for (int block = 0; block < 4; ++block) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const Piece value = unpack_bf16(value_raw[block][r]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    accumulator[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                        score[block][r], value.v[e], accumulator[e], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // The row's own key and value (floats, not in the cache): the first wave of
+    // the share that holds them.
+    if (has_current && wave == 0) {
+        const float* key = a.block_key + head_offset + 8 * j;
+        float dot = 0.0f;
+        if (i < heads_here) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float4 q_low = *reinterpret_cast<const float4*>(query + 32 * s);
+                const float4 q_high = *reinterpret_cast<const float4*>(query + 32 * s + 4);
+                const float4 k_low = *reinterpret_cast<const float4*>(key + 32 * s);
+                const float4 k_high = *reinterpret_cast<const float4*>(key + 32 * s + 4);
+                dot = fmaf(q_low.x, k_low.x, dot);
+                dot = fmaf(q_low.y, k_low.y, dot);
+                dot = fmaf(q_low.z, k_low.z, dot);
+                dot = fmaf(q_low.w, k_low.w, dot);
+                dot = fmaf(q_high.x, k_high.x, dot);
+                dot = fmaf(q_high.y, k_high.y, dot);
+                dot = fmaf(q_high.z, k_high.z, dot);
+                dot = fmaf(q_high.w, k_high.w, dot);
+            }
+        }
+        const float score = across_j_sum(dot) * a.scale;
+        const float next_maximum = fmaxf(maximum, score);
+        const float keep = expf(maximum - next_maximum);
+        const float weight = expf(score - next_maximum);
+        denominator = denominator * keep + weight;
+        maximum = next_maximum;
+        rescale(keep);
+        const float* value_row = a.block_value + head_offset + 8 * i;
+        const float4 v_low = *reinterpret_cast<const float4*>(value_row);
+        const float4 v_high = *reinterpret_cast<const float4*>(value_row + 4);
+        const float value[8] = {v_low.x, v_low.y, v_low.z, v_low.w,
+                                v_high.x, v_high.y, v_high.z, v_high.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float weight_r = __shfl(weight, 4 * j + r);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                accumulator[e][r] = fmaf(weight_r, value[e], accumulator[e][r]);
+            }
+        }
+    }
+
+    if (j == 0) {
+        wave_maximum[wave][i] = maximum;
+        wave_denominator[wave][i] = denominator;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float* target = &wave_accumulator[wave][4 * j + r][8 * i];
+        *reinterpret_cast<float4*>(target) = make_float4(
+            accumulator[0][r], accumulator[1][r], accumulator[2][r], accumulator[3][r]);
+        *reinterpret_cast<float4*>(target + 4) = make_float4(
+            accumulator[4][r], accumulator[5][r], accumulator[6][r], accumulator[7][r]);
+    }
+    __syncthreads();
+
+    // unnormalised, relative to this share's maximum; an empty share says (-inf, 0, 0).
+    // A thread takes eight dimensions of a head.
+    for (int item = tid; item < heads_here * (kGroupHeadDim / 8); item += blockDim.x) {
+        const int head = item / (kGroupHeadDim / 8);
+        const int piece = item % (kGroupHeadDim / 8);
+        float overall = active > 0 ? wave_maximum[0][head] : -INFINITY;
+        for (int w = 1; w < active; ++w) overall = fmaxf(overall, wave_maximum[w][head]);
+        float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        float total = 0.0f;
+        for (int w = 0; w < active; ++w) {
+            const float factor = expf(wave_maximum[w][head] - overall);
+            const float* row = &wave_accumulator[w][head][8 * piece];
+            const float4 low = *reinterpret_cast<const float4*>(row);
+            const float4 high = *reinterpret_cast<const float4*>(row + 4);
+            sum[0] = fmaf(low.x, factor, sum[0]);
+            sum[1] = fmaf(low.y, factor, sum[1]);
+            sum[2] = fmaf(low.z, factor, sum[2]);
+            sum[3] = fmaf(low.w, factor, sum[3]);
+            sum[4] = fmaf(high.x, factor, sum[4]);
+            sum[5] = fmaf(high.y, factor, sum[5]);
+            sum[6] = fmaf(high.z, factor, sum[6]);
+            sum[7] = fmaf(high.w, factor, sum[7]);
+            total = fmaf(wave_denominator[w][head], factor, total);
+        }
+        // a partial row starts 8-byte aligned, and so does its third float
+        float* partial = a.partials +
+            ((first_head + head) * a.splits + blockIdx.y) * partial_floats(kGroupHeadDim);
+        if (piece == 0) *reinterpret_cast<float2*>(partial) = make_float2(overall, total);
+        float2* target = reinterpret_cast<float2*>(partial + 2 + 8 * piece);
+        target[0] = make_float2(sum[0], sum[1]);
+        target[1] = make_float2(sum[2], sum[3]);
+        target[2] = make_float2(sum[4], sum[5]);
+        target[3] = make_float2(sum[6], sum[7]);
+    }
 }
 
 bool vector_form_fits(const AttentionArguments& arguments) {
@@ -759,28 +1105,71 @@ std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int
     return query_heads * kMaxSplits * partial_floats(head_dim) * 4;
 }
 
+namespace {
+
+// Split form of the one-token call.  `tiles`: the 64-key tiles of the row, or
+// with a position in device memory the most it can have (the shares are cut
+// from the row's real key count when the kernel runs; surplus shares are empty).
+void launch_split(AttentionArguments a, std::int64_t tiles, float* partials, hipStream_t stream) {
+    a.partials = partials;
+    const std::int64_t heads_per_kv = a.heads_per_kv;
+    if (a.head_dim == kGroupHeadDim && heads_per_kv >= kGroupMinHeads) {
+        // Matrix-core form: a workgroup serves up to 16 query heads of one key/value
+        // head.  As many shares as fill the chip, then up to four waves a share.
+        const std::int64_t groups = a.kv_heads * ((heads_per_kv + kGroupHeads - 1) / kGroupHeads);
+        std::int64_t splits = compute_units() / groups;
+        if (splits > kMaxSplits) splits = kMaxSplits;
+        if (splits > tiles) splits = tiles;
+        if (splits < 2) splits = 2;
+        a.splits = static_cast<int>(splits);
+        std::int64_t waves = (tiles + splits - 1) / splits;
+        if (waves > kGroupWaves) waves = kGroupWaves;
+        hipLaunchKernelGGL(attention_grouped_kernel,
+                           dim3(static_cast<unsigned>(groups), static_cast<unsigned>(splits)),
+                           dim3(static_cast<unsigned>(waves * kWave)), 0, stream, a);
+    } else {
+        // About one workgroup of up to eight waves per compute unit.
+        std::int64_t splits = compute_units() / a.query_heads;
+        if (splits > kVectorSplits) splits = kVectorSplits;
+        if (splits > tiles) splits = tiles;
+        if (splits < 2) splits = 2;
+        a.splits = static_cast<int>(splits);
+        launch_attention(a, 1, (tiles + a.splits - 1) / a.splits, stream);
+    }
+    const int threads = static_cast<int>((a.head_dim + kWave - 1) / kWave * kWave) * kMergeLanes;
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(static_cast<unsigned>(a.query_heads)),
+                       dim3(threads), 0, stream, partials, a.output, a.splits,
+                       static_cast<int>(a.head_dim));
+}
+
+}  // namespace
+
 void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d, float* partials,
                              hipStream_t stream) {
-    AttentionArguments a = decode_arguments(d);
+    const AttentionArguments a = decode_arguments(d);
     const std::int64_t tiles = tiles_of(a.sliding_window);
     if (!vector_form_fits(a) || tiles < 2) {
         launch_attention(a, 1, tiles, stream);  // nothing to split, or no vector form: one launch
         return;
     }
-    a.partials = partials;
-    // About one workgroup of up to eight waves per compute unit: fewer, fatter
-    // shares beat many small ones (every workgroup pays for the query load, the
-    // ring arithmetic and a partial row).
-    std::int64_t splits = compute_units() / d.query_heads;
-    if (splits > kMaxSplits) splits = kMaxSplits;
-    if (splits > tiles) splits = tiles;
-    if (splits < 2) splits = 2;
-    a.splits = static_cast<int>(splits);
-    launch_attention(a, 1, (tiles + a.splits - 1) / a.splits, stream);
-    const int threads = static_cast<int>((d.head_dim + kWave - 1) / kWave * kWave);
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(static_cast<unsigned>(d.query_heads)),
-                       dim3(threads), 0, stream, partials, d.output, a.splits,
-                       static_cast<int>(d.head_dim));
+    launch_split(a, tiles, partials, stream);
+}
+
+void launch_gqa_decode_split_device_position(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d,
+                                             const std::int64_t* device_position,
+                                             std::int64_t sliding_window, bool whole_context,
+                                             float* partials, hipStream_t stream) {
+    AttentionArguments a = decode_arguments(d);
+    a.device_position = device_position;
+    a.sliding_window = sliding_window;
+    a.whole_context = whole_context ? 1 : 0;
+    if (!vector_form_fits(a)) {
+        launch_attention(a, 1, kMaxWaves, stream);
+        return;
+    }
+    // a global layer sees at most the ring and the row's own key
+    launch_split(a, tiles_of(whole_context ? d.cache_capacity + 1 : sliding_window), partials,
+                 stream);
 }
 
 void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& d,

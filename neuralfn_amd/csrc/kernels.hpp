@@ -104,6 +104,11 @@ void launch_gqa_decode_device_position(const NfnNativeTileGlimmerGqaDecodeDescri
 std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int64_t head_dim);
 void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
                              float* partials, hipStream_t stream);
+// The same with the position read from device memory when the kernels run (the
+// meaning of `sliding_window` and `whole_context` as in the one-launch form).
+void launch_gqa_decode_split_device_position(
+    const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor, const std::int64_t* device_position,
+    std::int64_t sliding_window, bool whole_context, float* partials, hipStream_t stream);
 
 // clock_probe.hip — out[0] = shader cycles, out[1] = ticks of the constant
 // clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.

@@ -125,7 +125,11 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     d.rope_layout = layout
     d.apply_rope = 1 if apply_rope else 0
     d.cuda_stream = stream
-    if workspace is not None:
+    if workspace is not None and device_position is not None:
+        check(load().nfn_mi355_fused_decode_attention_split_device_position_v1(
+            ctypes.byref(d), device_position.data_ptr(), sliding_window, workspace.data_ptr(),
+            workspace.numel()), "fused_decode_attention_split_device_position")
+    elif workspace is not None:
         check(load().nfn_mi355_fused_decode_attention_split_v1(
             ctypes.byref(d), workspace.data_ptr(), workspace.numel()), "fused_decode_attention_split")
     elif device_position is not None:

@@ -194,6 +194,8 @@ SIGNATURES = {
     "nfn_mi355_gqa_decode_split_v1": (ctypes.c_int, [ctypes.POINTER(GqaDecodeDescriptor), _P, _I64]),
     "nfn_mi355_fused_decode_attention_split_v1": (
         ctypes.c_int, [ctypes.POINTER(FusedDecodeAttentionDescriptor), _P, _I64]),
+    "nfn_mi355_fused_decode_attention_split_device_position_v1": (
+        ctypes.c_int, [ctypes.POINTER(FusedDecodeAttentionDescriptor), _P, _I64, _P, _I64]),
     "nfn_native_tile_glimmer_embedding_gather_float32_v1": (ctypes.c_int, [_DESC, _I64, _P]),
     "nfn_native_tile_glimmer_embedding_gather_device_i64_float32_v1": (ctypes.c_int, [_DESC, _P, _P]),
     "nfn_native_tile_glimmer_embedding_batch_i32_float32_v1": (ctypes.c_int, [_DESC, _P, _P, _I64]),

@@ -250,6 +250,13 @@ def test_gqa_against_oracle(cuda, oracle, query_heads, kv_heads, head_dim, posit
     (4, 1, 256, 130, 2, 2048),        # three tiles
     (6, 3, 128, 70, 7, 64),           # one tile: nothing to split
     (6, 3, 50, 300, 100, 256),        # no vector form: the ordinary kernel
+    # head_dim 128 with four or more query heads per key/value head: the matrix-core kernel
+    (32, 2, 128, 2047, 0, 2048),      # 2048 keys: 32 full tiles, the current key closes the last
+    (32, 2, 128, 2048, 1, 2048),      # the current key alone in its tile; the ring is full and wraps
+    (8, 2, 128, 64, 0, 128),          # one cached tile and the current key
+    (20, 1, 128, 333, 40, 512),       # two groups of query heads (16 + 4), a window, ragged last tile
+    (48, 3, 128, 40000, 0, 65536),    # 626 tiles: 85 shares, more than one tile a wave
+    (4, 1, 128, 700, 130, 640),       # the fewest grouped heads; window wraps the ring
 ])
 def test_gqa_split_form_against_oracle(cuda, oracle, query_heads, kv_heads, head_dim, position, first,
                                        capacity):
@@ -601,9 +608,24 @@ def test_fused_decode_attention_with_the_position_on_the_device(cuda, oracle, ap
     assert_bits_equal(q2, q1, "query")
     assert_bits_equal(k2, k1, "key")
     assert np.array_equal(bits_of(kc2), bits_of(kc1)) and np.array_equal(bits_of(vc2), bits_of(vc1))
+    # the split form with the position on the device: one workspace and one launch geometry
+    # for every position (shares are cut on the device; those past the row's keys stay empty)
+    q3, k3, v3 = to_device(query, cuda), to_device(key, cuda), to_device(value, cuda)
+    kc3, vc3 = bf16_tensor(keys, cuda), bf16_tensor(values, cuda)
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+    workspace.fill_(0xFF)
+    split = engine_ops.fused_decode_attention(q3, k3, v3, kc3, vc3, 7, 3, head_dim ** -0.5,
+                                              device_position=device_position,
+                                              sliding_window=window, workspace=workspace, **common)
+    assert np.abs(split.cpu().numpy() - host.cpu().numpy()).max() <= 4e-6
+    assert_bits_equal(q3, q1, "query, split form")
+    assert np.array_equal(bits_of(kc3), bits_of(kc1)) and np.array_equal(bits_of(vc3), bits_of(vc1))
     lib = tile_ops.load()
     call = lib.nfn_native_tile_glimmer_fused_decode_attention_device_position_float32_v1
     assert call(None, device_position.data_ptr(), window) == 1
+    split_call = lib.nfn_mi355_fused_decode_attention_split_device_position_v1
+    assert split_call(None, device_position.data_ptr(), window, workspace.data_ptr(),
+                      workspace.numel()) == 1
 
 
 def test_cache_commit_layers_and_pack_target_taps(cuda, oracle):
