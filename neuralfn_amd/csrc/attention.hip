@@ -10,7 +10,9 @@
 // form for head sizes that are multiples of 32 (everything in 16-byte pieces,
 // all loads of a phase in flight together) and a generic element-wise form.
 // The one-token form is the block form with one query row whose own key is
-// the only block row.
+// the only block row.  A third kernel serves head_dim 128 with four or more
+// query heads per key/value head on the matrix cores, one workgroup per group
+// of up to 16 such heads: the split one-token form and blocks of many rows.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -711,24 +713,33 @@ __global__ __launch_bounds__(kMaxHeadDim * kMergeLanes) void attention_merge_ker
 // one workgroup per (key/value head, group of up to 16 of its query heads,
 // share of the keys).  All query heads of a group read a key/value row once.
 //
-// Lane = (j, i) = (lane / 16, lane % 16).  Scores of 16 keys x 16 heads are one
-// accumulator of v_mfma_f32_16x16x32_bf16 per 32 dimensions: operand A is the
-// cached key as it lies in memory (lane (j, i): key i, dimensions 8j..8j+7 of
-// the 32), operand B the query of head i cut into three bf16 terms whose sum is
-// the float, so that every product is exact.  The result leaves lane (j, i)
-// with keys 4j..4j+3 of head i -- which is operand A of v_mfma_f32_16x16x4_f32
-// (head i, k = j) for the weighted sum if the instruction's k index is read as
-// "key 4j + r"; operand B is then lane (j, i)'s own load of value row 4j + r,
-// dimensions 8i..8i+7, one instruction per dimension e of the eight with
-// column i standing for dimension 8i + e.  Values and weights stay floats.
+// Lane = (j, i) = (lane / 16, lane % 16).  Both products run on
+// v_mfma_f32_16x16x32_bf16 with float operands cut into three bf16 terms whose sum
+// is the float, so that every product is exact (cache rows are bf16 already).
+//
+// Scores of 16 keys x 16 heads, one accumulator per 32 dimensions: operand A is the
+// cached key as it lies in memory (lane (j, i): key i, dimensions 8j..8j+7 of the
+// 32), operand B the query of head i.  The result leaves lane (j, i) with keys
+// 4j..4j+3 of head i, for four blocks of 16 keys a tile.
+//
+// Weighted sum over 32 keys at a time: operand A is the weights of head i as the
+// lane holds them (the instruction's k index 8j + e read as "key 4j + e % 4 of
+// block e / 4" of the 32), operand B wants, for one dimension, the values of those
+// eight keys -- a column of the cache.  A wave therefore stages its tile's value
+// rows in LDS (rows of 272 bytes: a row's 256 and a pad that spreads the four j
+// over the banks) and reads them back a dword at a time: dimensions 2i and 2i + 1
+// of a key, whose halves go to two instructions (column i standing for dimension
+// 32p + 2i in one and 32p + 2i + 1 in the other).
 // ---------------------------------------------------------------------------
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kGroupWaves = 4;
+constexpr int kGroupWaves = 8;
 constexpr int kGroupHeads = 16;
 constexpr int kGroupHeadDim = 128;
 constexpr int kGroupRowPad = 4;  // floats between the rows of a wave's result in LDS
+constexpr int kStageRowBytes = 2 * kGroupHeadDim + 16;  // a staged value row and its pad
+constexpr int kStageBytes = kWave * kStageRowBytes;      // a wave's tile of value rows
 constexpr int kGroupMinHeads = 4;  // fewer query heads per key/value head: the vector form
 
 struct QueryTerms {
@@ -752,7 +763,9 @@ __device__ __forceinline__ QueryTerms split_query(const float (&x)[8]) {
             }
         }
 #pragma unroll
-        for (int t = 0; t < 3; ++t) words[t][w] = (term[t][0] >> 16) | term[t][1];
+        for (int t = 0; t < 3; ++t) {
+            words[t][w] = __builtin_amdgcn_perm(term[t][1], term[t][0], 0x07060302u);
+        }
     }
     QueryTerms terms;
     terms.high = __builtin_bit_cast(bf16x8, make_uint4(words[0][0], words[0][1], words[0][2], words[0][3]));
@@ -761,11 +774,20 @@ __device__ __forceinline__ QueryTerms split_query(const float (&x)[8]) {
     return terms;
 }
 
+// eight floats as the bf16 row the cache would hold of them
+__device__ __forceinline__ uint4 pack_as_cached(float4 low, float4 high) {
+    const auto pair = [](float first, float second) {
+        return static_cast<std::uint32_t>(to_bf16(first)) |
+            (static_cast<std::uint32_t>(to_bf16(second)) << 16);
+    };
+    return make_uint4(pair(low.x, low.y), pair(low.z, low.w), pair(high.x, high.y),
+                      pair(high.z, high.w));
+}
+
 __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(AttentionArguments a) {
-    __shared__ float wave_maximum[kGroupWaves][kGroupHeads];
-    __shared__ float wave_denominator[kGroupWaves][kGroupHeads];
-    __shared__ __attribute__((aligned(16))) float
-        wave_accumulator[kGroupWaves][kGroupHeads][kGroupHeadDim + kGroupRowPad];
+    // waves x kStageBytes: a value tile per wave; at the end the waves' results
+    // (maxima, denominators, accumulators: less than that) in the same memory
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t grouped_lds[];
 
     resolve_position(a);
     const int tid = threadIdx.x;
@@ -774,23 +796,35 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
     const int waves = static_cast<int>(blockDim.x >> 6);
     const int j = lane >> 4;
     const int i = lane & 15;
+    std::uint8_t* stage = grouped_lds + wave * kStageBytes;
+    // workgroup = (query row, key/value head, group of its query heads); all fit 32 bits
     const std::uint32_t groups_per_kv = (a.heads_per_kv + kGroupHeads - 1) / kGroupHeads;
-    const std::uint32_t kv_head = blockIdx.x / groups_per_kv;
-    const std::uint32_t head_group = blockIdx.x % groups_per_kv;
+    const std::uint32_t groups_per_row = static_cast<std::uint32_t>(a.kv_heads) * groups_per_kv;
+    const std::int64_t query_row = blockIdx.x / groups_per_row;
+    const std::uint32_t in_row = blockIdx.x % groups_per_row;
+    const std::uint32_t kv_head = in_row / groups_per_kv;
+    const std::uint32_t head_group = in_row % groups_per_kv;
     const int heads_here = static_cast<int>(
         a.heads_per_kv - head_group * kGroupHeads < kGroupHeads
             ? a.heads_per_kv - head_group * kGroupHeads : kGroupHeads);
     const std::int64_t first_head =
         static_cast<std::int64_t>(kv_head) * a.heads_per_kv + head_group * kGroupHeads;
-    const KeyRange range = key_range(a, 0, waves);
+    const KeyRange range = key_range(a, query_row, waves);
     const int active = range.active;
-    // the row's own key is the block row, everything before it is in the cache
-    const bool has_current = active > 0 && range.last >= a.context_length;
-    const std::int64_t cached_last = has_current ? a.context_length - 1 : range.last;
+    // Keys that are bf16 rows go through the matrix cores in tiles: the cache and, for a
+    // causal block, the rows before the query's own (the cache will hold them rounded).
+    // The others are float rows, taken one at a time: the query's own row, or every
+    // row of a block that is not causal.
+    const std::int64_t tiled_end = a.causal != 0 ? a.context_length + query_row : a.context_length;
+    const std::int64_t tiled_last = range.last < tiled_end ? range.last : tiled_end - 1;
+    const std::int64_t float_first = range.first > tiled_end ? range.first : tiled_end;
     const std::int64_t head_offset = static_cast<std::int64_t>(kv_head) * kGroupHeadDim;
+    const std::int64_t block_stride = a.kv_heads * kGroupHeadDim;
 
-    // query of head i, dimensions 32s + 8j .. + 7 (zeros for the heads a group lacks)
-    const float* query = a.query + (first_head + i) * kGroupHeadDim + 8 * j;
+    // query of head i, dimensions 32s + 8j .. + 7 (zeros for the heads a group lacks), as
+    // operand B of the score instructions
+    const float* query =
+        a.query + (query_row * a.query_heads + first_head + i) * kGroupHeadDim + 8 * j;
     QueryTerms q[4];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -814,12 +848,18 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
 
     float maximum = -INFINITY;  // of head i; the same in the four lanes (., i)
     float denominator = 0.0f;
-    f32x4 accumulator[8];  // [e][r]: head 4j + r, dimension 8i + e
+    f32x4 accumulator[8];  // [2p + parity][r]: head 4j + r, dimension 32p + 2i + parity
 #pragma unroll
     for (int e = 0; e < 8; ++e) accumulator[e] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // what a lane wrote to its wave's stage is seen by the other lanes after this, and
+    // the compiler moves no LDS access across it
+    const auto wave_sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
 
-    // running state of head i takes in `tile_maximum` and the weights' sum; the
-    // accumulator rows (heads 4j + r) are scaled by their heads' factors
+    // the accumulator rows (heads 4j + r) are scaled by their heads' factors
     const auto rescale = [&](float keep) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -837,18 +877,19 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
         return value + __shfl_xor(value, 32);
     };
 
-    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
-         wave < active && tile <= cached_last;
-         tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
-        // keys past the range repeat the last key of the tile with weight 0
-        const int in_tile =
-            static_cast<int>(cached_last - tile < kWave - 1 ? cached_last - tile : kWave - 1);
-        uint4 key_raw[4][4], value_raw[4][4];
+    // Loads of one tile of up to 64 bf16 rows starting at key `tile` (ring slot `slot`).
+    // Keys past the range repeat the last key of the tile (their weight will be 0).
+    uint4 key_raw[4][4], value_raw[4][4];
+    // ... a full tile that lies in the cache and does not wrap: one pointer per lane
+    // and operand, the rest are wave-uniform steps
+    const auto load_straight = [&](std::int64_t slot) {
+        const std::uint16_t* key_rows =
+            a.key_cache + (slot + i) * a.cache_row_stride + head_offset + 8 * j;
+        const std::uint16_t* value_rows =
+            a.value_cache + (slot + 4 * j) * a.cache_row_stride + head_offset + 8 * i;
 #pragma unroll
         for (int block = 0; block < 4; ++block) {
-            const int key = block * 16 + i < in_tile ? block * 16 + i : in_tile;
-            const std::uint16_t* row = a.key_cache +
-                ring_row(tile_slot + key) * a.cache_row_stride + head_offset + 8 * j;
+            const std::uint16_t* row = key_rows + block * 16 * a.cache_row_stride;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 key_raw[block][s] = *reinterpret_cast<const uint4*>(row + 32 * s);
@@ -858,35 +899,80 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
         for (int block = 0; block < 4; ++block) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int wanted = block * 16 + 4 * j + r;
-                const int key = wanted < in_tile ? wanted : in_tile;
                 value_raw[block][r] = *reinterpret_cast<const uint4*>(
-                    a.value_cache + ring_row(tile_slot + key) * a.cache_row_stride + head_offset +
-                    8 * i);
+                    value_rows + (block * 16 + r) * a.cache_row_stride);
             }
+        }
+    };
+    // ... any tile: rows of the block are read as floats and rounded the way the cache
+    // commit rounds them
+    const auto load_general = [&](std::int64_t tile, std::int64_t slot, int in_tile) {
+        const auto key_piece = [&](int key, int s) {
+            if (tile + key >= a.context_length) {
+                const float* row = a.block_key +
+                    (tile + key - a.context_length) * block_stride + head_offset + 8 * j + 32 * s;
+                return pack_as_cached(*reinterpret_cast<const float4*>(row),
+                                      *reinterpret_cast<const float4*>(row + 4));
+            }
+            return *reinterpret_cast<const uint4*>(
+                a.key_cache + ring_row(slot + key) * a.cache_row_stride + head_offset + 8 * j +
+                32 * s);
+        };
+        const auto value_piece = [&](int key) {
+            if (tile + key >= a.context_length) {
+                const float* row = a.block_value +
+                    (tile + key - a.context_length) * block_stride + head_offset + 8 * i;
+                return pack_as_cached(*reinterpret_cast<const float4*>(row),
+                                      *reinterpret_cast<const float4*>(row + 4));
+            }
+            return *reinterpret_cast<const uint4*>(
+                a.value_cache + ring_row(slot + key) * a.cache_row_stride + head_offset + 8 * i);
+        };
+        for (int block = 0; block < 4; ++block) {
+            const int key = block * 16 + i < in_tile ? block * 16 + i : in_tile;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) key_raw[block][s] = key_piece(key, s);
+        }
+        for (int block = 0; block < 4; ++block) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int wanted = block * 16 + 4 * j + r;
+                value_raw[block][r] = value_piece(wanted < in_tile ? wanted : in_tile);
+            }
+        }
+    };
+    const auto is_straight = [&](std::int64_t tile, std::int64_t slot) {  // wave-uniform
+        return tile + kWave - 1 <= tiled_last && tile + kWave - 1 < a.context_length &&
+            slot + kWave <= capacity;
+    };
+
+    for (std::int64_t tile = range.first + static_cast<std::int64_t>(wave) * kWave;
+         wave < active && tile <= tiled_last;
+         tile += tile_step, tile_slot = ring_row(tile_slot + slot_step)) {
+        const int in_tile =
+            static_cast<int>(tiled_last - tile < kWave - 1 ? tiled_last - tile : kWave - 1);
+        if (is_straight(tile, tile_slot)) {
+            load_straight(tile_slot);
+        } else {
+            load_general(tile, tile_slot, in_tile);
         }
 
         // scores: the small terms of the query first
         f32x4 score[4];
 #pragma unroll
-        for (int block = 0; block < 4; ++block) {
-            f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int block = 0; block < 4; ++block) score[block] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int term = 0; term < 3; ++term) {
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].low, sum, 0, 0, 0);
-            }
+                const bf16x8 query_term = term == 0 ? q[s].low : term == 1 ? q[s].middle : q[s].high;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].middle, sum, 0, 0, 0);
+                for (int block = 0; block < 4; ++block) {
+                    score[block] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(bf16x8, key_raw[block][s]), query_term, score[block], 0,
+                        0, 0);
+                }
             }
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                sum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8, key_raw[block][s]), q[s].high, sum, 0, 0, 0);
-            }
-            score[block] = sum;
         }
 
         float tile_maximum = -INFINITY;
@@ -900,13 +986,13 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
             }
         }
         const float next_maximum = fmaxf(maximum, across_j_max(tile_maximum));
-        const float keep = expf(maximum - next_maximum);  // 0 on the first tile
+        const float keep = __expf(maximum - next_maximum);  // 0 on the first tile
         float weights = 0.0f;
 #pragma unroll
         for (int block = 0; block < 4; ++block) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                score[block][r] = expf(score[block][r] - next_maximum);  // 0 for a dead key
+                score[block][r] = __expf(score[block][r] - next_maximum);  // 0 for a dead key
                 weights += score[block][r];
             }
         }
@@ -914,24 +1000,69 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
         maximum = next_maximum;
         rescale(keep);
 
+        // the tile's value rows into the stage: key block * 16 + 4j + r, dimensions 8i..
+        wave_sync();  // the reads of the previous tile are done
 #pragma unroll
         for (int block = 0; block < 4; ++block) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const Piece value = unpack_bf16(value_raw[block][r]);
+                *reinterpret_cast<uint4*>(stage + (block * 16 + 4 * j + r) * kStageRowBytes + 16 * i) =
+                    value_raw[block][r];
+            }
+        }
+        wave_sync();
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {  // 32 keys: blocks 2 * half and 2 * half + 1
+            const float weights_here[8] = {
+                score[2 * half][0], score[2 * half][1], score[2 * half][2], score[2 * half][3],
+                score[2 * half + 1][0], score[2 * half + 1][1], score[2 * half + 1][2],
+                score[2 * half + 1][3]};
+            const QueryTerms weight = split_query(weights_here);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                // element e of the operands: key 16 * (2 * half + e / 4) + 4j + e % 4
+                std::uint32_t pair[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    accumulator[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                        score[block][r], value.v[e], accumulator[e], 0, 0, 0);
+                    const int key = 16 * (2 * half + e / 4) + 4 * j + e % 4;
+                    pair[e] = *reinterpret_cast<const std::uint32_t*>(
+                        stage + key * kStageRowBytes + 64 * p + 4 * i);
                 }
+                // dimensions 32p + 2i and 32p + 2i + 1 of the eight keys: the low halves of
+                // two dwords side by side, and the high halves (v_perm_b32 byte selectors)
+                uint4 even, odd;
+                even.x = __builtin_amdgcn_perm(pair[1], pair[0], 0x05040100u);
+                even.y = __builtin_amdgcn_perm(pair[3], pair[2], 0x05040100u);
+                even.z = __builtin_amdgcn_perm(pair[5], pair[4], 0x05040100u);
+                even.w = __builtin_amdgcn_perm(pair[7], pair[6], 0x05040100u);
+                odd.x = __builtin_amdgcn_perm(pair[1], pair[0], 0x07060302u);
+                odd.y = __builtin_amdgcn_perm(pair[3], pair[2], 0x07060302u);
+                odd.z = __builtin_amdgcn_perm(pair[5], pair[4], 0x07060302u);
+                odd.w = __builtin_amdgcn_perm(pair[7], pair[6], 0x07060302u);
+                const bf16x8 even_values = __builtin_bit_cast(bf16x8, even);
+                const bf16x8 odd_values = __builtin_bit_cast(bf16x8, odd);
+                accumulator[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.low, even_values, accumulator[2 * p], 0, 0, 0);
+                accumulator[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.low, odd_values, accumulator[2 * p + 1], 0, 0, 0);
+                accumulator[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.middle, even_values, accumulator[2 * p], 0, 0, 0);
+                accumulator[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.middle, odd_values, accumulator[2 * p + 1], 0, 0, 0);
+                accumulator[2 * p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.high, even_values, accumulator[2 * p], 0, 0, 0);
+                accumulator[2 * p + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    weight.high, odd_values, accumulator[2 * p + 1], 0, 0, 0);
             }
         }
     }
 
-    // The row's own key and value (floats, not in the cache): the first wave of
-    // the share that holds them.
-    if (has_current && wave == 0) {
-        const float* key = a.block_key + head_offset + 8 * j;
+    // Float rows of the block, dealt over the waves that have work (the one-token form has
+    // one, the query's own key, and its first wave takes it).
+    for (std::int64_t position = float_first + wave; wave < active && position <= range.last;
+         position += active) {
+        const std::int64_t block_row = position - a.context_length;
+        const float* key = a.block_key + block_row * block_stride + head_offset + 8 * j;
         float dot = 0.0f;
         if (i < heads_here) {
 #pragma unroll
@@ -957,11 +1088,14 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
         denominator = denominator * keep + weight;
         maximum = next_maximum;
         rescale(keep);
-        const float* value_row = a.block_value + head_offset + 8 * i;
-        const float4 v_low = *reinterpret_cast<const float4*>(value_row);
-        const float4 v_high = *reinterpret_cast<const float4*>(value_row + 4);
-        const float value[8] = {v_low.x, v_low.y, v_low.z, v_low.w,
-                                v_high.x, v_high.y, v_high.z, v_high.w};
+        const float* value_row = a.block_value + block_row * block_stride + head_offset + 2 * i;
+        float value[8];  // [2p + parity]: dimension 32p + 2i + parity
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const float2 two = *reinterpret_cast<const float2*>(value_row + 32 * p);
+            value[2 * p] = two.x;
+            value[2 * p + 1] = two.y;
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float weight_r = __shfl(weight, 4 * j + r);
@@ -972,32 +1106,42 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
         }
     }
 
+    // the stages have been read; the waves' results take their place
+    __syncthreads();
+    constexpr int kRowFloats = kGroupHeadDim + kGroupRowPad;
+    float* wave_maximum = reinterpret_cast<float*>(grouped_lds);           // [waves][16]
+    float* wave_denominator = wave_maximum + waves * kGroupHeads;           // [waves][16]
+    float* wave_accumulator = wave_denominator + waves * kGroupHeads;       // [waves][16][132]
     if (j == 0) {
-        wave_maximum[wave][i] = maximum;
-        wave_denominator[wave][i] = denominator;
+        wave_maximum[wave * kGroupHeads + i] = maximum;
+        wave_denominator[wave * kGroupHeads + i] = denominator;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        float* target = &wave_accumulator[wave][4 * j + r][8 * i];
-        *reinterpret_cast<float4*>(target) = make_float4(
-            accumulator[0][r], accumulator[1][r], accumulator[2][r], accumulator[3][r]);
-        *reinterpret_cast<float4*>(target + 4) = make_float4(
-            accumulator[4][r], accumulator[5][r], accumulator[6][r], accumulator[7][r]);
+        float* target = wave_accumulator + (wave * kGroupHeads + 4 * j + r) * kRowFloats + 2 * i;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            *reinterpret_cast<float2*>(target + 32 * p) =
+                make_float2(accumulator[2 * p][r], accumulator[2 * p + 1][r]);
+        }
     }
     __syncthreads();
 
-    // unnormalised, relative to this share's maximum; an empty share says (-inf, 0, 0).
-    // A thread takes eight dimensions of a head.
+    // The waves' results meet; a thread takes eight dimensions of a head.  The split form
+    // leaves them unnormalised, relative to the share's maximum (an empty share says
+    // (-inf, 0, 0)); otherwise the output row is written.
     for (int item = tid; item < heads_here * (kGroupHeadDim / 8); item += blockDim.x) {
         const int head = item / (kGroupHeadDim / 8);
         const int piece = item % (kGroupHeadDim / 8);
-        float overall = active > 0 ? wave_maximum[0][head] : -INFINITY;
-        for (int w = 1; w < active; ++w) overall = fmaxf(overall, wave_maximum[w][head]);
+        float overall = active > 0 ? wave_maximum[head] : -INFINITY;
+        for (int w = 1; w < active; ++w) {
+            overall = fmaxf(overall, wave_maximum[w * kGroupHeads + head]);
+        }
         float sum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
         float total = 0.0f;
         for (int w = 0; w < active; ++w) {
-            const float factor = expf(wave_maximum[w][head] - overall);
-            const float* row = &wave_accumulator[w][head][8 * piece];
+            const float factor = expf(wave_maximum[w * kGroupHeads + head] - overall);
+            const float* row = wave_accumulator + (w * kGroupHeads + head) * kRowFloats + 8 * piece;
             const float4 low = *reinterpret_cast<const float4*>(row);
             const float4 high = *reinterpret_cast<const float4*>(row + 4);
             sum[0] = fmaf(low.x, factor, sum[0]);
@@ -1008,17 +1152,25 @@ __global__ __launch_bounds__(kGroupWaves * kWave) void attention_grouped_kernel(
             sum[5] = fmaf(high.y, factor, sum[5]);
             sum[6] = fmaf(high.z, factor, sum[6]);
             sum[7] = fmaf(high.w, factor, sum[7]);
-            total = fmaf(wave_denominator[w][head], factor, total);
+            total = fmaf(wave_denominator[w * kGroupHeads + head], factor, total);
         }
-        // a partial row starts 8-byte aligned, and so does its third float
-        float* partial = a.partials +
-            ((first_head + head) * a.splits + blockIdx.y) * partial_floats(kGroupHeadDim);
-        if (piece == 0) *reinterpret_cast<float2*>(partial) = make_float2(overall, total);
-        float2* target = reinterpret_cast<float2*>(partial + 2 + 8 * piece);
-        target[0] = make_float2(sum[0], sum[1]);
-        target[1] = make_float2(sum[2], sum[3]);
-        target[2] = make_float2(sum[4], sum[5]);
-        target[3] = make_float2(sum[6], sum[7]);
+        const std::int64_t row_index = query_row * a.query_heads + first_head + head;
+        if (a.partials != nullptr) {
+            // a partial row starts 8-byte aligned, and so does its third float
+            float* partial =
+                a.partials + (row_index * a.splits + blockIdx.y) * partial_floats(kGroupHeadDim);
+            if (piece == 0) *reinterpret_cast<float2*>(partial) = make_float2(overall, total);
+            float2* target = reinterpret_cast<float2*>(partial + 2 + 8 * piece);
+            target[0] = make_float2(sum[0], sum[1]);
+            target[1] = make_float2(sum[2], sum[3]);
+            target[2] = make_float2(sum[4], sum[5]);
+            target[3] = make_float2(sum[6], sum[7]);
+        } else {
+            float4* target =
+                reinterpret_cast<float4*>(a.output + row_index * kGroupHeadDim + 8 * piece);
+            target[0] = make_float4(sum[0] / total, sum[1] / total, sum[2] / total, sum[3] / total);
+            target[1] = make_float4(sum[4] / total, sum[5] / total, sum[6] / total, sum[7] / total);
+        }
     }
 }
 
@@ -1034,6 +1186,17 @@ bool vector_form_fits(const AttentionArguments& arguments) {
         aligned(arguments.block_key) && aligned(arguments.block_value);
 }
 
+// The matrix-core kernel: head_dim 128, enough query heads per key/value head to fill
+// a useful part of its 16-head tiles, 16-byte aligned rows everywhere.
+bool grouped_form_fits(const AttentionArguments& arguments) {
+    const auto aligned = [](const void* pointer) {
+        return reinterpret_cast<std::uintptr_t>(pointer) % 16 == 0;
+    };
+    return vector_form_fits(arguments) && arguments.head_dim == kGroupHeadDim &&
+        arguments.heads_per_kv >= kGroupMinHeads && aligned(arguments.query) &&
+        aligned(arguments.output);
+}
+
 // `tiles_per_group`: the most 64-key tiles one workgroup has to cover.
 void launch_attention(const AttentionArguments& arguments, std::int64_t query_rows,
                       std::int64_t tiles_per_group, hipStream_t stream) {
@@ -1042,6 +1205,26 @@ void launch_attention(const AttentionArguments& arguments, std::int64_t query_ro
     if (waves > kMaxWaves) waves = kMaxWaves;
     const std::int64_t head_dim = arguments.head_dim;
     const unsigned splits = arguments.partials != nullptr ? arguments.splits : 1;
+    // A workgroup that walks a whole key range alone takes its rows in at what one
+    // compute unit can pull from memory, whatever the arithmetic costs: the matrix-core
+    // kernel pays where its workgroups are many (the split form) or where the vector
+    // kernel's would not fit the chip at once (blocks of many rows).
+    if (grouped_form_fits(arguments) &&
+        (arguments.partials != nullptr || query_rows * arguments.query_heads > compute_units())) {
+        static_assert(kGroupWaves == kMaxWaves, "one wave rule for both kernels");
+        const std::int64_t groups = arguments.kv_heads *
+            ((arguments.heads_per_kv + kGroupHeads - 1) / kGroupHeads);
+        static const bool raised =
+            hipFuncSetAttribute(reinterpret_cast<const void*>(attention_grouped_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kGroupWaves * kStageBytes) == hipSuccess;
+        (void)raised;
+        hipLaunchKernelGGL(attention_grouped_kernel,
+                           dim3(static_cast<unsigned>(query_rows * groups), splits),
+                           dim3(static_cast<unsigned>(waves * kWave)),
+                           static_cast<std::size_t>(waves) * kStageBytes, stream, arguments);
+        return;
+    }
     const dim3 grid(static_cast<unsigned>(query_rows * arguments.query_heads), splits);
     const dim3 block(static_cast<unsigned>(waves * kWave));
     if (!vector_form_fits(arguments)) {
@@ -1112,30 +1295,18 @@ namespace {
 // from the row's real key count when the kernel runs; surplus shares are empty).
 void launch_split(AttentionArguments a, std::int64_t tiles, float* partials, hipStream_t stream) {
     a.partials = partials;
-    const std::int64_t heads_per_kv = a.heads_per_kv;
-    if (a.head_dim == kGroupHeadDim && heads_per_kv >= kGroupMinHeads) {
-        // Matrix-core form: a workgroup serves up to 16 query heads of one key/value
-        // head.  As many shares as fill the chip, then up to four waves a share.
-        const std::int64_t groups = a.kv_heads * ((heads_per_kv + kGroupHeads - 1) / kGroupHeads);
-        std::int64_t splits = compute_units() / groups;
-        if (splits > kMaxSplits) splits = kMaxSplits;
-        if (splits > tiles) splits = tiles;
-        if (splits < 2) splits = 2;
-        a.splits = static_cast<int>(splits);
-        std::int64_t waves = (tiles + splits - 1) / splits;
-        if (waves > kGroupWaves) waves = kGroupWaves;
-        hipLaunchKernelGGL(attention_grouped_kernel,
-                           dim3(static_cast<unsigned>(groups), static_cast<unsigned>(splits)),
-                           dim3(static_cast<unsigned>(waves * kWave)), 0, stream, a);
-    } else {
-        // About one workgroup of up to eight waves per compute unit.
-        std::int64_t splits = compute_units() / a.query_heads;
-        if (splits > kVectorSplits) splits = kVectorSplits;
-        if (splits > tiles) splits = tiles;
-        if (splits < 2) splits = 2;
-        a.splits = static_cast<int>(splits);
-        launch_attention(a, 1, (tiles + a.splits - 1) / a.splits, stream);
-    }
+    // As many shares as fill the chip with about one workgroup per compute unit (a
+    // workgroup of the matrix-core kernel serves up to 16 query heads, one of the
+    // vector kernel a single head), then up to eight waves a share.
+    const bool grouped = grouped_form_fits(a);
+    const std::int64_t groups = grouped
+        ? a.kv_heads * ((a.heads_per_kv + kGroupHeads - 1) / kGroupHeads) : a.query_heads;
+    std::int64_t splits = compute_units() / groups;
+    if (splits > (grouped ? kMaxSplits : kVectorSplits)) splits = grouped ? kMaxSplits : kVectorSplits;
+    if (splits > tiles) splits = tiles;
+    if (splits < 2) splits = 2;
+    a.splits = static_cast<int>(splits);
+    launch_attention(a, 1, (tiles + splits - 1) / splits, stream);
     const int threads = static_cast<int>((a.head_dim + kWave - 1) / kWave * kWave) * kMergeLanes;
     hipLaunchKernelGGL(attention_merge_kernel, dim3(static_cast<unsigned>(a.query_heads)),
                        dim3(threads), 0, stream, partials, a.output, a.splits,
