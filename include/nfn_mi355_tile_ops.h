@@ -793,6 +793,21 @@ int nfn_mi355_fused_decode_attention_split_device_position_v1(
     void* workspace,
     int64_t workspace_nbytes);
 
+/* Lends the one-token attention entry points that have no workspace argument
+ * (nfn_native_tile_glimmer_gqa_decode_float32_v1, the fused decode-attention
+ * call and its device-position form) a workspace for the split form above, so
+ * that an engine's unchanged call sites take it: from this call on they run as
+ * their nfn_mi355_*_split_* counterparts whenever the workspace is on the
+ * current device and large enough for the call's geometry
+ * (nfn_mi355_gqa_decode_split_workspace_bytes_v1), and as before otherwise.
+ * (nullptr, 0) takes it back.  No counterpart in the reference.  The memory
+ * stays the caller's; every such call uses the same memory, so calls that
+ * overlap on the device (different streams, concurrently replayed graphs) race
+ * on it -- lend one only to an engine that issues its attention calls in stream
+ * order.  Calls already captured into a graph keep the form they were captured
+ * with.  0 on success, 1 for a misaligned pointer or a size without a pointer. */
+int nfn_mi355_attention_workspace_v1(void* workspace, int64_t workspace_nbytes);
+
 /* Shader clock under load, a measurement aid (no counterpart in the reference;
  * for benchmarks that price a kernel against the matrix-core peak at the clock
  * the chip really ran at).  Enqueues one wave that waits about `microseconds`

@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <limits>
+#include <mutex>
 
 namespace nfn {
 
@@ -17,6 +18,30 @@ constexpr std::int64_t kMaxBlockRows = 64;
 constexpr std::int64_t kLimit = std::numeric_limits<std::int64_t>::max();
 
 bool positive_finite(float value) { return std::isfinite(value) && value > 0.0f; }
+
+// The workspace an engine lent to the reference-named one-token attention entry
+// points (nfn_mi355_attention_workspace_v1): device it belongs to, address, size.
+struct LentWorkspace {
+    int device = -1;
+    float* memory = nullptr;
+    std::int64_t nbytes = 0;
+};
+std::mutex lent_mutex;
+LentWorkspace lent_workspace;
+
+// The lent workspace if it is on the current device and large enough for this geometry.
+float* lent_partials(std::int64_t query_heads, std::int64_t head_dim) {
+    LentWorkspace lent;
+    {
+        std::lock_guard<std::mutex> guard(lent_mutex);
+        lent = lent_workspace;
+    }
+    if (lent.memory == nullptr) return nullptr;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device != lent.device) return nullptr;
+    const std::int64_t required = gqa_decode_split_workspace_bytes(query_heads, head_dim);
+    return lent.nbytes >= required ? lent.memory : nullptr;
+}
 
 // kv_heads * head_dim, both positive, fits and does not exceed the row stride
 bool cache_rows_fit(std::int64_t kv_heads, std::int64_t head_dim, std::int64_t row_stride) {
@@ -123,6 +148,7 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
         return kInvalid;
     }
     const hipStream_t stream = as_stream(d->cuda_stream);
+    if (split_partials == nullptr) split_partials = lent_partials(d->query_heads, d->head_dim);
     // The new cache row is written by the first launch, before the attention
     // runs: right as long as the attention does not read that ring row, which
     // holds for every key range shorter than the ring (and for the device
@@ -320,8 +346,26 @@ int nfn_mi355_fused_decode_attention_split_device_position_v1(
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(
     const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
     if (!gqa_descriptor_valid(d)) return kInvalid;
-    launch_gqa_decode(*d, as_stream(d->cuda_stream));
+    if (float* partials = lent_partials(d->query_heads, d->head_dim)) {
+        launch_gqa_decode_split(*d, partials, as_stream(d->cuda_stream));
+    } else {
+        launch_gqa_decode(*d, as_stream(d->cuda_stream));
+    }
     return launch_status();
+}
+
+int nfn_mi355_attention_workspace_v1(void* workspace, std::int64_t workspace_nbytes) {
+    if ((workspace == nullptr) != (workspace_nbytes == 0) || workspace_nbytes < 0 ||
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
+        return kInvalid;
+    }
+    int device = -1;
+    if (workspace != nullptr && hipGetDevice(&device) != hipSuccess) return kInvalid;
+    std::lock_guard<std::mutex> guard(lent_mutex);
+    lent_workspace.device = device;
+    lent_workspace.memory = static_cast<float*>(workspace);
+    lent_workspace.nbytes = workspace_nbytes;
+    return 0;
 }
 
 std::int64_t nfn_mi355_gqa_decode_split_workspace_bytes_v1(std::int64_t query_heads,

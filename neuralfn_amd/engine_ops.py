@@ -142,6 +142,16 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     return out
 
 
+def lend_attention_workspace(workspace=None) -> None:
+    """Lends the reference-named one-token attention calls a split-form workspace
+    (gqa_decode_workspace), or takes it back with None.  The tensor must outlive the loan."""
+    if workspace is None:
+        check(load().nfn_mi355_attention_workspace_v1(None, 0), "attention_workspace")
+    else:
+        check(load().nfn_mi355_attention_workspace_v1(workspace.data_ptr(), workspace.numel()),
+              "attention_workspace")
+
+
 def gqa_decode_workspace(query_heads: int, head_dim: int, device="cuda:0"):
     """Workspace of the split form of gqa_decode (nfn_mi355_gqa_decode_split_v1)."""
     import torch

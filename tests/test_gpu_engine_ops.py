@@ -638,6 +638,59 @@ def test_fused_decode_attention_with_the_position_on_the_device(cuda, oracle, ap
                       workspace.numel()) == 1
 
 
+def test_lent_workspace_turns_the_reference_named_calls_into_their_split_forms(cuda, oracle):
+    rng = np.random.default_rng(41)
+    query_heads, kv_heads, head_dim, capacity, position = 32, 2, 128, 2048, 3000
+    first = position - capacity + 1
+    stride = kv_heads * head_dim
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    keys = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    values = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    scale = head_dim ** -0.5
+    device_position = to_device(np.array([position], dtype=np.int64), cuda)
+    fused = dict(eps=1e-5, query_scale=1.0, theta=500000.0, layout=engine_ops.ROPE_INTERLEAVED,
+                 apply_rope=True)
+
+    def run(lent, explicit):
+        """(gqa_decode, fused host position, fused device position) outputs"""
+        outputs = []
+        engine_ops.lend_attention_workspace(lent)
+        try:
+            tensors = lambda: (to_device(query, cuda), to_device(key, cuda), to_device(value, cuda),
+                               bf16_tensor(keys, cuda), bf16_tensor(values, cuda))
+            outputs.append(engine_ops.gqa_decode(*tensors(), position, first, scale,
+                                                 workspace=explicit))
+            outputs.append(engine_ops.fused_decode_attention(*tensors(), position, first, scale,
+                                                             workspace=explicit, **fused))
+            outputs.append(engine_ops.fused_decode_attention(
+                *tensors(), 5, 2, scale, device_position=device_position, sliding_window=capacity,
+                workspace=explicit, **fused))
+        finally:
+            engine_ops.lend_attention_workspace(None)
+        return outputs
+
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+    plain = run(None, None)
+    split = run(None, workspace)
+    lent = run(workspace, None)
+    after = run(None, None)
+    for index, name in enumerate(("gqa_decode", "fused", "fused, device position")):
+        assert_bits_equal(lent[index], split[index], name + ": lent = explicit split form")
+        assert_bits_equal(after[index], plain[index], name + ": taken back")
+        assert not np.array_equal(bits_of(split[index]), bits_of(plain[index])), name
+        assert np.abs(split[index].cpu().numpy() - plain[index].cpu().numpy()).max() <= 4e-6
+    # too small for the geometry: the ordinary form; bad arguments are refused
+    small = torch_().empty(1024, dtype=torch_().uint8, device=cuda)
+    assert_bits_equal(run(small, None)[0], plain[0], "a workspace too small is not used")
+    lib = tile_ops.load()
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr() + 4, 1 << 20) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(None, 16) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 0) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(None, 0) == 0
+
+
 def test_cache_commit_layers_and_pack_target_taps(cuda, oracle):
     rng = np.random.default_rng(35)
     layers, source_rows, rows, kv_heads, head_dim, position = 5, 9, 6, 2, 64, 1021
