@@ -427,6 +427,58 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
     return result
 
 
+def attention_extra(device, stream, steps: int, warmup: int) -> dict:
+    """Attention alone at the workload's head geometry: the one-token call in the reference's
+    form (one workgroup per query head, no workspace) and in the split form, over a local
+    window and a long context, and the verifier's 16-row causal block."""
+    import torch
+    from neuralfn_amd import engine_ops
+    query_heads, kv_heads, head_dim = ATTN_DIM // 128, KV_DIM // 128, 128
+    scale = head_dim ** -0.5
+    steps, warmup = max(5, steps // 2), max(2, warmup // 2)
+    calls = 16  # per graph: a replay's own cost is not the call's
+
+    def time_calls(call) -> float:
+        def run():
+            for _ in range(calls):
+                call()
+        return time_graph(run, stream, steps, warmup) / calls
+
+    result = {"workload": f"{query_heads} query heads over {kv_heads} key/value heads of "
+                          f"{head_dim}, bf16 cache, {calls} calls a HIP-graph replay; GB/s = "
+                          "cache bytes of the attended keys / time"}
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim, device)
+    for keys in (2048, 32768):
+        query = torch.randn(query_heads, head_dim, device=device)
+        key = torch.randn(kv_heads, head_dim, device=device)
+        value = torch.randn(kv_heads, head_dim, device=device)
+        key_cache = torch.randn(keys, kv_heads * head_dim, device=device).to(torch.bfloat16)
+        value_cache = torch.randn(keys, kv_heads * head_dim, device=device).to(torch.bfloat16)
+        out = torch.empty_like(query)
+        position = 2 * keys - 1  # the ring is full and has wrapped once
+        first = position - keys + 1
+        cache_bytes = 2 * keys * kv_heads * head_dim * 2
+        entry = {}
+        for name, lent in (("reference_form", None), ("split_form", workspace)):
+            ms = time_calls(lambda: engine_ops.gqa_decode(query, key, value, key_cache, value_cache,
+                                                          position, first, scale, out=out,
+                                                          workspace=lent))
+            entry[name] = {"us": round(ms * 1e3, 2), "GB/s": round(cache_bytes / ms / 1e6, 1)}
+        result[f"one_token_{keys}_keys"] = entry
+    rows, window = 16, 2048
+    query = torch.randn(rows, query_heads, head_dim, device=device)
+    block_key = torch.randn(rows, kv_heads, head_dim, device=device)
+    block_value = torch.randn(rows, kv_heads, head_dim, device=device)
+    key_cache = torch.randn(window, kv_heads * head_dim, device=device).to(torch.bfloat16)
+    value_cache = torch.randn(window, kv_heads * head_dim, device=device).to(torch.bfloat16)
+    out = torch.empty_like(query)
+    ms = time_calls(lambda: engine_ops.block_attention(query, block_key, block_value, key_cache,
+                                                       value_cache, 4000, window, scale, True,
+                                                       out=out))
+    result[f"causal_block_{rows}_rows_{window}_window"] = {"us": round(ms * 1e3, 2)}
+    return result
+
+
 def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
     """Four layers of attention and FFN projections with per-tensor formats drawn by seed
     from {Q4_K, Q5_K, Q6_K, Q8_0} (V, O and down at least Q5_K), at one row (decode)
@@ -612,6 +664,7 @@ def main() -> int:
                 record["lm_head"] = lm_head_extra(device, stream, args.steps, args.warmup)
                 record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
                 record["mixed_profile"] = mixed_profile_extra(device, stream, args.steps, args.warmup)
+                record["attention"] = attention_extra(device, stream, args.steps, args.warmup)
                 record["decode_layer"] = decode_layer_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
             record["extras_error"] = repr(error)
