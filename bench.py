@@ -472,10 +472,13 @@ def attention_extra(device, stream, steps: int, warmup: int) -> dict:
     key_cache = torch.randn(window, kv_heads * head_dim, device=device).to(torch.bfloat16)
     value_cache = torch.randn(window, kv_heads * head_dim, device=device).to(torch.bfloat16)
     out = torch.empty_like(query)
-    ms = time_calls(lambda: engine_ops.block_attention(query, block_key, block_value, key_cache,
-                                                       value_cache, 4000, window, scale, True,
-                                                       out=out))
-    result[f"causal_block_{rows}_rows_{window}_window"] = {"us": round(ms * 1e3, 2)}
+    entry = {}
+    for name, lent in (("reference_form", None), ("split_form", workspace)):
+        ms = time_calls(lambda: engine_ops.block_attention(query, block_key, block_value, key_cache,
+                                                           value_cache, 4000, window, scale, True,
+                                                           out=out, workspace=lent))
+        entry[name] = {"us": round(ms * 1e3, 2)}
+    result[f"causal_block_{rows}_rows_{window}_window"] = entry
     return result
 
 

@@ -793,13 +793,27 @@ int nfn_mi355_fused_decode_attention_split_device_position_v1(
     void* workspace,
     int64_t workspace_nbytes);
 
-/* Lends the one-token attention entry points that have no workspace argument
+/* nfn_native_tile_dflash_block_attention_float32_v1 with a workspace: the keys
+ * of every query row are shared out over workgroups like those of the
+ * one-token split form (as many shares as the workspace has room for,
+ * query_rows * query_heads * (head_dim + 2) floats each; with room for fewer
+ * than two the ordinary form runs).  Same descriptor, same semantics and
+ * tolerance; the bits can differ from the ordinary entry point.  The workspace
+ * of the one-token form is a good size for blocks of up to 16 rows. */
+int nfn_mi355_dflash_block_attention_split_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* descriptor,
+    void* workspace,
+    int64_t workspace_nbytes);
+
+/* Lends the attention entry points that have no workspace argument
  * (nfn_native_tile_glimmer_gqa_decode_float32_v1, the fused decode-attention
- * call and its device-position form) a workspace for the split form above, so
+ * call and its device-position form, nfn_native_tile_dflash_block_attention_float32_v1
+ * and its short_split form) a workspace for the split forms above, so
  * that an engine's unchanged call sites take it: from this call on they run as
  * their nfn_mi355_*_split_* counterparts whenever the workspace is on the
  * current device and large enough for the call's geometry
- * (nfn_mi355_gqa_decode_split_workspace_bytes_v1), and as before otherwise.
+ * (nfn_mi355_gqa_decode_split_workspace_bytes_v1; a block takes as many shares
+ * as fit), and as before otherwise.
  * (nullptr, 0) takes it back.  No counterpart in the reference.  The memory
  * stays the caller's; every such call uses the same memory, so calls that
  * overlap on the device (different streams, concurrently replayed graphs) race

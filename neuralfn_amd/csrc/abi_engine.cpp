@@ -29,16 +29,24 @@ struct LentWorkspace {
 std::mutex lent_mutex;
 LentWorkspace lent_workspace;
 
-// The lent workspace if it is on the current device and large enough for this geometry.
-float* lent_partials(std::int64_t query_heads, std::int64_t head_dim) {
+// The lent workspace if it is on the current device (memory null otherwise).
+LentWorkspace lent_here() {
     LentWorkspace lent;
     {
         std::lock_guard<std::mutex> guard(lent_mutex);
         lent = lent_workspace;
     }
-    if (lent.memory == nullptr) return nullptr;
     int device = -1;
-    if (hipGetDevice(&device) != hipSuccess || device != lent.device) return nullptr;
+    if (lent.memory != nullptr && (hipGetDevice(&device) != hipSuccess || device != lent.device)) {
+        lent = LentWorkspace{};
+    }
+    return lent;
+}
+
+// ... if it is also large enough for the one-token split form of this geometry.
+float* lent_partials(std::int64_t query_heads, std::int64_t head_dim) {
+    const LentWorkspace lent = lent_here();
+    if (lent.memory == nullptr) return nullptr;
     const std::int64_t required = gqa_decode_split_workspace_bytes(query_heads, head_dim);
     return lent.nbytes >= required ? lent.memory : nullptr;
 }
@@ -116,6 +124,23 @@ bool gqa_descriptor_valid(const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
         d->cache_row_stride <= 0 || !positive_finite(d->scale) ||
         !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
         d->query_heads > std::numeric_limits<std::int32_t>::max());
+}
+
+bool block_descriptor_valid(const NfnNativeTileDFlashBlockAttentionDescriptorV1* d) {
+    return d != nullptr && d->struct_size >= sizeof(*d) &&
+        d->version == NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 &&
+        (d->flags & ~static_cast<std::uint32_t>(NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL)) == 0 &&
+        d->reserved0 == 0 && d->reserved1 == 0 && d->query != nullptr &&
+        d->block_key != nullptr && d->block_value != nullptr && d->key_cache_bf16 != nullptr &&
+        d->value_cache_bf16 != nullptr && d->output != nullptr && d->query_rows > 0 &&
+        d->block_rows > 0 && d->query_rows <= d->block_rows && d->block_rows <= kMaxBlockRows &&
+        d->query_heads > 0 && d->kv_heads > 0 && d->query_heads % d->kv_heads == 0 &&
+        d->head_dim > 0 && d->head_dim <= kMaxHeadDim && d->context_length >= 0 &&
+        d->context_length <= kLimit - kMaxBlockRows && d->sliding_window > 0 &&
+        d->cache_capacity >= d->sliding_window && d->cache_row_stride > 0 &&
+        positive_finite(d->scale) &&
+        cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) &&
+        d->query_heads <= std::numeric_limits<std::int32_t>::max() / kMaxBlockRows;
 }
 
 // Shared body of the fused decode entry points; device_position null = the
@@ -413,23 +438,21 @@ int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
 
 int nfn_native_tile_dflash_block_attention_float32_v1(
     const NfnNativeTileDFlashBlockAttentionDescriptorV1* d) {
-    if (d == nullptr || d->struct_size < sizeof(*d) ||
-        d->version != NFN_NATIVE_TILE_GLIMMER_INFERENCE_V1 ||
-        (d->flags & ~static_cast<std::uint32_t>(NFN_NATIVE_TILE_BLOCK_ATTENTION_CAUSAL)) != 0 ||
-        d->reserved0 != 0 || d->reserved1 != 0 || d->query == nullptr ||
-        d->block_key == nullptr || d->block_value == nullptr || d->key_cache_bf16 == nullptr ||
-        d->value_cache_bf16 == nullptr || d->output == nullptr || d->query_rows <= 0 ||
-        d->block_rows <= 0 || d->query_rows > d->block_rows || d->block_rows > kMaxBlockRows ||
-        d->query_heads <= 0 || d->kv_heads <= 0 || d->query_heads % d->kv_heads != 0 ||
-        d->head_dim <= 0 || d->head_dim > kMaxHeadDim || d->context_length < 0 ||
-        d->context_length > kLimit - kMaxBlockRows || d->sliding_window <= 0 ||
-        d->cache_capacity < d->sliding_window || d->cache_row_stride <= 0 ||
-        !positive_finite(d->scale) ||
-        !cache_rows_fit(d->kv_heads, d->head_dim, d->cache_row_stride) ||
-        d->query_heads > std::numeric_limits<std::int32_t>::max() / kMaxBlockRows) {
+    if (!block_descriptor_valid(d)) return kInvalid;
+    const LentWorkspace lent = lent_here();
+    launch_block_attention(*d, lent.memory, lent.nbytes, as_stream(d->cuda_stream));
+    return launch_status();
+}
+
+int nfn_mi355_dflash_block_attention_split_v1(
+    const NfnNativeTileDFlashBlockAttentionDescriptorV1* d, void* workspace,
+    std::int64_t workspace_nbytes) {
+    if (!block_descriptor_valid(d) || workspace == nullptr || workspace_nbytes <= 0 ||
+        reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
         return kInvalid;
     }
-    launch_block_attention(*d, as_stream(d->cuda_stream));
+    launch_block_attention(*d, static_cast<float*>(workspace), workspace_nbytes,
+                           as_stream(d->cuda_stream));
     return launch_status();
 }
 

@@ -1290,27 +1290,36 @@ std::int64_t gqa_decode_split_workspace_bytes(std::int64_t query_heads, std::int
 
 namespace {
 
-// Split form of the one-token call.  `tiles`: the 64-key tiles of the row, or
-// with a position in device memory the most it can have (the shares are cut
-// from the row's real key count when the kernel runs; surplus shares are empty).
-void launch_split(AttentionArguments a, std::int64_t tiles, float* partials, hipStream_t stream) {
-    a.partials = partials;
+// Split form.  `tiles`: the 64-key tiles of the longest row, or with a position in
+// device memory the most it can have (the shares are cut from each row's real key
+// count when the kernel runs; surplus shares are empty).  `partial_bytes` bounds the
+// shares; with room for fewer than two the ordinary form runs.
+void launch_split(AttentionArguments a, std::int64_t query_rows, std::int64_t tiles,
+                  float* partials, std::int64_t partial_bytes, hipStream_t stream) {
     // As many shares as fill the chip with about one workgroup per compute unit (a
     // workgroup of the matrix-core kernel serves up to 16 query heads, one of the
     // vector kernel a single head), then up to eight waves a share.
+    a.partials = partials;  // (decides the kernel)
     const bool grouped = grouped_form_fits(a);
-    const std::int64_t groups = grouped
-        ? a.kv_heads * ((a.heads_per_kv + kGroupHeads - 1) / kGroupHeads) : a.query_heads;
+    const std::int64_t groups = query_rows *
+        (grouped ? a.kv_heads * ((a.heads_per_kv + kGroupHeads - 1) / kGroupHeads) : a.query_heads);
+    const std::int64_t share_bytes = query_rows * a.query_heads * partial_floats(a.head_dim) * 4;
     std::int64_t splits = compute_units() / groups;
     if (splits > (grouped ? kMaxSplits : kVectorSplits)) splits = grouped ? kMaxSplits : kVectorSplits;
     if (splits > tiles) splits = tiles;
     if (splits < 2) splits = 2;
+    if (splits > partial_bytes / share_bytes) splits = partial_bytes / share_bytes;
+    if (splits < 2) {
+        a.partials = nullptr;
+        launch_attention(a, query_rows, tiles, stream);
+        return;
+    }
     a.splits = static_cast<int>(splits);
-    launch_attention(a, 1, (tiles + splits - 1) / splits, stream);
+    launch_attention(a, query_rows, (tiles + splits - 1) / splits, stream);
     const int threads = static_cast<int>((a.head_dim + kWave - 1) / kWave * kWave) * kMergeLanes;
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(static_cast<unsigned>(a.query_heads)),
-                       dim3(threads), 0, stream, partials, a.output, a.splits,
-                       static_cast<int>(a.head_dim));
+    hipLaunchKernelGGL(attention_merge_kernel,
+                       dim3(static_cast<unsigned>(query_rows * a.query_heads)), dim3(threads), 0,
+                       stream, partials, a.output, a.splits, static_cast<int>(a.head_dim));
 }
 
 }  // namespace
@@ -1323,7 +1332,8 @@ void launch_gqa_decode_split(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d,
         launch_attention(a, 1, tiles, stream);  // nothing to split, or no vector form: one launch
         return;
     }
-    launch_split(a, tiles, partials, stream);
+    launch_split(a, 1, tiles, partials, gqa_decode_split_workspace_bytes(d.query_heads, d.head_dim),
+                 stream);
 }
 
 void launch_gqa_decode_split_device_position(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& d,
@@ -1339,12 +1349,12 @@ void launch_gqa_decode_split_device_position(const NfnNativeTileGlimmerGqaDecode
         return;
     }
     // a global layer sees at most the ring and the row's own key
-    launch_split(a, tiles_of(whole_context ? d.cache_capacity + 1 : sliding_window), partials,
-                 stream);
+    launch_split(a, 1, tiles_of(whole_context ? d.cache_capacity + 1 : sliding_window), partials,
+                 gqa_decode_split_workspace_bytes(d.query_heads, d.head_dim), stream);
 }
 
-void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& d,
-                            hipStream_t stream) {
+void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& d, float* partials,
+                            std::int64_t partial_bytes, hipStream_t stream) {
     AttentionArguments a{};
     a.query = d.query;
     a.block_key = d.block_key;
@@ -1368,7 +1378,12 @@ void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1&
         const std::int64_t window = a.causal ? d.sliding_window : 2 * d.sliding_window + 1;
         if (window < longest) longest = window;
     }
-    launch_attention(a, d.query_rows, tiles_of(longest), stream);
+    const std::int64_t tiles = tiles_of(longest);
+    if (partials != nullptr && vector_form_fits(a) && tiles >= 2) {
+        launch_split(a, d.query_rows, tiles, partials, partial_bytes, stream);
+    } else {
+        launch_attention(a, d.query_rows, tiles, stream);
+    }
 }
 
 }  // namespace nfn

@@ -91,8 +91,10 @@ void launch_scale(float* values, std::int64_t count, float scale, hipStream_t st
 // attention.hip — descriptors already checked.
 void launch_gqa_decode(const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor,
                        hipStream_t stream);
+// `partials` (16-byte aligned, `partial_bytes` bytes) or null: with it the keys of every
+// row are shared out over workgroups as in the split one-token form.
 void launch_block_attention(const NfnNativeTileDFlashBlockAttentionDescriptorV1& descriptor,
-                            hipStream_t stream);
+                            float* partials, std::int64_t partial_bytes, hipStream_t stream);
 // One-token attention with the keys of every head dealt over several
 // workgroups; `partials` holds gqa_decode_split_workspace_bytes() bytes.
 // One-token attention whose position is read from device memory when the kernel

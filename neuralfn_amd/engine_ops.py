@@ -208,8 +208,9 @@ def cache_commit(keys, values, key_cache, value_cache, position: int, rows: int 
 
 
 def block_attention(query, block_key, block_value, key_cache, value_cache, context_length: int,
-                    sliding_window: int, scale: float, causal: bool, out=None):
-    """query [query_rows, query_heads, head_dim]; block_key/value [block_rows, kv_heads, head_dim]."""
+                    sliding_window: int, scale: float, causal: bool, out=None, workspace=None):
+    """query [query_rows, query_heads, head_dim]; block_key/value [block_rows, kv_heads, head_dim].
+    With `workspace` (any 16-byte aligned uint8 tensor, e.g. gqa_decode_workspace) the split form."""
     import torch
     if out is None:
         out = torch.empty_like(query)
@@ -227,8 +228,12 @@ def block_attention(query, block_key, block_value, key_cache, value_cache, conte
     d.cache_capacity, d.cache_row_stride = key_cache.shape
     d.scale = scale
     d.cuda_stream = _stream()
-    check(load().nfn_native_tile_dflash_block_attention_float32_v1(ctypes.byref(d)),
-          "block_attention")
+    if workspace is not None:
+        check(load().nfn_mi355_dflash_block_attention_split_v1(
+            ctypes.byref(d), workspace.data_ptr(), workspace.numel()), "block_attention_split")
+    else:
+        check(load().nfn_native_tile_dflash_block_attention_float32_v1(ctypes.byref(d)),
+              "block_attention")
     return out
 
 

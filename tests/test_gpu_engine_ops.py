@@ -405,6 +405,44 @@ def test_causal_block_is_token_at_a_time_decode(cuda, oracle, query_heads, kv_he
         assert np.abs(block.cpu().numpy() - serial.cpu().numpy()).max() <= 4e-6
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("rows,block_rows,query_heads,kv_heads,context,window,capacity,head_dim", [
+    (16, 16, 32, 2, 3000, 2048, 2048, 128),  # the verifier's block: matrix-core kernel, eight shares
+    (5, 7, 8, 2, 150, 60, 96, 64),           # vector kernel, shares of one tile; the ring has wrapped
+    (64, 64, 8, 2, 3000, 2048, 2048, 128),   # more rows than the workspace has room to split well
+    (3, 9, 6, 3, 20, 90, 128, 50),           # no vector form: the ordinary kernel, workspace untouched
+    (2, 2, 16, 1, 40, 64, 64, 128),          # one tile: nothing to split
+])
+def test_block_attention_split_form(cuda, oracle, causal, rows, block_rows, query_heads, kv_heads,
+                                    context, window, capacity, head_dim):
+    rng = np.random.default_rng(rows * 100 + context + head_dim)
+    stride = kv_heads * head_dim
+    query = rng.standard_normal((rows, query_heads, head_dim)).astype(np.float32)
+    block_key = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    block_value = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    key_cache = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    value_cache = oracle.to_bf16(rng.standard_normal((capacity, stride)).astype(np.float32))
+    scale = 1.0 / np.sqrt(head_dim)
+    arguments = (to_device(query, cuda), to_device(block_key, cuda), to_device(block_value, cuda),
+                 bf16_tensor(key_cache, cuda), bf16_tensor(value_cache, cuda), context, window, scale,
+                 causal)
+    workspace = engine_ops.gqa_decode_workspace(32, 128)  # what an engine would have at hand
+    workspace.fill_(0xFF)
+    out = engine_ops.block_attention(*arguments, workspace=workspace)
+    expected = oracle.block_attention(query, block_key, block_value, key_cache, value_cache, context,
+                                      window, scale, causal)
+    assert np.abs(out.cpu().numpy() - expected).max() <= 4e-6
+    # the reference-named call takes the same form while the workspace is lent
+    engine_ops.lend_attention_workspace(workspace)
+    try:
+        lent = engine_ops.block_attention(*arguments)
+    finally:
+        engine_ops.lend_attention_workspace(None)
+    assert_bits_equal(lent, out, "lent = explicit split form")
+    lib = tile_ops.load()
+    assert lib.nfn_mi355_dflash_block_attention_split_v1(None, workspace.data_ptr(), 1 << 20) == 1
+
+
 def test_block_attention_fails_closed(cuda):
     lib = tile_ops.load()
     x = torch_().zeros(1 << 16, dtype=torch_().float32, device=cuda)
