@@ -427,6 +427,25 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
     return result
 
 
+def memory_rate_extra(device, stream, steps: int, warmup: int) -> dict:
+    """What the vendor library's own streaming kernels reach on this GPU: a float sum (read
+    only) and a copy (read + write) over buffers below and far above the 256 MB the memory-side
+    cache holds.  The comparator for every HBM-bound figure here, next to the published 8 TB/s."""
+    import torch
+    result = {"workload": "torch.sum / Tensor.copy_ over a float32 buffer, TB/s of bytes moved"}
+    steps, warmup = max(5, steps // 2), max(2, warmup // 2)
+    for mib in (256, 2048):
+        source = torch.empty(mib * (1 << 20) // 4, dtype=torch.float32, device=device).normal_()
+        target = torch.empty_like(source)
+        nbytes = source.numel() * 4
+        read_ms = time_replays(lambda: source.sum(), steps, warmup)
+        copy_ms = time_replays(lambda: target.copy_(source), steps, warmup)
+        result[f"{mib}_MiB"] = {"sum_read_TB/s": round(nbytes / read_ms / 1e9, 2),
+                                "copy_read_plus_write_TB/s": round(2 * nbytes / copy_ms / 1e9, 2)}
+        del source, target
+    return result
+
+
 def attention_extra(device, stream, steps: int, warmup: int) -> dict:
     """Attention alone at the workload's head geometry: the one-token call in the reference's
     form (one workgroup per query head, no workspace) and in the split form, over a local
@@ -668,6 +687,8 @@ def main() -> int:
                 record["prefill"] = prefill_extra(device, stream, args.steps, args.warmup)
                 record["mixed_profile"] = mixed_profile_extra(device, stream, args.steps, args.warmup)
                 record["attention"] = attention_extra(device, stream, args.steps, args.warmup)
+                record["library_memory_rate"] = memory_rate_extra(device, stream, args.steps,
+                                                                  args.warmup)
                 record["decode_layer"] = decode_layer_extra(device, stream, args.steps, args.warmup)
         except Exception as error:  # side measurements never hide the headline
             record["extras_error"] = repr(error)
