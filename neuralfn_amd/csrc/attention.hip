@@ -709,9 +709,10 @@ __global__ __launch_bounds__(kMaxHeadDim * kMergeLanes) void attention_merge_ker
 }
 
 // ---------------------------------------------------------------------------
-// Grouped one-token form on the matrix cores (split form only, head_dim 128):
-// one workgroup per (key/value head, group of up to 16 of its query heads,
-// share of the keys).  All query heads of a group read a key/value row once.
+// Grouped form on the matrix cores (head_dim 128): one workgroup per (query row,
+// key/value head, group of up to 16 of its query heads[, share of the keys]).
+// All query heads of a group read a key/value row once.  Same semantics as the
+// vector kernel for one-token calls and blocks, with or without the split.
 //
 // Lane = (j, i) = (lane / 16, lane % 16).  Both products run on
 // v_mfma_f32_16x16x32_bf16 with float operands cut into three bf16 terms whose sum
@@ -1214,11 +1215,7 @@ void launch_attention(const AttentionArguments& arguments, std::int64_t query_ro
         static_assert(kGroupWaves == kMaxWaves, "one wave rule for both kernels");
         const std::int64_t groups = arguments.kv_heads *
             ((arguments.heads_per_kv + kGroupHeads - 1) / kGroupHeads);
-        static const bool raised =
-            hipFuncSetAttribute(reinterpret_cast<const void*>(attention_grouped_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kGroupWaves * kStageBytes) == hipSuccess;
-        (void)raised;
+        allow_large_lds<attention_grouped_kernel>(kGroupWaves * kStageBytes);
         hipLaunchKernelGGL(attention_grouped_kernel,
                            dim3(static_cast<unsigned>(query_rows * groups), splits),
                            dim3(static_cast<unsigned>(waves * kWave)),

@@ -9,6 +9,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdint>
 
 #include "../../include/nfn_mi355_tile_ops.h"
@@ -60,18 +61,39 @@ bool validate_k_descriptor(const Descriptor* descriptor, std::int64_t input_dim,
                            void* stream, bool allow_q8_0);
 
 // Compute units of the current device (256 on MI355X), cached.
+constexpr int kMaxDevices = 64;
+
+// The current device's index, 0 if it cannot be told or is beyond the tables below.
+inline int current_device() {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 0;
+    return device;
+}
+
 inline int compute_units() {
-    static const int count = [] {
-        int device = 0;
-        int value = 0;
-        if (hipGetDevice(&device) != hipSuccess ||
-            hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
-            value <= 0) {
-            return 256;
+    static std::atomic<int> counts[kMaxDevices];  // 0 = not asked yet
+    const int device = current_device();
+    int count = counts[device].load(std::memory_order_relaxed);
+    if (count == 0) {
+        if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+            count <= 0) {
+            count = 256;
         }
-        return value;
-    }();
+        counts[device].store(count, std::memory_order_relaxed);
+    }
     return count;
+}
+
+// More than 64 KB of dynamic LDS has to be allowed once per kernel and device.
+template <auto Kernel>
+inline void allow_large_lds(int bytes = 160 * 1024) {
+    static std::atomic<std::uint64_t> allowed{0};  // one bit per device
+    const std::uint64_t bit = std::uint64_t(1) << current_device();
+    if ((allowed.load(std::memory_order_acquire) & bit) != 0) return;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess) {
+        allowed.fetch_or(bit, std::memory_order_release);
+    }
 }
 
 inline hipStream_t as_stream(void* stream) { return reinterpret_cast<hipStream_t>(stream); }

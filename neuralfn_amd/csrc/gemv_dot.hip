@@ -304,10 +304,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     const std::int64_t blocks = set.input_dim >> 8;
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes_host(blocks);
     auto kernel = gemv_dot_kernel<ENC, T, P>;
-    static const bool raised =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
-    (void)raised;
+    allow_large_lds<gemv_dot_kernel<ENC, T, P>>();
     const int passes = (tokens + T - 1) / T;
     const std::int64_t groups = decode_groups(rows, kDotWaves);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,

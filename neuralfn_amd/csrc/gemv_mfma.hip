@@ -736,11 +736,7 @@ void launch_variant(ProjectionSet set, const Pass& pass) {
         *pass.quantized = true;
     }
     auto kernel = gemv_mfma_kernel<ENC, S, MODE, P, ARGMAX>;
-    // More than 64 KB of dynamic LDS has to be allowed once per kernel.
-    static const bool raised =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
-    (void)raised;
+    allow_large_lds<gemv_mfma_kernel<ENC, S, MODE, P, ARGMAX>>();
     const int pass_capacity = 2 * S;
     const int passes = (pass.tokens + pass_capacity - 1) / pass_capacity;
     // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles

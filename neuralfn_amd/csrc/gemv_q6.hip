@@ -635,10 +635,7 @@ std::int64_t launch_variant(ProjectionSet set, const float* first, const float* 
     std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8);
     if (lds < 1024) lds = 1024;  // room for the per-wave candidates
     auto kernel = gemv_q6_kernel<T, P, ARGMAX>;
-    static const bool raised =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
-    (void)raised;
+    allow_large_lds<gemv_q6_kernel<T, P, ARGMAX>>();
     const std::int64_t groups = decode_groups(rows, kWaves);
     const int passes = (tokens + T - 1) / T;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
@@ -677,10 +674,7 @@ std::int64_t launch_stream(const ProjectionSet& set, const float* first, const f
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8) +
         W * kStagingBytes;
     auto kernel = gemv_q6_stream_kernel<T, P, ARGMAX, W>;
-    static const bool raised =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
-    (void)raised;
+    allow_large_lds<gemv_q6_stream_kernel<T, P, ARGMAX, W>>();
     const int passes = (tokens + T - 1) / T;
     // one launch: the projections take consecutive ranges of waves
     std::int64_t rows = 0;

@@ -256,10 +256,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     }
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8);
     auto kernel = gemv_q8_kernel<T, P>;
-    static const bool raised =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess;
-    (void)raised;
+    allow_large_lds<gemv_q8_kernel<T, P>>();
     const int passes = (tokens + T - 1) / T;
     const std::int64_t groups = decode_groups(rows, kWaves);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kThreads), lds,
