@@ -364,12 +364,12 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
 
 def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
     """Whole decode layers at the workload's geometry, every operator through the C ABI in the
-    engine's order (neuralfn_amd/decode_layer.py): what a token costs beyond the projections."""
+    engine's order (neuralfn_amd/decode_layer.py): what a token costs beyond the projections.
+    Local layers (2048-key window) and global ones at a 32768-token context, each with the
+    reference's fused attention call and with the split form."""
     import torch
-    from neuralfn_amd import decode_layer as dl, kquant, tile_ops
-    layers, position = 8, 5000
-    g = dl.LayerGeometry(model_dim=MODEL_DIM, query_heads=ATTN_DIM // 128, kv_heads=KV_DIM // 128,
-                         head_dim=128, ffn_dim=FFN_DIM, sliding_window=2048)
+    from neuralfn_amd import decode_layer as dl, engine_ops, kquant, tile_ops
+    layers = 8
     ones = {width: tile_ops.PackedWeight(
         kquant.F32, 1, width, torch.ones(width, dtype=torch.float32, device=device).view(torch.uint8))
         for width in (MODEL_DIM, 128)}
@@ -377,53 +377,87 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
                   attention_gate=(ATTN_DIM, MODEL_DIM), output=(MODEL_DIM, ATTN_DIM),
                   mlp_gate=(FFN_DIM, MODEL_DIM), mlp_up=(FFN_DIM, MODEL_DIM),
                   mlp_down=(MODEL_DIM, FFN_DIM))
-    stack = []
+    weights = []
     for layer in range(layers):
         packed = {name: random_packed_on_device(kquant.Q4_K, out_dim, in_dim, device,
                                                 1000 + 10 * layer + index)
                   for index, (name, (out_dim, in_dim)) in enumerate(shapes.items())}
-        weights = dl.LayerWeights(
+        weights.append(dl.LayerWeights(
             **packed, input_norm=ones[MODEL_DIM], q_norm=ones[128], k_norm=ones[128],
             post_attention_norm=ones[MODEL_DIM], pre_feedforward_norm=ones[MODEL_DIM],
-            post_feedforward_norm=ones[MODEL_DIM])
-        cache = dl.LayerCache(g, device)
-        cache.keys.copy_(torch.randn(cache.keys.shape, device=device).to(torch.bfloat16).view(torch.int16))
-        cache.values.copy_(torch.randn(cache.values.shape, device=device).to(torch.bfloat16).view(torch.int16))
-        stack.append((weights, cache))
+            post_feedforward_norm=ones[MODEL_DIM]))
+    weight_bytes = sum(w.packed_bytes() for w in weights)
     workspace = tile_ops.small_batch_workspace(1, FFN_DIM, device)
     embedding = torch.from_numpy(kquant.synthetic_activations(41, 1, MODEL_DIM)).to(device)
     zeros = torch.zeros_like(embedding)
     last = {}
-
-    weight_bytes = sum(weights.packed_bytes() for weights, _ in stack)
-    cache_bytes = layers * 2 * g.sliding_window * g.kv_dim * 2
     result = {
         "workload": f"{layers} whole decode layers (Q4_K projections incl. attention gate and FFN "
-                    f"{MODEL_DIM}<->{FFN_DIM}, 2048-key local attention), one token, HIP-graph replay"}
-    from neuralfn_amd import engine_ops
-    forms = (("reference_fused_attention", None, dl.LAUNCHES_PER_LAYER),
-             ("split_attention", engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim, device),
-              dl.LAUNCHES_PER_LAYER_SPLIT))
-    for name, attention_workspace, launches in forms:
-        def token():
-            pending, residual, pending_norm = embedding, zeros, None
-            for weights, cache in stack:
-                pending, residual = dl.decode_layer(g, weights, cache, pending, residual,
-                                                    pending_norm, position, workspace, True,
-                                                    attention_workspace)
-                pending_norm = weights.post_feedforward_norm
-            last["hidden"] = residual
+                    f"{MODEL_DIM}<->{FFN_DIM}), one token, HIP-graph replay; local = 2048-key "
+                    "window, global = every key of a 32768-token context"}
+    for kind, keys, local in (("local", 2048, True), ("global", 32768, False)):
+        g = dl.LayerGeometry(model_dim=MODEL_DIM, query_heads=ATTN_DIM // 128,
+                             kv_heads=KV_DIM // 128, head_dim=128, ffn_dim=FFN_DIM,
+                             sliding_window=keys)
+        position = 5000 if local else keys - 1
+        caches = []
+        for _ in range(layers):
+            cache = dl.LayerCache(g, device)
+            cache.keys.copy_(torch.randn(cache.keys.shape, device=device).to(torch.bfloat16).view(torch.int16))
+            cache.values.copy_(torch.randn(cache.values.shape, device=device).to(torch.bfloat16).view(torch.int16))
+            caches.append(cache)
+        cache_bytes = layers * 2 * keys * g.kv_dim * 2
+        forms = (("reference_fused_attention", None, dl.LAUNCHES_PER_LAYER),
+                 ("split_attention", engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim, device),
+                  dl.LAUNCHES_PER_LAYER_SPLIT))
+        for name, attention_workspace, launches in forms:
+            def token():
+                pending, residual, pending_norm = embedding, zeros, None
+                for layer_weights, cache in zip(weights, caches):
+                    pending, residual = dl.decode_layer(g, layer_weights, cache, pending, residual,
+                                                        pending_norm, position, workspace, local,
+                                                        attention_workspace)
+                    pending_norm = layer_weights.post_feedforward_norm
+                last["hidden"] = residual
 
-        ms = time_graph(token, stream, max(5, steps // 2), max(2, warmup // 2))
-        if not bool(torch.isfinite(last["hidden"]).all()):
-            raise RuntimeError("the decode-layer chain produced a non-finite hidden state")
-        per_layer_us = ms * 1e3 / layers
-        result[name] = {
-            "us_per_layer": round(per_layer_us, 2),
-            "launches_per_layer": launches,
-            "weight_GB/s": round(weight_bytes / ms / 1e6, 1),
-            "frac_hbm": round((weight_bytes + cache_bytes) / ms / 1e6 / HBM_PEAK_GBS, 4),
-            "tokens/s_at_48_layers_without_lm_head": round(1e6 / (48 * per_layer_us), 1)}
+            ms = time_graph(token, stream, max(5, steps // 2), max(2, warmup // 2))
+            if not bool(torch.isfinite(last["hidden"]).all()):
+                raise RuntimeError("the decode-layer chain produced a non-finite hidden state")
+            per_layer_us = ms * 1e3 / layers
+            entry = {
+                "us_per_layer": round(per_layer_us, 2),
+                "launches_per_layer": launches,
+                "weight_GB/s": round(weight_bytes / ms / 1e6, 1),
+                "frac_hbm": round((weight_bytes + cache_bytes) / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            if local:
+                entry["tokens/s_at_48_layers_without_lm_head"] = round(1e6 / (48 * per_layer_us), 1)
+                result[name] = entry
+            else:
+                result.setdefault("global_32768_keys", {})[name] = entry
+        if local:
+            # the verifier's block of 16 tokens through the same layers (batch forms of the
+            # operators, causal block attention, no commit)
+            rows = 16
+            block = torch.from_numpy(kquant.synthetic_activations(42, rows, MODEL_DIM)).to(device)
+            block_zeros = torch.zeros_like(block)
+            block_workspace = tile_ops.small_batch_workspace(rows, FFN_DIM, device)
+            for name, attention_workspace, _ in forms:
+                def verify():
+                    pending, residual, pending_norm = block, block_zeros, None
+                    for layer_weights, cache in zip(weights, caches):
+                        pending, residual, _, _ = dl.verify_layer(
+                            g, layer_weights, cache, pending, residual, pending_norm, position,
+                            block_workspace, True, attention_workspace)
+                        pending_norm = layer_weights.post_feedforward_norm
+                    last["hidden"] = residual
+
+                ms = time_graph(verify, stream, max(5, steps // 2), max(2, warmup // 2))
+                if not bool(torch.isfinite(last["hidden"]).all()):
+                    raise RuntimeError("the verifier chain produced a non-finite hidden state")
+                result.setdefault("verify_block_16_rows", {})[name] = {
+                    "us_per_layer": round(ms * 1e3 / layers, 2),
+                    "weight_GB/s": round(weight_bytes / ms / 1e6, 1)}
+        del caches
     return result
 
 

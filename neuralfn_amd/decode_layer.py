@@ -122,5 +122,47 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     return down, hidden
 
 
+def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
+                 pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
+                 attention_workspace=None):
+    """A block of tokens (rows of `pending`, at positions position, position + 1, ...) through
+    one layer the way the verifier runs it (resident_glimmer_cuda.cpp:2913-2960, 3437-3520): the
+    same operators in their batch forms, a causal block attention over the cache and the
+    block's own rows, and no cache commit -- the block's key/value rows are returned for the
+    commit of the accepted ones (cache_commit, cache_commit_layers).  Row r equals decode_layer
+    at position + r after the commits of the rows before it, to rounding.
+
+    Returns (down, hidden, key_rows, value_rows).
+    """
+    g = geometry
+    rows = pending.shape[0]
+    hidden, normalized, _ = tile_ops.dual_rms_add_capture(
+        pending, residual, pending_norm, False, weights.input_norm, False,
+        g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps)
+    query, key, value, gate = tile_ops.multi_linear(
+        [weights.q, weights.k, weights.v, weights.attention_gate], normalized, workspace)
+    query = query.view(rows, g.query_heads, g.head_dim)
+    key = key.view(rows, g.kv_heads, g.head_dim)
+    value = value.view(rows, g.kv_heads, g.head_dim)
+    layout = engine_ops.ROPE_INTERLEAVED if g.interleaved_rope else engine_ops.ROPE_HALF_SPLIT
+    engine_ops.qk_norm_scale_rope(query, key, weights.q_norm, weights.k_norm, g.norm_eps, 1.0,
+                                  position, g.rope_theta, layout, local)
+    # a local layer's row sees its last sliding_window keys, a global one everything
+    window = g.sliding_window if local else position + rows
+    attention = engine_ops.block_attention(query, key, value, cache.keys, cache.values, position,
+                                           window, g.head_dim ** -0.5, True,
+                                           workspace=attention_workspace)
+    (projected,) = tile_ops.multi_linear([weights.output], attention.view(rows, g.attention_dim),
+                                         workspace, second=gate, prologue="gated")
+    hidden, normalized, _ = tile_ops.dual_rms_add_capture(
+        projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
+        g.post_norm_eps, g.norm_eps)
+    mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
+                                             workspace)
+    (down,) = tile_ops.multi_linear([weights.mlp_down], mlp_gate, workspace, second=mlp_up,
+                                    prologue="swiglu")
+    return down, hidden, key, value
+
+
 LAUNCHES_PER_LAYER = 8           # with the reference's fused attention call
 LAUNCHES_PER_LAYER_SPLIT = 9     # with the split attention form (one more: the merge)

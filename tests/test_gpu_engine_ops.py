@@ -908,3 +908,91 @@ def test_two_decode_layers_against_the_cpu_engine_arithmetic(cuda, oracle):
             assert np.max(np.abs(committed - expected)) <= 2e-3 * np.max(np.abs(expected)) + 2.0 ** -8 * np.max(np.abs(expected))
         untouched = np.delete(np.arange(g.sliding_window), slot)
         assert np.array_equal(bits_of(cache.keys)[untouched], keys[untouched])
+
+
+@pytest.mark.parametrize("split", [False, True])
+def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, oracle, split):
+    """decode_layer.verify_layer runs a block of tokens through a layer in the batch forms of the
+    operators with a causal block attention and no commit; every row must come out as the
+    token-at-a-time chain (decode_layer, which commits) leaves it."""
+    from neuralfn_amd import decode_layer as dl
+    rng = np.random.default_rng(22)
+    g = dl.LayerGeometry(model_dim=512, query_heads=8, kv_heads=2, head_dim=128, ffn_dim=768,
+                         sliding_window=256)
+    rows, position, layers = 5, 700, 2  # the ring has wrapped
+    formats = dict(q=kquant.Q4_K, k=kquant.Q5_K, v=kquant.Q6_K, attention_gate=kquant.Q4_K,
+                   output=kquant.Q5_K, mlp_gate=kquant.Q4_K, mlp_up=kquant.Q8_0, mlp_down=kquant.Q6_K)
+    shapes = dict(q=(g.attention_dim, g.model_dim), k=(g.kv_dim, g.model_dim),
+                  v=(g.kv_dim, g.model_dim), attention_gate=(g.attention_dim, g.model_dim),
+                  output=(g.model_dim, g.attention_dim), mlp_gate=(g.ffn_dim, g.model_dim),
+                  mlp_up=(g.ffn_dim, g.model_dim), mlp_down=(g.model_dim, g.ffn_dim))
+    norms = dict(input_norm=g.model_dim, q_norm=g.head_dim, k_norm=g.head_dim,
+                 post_attention_norm=g.model_dim, pre_feedforward_norm=g.model_dim,
+                 post_feedforward_norm=g.model_dim)
+    stack, rings = [], []
+    for _ in range(layers):
+        device = {}
+        for name, (out_dim, in_dim) in shapes.items():
+            packed = kquant.quantize(formats[name],
+                                     (rng.standard_normal((out_dim, in_dim)) * 0.05).astype(np.float32))
+            device[name] = tile_ops.PackedWeight.from_numpy(formats[name], packed, out_dim, in_dim)
+        for name, width in norms.items():
+            row = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+            device[name] = tile_ops.PackedWeight.from_numpy(kquant.F32, row.view(np.uint8).copy(), 1, width)
+        stack.append(dl.LayerWeights(**device))
+        rings.append((oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32)),
+                      oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))))
+
+    def caches():
+        made = []
+        for keys, values in rings:
+            cache = dl.LayerCache(g, cuda)
+            cache.keys.copy_(bf16_tensor(keys, cuda))
+            cache.values.copy_(bf16_tensor(values, cuda))
+            made.append(cache)
+        return made
+
+    embeddings = rng.standard_normal((rows, g.model_dim)).astype(np.float32)
+    attention_workspace = engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim) if split else None
+
+    # token at a time, committing
+    serial_caches = caches()
+    workspace = tile_ops.small_batch_workspace(1, max(g.model_dim, g.ffn_dim, g.attention_dim))
+    serial_down, serial_hidden = [], []
+    for row in range(rows):
+        pending = to_device(embeddings[row:row + 1], cuda)
+        residual, pending_norm = torch_().zeros_like(pending), None
+        for weights, cache in zip(stack, serial_caches):
+            pending, residual = dl.decode_layer(g, weights, cache, pending, residual, pending_norm,
+                                                position + row, workspace, True, attention_workspace)
+            pending_norm = weights.post_feedforward_norm
+        serial_down.append(pending.cpu().numpy()[0])
+        serial_hidden.append(residual.cpu().numpy()[0])
+
+    # the block, then the commit of all its rows
+    block_caches = caches()
+    workspace = tile_ops.small_batch_workspace(rows, max(g.model_dim, g.ffn_dim, g.attention_dim))
+    pending = to_device(embeddings, cuda)
+    residual, pending_norm = torch_().zeros_like(pending), None
+    staged = []
+    for weights, cache in zip(stack, block_caches):
+        pending, residual, key_rows, value_rows = dl.verify_layer(
+            g, weights, cache, pending, residual, pending_norm, position, workspace, True,
+            attention_workspace)
+        pending_norm = weights.post_feedforward_norm
+        staged.append((key_rows, value_rows))
+
+    def error(actual, expected):
+        return float(np.max(np.abs(actual - expected)) / np.max(np.abs(expected)))
+
+    # the projections of a block and of one token quantize their activations in different
+    # kernels: each within 2e-3 of the float formula, here about 1e-4 apart
+    assert error(residual.cpu().numpy(), np.stack(serial_hidden)) <= 1e-3
+    assert error(pending.cpu().numpy(), np.stack(serial_down)) <= 1e-3
+    for cache, serial_cache, (key_rows, value_rows) in zip(block_caches, serial_caches, staged):
+        engine_ops.cache_commit(key_rows, value_rows, cache.keys, cache.values, position, rows=rows)
+        # committed rows carry the upstream rounding differences: a bf16 step apart at most
+        for ours, theirs in ((cache.keys, serial_cache.keys), (cache.values, serial_cache.values)):
+            ours = oracle.bf16_to_float(bits_of(ours)).astype(np.float64)
+            theirs = oracle.bf16_to_float(bits_of(theirs)).astype(np.float64)
+            assert np.max(np.abs(ours - theirs)) <= 2.0 ** -7 * np.max(np.abs(theirs))
