@@ -171,3 +171,71 @@ def test_attention_random_case(cuda, oracle, seed):
             to_device(block_query, cuda), to_device(block_key, cuda), to_device(block_value, cuda),
             device_keys, device_values, context, window, scale, causal).cpu().numpy()
         assert np.abs(actual - expected).max() <= 4e-6, f"{label}, block {rows}/{block_rows}, causal {causal}"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_matrix_core_attention_random_case(cuda, oracle, seed):
+    """Geometries of the matrix-core kernel (head size 128, four or more query heads per key/value
+    head, also more than 16 and not a multiple of 16): the split one-token form with the position on
+    the host and on the device, and blocks large enough to take that kernel, unsplit and split, in
+    both modes.  Padded cache rows, rings that wrapped, windows that cut the context, short rings."""
+    from neuralfn_amd import engine_ops
+    rng = np.random.default_rng(5000 + seed)
+    head_dim = 128
+    kv_heads = int(rng.choice([1, 2, 3, 8]))
+    per_kv = int(rng.choice([4, 5, 16, 17, 20, 32]))
+    query_heads = kv_heads * per_kv
+    capacity = int(rng.choice([64, 100, 130, 512, 2048, 5000]))
+    padding = int(rng.choice([0, 0, 8, 24]))
+    stride = kv_heads * head_dim + padding
+    position = int(rng.integers(0, 3 * capacity))
+    window = int(rng.integers(1, capacity + 1))
+    first = max(0, position - window + 1)
+    scale = float(head_dim ** -0.5)
+    key_cache, value_cache = _bf16(oracle, rng, (capacity, stride)), _bf16(oracle, rng, (capacity, stride))
+    device_keys, device_values = _bf16_tensor(key_cache, cuda), _bf16_tensor(value_cache, cuda)
+    label = (f"heads {query_heads}/{kv_heads}, ring {capacity} x {stride}, position {position}, "
+             f"window {window}")
+
+    query = rng.standard_normal((query_heads, head_dim)).astype(np.float32)
+    key = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    value = rng.standard_normal((kv_heads, head_dim)).astype(np.float32)
+    expected = oracle.gqa_decode(query, key, value, key_cache, value_cache, position, first, scale)
+    workspace = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+    workspace.fill_(0xFF)
+    split = engine_ops.gqa_decode(to_device(query, cuda), to_device(key, cuda), to_device(value, cuda),
+                                  device_keys, device_values, position, first, scale,
+                                  workspace=workspace).cpu().numpy()
+    assert np.abs(split - expected).max() <= 4e-6, label + " (split form)"
+    # position on the device, no norm weights and no rope: the fused call is attention + commit
+    device_position = to_device(np.array([position], dtype=np.int64), cuda)
+    keys_copy, values_copy = device_keys.clone(), device_values.clone()
+    fused = engine_ops.fused_decode_attention(
+        to_device(query, cuda), to_device(key, cuda), to_device(value, cuda), keys_copy, values_copy,
+        3, 1, scale, None, None, 1e-5, 1.0, 500000.0, engine_ops.ROPE_INTERLEAVED, True,
+        device_position=device_position, sliding_window=window, workspace=workspace)
+    # that call normalises query and key per head first (no weights): compare with the oracle on those
+    normalized_query = oracle.rope(np.stack([oracle.rms_norm(row, None, False, 1e-5) for row in query]),
+                                   position, 500000.0, True)
+    normalized_key = oracle.rope(np.stack([oracle.rms_norm(row, None, False, 1e-5) for row in key]),
+                                 position, 500000.0, True)
+    expected_fused = oracle.gqa_decode(normalized_query, normalized_key, value, key_cache, value_cache,
+                                       position, first, scale)
+    assert np.abs(fused.cpu().numpy() - expected_fused).max() <= 6e-6, label + " (fused, device position)"
+
+    rows = int(rng.integers(1, 17))
+    # more rows x heads than compute units where 64 block rows allow it: the matrix cores
+    rows = min(max(rows, 256 // query_heads + 1), 62)
+    block_rows = rows + int(rng.integers(0, 3))
+    block_query = rng.standard_normal((rows, query_heads, head_dim)).astype(np.float32)
+    block_key = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    block_value = rng.standard_normal((block_rows, kv_heads, head_dim)).astype(np.float32)
+    for causal in (True, False):
+        expected = oracle.block_attention(block_query, block_key, block_value, key_cache, value_cache,
+                                          position, window, scale, causal)
+        arguments = (to_device(block_query, cuda), to_device(block_key, cuda), to_device(block_value, cuda),
+                     device_keys, device_values, position, window, scale, causal)
+        for lent in (None, workspace):
+            actual = engine_ops.block_attention(*arguments, workspace=lent).cpu().numpy()
+            assert np.abs(actual - expected).max() <= 4e-6, \
+                f"{label}, block {rows}/{block_rows}, causal {causal}, split {lent is not None}"
