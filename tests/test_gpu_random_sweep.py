@@ -157,6 +157,26 @@ def test_attention_random_case(cuda, oracle, seed):
     workspace.fill_(0xFF)
     split = engine_ops.gqa_decode(*arguments, workspace=workspace).cpu().numpy()
     assert np.abs(split - expected).max() <= 4e-6, label + " (split form)"
+    # the fused call with the position on the device and the split form (no norm weights):
+    # per-head norm and rope of query and key, then the same attention, then the commit
+    device_position = to_device(np.array([position], dtype=np.int64), cuda)
+    keys_copy, values_copy = device_keys.clone(), device_values.clone()
+    fused = engine_ops.fused_decode_attention(
+        to_device(query, cuda), to_device(key, cuda), to_device(value, cuda), keys_copy, values_copy,
+        3, 1, scale, None, None, 1e-5, 1.0, 500000.0, engine_ops.ROPE_HALF_SPLIT, True,
+        device_position=device_position, sliding_window=window, workspace=workspace).cpu().numpy()
+    normalized_query = oracle.rope(np.stack([oracle.rms_norm(row, None, False, 1e-5) for row in query]),
+                                   position, 500000.0, False)
+    normalized_key = oracle.rope(np.stack([oracle.rms_norm(row, None, False, 1e-5) for row in key]),
+                                 position, 500000.0, False)
+    expected_fused = oracle.gqa_decode(normalized_query, normalized_key, value, key_cache, value_cache,
+                                       position, first, scale)
+    assert np.abs(fused - expected_fused).max() <= 6e-6, label + " (fused, device position, split)"
+    # the committed key row: the normalised, rotated key, a bf16 rounding step apart at most
+    committed = oracle.bf16_to_float(
+        keys_copy.cpu().numpy().view(np.uint16)[position % capacity, :kv_heads * head_dim])
+    assert np.abs(committed - normalized_key.reshape(-1)).max() <= \
+        2.0 ** -7 * np.abs(normalized_key).max(), label
 
     rows = int(rng.integers(1, 9))
     block_rows = rows + int(rng.integers(0, 5))
