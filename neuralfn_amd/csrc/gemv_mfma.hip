@@ -762,10 +762,18 @@ void launch_tokens(const ProjectionSet& set, const Pass& pass) {
         }
     }
     if constexpr (kStreamFits) {
-        launch_variant<ENC, S, kStream, P, ARGMAX>(set, pass);
-    } else {
-        launch_variant<ENC, S, kWorkspace, kPlain, ARGMAX>(set, pass);
+        // Streamed quantization repeats for every tile of a workgroup: with two or more
+        // tiles each, one quantizer launch and records read from the workspace are cheaper.
+        std::int64_t tiles = 0;
+        for (int index = 0; index < set.count; ++index) {
+            tiles += (set.op[index].output_dim + kTileRows - 1) / kTileRows;
+        }
+        if (tiles < 2 * static_cast<std::int64_t>(compute_units()) || pass.workspace == nullptr) {
+            launch_variant<ENC, S, kStream, P, ARGMAX>(set, pass);
+            return;
+        }
     }
+    launch_variant<ENC, S, kWorkspace, kPlain, ARGMAX>(set, pass);
 }
 
 template <std::uint32_t ENC, int P, bool ARGMAX>

@@ -894,3 +894,25 @@ def test_shader_clock_probe_reports_a_plausible_clock():
     assert lib.nfn_mi355_shader_clock_probe_v1(None, 100, None) == 1
     assert lib.nfn_mi355_shader_clock_probe_v1(probe.result.data_ptr(), 0, None) == 1
     assert lib.nfn_mi355_shader_clock_probe_v1(probe.result.data_ptr(), 100001, None) == 1
+
+
+@pytest.mark.parametrize("prologue", ["plain", "swiglu"])
+@pytest.mark.parametrize("rows", [5, 8])
+def test_many_tile_launches_at_five_to_eight_rows_equal_narrow_ones(cuda, prologue, rows):
+    """With two or more 32-row tiles per compute unit the 5..8-row launches quantize the
+    activations once (a quantizer launch and the workspace) instead of once per tile in the
+    kernel: same records, so the same bits as a launch over a slice of the rows."""
+    in_dim, out_dim, narrow = 512, 16640, 96  # 2 x 520 tiles; the slice is three tiles
+    packed = [random_packed(kquant.Q4_K, out_dim, in_dim, 70 + index) for index in range(2)]
+    wide = [tile_ops.PackedWeight.from_numpy(kquant.Q4_K, p, out_dim, in_dim) for p in packed]
+    row_bytes = packed[0].size // out_dim
+    first, last = out_dim - narrow, out_dim
+    sliced = [tile_ops.PackedWeight.from_numpy(kquant.Q4_K, p.reshape(-1)[first * row_bytes:].copy(),
+                                               narrow, in_dim) for p in packed]
+    x = to_device(kquant.synthetic_activations(71, rows, in_dim), cuda)
+    second = to_device(kquant.synthetic_activations(72, rows, in_dim), cuda) if prologue != "plain" else None
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    many = tile_ops.multi_linear(wide, x, workspace, second, "mmq", prologue)
+    few = tile_ops.multi_linear(sliced, x, workspace, second, "mmq", prologue)
+    for whole, part in zip(many, few):
+        assert_bits_equal(whole[:, first:last].contiguous(), part, "many tiles vs few")
