@@ -38,7 +38,16 @@
 //                       reference probe's equality rule
 //                       (tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:968-1007).
 //   nfo_linear_q8_1     closed form over reconstructed activations, same rule
-//                       as tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1009-1023.
+//                       as tests/cpp/muse_glimmer_cuda_kernel_probe.cpp:1009-1023;
+//                       checked against an independent float64 numpy statement
+//                       (round_fp16(scale) * code) @ dequantized.T, which the
+//                       unrounded scale fails.
+//   nfo_sigmoid_gate    bit-equal to the reference's CPU stand-in for its sidecar
+//                       (tests/cpp/fake_glimmer_tile_ops.cpp:570), live and by
+//                       committed vectors; float64 closed form; operand swap fails.
+//   nfo_swiglu          within 4 ulp of that stand-in (:1105, which associates
+//                       gate*sigmoid*up differently from the device form restated
+//                       here), live and by committed vectors; float64 closed form.
 //   nfo_rms_norm        equals the compiled reference rms_norm() bit for bit where
 //                       that builds; closed form x / sqrt(mean(x^2) + eps) in numpy.
 //   nfo_rms_norm_strict, nfo_dual_rms_add_capture  within the reference probe's 2e-5 of the double
