@@ -737,6 +737,22 @@ int nfn_mi355_k_quant_gemm_float32_v1(
     int mode,
     void* cuda_stream);
 
+/* How the call above cuts a problem of this geometry on the current device
+ * (no counterpart in the reference; for tests and benchmarks that want to know
+ * which launch form they exercised): *tile_rows = output rows per workgroup
+ * tile (128 or 256), *k_shares = workgroups that share the K range of a tile
+ * (1 = unsplit; with more, each writes a partial output into the workspace and
+ * a second launch adds them in share order).  0 on success, 1 for an encoding
+ * or width the matrix-core path does not take, or the reserved mode. */
+int nfn_mi355_k_quant_gemm_plan_v1(
+    uint32_t encoding,
+    int64_t rows,
+    int64_t input_dim,
+    int64_t output_dim,
+    int mode,
+    int* tile_rows,
+    int* k_shares);
+
 /* The same for 1..4 projections of one input (Q/K/V, gate/up), the way the
  * small-batch entry points group them: the activations are converted once and
  * every projection runs from that copy.  All descriptors share input_dim (a

@@ -540,6 +540,17 @@ std::int64_t nfn_mi355_k_quant_gemm_workspace_bytes_v1(std::int64_t rows, std::i
     return gemm_f16_workspace_bytes(rows, input_dim, output_dim);
 }
 
+int nfn_mi355_k_quant_gemm_plan_v1(std::uint32_t encoding, std::int64_t rows, std::int64_t input_dim,
+                                   std::int64_t output_dim, int mode, int* tile_rows,
+                                   int* k_shares) {
+    if (tile_rows == nullptr || k_shares == nullptr || rows <= 0 || output_dim <= 0 ||
+        input_dim <= 0 || mode != NFN_MI355_GEMM_F16 || !gemm_f16_supports(encoding, input_dim)) {
+        return kInvalid;
+    }
+    gemm_f16_plan(encoding, rows, input_dim, output_dim, tile_rows, k_shares);
+    return 0;
+}
+
 int nfn_mi355_k_quant_gemm_float32_v1(const Descriptor* descriptor, const float* input,
                                       float* output, std::int64_t rows, void* workspace,
                                       std::int64_t workspace_nbytes, int mode,

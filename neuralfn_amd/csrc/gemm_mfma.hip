@@ -817,6 +817,13 @@ std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim,
     return activation_bytes(rows, input_dim) + (shares > 1 ? shares * rows * output_dim * 4 : 0) + 256;
 }
 
+void gemm_f16_plan(std::uint32_t encoding, std::int64_t rows, std::int64_t input_dim,
+                   std::int64_t output_dim, int* tile_rows, int* k_shares) {
+    const Plan chosen = plan(encoding, rows, output_dim, input_dim);
+    *tile_rows = 128 * chosen.row_blocks;
+    *k_shares = chosen.shares;
+}
+
 bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
     return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K ||
             encoding == kEncQ8_0) && input_dim % 256 == 0;

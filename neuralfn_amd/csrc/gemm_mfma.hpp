@@ -12,6 +12,11 @@ namespace nfn {
 std::int64_t gemm_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim,
                                       std::int64_t output_dim);
 bool gemm_f16_supports(std::uint32_t encoding, std::int64_t input_dim);
+// How a launch of this geometry is cut on the current device: rows of the
+// output tile a workgroup owns (128 or 256) and the number of K shares (1 =
+// unsplit; more = one partial output per share, summed by a second launch).
+void gemm_f16_plan(std::uint32_t encoding, std::int64_t rows, std::int64_t input_dim,
+                   std::int64_t output_dim, int* tile_rows, int* k_shares);
 // output[rows, output_dim] = input[rows, input_dim] * W^T, float accumulation.
 void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,
                       std::int64_t rows, void* workspace, hipStream_t stream);

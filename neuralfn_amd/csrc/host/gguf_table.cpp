@@ -10,6 +10,7 @@
 
 #include <algorithm>
 #include <cstring>
+#include <exception>
 #include <limits>
 #include <string>
 #include <unordered_map>
@@ -162,8 +163,9 @@ int parse(NfnMi355GgufFileV1* file) {
     if (version != 3) return kVersion;
     if (!cursor.read(&tensor_count) || !cursor.read(&file->metadata_count)) return kTruncated;
     if (tensor_count == 0) return kEmpty;
-    // every entry takes bytes: counts larger than the file are malformed
-    if (tensor_count > file->size || file->metadata_count > file->size) return kTruncated;
+    // every entry takes bytes: a tensor info is at least 32 (name length, rank, one
+    // dimension, encoding, offset), a metadata entry at least 13 (key length, type, one byte)
+    if (tensor_count > file->size / 32 || file->metadata_count > file->size / 13) return kTruncated;
 
     for (std::uint64_t entry = 0; entry < file->metadata_count; ++entry) {
         std::string key;
@@ -173,7 +175,7 @@ int parse(NfnMi355GgufFileV1* file) {
         if (!skip_value(&cursor, type, 0)) return kMetadata;
     }
 
-    file->tensors.reserve(tensor_count);
+    file->tensors.reserve(static_cast<std::size_t>(tensor_count < 4096 ? tensor_count : 4096));
     for (std::uint64_t index = 0; index < tensor_count; ++index) {
         Tensor tensor;
         std::uint64_t dimensions[2] = {1, 1};
@@ -267,7 +269,12 @@ int nfn_mi355_gguf_open_v1(const char* path, NfnMi355GgufFileV1** file) {
     auto* handle = new NfnMi355GgufFileV1();
     handle->data = static_cast<const std::uint8_t*>(mapping);
     handle->size = static_cast<std::uint64_t>(status.st_size);
-    const int code = parse(handle);
+    int code = kArgument;
+    try {
+        code = parse(handle);
+    } catch (const std::exception&) {  // allocation failure or the like: no exception leaves this call
+        code = kTruncated;
+    }
     if (code != kOk) {
         nfn_mi355_gguf_close_v1(handle);
         return code;

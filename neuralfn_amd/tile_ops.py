@@ -185,6 +185,8 @@ SIGNATURES = {
     "nfn_mi355_lm_head_argmax_workspace_bytes_v1": (_I64, [_I64, _I64]),
     "nfn_mi355_lm_head_argmax_v1": (ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P, _I64, _P]),
     "nfn_mi355_k_quant_gemm_workspace_bytes_v1": (_I64, [_I64, _I64, _I64, ctypes.c_int]),
+    "nfn_mi355_k_quant_gemm_plan_v1": (
+        ctypes.c_int, [ctypes.c_uint32, _I64, _I64, _I64, ctypes.c_int, _P, _P]),
     "nfn_mi355_k_quant_gemm_float32_v1": (
         ctypes.c_int, [_DESC, _P, _P, _I64, _P, _I64, ctypes.c_int, _P]),
     "nfn_mi355_k_quant_gemm_multi_float32_v1": (
@@ -590,6 +592,15 @@ def gemm(weight: PackedWeight, x, mode: int = GEMM_F16, workspace=None, out=None
         ctypes.byref(descriptor), x.data_ptr(), out.data_ptr(), rows, workspace.data_ptr(),
         workspace.numel(), mode, stream), "k_quant_gemm")
     return out
+
+
+def gemm_plan(encoding: int, rows: int, input_dim: int, output_dim: int, mode: int = GEMM_F16):
+    """nfn_mi355_k_quant_gemm_plan_v1: (rows per workgroup tile, K shares) of a launch."""
+    tile_rows, shares = ctypes.c_int(0), ctypes.c_int(0)
+    check(load().nfn_mi355_k_quant_gemm_plan_v1(
+        encoding, rows, input_dim, output_dim, mode, ctypes.addressof(tile_rows),
+        ctypes.addressof(shares)), "k_quant_gemm_plan")
+    return tile_rows.value, shares.value
 
 
 def gemm_multi(weights: Sequence[PackedWeight], x, mode: int = GEMM_F16, workspace=None,

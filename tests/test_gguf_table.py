@@ -183,6 +183,17 @@ def test_malformed_files_are_refused(tmp_path):
     path.write_bytes(blob)
     _expect(path, 6)
     _expect(tmp_path / "absent.gguf", 2)
+    # a header that claims more tensors (or metadata entries) than the file has bytes for is
+    # refused before anything is reserved for them
+    write_gguf(good, tensors, METADATA)
+    for field_offset in (8, 16):
+        blob = bytearray(good.read_bytes())
+        blob[field_offset:field_offset + 8] = struct.pack("<Q", len(blob) // 32 + 1)
+        path.write_bytes(blob)
+        _expect(path, 3)
+        blob[field_offset:field_offset + 8] = struct.pack("<Q", (1 << 63) - 1)
+        path.write_bytes(blob)
+        _expect(path, 3)
 
 
 @pytest.mark.gpu

@@ -784,12 +784,19 @@ def test_prefill_gemm_tall_tiles(cuda, oracle, encoding):
     assert normalised_error(y[picked], expected) <= TOLERANCE
 
 
-@pytest.mark.parametrize("in_dim", [4096, 6144])
+@pytest.mark.parametrize("rows,in_dim,plan", [
+    (96, 4096, (128, 1)),    # sixteen blocks: too short to give two shares twelve each
+    (96, 6144, (128, 2)),    # 24 blocks -> two shares of 128-row tiles
+    (96, 9216, (128, 3)),    # 36 blocks -> three
+    (200, 9216, (256, 3)),   # more than 128 rows keep 256-row tiles while two shares or more fit
+    (200, 12544, (256, 4)),  # 49 blocks -> four shares of unequal length (13, 12, 12, 12)
+])
 @pytest.mark.parametrize("encoding", ALL_PACKED)
-def test_prefill_gemm_split_k(cuda, oracle, encoding, in_dim):
-    # few tiles and a long K: the launch splits K into shares (two at 16 blocks,
-    # three at 24) and a second launch sums them
-    rows, out_dim = 96, 130
+def test_prefill_gemm_split_k(cuda, oracle, encoding, rows, in_dim, plan):
+    # few tiles and a long K: the launch splits K into shares of at least twelve
+    # 256-value blocks (at most four) and a second launch sums them in share order
+    out_dim = 130
+    assert tile_ops.gemm_plan(encoding, rows, in_dim, out_dim) == plan
     packed = kquant.quantize(encoding, kquant.synthetic_weights(70 + encoding, out_dim, in_dim))
     x = kquant.synthetic_activations(71, rows, in_dim)
     weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
@@ -865,6 +872,50 @@ def test_prefill_gemm_full_size_row_subset(cuda, oracle):
     assert normalised_error(y[:, :256], expected) <= TOLERANCE
     # every 256-column stripe repeats the same weights
     assert np.array_equal(y[:, :256], y[:, out_dim - 256:])
+
+
+def gemm_subset_check(cuda, oracle, encoding, rows, out_dim, in_dim, seed, plan):
+    """A full-size GEMM with distinct random weights in every column, compared with the oracle on a
+    spread of rows (tile edges, both halves of every 256-row tile kind) and of column stripes
+    (first, last and interior 128-column tiles, edges of each)."""
+    assert tile_ops.gemm_plan(encoding, rows, in_dim, out_dim) == plan
+    packed = random_packed(encoding, out_dim, in_dim, seed)
+    x = kquant.synthetic_activations(seed + 1, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.gemm(weight, to_device(x, cuda), tile_ops.GEMM_F16).cpu().numpy()
+    rng = np.random.default_rng(seed + 2)
+    picked_rows = np.unique(np.concatenate([
+        np.array([0, 1, 31, 32, 127, 128, 255, rows - 256, rows - 129, rows - 128, rows - 33, rows - 1]),
+        rng.integers(0, rows, 12)]))
+    starts = [0, 120, out_dim // 2 - 8, out_dim - 136, out_dim - 16]
+    picked_columns = np.unique(np.concatenate([np.arange(start, start + 16) for start in starts] +
+                                              [rng.integers(0, out_dim, 48)]))
+    row_bytes = packed.size // out_dim
+    stripe = np.ascontiguousarray(packed.reshape(out_dim, row_bytes)[picked_columns]).reshape(-1)
+    expected = oracle.linear(encoding, stripe, picked_columns.size, in_dim,
+                             np.ascontiguousarray(x[picked_rows]))
+    assert normalised_error(y[np.ix_(picked_rows, picked_columns)], expected) <= TOLERANCE
+    return y
+
+
+@pytest.mark.parametrize("rows", [512, 2048])
+def test_prefill_gemm_config3_gate_up_shape(cuda, oracle, rows):
+    # SwiGLU FFN prefill, gate / up projection: 6,656 -> 16,384 at both row counts
+    gemm_subset_check(cuda, oracle, kquant.Q4_K, rows, 16384, 6656, 300 + rows, (256, 1))
+
+
+@pytest.mark.parametrize("rows,plan", [(512, (256, 4)), (2048, (256, 1))])
+def test_prefill_gemm_config3_down_shape(cuda, oracle, rows, plan):
+    # the down projection 16,384 -> 6,656 (64 blocks of K): 512 rows give 104 tall tiles for 256
+    # compute units, so K is split into four shares; 2,048 rows run unsplit
+    y = gemm_subset_check(cuda, oracle, kquant.Q4_K, rows, 6656, 16384, 400 + rows, plan)
+    assert np.all(np.isfinite(y))
+
+
+@pytest.mark.parametrize("encoding", [kquant.Q5_K, kquant.Q6_K, kquant.Q8_0])
+def test_prefill_gemm_config4_prefill_shapes(cuda, oracle, encoding):
+    # the mixed-format profile's prefill half: 1,024 rows, FFN down in the formats it may draw
+    gemm_subset_check(cuda, oracle, encoding, 1024, 6656, 16384, 500 + encoding, (256, 2))
 
 
 def test_decode_gemv_is_deterministic(cuda):
