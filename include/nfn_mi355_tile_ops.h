@@ -715,6 +715,31 @@ int nfn_mi355_lm_head_argmax_v1(
     int64_t workspace_nbytes,
     void* cuda_stream);
 
+/* nfn_mi355_lm_head_argmax_v1 for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc) and therefore have no workspace to pass.  No counterpart in the
+ * reference.  Same arguments without the workspace, same kernels, same
+ * results bit for bit: the candidate records of the first pass live in a
+ * device array inside the library, NFN_MI355_LM_HEAD_NO_ALLOC_SCRATCH_BYTES
+ * per GPU, held from library load until the process ends.  The call allocates
+ * and frees nothing.  A problem whose workspace
+ * (nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, output_dim)) exceeds that
+ * size is refused with NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED; the full
+ * 202,048-row vocabulary at 8 rows needs 808,192 bytes and fits.  Every call
+ * on a GPU uses that GPU's one array: calls that overlap on a device
+ * (different streams, concurrently replayed graphs) race on it.  The first
+ * call on a device looks the array's address up in the runtime
+ * (hipGetSymbolAddress); make that call before a capture begins. */
+#define NFN_MI355_LM_HEAD_NO_ALLOC_SCRATCH_BYTES (1 << 20)
+#define NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED 0x4e46
+int nfn_mi355_lm_head_argmax_no_alloc_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* descriptor,
+    const float* input,
+    int64_t* output_indices,
+    float* output_values,
+    int64_t rows,
+    void* cuda_stream);
+
 /* Prefill dequant-GEMM for any row count: output[rows, output_dim] =
  * input[rows, input_dim] * W^T.  The reference's small-batch entry points stop
  * at 16 rows (glimmer_k_mmq.cu:1326-1328) and its only route for more rows is

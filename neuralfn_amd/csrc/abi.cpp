@@ -136,6 +136,9 @@ int nfn_native_tile_k_quant_mmq_abi_version(void) { return NFN_NATIVE_TILE_K_QUA
 int nfn_mi355_abi_version(void) { return 1; }
 
 const char* nfn_native_tile_ops_error_string(int code) {
+    if (code == NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED) {
+        return "the problem needs more scratch than the no-allocation entry point holds";
+    }
     const char* text = hipGetErrorString(static_cast<hipError_t>(code));
     return text != nullptr ? text : "unknown error";
 }

@@ -184,6 +184,7 @@ SIGNATURES = {
     "nfn_native_tile_swiglu_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
     "nfn_mi355_lm_head_argmax_workspace_bytes_v1": (_I64, [_I64, _I64]),
     "nfn_mi355_lm_head_argmax_v1": (ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P, _I64, _P]),
+    "nfn_mi355_lm_head_argmax_no_alloc_v1": (ctypes.c_int, [_DESC, _P, _P, _P, _I64, _P]),
     "nfn_mi355_k_quant_gemm_workspace_bytes_v1": (_I64, [_I64, _I64, _I64, ctypes.c_int]),
     "nfn_mi355_k_quant_gemm_plan_v1": (
         ctypes.c_int, [ctypes.c_uint32, _I64, _I64, _I64, ctypes.c_int, _P, _P]),
@@ -571,6 +572,21 @@ def lm_head_argmax(weight: PackedWeight, x, workspace=None, indices=None, maxima
     check(load().nfn_mi355_lm_head_argmax_v1(
         ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), rows,
         workspace.data_ptr(), workspace.numel(), stream), "lm_head_argmax")
+    return indices, maxima
+
+
+STATIC_SCRATCH_EXCEEDED = 0x4e46  # NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED
+LM_HEAD_NO_ALLOC_SCRATCH_BYTES = 1 << 20
+
+
+def lm_head_argmax_no_alloc(weight: PackedWeight, x, indices, maxima):
+    """nfn_mi355_lm_head_argmax_no_alloc_v1: the fused lm_head argmax with the library's own
+    scratch; the caller passes inputs and outputs only and nothing is allocated."""
+    stream = _stream_handle()
+    descriptor = weight.descriptor(stream)
+    check(load().nfn_mi355_lm_head_argmax_no_alloc_v1(
+        ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), x.shape[0],
+        stream), "lm_head_argmax_no_alloc")
     return indices, maxima
 
 
