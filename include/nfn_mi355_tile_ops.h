@@ -852,16 +852,20 @@ int nfn_mi355_dflash_block_attention_split_v1(
  * and its short_split form) a workspace for the split forms above, so
  * that an engine's unchanged call sites take it: from this call on they run as
  * their nfn_mi355_*_split_* counterparts whenever the workspace is on the
- * current device and large enough for the call's geometry
+ * current device, was lent for the stream the call is issued on
+ * (descriptor->cuda_stream) and is large enough for the call's geometry
  * (nfn_mi355_gqa_decode_split_workspace_bytes_v1; a block takes as many shares
- * as fit), and as before otherwise.
- * (nullptr, 0) takes it back.  No counterpart in the reference.  The memory
- * stays the caller's; every such call uses the same memory, so calls that
- * overlap on the device (different streams, concurrently replayed graphs) race
- * on it -- lend one only to an engine that issues its attention calls in stream
- * order.  Calls already captured into a graph keep the form they were captured
- * with.  0 on success, 1 for a misaligned pointer or a size without a pointer. */
-int nfn_mi355_attention_workspace_v1(void* workspace, int64_t workspace_nbytes);
+ * as fit), and as before otherwise.  One loan per (device, stream), at most 32
+ * at a time; lending again for the same stream replaces the loan;
+ * (nullptr, 0, stream) takes that stream's loan back.  No counterpart in the
+ * reference.  The memory stays the caller's.  Calls on the loan's stream run
+ * in stream order, so they never write the workspace at once; calls on other
+ * streams do not see it.  What still races: graphs captured from that stream
+ * and replayed concurrently with each other or with it -- give such graphs
+ * the explicit *_split_v1 entry points with a workspace each.  Calls already
+ * captured into a graph keep the form they were captured with.  0 on success,
+ * 1 for a misaligned pointer, a size without a pointer, or a 33rd loan. */
+int nfn_mi355_attention_workspace_v1(void* workspace, int64_t workspace_nbytes, void* cuda_stream);
 
 /* Shader clock under load, a measurement aid (no counterpart in the reference;
  * for benchmarks that price a kernel against the matrix-core peak at the clock

@@ -19,33 +19,34 @@ constexpr std::int64_t kLimit = std::numeric_limits<std::int64_t>::max();
 
 bool positive_finite(float value) { return std::isfinite(value) && value > 0.0f; }
 
-// The workspace an engine lent to the reference-named one-token attention entry
-// points (nfn_mi355_attention_workspace_v1): device it belongs to, address, size.
+// Workspaces an engine lent to the reference-named attention entry points
+// (nfn_mi355_attention_workspace_v1), one per (device, stream): a loan serves
+// only calls issued on the stream it was made for, whose work is ordered, so
+// two calls never write the same partial results at once.
 struct LentWorkspace {
     int device = -1;
-    float* memory = nullptr;
+    void* stream = nullptr;
+    float* memory = nullptr;  // null = free slot
     std::int64_t nbytes = 0;
 };
+constexpr int kMaxLoans = 32;
 std::mutex lent_mutex;
-LentWorkspace lent_workspace;
+LentWorkspace lent_workspaces[kMaxLoans];
 
-// The lent workspace if it is on the current device (memory null otherwise).
-LentWorkspace lent_here() {
-    LentWorkspace lent;
-    {
-        std::lock_guard<std::mutex> guard(lent_mutex);
-        lent = lent_workspace;
-    }
+// The workspace lent for `stream` on the current device (memory null if none).
+LentWorkspace lent_here(void* stream) {
     int device = -1;
-    if (lent.memory != nullptr && (hipGetDevice(&device) != hipSuccess || device != lent.device)) {
-        lent = LentWorkspace{};
+    if (hipGetDevice(&device) != hipSuccess) return LentWorkspace{};
+    std::lock_guard<std::mutex> guard(lent_mutex);
+    for (const LentWorkspace& loan : lent_workspaces) {
+        if (loan.memory != nullptr && loan.device == device && loan.stream == stream) return loan;
     }
-    return lent;
+    return LentWorkspace{};
 }
 
 // ... if it is also large enough for the one-token split form of this geometry.
-float* lent_partials(std::int64_t query_heads, std::int64_t head_dim) {
-    const LentWorkspace lent = lent_here();
+float* lent_partials(void* stream, std::int64_t query_heads, std::int64_t head_dim) {
+    const LentWorkspace lent = lent_here(stream);
     if (lent.memory == nullptr) return nullptr;
     const std::int64_t required = gqa_decode_split_workspace_bytes(query_heads, head_dim);
     return lent.nbytes >= required ? lent.memory : nullptr;
@@ -173,7 +174,7 @@ int run_fused_decode(const NfnNativeTileGlimmerFusedDecodeAttentionDescriptorV1*
         return kInvalid;
     }
     const hipStream_t stream = as_stream(d->cuda_stream);
-    if (split_partials == nullptr) split_partials = lent_partials(d->query_heads, d->head_dim);
+    if (split_partials == nullptr) split_partials = lent_partials(d->cuda_stream, d->query_heads, d->head_dim);
     // The new cache row is written by the first launch, before the attention
     // runs: right as long as the attention does not read that ring row, which
     // holds for every key range shorter than the ring (and for the device
@@ -371,7 +372,7 @@ int nfn_mi355_fused_decode_attention_split_device_position_v1(
 int nfn_native_tile_glimmer_gqa_decode_float32_v1(
     const NfnNativeTileGlimmerGqaDecodeDescriptorV1* d) {
     if (!gqa_descriptor_valid(d)) return kInvalid;
-    if (float* partials = lent_partials(d->query_heads, d->head_dim)) {
+    if (float* partials = lent_partials(d->cuda_stream, d->query_heads, d->head_dim)) {
         launch_gqa_decode_split(*d, partials, as_stream(d->cuda_stream));
     } else {
         launch_gqa_decode(*d, as_stream(d->cuda_stream));
@@ -379,17 +380,32 @@ int nfn_native_tile_glimmer_gqa_decode_float32_v1(
     return launch_status();
 }
 
-int nfn_mi355_attention_workspace_v1(void* workspace, std::int64_t workspace_nbytes) {
+int nfn_mi355_attention_workspace_v1(void* workspace, std::int64_t workspace_nbytes,
+                                     void* cuda_stream) {
     if ((workspace == nullptr) != (workspace_nbytes == 0) || workspace_nbytes < 0 ||
         reinterpret_cast<std::uintptr_t>(workspace) % 16 != 0) {
         return kInvalid;
     }
     int device = -1;
-    if (workspace != nullptr && hipGetDevice(&device) != hipSuccess) return kInvalid;
+    if (hipGetDevice(&device) != hipSuccess) return kInvalid;
     std::lock_guard<std::mutex> guard(lent_mutex);
-    lent_workspace.device = device;
-    lent_workspace.memory = static_cast<float*>(workspace);
-    lent_workspace.nbytes = workspace_nbytes;
+    LentWorkspace* slot = nullptr;
+    for (LentWorkspace& loan : lent_workspaces) {
+        if (loan.memory != nullptr && loan.device == device && loan.stream == cuda_stream) {
+            slot = &loan;
+            break;
+        }
+        if (loan.memory == nullptr && slot == nullptr) slot = &loan;
+    }
+    if (workspace == nullptr) {  // taking back what was never lent is not an error
+        if (slot != nullptr && slot->memory != nullptr) *slot = LentWorkspace{};
+        return 0;
+    }
+    if (slot == nullptr) return kInvalid;  // every slot holds another stream's loan
+    slot->device = device;
+    slot->stream = cuda_stream;
+    slot->memory = static_cast<float*>(workspace);
+    slot->nbytes = workspace_nbytes;
     return 0;
 }
 
@@ -439,7 +455,7 @@ int nfn_native_tile_glimmer_cache_commit_rows_bf16_v1(
 int nfn_native_tile_dflash_block_attention_float32_v1(
     const NfnNativeTileDFlashBlockAttentionDescriptorV1* d) {
     if (!block_descriptor_valid(d)) return kInvalid;
-    const LentWorkspace lent = lent_here();
+    const LentWorkspace lent = lent_here(d->cuda_stream);
     launch_block_attention(*d, lent.memory, lent.nbytes, as_stream(d->cuda_stream));
     return launch_status();
 }

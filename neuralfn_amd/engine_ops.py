@@ -142,13 +142,15 @@ def fused_decode_attention(query, key, value, key_cache, value_cache, position: 
     return out
 
 
-def lend_attention_workspace(workspace=None) -> None:
-    """Lends the reference-named one-token attention calls a split-form workspace
-    (gqa_decode_workspace), or takes it back with None.  The tensor must outlive the loan."""
+def lend_attention_workspace(workspace=None, stream=None) -> None:
+    """Lends the reference-named attention calls issued on `stream` (a raw handle; default: torch's
+    current stream) a split-form workspace (gqa_decode_workspace), or takes that stream's loan
+    back with None.  The tensor must outlive the loan."""
+    handle = _stream() if stream is None else stream
     if workspace is None:
-        check(load().nfn_mi355_attention_workspace_v1(None, 0), "attention_workspace")
+        check(load().nfn_mi355_attention_workspace_v1(None, 0, handle), "attention_workspace")
     else:
-        check(load().nfn_mi355_attention_workspace_v1(workspace.data_ptr(), workspace.numel()),
+        check(load().nfn_mi355_attention_workspace_v1(workspace.data_ptr(), workspace.numel(), handle),
               "attention_workspace")
 
 

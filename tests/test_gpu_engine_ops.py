@@ -723,10 +723,45 @@ def test_lent_workspace_turns_the_reference_named_calls_into_their_split_forms(c
     small = torch_().empty(1024, dtype=torch_().uint8, device=cuda)
     assert_bits_equal(run(small, None)[0], plain[0], "a workspace too small is not used")
     lib = tile_ops.load()
-    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr() + 4, 1 << 20) == 1
-    assert lib.nfn_mi355_attention_workspace_v1(None, 16) == 1
-    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 0) == 1
-    assert lib.nfn_mi355_attention_workspace_v1(None, 0) == 0
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr() + 4, 1 << 20, None) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(None, 16, None) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 0, None) == 1
+    assert lib.nfn_mi355_attention_workspace_v1(None, 0, None) == 0
+    # a loan serves the stream it was made for and no other: a call on a second stream keeps
+    # the ordinary form (and its bits) while the first stream's loan stands
+    torch = torch_()
+    side = torch.cuda.Stream(device=cuda)
+    engine_ops.lend_attention_workspace(workspace)           # for the current (default) stream
+    try:
+        tensors = (to_device(query, cuda), to_device(key, cuda), to_device(value, cuda),
+                   bf16_tensor(keys, cuda), bf16_tensor(values, cuda))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            elsewhere = engine_ops.gqa_decode(*tensors, position, first, scale)
+        side.synchronize()
+        assert_bits_equal(elsewhere, plain[0], "another stream does not see the loan")
+        here = engine_ops.gqa_decode(*tensors, position, first, scale)
+        assert_bits_equal(here, split[0], "the loan's stream does")
+        # the side stream can hold a loan of its own; taking it back leaves the first in place
+        own = engine_ops.gqa_decode_workspace(query_heads, head_dim)
+        engine_ops.lend_attention_workspace(own, side.cuda_stream)
+        with torch.cuda.stream(side):
+            elsewhere = engine_ops.gqa_decode(*tensors, position, first, scale)
+        side.synchronize()
+        assert_bits_equal(elsewhere, split[0], "the side stream's own loan")
+        engine_ops.lend_attention_workspace(None, side.cuda_stream)
+        assert_bits_equal(engine_ops.gqa_decode(*tensors, position, first, scale), split[0])
+    finally:
+        engine_ops.lend_attention_workspace(None, side.cuda_stream)
+        engine_ops.lend_attention_workspace(None)
+    # the table is bounded: a 33rd stream's loan is refused, the 32 others stand until taken back
+    for handle in range(1, 33):
+        assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 1 << 20, handle << 8) == 0
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 1 << 20, 33 << 8) == 1
+    for handle in range(1, 33):
+        assert lib.nfn_mi355_attention_workspace_v1(None, 0, handle << 8) == 0
+    assert lib.nfn_mi355_attention_workspace_v1(workspace.data_ptr(), 1 << 20, 33 << 8) == 0
+    assert lib.nfn_mi355_attention_workspace_v1(None, 0, 33 << 8) == 0
 
 
 def test_cache_commit_layers_and_pack_target_taps(cuda, oracle):
