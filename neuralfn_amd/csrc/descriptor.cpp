@@ -30,6 +30,8 @@ bool normalize_descriptor(const Descriptor* source, Descriptor* output) {
         source->row_stride_bytes <= 0) {
         return false;
     }
+    // device addresses have 48 bits (the decode kernels pass four of them in six dwords)
+    if ((reinterpret_cast<std::uintptr_t>(source->data) >> 48) != 0) return false;
     const std::int64_t elements = block_elements(source->encoding);
     const std::int64_t bytes = block_bytes(source->encoding);
     if (elements == 0 || source->input_dim % elements != 0) {

@@ -8,10 +8,20 @@
 // consecutive units read consecutive 16-byte slots; the first weight loads of
 // every wave are already in flight while it does so.  Per unit a lane then
 // spends 24 logic operations on unpacking and 32 dot4 on the two planes, and
-// folds the 6-bit sub-scales in with 24-bit integer multiplies; one float
-// conversion per unit, one butterfly per row.  No LDS round trip for weights,
-// no synchronisation after the single barrier, small register footprint: the
-// latency of HBM is hidden by many resident waves.
+// folds the 6-bit sub-scales in with integer multiply-adds; two float
+// conversions per unit, one butterfly per row.  No LDS round trip for weights,
+// no synchronisation after the single barrier.
+//
+// What the launch is bound by at the sizes of one decode layer (16 MB) is the
+// number of instructions a wave issues between its start and its last row, so:
+// the arguments the first loads need (activation pointer, the four weight
+// pointers as 48-bit addresses, the row split) are the kernel's first 14
+// dwords, which arrive in registers at wave start, and everything else sits in
+// a struct the kernel reads while those loads are in flight; a lane's byte
+// offsets inside a row are computed once and the loads take the row address
+// from scalar registers; and with one token and rows of at most two 64-unit
+// slices (up to 8,192 columns) a lane's activation operands stay in registers
+// for all rows of the launch instead of being read from LDS for every unit.
 //
 // Every row gets the same arithmetic whatever the number of tokens in the
 // launch (T token planes are walked one after another against the same
@@ -89,11 +99,206 @@ struct Stage {
     uint4 h0, h1;  // Q5_K: the block's 32 high-bit bytes
 };
 
-template <std::uint32_t ENC, int T, int P>
+// The activation operands of one unit for one token: the two int8 planes of
+// both sub-blocks (two 16-value halves each), the sub-blocks' code sums and the
+// block's scale.
+struct UnitActivations {
+    v4i a_hi[2], a_lo[2], b_hi[2], b_lo[2];
+    int2 sums;
+    float scale;
+};
+
+__device__ __forceinline__ UnitActivations load_unit_activations(const std::uint8_t* lds, int token,
+                                                                 int unit, int blocks) {
+    const TokenImage image = token_image(const_cast<std::uint8_t*>(lds), token, blocks);
+    const int units = 4 * blocks;
+    const std::uint8_t* slot = image.planes + unit * 16;
+    const int stride = units * 16;
+    UnitActivations acts;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        acts.a_hi[half] = *reinterpret_cast<const v4i*>(slot + (0 + half) * stride);
+        acts.a_lo[half] = *reinterpret_cast<const v4i*>(slot + (2 + half) * stride);
+        acts.b_hi[half] = *reinterpret_cast<const v4i*>(slot + (4 + half) * stride);
+        acts.b_lo[half] = *reinterpret_cast<const v4i*>(slot + (6 + half) * stride);
+    }
+    acts.sums = *reinterpret_cast<const int2*>(image.sums + (unit >> 2) * 8 + 2 * (unit & 3));
+    acts.scale = image.scale[unit >> 2];
+    return acts;
+}
+
+// The weights of one unit, unpacked once for all tokens.
+struct UnitWeights {
+    std::uint32_t low[8], high[8];  // 4-bit (Q5_K: 5-bit) codes of the two sub-blocks, a byte each
+    int scale_a, scale_b, min_a, min_b;  // 6-bit sub-block scales and minimums
+    float d, dmin;
+};
+
+template <bool Q5>
+__device__ __forceinline__ UnitWeights unpack_unit(const Stage<Q5>& stage, int pair) {
+    UnitWeights weights;
+    // the low nibbles are sub-block 2*pair, the high nibbles 2*pair+1
+    const std::uint32_t packed[8] = {stage.q0.x, stage.q0.y, stage.q0.z, stage.q0.w,
+                                     stage.q1.x, stage.q1.y, stage.q1.z, stage.q1.w};
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+        weights.low[w] = packed[w] & 0x0f0f0f0fu;
+        weights.high[w] = (packed[w] >> 4) & 0x0f0f0f0fu;
+    }
+    if constexpr (Q5) {
+        const std::uint32_t bits[8] = {stage.h0.x, stage.h0.y, stage.h0.z, stage.h0.w,
+                                       stage.h1.x, stage.h1.y, stage.h1.z, stage.h1.w};
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            // bit 2*pair of the high-bit byte belongs to the first sub-block, 2*pair+1 to the second
+            const std::uint32_t shifted = bits[w] >> (2 * pair);
+            weights.low[w] |= (shifted & 0x01010101u) << 4;
+            weights.high[w] |= (shifted & 0x02020202u) << 3;
+        }
+    }
+    // the pair's two 6-bit scales and minimums, packed [second:first] in 16 bits
+    const int shift = 16 * (pair & 1);
+    const std::uint32_t y = stage.header.y >> shift;
+    const std::uint32_t z = stage.header.z >> shift;
+    const std::uint32_t w = stage.header.w >> shift;
+    const bool upper = pair >= 2;
+    const std::uint32_t scales = upper ? ((w & 0x0f0fu) | ((y >> 2) & 0x3030u)) : (y & 0x3f3fu);
+    const std::uint32_t minimums =
+        upper ? (((w >> 4) & 0x0f0fu) | ((z >> 2) & 0x3030u)) : (z & 0x3f3fu);
+    weights.scale_a = static_cast<int>(scales & 0xffu);
+    weights.scale_b = static_cast<int>(scales >> 8);
+    weights.min_a = static_cast<int>(minimums & 0xffu);
+    weights.min_b = static_cast<int>(minimums >> 8);
+    weights.d = half_bits_to_float(stage.header.x & 0xffffu);
+    weights.dmin = half_bits_to_float(stage.header.x >> 16);
+    return weights;
+}
+
+// acc += scale * (d * sum_sub sc * dot(q, codes) - dmin * sum_sub m * sum(codes)) for one
+// unit and one token.  `live` is false for the lanes past the end of a row's last slice.
+__device__ __forceinline__ float unit_product(const UnitWeights& weights, const UnitActivations& acts,
+                                              bool live, float acc) {
+    int dot_a_hi = 0, dot_a_lo = 0, dot_b_hi = 0, dot_b_lo = 0;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int lo_codes = static_cast<int>(weights.low[half * 4 + v]);
+            const int hi_codes = static_cast<int>(weights.high[half * 4 + v]);
+            dot_a_hi = __builtin_amdgcn_sdot4(lo_codes, acts.a_hi[half][v], dot_a_hi, false);
+            dot_a_lo = __builtin_amdgcn_sdot4(lo_codes, acts.a_lo[half][v], dot_a_lo, false);
+            dot_b_hi = __builtin_amdgcn_sdot4(hi_codes, acts.b_hi[half][v], dot_b_hi, false);
+            dot_b_lo = __builtin_amdgcn_sdot4(hi_codes, acts.b_lo[half][v], dot_b_lo, false);
+        }
+    }
+    // Integer up to the last step: every sub-block scale times its dot product and the
+    // sums of two of them stay below 2^24 (31 * 32 * 127 * 63 * 2), so the two
+    // conversions are exact and the float code sum is rounded once.
+    const int weighted_hi = weights.scale_a * dot_a_hi + weights.scale_b * dot_b_hi;
+    const int weighted_lo = weights.scale_a * dot_a_lo + weights.scale_b * dot_b_lo;
+    const int weighted_min = weights.min_a * acts.sums.x + weights.min_b * acts.sums.y;
+    const float codes = fmaf(static_cast<float>(weighted_hi), 256.0f, static_cast<float>(weighted_lo));
+    const float value = fmaf(-weights.dmin, static_cast<float>(weighted_min), weights.d * codes);
+    return fmaf(live ? acts.scale : 0.0f, value, acc);
+}
+
+// One unit (a 64-value pair of sub-blocks of one block) against the token planes in LDS.
+template <bool Q5, int T>
+__device__ __forceinline__ void accumulate_unit(const Stage<Q5>& stage, const std::uint8_t* lds,
+                                                int unit, bool live, int blocks, float (&acc)[T]) {
+    const UnitWeights weights = unpack_unit<Q5>(stage, unit & 3);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        acc[t] = unit_product(weights, load_unit_activations(lds, t, unit, blocks), live, acc[t]);
+    }
+}
+
+typedef const __attribute__((address_space(1))) std::uint8_t* GlobalBytes;
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(1))) v4u* GlobalVec;
+
+// Arguments the kernel needs late (row ends, prologues): read from the argument
+// block while the first loads are in flight.
+struct DotTail {
+    const float* second;
+    std::uint8_t* records_out;
+    int tokens;
+    int pad;
+    float* output[4];
+    std::int64_t output_dim[4];
+};
+
+
+// Four 48-bit device addresses in three 64-bit words.
+struct PackedPointers {
+    std::uint64_t a, b, c;
+};
+constexpr std::uint64_t kAddressMask = (std::uint64_t(1) << 48) - 1;
+inline PackedPointers pack_pointers(const void* const p[4]) {
+    std::uint64_t v[4];
+    for (int i = 0; i < 4; ++i) v[i] = reinterpret_cast<std::uint64_t>(p[i]) & kAddressMask;
+    PackedPointers packed;
+    packed.a = v[0] | (v[1] << 48);
+    packed.b = (v[1] >> 16) | (v[2] << 32);
+    packed.c = (v[2] >> 32) | (v[3] << 16);
+    return packed;
+}
+__device__ __forceinline__ GlobalBytes unpack_pointer(std::uint64_t a, std::uint64_t b,
+                                                      std::uint64_t c, int index) {
+    const std::uint64_t p0 = a & kAddressMask;
+    const std::uint64_t p1 = (a >> 48) | ((b & 0xffffffffull) << 16);
+    const std::uint64_t p2 = (b >> 32) | ((c & 0xffffull) << 32);
+    const std::uint64_t p3 = c >> 16;
+    std::uint64_t p = p0;
+    p = index == 1 ? p1 : p;
+    p = index == 2 ? p2 : p;
+    p = index == 3 ? p3 : p;
+    return reinterpret_cast<GlobalBytes>(p);
+}
+
+// Walks the (row, 64-unit slice) pairs of one wave; everything is uniform.
+struct DotCursor {
+    int op, row, first_row, next_bound, iteration;
+    GlobalBytes row_ptr;
+
+    __device__ __forceinline__ void bounds(int b1, int b2, int b3) {
+        first_row = op == 0 ? 0 : op == 1 ? b1 : op == 2 ? b2 : b3;
+        next_bound = op == 0 ? b1 : op == 1 ? b2 : op == 2 ? b3 : 0x7fffffff;
+    }
+    __device__ __forceinline__ void start(int global_row, std::int64_t stride, std::uint64_t a,
+                                          std::uint64_t b, std::uint64_t c, int b1, int b2, int b3) {
+        op = (global_row >= b1 ? 1 : 0) + (global_row >= b2 ? 1 : 0) + (global_row >= b3 ? 1 : 0);
+        row = global_row;
+        iteration = 0;
+        bounds(b1, b2, b3);
+        row_ptr = unpack_pointer(a, b, c, op) + (row - first_row) * stride;
+    }
+    __device__ __forceinline__ void advance(int iterations, std::int64_t stride, std::uint64_t a,
+                                            std::uint64_t b, std::uint64_t c, int b1, int b2, int b3) {
+        if (++iteration < iterations) return;
+        iteration = 0;
+        ++row;
+        row_ptr += stride;
+        if (row == next_bound) {
+            ++op;
+            bounds(b1, b2, b3);
+            row_ptr = unpack_pointer(a, b, c, op);
+        }
+    }
+};
+
+// The leading arguments (14 dwords) arrive in registers at wave start: the first
+// activation and weight loads depend on nothing else.  Rows of projection k are
+// [bound_k, bound_k+1) of the launch (bound_0 = 0; unused bounds are INT_MAX).
+// ITER > 0 (one token only): a row has exactly ITER 64-unit slices, and since a
+// lane's units are then the same in every row, their activation operands stay in
+// registers for the whole launch instead of being read from LDS per row.
+template <std::uint32_t ENC, int T, int P, int ITER>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
-    const float* __restrict__ first, const float* __restrict__ second, int tokens, int input_dim,
-    int total_rows, int rows_per_group, int longer_groups, std::uint8_t* __restrict__ records_out,
-    ProjectionSet set) {
+    const float* __restrict__ first, std::uint64_t data_a, std::uint64_t data_b,
+    std::uint64_t data_c, int input_dim, int rows_per_group, int longer_groups, int bound1,
+    int bound2, int bound3, DotTail tail) {
+    static_assert(ITER == 0 || (T == 1 && ITER <= 2), "register-resident activations: one token, two slices");
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
     constexpr int kQuants = kQ5 ? 48 : 16;
@@ -103,12 +308,13 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int blocks = input_dim >> 8;
     const int units = 4 * blocks;
-    const int iterations = (units + kWave - 1) / kWave;
+    const int iterations = ITER > 0 ? ITER : (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
-    const int pass_tokens = min(tokens - token0, T);
+    const int pass_tokens = T == 1 ? 1 : min(tail.tokens - token0, T);
     const float* pass_first = pass_input<P>(first, token0, input_dim);
     const float* pass_second = P == kGated || P == kSwiGlu
-        ? second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
+        ? tail.second + static_cast<std::int64_t>(token0) * input_dim : nullptr;
+    const std::int64_t stride = static_cast<std::int64_t>(blocks) * kBlockBytes;
 
     // rows of this wave: dealt out evenly over the workgroups, then over the waves
     const WaveRows mine =
@@ -132,30 +338,60 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
                                        static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
     }
 
-    // (2) weight loads of the first two (row, iteration) pairs
-    PairCursor fetch;
-    fetch.start(set, min(row_begin, total_rows - 1));
-    int fetch_left = total;  // pairs not fetched yet; the cursor rests on the last one
-    auto issue = [&](Stage<kQ5>& stage) {
-        const int unit = min(fetch.iteration * kWave + lane, units - 1);
-        const std::uint8_t* block = fetch.row + (unit >> 2) * kBlockBytes;
-        stage.header = *reinterpret_cast<const uint4*>(block);
-        const std::uint8_t* quants = block + kQuants + (unit & 3) * 32;
-        stage.q0 = *reinterpret_cast<const uint4*>(quants);
-        stage.q1 = *reinterpret_cast<const uint4*>(quants + 16);
-        if constexpr (kQ5) {
-            stage.h0 = *reinterpret_cast<const uint4*>(block + 16);
-            stage.h1 = *reinterpret_cast<const uint4*>(block + 32);
+    // (2) weight loads of the first two (row, slice) pairs.  A stage beyond the wave's
+    // last pair loads one fixed address in every lane (one cache line per instruction),
+    // so the number of loads in flight is the same on every path.
+    DotCursor fetch;
+    fetch.start(row_count > 0 ? row_begin : 0, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+    int fetch_left = total;  // pairs not fetched yet
+    // A lane's byte offsets inside a row depend on the slice only (and a slice of a
+    // two-slice row always lands in the same stage): computed once, added to the
+    // uniform row address by the load instruction itself.
+    auto unit_offset = [&](int slice) {
+        const int unit = min(slice * kWave + lane, units - 1);
+        return (unit >> 2) * kBlockBytes;
+    };
+    auto quant_offset = [&](int slice) {
+        const int unit = min(slice * kWave + lane, units - 1);
+        return (unit >> 2) * kBlockBytes + kQuants + (unit & 3) * 32;
+    };
+    const int block_offsets[2] = {unit_offset(0), unit_offset(1)};
+    const int quant_offsets[2] = {quant_offset(0), quant_offset(1)};
+    auto issue = [&](Stage<kQ5>& stage, int slice) {
+        const bool real = fetch_left > 0;
+        std::uint32_t block_offset, quants_offset;
+        if constexpr (ITER > 0) {
+            block_offset = real ? block_offsets[slice] : 0;
+            quants_offset = real ? quant_offsets[slice] : 0;
+        } else {
+            const int unit = real ? min(fetch.iteration * kWave + lane, units - 1) : 0;
+            block_offset = (unit >> 2) * kBlockBytes;
+            quants_offset = block_offset + kQuants + (unit & 3) * 32;
         }
-        if (--fetch_left > 0) fetch.advance(set, iterations);
+        GlobalBytes block = fetch.row_ptr + block_offset;
+        const v4u header = *reinterpret_cast<GlobalVec>(block);
+        GlobalBytes quants = fetch.row_ptr + quants_offset;
+        const v4u q0 = *reinterpret_cast<GlobalVec>(quants);
+        const v4u q1 = *reinterpret_cast<GlobalVec>(quants + 16);
+        stage.header = make_uint4(header.x, header.y, header.z, header.w);
+        stage.q0 = make_uint4(q0.x, q0.y, q0.z, q0.w);
+        stage.q1 = make_uint4(q1.x, q1.y, q1.z, q1.w);
+        if constexpr (kQ5) {
+            const v4u h0 = *reinterpret_cast<GlobalVec>(block + 16);
+            const v4u h1 = *reinterpret_cast<GlobalVec>(block + 32);
+            stage.h0 = make_uint4(h0.x, h0.y, h0.z, h0.w);
+            stage.h1 = make_uint4(h1.x, h1.y, h1.z, h1.w);
+        }
+        if (--fetch_left > 0) fetch.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     };
     Stage<kQ5> stage0, stage1;
-    issue(stage0);
-    issue(stage1);
+    issue(stage0, 0);
+    issue(stage1, ITER == 2 ? 1 : 0);
 
     // (3) quantize; one barrier; after it the workgroup never synchronises again.
     // The first workgroup also leaves the records in the caller's workspace
     // for a later launch that shares this input.
+    std::uint8_t* const records_out = tail.records_out;
     const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
     auto quantize_record = [&](float4 loaded, int record) {
         const int token = token_of_record<T>(record, blocks);
@@ -182,97 +418,42 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     }
     __syncthreads();
 
+    UnitActivations held[ITER > 0 ? ITER : 1];
+    if constexpr (ITER > 0) {
+#pragma unroll
+        for (int slice = 0; slice < ITER; ++slice) {
+            held[slice] = load_unit_activations(lds, 0, min(slice * kWave + lane, units - 1), blocks);
+        }
+    }
+
     float acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = 0.0f;
 
-    PairCursor work;
-    work.start(set, min(row_begin, total_rows - 1));
-    auto compute = [&](const Stage<kQ5>& stage) {
+    DotCursor work;
+    work.start(row_count > 0 ? row_begin : 0, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+    // `slice`: for ITER > 0 the slice this stage always holds (stage s of a row of
+    // two slices holds slice s; rows of one slice use both stages for slice 0)
+    auto compute = [&](const Stage<kQ5>& stage, int slice) {
         const int iteration = work.iteration;
         const int raw_unit = iteration * kWave + lane;
         const bool live = raw_unit < units;
         const int unit = min(raw_unit, units - 1);
-        const int block = unit >> 2;
-        const int pair = unit & 3;
-
-        // unpack: the low nibbles are sub-block 2*pair, the high nibbles 2*pair+1
-        const std::uint32_t packed[8] = {stage.q0.x, stage.q0.y, stage.q0.z, stage.q0.w,
-                                         stage.q1.x, stage.q1.y, stage.q1.z, stage.q1.w};
-        std::uint32_t low[8], high[8];
-#pragma unroll
-        for (int w = 0; w < 8; ++w) {
-            low[w] = packed[w] & 0x0f0f0f0fu;
-            high[w] = (packed[w] >> 4) & 0x0f0f0f0fu;
+        if constexpr (ITER > 0) {
+            acc[0] = unit_product(unpack_unit<kQ5>(stage, lane & 3), held[slice], live, acc[0]);
+        } else {
+            accumulate_unit<kQ5, T>(stage, lds, unit, live, blocks, acc);
         }
-        if constexpr (kQ5) {
-            const std::uint32_t bits[8] = {stage.h0.x, stage.h0.y, stage.h0.z, stage.h0.w,
-                                           stage.h1.x, stage.h1.y, stage.h1.z, stage.h1.w};
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                // bit 2*pair of the high-bit byte belongs to the first sub-block, 2*pair+1 to the second
-                const std::uint32_t shifted = bits[w] >> (2 * pair);
-                low[w] |= (shifted & 0x01010101u) << 4;
-                high[w] |= (shifted & 0x02020202u) << 3;
-            }
-        }
-        // the pair's two 6-bit scales and minimums, packed [second:first] in 16 bits
-        const int shift = 16 * (pair & 1);
-        const std::uint32_t y = stage.header.y >> shift;
-        const std::uint32_t z = stage.header.z >> shift;
-        const std::uint32_t w = stage.header.w >> shift;
-        const bool upper = pair >= 2;
-        const std::uint32_t scales = upper ? ((w & 0x0f0fu) | ((y >> 2) & 0x3030u)) : (y & 0x3f3fu);
-        const std::uint32_t minimums =
-            upper ? (((w >> 4) & 0x0f0fu) | ((z >> 2) & 0x3030u)) : (z & 0x3f3fu);
-        // as floats: every product and sum below stays under 2^24, so the
-        // float arithmetic on the integer dot products is exact
-        const float scale_a = static_cast<float>(scales & 0xffu);
-        const float scale_b = static_cast<float>((scales >> 8) & 0xffu);
-        const float min_a = static_cast<float>(minimums & 0xffu);
-        const float min_b = static_cast<float>((minimums >> 8) & 0xffu);
-        const float d = half_bits_to_float(stage.header.x & 0xffffu);
-        const float dmin = half_bits_to_float(stage.header.x >> 16);
-
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const TokenImage image = token_image(lds, t, blocks);
-            const std::uint8_t* slot = image.planes + unit * 16;
-            const int stride = units * 16;
-            int dot_a_hi = 0, dot_a_lo = 0, dot_b_hi = 0, dot_b_lo = 0;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const v4i a_hi = *reinterpret_cast<const v4i*>(slot + (0 + half) * stride);
-                const v4i a_lo = *reinterpret_cast<const v4i*>(slot + (2 + half) * stride);
-                const v4i b_hi = *reinterpret_cast<const v4i*>(slot + (4 + half) * stride);
-                const v4i b_lo = *reinterpret_cast<const v4i*>(slot + (6 + half) * stride);
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int lo_codes = static_cast<int>(low[half * 4 + v]);
-                    const int hi_codes = static_cast<int>(high[half * 4 + v]);
-                    dot_a_hi = __builtin_amdgcn_sdot4(lo_codes, a_hi[v], dot_a_hi, false);
-                    dot_a_lo = __builtin_amdgcn_sdot4(lo_codes, a_lo[v], dot_a_lo, false);
-                    dot_b_hi = __builtin_amdgcn_sdot4(hi_codes, b_hi[v], dot_b_hi, false);
-                    dot_b_lo = __builtin_amdgcn_sdot4(hi_codes, b_lo[v], dot_b_lo, false);
-                }
-            }
-            const int2 sums = *reinterpret_cast<const int2*>(image.sums + block * 8 + 2 * pair);
-            const float scale = image.scale[block];
-            const float weighted_hi = fmaf(scale_b, static_cast<float>(dot_b_hi),
-                                           scale_a * static_cast<float>(dot_a_hi));
-            const float weighted_lo = fmaf(scale_b, static_cast<float>(dot_b_lo),
-                                           scale_a * static_cast<float>(dot_a_lo));
-            const float weighted_min = fmaf(min_b, static_cast<float>(sums.y),
-                                            min_a * static_cast<float>(sums.x));
-            const float codes = fmaf(weighted_hi, 256.0f, weighted_lo);
-            const float value = fmaf(-dmin, weighted_min, d * codes);
-            acc[t] = fmaf(live ? scale : 0.0f, value, acc[t]);
-        }
-
         if (iteration == iterations - 1) {
             // the row is complete: fixed-order butterfly, lane 0 writes
-            float* output = work.current.output + work.local_row;
-            const std::int64_t output_dim = work.current.output_dim;
+            float* base = tail.output[0];
+            std::int64_t output_dim = tail.output_dim[0];
+#pragma unroll
+            for (int k = 1; k < 4; ++k) {
+                base = work.op == k ? tail.output[k] : base;
+                output_dim = work.op == k ? tail.output_dim[k] : output_dim;
+            }
+            float* output = base + (work.row - work.first_row);
 #pragma unroll
             for (int t = 0; t < T; ++t) {
                 const float total_value = wave_total(acc[t]);
@@ -282,14 +463,14 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
                 acc[t] = 0.0f;
             }
         }
-        work.advance(set, iterations);
+        work.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     };
 
     for (int n = 0; n < total; n += 2) {
-        compute(stage0);
-        issue(stage0);
-        if (n + 1 < total) compute(stage1);
-        issue(stage1);
+        compute(stage0, 0);
+        issue(stage0, 0);
+        if (n + 1 < total) compute(stage1, ITER == 2 ? 1 : 0);
+        issue(stage1, ITER == 2 ? 1 : 0);
     }
 }
 
@@ -297,20 +478,45 @@ template <std::uint32_t ENC, int T, int P>
 void launch_variant(ProjectionSet set, const float* first, const float* second,
                     std::uint8_t* records_out, int tokens, hipStream_t stream) {
     std::int64_t rows = 0;
+    int bounds[4] = {0, 0x7fffffff, 0x7fffffff, 0x7fffffff};
+    const void* data[4] = {set.op[0].data, set.op[0].data, set.op[0].data, set.op[0].data};
+    DotTail tail{};
+    tail.second = second;
+    tail.records_out = records_out;
+    tail.tokens = tokens;
     for (int index = 0; index < set.count; ++index) {
-        set.op[index].first_tile = static_cast<std::uint32_t>(rows);  // first row here
+        bounds[index] = static_cast<int>(rows);
+        data[index] = set.op[index].data;
+        tail.output[index] = set.op[index].output;
+        tail.output_dim[index] = set.op[index].output_dim;
         rows += set.op[index].output_dim;
     }
+    const PackedPointers packed = pack_pointers(data);
     const std::int64_t blocks = set.input_dim >> 8;
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes_host(blocks);
-    auto kernel = gemv_dot_kernel<ENC, T, P>;
-    allow_large_lds<gemv_dot_kernel<ENC, T, P>>();
     const int passes = (tokens + T - 1) / T;
     const std::int64_t groups = decode_groups(rows, kDotWaves);
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
-                       stream, first, second, tokens, static_cast<int>(set.input_dim),
-                       static_cast<int>(rows), static_cast<int>(rows / groups),
-                       static_cast<int>(rows % groups), records_out, set);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), passes), dim3(kDotThreads), lds,
+                           stream, first, packed.a, packed.b, packed.c,
+                           static_cast<int>(set.input_dim), static_cast<int>(rows / groups),
+                           static_cast<int>(rows % groups), bounds[1], bounds[2], bounds[3], tail);
+    };
+    const std::int64_t slices = (4 * blocks + kWave - 1) / kWave;
+    if constexpr (T == 1) {
+        if (slices == 1) {
+            allow_large_lds<gemv_dot_kernel<ENC, T, P, 1>>();
+            launch(gemv_dot_kernel<ENC, T, P, 1>);
+            return;
+        }
+        if (slices == 2) {
+            allow_large_lds<gemv_dot_kernel<ENC, T, P, 2>>();
+            launch(gemv_dot_kernel<ENC, T, P, 2>);
+            return;
+        }
+    }
+    allow_large_lds<gemv_dot_kernel<ENC, T, P, 0>>();
+    launch(gemv_dot_kernel<ENC, T, P, 0>);
 }
 
 template <std::uint32_t ENC, int P>
