@@ -246,6 +246,201 @@ def cpu_baseline(host_layers, rows: int, budget_seconds: float = 20.0) -> dict:
     }
 
 
+def launch_floor_extra(layers, device, stream, steps: int, warmup: int) -> dict:
+    """What the headline's launches would cost with no arithmetic at all: the same number of
+    back-to-back launches in a HIP graph, each one workgroup per compute unit that only reads
+    the bytes a decode launch streams (nfn_mi355_read_probe_v1), and the same with an empty
+    kernel.  The ceiling these two put over the headline is a property of 16 MB launches on
+    this chip, not of the kernels."""
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    lib = tile_ops.load()
+    qkv = (kquant.packed_nbytes(kquant.Q4_K, ATTN_DIM, MODEL_DIM)
+           + 2 * kquant.packed_nbytes(kquant.Q4_K, KV_DIM, MODEL_DIM))
+    out = kquant.packed_nbytes(kquant.Q4_K, MODEL_DIM, ATTN_DIM)
+    per_layer = qkv + out
+    pool = torch.randint(0, 256, (len(layers) * per_layer,), dtype=torch.uint8, device=device)
+    sink = torch.zeros(1024, dtype=torch.int32, device=device)
+
+    def enqueue(read: bool):
+        handle = int(torch.cuda.current_stream().cuda_stream)
+        for layer in range(len(layers)):
+            base = pool.data_ptr() + layer * per_layer
+            for offset, nbytes in ((0, qkv), (qkv, out)):
+                tile_ops.check(lib.nfn_mi355_read_probe_v1(
+                    base + offset, nbytes if read else 0, sink.data_ptr(), handle), "read probe")
+
+    launches = 2 * len(layers)
+    read_ms = time_graph(lambda: enqueue(True), stream, steps, warmup)
+    empty_ms = time_graph(lambda: enqueue(False), stream, steps, warmup)
+    bytes_per_launch = per_layer / 2
+    return {
+        "workload": f"{launches} launches a HIP-graph replay, one workgroup of 512 per compute unit: "
+                    "read only the packed bytes of a decode launch / an empty kernel",
+        "read_only_us_per_launch": round(read_ms * 1e3 / launches, 3),
+        "empty_kernel_us_per_launch": round(empty_ms * 1e3 / launches, 3),
+        "read_only_GB/s": round(bytes_per_launch / (read_ms * 1e3 / launches) / 1e3, 1),
+        "read_only_frac_hbm": round(bytes_per_launch / (read_ms * 1e3 / launches) / 1e3 / HBM_PEAK_GBS, 4)}
+
+
+def patterned_packed_on_device(encoding: int, out_dim: int, in_dim: int, device):
+    """The reference benchmark's weights (tools/bench_muse_glimmer_packed_linear.py:161-177):
+    byte i of the tensor is (29 i + 17) mod 256, then every block gets d = 0x2800 and (Q4_K,
+    Q5_K) dmin = 0x2400."""
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    elements, nbytes = kquant.BLOCKS[encoding]
+    total = out_dim * in_dim // elements * nbytes
+    data = ((torch.arange(total, dtype=torch.int64, device=device) * 29 + 17) & 0xFF).to(torch.uint8)
+    blocks = data.view(-1, nbytes)
+    if encoding == kquant.Q6_K:
+        blocks[:, 208], blocks[:, 209] = 0x00, 0x28
+    else:
+        blocks[:, 0], blocks[:, 1], blocks[:, 2], blocks[:, 3] = 0x00, 0x28, 0x00, 0x24
+    return tile_ops.PackedWeight(encoding, out_dim, in_dim, data)
+
+
+# ms on an RTX 5090 as the reference publishes them (docs/glimmer-support-todo.md:730-739, 746-750)
+PUBLISHED_SHAPES = (
+    ("q4_k", 6656, 4096, {1: 0.018, 16: 0.106}),
+    ("q4_k", 6656, 19968, {1: 0.055, 16: 0.376}),
+    ("q6_k", 19968, 6656, {1: 0.083, 16: 0.454}),
+    ("q5_k", 6656, VOCAB, {1: 0.626, 16: 4.198}),
+    ("q4_k", 6656, 256, {1: 0.008, 16: 0.032}),
+    ("q6_k", 6656, 256, {16: 0.038}),
+)
+
+
+def published_shapes_extra(device, stream, steps: int, warmup: int) -> dict:
+    """The reference's own microbenchmark shapes with its patterned bytes and inputs, one and 16
+    rows, through the same entry point (k_quant_mmq_multi_linear), timed the way it times them
+    (back-to-back enqueues of one call, events around them), beside its published RTX 5090 times."""
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    names = {"q4_k": kquant.Q4_K, "q5_k": kquant.Q5_K, "q6_k": kquant.Q6_K}
+    result = {"workload": "patterned bytes (29 i + 17 mod 256, d 0x2800, dmin 0x2400), inputs "
+                          "((37 r + 13 c) mod 257 - 128) / 257; ms per call, 30 back-to-back enqueues"}
+    for name, in_dim, out_dim, published in PUBLISHED_SHAPES:
+        weight = patterned_packed_on_device(names[name], out_dim, in_dim, device)
+        workspace = tile_ops.small_batch_workspace(16, in_dim, device)
+        for rows in (1, 16):
+            if rows not in published:
+                continue
+            r = torch.arange(rows, dtype=torch.int64, device=device)[:, None]
+            c = torch.arange(in_dim, dtype=torch.int64, device=device)[None, :]
+            x = (((r * 37 + c * 13) % 257 - 128).to(torch.float32) / 257.0).contiguous()
+            out = torch.empty((rows, out_dim), dtype=torch.float32, device=device)
+            ms = time_replays(lambda: tile_ops.multi_linear([weight], x, workspace, outputs=[out]),
+                              30, 5)
+            if not bool(torch.isfinite(out).all()):
+                raise RuntimeError(f"{name} {in_dim}->{out_dim}: non-finite output")
+            traffic = weight.nbytes + rows * (in_dim + out_dim) * 4
+            result[f"{name}_{in_dim}_to_{out_dim}_rows{rows}"] = {
+                "ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
+                "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
+                "reference_rtx5090_ms": published[rows]}
+        del weight
+    return result
+
+
+def large_projection_extra(device, stream, steps: int, warmup: int) -> dict:
+    """One-token GEMV of one projection large enough (65,536 rows of 6,656) that the launch's
+    fixed costs vanish: what the decode kernels stream at per format."""
+    import torch
+    from neuralfn_amd import kquant, tile_ops
+    out_dim = 65536
+    x = torch.from_numpy(kquant.synthetic_activations(51, 1, MODEL_DIM)).to(device)
+    workspace = tile_ops.small_batch_workspace(1, MODEL_DIM, device)
+    out = torch.empty((1, out_dim), dtype=torch.float32, device=device)
+    result = {"workload": f"one token, {MODEL_DIM}->{out_dim}, one projection per launch, HIP-graph replay"}
+    for encoding in (kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0):
+        # two tensors visited in turn, together beyond the 256 MB memory-side cache
+        weights = [random_packed_on_device(encoding, out_dim, MODEL_DIM, device, 60 + k) for k in range(2)]
+
+        def run():
+            for weight in weights:
+                tile_ops.multi_linear([weight], x, workspace, outputs=[out])
+
+        ms = time_graph(run, stream, max(5, steps // 2), max(2, warmup // 2)) / len(weights)
+        traffic = weights[0].nbytes + (MODEL_DIM + out_dim) * 4
+        result[kquant.NAMES[encoding]] = {
+            "MB": round(weights[0].nbytes / 1e6, 1), "us": round(ms * 1e3, 2),
+            "GB/s": round(traffic / ms / 1e6, 1),
+            "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        del weights
+    return result
+
+
+def cpu_baselines_other_configs(host_layers) -> dict:
+    """The CPU path on the other configurations: config 0 (one Q4_K GEMV 6656->4096) and config 2
+    (the whole Q6_K lm_head, one row) in full with the reference's own linear() where it is
+    built; config 3 as a stated slice of the reference's batched form (linear_rows,
+    resident_glimmer_assistant.cpp:459-483: one flat loop over rows x outputs, every weight decoded
+    again for every row), restated by the oracle, and extrapolated linearly in the rows."""
+    from neuralfn_amd import kquant
+    from oracle import kquant_oracle
+    use_reference = kquant_oracle.reference_available()
+    kind = "reference" if use_reference else "port"
+
+    def single(encoding, packed, out_dim, in_dim, x):
+        if use_reference:
+            return kquant_oracle.ref_linear(encoding, packed, out_dim, in_dim, x)
+        return kquant_oracle.linear(encoding, packed, out_dim, in_dim, x, as_written=True)
+
+    result = {}
+    # config 0
+    x = kquant.synthetic_activations(11, 1, MODEL_DIM)
+    packed = host_layers[0]["q"]
+    single(kquant.Q4_K, packed, ATTN_DIM, MODEL_DIM, x)
+    calls, began = 0, time.perf_counter()
+    while time.perf_counter() - began < 3.0:
+        single(kquant.Q4_K, packed, ATTN_DIM, MODEL_DIM, x)
+        calls += 1
+    seconds = (time.perf_counter() - began) / calls
+    traffic = packed.size + (MODEL_DIM + ATTN_DIM) * 4
+    result["config0_q4_k_gemv_6656_to_4096"] = {
+        "value": round(traffic / seconds / 1e9, 4), "unit": "GB/s", "ms_per_call": round(seconds * 1e3, 3),
+        "cores": kquant_oracle.worker_count(ATTN_DIM, 128), "kind": kind,
+        "sample": f"{calls} full calls at one row"}
+    # config 2: the byte values do not change what the CPU path costs
+    rng = np.random.default_rng(7)
+    stride = kquant.row_stride_bytes(kquant.Q6_K, MODEL_DIM)
+    lm_head = rng.integers(0, 256, VOCAB * stride, dtype=np.uint8).reshape(-1, 210)
+    lm_head[:, 208], lm_head[:, 209] = 0, 0x14
+    lm_head = lm_head.reshape(-1)
+    x = kquant.synthetic_activations(21, 1, MODEL_DIM, True)
+    began = time.perf_counter()
+    logits = single(kquant.Q6_K, lm_head, VOCAB, MODEL_DIM, x)
+    kquant_oracle.argmax(logits[0])
+    seconds = time.perf_counter() - began
+    result["config2_q6_k_lm_head_argmax_one_row"] = {
+        "value": round((lm_head.size + MODEL_DIM * 4 + 12) / seconds / 1e9, 4), "unit": "GB/s",
+        "ms_per_call": round(seconds * 1e3, 1), "cores": kquant_oracle.worker_count(VOCAB, 128),
+        "kind": kind, "sample": "one full call: 202,048 x 6,656 Q6_K rows and the argmax over the logits"}
+    del lm_head, logits
+    # config 3: 8 rows of the gate projection in the batched form, then times M / 8 and three projections
+    rng = np.random.default_rng(8)
+    stride = kquant.row_stride_bytes(kquant.Q4_K, MODEL_DIM)
+    gate = rng.integers(0, 256, FFN_DIM * stride, dtype=np.uint8).reshape(-1, 144)
+    gate[:, 0], gate[:, 1], gate[:, 2], gate[:, 3] = 0, 0x14, 0, 0x14
+    gate = gate.reshape(-1)
+    slice_rows = 8
+    x = kquant.synthetic_activations(31, slice_rows, MODEL_DIM)
+    began = time.perf_counter()
+    kquant_oracle.linear(kquant.Q4_K, gate, FFN_DIM, MODEL_DIM, x, as_written=True)
+    seconds = time.perf_counter() - began
+    flops = 2.0 * slice_rows * MODEL_DIM * FFN_DIM
+    result["config3_q4_k_ffn_prefill_slice"] = {
+        "value": round(flops / seconds / 1e12, 6), "unit": "TFLOP/s",
+        "cores": kquant_oracle.worker_count(slice_rows * FFN_DIM, 128), "kind": "port",
+        "sample": f"{slice_rows} rows x 6656->16384 in the reference's batched CPU form (every weight "
+                  f"decoded again per row) in {seconds:.2f} s",
+        "extrapolated_seconds_for_one_ffn": {
+            f"M={rows}": round(seconds / slice_rows * rows * 3, 1) for rows in (512, 2048)},
+        "note": "extrapolation: cost is linear in rows and the three projections have the same size"}
+    return result
+
+
 def decode_batch_extra(layers, device, stream, steps: int, warmup: int, headline_rows: int) -> dict:
     """The headline workload at the other batch sizes of the same configuration."""
     import torch
@@ -706,6 +901,8 @@ def main() -> int:
             "unit": "GB/s",
             "frac": round(value / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.rows),
+            "traffic_source": "stored result of a counter run of this workload (FETCH_SIZE + "
+                              "WRITE_SIZE, see profiles/); not measured in this run",
             "kernel": "decode GEMV (Q/K/V grouped launch and O launch, averaged)",
             "bytes_per_launch": bytes_per_step // launches,
             "us_per_launch": round(ms_per_step * 1e3 / launches, 3),
@@ -724,12 +921,19 @@ def main() -> int:
                 record["library_memory_rate"] = memory_rate_extra(device, stream, args.steps,
                                                                   args.warmup)
                 record["decode_layer"] = decode_layer_extra(device, stream, args.steps, args.warmup)
-        except Exception as error:  # side measurements never hide the headline
+                record["launch_floor"] = launch_floor_extra(layers, device, stream, args.steps,
+                                                            args.warmup)
+                record["large_projection_rows1"] = large_projection_extra(device, stream, args.steps,
+                                                                          args.warmup)
+                record["published_shapes"] = published_shapes_extra(device, stream, args.steps,
+                                                                    args.warmup)
+        except Exception as error:  # the headline is still printed; the exit code says it failed
             record["extras_error"] = repr(error)
     if not args.no_cpu_baseline:
         record["cpu_baseline"] = cpu_baseline(host_layers, args.rows)
+        record["cpu_baselines_other_configs"] = cpu_baselines_other_configs(host_layers)
     print(json.dumps(record))
-    return 0
+    return 1 if "extras_error" in record else 0
 
 
 if __name__ == "__main__":

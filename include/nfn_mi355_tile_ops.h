@@ -880,6 +880,20 @@ int nfn_mi355_shader_clock_probe_v1(
     int64_t microseconds,
     void* cuda_stream);
 
+/* The floor under a launch, a measurement aid like the clock probe (no
+ * counterpart in the reference): one workgroup per compute unit reads
+ * `nbytes` of `data` (16-byte aligned; rounded down to whole 16-byte pieces per
+ * workgroup) with plain coalesced loads and stores nothing; with nbytes = 0 it
+ * is an empty kernel of the same grid.  Timed back to back in a graph over
+ * the bytes a decode launch streams, it is what that launch would cost with
+ * no arithmetic at all.  `sink`: device memory of one uint32 per compute unit
+ * (1,024 bytes are enough), never written in practice. */
+int nfn_mi355_read_probe_v1(
+    const void* data,
+    int64_t nbytes,
+    uint32_t* sink,
+    void* cuda_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -639,4 +639,14 @@ int nfn_mi355_shader_clock_probe_v1(std::uint64_t* cycles_and_ticks, std::int64_
     return launch_status();
 }
 
+int nfn_mi355_read_probe_v1(const void* data, std::int64_t nbytes, std::uint32_t* sink,
+                            void* cuda_stream) {
+    if (nbytes < 0 || sink == nullptr || (nbytes > 0 && data == nullptr) ||
+        reinterpret_cast<std::uintptr_t>(data) % 16 != 0) {
+        return kInvalid;
+    }
+    launch_read_probe(data, nbytes, sink, as_stream(cuda_stream));
+    return launch_status();
+}
+
 }  // extern "C"

@@ -116,5 +116,9 @@ void launch_gqa_decode_split_device_position(
 // clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.
 void launch_clock_probe(std::uint64_t* out, std::int64_t ticks, std::uint64_t ticks_per_second,
                         hipStream_t stream);
+// clock_probe.hip — one workgroup per compute unit reads `nbytes` (rounded down to a
+// whole 16 bytes per workgroup) and stores nothing; nbytes 0 = an empty kernel.
+void launch_read_probe(const void* data, std::int64_t nbytes, std::uint32_t* sink,
+                       hipStream_t stream);
 
 }  // namespace nfn
