@@ -90,76 +90,116 @@ __device__ __forceinline__ void scale_bytes(std::uint32_t word, f16x2 bias, f16x
 
 // ---------------------------------------------------------------------------
 // activations: fp32 -> row-scaled fp16 in operand order, whole 256-row tiles
-// (rows past the end are zeros), in two launches.
+// (rows past the end are zeros), in one launch that reads the input once.
 // ---------------------------------------------------------------------------
 
-// One workgroup per row: the power of two that brings the row's largest
-// magnitude into [2^14, 2^15), and its inverse.  Zero, subnormal, infinite or
-// NaN maxima keep scale 1; padding rows get inverse 0.
-__global__ __launch_bounds__(256) void row_scale_kernel(
-    const float* __restrict__ input, float* __restrict__ scale, float* __restrict__ inverse_scale,
-    std::int64_t rows, std::int64_t width) {
-    __shared__ float partial[4];
-    const std::int64_t row = blockIdx.x;
-    const int tid = threadIdx.x;
-    if (row >= rows) {
-        if (tid == 0) {
-            scale[row] = 0.0f;
-            inverse_scale[row] = 0.0f;
-        }
-        return;
-    }
-    const float4* source = reinterpret_cast<const float4*>(input + row * width);
+// One wave per row, four rows per workgroup.  A lane owns groups of eight
+// consecutive columns (one 16-byte piece of the fp16 copy each); rows of up to
+// 8,192 columns stay in the lane's registers between the search for the row's
+// largest magnitude and the conversion, wider rows are read again (from L2).
+// The row's scale is the power of two that brings that magnitude into
+// [2^14, 2^15); zero, subnormal, infinite or NaN maxima keep scale 1; padding
+// rows get inverse 0 and zeros.
+// The eight workgroups that fill one 32-row block of the operand-order copy
+// are the ones a round-robin placement over the eight XCDs puts on the same
+// XCD (workgroup w lands on XCD w % 8), so that the 16-byte pieces they
+// scatter into the same cache lines merge in one L2 before going to memory.
+// SPLIT waves share a row (each takes a contiguous part of its columns and they exchange
+// their maxima through LDS): rows of up to 16,384 columns still fit the registers.
+template <int HELD, int SPLIT>  // HELD: 8-column groups a lane keeps in registers; 0 = read the row twice
+__global__ __launch_bounds__(256) void prepare_activations_kernel(
+    const float* __restrict__ input, std::uint8_t* __restrict__ output,
+    float* __restrict__ inverse_scale, std::int64_t rows, std::int64_t width) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const std::int64_t group_index = blockIdx.x;
+    const std::int64_t xcd = group_index & 7;
+    const std::int64_t turn = group_index >> 3;
+    constexpr int kRowsPerGroup = 4 / SPLIT;
+    constexpr int kGroupsPerBlock = 32 / kRowsPerGroup;  // workgroups that fill a 32-row block
+    const std::int64_t block_index = (turn / kGroupsPerBlock) * 8 + xcd;  // 32-row block of the copy
+    const int r = static_cast<int>(turn % kGroupsPerBlock) * kRowsPerGroup + wave / SPLIT;  // row inside it
+    const int part = wave % SPLIT;  // which part of the row's columns this wave takes
+    const std::int64_t row = block_index * 32 + r;
+    const bool live = row < rows;
+    const float* source = input + (live ? row : 0) * width;
+    const std::int64_t all_groups = width / 8;
+    const std::int64_t part_groups = (all_groups + SPLIT - 1) / SPLIT;
+    const std::int64_t first_group = part * part_groups;
+    const std::int64_t groups = min(all_groups, first_group + part_groups);  // end of this wave's groups
+
+    float4 held_x[HELD > 0 ? HELD : 1], held_y[HELD > 0 ? HELD : 1];
     float largest = 0.0f;
-    for (std::int64_t i = tid; i < width / 4; i += 256) {
-        const float4 x = source[i];
-        largest = fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+    if constexpr (HELD > 0) {
+#pragma unroll
+        for (int j = 0; j < HELD; ++j) {
+            const std::int64_t g = first_group + lane + 64 * j;
+            held_x[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            held_y[j] = held_x[j];
+            if (live && g < groups) {
+                held_x[j] = *reinterpret_cast<const float4*>(source + g * 8);
+                held_y[j] = *reinterpret_cast<const float4*>(source + g * 8 + 4);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < HELD; ++j) {
+            const float4 x = held_x[j], y = held_y[j];
+            largest = fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+            largest = fmaxf(largest, fmaxf(fmaxf(fabsf(y.x), fabsf(y.y)), fmaxf(fabsf(y.z), fabsf(y.w))));
+        }
+    } else {
+        for (std::int64_t g = first_group + lane; live && g < groups; g += 64) {
+            const float4 x = *reinterpret_cast<const float4*>(source + g * 8);
+            const float4 y = *reinterpret_cast<const float4*>(source + g * 8 + 4);
+            largest = fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+            largest = fmaxf(largest, fmaxf(fmaxf(fabsf(y.x), fabsf(y.y)), fmaxf(fabsf(y.z), fabsf(y.w))));
+        }
     }
+    // NaN never wins fmaxf: a row with NaN keeps the largest finite magnitude, as before
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {
         largest = fmaxf(largest, __shfl_xor(largest, offset));
     }
-    if ((tid & 63) == 0) partial[tid >> 6] = largest;
-    __syncthreads();
-    if (tid == 0) {
-        largest = fmaxf(fmaxf(partial[0], partial[1]), fmaxf(partial[2], partial[3]));
-        const std::uint32_t exponent = (__float_as_uint(largest) >> 23) & 0xffu;
-        const bool usable = exponent >= 16u && exponent <= 254u;
-        scale[row] = usable ? __uint_as_float((127u + 14u + 127u - exponent) << 23) : 1.0f;
-        inverse_scale[row] = usable ? __uint_as_float((exponent - 14u) << 23) : 1.0f;
+    if constexpr (SPLIT > 1) {
+        __shared__ float maxima[4];
+        if (lane == 0) maxima[wave] = largest;
+        __syncthreads();
+        const int first_wave = wave - part;
+#pragma unroll
+        for (int k = 0; k < SPLIT; ++k) largest = fmaxf(largest, maxima[first_wave + k]);
     }
-}
+    const std::uint32_t exponent = (__float_as_uint(largest) >> 23) & 0xffu;
+    const bool usable = exponent >= 16u && exponent <= 254u;
+    const float factor = !live ? 0.0f
+        : usable ? __uint_as_float((127u + 14u + 127u - exponent) << 23) : 1.0f;
+    if (lane == 0 && part == 0) {
+        inverse_scale[row] = !live ? 0.0f : usable ? __uint_as_float((exponent - 14u) << 23) : 1.0f;
+    }
 
-// Workgroup (x, y): rows 32x .. 32x+31, K values 512y .. 512y+511.  Thread t
-// handles row t%32 and the groups of 8 K values t/32, t/32+8, ...; the two
-// groups of a K chunk of 16 are handled by the two halves of one wave, so a
-// wave writes one whole 1 KB fragment per store.  Fragment (row block b, K
-// chunk c) starts at ((b * K/16) + c) * 1 KB; inside it lane (K half)*32 + row
-// holds that row's 8 values.
-__global__ __launch_bounds__(256) void convert_activations_kernel(
-    const float* __restrict__ input, const float* __restrict__ scale,
-    std::uint8_t* __restrict__ output, std::int64_t rows, std::int64_t width) {
-    const int tid = threadIdx.x;
-    const int r = tid & 31;
-    const std::int64_t row = static_cast<std::int64_t>(blockIdx.x) * 32 + r;
-    const bool live = row < rows;
-    const float* source = input + (live ? row : 0) * width;
-    const float factor = scale[row];
-    std::uint8_t* block = output + static_cast<std::int64_t>(blockIdx.x) * (width / 16) * kFragmentBytes;
-    const std::int64_t first = static_cast<std::int64_t>(blockIdx.y) * 64;
-    const std::int64_t end = min(first + 64, width / 8);
-    for (std::int64_t g = first + (tid >> 5); g < end; g += 8) {
-        float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f), y = x;
-        if (live) {
-            x = *reinterpret_cast<const float4*>(source + g * 8);
-            y = *reinterpret_cast<const float4*>(source + g * 8 + 4);
-        }
+    std::uint8_t* block = output + block_index * (width / 16) * kFragmentBytes;
+    auto store = [&](std::int64_t g, float4 x, float4 y) {
         const f16x2 h0 = {static_cast<_Float16>(x.x * factor), static_cast<_Float16>(x.y * factor)};
         const f16x2 h1 = {static_cast<_Float16>(x.z * factor), static_cast<_Float16>(x.w * factor)};
         const f16x2 h2 = {static_cast<_Float16>(y.x * factor), static_cast<_Float16>(y.y * factor)};
         const f16x2 h3 = {static_cast<_Float16>(y.z * factor), static_cast<_Float16>(y.w * factor)};
         std::uint8_t* target = block + (g >> 1) * kFragmentBytes + ((g & 1) * 32 + r) * 16;
         *reinterpret_cast<u32x4*>(target) = u32x4{bits_of(h0), bits_of(h1), bits_of(h2), bits_of(h3)};
+    };
+    if constexpr (HELD > 0) {
+#pragma unroll
+        for (int j = 0; j < HELD; ++j) {
+            const std::int64_t g = first_group + lane + 64 * j;
+            if (g < groups) store(g, held_x[j], held_y[j]);
+        }
+    } else {
+        for (std::int64_t g = first_group + lane; g < groups; g += 64) {
+            float4 x = make_float4(0.0f, 0.0f, 0.0f, 0.0f), y = x;
+            if (live) {
+                x = *reinterpret_cast<const float4*>(source + g * 8);
+                y = *reinterpret_cast<const float4*>(source + g * 8 + 4);
+            }
+            store(g, x, y);
+        }
     }
 }
 
@@ -802,7 +842,8 @@ void launch_encoding(const Descriptor& descriptor, const std::uint8_t* activatio
 
 std::int64_t padded_rows(std::int64_t rows) { return (rows + kBM - 1) / kBM * kBM; }
 
-// fp16 activations in whole 256-row tiles, then a scale and its inverse per row
+// fp16 activations in whole 256-row tiles, then the inverse scale of every row (8 bytes a row
+// are kept for it: the size is part of what callers were told to allocate)
 std::int64_t activation_bytes(std::int64_t rows, std::int64_t input_dim) {
     return (padded_rows(rows) * input_dim * 2 + padded_rows(rows) * 8 + 255) & ~std::int64_t(255);
 }
@@ -833,13 +874,21 @@ void convert_gemm_activations(const float* input, std::int64_t rows, std::int64_
                               void* workspace, hipStream_t stream) {
     std::uint8_t* activations = static_cast<std::uint8_t*>(workspace);
     float* inverse_scale = reinterpret_cast<float*>(activations + padded_rows(rows) * input_dim * 2);
-    float* scale = inverse_scale + padded_rows(rows);
-    hipLaunchKernelGGL(row_scale_kernel, dim3(static_cast<unsigned>(padded_rows(rows))), dim3(256),
-                       0, stream, input, scale, inverse_scale, rows, input_dim);
-    hipLaunchKernelGGL(convert_activations_kernel,
-                       dim3(static_cast<unsigned>(padded_rows(rows) / 32),
-                            static_cast<unsigned>((input_dim + 511) / 512)),
-                       dim3(256), 0, stream, input, scale, activations, rows, input_dim);
+    const std::int64_t groups = input_dim / 8;
+    const unsigned whole_rows = static_cast<unsigned>(padded_rows(rows) / 4);  // a wave per row
+    if (groups <= 64 * 8) {
+        hipLaunchKernelGGL((prepare_activations_kernel<8, 1>), dim3(whole_rows), dim3(256), 0, stream,
+                           input, activations, inverse_scale, rows, input_dim);
+    } else if (groups <= 64 * 16) {
+        hipLaunchKernelGGL((prepare_activations_kernel<16, 1>), dim3(whole_rows), dim3(256), 0, stream,
+                           input, activations, inverse_scale, rows, input_dim);
+    } else if (groups <= 2 * 64 * 16) {
+        hipLaunchKernelGGL((prepare_activations_kernel<16, 2>), dim3(2 * whole_rows), dim3(256), 0,
+                           stream, input, activations, inverse_scale, rows, input_dim);
+    } else {
+        hipLaunchKernelGGL((prepare_activations_kernel<0, 1>), dim3(whole_rows), dim3(256), 0, stream,
+                           input, activations, inverse_scale, rows, input_dim);
+    }
 }
 
 void launch_gemm_f16(const Descriptor& descriptor, const float* input, float* output,
