@@ -553,6 +553,26 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     result["library_f16_gemm_same_shape_M2048"] = {
         "ms": round(ms, 4), "TFLOP/s": round(library, 1),
         "frac_mfma": round(library / MFMA_PEAK_TFLOPS["f16"], 4)}
+    # Config 3's int8 leg: what the int8 matrix cores would have to run, from registers
+    # (nfn_mi355_mfma_rate_probe_v1), beside the fp16 instruction the GEMM uses.  One step =
+    # one 32 x 32 x 32 product per wave = 65,536 flop.
+    lib = tile_ops.load()
+    sink = torch.zeros(4096, dtype=torch.float32, device=device)
+    probe_steps, groups = 20000, 2 * CU_COUNT
+    legs = {}
+    for mode, label in ((0, "f16_mfma"), (1, "int8_mfma_one_plane_no_rescale"),
+                        (2, "int8_mfma_two_planes_rescaled_per_32")):
+        def run():
+            tile_ops.check(lib.nfn_mi355_mfma_rate_probe_v1(
+                mode, probe_steps, groups, sink.data_ptr(),
+                int(torch.cuda.current_stream().cuda_stream)), "mfma rate probe")
+        ms = time_replays(run, 5, 2)
+        legs[label] = round(65536.0 * probe_steps * groups * 4 / ms / 1e9, 1)
+    result["matrix_core_probe_TFLOP/s_equivalent"] = {
+        **legs,
+        "note": "useful 32x32x32 products per second x 65,536; the last row is the only int8 form "
+                "whose results can meet the 2e-3 bound (16-bit activation codes), and the reason "
+                "NFN_MI355_GEMM_INT8 stays reserved when it is below the fp16 row"}
     return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}, dequant-GEMM "
                         "incl. activation conversion", **result}
 

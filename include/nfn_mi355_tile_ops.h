@@ -880,6 +880,18 @@ int nfn_mi355_shader_clock_probe_v1(
     int64_t microseconds,
     void* cuda_stream);
 
+/* Matrix-core rates from registers, a measurement aid (no counterpart in the
+ * reference): `groups` workgroups of four waves each run `steps` steps of one
+ * 32 x 32 x 32 product per wave.  mode 0: fp16 operands (two
+ * v_mfma_f32_32x32x16_f16); mode 1: int8 operands (one
+ * v_mfma_i32_32x32x32_i8); mode 2: the int8 form a K-quant prefill with 16-bit
+ * activation codes would need -- two int8 planes into fresh accumulators and,
+ * after every 32 values, the rescale of all 16 accumulators by the sub-block's
+ * scale.  The benchmark times the three and reports their ratio: the
+ * measurement behind the reserved NFN_MI355_GEMM_INT8 mode.  `sink`: device
+ * memory of one float per workgroup, never written in practice. */
+int nfn_mi355_mfma_rate_probe_v1(int mode, int steps, int groups, float* sink, void* cuda_stream);
+
 /* The floor under a launch, a measurement aid like the clock probe (no
  * counterpart in the reference): one workgroup per compute unit reads
  * `nbytes` of `data` (16-byte aligned; rounded down to whole 16-byte pieces per

@@ -639,6 +639,15 @@ int nfn_mi355_shader_clock_probe_v1(std::uint64_t* cycles_and_ticks, std::int64_
     return launch_status();
 }
 
+int nfn_mi355_mfma_rate_probe_v1(int mode, int steps, int groups, float* sink, void* cuda_stream) {
+    if (mode < 0 || mode > 2 || steps < 1 || steps > (1 << 20) || groups < 1 || groups > 65536 ||
+        sink == nullptr) {
+        return kInvalid;
+    }
+    launch_mfma_rate_probe(mode, steps, groups, sink, as_stream(cuda_stream));
+    return launch_status();
+}
+
 int nfn_mi355_read_probe_v1(const void* data, std::int64_t nbytes, std::uint32_t* sink,
                             void* cuda_stream) {
     if (nbytes < 0 || sink == nullptr || (nbytes > 0 && data == nullptr) ||

@@ -56,7 +56,73 @@ __global__ __launch_bounds__(512) void read_probe_kernel(const v4u* __restrict__
     if (folded == 0x9e3779b9u && vectors_per_group > 0) sink[blockIdx.x] = folded;
 }
 
+// What the matrix cores sustain per 32 x 32 x 32 step, operands in registers, for
+// the three ways a prefill tile could be computed:
+//   mode 0: two v_mfma_f32_32x32x16_f16 (fp16 operands, float accumulation);
+//   mode 1: one v_mfma_i32_32x32x32_i8 (what an 8-bit activation would cost);
+//   mode 2: two v_mfma_i32_32x32x32_i8 (the two int8 planes of a 16-bit activation
+//           code) into fresh integer accumulators, then what the K-quant formats
+//           force after every 32 values: 256*high + low, conversion to float and a
+//           multiply-add with the sub-block's scale, for each of the 16 accumulators.
+// Eight waves per compute unit and several workgroups per unit, as the GEMM runs.
+typedef float probe_v16f __attribute__((ext_vector_type(16)));
+typedef int probe_v16i __attribute__((ext_vector_type(16)));
+typedef int probe_v4i __attribute__((ext_vector_type(4)));
+typedef _Float16 probe_v8h __attribute__((ext_vector_type(8)));
+
+template <int MODE>
+__global__ __launch_bounds__(256) void mfma_rate_kernel(int steps, float* __restrict__ sink) {
+    const int lane = threadIdx.x;
+    probe_v16f total;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) total[r] = 0.0f;
+    probe_v4i a8 = {lane, lane * 3, lane * 5, lane * 7}, b8 = {lane * 11, lane * 13, lane * 17, lane * 19};
+    probe_v8h a16, b16;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        a16[k] = static_cast<_Float16>(0.001f * static_cast<float>((lane + k) & 15));
+        b16[k] = static_cast<_Float16>(0.002f * static_cast<float>((lane * 3 + k) & 15));
+    }
+    float scale = 1.0f + 1.0e-6f * static_cast<float>(lane);
+    for (int step = 0; step < steps; ++step) {
+        if constexpr (MODE == 0) {
+            total = __builtin_amdgcn_mfma_f32_32x32x16_f16(a16, b16, total, 0, 0, 0);
+            total = __builtin_amdgcn_mfma_f32_32x32x16_f16(b16, a16, total, 0, 0, 0);
+        } else if constexpr (MODE == 1) {
+            probe_v16i whole = __builtin_bit_cast(probe_v16i, total);
+            whole = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b8, whole, 0, 0, 0);
+            total = __builtin_bit_cast(probe_v16f, whole);
+        } else {
+            probe_v16i zero;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) zero[r] = 0;
+            const probe_v16i high = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b8, zero, 0, 0, 0);
+            const probe_v16i low = __builtin_amdgcn_mfma_i32_32x32x32_i8(b8, a8, zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                total[r] = fmaf(static_cast<float>((high[r] << 8) + low[r]), scale, total[r]);
+            }
+            a8[0] += step;  // the next sub-block's operands and scale differ
+            scale *= 1.0000001f;
+        }
+    }
+    float folded = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) folded += total[r];
+    if (folded == 1.2345e30f) sink[blockIdx.x] = folded;
+}
+
 }  // namespace
+
+void launch_mfma_rate_probe(int mode, int steps, int groups, float* sink, hipStream_t stream) {
+    if (mode == 0) {
+        hipLaunchKernelGGL(mfma_rate_kernel<0>, dim3(groups), dim3(256), 0, stream, steps, sink);
+    } else if (mode == 1) {
+        hipLaunchKernelGGL(mfma_rate_kernel<1>, dim3(groups), dim3(256), 0, stream, steps, sink);
+    } else {
+        hipLaunchKernelGGL(mfma_rate_kernel<2>, dim3(groups), dim3(256), 0, stream, steps, sink);
+    }
+}
 
 void launch_read_probe(const void* data, std::int64_t nbytes, std::uint32_t* sink,
                        hipStream_t stream) {

@@ -120,5 +120,8 @@ void launch_clock_probe(std::uint64_t* out, std::int64_t ticks, std::uint64_t ti
 // whole 16 bytes per workgroup) and stores nothing; nbytes 0 = an empty kernel.
 void launch_read_probe(const void* data, std::int64_t nbytes, std::uint32_t* sink,
                        hipStream_t stream);
+// clock_probe.hip — `groups` workgroups of four waves run `steps` 32 x 32 x 32 matrix-core steps
+// each from registers: mode 0 fp16, 1 int8, 2 two int8 planes + the per-32 rescale.
+void launch_mfma_rate_probe(int mode, int steps, int groups, float* sink, hipStream_t stream);
 
 }  // namespace nfn

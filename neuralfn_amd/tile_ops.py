@@ -194,6 +194,7 @@ SIGNATURES = {
         ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, ctypes.c_int, _P]),
     "nfn_mi355_shader_clock_probe_v1": (ctypes.c_int, [_P, _I64, _P]),
     "nfn_mi355_read_probe_v1": (ctypes.c_int, [_P, _I64, _P, _P]),
+    "nfn_mi355_mfma_rate_probe_v1": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, _P, _P]),
     "nfn_mi355_gqa_decode_split_workspace_bytes_v1": (_I64, [_I64, _I64]),
     "nfn_mi355_attention_workspace_v1": (ctypes.c_int, [_P, _I64, _P]),
     "nfn_mi355_dflash_block_attention_split_v1": (

@@ -947,6 +947,32 @@ def test_shader_clock_probe_reports_a_plausible_clock():
     assert lib.nfn_mi355_shader_clock_probe_v1(probe.result.data_ptr(), 100001, None) == 1
 
 
+@pytest.mark.gpu
+def test_measurement_probes_run_and_check_their_arguments():
+    """nfn_mi355_read_probe_v1 and nfn_mi355_mfma_rate_probe_v1: launches that finish, store nothing,
+    and refuse bad arguments."""
+    import torch
+    device = torch.device("cuda:0")
+    lib = tile_ops.load()
+    data = torch.randint(0, 256, (1 << 20,), dtype=torch.uint8, device=device)
+    sink = torch.full((4096,), -1, dtype=torch.int32, device=device)
+    assert lib.nfn_mi355_read_probe_v1(data.data_ptr(), data.numel(), sink.data_ptr(), None) == 0
+    assert lib.nfn_mi355_read_probe_v1(None, 0, sink.data_ptr(), None) == 0          # empty kernel
+    assert lib.nfn_mi355_read_probe_v1(data.data_ptr(), 5000, sink.data_ptr(), None) == 0  # less than a piece per group
+    assert lib.nfn_mi355_read_probe_v1(None, 1024, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_read_probe_v1(data.data_ptr() + 4, 1024, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_read_probe_v1(data.data_ptr(), -1, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_read_probe_v1(data.data_ptr(), 1024, None, None) == 1
+    for mode in (0, 1, 2):
+        assert lib.nfn_mi355_mfma_rate_probe_v1(mode, 16, 8, sink.data_ptr(), None) == 0
+    assert lib.nfn_mi355_mfma_rate_probe_v1(3, 16, 8, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_mfma_rate_probe_v1(0, 0, 8, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_mfma_rate_probe_v1(0, 16, 0, sink.data_ptr(), None) == 1
+    assert lib.nfn_mi355_mfma_rate_probe_v1(0, 16, 8, None, None) == 1
+    torch.cuda.synchronize()
+    assert bool((sink == -1).all())
+
+
 @pytest.mark.parametrize("prologue", ["plain", "swiglu"])
 @pytest.mark.parametrize("rows", [5, 8])
 def test_many_tile_launches_at_five_to_eight_rows_equal_narrow_ones(cuda, prologue, rows):
