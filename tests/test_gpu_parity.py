@@ -335,6 +335,31 @@ def test_small_batch_quantized_weights(cuda, oracle, encoding, rows):
     assert normalised_error(y, expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("in_dim", [4096, 8192, 8448, 16384])
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
+def test_decode_dot_kernel_row_lengths(cuda, oracle, encoding, in_dim):
+    """The one-token kernel keeps a lane's activation operands in registers for rows of one or two
+    64-unit slices (up to 8,192 columns) and reads them from LDS for longer rows; the verifier
+    rows must equal it bit for bit at every length, grouped projections the single one."""
+    out_dims = (40, 8, 19)  # a wave's rows cross the boundaries between the projections
+    packed = [random_packed(encoding, n, in_dim, 80 + i) for i, n in enumerate(out_dims)]
+    weights = [tile_ops.PackedWeight.from_numpy(encoding, p, n, in_dim) for p, n in zip(packed, out_dims)]
+    x = kquant.synthetic_activations(81, 4, in_dim)
+    workspace = tile_ops.small_batch_workspace(4, in_dim)
+    one = tile_ops.multi_linear(weights, to_device(x[:1], cuda), workspace)
+    for y, p, n in zip(one, packed, out_dims):
+        expected = oracle.linear(encoding, p, n, in_dim, x[:1])
+        assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE
+    single = tile_ops.mmvq_linear(weights[1], to_device(x[:1], cuda), workspace)
+    assert_bits_equal(single, one[1], "single projection = its place in the group")
+    for rows in (2, 4):
+        batch = tile_ops.multi_linear(weights, to_device(x[:rows], cuda), workspace, family="mmvq")
+        for row in range(rows):
+            alone = tile_ops.multi_linear(weights, to_device(x[row:row + 1], cuda), workspace)
+            for whole, part in zip(batch, alone):
+                assert_bits_equal(whole[row:row + 1].contiguous(), part, f"verifier row {row} of {rows}")
+
+
 # ------------------------------------------------------------------- argmax
 
 def test_argmax_rows_tie_rule_at_vocabulary_width(cuda):
