@@ -6,6 +6,7 @@
 #include "common.hpp"
 #include "gemv_dot.hpp"
 #include "gemm_mfma.hpp"
+#include "gemv_f16.hpp"
 #include "gemv_mfma.hpp"
 #include "gemv_q6.hpp"
 #include "gemv_q8.hpp"
@@ -72,13 +73,17 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     const std::int64_t required = small_batch_workspace_bytes(rows, input_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
     // One or two rows, and the verifier entry points at any row count: the
-    // vector-ALU kernels.  3..16 rows otherwise: the matrix-core kernel (Q8_0:
-    // its dot kernel).  Encodings and widths without either: the float kernel.
-    // (two rows are also faster there: the dot kernels walk the token planes
+    // vector-ALU kernels.  Otherwise 3 and 4 rows: the int8 matrix-core kernel,
+    // which quantizes inside the kernel; 5..16 rows: the fp16 matrix-core kernel
+    // behind its conversion launch (Q8_0: its dot kernel at any row count).
+    // Encodings and widths without either: the float kernel.
+    // (two rows are also faster on the dot kernels: they walk the token planes
     // against the same unpacked weights)
+    constexpr std::int64_t kFirstHalfRows = 5;
     const bool one_row_arithmetic = rows <= 2 || verifier;
-    ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, exact{};
-    dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = exact.input_dim = input_dim;
+    ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, half{}, exact{};
+    dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = half.input_dim =
+        exact.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
         const std::uint32_t encoding = set.op[index].encoding;
         ProjectionSet* target = &exact;
@@ -88,13 +93,15 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
             target = &dot6;
         } else if (gemv_q8_supports(encoding, input_dim)) {
             target = &dot8;  // Q8_0 has no matrix-core kernel: the dot kernel at any row count
+        } else if (rows >= kFirstHalfRows && gemv_f16_supports(encoding, input_dim)) {
+            target = &half;
         } else if (rows >= 2 && gemv_mfma_supports(encoding, input_dim)) {
             target = &matrix;
         }
         target->op[target->count++] = set.op[index];
     }
     // Prequantized input: only the dot kernels read activation records.
-    if (prologue == kRecords && (matrix.count > 0 || exact.count > 0)) return kInvalid;
+    if (prologue == kRecords && (matrix.count > 0 || half.count > 0 || exact.count > 0)) return kInvalid;
     // In the verifier family the dot kernels leave their activation records in
     // the workspace, where a following prequantized call with the same input
     // finds them (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:3649-3666).
@@ -111,6 +118,9 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     }
     if (matrix.count > 0) {
         launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));
+    }
+    if (half.count > 0) {
+        launch_gemv_f16(half, first, second, prologue, rows, workspace, as_stream(stream));
     }
     if (exact.count > 0) {
         launch_gemv_f32(exact, first, second, prologue, nullptr, rows, as_stream(stream));

@@ -38,6 +38,7 @@
 // the float kernel neuralfn/csrc/tile_cuda/kernels.cu:1398-1525.  Weight
 // layouts and decode: neuralfn/csrc/native_gpt2/resident_glimmer.cpp:542-616.
 #include "common.hpp"
+#include "f16_decode.hpp"
 #include "gemm_mfma.hpp"
 
 namespace nfn {
@@ -45,9 +46,6 @@ namespace nfn {
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef std::uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBM = 256;
 constexpr int kBN = 128;
@@ -61,32 +59,6 @@ constexpr int kFragmentBytes = 1024;  // 32 rows x 16 K values of fp16 in operan
 struct __attribute__((packed, aligned(2))) Chunk16 {
     std::uint32_t v[4];
 };
-
-__device__ __forceinline__ std::uint32_t bits_of(f16x2 value) {
-    return __builtin_bit_cast(std::uint32_t, value);
-}
-__device__ __forceinline__ f16x2 splat(float value) {
-    const _Float16 h = static_cast<_Float16>(value);
-    return f16x2{h, h};
-}
-
-// Two code bytes of `word` (byte indices 2*pair, 2*pair+1) as fp16 (1024+b0, 1024+b1):
-// 0x6400 is 1024.0 and its ten mantissa bits count in ones.
-template <int PAIR>
-__device__ __forceinline__ f16x2 bytes_to_biased_half(std::uint32_t word) {
-    constexpr std::uint32_t selector = PAIR == 0 ? 0x04010400u : 0x04030402u;
-    return __builtin_bit_cast(f16x2, __builtin_amdgcn_perm(0x64646464u, word, selector));
-}
-
-// (bytes + bias) * scale + shift for the four code bytes of `word`
-__device__ __forceinline__ void scale_bytes(std::uint32_t word, f16x2 bias, f16x2 scale,
-                                            f16x2 shift, std::uint32_t& out0,
-                                            std::uint32_t& out1) {
-    const f16x2 x0 = bytes_to_biased_half<0>(word) + bias;
-    const f16x2 x1 = bytes_to_biased_half<1>(word) + bias;
-    out0 = bits_of(__builtin_elementwise_fma(x0, scale, shift));
-    out1 = bits_of(__builtin_elementwise_fma(x1, scale, shift));
-}
 
 // ---------------------------------------------------------------------------
 // activations: fp32 -> row-scaled fp16 in operand order, whole 256-row tiles
@@ -218,29 +190,6 @@ struct PackedSlice;
 template <std::uint32_t ENC>
 struct BlockHeader;
 
-// shared by Q4_K and Q5_K: d, dmin and the 6-bit scale/min pair of the step
-struct KBlockScales {
-    std::uint32_t sc, mn;  // low byte: first group, next byte: second group
-    f16x2 scale_a, shift_a, scale_b, shift_b;
-    __device__ __forceinline__ void bits(u32x4 header, int pair) {
-        const int shift = 16 * (pair & 1);
-        const std::uint32_t ys = header.y >> shift, zs = header.z >> shift, ws = header.w >> shift;
-        // sub-blocks 4..7 keep their 6-bit values split over two bytes; bit masks
-        // instead of a branch keep the K step free of control flow
-        const std::uint32_t upper = 0u - static_cast<std::uint32_t>(pair >> 1);
-        sc = (((ws & 0x0f0fu) | ((ys >> 2) & 0x3030u)) & upper) | ((ys & 0x3f3fu) & ~upper);
-        mn = ((((ws >> 4) & 0x0f0fu) | ((zs >> 2) & 0x3030u)) & upper) | ((zs & 0x3f3fu) & ~upper);
-    }
-    __device__ __forceinline__ void scales(u32x4 header) {
-        const float d = half_bits_to_float(header.x & 0xffffu);
-        const float dmin = half_bits_to_float(header.x >> 16);
-        scale_a = splat(d * static_cast<float>(sc & 0xffu));
-        scale_b = splat(d * static_cast<float>((sc >> 8) & 0xffu));
-        shift_a = splat(-(dmin * static_cast<float>(mn & 0xffu)));
-        shift_b = splat(-(dmin * static_cast<float>((mn >> 8) & 0xffu)));
-    }
-};
-
 template <>
 struct BlockHeader<kEncQ4K> {
     u32x4 words;  // d, dmin and the twelve scale bytes
@@ -314,12 +263,17 @@ struct PackedSlice<kEncQ5K> {
 
 template <>
 struct BlockHeader<kEncQ6K> {
-    u32x4 scales;  // sixteen int8 sub-scales
+    // sixteen int8 sub-scales in four words, then d; five plain words, so that the
+    // struct has no padding for a copy to carry through scratch memory
+    std::uint32_t scales_x, scales_y, scales_z, scales_w;
     std::uint32_t d_bits;
     __device__ __forceinline__ void load(const std::uint8_t* row, int block) {
         const std::uint8_t* p = row + block * 210;
         const Chunk16 s = *reinterpret_cast<const Chunk16*>(p + 192);
-        scales = u32x4{s.v[0], s.v[1], s.v[2], s.v[3]};
+        scales_x = s.v[0];
+        scales_y = s.v[1];
+        scales_z = s.v[2];
+        scales_w = s.v[3];
         d_bits = *reinterpret_cast<const std::uint16_t*>(p + 208);
     }
 };
@@ -345,8 +299,8 @@ struct PackedSlice<kEncQ6K> {
                                                  int half) {
         // sub-scale index = 8*half_of_block + 2*quarter + position/16: the step's four
         // are word `pair` of the sixteen, and this thread's 16 positions share one per quarter
-        const std::uint32_t sub_scales = pair == 0 ? header.scales.x
-            : pair == 1 ? header.scales.y : pair == 2 ? header.scales.z : header.scales.w;
+        const std::uint32_t sub_scales = pair == 0 ? header.scales_x
+            : pair == 1 ? header.scales_y : pair == 2 ? header.scales_z : header.scales_w;
         sa = static_cast<std::int8_t>((sub_scales >> (8 * half)) & 0xffu);
         sb = static_cast<std::int8_t>((sub_scales >> (8 * (2 + half))) & 0xffu);
         upper = (pair & 1) * 4;  // quarters 2,3: high nibbles, high-bit pairs 4..7

@@ -1,0 +1,531 @@
+// Small-batch (3..16 rows) GEMV on the fp16 matrix cores.
+//
+// A small launch first turns the activations into fp16, every row scaled by
+// the power of two that brings its largest magnitude into [2^14, 2^15), and
+// stores them in the caller's workspace by groups of eight columns:
+// [column / 8][row][8 values], so that the 16 bytes one lane feeds to a matrix
+// instruction are contiguous and the lanes of a quarter wave read one segment.
+// Fused prologues (sigmoid gate, SwiGLU) are applied there.
+//
+// In the main kernel a workgroup of 8 waves owns tiles of 16 consecutive
+// weight rows (persistent: tiles blockIdx.x, blockIdx.x + gridDim.x, ...).
+// The waves split K by 256-value blocks and meet once per tile in a
+// fixed-order sum.  Per block a lane (row i = lane % 16, quarter j = lane / 16)
+// loads its share of the packed bytes of row i straight into registers (the
+// block's header and a quarter of its codes), dequantizes them to fp16 with
+// packed arithmetic and feeds eight v_mfma_f32_16x16x32_f16: operand B is the
+// weights (column = weight row), operand A the activations (row = token).
+// The K index of a matrix instruction is only a pairing of A and B elements,
+// so every format picks the eight columns a lane contributes from the bytes
+// it already holds; the activation address follows that choice.  Weights are
+// read from HBM once; no weight byte goes through LDS.
+//
+// Arithmetic it replaces: the reference's small-batch kernel
+// (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:1174-1303), which multiplies 8-bit
+// activation codes with the integer codes; here the weights are dequantized
+// ((q * d*sc - dmin*m) rounded to fp16, 11 significant bits) and the
+// activations keep 11 significant bits each, which stays within 2e-3 of the
+// float-activation CPU engine
+// (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:655-679) like the prefill
+// GEMM with the same number formats.  Results do not depend on the launch
+// geometry: the sum over K runs block by block inside a wave and the eight
+// waves' partial sums are added in wave order.
+#include "common.hpp"
+#include "f16_decode.hpp"
+#include "gemv_f16.hpp"
+#include "wave_rows.hpp"
+
+namespace nfn {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTileRows = 16;
+constexpr int kWaves = 8;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kDepth = 4;  // blocks in flight per wave
+
+struct __attribute__((packed, aligned(2))) Chunk8 {
+    std::uint32_t v[2];
+};
+struct __attribute__((packed, aligned(2))) Chunk16 {
+    std::uint32_t v[4];
+};
+
+// ---- activations: fp32 -> row-scaled fp16, [column / 8][row][8] ----------------
+
+constexpr int kImageThreads = 256;
+constexpr int kImageHeld = 8;  // 8-column groups a thread keeps: rows of up to 16,384 columns are read once
+
+__device__ __forceinline__ float largest_of(float4 x, float largest) {
+    return fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+}
+
+// One workgroup per row.
+template <int P>
+__global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
+    const float* __restrict__ first, const float* __restrict__ second,
+    std::uint8_t* __restrict__ image, float* __restrict__ inverse_scale, int tokens,
+    int input_dim) {
+    __shared__ float maxima[kImageThreads / kWave];
+    const int token = blockIdx.x;
+    const int groups = input_dim >> 3;
+    const std::int64_t base = static_cast<std::int64_t>(token) * input_dim;
+    const bool held = groups <= kImageThreads * kImageHeld;  // uniform
+    float4 x[kImageHeld][2];
+    float largest = 0.0f;
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j) {
+            const int g = threadIdx.x + kImageThreads * j;
+            x[j][0] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            x[j][1] = x[j][0];
+            if (g < groups) {
+                x[j][0] = load_activations<P>(first, second, base + g * 8);
+                x[j][1] = load_activations<P>(first, second, base + g * 8 + 4);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j) largest = largest_of(x[j][1], largest_of(x[j][0], largest));
+    } else {
+        for (int g = threadIdx.x; g < groups; g += kImageThreads) {
+            largest = largest_of(load_activations<P>(first, second, base + g * 8), largest);
+            largest = largest_of(load_activations<P>(first, second, base + g * 8 + 4), largest);
+        }
+    }
+    // NaN never wins fmaxf: a row with NaN keeps its largest finite magnitude
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) largest = fmaxf(largest, __shfl_xor(largest, offset));
+    if ((threadIdx.x & 63) == 0) maxima[threadIdx.x >> 6] = largest;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kImageThreads / kWave; ++w) largest = fmaxf(largest, maxima[w]);
+    // zero, subnormal-range, infinite maxima keep scale 1
+    const std::uint32_t exponent = (__float_as_uint(largest) >> 23) & 0xffu;
+    const bool usable = exponent >= 16u && exponent <= 254u;
+    const float factor = usable ? __uint_as_float((127u + 14u + 127u - exponent) << 23) : 1.0f;
+    if (threadIdx.x == 0) {
+        inverse_scale[token] = usable ? __uint_as_float((exponent - 14u) << 23) : 1.0f;
+    }
+    auto store = [&](int g, float4 a, float4 b) {
+        const f16x2 h0 = {static_cast<_Float16>(a.x * factor), static_cast<_Float16>(a.y * factor)};
+        const f16x2 h1 = {static_cast<_Float16>(a.z * factor), static_cast<_Float16>(a.w * factor)};
+        const f16x2 h2 = {static_cast<_Float16>(b.x * factor), static_cast<_Float16>(b.y * factor)};
+        const f16x2 h3 = {static_cast<_Float16>(b.z * factor), static_cast<_Float16>(b.w * factor)};
+        std::uint8_t* target = image + (static_cast<std::int64_t>(g) * tokens + token) * 16;
+        *reinterpret_cast<u32x4*>(target) = u32x4{bits_of(h0), bits_of(h1), bits_of(h2), bits_of(h3)};
+    };
+    if (held) {
+#pragma unroll
+        for (int j = 0; j < kImageHeld; ++j) {
+            const int g = threadIdx.x + kImageThreads * j;
+            if (g < groups) store(g, x[j][0], x[j][1]);
+        }
+    } else {
+        for (int g = threadIdx.x; g < groups; g += kImageThreads) {
+            store(g, load_activations<P>(first, second, base + g * 8),
+                  load_activations<P>(first, second, base + g * 8 + 4));
+        }
+    }
+}
+
+// ---- what one lane holds of one 256-value block of its weight row ---------------
+// load(): the packed bytes (header and this quarter's codes).
+// prepare(): the fp16 scale constants.
+// operand<M>(): the eight weights of matrix instruction M as fp16.
+// group(m, j): which group of eight columns of the block those are.
+
+__device__ __forceinline__ f16x8 as_operand(std::uint32_t a, std::uint32_t b, std::uint32_t c,
+                                            std::uint32_t d) {
+    return __builtin_bit_cast(f16x8, u32x4{a, b, c, d});
+}
+
+template <std::uint32_t ENC>
+struct PackedBlock;
+
+// Q4_K: a 16-byte piece c of the 128 code bytes holds values 16*(c%2)..+15 of
+// sub-blocks 2*(c/2) (low nibbles) and 2*(c/2)+1 (high nibbles).  Quarter j
+// takes pieces j and j + 4; instructions 0..3 use the first, 4..7 the second:
+// M % 4 = 2*(high nibbles) + (second eight values).
+template <>
+struct PackedBlock<kEncQ4K> {
+    static constexpr int kBytes = 144;
+    u32x4 header, piece[2];
+    KBlockScales scales[2];
+    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
+        header = *reinterpret_cast<const u32x4*>(block);
+        piece[0] = *reinterpret_cast<const u32x4*>(block + 16 + 16 * j);
+        piece[1] = *reinterpret_cast<const u32x4*>(block + 16 + 64 + 16 * j);
+    }
+    __device__ __forceinline__ void prepare(int j) {
+        scales[0].bits(header, j >> 1);
+        scales[0].scales(header);
+        scales[1].bits(header, (j >> 1) + 2);
+        scales[1].scales(header);
+    }
+    __device__ __forceinline__ static int group(int m, int j) {
+        return 8 * ((j >> 1) + 2 * (m >> 2)) + 4 * ((m >> 1) & 1) + 2 * (j & 1) + (m & 1);
+    }
+    template <int M>
+    __device__ __forceinline__ f16x8 operand() const {
+        constexpr int kPiece = M >> 2, kHigh = (M >> 1) & 1, kWord = 2 * (M & 1);
+        const KBlockScales& s = scales[kPiece];
+        const std::uint32_t a = (kHigh ? piece[kPiece][kWord] >> 4 : piece[kPiece][kWord]) & 0x0f0f0f0fu;
+        const std::uint32_t b =
+            (kHigh ? piece[kPiece][kWord + 1] >> 4 : piece[kPiece][kWord + 1]) & 0x0f0f0f0fu;
+        std::uint32_t out[4];
+        scale_bytes(a, splat(-1024.0f), kHigh ? s.scale_b : s.scale_a, kHigh ? s.shift_b : s.shift_a,
+                    out[0], out[1]);
+        scale_bytes(b, splat(-1024.0f), kHigh ? s.scale_b : s.scale_a, kHigh ? s.shift_b : s.shift_a,
+                    out[2], out[3]);
+        return as_operand(out[0], out[1], out[2], out[3]);
+    }
+};
+
+// Q5_K: as Q4_K, and bit s of high-bit byte v is the fifth bit of value v of
+// sub-block s; both pieces of a quarter cover values 16*(j%2)..+15.
+template <>
+struct PackedBlock<kEncQ5K> {
+    static constexpr int kBytes = 176;
+    u32x4 header, fifth, piece[2];
+    KBlockScales scales[2];
+    int fifth_shift;  // sub-block of the first piece's low nibbles
+    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
+        header = *reinterpret_cast<const u32x4*>(block);
+        fifth = *reinterpret_cast<const u32x4*>(block + 16 + 16 * (j & 1));
+        piece[0] = *reinterpret_cast<const u32x4*>(block + 48 + 16 * j);
+        piece[1] = *reinterpret_cast<const u32x4*>(block + 48 + 64 + 16 * j);
+    }
+    __device__ __forceinline__ void prepare(int j) {
+        scales[0].bits(header, j >> 1);
+        scales[0].scales(header);
+        scales[1].bits(header, (j >> 1) + 2);
+        scales[1].scales(header);
+        fifth_shift = 2 * (j >> 1);
+    }
+    __device__ __forceinline__ static int group(int m, int j) {
+        return PackedBlock<kEncQ4K>::group(m, j);
+    }
+    template <int M>
+    __device__ __forceinline__ f16x8 operand() const {
+        constexpr int kPiece = M >> 2, kHigh = (M >> 1) & 1, kWord = 2 * (M & 1);
+        const KBlockScales& s = scales[kPiece];
+        const int shift = fifth_shift + 4 * kPiece + kHigh;  // the sub-block's bit
+        std::uint32_t out[4];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            const std::uint32_t word = piece[kPiece][kWord + w];
+            const std::uint32_t nibbles = (kHigh ? word >> 4 : word) & 0x0f0f0f0fu;
+            const std::uint32_t bit = ((fifth[kWord + w] >> shift) & 0x01010101u) << 4;
+            scale_bytes(nibbles | bit, splat(-1024.0f), kHigh ? s.scale_b : s.scale_a,
+                        kHigh ? s.shift_b : s.shift_a, out[2 * w], out[2 * w + 1]);
+        }
+        return as_operand(out[0], out[1], out[2], out[3]);
+    }
+};
+
+// Q6_K: value v (0..31) of quarter q (0..3) of half n (0, 1) of the block has
+// its low nibble in ql[64n + 32*(q%2) + v] (high nibble for q >= 2) and bits
+// 2q, 2q+1 of qh[32n + v] on top; one int8 sub-scale per 16 values.  Quarter j
+// of the wave takes values 16*(j%2)..+15 of every quarter of half j/2:
+// instruction M = 2q + (second eight values).
+template <>
+struct PackedBlock<kEncQ6K> {
+    static constexpr int kBytes = 210;
+    u32x4 low_a, low_b, top;
+    std::uint32_t sub_scales[2];  // the eight of this lane's half
+    std::uint32_t d_bits;
+    f16x2 scale[4];  // per quarter
+    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
+        const int n = j >> 1, h = j & 1;
+        const Chunk16 a = *reinterpret_cast<const Chunk16*>(block + 64 * n + 16 * h);
+        const Chunk16 b = *reinterpret_cast<const Chunk16*>(block + 64 * n + 32 + 16 * h);
+        const Chunk16 t = *reinterpret_cast<const Chunk16*>(block + 128 + 32 * n + 16 * h);
+        const Chunk8 s = *reinterpret_cast<const Chunk8*>(block + 192 + 8 * n);
+        low_a = u32x4{a.v[0], a.v[1], a.v[2], a.v[3]};
+        low_b = u32x4{b.v[0], b.v[1], b.v[2], b.v[3]};
+        top = u32x4{t.v[0], t.v[1], t.v[2], t.v[3]};
+        sub_scales[0] = s.v[0];
+        sub_scales[1] = s.v[1];
+        d_bits = *reinterpret_cast<const std::uint16_t*>(block + 208);
+    }
+    __device__ __forceinline__ void prepare(int j) {
+        const float d = half_bits_to_float(d_bits);
+        const int within = 8 * (j & 1);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            // sub-scale 8n + 2q + j%2: byte (2q + j%2) % 4 of word q/2 of this half's eight
+            const std::uint32_t pair = sub_scales[q >> 1] >> (16 * (q & 1));
+            const int value = static_cast<std::int8_t>((pair >> within) & 0xffu);
+            scale[q] = splat(d * static_cast<float>(value));
+        }
+    }
+    __device__ __forceinline__ static int group(int m, int j) {
+        return 16 * (j >> 1) + 4 * (m >> 1) + 2 * (j & 1) + (m & 1);
+    }
+    template <int M>
+    __device__ __forceinline__ f16x8 operand() const {
+        constexpr int kQuarter = M >> 1, kWord = 2 * (M & 1);
+        std::uint32_t out[4];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            const std::uint32_t low = (kQuarter & 1) ? low_b[kWord + w] : low_a[kWord + w];
+            const std::uint32_t nibbles = (kQuarter >= 2 ? low >> 4 : low) & 0x0f0f0f0fu;
+            const std::uint32_t bits = top[kWord + w];
+            const std::uint32_t upper =
+                (kQuarter < 2 ? bits << (4 - 2 * kQuarter) : bits >> (2 * kQuarter - 4)) & 0x30303030u;
+            // bias: 1024 + the format's offset of 32
+            scale_bytes(nibbles | upper, splat(-1056.0f), scale[kQuarter], splat(0.0f), out[2 * w],
+                        out[2 * w + 1]);
+        }
+        return as_operand(out[0], out[1], out[2], out[3]);
+    }
+};
+
+// Projection a tile belongs to.
+__device__ __forceinline__ Projection tile_projection(const ProjectionSet& set, std::uint32_t tile) {
+    int which = 0;
+#pragma unroll
+    for (int index = 1; index < 4; ++index) {
+        if (index < set.count && tile >= set.op[index].first_tile) which = index;
+    }
+    return pick(set, which);
+}
+
+// What a wave keeps of one step in flight: the packed weights, and, when the
+// activations stream with them, the eight operand fragments of the block.
+template <std::uint32_t ENC, bool RESIDENT>
+struct Stage {
+    PackedBlock<ENC> weights;
+    f16x8 activations[RESIDENT ? 1 : 8];
+};
+
+// RESIDENT: rows of up to 8,192 columns.  A wave's K range is at most four
+// blocks, whose activation fragments it loads once and keeps in registers for
+// all its tiles (128 registers); a tile is four steps, step s of every tile
+// uses stage s and fragment set s, and only packed weights stream.
+// Otherwise: the fragments of a block are loaded again with its weights for
+// every tile.
+template <std::uint32_t ENC, bool RESIDENT>
+__global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
+    const std::uint8_t* __restrict__ image, const float* __restrict__ inverse_scale, int tokens,
+    std::uint32_t total_tiles, int input_dim, ProjectionSet set) {
+    using Block = PackedBlock<ENC>;
+    __shared__ float partial[2 * kWaves * kWave * 4];
+
+    const int lane = threadIdx.x & 63;
+    // the wave index is uniform; saying so keeps tile bookkeeping in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15;
+    const int j = lane >> 4;
+    const int blocks = input_dim >> 8;
+    const int begin = blocks * wave / kWaves;
+    const int end = blocks * (wave + 1) / kWaves;
+    const int count = end - begin;
+    // steps of a tile, the same for every wave (a wave whose K range is shorter idles in the last ones)
+    const int steps = RESIDENT ? kDepth : (blocks + kWaves - 1) / kWaves;
+
+    // This lane's 16 bytes of the group g of eight columns: image + (g * tokens + i) * 16.
+    // Lanes past the last token read token 0 again: a row of A only reaches its own row of
+    // the result, and those rows are never stored.
+    const std::uint8_t* lane_image = image + (i < tokens ? i : 0) * 16;
+    const std::int64_t group_bytes = static_cast<std::int64_t>(tokens) * 16;
+    std::uint32_t group_offset[8];  // of instruction m's group inside a block
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        group_offset[m] = static_cast<std::uint32_t>(Block::group(m, j)) * static_cast<std::uint32_t>(group_bytes);
+    }
+    auto load_fragments = [&](int block, f16x8 (&fragments)[8]) {
+        const std::uint8_t* block_image = lane_image + static_cast<std::int64_t>(block) * 32 * group_bytes;
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            fragments[m] = *reinterpret_cast<const f16x8*>(block_image + group_offset[m]);
+        }
+    };
+    f16x8 resident[RESIDENT ? kDepth : 1][8];
+    if constexpr (RESIDENT) {
+#pragma unroll
+        for (int s = 0; s < kDepth; ++s) load_fragments(begin + max(min(s, count - 1), 0), resident[s]);
+    }
+
+    // register r of quarter j of the result: token 4j + r
+    float token_scale[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) token_scale[r] = inverse_scale[min(4 * j + r, tokens - 1)];
+
+    const std::uint32_t first_tile = blockIdx.x;
+    const int tile_count = static_cast<int>((total_tiles - first_tile + gridDim.x - 1) / gridDim.x);
+    const int total = tile_count * steps;
+
+    // Every wave walks the same flat stream of (tile, step) pairs, so the waves
+    // meet at the end of a tile in uniform control flow.  Loads run kDepth steps
+    // ahead; they are unconditional (a step without work reads the first bytes
+    // of the first projection, one line for the whole wave), so a step waits
+    // for nothing but its own.
+    std::uint32_t fetch_tile = first_tile;
+    int fetch_step = 0;
+    bool fetch_live = true;
+    const std::uint8_t* fetch_row = nullptr;
+    auto fetch_setup = [&]() {
+        const Projection op = tile_projection(set, fetch_tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(fetch_tile - op.first_tile) * kTileRows;
+        const std::int64_t last = op.output_dim - 1 - row0;  // rows past the end repeat the last one
+        fetch_row = op.data + (row0 + min(static_cast<std::int64_t>(i), last)) * op.row_stride;
+    };
+    fetch_setup();
+    auto fetch = [&](Stage<ENC, RESIDENT>& stage) {
+        const bool work = fetch_live && fetch_step < count;
+        const int block = begin + max(min(fetch_step, count - 1), 0);
+        const std::uint8_t* source =
+            work ? fetch_row + static_cast<std::int64_t>(block) * Block::kBytes : set.op[0].data;
+        stage.weights.load(source, work ? j : 0);
+        if constexpr (!RESIDENT) load_fragments(work ? block : 0, stage.activations);
+        if (++fetch_step == steps) {
+            fetch_step = 0;
+            if (fetch_tile + gridDim.x < total_tiles) {
+                fetch_tile += gridDim.x;
+                fetch_setup();
+            } else {
+                fetch_live = false;  // stream exhausted
+            }
+        }
+    };
+    Stage<ENC, RESIDENT> stages[kDepth];
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) fetch(stages[d]);
+
+    std::uint32_t tile = first_tile;
+    int work_step = 0;
+    int parity = 0;
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto step = [&](Stage<ENC, RESIDENT>& stage, const f16x8 (&a)[8], int position) {
+        if (position < total) {
+            if (work_step < count) {
+                stage.weights.prepare(j);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[0], stage.weights.template operand<0>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[1], stage.weights.template operand<1>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2], stage.weights.template operand<2>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[3], stage.weights.template operand<3>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[4], stage.weights.template operand<4>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[5], stage.weights.template operand<5>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[6], stage.weights.template operand<6>(), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], stage.weights.template operand<7>(), acc, 0, 0, 0);
+            }
+            if (++work_step == steps) {
+                // Cross-wave sum in wave order; the two buffers alternate so one
+                // barrier per tile is enough.
+                float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * 4;
+                *reinterpret_cast<f32x4*>(mine) = acc;
+                __syncthreads();
+                if (wave == (parity ? kWaves - 1 : 0)) {
+                    const Projection op = tile_projection(set, tile);
+                    const std::int64_t row = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows + i;
+                    f32x4 sum = *reinterpret_cast<const f32x4*>(partial + ((parity * kWaves + 0) * kWave + lane) * 4);
+#pragma unroll
+                    for (int w = 1; w < kWaves; ++w) {
+                        sum += *reinterpret_cast<const f32x4*>(partial + ((parity * kWaves + w) * kWave + lane) * 4);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int token = 4 * j + r;
+                        if (token < tokens && row < op.output_dim) {
+                            op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
+                                sum[r] * token_scale[r];
+                        }
+                    }
+                }
+                parity ^= 1;
+                work_step = 0;
+                tile += gridDim.x;
+                acc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+        fetch(stage);
+    };
+
+    for (int position = 0; position < total; position += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            if constexpr (RESIDENT) {
+                step(stages[d], resident[d], position + d);
+            } else {
+                step(stages[d], stages[d].activations, position + d);
+            }
+        }
+    }
+}
+
+template <std::uint32_t ENC>
+void launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* inverse_scale,
+                     int tokens, hipStream_t stream) {
+    std::uint32_t tiles = 0;
+    for (int index = 0; index < set.count; ++index) {
+        set.op[index].first_tile = tiles;
+        tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
+    }
+    // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
+    const std::uint32_t slots = static_cast<std::uint32_t>(compute_units());
+    const std::uint32_t grid = tiles < slots ? tiles : slots;
+    if ((set.input_dim >> 8) <= kWaves * kDepth) {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, true>), dim3(grid), dim3(kThreads), 0, stream, image,
+                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
+    } else {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, false>), dim3(grid), dim3(kThreads), 0, stream, image,
+                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
+    }
+}
+
+}  // namespace
+
+bool gemv_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
+    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
+        input_dim % 256 == 0 && input_dim <= 65536;
+}
+
+std::int64_t gemv_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
+    return rows * input_dim * 2 + rows * 4;
+}
+
+void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* second, int prologue,
+                     std::int64_t rows, void* workspace, hipStream_t stream) {
+    std::uint8_t* image = static_cast<std::uint8_t*>(workspace);
+    float* inverse_scale = reinterpret_cast<float*>(image + rows * set.input_dim * 2);
+    const int tokens = static_cast<int>(rows);
+    const int input_dim = static_cast<int>(set.input_dim);
+    const dim3 grid(static_cast<unsigned>(rows));
+    switch (prologue) {
+        case kGated:
+            hipLaunchKernelGGL((f16_image_kernel<kGated>), grid, dim3(kImageThreads), 0, stream, first,
+                               second, image, inverse_scale, tokens, input_dim);
+            break;
+        case kSwiGlu:
+            hipLaunchKernelGGL((f16_image_kernel<kSwiGlu>), grid, dim3(kImageThreads), 0, stream, first,
+                               second, image, inverse_scale, tokens, input_dim);
+            break;
+        default:
+            hipLaunchKernelGGL((f16_image_kernel<kPlain>), grid, dim3(kImageThreads), 0, stream, first,
+                               second, image, inverse_scale, tokens, input_dim);
+            break;
+    }
+    // one launch per encoding present
+    const std::uint32_t encodings[3] = {kEncQ4K, kEncQ5K, kEncQ6K};
+    for (const std::uint32_t encoding : encodings) {
+        ProjectionSet group{};
+        group.input_dim = set.input_dim;
+        for (int index = 0; index < set.count; ++index) {
+            if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
+        }
+        if (group.count == 0) continue;
+        if (encoding == kEncQ4K) {
+            launch_encoding<kEncQ4K>(group, image, inverse_scale, tokens, stream);
+        } else if (encoding == kEncQ5K) {
+            launch_encoding<kEncQ5K>(group, image, inverse_scale, tokens, stream);
+        } else {
+            launch_encoding<kEncQ6K>(group, image, inverse_scale, tokens, stream);
+        }
+    }
+}
+
+}  // namespace nfn

@@ -1020,10 +1020,12 @@ def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, o
     def error(actual, expected):
         return float(np.max(np.abs(actual - expected)) / np.max(np.abs(expected)))
 
-    # the projections of a block and of one token quantize their activations in different
-    # kernels: each within 2e-3 of the float formula, here about 1e-4 apart
-    assert error(residual.cpu().numpy(), np.stack(serial_hidden)) <= 1e-3
-    assert error(pending.cpu().numpy(), np.stack(serial_down)) <= 1e-3
+    # the projections of a block (fp16 weights and activations on the matrix cores, 11
+    # significant bits each) and of one token (integer codes against 16-bit activation codes)
+    # run in different kernels: each within 2e-3 of the float formula, and after two layers
+    # about 1e-3 apart
+    assert error(residual.cpu().numpy(), np.stack(serial_hidden)) <= 2e-3
+    assert error(pending.cpu().numpy(), np.stack(serial_down)) <= 2e-3
     for cache, serial_cache, (key_rows, value_rows) in zip(block_caches, serial_caches, staged):
         engine_ops.cache_commit(key_rows, value_rows, cache.keys, cache.values, position, rows=rows)
         # committed rows carry the upstream rounding differences: a bf16 step apart at most

@@ -335,6 +335,33 @@ def test_small_batch_quantized_weights(cuda, oracle, encoding, rows):
     assert normalised_error(y, expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("rows", [5, 9, 16])
+@pytest.mark.parametrize("in_dim", [256, 2304, 8192, 8448])
+def test_small_batch_half_kernel_shapes(cuda, oracle, in_dim, rows):
+    """Five rows and more run on the fp16 matrix cores behind a conversion launch.  Row lengths:
+    one block (seven of the eight waves of a workgroup have no K range), nine blocks (ranges
+    of one and two blocks), the longest row whose activation fragments stay in registers and
+    the first length past it.  Projections of 40, 8 and 19 rows: partial 16-row tiles and
+    tiles of different projections and formats in one call.  Activations of very different
+    magnitude per row: every row carries its own power-of-two scale."""
+    specs = [(kquant.Q4_K, 40), (kquant.Q5_K, 8), (kquant.Q6_K, 19), (kquant.Q4_K, 16)]
+    packed = [random_packed(e, n, in_dim, 90 + i) for i, (e, n) in enumerate(specs)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, p, n, in_dim) for (e, n), p in zip(specs, packed)]
+    x = kquant.synthetic_activations(91 + rows, rows, in_dim)
+    x *= (10.0 ** np.linspace(-6, 5, rows)).astype(np.float32)[:, None]
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    outputs = tile_ops.multi_linear(weights, to_device(x, cuda), workspace)
+    again = tile_ops.multi_linear(weights, to_device(x, cuda), workspace)
+    for (encoding, out_dim), p, y, z in zip(specs, packed, outputs, again):
+        expected = oracle.linear(encoding, p, out_dim, in_dim, x)
+        for row in range(rows):  # per row: the rows differ by eleven orders of magnitude
+            assert normalised_error(y[row:row + 1].cpu().numpy(), expected[row:row + 1]) <= TOLERANCE
+        assert_bits_equal(y, z, "the same call twice")
+    # a single projection alone gives the bits it gives inside the group
+    alone = tile_ops.multi_linear(weights[2:3], to_device(x, cuda), workspace)[0]
+    assert_bits_equal(alone, outputs[2], "single projection = its place in the group")
+
+
 @pytest.mark.parametrize("in_dim", [4096, 8192, 8448, 16384])
 @pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
 def test_decode_dot_kernel_row_lengths(cuda, oracle, encoding, in_dim):
