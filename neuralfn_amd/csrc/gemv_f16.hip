@@ -46,13 +46,6 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kDepth = 4;  // blocks in flight per wave
 
-struct __attribute__((packed, aligned(2))) Chunk8 {
-    std::uint32_t v[2];
-};
-struct __attribute__((packed, aligned(2))) Chunk16 {
-    std::uint32_t v[4];
-};
-
 // ---- activations: fp32 -> row-scaled fp16, [column / 8][row][8] ----------------
 
 constexpr int kImageThreads = 256;
@@ -131,10 +124,16 @@ __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
 }
 
 // ---- what one lane holds of one 256-value block of its weight row ---------------
-// load(): the packed bytes (header and this quarter's codes).
+// load(): the packed bytes (header and this quarter's codes) of the block at
+//   `block` (uniform) + `row` (this lane's byte offset, 32 bits): a scalar base
+//   and a 32-bit lane offset, the addressing form that needs no address arithmetic.
 // prepare(): the fp16 scale constants.
 // operand<M>(): the eight weights of matrix instruction M as fp16.
-// group(m, j): which group of eight columns of the block those are.
+// lane_group(j) + step_group(m): which group of eight columns of the block those are.
+
+typedef const __attribute__((address_space(1))) std::uint8_t* GlobalBytes;
+typedef const __attribute__((address_space(1))) u32x4* GlobalVec;
+typedef const __attribute__((address_space(1))) f16x8* GlobalFragment;
 
 __device__ __forceinline__ f16x8 as_operand(std::uint32_t a, std::uint32_t b, std::uint32_t c,
                                             std::uint32_t d) {
@@ -153,10 +152,11 @@ struct PackedBlock<kEncQ4K> {
     static constexpr int kBytes = 144;
     u32x4 header, piece[2];
     KBlockScales scales[2];
-    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
-        header = *reinterpret_cast<const u32x4*>(block);
-        piece[0] = *reinterpret_cast<const u32x4*>(block + 16 + 16 * j);
-        piece[1] = *reinterpret_cast<const u32x4*>(block + 16 + 64 + 16 * j);
+    __device__ __forceinline__ void load(GlobalBytes block, std::uint32_t row, int j) {
+        header = *reinterpret_cast<GlobalVec>(block + row);
+        const std::uint32_t mine = row + 16 + 16 * j;
+        piece[0] = *reinterpret_cast<GlobalVec>(block + mine);
+        piece[1] = *reinterpret_cast<GlobalVec>(block + mine + 64);
     }
     __device__ __forceinline__ void prepare(int j) {
         scales[0].bits(header, j >> 1);
@@ -164,9 +164,8 @@ struct PackedBlock<kEncQ4K> {
         scales[1].bits(header, (j >> 1) + 2);
         scales[1].scales(header);
     }
-    __device__ __forceinline__ static int group(int m, int j) {
-        return 8 * ((j >> 1) + 2 * (m >> 2)) + 4 * ((m >> 1) & 1) + 2 * (j & 1) + (m & 1);
-    }
+    __device__ __forceinline__ static int lane_group(int j) { return 8 * (j >> 1) + 2 * (j & 1); }
+    static constexpr int step_group(int m) { return 16 * (m >> 2) + 4 * ((m >> 1) & 1) + (m & 1); }
     template <int M>
     __device__ __forceinline__ f16x8 operand() const {
         constexpr int kPiece = M >> 2, kHigh = (M >> 1) & 1, kWord = 2 * (M & 1);
@@ -191,11 +190,12 @@ struct PackedBlock<kEncQ5K> {
     u32x4 header, fifth, piece[2];
     KBlockScales scales[2];
     int fifth_shift;  // sub-block of the first piece's low nibbles
-    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
-        header = *reinterpret_cast<const u32x4*>(block);
-        fifth = *reinterpret_cast<const u32x4*>(block + 16 + 16 * (j & 1));
-        piece[0] = *reinterpret_cast<const u32x4*>(block + 48 + 16 * j);
-        piece[1] = *reinterpret_cast<const u32x4*>(block + 48 + 64 + 16 * j);
+    __device__ __forceinline__ void load(GlobalBytes block, std::uint32_t row, int j) {
+        header = *reinterpret_cast<GlobalVec>(block + row);
+        fifth = *reinterpret_cast<GlobalVec>(block + (row + 16 + 16 * (j & 1)));
+        const std::uint32_t mine = row + 48 + 16 * j;
+        piece[0] = *reinterpret_cast<GlobalVec>(block + mine);
+        piece[1] = *reinterpret_cast<GlobalVec>(block + mine + 64);
     }
     __device__ __forceinline__ void prepare(int j) {
         scales[0].bits(header, j >> 1);
@@ -204,9 +204,8 @@ struct PackedBlock<kEncQ5K> {
         scales[1].scales(header);
         fifth_shift = 2 * (j >> 1);
     }
-    __device__ __forceinline__ static int group(int m, int j) {
-        return PackedBlock<kEncQ4K>::group(m, j);
-    }
+    __device__ __forceinline__ static int lane_group(int j) { return PackedBlock<kEncQ4K>::lane_group(j); }
+    static constexpr int step_group(int m) { return PackedBlock<kEncQ4K>::step_group(m); }
     template <int M>
     __device__ __forceinline__ f16x8 operand() const {
         constexpr int kPiece = M >> 2, kHigh = (M >> 1) & 1, kWord = 2 * (M & 1);
@@ -237,18 +236,25 @@ struct PackedBlock<kEncQ6K> {
     std::uint32_t sub_scales[2];  // the eight of this lane's half
     std::uint32_t d_bits;
     f16x2 scale[4];  // per quarter
-    __device__ __forceinline__ void load(const std::uint8_t* block, int j) {
+    __device__ __forceinline__ void load(GlobalBytes block, std::uint32_t row, int j) {
         const int n = j >> 1, h = j & 1;
-        const Chunk16 a = *reinterpret_cast<const Chunk16*>(block + 64 * n + 16 * h);
-        const Chunk16 b = *reinterpret_cast<const Chunk16*>(block + 64 * n + 32 + 16 * h);
-        const Chunk16 t = *reinterpret_cast<const Chunk16*>(block + 128 + 32 * n + 16 * h);
-        const Chunk8 s = *reinterpret_cast<const Chunk8*>(block + 192 + 8 * n);
-        low_a = u32x4{a.v[0], a.v[1], a.v[2], a.v[3]};
-        low_b = u32x4{b.v[0], b.v[1], b.v[2], b.v[3]};
-        top = u32x4{t.v[0], t.v[1], t.v[2], t.v[3]};
-        sub_scales[0] = s.v[0];
-        sub_scales[1] = s.v[1];
-        d_bits = *reinterpret_cast<const std::uint16_t*>(block + 208);
+        // the block is 210 bytes long: its parts are aligned to two bytes only
+        typedef std::uint32_t Words4 __attribute__((ext_vector_type(4), aligned(2)));
+        typedef std::uint32_t Words2 __attribute__((ext_vector_type(2), aligned(2)));
+        typedef const __attribute__((address_space(1))) Words4* GlobalWords4;
+        typedef const __attribute__((address_space(1))) Words2* GlobalWords2;
+        typedef const __attribute__((address_space(1))) std::uint16_t* GlobalHalf;
+        const std::uint32_t low = row + 64 * n + 16 * h;
+        const Words4 a = *reinterpret_cast<GlobalWords4>(block + low);
+        const Words4 b = *reinterpret_cast<GlobalWords4>(block + low + 32);
+        const Words4 t = *reinterpret_cast<GlobalWords4>(block + (row + 128 + 32 * n + 16 * h));
+        const Words2 s = *reinterpret_cast<GlobalWords2>(block + (row + 192 + 8 * n));
+        low_a = u32x4{a[0], a[1], a[2], a[3]};
+        low_b = u32x4{b[0], b[1], b[2], b[3]};
+        top = u32x4{t[0], t[1], t[2], t[3]};
+        sub_scales[0] = s[0];
+        sub_scales[1] = s[1];
+        d_bits = *reinterpret_cast<GlobalHalf>(block + (row + 208));
     }
     __device__ __forceinline__ void prepare(int j) {
         const float d = half_bits_to_float(d_bits);
@@ -261,9 +267,8 @@ struct PackedBlock<kEncQ6K> {
             scale[q] = splat(d * static_cast<float>(value));
         }
     }
-    __device__ __forceinline__ static int group(int m, int j) {
-        return 16 * (j >> 1) + 4 * (m >> 1) + 2 * (j & 1) + (m & 1);
-    }
+    __device__ __forceinline__ static int lane_group(int j) { return 16 * (j >> 1) + 2 * (j & 1); }
+    static constexpr int step_group(int m) { return 4 * (m >> 1) + (m & 1); }
     template <int M>
     __device__ __forceinline__ f16x8 operand() const {
         constexpr int kQuarter = M >> 1, kWord = 2 * (M & 1);
@@ -293,26 +298,21 @@ __device__ __forceinline__ Projection tile_projection(const ProjectionSet& set, 
     return pick(set, which);
 }
 
-// What a wave keeps of one step in flight: the packed weights, and, when the
-// activations stream with them, the eight operand fragments of the block.
-template <std::uint32_t ENC, bool RESIDENT>
-struct Stage {
-    PackedBlock<ENC> weights;
-    f16x8 activations[RESIDENT ? 1 : 8];
-};
+constexpr int kGroupTiles = 2;  // tiles a workgroup accumulates side by side
 
-// RESIDENT: rows of up to 8,192 columns.  A wave's K range is at most four
-// blocks, whose activation fragments it loads once and keeps in registers for
-// all its tiles (128 registers); a tile is four steps, step s of every tile
-// uses stage s and fragment set s, and only packed weights stream.
-// Otherwise: the fragments of a block are loaded again with its weights for
-// every tile.
-template <std::uint32_t ENC, bool RESIDENT>
+// A workgroup takes its tiles in groups of up to kGroupTiles and K in chunks of
+// 8 x kDepth blocks.  Per (group, chunk) a wave loads the activation fragments
+// of its share of the chunk (at most kDepth blocks) once, into registers, and
+// walks the group's tiles: step s of every tile uses fragment set s and stage
+// s, so only packed weights stream, kDepth steps (one tile) ahead.  Rows of up
+// to 8,192 columns are one chunk: the fragments are loaded once per launch.
+// After the last chunk the eight waves' partial sums of the group meet in LDS.
+template <std::uint32_t ENC>
 __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const std::uint8_t* __restrict__ image, const float* __restrict__ inverse_scale, int tokens,
     std::uint32_t total_tiles, int input_dim, ProjectionSet set) {
     using Block = PackedBlock<ENC>;
-    __shared__ float partial[2 * kWaves * kWave * 4];
+    __shared__ float partial[2 * kGroupTiles * kWaves * kWave * 4];
 
     const int lane = threadIdx.x & 63;
     // the wave index is uniform; saying so keeps tile bookkeeping in scalar registers
@@ -323,135 +323,143 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const int begin = blocks * wave / kWaves;
     const int end = blocks * (wave + 1) / kWaves;
     const int count = end - begin;
-    // steps of a tile, the same for every wave (a wave whose K range is shorter idles in the last ones)
-    const int steps = RESIDENT ? kDepth : (blocks + kWaves - 1) / kWaves;
+    const int chunks = ((blocks + kWaves - 1) / kWaves + kDepth - 1) / kDepth;  // the same for every wave
 
-    // This lane's 16 bytes of the group g of eight columns: image + (g * tokens + i) * 16.
+    // The 16 bytes of group g of eight columns for token i: image + (g * tokens + i) * 16, as
+    // a uniform part (block and instruction) and this lane's part (its quarter and token).
     // Lanes past the last token read token 0 again: a row of A only reaches its own row of
     // the result, and those rows are never stored.
-    const std::uint8_t* lane_image = image + (i < tokens ? i : 0) * 16;
-    const std::int64_t group_bytes = static_cast<std::int64_t>(tokens) * 16;
-    std::uint32_t group_offset[8];  // of instruction m's group inside a block
+    const GlobalBytes global_image = (GlobalBytes)image;
+    const std::uint32_t group_bytes = static_cast<std::uint32_t>(tokens) * 16;
+    const std::uint32_t lane_fragment =
+        static_cast<std::uint32_t>(Block::lane_group(j)) * group_bytes + (i < tokens ? i : 0) * 16;
+    f16x8 fragments[kDepth][8];
+    auto load_fragments = [&](int chunk) {
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-        group_offset[m] = static_cast<std::uint32_t>(Block::group(m, j)) * static_cast<std::uint32_t>(group_bytes);
-    }
-    auto load_fragments = [&](int block, f16x8 (&fragments)[8]) {
-        const std::uint8_t* block_image = lane_image + static_cast<std::int64_t>(block) * 32 * group_bytes;
+        for (int s = 0; s < kDepth; ++s) {
+            const int block = begin + max(min(chunk * kDepth + s, count - 1), 0);
+            const GlobalBytes block_image = global_image + static_cast<std::int64_t>(block) * 32 * group_bytes;
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            fragments[m] = *reinterpret_cast<const f16x8*>(block_image + group_offset[m]);
+            for (int m = 0; m < 8; ++m) {
+                fragments[s][m] = *reinterpret_cast<GlobalFragment>(
+                    block_image + Block::step_group(m) * group_bytes + lane_fragment);
+            }
         }
     };
-    f16x8 resident[RESIDENT ? kDepth : 1][8];
-    if constexpr (RESIDENT) {
-#pragma unroll
-        for (int s = 0; s < kDepth; ++s) load_fragments(begin + max(min(s, count - 1), 0), resident[s]);
-    }
 
     // register r of quarter j of the result: token 4j + r
     float token_scale[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) token_scale[r] = inverse_scale[min(4 * j + r, tokens - 1)];
 
-    const std::uint32_t first_tile = blockIdx.x;
-    const int tile_count = static_cast<int>((total_tiles - first_tile + gridDim.x - 1) / gridDim.x);
-    const int total = tile_count * steps;
+    // this workgroup's tiles: blockIdx.x + n * gridDim.x
+    const int tile_count =
+        static_cast<int>((total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x);
+    const int groups = (tile_count + kGroupTiles - 1) / kGroupTiles;
 
-    // Every wave walks the same flat stream of (tile, step) pairs, so the waves
-    // meet at the end of a tile in uniform control flow.  Loads run kDepth steps
-    // ahead; they are unconditional (a step without work reads the first bytes
-    // of the first projection, one line for the whole wave), so a step waits
-    // for nothing but its own.
-    std::uint32_t fetch_tile = first_tile;
-    int fetch_step = 0;
+    // Every wave walks the same stream of (group, chunk, tile of the group, step)
+    // in uniform control flow (a group's tiles: kGroupTiles, fewer in the last group).  Weight loads run kDepth steps ahead; they are
+    // unconditional (a step without work reads the first bytes of the first
+    // projection, one line for the whole wave), so a step waits for nothing but
+    // its own.  The fetch cursor walks the same stream, one tile ahead.
+    int fetch_group = 0, fetch_chunk = 0, fetch_slot = 0;
+    GlobalBytes fetch_tile = nullptr;  // first row of the tile being fetched (uniform)
+    std::uint32_t fetch_row = 0;       // this lane's row of it, in bytes
     bool fetch_live = true;
-    const std::uint8_t* fetch_row = nullptr;
     auto fetch_setup = [&]() {
-        const Projection op = tile_projection(set, fetch_tile);
-        const std::int64_t row0 = static_cast<std::int64_t>(fetch_tile - op.first_tile) * kTileRows;
-        const std::int64_t last = op.output_dim - 1 - row0;  // rows past the end repeat the last one
-        fetch_row = op.data + (row0 + min(static_cast<std::int64_t>(i), last)) * op.row_stride;
+        const int index = fetch_group * kGroupTiles + fetch_slot;
+        fetch_live = fetch_group < groups && index < tile_count;
+        const std::uint32_t tile = blockIdx.x + static_cast<std::uint32_t>(fetch_live ? index : 0) * gridDim.x;
+        const Projection op = tile_projection(set, tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
+        const int last = static_cast<int>(min(static_cast<std::int64_t>(kTileRows - 1), op.output_dim - 1 - row0));
+        fetch_tile = (GlobalBytes)op.data + row0 * op.row_stride;
+        fetch_row = static_cast<std::uint32_t>(min(i, last)) * static_cast<std::uint32_t>(op.row_stride);  // rows past the end repeat the last one
+    };
+    auto fetch_advance = [&]() {  // to the next (group, chunk, tile of the group)
+        if (++fetch_slot >= min(kGroupTiles, tile_count - fetch_group * kGroupTiles)) {
+            fetch_slot = 0;
+            if (++fetch_chunk == chunks) {
+                fetch_chunk = 0;
+                ++fetch_group;
+            }
+        }
+        fetch_setup();
     };
     fetch_setup();
-    auto fetch = [&](Stage<ENC, RESIDENT>& stage) {
-        const bool work = fetch_live && fetch_step < count;
-        const int block = begin + max(min(fetch_step, count - 1), 0);
-        const std::uint8_t* source =
-            work ? fetch_row + static_cast<std::int64_t>(block) * Block::kBytes : set.op[0].data;
-        stage.weights.load(source, work ? j : 0);
-        if constexpr (!RESIDENT) load_fragments(work ? block : 0, stage.activations);
-        if (++fetch_step == steps) {
-            fetch_step = 0;
-            if (fetch_tile + gridDim.x < total_tiles) {
-                fetch_tile += gridDim.x;
-                fetch_setup();
-            } else {
-                fetch_live = false;  // stream exhausted
-            }
-        }
+    auto fetch = [&](PackedBlock<ENC>& stage, int s) {
+        const int local = fetch_chunk * kDepth + s;  // block of this wave's K range
+        const bool work = fetch_live && local < count;
+        const GlobalBytes source = work
+            ? fetch_tile + static_cast<std::int64_t>(begin + local) * Block::kBytes : (GlobalBytes)set.op[0].data;
+        stage.load(source, work ? fetch_row : 0u, work ? j : 0);
     };
-    Stage<ENC, RESIDENT> stages[kDepth];
+    PackedBlock<ENC> stages[kDepth];
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) fetch(stages[d]);
+    for (int s = 0; s < kDepth; ++s) fetch(stages[s], s);
+    fetch_advance();
 
-    std::uint32_t tile = first_tile;
-    int work_step = 0;
-    int parity = 0;
-    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-
-    auto step = [&](Stage<ENC, RESIDENT>& stage, const f16x8 (&a)[8], int position) {
-        if (position < total) {
-            if (work_step < count) {
-                stage.weights.prepare(j);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[0], stage.weights.template operand<0>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[1], stage.weights.template operand<1>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2], stage.weights.template operand<2>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[3], stage.weights.template operand<3>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[4], stage.weights.template operand<4>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[5], stage.weights.template operand<5>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[6], stage.weights.template operand<6>(), acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], stage.weights.template operand<7>(), acc, 0, 0, 0);
-            }
-            if (++work_step == steps) {
-                // Cross-wave sum in wave order; the two buffers alternate so one
-                // barrier per tile is enough.
-                float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * 4;
-                *reinterpret_cast<f32x4*>(mine) = acc;
-                __syncthreads();
-                if (wave == (parity ? kWaves - 1 : 0)) {
-                    const Projection op = tile_projection(set, tile);
-                    const std::int64_t row = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows + i;
-                    f32x4 sum = *reinterpret_cast<const f32x4*>(partial + ((parity * kWaves + 0) * kWave + lane) * 4);
+    for (int group = 0; group < groups; ++group) {
+        f32x4 acc[kGroupTiles];
 #pragma unroll
-                    for (int w = 1; w < kWaves; ++w) {
-                        sum += *reinterpret_cast<const f32x4*>(partial + ((parity * kWaves + w) * kWave + lane) * 4);
-                    }
+        for (int t = 0; t < kGroupTiles; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        const int group_tiles = min(kGroupTiles, tile_count - group * kGroupTiles);
+        for (int chunk = 0; chunk < chunks; ++chunk) {
+            if (chunks > 1 || group == 0) load_fragments(chunk);
+            const int chunk_count = min(kDepth, count - chunk * kDepth);  // this wave's blocks of the chunk
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int token = 4 * j + r;
-                        if (token < tokens && row < op.output_dim) {
-                            op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
-                                sum[r] * token_scale[r];
-                        }
+            for (int t = 0; t < kGroupTiles; ++t) {
+                if (t >= group_tiles) break;
+#pragma unroll
+                for (int s = 0; s < kDepth; ++s) {
+                    PackedBlock<ENC>& stage = stages[s];
+                    if (s < chunk_count) {
+                        const f16x8 (&a)[8] = fragments[s];
+                        stage.prepare(j);
+                        f32x4 sum = acc[t];
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[0], stage.template operand<0>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[1], stage.template operand<1>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2], stage.template operand<2>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[3], stage.template operand<3>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[4], stage.template operand<4>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[5], stage.template operand<5>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[6], stage.template operand<6>(), sum, 0, 0, 0);
+                        sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], stage.template operand<7>(), sum, 0, 0, 0);
+                        acc[t] = sum;
                     }
+                    fetch(stage, s);
                 }
-                parity ^= 1;
-                work_step = 0;
-                tile += gridDim.x;
-                acc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                fetch_advance();
             }
         }
-        fetch(stage);
-    };
-
-    for (int position = 0; position < total; position += kDepth) {
+        // Cross-wave sums in wave order, wave t adds up tile t of the group; the
+        // two buffers alternate so one barrier per group is enough.
+        float* buffer = partial + (group & 1) * kGroupTiles * kWaves * kWave * 4;
 #pragma unroll
-        for (int d = 0; d < kDepth; ++d) {
-            if constexpr (RESIDENT) {
-                step(stages[d], resident[d], position + d);
-            } else {
-                step(stages[d], stages[d].activations, position + d);
+        for (int t = 0; t < kGroupTiles; ++t) {
+            if (t < group_tiles) {
+                *reinterpret_cast<f32x4*>(buffer + ((t * kWaves + wave) * kWave + lane) * 4) = acc[t];
+            }
+        }
+        __syncthreads();
+        if (wave < group_tiles) {
+            const float* mine = buffer + wave * kWaves * kWave * 4;
+            const std::uint32_t tile =
+                blockIdx.x + static_cast<std::uint32_t>(group * kGroupTiles + wave) * gridDim.x;
+            const Projection op = tile_projection(set, tile);
+            const std::int64_t row = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows + i;
+            f32x4 sum = *reinterpret_cast<const f32x4*>(mine + lane * 4);
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                sum += *reinterpret_cast<const f32x4*>(mine + (w * kWave + lane) * 4);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int token = 4 * j + r;
+                if (token < tokens && row < op.output_dim) {
+                    op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
+                        sum[r] * token_scale[r];
+                }
             }
         }
     }
@@ -468,13 +476,8 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* 
     // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
     const std::uint32_t slots = static_cast<std::uint32_t>(compute_units());
     const std::uint32_t grid = tiles < slots ? tiles : slots;
-    if ((set.input_dim >> 8) <= kWaves * kDepth) {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, true>), dim3(grid), dim3(kThreads), 0, stream, image,
-                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
-    } else {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, false>), dim3(grid), dim3(kThreads), 0, stream, image,
-                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
-    }
+    hipLaunchKernelGGL((gemv_f16_kernel<ENC>), dim3(grid), dim3(kThreads), 0, stream, image,
+                       inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
 }
 
 }  // namespace

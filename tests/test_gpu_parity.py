@@ -336,12 +336,13 @@ def test_small_batch_quantized_weights(cuda, oracle, encoding, rows):
 
 
 @pytest.mark.parametrize("rows", [5, 9, 16])
-@pytest.mark.parametrize("in_dim", [256, 2304, 8192, 8448])
+@pytest.mark.parametrize("in_dim", [256, 2304, 8192, 8448, 19968])
 def test_small_batch_half_kernel_shapes(cuda, oracle, in_dim, rows):
     """Five rows and more run on the fp16 matrix cores behind a conversion launch.  Row lengths:
     one block (seven of the eight waves of a workgroup have no K range), nine blocks (ranges
-    of one and two blocks), the longest row whose activation fragments stay in registers and
-    the first length past it.  Projections of 40, 8 and 19 rows: partial 16-row tiles and
+    of one and two blocks), the longest row that is one chunk of K (activation fragments loaded
+    once), the first length past it (two chunks, the second of one block for some waves) and
+    three chunks.  Projections of 40, 8 and 19 rows: partial 16-row tiles and
     tiles of different projections and formats in one call.  Activations of very different
     magnitude per row: every row carries its own power-of-two scale."""
     specs = [(kquant.Q4_K, 40), (kquant.Q5_K, 8), (kquant.Q6_K, 19), (kquant.Q4_K, 16)]
@@ -360,6 +361,25 @@ def test_small_batch_half_kernel_shapes(cuda, oracle, in_dim, rows):
     # a single projection alone gives the bits it gives inside the group
     alone = tile_ops.multi_linear(weights[2:3], to_device(x, cuda), workspace)[0]
     assert_bits_equal(alone, outputs[2], "single projection = its place in the group")
+
+
+@pytest.mark.parametrize("in_dim", [512, 8448])
+def test_small_batch_half_kernel_many_tiles(cuda, oracle, in_dim):
+    """More 16-row tiles than twice the compute units: workgroups take three tiles, in a group of
+    two and a group of one, and with two chunks of K they load their activation fragments
+    again for every (group, chunk)."""
+    rows = 7
+    units = torch_().cuda.get_device_properties(0).multi_processor_count
+    specs = [(kquant.Q4_K, 16 * 2 * units + 200), (kquant.Q6_K, 16 * units - 200 + 5)]
+    packed = [random_packed(e, n, in_dim, 95 + i) for i, (e, n) in enumerate(specs)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, p, n, in_dim) for (e, n), p in zip(specs, packed)]
+    x = kquant.synthetic_activations(96, rows, in_dim)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    for group in (weights[:1], weights):  # 2 x units + 13 tiles of one format, then both formats
+        outputs = tile_ops.multi_linear(group, to_device(x, cuda), workspace)
+        for (encoding, out_dim), p, y in zip(specs, packed, outputs):
+            expected = oracle.linear(encoding, p, out_dim, in_dim, x)
+            assert normalised_error(y.cpu().numpy(), expected) <= TOLERANCE
 
 
 @pytest.mark.parametrize("in_dim", [4096, 8192, 8448, 16384])
