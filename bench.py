@@ -446,7 +446,7 @@ def decode_batch_extra(layers, device, stream, steps: int, warmup: int, headline
     import torch
 
     result = {"workload": "decode attention projections as the headline, other batch sizes, HIP-graph replay"}
-    for rows in (1, 4, 8):
+    for rows in (1, 4, 8, 16):
         if rows == headline_rows:
             continue
         step = DecodeStep(layers, rows, device)
@@ -523,6 +523,16 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
                     "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
                     "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS[name], 4),
                     "tokens/s": round(rows / ms * 1e3, 1)}
+    # The same gate projection at M = 512 through the generic v1 call, which has no workspace
+    # argument and therefore runs the float kernel (fp32 activations against weights
+    # dequantized to fp32 in registers): the only v1 call that takes more than 16 rows.
+    rows = 512
+    x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
+    ms = time_replays(lambda: tile_ops.linear(gate, x), 3, 1)
+    tflops = 2.0 * rows * MODEL_DIM * FFN_DIM / ms / 1e9
+    result["generic_v1_linear_float_kernel_gate_M512"] = {
+        "ms": round(ms, 4), "TFLOP/s": round(tflops, 2),
+        "x_workspace_gemm": round(ms / result["f16_gate_up_M512"]["ms"], 1)}
     # The shader clock while the largest shape runs, and the matrix-core peak at
     # that clock: 256 CUs x 4096 fp16 flop per cycle per CU.
     rows = 2048

@@ -75,7 +75,7 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // One or two rows, and the verifier entry points at any row count: the
     // vector-ALU kernels.  Otherwise 3 and 4 rows: the int8 matrix-core kernel,
     // which quantizes inside the kernel; 5..16 rows: the fp16 matrix-core kernel
-    // behind its conversion launch (Q8_0: its dot kernel at any row count).
+    // behind its conversion launch (Q8_0 below five rows: its dot kernel).
     // Encodings and widths without either: the float kernel.
     // (two rows are also faster on the dot kernels: they walk the token planes
     // against the same unpacked weights)
@@ -91,10 +91,10 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
             target = &dot;
         } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
             target = &dot6;
-        } else if (gemv_q8_supports(encoding, input_dim)) {
-            target = &dot8;  // Q8_0 has no matrix-core kernel: the dot kernel at any row count
-        } else if (rows >= kFirstHalfRows && gemv_f16_supports(encoding, input_dim)) {
+        } else if (rows >= kFirstHalfRows && !verifier && gemv_f16_supports(encoding, input_dim)) {
             target = &half;
+        } else if (gemv_q8_supports(encoding, input_dim)) {
+            target = &dot8;  // Q8_0 below five rows and in the verifier family: its dot kernel
         } else if (rows >= 2 && gemv_mfma_supports(encoding, input_dim)) {
             target = &matrix;
         }

@@ -288,6 +288,60 @@ struct PackedBlock<kEncQ6K> {
     }
 };
 
+// Q8_0: eight 34-byte blocks (fp16 scale, 32 int8 codes) per 256 values.  Quarter j takes
+// blocks 2j and 2j + 1; instruction M uses codes 8*(M%4)..+7 of block 2j + M/4.
+template <>
+struct PackedBlock<kEncQ8_0> {
+    static constexpr int kBytes = 272;
+    std::uint32_t codes[2][8];
+    std::uint32_t d_bits[2];
+    f16x2 scale[2];
+    __device__ __forceinline__ void load(GlobalBytes block, std::uint32_t row, int j) {
+        // The quarter's two blocks are 68 bytes = 17 aligned words: the first block's codes
+        // start in the middle of word 0 and are shifted into place, the second block's
+        // scale is the upper half of word 8 and its codes are words 9..16.
+        typedef const __attribute__((address_space(1))) std::uint32_t* GlobalWord;
+        const std::uint32_t mine = row + 68 * j;
+        std::uint32_t word[17];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const u32x4 four = *reinterpret_cast<GlobalVec>(block + (mine + 16 * q));
+            word[4 * q] = four[0];
+            word[4 * q + 1] = four[1];
+            word[4 * q + 2] = four[2];
+            word[4 * q + 3] = four[3];
+        }
+        word[16] = *reinterpret_cast<GlobalWord>(block + (mine + 64));
+        d_bits[0] = word[0] & 0xffffu;
+        d_bits[1] = word[8] >> 16;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            codes[0][w] = __builtin_amdgcn_alignbit(word[w + 1], word[w], 16);
+            codes[1][w] = word[9 + w];
+        }
+    }
+    __device__ __forceinline__ void prepare(int) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const _Float16 d = __builtin_bit_cast(_Float16, static_cast<std::uint16_t>(d_bits[b]));
+            scale[b] = f16x2{d, d};
+        }
+    }
+    __device__ __forceinline__ static int lane_group(int j) { return 8 * j; }
+    static constexpr int step_group(int m) { return m; }
+    template <int M>
+    __device__ __forceinline__ f16x8 operand() const {
+        constexpr int kBlock = M >> 2, kWord = 2 * (M & 3);
+        std::uint32_t out[4];
+        // flipping the sign bit turns the int8 code q into the byte q + 128: bias 1024 + 128
+        scale_bytes(codes[kBlock][kWord] ^ 0x80808080u, splat(-1152.0f), scale[kBlock], splat(0.0f),
+                    out[0], out[1]);
+        scale_bytes(codes[kBlock][kWord + 1] ^ 0x80808080u, splat(-1152.0f), scale[kBlock],
+                    splat(0.0f), out[2], out[3]);
+        return as_operand(out[0], out[1], out[2], out[3]);
+    }
+};
+
 // Projection a tile belongs to.
 __device__ __forceinline__ Projection tile_projection(const ProjectionSet& set, std::uint32_t tile) {
     int which = 0;
@@ -483,7 +537,8 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* 
 }  // namespace
 
 bool gemv_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
-    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K) &&
+    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K ||
+            encoding == kEncQ8_0) &&
         input_dim % 256 == 0 && input_dim <= 65536;
 }
 
@@ -513,7 +568,7 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
             break;
     }
     // one launch per encoding present
-    const std::uint32_t encodings[3] = {kEncQ4K, kEncQ5K, kEncQ6K};
+    const std::uint32_t encodings[4] = {kEncQ4K, kEncQ5K, kEncQ6K, kEncQ8_0};
     for (const std::uint32_t encoding : encodings) {
         ProjectionSet group{};
         group.input_dim = set.input_dim;
@@ -525,8 +580,10 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
             launch_encoding<kEncQ4K>(group, image, inverse_scale, tokens, stream);
         } else if (encoding == kEncQ5K) {
             launch_encoding<kEncQ5K>(group, image, inverse_scale, tokens, stream);
-        } else {
+        } else if (encoding == kEncQ6K) {
             launch_encoding<kEncQ6K>(group, image, inverse_scale, tokens, stream);
+        } else {
+            launch_encoding<kEncQ8_0>(group, image, inverse_scale, tokens, stream);
         }
     }
 }

@@ -345,7 +345,7 @@ def test_small_batch_half_kernel_shapes(cuda, oracle, in_dim, rows):
     three chunks.  Projections of 40, 8 and 19 rows: partial 16-row tiles and
     tiles of different projections and formats in one call.  Activations of very different
     magnitude per row: every row carries its own power-of-two scale."""
-    specs = [(kquant.Q4_K, 40), (kquant.Q5_K, 8), (kquant.Q6_K, 19), (kquant.Q4_K, 16)]
+    specs = [(kquant.Q4_K, 40), (kquant.Q5_K, 8), (kquant.Q6_K, 19), (kquant.Q8_0, 24)]
     packed = [random_packed(e, n, in_dim, 90 + i) for i, (e, n) in enumerate(specs)]
     weights = [tile_ops.PackedWeight.from_numpy(e, p, n, in_dim) for (e, n), p in zip(specs, packed)]
     x = kquant.synthetic_activations(91 + rows, rows, in_dim)
