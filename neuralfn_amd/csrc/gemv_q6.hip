@@ -357,9 +357,9 @@ __global__ __launch_bounds__(kThreads) void gemv_q6_kernel(
 // LDS staging area instead: per pass 16 blocks, read as 224 consecutive 16-byte
 // pieces (four load instructions whose lanes touch neighbouring bytes) and
 // written to 224-byte slots, one per block, so that every piece of a block is
-// 16-byte aligned in LDS.  Piece 13 of a block is read from byte 194, not 208,
-// so that no load reaches past the block; it lands at slot offset 208 and puts
-// d at slot offset 222.  The 64 lanes then read one unit each from the slots
+// 16-byte aligned in LDS.  Piece 13 of a block holds the block's last 16 bytes
+// (bytes 194..209, not 208..223, so that no load reaches past the block); it
+// lands at slot offset 208 and puts d at slot offset 222.  The 64 lanes then read one unit each from the slots
 // and run the same arithmetic as above.  Nothing but the first barrier (for
 // the activation image) synchronises the workgroup; a wave's own LDS accesses
 // execute in order.
@@ -417,24 +417,60 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
         min(row_begin, op.output_dim - 1) * op.row_stride;
     const int stream_blocks = max(wave_blocks, 1);  // blocks that may be read from `stream`
 
+    // Blocks are 210 bytes long, so every other block of a tensor that starts on a
+    // four-byte boundary starts two bytes past one, and 16-byte loads that are not
+    // word aligned run at a fraction of the rate of aligned ones.  Loads 0 and 1
+    // of a pass fetch the eight blocks that start on a word (112 pieces, the last
+    // 16 lanes repeat the last one), loads 2 and 3 the eight that do not: their
+    // pieces are read from two bytes earlier and shifted into place with the first
+    // two bytes of the next piece, which the next lane holds.  Piece 13 of such a
+    // block is read from byte 194 (aligned; its bytes 12, 13 are what piece 12
+    // lacks); piece 13 of an aligned block from byte 196 (aligned; d moves from
+    // bytes 12, 13 to the place it has in a read from 194).  That read reaches two
+    // bytes into the next block, and a shifted read two bytes into the previous
+    // one: a pass that holds the last block of the tensor, or blocks that only
+    // stand in for ones past the wave's range, reads every piece the plain way.
+    // A tensor that does not start on a word is read the plain way throughout.
+    const bool realign = (reinterpret_cast<std::uintptr_t>(op.data) & 3u) == 0;
+    const int stream_parity =
+        static_cast<int>((reinterpret_cast<std::uintptr_t>(stream) >> 1) & 1u);
+    // the tensor's last block as a block of this wave's stream (beyond it for most waves)
+    const std::int64_t blocks_to_end =
+        (op.output_dim - min(row_begin, op.output_dim - 1)) * static_cast<std::int64_t>(blocks);
+    const int tensor_last_block =
+        static_cast<int>(min(blocks_to_end - 1, static_cast<std::int64_t>(0x7fffffff)));
+    static_assert(kPassBlocks % 2 == 0, "a block of a pass keeps its alignment from pass to pass");
+    // passes read the plain way: from plain_from on, and plain_also
+    const int plain_from = realign ? stream_blocks / kPassBlocks : 0;
+    const int plain_also = tensor_last_block / kPassBlocks;
+
     // which piece of a pass each of this lane's four loads fetches: loop invariant
-    int source_offset[4], target_offset[4], piece_block[4];
+    constexpr int kHalfPieces = kPassPieces / 2;  // of the aligned blocks, of the others
+    // (source_offset: of the plain read; aligned_step: what the word-aligned read adds to it)
+    int source_offset[4], aligned_step[4], target_offset[4], piece_block[4];
+    bool last_piece0 = false, last_piece1 = false;  // loads k and k + 2 fetch the same piece of their blocks
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const int piece = min(k * kWave + lane, kPassPieces - 1);
-        const int block = piece / kPiecesPerBlock;
-        const int within = piece - block * kPiecesPerBlock;
+        const int piece = min((k & 1) * kWave + lane, kHalfPieces - 1);
+        const int pair = piece / kPiecesPerBlock;  // block pair of the pass
+        const int within = piece - pair * kPiecesPerBlock;
+        const int block = 2 * pair + ((k >> 1) ^ stream_parity);
         piece_block[k] = block;
         source_offset[k] = within == 13 ? 194 : within * 16;
+        aligned_step[k] = k < 2 ? (within == 13 ? 2 : 0) : (within == 13 ? 0 : -2);
         target_offset[k] = block * kSlotBytes + within * 16;
+        if (k == 0) last_piece0 = within == 13;
+        if (k == 1) last_piece1 = within == 13;
     }
     auto issue = [&](PassLoads& loads, int pass) {
+        const bool plain = pass >= plain_from || pass == plain_also;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             // blocks past the wave's range are read from its last block instead
             const int block = min(pass * kPassBlocks + piece_block[k], stream_blocks - 1);
             loads.piece[k] = *reinterpret_cast<const Unaligned16*>(
-                stream + static_cast<std::int64_t>(block) * kBlockBytes + source_offset[k]);
+                stream + static_cast<std::int64_t>(block) * kBlockBytes + source_offset[k] +
+                (plain ? 0 : aligned_step[k]));
         }
     };
 
@@ -506,11 +542,39 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
     auto consume = [&](const PassLoads& loads, int pass) {
         // stage: every lane writes its pieces (lanes 32..63 of the fourth load hold
         // duplicates of the last piece and write the same bytes to the same place)
+        if (pass >= plain_from || pass == plain_also) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            *reinterpret_cast<u32x4*>(staging + target_offset[k]) =
-                u32x4{loads.piece[k].v[0], loads.piece[k].v[1], loads.piece[k].v[2],
-                      loads.piece[k].v[3]};
+            for (int k = 0; k < 4; ++k) {
+                *reinterpret_cast<u32x4*>(staging + target_offset[k]) =
+                    u32x4{loads.piece[k].v[0], loads.piece[k].v[1], loads.piece[k].v[2],
+                          loads.piece[k].v[3]};
+            }
+        } else {
+            // aligned blocks: only d of piece 13 moves
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const std::uint32_t v3 = loads.piece[k].v[3];
+                *reinterpret_cast<u32x4*>(staging + target_offset[k]) =
+                    u32x4{loads.piece[k].v[0], loads.piece[k].v[1], loads.piece[k].v[2],
+                          (k == 0 ? last_piece0 : last_piece1) ? v3 << 16 : v3};
+            }
+            // the others: two bytes up, the last two from the next piece (piece 13 as read)
+            const std::uint32_t give2 = last_piece0 ? loads.piece[2].v[3] : loads.piece[2].v[0];
+            const std::uint32_t give3 = last_piece1 ? loads.piece[3].v[3] : loads.piece[3].v[0];
+#pragma unroll
+            for (int k = 2; k < 4; ++k) {
+                const std::uint32_t v0 = loads.piece[k].v[0], v1 = loads.piece[k].v[1];
+                const std::uint32_t v2 = loads.piece[k].v[2], v3 = loads.piece[k].v[3];
+                // the next piece's word: from the next lane, for lane 63 from lane 0 of the next load
+                const std::uint32_t wrapped = k == 2 ? __builtin_amdgcn_readfirstlane(give3) : 0u;
+                const std::uint32_t next = static_cast<std::uint32_t>(__builtin_amdgcn_update_dpp(
+                    static_cast<int>(wrapped), static_cast<int>(k == 2 ? give2 : give3),
+                    0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+                const std::uint32_t shift = (k == 2 ? last_piece0 : last_piece1) ? 0u : 16u;
+                *reinterpret_cast<u32x4*>(staging + target_offset[k]) =
+                    u32x4{__builtin_amdgcn_alignbit(v1, v0, shift), __builtin_amdgcn_alignbit(v2, v1, shift),
+                          __builtin_amdgcn_alignbit(v3, v2, shift), __builtin_amdgcn_alignbit(next, v3, shift)};
+            }
         }
         // read back this lane's unit
         UnitData data;

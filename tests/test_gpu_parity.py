@@ -491,7 +491,7 @@ def test_q8_0_one_token_and_verifier(cuda, oracle, shape):
 
 # ------------------------------------------------ Q6_K rows of 16 blocks and more (streaming kernel)
 
-@pytest.mark.parametrize("shape", [(777, 4096), (1301, 6656), (64, 8192)])
+@pytest.mark.parametrize("shape", [(777, 4096), (1301, 6656), (64, 8192), (33, 4352)])
 def test_q6_k_long_rows_one_token_and_verifier(cuda, oracle, shape):
     # row counts that leave partial passes and waves without rows; K of exactly
     # 16 blocks, of 26 (rows straddle passes) and of 32
@@ -508,6 +508,24 @@ def test_q6_k_long_rows_one_token_and_verifier(cuda, oracle, shape):
         assert_bits_equal(single, batched[row:row + 1], f"row {row}")
     one = tile_ops.multi_linear([weight], to_device(x[:1], cuda), workspace, family="mmq")[0]
     assert_bits_equal(one, batched[:1], "mmq at one row")
+
+
+def test_q6_k_long_rows_tensor_two_bytes_off_a_word(cuda, oracle):
+    """The streaming kernel reads word-aligned pieces when the tensor starts on a four-byte
+    boundary; a tensor that does not is read the plain way and gives the same bits."""
+    out_dim, in_dim = 33, 4352
+    packed = random_packed(kquant.Q6_K, out_dim, in_dim, 53)
+    aligned = tile_ops.PackedWeight.from_numpy(kquant.Q6_K, packed, out_dim, in_dim)
+    holder = torch_().empty(packed.size + 2, dtype=torch_().uint8, device=cuda)
+    holder[2:].copy_(torch_().from_numpy(packed.reshape(-1)))
+    shifted = tile_ops.PackedWeight(kquant.Q6_K, out_dim, in_dim, holder[2:])
+    assert shifted.data.data_ptr() % 4 == 2
+    x = kquant.synthetic_activations(54, 1, in_dim)
+    workspace = tile_ops.small_batch_workspace(1, in_dim)
+    a = tile_ops.mmvq_linear(aligned, to_device(x, cuda), workspace)
+    b = tile_ops.mmvq_linear(shifted, to_device(x, cuda), workspace)
+    assert normalised_error(a.cpu().numpy(), oracle.linear(kquant.Q6_K, packed, out_dim, in_dim, x)) <= TOLERANCE
+    assert_bits_equal(a, b, "aligned and shifted tensor")
 
 
 @pytest.mark.parametrize("rows", [1, 3])
