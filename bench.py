@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # WRITE_SIZE counters of a `--traffic-probe` run, each calibrated on a plain
 # copy of known size; the figures and commands are in
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_643_284}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_641_434}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
 CU_COUNT = 256
 F16_FLOP_PER_CYCLE_PER_CU = 4096   # 4 SIMDs x one 32x32x16 fp16 matrix instruction per 32 cycles
@@ -145,9 +145,31 @@ class DecodeStep:
         return 2 * len(self.calls)
 
 
-def time_replays(run, steps: int, warmup: int) -> float:
-    """Milliseconds per call of run(), measured with events on the current stream."""
+SETTLE_SECONDS = 0.08
+
+
+def settle(run) -> None:
+    """Untimed calls of run() for SETTLE_SECONDS before a measurement's warm-up.
+
+    The memory-side clocks take tens of milliseconds of load to reach their steady
+    state after the idle time of a host-side set-up: the same lm_head launch measured
+    249 us in the first 6 ms of load and 208 us from about 60 ms on.  A decode loop runs
+    in that steady state; the figures here are meant to be its figures.
+    """
     import torch
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    while time.perf_counter() - start < SETTLE_SECONDS:
+        for _ in range(8):
+            run()
+        torch.cuda.synchronize()
+
+
+def time_replays(run, steps: int, warmup: int) -> float:
+    """Milliseconds per call of run(), measured with events on the current stream
+    (after settle(): untimed calls until the clocks are steady, then `warmup` more)."""
+    import torch
+    settle(run)
     for _ in range(warmup):
         run()
     torch.cuda.synchronize()
