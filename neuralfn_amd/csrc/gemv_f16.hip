@@ -48,8 +48,8 @@ constexpr int kDepth = 4;  // blocks in flight per wave
 
 // ---- activations: fp32 -> row-scaled fp16, [column / 8][row][8] ----------------
 
-constexpr int kImageThreads = 256;
-constexpr int kImageHeld = 8;  // 8-column groups a thread keeps: rows of up to 16,384 columns are read once
+constexpr int kImageThreads = 1024;  // there are at most 16 rows: a large workgroup per row
+constexpr int kImageHeld = 2;  // 8-column groups a thread keeps: rows of up to 16,384 columns are read once
 
 __device__ __forceinline__ float largest_of(float4 x, float largest) {
     return fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
