@@ -8,8 +8,9 @@
 // the caller's small-batch workspace, so that the projection that follows can
 // skip its own quantization.
 //
-// One workgroup of 256 threads per row; rows of up to 8192 columns take the
-// register-resident kernel, wider ones the kernel that walks memory in batches.
+// One workgroup per row; rows of up to 8192 columns take the kernel whose loads
+// are all in flight at once (1024 threads), wider ones the 256-thread kernel that
+// walks memory in batches.
 // The float arithmetic follows the
 // reference kernel operation for operation
 // (neuralfn/csrc/tile_cuda/kernels.cu:2155-2243): thread t accumulates the
@@ -195,21 +196,48 @@ __device__ __forceinline__ float tree_total(float square_sum, float* partials) {
     return total;
 }
 
-// Rows of up to 8192 columns: a thread keeps its (at most 32) columns of every
-// operand in registers.  All loads of the kernel go out at its start; the
-// second normalisation needs no second pass over memory because the columns a
-// thread sums in the second reduction are the ones it produced in the first.
-// Same arithmetic, same order, same bits as the kernel above.
-constexpr int kOwned = 32;
+// Rows of up to 8192 columns: one workgroup of 1024 threads per row.  The sums
+// keep the 256-thread order above (sum t adds the squares of columns t, t + 256,
+// ... one after another, then the halving tree), but the loads are spread over
+// four threads per sum: thread (q, t) loads columns t + 256 * (q + 4k) of every
+// operand, eight per operand, so that all loads of the kernel are in flight at
+// once (one thread per sum would have 104 outstanding where the hardware counts
+// 63), hands its values to thread (0, t) through LDS for the ordered sum, and
+// does the element-wise arithmetic of its own columns.  The second
+// normalisation needs no second pass over memory.  Same arithmetic, same order,
+// same bits as the kernel above.
+constexpr int kOwned = 32;      // columns per sum
+constexpr int kLoaders = 4;     // threads that share the loads of a sum
+constexpr int kWideThreads = kRmsThreads * kLoaders;
+constexpr int kLoaded = kOwned / kLoaders;  // columns per thread
+
+// The halving tree over the 256 sums of threads (0, t), additions in the order of
+// tree_total: (p[t] + p[t+128]) + (p[t+64] + p[t+192]) is its first two levels,
+// the last six run inside the first wave.  Every thread of the workgroup calls it.
+__device__ __forceinline__ float tree_total_wide(float square_sum, float* partials) {
+    if (threadIdx.x < kRmsThreads) partials[threadIdx.x] = square_sum;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const float a = partials[threadIdx.x] + partials[threadIdx.x + 128];
+        const float b = partials[threadIdx.x + 64] + partials[threadIdx.x + 192];
+        float value = a + b;
+#pragma unroll
+        for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
+        if (threadIdx.x == 0) partials[kRmsThreads] = value;
+    }
+    __syncthreads();
+    return partials[kRmsThreads];
+}
 
 template <bool HANDOFF>
-__global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
+__global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     const float* __restrict__ input, NormWeight first_weight,
     const float* __restrict__ residual_input, float* __restrict__ hidden_output,
     NormWeight second_weight, float* __restrict__ normalized_output,
     float* __restrict__ residual_output, int width, float first_eps, float second_eps,
     std::uint8_t* __restrict__ records) {
-    __shared__ float partials[kRmsThreads];
+    __shared__ float partials[kRmsThreads + 1];
+    __shared__ float handed[kOwned * kRmsThreads];  // [k][t]: column t + 256 k
     extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF: the normalized row
     const std::int64_t row = blockIdx.x;
     const float* source = input + row * width;
@@ -217,12 +245,14 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
     float* hidden = hidden_output + row * width;
     float* captured = residual_output + row * width;
     float* normalized = normalized_output + row * width;
+    const int t = threadIdx.x & (kRmsThreads - 1);
+    const int q = threadIdx.x / kRmsThreads;
 
-    float value[kOwned], other[kOwned], first_scale[kOwned], second_scale[kOwned];
-    int clamped[kOwned];
+    float value[kLoaded], other[kLoaded], first_scale[kLoaded], second_scale[kLoaded];
+    int clamped[kLoaded];
 #pragma unroll
-    for (int i = 0; i < kOwned; ++i) {
-        const int column = threadIdx.x + i * kRmsThreads;
+    for (int i = 0; i < kLoaded; ++i) {
+        const int column = t + (q + kLoaders * i) * kRmsThreads;
         clamped[i] = min(column, width - 1);
         value[i] = column < width ? source[clamped[i]] : 0.0f;
         other[i] = residual[clamped[i]];
@@ -230,16 +260,28 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
     norm_scales(first_weight, clamped, first_scale);
     norm_scales(second_weight, clamped, second_scale);
 
-    float square_sum = 0.0f;
+    // sum t over its columns in order (a column past the end contributes fma(0, 0, sum) = sum)
+    auto ordered_sum = [&]() {
+        float square_sum = 0.0f;
+        if (q == 0) {
 #pragma unroll
-    for (int i = 0; i < kOwned; ++i) square_sum = fmaf(value[i], value[i], square_sum);
-    const float first_inverse =
-        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + first_eps);
+            for (int k = 0; k < kOwned; ++k) {
+                const float v = handed[k * kRmsThreads + t];
+                square_sum = fmaf(v, v, square_sum);
+            }
+        }
+        return square_sum;
+    };
 
-    square_sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kOwned; ++i) {
-        const int column = threadIdx.x + i * kRmsThreads;
+    for (int i = 0; i < kLoaded; ++i) handed[(q + kLoaders * i) * kRmsThreads + t] = value[i];
+    __syncthreads();
+    const float first_inverse =
+        1.0f / sqrtf(tree_total_wide(ordered_sum(), partials) / static_cast<float>(width) + first_eps);
+
+#pragma unroll
+    for (int i = 0; i < kLoaded; ++i) {
+        const int column = t + (q + kLoaders * i) * kRmsThreads;
         const float sum =
             __fadd_rn(__fmul_rn(__fmul_rn(value[i], first_inverse), first_scale[i]), other[i]);
         value[i] = column < width ? sum : 0.0f;
@@ -247,14 +289,16 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
             hidden[column] = sum;
             captured[column] = sum;
         }
-        square_sum = fmaf(value[i], value[i], square_sum);
+        // every sum has read its old values: tree_total_wide's barriers lie in between
+        handed[(q + kLoaders * i) * kRmsThreads + t] = value[i];
     }
+    __syncthreads();
     const float second_inverse =
-        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + second_eps);
+        1.0f / sqrtf(tree_total_wide(ordered_sum(), partials) / static_cast<float>(width) + second_eps);
 
 #pragma unroll
-    for (int i = 0; i < kOwned; ++i) {
-        const int column = threadIdx.x + i * kRmsThreads;
+    for (int i = 0; i < kLoaded; ++i) {
+        const int column = t + (q + kLoaders * i) * kRmsThreads;
         const float result = __fmul_rn(__fmul_rn(value[i], second_inverse), second_scale[i]);
         if (column < width) {
             normalized[column] = result;
@@ -267,7 +311,7 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_resident_kernel(
         // one wave per 256-value block: the quantizer of the decode kernels
         const int lane = threadIdx.x & 63;
         const int wave = threadIdx.x >> 6;
-        for (int block = wave; block < (width >> 8); block += kRmsThreads / kWave) {
+        for (int block = wave; block < (width >> 8); block += kWideThreads / kWave) {
             const float4 x = *reinterpret_cast<const float4*>(staged + block * 256 + lane * 4);
             store_record(records + static_cast<std::int64_t>(block) * kActRecord, lane,
                          encode_activations(x));
@@ -472,12 +516,12 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
     if (width <= kOwned * kRmsThreads) {
         const int columns = static_cast<int>(width);
         if (records != nullptr) {
-            hipLaunchKernelGGL((dual_rms_resident_kernel<true>), grid, dim3(kRmsThreads),
+            hipLaunchKernelGGL((dual_rms_resident_kernel<true>), grid, dim3(kWideThreads),
                                static_cast<std::size_t>(columns) * sizeof(float), stream, input,
                                first, residual_input, hidden_output, second, normalized_output,
                                residual_output, columns, first_eps, second_eps, records);
         } else {
-            hipLaunchKernelGGL((dual_rms_resident_kernel<false>), grid, dim3(kRmsThreads), 0, stream,
+            hipLaunchKernelGGL((dual_rms_resident_kernel<false>), grid, dim3(kWideThreads), 0, stream,
                                input, first, residual_input, hidden_output, second,
                                normalized_output, residual_output, columns, first_eps, second_eps,
                                records);
