@@ -293,7 +293,7 @@ struct DotCursor {
 // ITER > 0 (one token only): a row has exactly ITER 64-unit slices, and since a
 // lane's units are then the same in every row, their activation operands stay in
 // registers for the whole launch instead of being read from LDS per row.
-template <std::uint32_t ENC, int T, int P, int ITER>
+template <std::uint32_t ENC, int T, int P, int ITER, int STAGES>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const float* __restrict__ first, std::uint64_t data_a, std::uint64_t data_b,
     std::uint64_t data_c, int input_dim, int rows_per_group, int longer_groups, int bound1,
@@ -384,9 +384,21 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         }
         if (--fetch_left > 0) fetch.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     };
-    Stage<kQ5> stage0, stage1;
-    issue(stage0, 0);
-    issue(stage1, ITER == 2 ? 1 : 0);
+    // STAGES register stages.  Two are requested here; a third only once this wave's
+    // activations have arrived (below): weight requests that go out ahead of the activation
+    // loads of waves that start later delay those, and with them the barrier every wave
+    // waits at (three at the start: 6.0 us per launch of the headline workload; two: 6.0;
+    // this way 5.6).  Launches of more than one workgroup per compute unit are faster with
+    // two (a 16,384-row projection: 12.3 against 14.0 us).
+    // With ITER > 0 the slices of consecutive steps run 0, .., ITER - 1, 0, ..; the loop
+    // below is unrolled over the steps after which (stage, slice) repeats.
+    static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
+    constexpr int kStages = STAGES;
+    constexpr int kSlices = ITER > 0 ? ITER : 1;
+    constexpr int kPeriod = kStages % kSlices == 0 ? kStages : kStages * kSlices;
+    Stage<kQ5> stages[kStages];
+    issue(stages[0], 0);
+    issue(stages[1], 1 % kSlices);
 
     // (3) quantize; one barrier; after it the workgroup never synchronises again.
     // The first workgroup also leaves the records in the caller's workspace
@@ -416,6 +428,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_record(x, record);
     }
+    if constexpr (kStages == 3) issue(stages[2], 2 % kSlices);
     __syncthreads();
 
     UnitActivations held[ITER > 0 ? ITER : 1];
@@ -432,8 +445,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 
     DotCursor work;
     work.start(row_count > 0 ? row_begin : 0, stride, data_a, data_b, data_c, bound1, bound2, bound3);
-    // `slice`: for ITER > 0 the slice this stage always holds (stage s of a row of
-    // two slices holds slice s; rows of one slice use both stages for slice 0)
+    // `slice`: for ITER > 0 the slice of its row this step works on
     auto compute = [&](const Stage<kQ5>& stage, int slice) {
         const int iteration = work.iteration;
         const int raw_unit = iteration * kWave + lane;
@@ -466,11 +478,12 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         work.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     };
 
-    for (int n = 0; n < total; n += 2) {
-        compute(stage0, 0);
-        issue(stage0, 0);
-        if (n + 1 < total) compute(stage1, ITER == 2 ? 1 : 0);
-        issue(stage1, ITER == 2 ? 1 : 0);
+    for (int n = 0; n < total; n += kPeriod) {
+#pragma unroll
+        for (int k = 0; k < kPeriod; ++k) {
+            if (k == 0 || n + k < total) compute(stages[k % kStages], k % kSlices);
+            issue(stages[k % kStages], (k + kStages) % kSlices);
+        }
     }
 }
 
@@ -504,19 +517,36 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     };
     const std::int64_t slices = (4 * blocks + kWave - 1) / kWave;
     if constexpr (T == 1) {
+        // one workgroup per compute unit: three stages, the third requested late
+        const bool small = groups <= compute_units();
         if (slices == 1) {
-            allow_large_lds<gemv_dot_kernel<ENC, T, P, 1>>();
-            launch(gemv_dot_kernel<ENC, T, P, 1>);
+            if (small) {
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 3>>();
+                launch(gemv_dot_kernel<ENC, T, P, 1, 3>);
+            } else {
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 2>>();
+                launch(gemv_dot_kernel<ENC, T, P, 1, 2>);
+            }
             return;
         }
         if (slices == 2) {
-            allow_large_lds<gemv_dot_kernel<ENC, T, P, 2>>();
-            launch(gemv_dot_kernel<ENC, T, P, 2>);
+            if (small) {
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 3>>();
+                launch(gemv_dot_kernel<ENC, T, P, 2, 3>);
+            } else {
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 2>>();
+                launch(gemv_dot_kernel<ENC, T, P, 2, 2>);
+            }
+            return;
+        }
+        if (small) {
+            allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 3>>();
+            launch(gemv_dot_kernel<ENC, T, P, 0, 3>);
             return;
         }
     }
-    allow_large_lds<gemv_dot_kernel<ENC, T, P, 0>>();
-    launch(gemv_dot_kernel<ENC, T, P, 0>);
+    allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 2>>();
+    launch(gemv_dot_kernel<ENC, T, P, 0, 2>);
 }
 
 template <std::uint32_t ENC, int P>
