@@ -490,7 +490,6 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
     }
     PassLoads loads0, loads1;
     issue(loads0, 0);
-    issue(loads1, min(1, max(passes - 1, 0)));
 
     // (3) quantize; one barrier
     // (the first workgroup also leaves the records in the caller's workspace
@@ -519,6 +518,10 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_record(x, record);
     }
+    // the second pass's weights are requested only now: requests that go out ahead of the
+    // activation loads of waves that start later delay those, and every wave waits at
+    // the barrier for all activations
+    issue(loads1, min(1, max(passes - 1, 0)));
     __syncthreads();
 
     float acc_current[T], acc_next[T];

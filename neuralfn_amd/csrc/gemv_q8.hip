@@ -132,7 +132,6 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
     };
     Stage stage0, stage1;
     issue(stage0);
-    issue(stage1);
 
     // (3) quantize; one barrier
     // (the first workgroup also leaves the records in the caller's workspace
@@ -161,6 +160,10 @@ __global__ __launch_bounds__(kThreads) void gemv_q8_kernel(
             static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
         quantize_record(x, record);
     }
+    // the second stage's weights are requested only now: requests that go out ahead of the
+    // activation loads of waves that start later delay those, and every wave waits at
+    // the barrier for all activations
+    issue(stage1);
     __syncthreads();
 
     float acc[T];
