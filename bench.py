@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # copy of known size; the figures and commands are in
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_641_434}
-MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0, "f32": 157.3}
 CU_COUNT = 256
 F16_FLOP_PER_CYCLE_PER_CU = 4096   # 4 SIMDs x one 32x32x16 fp16 matrix instruction per 32 cycles
 MODEL_DIM, ATTN_DIM, KV_DIM = 6656, 4096, 256
@@ -545,15 +545,17 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
                     "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
                     "frac_mfma": round(tflops / MFMA_PEAK_TFLOPS[name], 4),
                     "tokens/s": round(rows / ms * 1e3, 1)}
-    # The same gate projection at M = 512 through the generic v1 call, which has no workspace
-    # argument and therefore runs the float kernel (fp32 activations against weights
-    # dequantized to fp32 in registers): the only v1 call that takes more than 16 rows.
+    # The same gate projection at M = 512 through the generic v1 call, the only v1 call that
+    # takes more than 16 rows.  It has no workspace argument, so it stays in the exact tier:
+    # float activations against weights decoded to float, on the float matrix instruction
+    # (256 flop per cycle and compute unit, a sixteenth of the fp16 one).
     rows = 512
     x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
-    ms = time_replays(lambda: tile_ops.linear(gate, x), 3, 1)
+    ms = time_replays(lambda: tile_ops.linear(gate, x), 5, 2)
     tflops = 2.0 * rows * MODEL_DIM * FFN_DIM / ms / 1e9
-    result["generic_v1_linear_float_kernel_gate_M512"] = {
+    result["generic_v1_linear_f32_matrix_cores_gate_M512"] = {
         "ms": round(ms, 4), "TFLOP/s": round(tflops, 2),
+        "frac_mfma_f32": round(tflops / MFMA_PEAK_TFLOPS["f32"], 4),
         "x_workspace_gemm": round(ms / result["f16_gate_up_M512"]["ms"], 1)}
     # The shader clock while the largest shape runs, and the matrix-core peak at
     # that clock: 256 CUs x 4096 fp16 flop per cycle per CU.

@@ -89,8 +89,9 @@ int nfn_native_tile_packed_weight_dequantize_float32_v1(
 
 /* ---- generic float-activation linear, any row count (tile_ops.h:614-620):
  *      float weights times float activations, no quantization of the input.
- *      It has no workspace argument, so large row counts take the same float
- *      kernel; nfn_mi355_k_quant_gemm_float32_v1 is the matrix-core route. -- */
+ *      It has no workspace argument, so every row count keeps that float
+ *      arithmetic (17 rows and more on the float matrix instruction);
+ *      nfn_mi355_k_quant_gemm_float32_v1 is the fp16 matrix-core route. -- */
 int nfn_native_tile_linear_packed_weight_float32_v1(
     const NfnNativeTilePackedWeightDescriptorV1* descriptor,
     const float* input,

@@ -12,6 +12,14 @@ void launch_dequantize(const Descriptor& descriptor, float* output, hipStream_t 
 void launch_gemv_f32(ProjectionSet set, const float* first, const float* second, int prologue,
                      const float* bias, std::int64_t rows, hipStream_t stream);
 
+// gemm_f32.hip — the same arithmetic on the float matrix cores, for many rows of one
+// projection: input_dim a multiple of 32.  gemm_f32_tile_passes: how many of its
+// 128 x 64 tiles a compute unit works through one after another (at least 1).
+bool gemm_f32_supports(const Descriptor& weight, std::int64_t rows);
+double gemm_f32_tile_passes(const Descriptor& weight, std::int64_t rows);
+void launch_gemm_f32(const Descriptor& weight, const float* input, const float* bias,
+                     float* output, std::int64_t rows, hipStream_t stream);
+
 // q8_1.hip — the public int8-activation path.
 void launch_quantize_q8_1(const float* input, std::int8_t* codes, float* scales, float* sums,
                           std::int64_t rows, std::int64_t width, hipStream_t stream);

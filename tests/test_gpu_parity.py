@@ -141,6 +141,40 @@ def test_generic_linear_against_oracle(cuda, oracle, encoding, rows):
     assert normalised_error(y, expected) <= TOLERANCE
 
 
+@pytest.mark.parametrize("encoding", ALL_PACKED + [kquant.F32, kquant.BF16])
+def test_generic_linear_many_rows_decodes_every_weight_exactly(cuda, oracle, encoding):
+    """More than 16 rows of the generic linear run on the float matrix cores.  One-hot input
+    rows make every output a single product with 1.0, so the result is the decoded weight
+    matrix itself and has to equal the dequantize entry point's bit for bit (all eight
+    sub-blocks of a K-quant block, both halves of every nibble, rows past the last tile)."""
+    out_dim, in_dim = 203, 768
+    if encoding in (kquant.F32, kquant.BF16):
+        packed = kquant.quantize(encoding, kquant.synthetic_weights(9, out_dim, in_dim, 1.0))
+    else:
+        packed = kquant.quantize(encoding, kquant.synthetic_weights(9 + encoding, out_dim, in_dim))
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    decoded = tile_ops.dequantize(weight).cpu().numpy()
+    assert np.array_equal(decoded, oracle.dequantize(encoding, packed, out_dim, in_dim))
+    x = np.eye(in_dim, dtype=np.float32)
+    bias = ((np.arange(out_dim) % 7 - 3) * 0.25).astype(np.float32)
+    y = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
+    assert np.array_equal(y, decoded.T)
+    y = tile_ops.linear(weight, to_device(x[:300] * 2.0, cuda), to_device(bias, cuda)).cpu().numpy()
+    assert np.array_equal(y, decoded.T[:300] * 2.0 + bias[None, :])
+
+
+@pytest.mark.parametrize("rows", [17, 128, 129, 300])
+@pytest.mark.parametrize("encoding", ALL_PACKED)
+def test_generic_linear_many_rows_against_oracle(cuda, oracle, encoding, rows):
+    out_dim, in_dim = 321, 2048
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(41 + encoding, out_dim, in_dim))
+    x = kquant.synthetic_activations(78 + rows, rows, in_dim)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    y = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    assert normalised_error(y, expected) <= 1e-5
+
+
 # ------------------------------------------------------------ public Q8_1 path
 
 def crafted_q8_input(rows, in_dim):

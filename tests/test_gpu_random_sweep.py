@@ -107,7 +107,7 @@ def test_gemm_random_case(cuda, oracle, seed):
         # (a row of a few outputs can cancel to nearly nothing, so only wide rows are asked)
         for row in range(rows):
             assert normalised_error(y[row], expected[row]) <= TOLERANCE, f"{label} row {row}"
-    # the generic linear has no workspace and stays on the float kernel at any row count
+    # the generic linear has no workspace: exact float arithmetic at any row count
     z = tile_ops.linear(weight, to_device(x, cuda)).cpu().numpy()
     for row in range(0, rows, 7):
         assert normalised_error(z[row], expected[row]) <= 1e-5, f"{label} row {row} (generic linear)"
