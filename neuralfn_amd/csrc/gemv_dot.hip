@@ -327,7 +327,8 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // that their short latency does not queue behind the weight loads.  All
     // loads are unconditional (clamped indices) to keep the load counters exact.
     const int records = pass_tokens * blocks;
-    constexpr int kEarly = 4;
+    // (rows of more than 8,192 columns: eight, i.e. every record of a 16,384-column row)
+    constexpr int kEarly = ITER > 0 ? 4 : 8;
     float4 early[kEarly];
 #pragma unroll
     for (int e = 0; e < kEarly; ++e) {
