@@ -327,6 +327,29 @@ def test_fused_prologue_equals_materialised(cuda, oracle, mixed, prologue, rows)
         assert_bits_equal(b, f, prologue)
 
 
+def test_elementwise_prologues_over_the_float_range(cuda, oracle):
+    """The sigmoid of the two element-wise operators (and of the fused prologues, which share
+    it) is built from the hardware's exp2 and reciprocal: 2e-6 of the oracle over twenty
+    decades of either sign, the saturated ends, zeros, infinities and NaN."""
+    rng = np.random.default_rng(5)
+    magnitudes = 10.0 ** rng.uniform(-20, 3, 4096)
+    gate = (magnitudes * rng.choice([-1.0, 1.0], 4096)).astype(np.float32)
+    special = np.array([0.0, -0.0, 86.9, -86.9, 87.0, -87.0, 88.4, -88.4, 88.8, -88.8, 104.0,
+                        -104.0, 1e30, -1e30, np.inf, -np.inf, np.nan, 1e-40, -1e-40],
+                       np.float32)
+    gate = np.concatenate([gate, special, np.linspace(-30, 30, 4096).astype(np.float32)])
+    other = rng.uniform(-3, 3, gate.size).astype(np.float32)
+    for name in ("sigmoid_gate", "swiglu"):
+        first, second = (other, gate) if name == "sigmoid_gate" else (gate, other)
+        got = getattr(tile_ops, name)(to_device(first[None, :], cuda),
+                                      to_device(second[None, :], cuda)).cpu().numpy()[0]
+        with np.errstate(all="ignore"):
+            want = getattr(oracle, name)(first[None, :], second[None, :])[0]
+        assert np.array_equal(np.isnan(got), np.isnan(want)), name
+        finite = ~np.isnan(want)
+        np.testing.assert_allclose(got[finite], want[finite], rtol=2e-6, atol=1e-35, err_msg=name)
+
+
 def test_small_batch_fails_closed_on_device(cuda, mixed):
     # probe :1834-1866 with real device buffers
     rows, in_dim = mixed["rows"], mixed["in_dim"]
