@@ -690,13 +690,17 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
             block = torch.from_numpy(kquant.synthetic_activations(42, rows, MODEL_DIM)).to(device)
             block_zeros = torch.zeros_like(block)
             block_workspace = tile_ops.small_batch_workspace(rows, FFN_DIM, device)
-            for name, attention_workspace, _ in forms:
+            # (the last form: the dual norms also hand their output to the projections behind
+            # them in the small-batch workspace, nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1)
+            block_forms = [(name, workspace, False) for name, workspace, _ in forms]
+            block_forms.append((forms[-1][0] + "_norm_handoff", forms[-1][1], True))
+            for name, attention_workspace, handoff in block_forms:
                 def verify():
                     pending, residual, pending_norm = block, block_zeros, None
                     for layer_weights, cache in zip(weights, caches):
                         pending, residual, _, _ = dl.verify_layer(
                             g, layer_weights, cache, pending, residual, pending_norm, position,
-                            block_workspace, True, attention_workspace)
+                            block_workspace, True, attention_workspace, handoff)
                         pending_norm = layer_weights.post_feedforward_norm
                     last["hidden"] = residual
 

@@ -335,6 +335,42 @@ int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
     void* mmvq_workspace,
     int64_t mmvq_workspace_nbytes,
     void* cuda_stream);
+/* The same handoff for a block of 5..16 rows (the verifier's block, a prefill
+ * chunk): the reference's pair (tile_ops.h:874-894 producer, :698-709 consumer)
+ * takes one row only, and at these row counts the small-batch entry points
+ * spend a launch per call on converting their input.  Here the norm kernel
+ * also leaves normalized_output in mmq_workspace in the form the
+ * nfn_native_tile_k_quant_mmq_* calls convert their input to, and
+ * nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1 multiplies from
+ * it: the same bits as the mmq call on normalized_output, one launch less per
+ * projection group.  width: a multiple of 256, at most 8192; the workspace at
+ * least nfn_native_tile_k_quant_mmq_workspace_bytes_v1(rows, width) bytes; the
+ * consumer fails closed unless every projection is Q4_K, Q5_K, Q6_K or Q8_0. */
+int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    void* mmq_workspace,
+    int64_t mmq_workspace_nbytes,
+    void* cuda_stream);
+int nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    float* const* outputs,
+    int64_t operation_count,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
 
 /* ---- row argmax, ties to the lowest column (tile_ops.h:757-764) --------- */
 int nfn_native_tile_argmax_rows_float32_v1(

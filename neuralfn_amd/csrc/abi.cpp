@@ -102,6 +102,8 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     }
     // Prequantized input: only the dot kernels read activation records.
     if (prologue == kRecords && (matrix.count > 0 || half.count > 0 || exact.count > 0)) return kInvalid;
+    // An fp16 image in the workspace: only the fp16 small-batch kernel reads one.
+    if (prologue == kHalfImage && half.count != set.count) return kInvalid;
     // In the verifier family the dot kernels leave their activation records in
     // the workspace, where a following prequantized call with the same input
     // finds them (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:3649-3666).
@@ -344,6 +346,17 @@ int nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1(
                            cuda_stream);
 }
 
+int nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1(
+    const Descriptor* const* descriptors, float* const* outputs, std::int64_t operation_count,
+    std::int64_t rows, void* workspace, std::int64_t workspace_nbytes, void* cuda_stream) {
+    // The workspace holds the fp16 image of `rows` rows, left there by
+    // nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1.
+    if (rows < 5) return kInvalid;
+    return run_small_batch(false, descriptors, static_cast<const float*>(workspace), nullptr,
+                           kHalfImage, outputs, operation_count, rows, workspace, workspace_nbytes,
+                           cuda_stream);
+}
+
 int nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1(
     const Descriptor* const* descriptors, const float* input, const float* gate,
     float* const* outputs, std::int64_t operation_count, std::int64_t rows, void* workspace,
@@ -491,7 +504,7 @@ int nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(
                                 residual_input, hidden_output,
                                 second_weight != nullptr ? &second : nullptr, second_centered,
                                 normalized_output, residual_output, rows, width, first_eps,
-                                second_eps, nullptr, as_stream(cuda_stream));
+                                second_eps, nullptr, nullptr, as_stream(cuda_stream));
     return launch_status();
 }
 
@@ -534,7 +547,34 @@ int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
                                 residual_input, hidden_output,
                                 second_weight != nullptr ? &second : nullptr, second_centered,
                                 normalized_output, residual_output, rows, width, first_eps,
-                                second_eps, static_cast<std::uint8_t*>(mmvq_workspace),
+                                second_eps, static_cast<std::uint8_t*>(mmvq_workspace), nullptr,
+                                as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t rows, std::int64_t width, float first_eps,
+    bool first_centered, float second_eps, bool second_centered, void* mmq_workspace,
+    std::int64_t mmq_workspace_nbytes, void* cuda_stream) {
+    Descriptor first{}, second{};
+    // Row counts that the small-batch entry points run on the fp16 kernel, rows that the
+    // register-resident norm kernel takes, a width that kernel reads.
+    const bool rows_fit = rows >= 5 && rows <= kMaxSmallRows;
+    const std::int64_t required = rows_fit ? small_batch_workspace_bytes(rows, width) : 0;
+    if (mmq_workspace == nullptr || !rows_fit || width % 256 != 0 || width > 8192 ||
+        required == 0 || mmq_workspace_nbytes < required ||
+        !dual_rms_arguments_valid(input, first_weight, residual_input, hidden_output,
+                                  second_weight, normalized_output, residual_output, rows, width,
+                                  first_eps, second_eps, &first, &second)) {
+        return kInvalid;
+    }
+    launch_dual_rms_add_capture(input, first_weight != nullptr ? &first : nullptr, first_centered,
+                                residual_input, hidden_output,
+                                second_weight != nullptr ? &second : nullptr, second_centered,
+                                normalized_output, residual_output, rows, width, first_eps,
+                                second_eps, nullptr, static_cast<std::uint8_t*>(mmq_workspace),
                                 as_stream(cuda_stream));
     return launch_status();
 }

@@ -118,8 +118,9 @@ struct ProjectionSet {
 // Activation prologues of the fused entry points (glimmer_k_mmq.cu:299-317).
 // kRecords is not a prologue of the floats: the input pointer holds activation
 // records that an earlier launch quantized (the prequantized entry point,
-// neuralfn/csrc/native_train/tile_ops.h:698-709).
-enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2, kRecords = 3 };
+// neuralfn/csrc/native_train/tile_ops.h:698-709).  kHalfImage likewise: the fp16 image of
+// the fp16 small-batch kernel already lies in the workspace (written by the dual RMS kernel).
+enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2, kRecords = 3, kHalfImage = 4 };
 
 #if defined(__HIPCC__)
 

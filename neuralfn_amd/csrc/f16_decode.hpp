@@ -38,6 +38,35 @@ __device__ __forceinline__ void scale_bytes(std::uint32_t word, f16x2 bias, f16x
     out1 = bits_of(__builtin_elementwise_fma(x1, scale, shift));
 }
 
+// The fp16 copy of a small batch of activation rows that the small-batch kernel reads
+// (gemv_f16.hip): [column / 8][row][8 halfs], every row scaled by a power of two so that its
+// largest magnitude lands near 2^14, and one float per row to multiply results back.
+struct HalfImageScale {
+    float factor, inverse;
+};
+// zero, subnormal-range and infinite maxima keep scale 1
+__device__ __forceinline__ HalfImageScale half_image_scale(float largest) {
+    const std::uint32_t exponent = (__float_as_uint(largest) >> 23) & 0xffu;
+    const bool usable = exponent >= 16u && exponent <= 254u;
+    HalfImageScale scale;
+    scale.factor = usable ? __uint_as_float((127u + 14u + 127u - exponent) << 23) : 1.0f;
+    scale.inverse = usable ? __uint_as_float((exponent - 14u) << 23) : 1.0f;
+    return scale;
+}
+__device__ __forceinline__ float largest_of(float4 x, float largest) {
+    return fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+}
+// columns 8 group .. 8 group + 7 of row `row` (a, then b) into the image of `rows` rows
+__device__ __forceinline__ void half_image_store(std::uint8_t* image, int group, int rows, int row,
+                                                 float4 a, float4 b, float factor) {
+    const f16x2 h0 = {static_cast<_Float16>(a.x * factor), static_cast<_Float16>(a.y * factor)};
+    const f16x2 h1 = {static_cast<_Float16>(a.z * factor), static_cast<_Float16>(a.w * factor)};
+    const f16x2 h2 = {static_cast<_Float16>(b.x * factor), static_cast<_Float16>(b.y * factor)};
+    const f16x2 h3 = {static_cast<_Float16>(b.z * factor), static_cast<_Float16>(b.w * factor)};
+    std::uint8_t* target = image + (static_cast<std::int64_t>(group) * rows + row) * 16;
+    *reinterpret_cast<u32x4*>(target) = u32x4{bits_of(h0), bits_of(h1), bits_of(h2), bits_of(h3)};
+}
+
 // Q4_K and Q5_K: d, dmin and the 6-bit scale/min pair of sub-blocks 2*pair, 2*pair+1
 // out of the block's first 16 bytes
 struct KBlockScales {

@@ -51,10 +51,6 @@ constexpr int kDepth = 4;  // blocks in flight per wave
 constexpr int kImageThreads = 1024;  // there are at most 16 rows: a large workgroup per row
 constexpr int kImageHeld = 2;  // 8-column groups a thread keeps: rows of up to 16,384 columns are read once
 
-__device__ __forceinline__ float largest_of(float4 x, float largest) {
-    return fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
-}
-
 // One workgroup per row.
 template <int P>
 __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
@@ -94,20 +90,10 @@ __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
     __syncthreads();
 #pragma unroll
     for (int w = 0; w < kImageThreads / kWave; ++w) largest = fmaxf(largest, maxima[w]);
-    // zero, subnormal-range, infinite maxima keep scale 1
-    const std::uint32_t exponent = (__float_as_uint(largest) >> 23) & 0xffu;
-    const bool usable = exponent >= 16u && exponent <= 254u;
-    const float factor = usable ? __uint_as_float((127u + 14u + 127u - exponent) << 23) : 1.0f;
-    if (threadIdx.x == 0) {
-        inverse_scale[token] = usable ? __uint_as_float((exponent - 14u) << 23) : 1.0f;
-    }
+    const HalfImageScale scale = half_image_scale(largest);
+    if (threadIdx.x == 0) inverse_scale[token] = scale.inverse;
     auto store = [&](int g, float4 a, float4 b) {
-        const f16x2 h0 = {static_cast<_Float16>(a.x * factor), static_cast<_Float16>(a.y * factor)};
-        const f16x2 h1 = {static_cast<_Float16>(a.z * factor), static_cast<_Float16>(a.w * factor)};
-        const f16x2 h2 = {static_cast<_Float16>(b.x * factor), static_cast<_Float16>(b.y * factor)};
-        const f16x2 h3 = {static_cast<_Float16>(b.z * factor), static_cast<_Float16>(b.w * factor)};
-        std::uint8_t* target = image + (static_cast<std::int64_t>(g) * tokens + token) * 16;
-        *reinterpret_cast<u32x4*>(target) = u32x4{bits_of(h0), bits_of(h1), bits_of(h2), bits_of(h3)};
+        half_image_store(image, g, tokens, token, a, b, scale.factor);
     };
     if (held) {
 #pragma unroll
@@ -554,6 +540,8 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
     const int input_dim = static_cast<int>(set.input_dim);
     const dim3 grid(static_cast<unsigned>(rows));
     switch (prologue) {
+        case kHalfImage:  // an earlier launch left the image in the workspace
+            break;
         case kGated:
             hipLaunchKernelGGL((f16_image_kernel<kGated>), grid, dim3(kImageThreads), 0, stream, first,
                                second, image, inverse_scale, tokens, input_dim);

@@ -12,7 +12,8 @@ bool gemv_f16_supports(std::uint32_t encoding, std::int64_t input_dim);
 std::int64_t gemv_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim);
 
 // rows 3..16: one launch converts the activations (with the prologue applied) into
-// `workspace`, then one launch per encoding present multiplies.
+// `workspace`, then one launch per encoding present multiplies.  Prologue kHalfImage: the
+// workspace already holds the converted rows and only the multiplying launches run.
 void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* second, int prologue,
                      std::int64_t rows, void* workspace, hipStream_t stream);
 

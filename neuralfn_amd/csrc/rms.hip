@@ -21,6 +21,7 @@
 // square root where the reference calls the device's approximate reciprocal
 // square root, so the two can differ in the last bits of that one factor.
 #include "common.hpp"
+#include "f16_decode.hpp"
 #include "kernels.hpp"
 #include "wave_rows.hpp"
 
@@ -229,7 +230,10 @@ __device__ __forceinline__ float tree_total_wide(float square_sum, float* partia
     return partials[kRmsThreads];
 }
 
-template <bool HANDOFF>
+// HANDOFF 0: nothing more; 1: the activation records of the normalized row (one row);
+// 2: the normalized rows as the fp16 image of the fp16 small-batch kernel, `records` being
+// the small-batch workspace of gridDim.x rows.
+template <int HANDOFF>
 __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     const float* __restrict__ input, NormWeight first_weight,
     const float* __restrict__ residual_input, float* __restrict__ hidden_output,
@@ -237,8 +241,9 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     float* __restrict__ residual_output, int width, float first_eps, float second_eps,
     std::uint8_t* __restrict__ records) {
     __shared__ float partials[kRmsThreads + 1];
-    __shared__ float handed[kOwned * kRmsThreads];  // [k][t]: column t + 256 k
-    extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF: the normalized row
+    __shared__ __attribute__((aligned(16))) float handed[kOwned * kRmsThreads];  // [k][t]: column t + 256 k
+    extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF 1: the normalized row
+    __shared__ float wave_largest[kWideThreads / kWave];
     const std::int64_t row = blockIdx.x;
     const float* source = input + row * width;
     const float* residual = residual_input + row * width;
@@ -296,17 +301,42 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     const float second_inverse =
         1.0f / sqrtf(tree_total_wide(ordered_sum(), partials) / static_cast<float>(width) + second_eps);
 
+    float largest = 0.0f;
 #pragma unroll
     for (int i = 0; i < kLoaded; ++i) {
         const int column = t + (q + kLoaders * i) * kRmsThreads;
         const float result = __fmul_rn(__fmul_rn(value[i], second_inverse), second_scale[i]);
         if (column < width) {
             normalized[column] = result;
-            if constexpr (HANDOFF) staged[column] = result;
+            if constexpr (HANDOFF == 1) staged[column] = result;
+            // (the sums have read `handed`: tree_total_wide's barriers lie in between)
+            if constexpr (HANDOFF == 2) handed[column] = result;
+            largest = fmaxf(largest, fabsf(result));
         }
     }
 
-    if constexpr (HANDOFF) {
+    if constexpr (HANDOFF == 2) {
+        // what f16_image_kernel would make of the normalized row, bit for bit
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) largest = fmaxf(largest, __shfl_xor(largest, offset));
+        if ((threadIdx.x & 63) == 0) wave_largest[threadIdx.x >> 6] = largest;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < kWideThreads / kWave; ++w) largest = fmaxf(largest, wave_largest[w]);
+        const HalfImageScale scale = half_image_scale(largest);
+        const int rows = static_cast<int>(gridDim.x);
+        float* inverse_scale =
+            reinterpret_cast<float*>(records + static_cast<std::int64_t>(rows) * width * 2);
+        if (threadIdx.x == 0) inverse_scale[row] = scale.inverse;
+        for (int group = threadIdx.x; group < (width >> 3); group += kWideThreads) {
+            half_image_store(records, group, rows, static_cast<int>(row),
+                             *reinterpret_cast<const float4*>(handed + group * 8),
+                             *reinterpret_cast<const float4*>(handed + group * 8 + 4),
+                             scale.factor);
+        }
+    }
+
+    if constexpr (HANDOFF == 1) {
         __syncthreads();
         // one wave per 256-value block: the quantizer of the decode kernels
         const int lane = threadIdx.x & 63;
@@ -509,19 +539,23 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
                                  bool second_centered, float* normalized_output,
                                  float* residual_output, std::int64_t rows, std::int64_t width,
                                  float first_eps, float second_eps, std::uint8_t* records,
-                                 hipStream_t stream) {
+                                 std::uint8_t* half_image, hipStream_t stream) {
     const NormWeight first = norm_weight(first_weight, first_centered);
     const NormWeight second = norm_weight(second_weight, second_centered);
     const dim3 grid(static_cast<unsigned>(rows));
     if (width <= kOwned * kRmsThreads) {
         const int columns = static_cast<int>(width);
-        if (records != nullptr) {
-            hipLaunchKernelGGL((dual_rms_resident_kernel<true>), grid, dim3(kWideThreads),
+        if (half_image != nullptr) {
+            hipLaunchKernelGGL((dual_rms_resident_kernel<2>), grid, dim3(kWideThreads), 0, stream, input,
+                               first, residual_input, hidden_output, second, normalized_output,
+                               residual_output, columns, first_eps, second_eps, half_image);
+        } else if (records != nullptr) {
+            hipLaunchKernelGGL((dual_rms_resident_kernel<1>), grid, dim3(kWideThreads),
                                static_cast<std::size_t>(columns) * sizeof(float), stream, input,
                                first, residual_input, hidden_output, second, normalized_output,
                                residual_output, columns, first_eps, second_eps, records);
         } else {
-            hipLaunchKernelGGL((dual_rms_resident_kernel<false>), grid, dim3(kWideThreads), 0, stream,
+            hipLaunchKernelGGL((dual_rms_resident_kernel<0>), grid, dim3(kWideThreads), 0, stream,
                                input, first, residual_input, hidden_output, second,
                                normalized_output, residual_output, columns, first_eps, second_eps,
                                records);

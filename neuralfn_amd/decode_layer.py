@@ -124,7 +124,7 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
 
 def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
                  pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
-                 attention_workspace=None):
+                 attention_workspace=None, handoff: bool = False):
     """A block of tokens (rows of `pending`, at positions position, position + 1, ...) through
     one layer the way the verifier runs it (resident_glimmer_cuda.cpp:2913-2960, 3437-3520): the
     same operators in their batch forms, a causal block attention over the cache and the
@@ -132,15 +132,25 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     commit of the accepted ones (cache_commit, cache_commit_layers).  Row r equals decode_layer
     at position + r after the commits of the rows before it, to rounding.
 
+    handoff (5..16 rows, a model width of at most 8,192): the two dual norms also leave their
+    output in `workspace` in the form the projections would convert it to
+    (nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1) and the projections behind them
+    multiply from it; the same bits, two launches less.
+
     Returns (down, hidden, key_rows, value_rows).
     """
     g = geometry
     rows = pending.shape[0]
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         pending, residual, pending_norm, False, weights.input_norm, False,
-        g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps)
-    query, key, value, gate = tile_ops.multi_linear(
-        [weights.q, weights.k, weights.v, weights.attention_gate], normalized, workspace)
+        g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps,
+        handoff_workspace=workspace if handoff else None)
+    attention_inputs = [weights.q, weights.k, weights.v, weights.attention_gate]
+    if handoff:
+        query, key, value, gate = tile_ops.multi_linear_prequantized(
+            attention_inputs, rows, workspace, family="mmq")
+    else:
+        query, key, value, gate = tile_ops.multi_linear(attention_inputs, normalized, workspace)
     query = query.view(rows, g.query_heads, g.head_dim)
     key = key.view(rows, g.kv_heads, g.head_dim)
     value = value.view(rows, g.kv_heads, g.head_dim)
@@ -156,9 +166,13 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
                                          workspace, second=gate, prologue="gated")
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
-        g.post_norm_eps, g.norm_eps)
-    mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
-                                             workspace)
+        g.post_norm_eps, g.norm_eps, handoff_workspace=workspace if handoff else None)
+    if handoff:
+        mlp_gate, mlp_up = tile_ops.multi_linear_prequantized(
+            [weights.mlp_gate, weights.mlp_up], rows, workspace, family="mmq")
+    else:
+        mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
+                                                 workspace)
     (down,) = tile_ops.multi_linear([weights.mlp_down], mlp_gate, workspace, second=mlp_up,
                                     prologue="swiglu")
     return down, hidden, key, value

@@ -156,6 +156,8 @@ SIGNATURES = {
         ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
+    "nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1": (
+        ctypes.c_int, [_DESC_ARRAY, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_gated_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _P, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, _P]),
     "nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1": (
@@ -177,6 +179,9 @@ SIGNATURES = {
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P]),
     "nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
+    "nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1": (
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
     "nfn_native_tile_argmax_rows_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
@@ -393,18 +398,22 @@ def multi_linear(weights: Sequence[PackedWeight], x, workspace, second=None, fam
     return outputs
 
 
-def multi_linear_prequantized(weights: Sequence[PackedWeight], rows: int, workspace, outputs=None):
-    """Projections of the input whose activation records a verifier-family call or the
-    dual-RMS handoff left in `workspace`."""
+def multi_linear_prequantized(weights: Sequence[PackedWeight], rows: int, workspace, outputs=None,
+                              family: str = "mmvq"):
+    """Projections of the input whose quantized form an earlier call left in `workspace`:
+    family "mmvq": the activation records of a verifier-family call or of the one-row dual-RMS
+    handoff; family "mmq": the fp16 rows of the 5..16-row dual-RMS handoff."""
     import torch
     stream = _stream_handle()
     if outputs is None:
         outputs = [torch.empty((rows, w.output_dim), dtype=torch.float32, device=workspace.device)
                    for w in weights]
     descriptors = [w.descriptor(stream) for w in weights]
-    check(load().nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1(
+    name = ("nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1" if family == "mmvq"
+            else "nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1")
+    check(getattr(load(), name)(
         _descriptor_array(descriptors), _pointer_array(outputs), len(weights), rows,
-        workspace.data_ptr(), workspace.numel(), stream), "mmvq_multi_linear_prequantized")
+        workspace.data_ptr(), workspace.numel(), stream), f"{family}_multi_linear_prequantized")
     return outputs
 
 
@@ -451,8 +460,9 @@ def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = Non
                          second_eps: float = 1e-6, handoff_workspace=None):
     """hidden = residual + rms(x, first); normalized = rms(hidden, second).
 
-    Returns (hidden, normalized, residual_output).  With `handoff_workspace` (one row) the
-    activation records of `normalized` are left there for multi_linear_prequantized.
+    Returns (hidden, normalized, residual_output).  With `handoff_workspace` the quantized form
+    of `normalized` is left there for multi_linear_prequantized: one row, family "mmvq";
+    5..16 rows, family "mmq".
     """
     import torch
     rows, width = x.shape
@@ -470,10 +480,14 @@ def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = Non
     if handoff_workspace is None:
         check(load().nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1(*arguments, stream),
               "dual_rms_add_capture")
-    else:
+    elif rows == 1:
         check(load().nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
             *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
             "dual_rms_add_capture_mmvq_q8")
+    else:
+        check(load().nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
+            *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
+            "dual_rms_add_capture_mmq_f16")
     return hidden, normalized, captured
 
 

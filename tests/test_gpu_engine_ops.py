@@ -1017,6 +1017,18 @@ def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, o
         pending_norm = weights.post_feedforward_norm
         staged.append((key_rows, value_rows))
 
+    # the same block with the dual norms handing their output to the projections in the
+    # small-batch workspace: two launches less per layer, the same bits
+    handed_pending = to_device(embeddings, cuda)
+    handed_residual, pending_norm = torch_().zeros_like(handed_pending), None
+    for weights, cache, (key_rows, value_rows) in zip(stack, caches(), staged):
+        handed_pending, handed_residual, handed_keys, handed_values = dl.verify_layer(
+            g, weights, cache, handed_pending, handed_residual, pending_norm, position, workspace,
+            True, attention_workspace, handoff=True)
+        pending_norm = weights.post_feedforward_norm
+        assert torch_().equal(handed_keys, key_rows) and torch_().equal(handed_values, value_rows)
+    assert torch_().equal(handed_pending, pending) and torch_().equal(handed_residual, residual)
+
     def error(actual, expected):
         return float(np.max(np.abs(actual - expected)) / np.max(np.abs(expected)))
 

@@ -805,6 +805,84 @@ def test_prequantized_reuses_the_records_of_a_verifier_call(cuda, rows):
         assert_bits_equal(a, b, kquant.NAMES[encoding])
 
 
+@pytest.mark.parametrize("rows,width", [(5, 6656), (16, 6656), (9, 256), (16, 8192)])
+def test_dual_rms_block_handoff_equals_ordinary_path(cuda, oracle, rows, width):
+    """The 5..16-row form of the handoff: the norm kernel leaves the fp16 rows that the
+    small-batch call would have converted its input to, and the projections fed from them
+    equal the ordinary dual RMS followed by the ordinary call, bit for bit; rows several
+    orders of magnitude apart keep their own scales."""
+    rng = np.random.default_rng(70 + rows)
+    x = probe_rms_input(rows, width) * (10.0 ** rng.integers(-3, 4, (rows, 1))).astype(np.float32)
+    residual = (rng.standard_normal((rows, width)) *
+                10.0 ** rng.integers(-2, 3, (rows, 1))).astype(np.float32)
+    scale = tile_ops.PackedWeight.from_numpy(
+        kquant.F32, kquant.quantize(kquant.F32, rng.uniform(0.5, 1.5, (1, width)).astype(np.float32)),
+        1, width)
+    specs = [(kquant.Q4_K, 129), (kquant.Q5_K, 33), (kquant.Q6_K, 70), (kquant.Q8_0, 17)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, width, 40 + i), n, width)
+               for i, (e, n) in enumerate(specs)]
+    workspace = tile_ops.small_batch_workspace(rows, width)
+    arguments = dict(first_weight=scale, second_weight=scale, first_eps=1e-8, second_eps=1e-5)
+    ordinary = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda), **arguments)
+    ordinary_out = tile_ops.multi_linear(weights, ordinary[1], workspace)
+    workspace.zero_()
+    handoff = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda),
+                                            handoff_workspace=workspace, **arguments)
+    handoff_out = tile_ops.multi_linear_prequantized(weights, rows, workspace, family="mmq")
+    again = tile_ops.multi_linear_prequantized(weights[1:3], rows, workspace, family="mmq")
+    for a, b, label in zip(ordinary, handoff, ("hidden", "normalized", "capture")):
+        assert_bits_equal(a, b, label)
+    for a, b, (encoding, _) in zip(ordinary_out, handoff_out, specs):
+        assert_bits_equal(a, b, kquant.NAMES[encoding])
+    for a, b in zip(ordinary_out[1:3], again):
+        assert_bits_equal(a, b, "a second consumer of the same rows")
+    normalized = ordinary[1].cpu().numpy()
+    for (encoding, out_dim), weight, y in zip(specs, weights, ordinary_out):
+        exact = oracle.linear(encoding, weight.data.cpu().numpy(), out_dim, width, normalized)
+        for row in range(rows):
+            assert normalised_error(y.cpu().numpy()[row], exact[row]) <= TOLERANCE
+
+
+def test_block_handoff_fails_closed(cuda):
+    width = 512
+    lib = tile_ops.load()
+    x = to_device(probe_rms_input(16, width), cuda)
+    outputs = [torch_().empty_like(x) for _ in range(3)]
+    workspace = tile_ops.small_batch_workspace(16, width)
+    head = [x.data_ptr(), None, x.data_ptr(), outputs[0].data_ptr(), None, outputs[1].data_ptr(),
+            outputs[2].data_ptr()]
+    tail = [1e-8, False, 1e-5, False]
+    handoff = lib.nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1
+    required = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(8, width)
+    assert handoff(*head, 8, width, *tail, workspace.data_ptr(), required, None) == 0
+    assert handoff(*head, 4, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 17, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 8, width, *tail, workspace.data_ptr(), required - 1, None) == 1
+    assert handoff(*head, 8, width, *tail, None, required, None) == 1
+    assert handoff(*head, 8, 384, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 8, 8448, *tail, workspace.data_ptr(), 1 << 30, None) == 1
+    assert handoff(*head, 8, width, 0.0, False, 1e-5, False, workspace.data_ptr(), required, None) == 1
+    torch_().cuda.synchronize()
+    out = torch_().empty((16, 8), dtype=torch_().float32, device=cuda)
+    packed = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, 8, width, 1),
+                                              8, width)
+    plain = tile_ops.PackedWeight.from_numpy(
+        kquant.F32, kquant.quantize(kquant.F32, kquant.synthetic_weights(2, 8, width, 1.0)), 8, width)
+    prequantized = lib.nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1
+    pointers = tile_ops._pointer_array([out])
+    good = tile_ops._descriptor_array([packed.descriptor(0)])
+    assert prequantized(good, pointers, 1, 8, workspace.data_ptr(), required, None) == 0
+    assert prequantized(good, pointers, 1, 4, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert prequantized(good, pointers, 1, 17, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert prequantized(good, pointers, 1, 8, workspace.data_ptr(), required - 1, None) == 1
+    assert prequantized(good, pointers, 0, 8, workspace.data_ptr(), required, None) == 1
+    assert prequantized(good, pointers, 1, 8, None, required, None) == 1
+    # a projection that the fp16 kernel does not take has no use for the rows in the workspace
+    other = tile_ops._descriptor_array([plain.descriptor(0)])
+    assert prequantized(other, pointers, 1, 8, workspace.data_ptr(), required, None) == 1
+    torch_().cuda.synchronize()
+
+
 def test_handoff_and_prequantized_fail_closed(cuda):
     width = 512
     lib = tile_ops.load()
