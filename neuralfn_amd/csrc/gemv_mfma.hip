@@ -359,38 +359,74 @@ struct TileSource {
     }
 };
 
-template <std::uint32_t ENC>
+// Q6_K blocks are 210 bytes: every other block of a row starts two bytes past a word, and a
+// 16-byte load that is not word aligned runs at a fraction of an aligned one's rate.  Such a
+// chunk is read from two bytes earlier and moved into place when it goes to LDS
+// (store_block), with the first word of the next chunk, which the next lane holds.
+// `flags` remembers per load: bit i: moved down two bytes; bit 8 + i: read at the tensor's end.
+// REALIGN false keeps the loads where the chunks are: the lm_head at two to eight tokens has
+// no vector instructions to spare for the moving (263 us as read, 272 us realigned), the short
+// launches of a decode layer are waiting for memory (17.2 -> 16.1 us on the attention
+// projections at four tokens).
+template <std::uint32_t ENC, bool REALIGN>
 __device__ __forceinline__ void fetch_block(const TileSource<ENC>& src, std::int64_t block,
-                                            int lane, uint4 (&staged)[TileSource<ENC>::kLoads]) {
+                                            int lane, uint4 (&staged)[TileSource<ENC>::kLoads],
+                                            std::uint32_t& flags) {
     using F = Format<ENC>;
     const std::uint8_t* block_base = src.base + block * F::kBlockBytes;
+    flags = 0;
 #pragma unroll
     for (int i = 0; i < TileSource<ENC>::kLoads; ++i) {
         const std::uint8_t* p = block_base + src.offset[i];
         if constexpr (F::kAligned) {
             staged[i] = load_chunk<ENC>(p);
         } else {
-            // The last chunk of a block reads 14 bytes past it; only its first
-            // two bytes (the block's d) are used.  At the very end of the
-            // tensor read the 16 bytes before the end instead and move those
-            // two bytes into place.
+            const std::uint32_t two =
+                REALIGN ? static_cast<std::uint32_t>(reinterpret_cast<std::uintptr_t>(p)) & 2u : 0u;
+            p -= two;
+            // The last chunk of a block reads past it; only its first two bytes (the block's
+            // d) are used.  At the very end of the tensor the 16 bytes before the end are
+            // read instead, whose last two bytes they are.
             const bool past = p + 16 > src.data_end;
-            uint4 v = load_chunk<ENC>(past ? src.data_end - 16 : p);
-            if (past) v.x = v.w >> 16;
-            staged[i] = v;
+            staged[i] = load_chunk<ENC>(past ? src.data_end - 16 : p);
+            flags |= (two >> 1) << i;
+            flags |= (past ? 1u : 0u) << (8 + i);
         }
     }
 }
 
-template <std::uint32_t ENC>
+template <std::uint32_t ENC, bool REALIGN>
 __device__ __forceinline__ void store_block(const uint4 (&staged)[TileSource<ENC>::kLoads],
-                                            int lane, std::uint8_t* wave_tile) {
+                                            std::uint32_t flags, int lane,
+                                            std::uint8_t* wave_tile) {
     using F = Format<ENC>;
 #pragma unroll
     for (int i = 0; i < TileSource<ENC>::kLoads; ++i) {
         const int chunk = min(i * kWave + lane, TileSource<ENC>::kTotalChunks - 1);
         const int row = chunk / F::kChunks;
         const int col = chunk - row * F::kChunks;
+        if constexpr (!F::kAligned) {
+            const uint4 read = staged[i];
+            // the next chunk's first word: the next lane's, for lane 63 lane 0 of the next load
+            // (a row's last chunk needs none: its two bytes are in the words it read)
+            const std::uint32_t wrapped = i + 1 < TileSource<ENC>::kLoads
+                ? __builtin_amdgcn_readfirstlane(staged[i + 1 < TileSource<ENC>::kLoads ? i + 1 : i].x)
+                : 0u;
+            const bool moved = REALIGN && ((flags >> i) & 1u) != 0;
+            const bool past = ((flags >> (8 + i)) & 1u) != 0;
+            // (a chunk read at the tensor's end holds those two bytes in its last word)
+            const std::uint32_t next = static_cast<std::uint32_t>(__builtin_amdgcn_update_dpp(
+                static_cast<int>(wrapped), static_cast<int>(past ? read.w : read.x),
+                0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+            uint4 placed;
+            placed.x = moved ? __builtin_amdgcn_alignbit(read.y, read.x, 16) : read.x;
+            placed.y = moved ? __builtin_amdgcn_alignbit(read.z, read.y, 16) : read.y;
+            placed.z = moved ? __builtin_amdgcn_alignbit(read.w, read.z, 16) : read.z;
+            placed.w = moved ? __builtin_amdgcn_alignbit(next, read.w, 16) : read.w;
+            if (past) placed.x = read.w >> 16;
+            *reinterpret_cast<uint4*>(wave_tile + row * F::kLdsRow + col * 16) = placed;
+            continue;
+        }
         *reinterpret_cast<uint4*>(wave_tile + row * F::kLdsRow + col * 16) = staged[i];
     }
 }
@@ -501,15 +537,17 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     int fetch_step = 0;
     fetch_source.setup(set, fetch_tile, lane);
     uint4 staged[kDepth][Source::kLoads];
+    std::uint32_t staged_flags[kDepth];
     float4 inputs[MODE == kStream ? kDepth : 1][MODE == kStream ? kTokens : 1];
-    auto fetch = [&](uint4 (&chunks)[Source::kLoads], float4 (&slot)[MODE == kStream ? kTokens : 1]) {
+    auto fetch = [&](uint4 (&chunks)[Source::kLoads], std::uint32_t& chunk_flags,
+                     float4 (&slot)[MODE == kStream ? kTokens : 1]) {
         const int block = max(min(fetch_step, count - 1), 0);
         if constexpr (MODE == kStream) {
             // the float activations of the block go out ahead of its chunks
 #pragma unroll
             for (int t = 0; t < kTokens; ++t) slot[t] = load_input(block, t);
         }
-        fetch_block<ENC>(fetch_source, begin + block, lane, chunks);
+        fetch_block<ENC, !ARGMAX>(fetch_source, begin + block, lane, chunks, chunk_flags);
         if (++fetch_step == steps) {
             fetch_step = 0;
             if (fetch_tile + gridDim.x < total_tiles) {
@@ -529,7 +567,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     // 10.8; none: 11.8).
     constexpr int kAhead = MODE == kResident ? 1 : kDepth;
 #pragma unroll
-    for (int d = 0; d < kAhead; ++d) fetch(staged[d], inputs[MODE == kStream ? d : 0]);
+    for (int d = 0; d < kAhead; ++d) fetch(staged[d], staged_flags[d], inputs[MODE == kStream ? d : 0]);
 
     if constexpr (MODE == kResident) {
 #pragma unroll
@@ -554,7 +592,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
         wave_lds_fence();
     }
 #pragma unroll
-    for (int d = kAhead; d < kDepth; ++d) fetch(staged[d], inputs[MODE == kStream ? d : 0]);
+    for (int d = kAhead; d < kDepth; ++d) fetch(staged[d], staged_flags[d], inputs[MODE == kStream ? d : 0]);
 
     // Which A row this lane supplies.
     const OperandRow<kQ6> a_row(j, kc);
@@ -568,11 +606,11 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
 #pragma unroll
     for (int u = 0; u < S; ++u) acc[u] = 0.0f;
 
-    auto step = [&](uint4 (&chunks)[Source::kLoads], float4 (&slot)[MODE == kStream ? kTokens : 1],
-                    int position) {
+    auto step = [&](uint4 (&chunks)[Source::kLoads], std::uint32_t& chunk_flags,
+                    float4 (&slot)[MODE == kStream ? kTokens : 1], int position) {
         if (position < total) {
             if (work_step < count) {
-                store_block<ENC>(chunks, lane, wave_tile);
+                store_block<ENC, !ARGMAX>(chunks, chunk_flags, lane, wave_tile);
                 if constexpr (MODE == kStream) {
 #pragma unroll
                     for (int t = 0; t < kTokens; ++t) {
@@ -664,13 +702,13 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
                 for (int u = 0; u < S; ++u) acc[u] = 0.0f;
             }
         }
-        fetch(chunks, slot);
+        fetch(chunks, chunk_flags, slot);
     };
 
     for (int position = 0; position < total; position += kDepth) {
 #pragma unroll
         for (int d = 0; d < kDepth; ++d) {
-            step(staged[d], inputs[MODE == kStream ? d : 0], position + d);
+            step(staged[d], staged_flags[d], inputs[MODE == kStream ? d : 0], position + d);
         }
     }
 }
