@@ -663,9 +663,12 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
             def token():
                 pending, residual, pending_norm = embedding, zeros, None
                 for layer_weights, cache in zip(weights, caches):
+                    # (the reference form keeps to the reference's entry points; the other
+                    # also takes gate and up with the activation folded into their row ends)
                     pending, residual = dl.decode_layer(g, layer_weights, cache, pending, residual,
                                                         pending_norm, position, workspace, local,
-                                                        attention_workspace)
+                                                        attention_workspace,
+                                                        fused_gate_up=attention_workspace is not None)
                     pending_norm = layer_weights.post_feedforward_norm
                 last["hidden"] = residual
 

@@ -225,6 +225,22 @@ int nfn_native_tile_k_quant_mmvq_linear_float32_v1(
     void* workspace,
     int64_t workspace_nbytes,
     void* cuda_stream);
+/* The gate and up projections of a feed-forward block for one token with the
+ * SwiGLU activation at the row ends: output[r] = (up_r * gate_r) * sigmoid(gate_r),
+ * output_dim floats.  No counterpart in the reference, whose engine runs the
+ * grouped one-row call on [gate, up] and then
+ * nfn_native_tile_k_quant_mmvq_multi_linear_swiglu_float32_v1 on the two
+ * results (resident_glimmer_cuda.cpp:2233-2585, glimmer_k_mmq.cu:299-317):
+ * here the down projection behind reads one plain vector of output_dim floats
+ * instead of two, and the plain call on `output` gives the bits of the SwiGLU
+ * call on the separate results.  gate and up: the same encoding (Q4_K or
+ * Q5_K), shape and row stride; input_dim a multiple of 256, at most 8192. */
+int nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* gate,
+    const NfnNativeTilePackedWeightDescriptorV1* up,
+    const float* input,
+    float* output,
+    void* cuda_stream);
 
 /* ---- the normalisation step upstream of the decode projections ----------
  * hidden = residual_input + rms(input, first_weight, first_eps);

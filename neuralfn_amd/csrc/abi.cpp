@@ -386,6 +386,26 @@ int nfn_native_tile_k_quant_mmvq_linear_float32_v1(const Descriptor* descriptor,
                            workspace_nbytes, cuda_stream);
 }
 
+int nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1(const Descriptor* gate, const Descriptor* up,
+                                                     const float* input, float* output,
+                                                     void* cuda_stream) {
+    if (gate == nullptr || up == nullptr || input == nullptr || output == nullptr ||
+        !validate_k_descriptor(gate, gate->input_dim, cuda_stream, false) ||
+        !validate_k_descriptor(up, gate->input_dim, cuda_stream, false) ||
+        gate->output_dim != up->output_dim || gate->output_dim > 0x3fffffff ||
+        !gemv_dot_pairs_supports(gate->encoding, up->encoding, gate->input_dim)) {
+        return kInvalid;
+    }
+    ProjectionSet set{};
+    set.count = 2;
+    set.input_dim = gate->input_dim;
+    set.op[0] = make_projection(*gate, output);
+    set.op[1] = make_projection(*up, output);
+    if (set.op[0].row_stride != set.op[1].row_stride) return kInvalid;
+    launch_gemv_dot_pairs(set, input, as_stream(cuda_stream));
+    return launch_status();
+}
+
 int nfn_native_tile_argmax_rows_float32_v1(const float* values, std::int64_t* output_indices,
                                            float* output_values, std::int64_t rows,
                                            std::int64_t width, void* cuda_stream) {

@@ -257,9 +257,12 @@ __device__ __forceinline__ GlobalBytes unpack_pointer(std::uint64_t a, std::uint
 }
 
 // Walks the (row, 64-unit slice) pairs of one wave; everything is uniform.
+// HALF > 0 (pair mode, one projection slot): "row" r stands for row r of the first
+// projection followed by row r of the second, HALF slices each.
 struct DotCursor {
     int op, row, first_row, next_bound, iteration;
     GlobalBytes row_ptr;
+    std::int64_t second_minus_first;  // pair mode: from a row of the first projection to its partner
 
     __device__ __forceinline__ void bounds(int b1, int b2, int b3) {
         first_row = op == 0 ? 0 : op == 1 ? b1 : op == 2 ? b2 : b3;
@@ -273,9 +276,19 @@ struct DotCursor {
         bounds(b1, b2, b3);
         row_ptr = unpack_pointer(a, b, c, op) + (row - first_row) * stride;
     }
+    template <int HALF>
     __device__ __forceinline__ void advance(int iterations, std::int64_t stride, std::uint64_t a,
                                             std::uint64_t b, std::uint64_t c, int b1, int b2, int b3) {
-        if (++iteration < iterations) return;
+        ++iteration;
+        if constexpr (HALF > 0) {
+            if (iteration == HALF) row_ptr += second_minus_first;
+            if (iteration < 2 * HALF) return;
+            iteration = 0;
+            ++row;
+            row_ptr += stride - second_minus_first;
+            return;
+        }
+        if (iteration < iterations) return;
         iteration = 0;
         ++row;
         row_ptr += stride;
@@ -293,12 +306,19 @@ struct DotCursor {
 // ITER > 0 (one token only): a row has exactly ITER 64-unit slices, and since a
 // lane's units are then the same in every row, their activation operands stay in
 // registers for the whole launch instead of being read from LDS per row.
-template <std::uint32_t ENC, int T, int P, int ITER, int STAGES>
+// PAIRS (one token, ITER > 0, two projections of one shape): a wave takes row r of the first
+// projection and row r of the second one after the other and stores
+// swiglu(first's sum, second's sum) as output r: the gate and up projections of a
+// feed-forward block with the activation folded into the row end, so that the down
+// projection behind it reads one plain vector.
+template <std::uint32_t ENC, int T, int P, int ITER, int STAGES, bool PAIRS = false>
 __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const float* __restrict__ first, std::uint64_t data_a, std::uint64_t data_b,
     std::uint64_t data_c, int input_dim, int rows_per_group, int longer_groups, int bound1,
     int bound2, int bound3, DotTail tail) {
     static_assert(ITER == 0 || (T == 1 && ITER <= 2), "register-resident activations: one token, two slices");
+    static_assert(!PAIRS || (ITER > 0 && P == kPlain), "pair mode: register-resident activations, plain input");
+    constexpr int kHalf = PAIRS ? ITER : 0;
     constexpr bool kQ5 = ENC == kEncQ5K;
     constexpr int kBlockBytes = kQ5 ? 176 : 144;
     constexpr int kQuants = kQ5 ? 48 : 16;
@@ -308,7 +328,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int blocks = input_dim >> 8;
     const int units = 4 * blocks;
-    const int iterations = ITER > 0 ? ITER : (units + kWave - 1) / kWave;
+    const int iterations = PAIRS ? 2 * ITER : ITER > 0 ? ITER : (units + kWave - 1) / kWave;
     const int token0 = blockIdx.y * T;
     const int pass_tokens = T == 1 ? 1 : min(tail.tokens - token0, T);
     const float* pass_first = pass_input<P>(first, token0, input_dim);
@@ -343,6 +363,8 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // last pair loads one fixed address in every lane (one cache line per instruction),
     // so the number of loads in flight is the same on every path.
     DotCursor fetch;
+    fetch.second_minus_first = PAIRS ? unpack_pointer(data_a, data_b, data_c, 1) -
+            unpack_pointer(data_a, data_b, data_c, 0) : 0;
     fetch.start(row_count > 0 ? row_begin : 0, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     int fetch_left = total;  // pairs not fetched yet
     // A lane's byte offsets inside a row depend on the slice only (and a slice of a
@@ -362,8 +384,8 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         const bool real = fetch_left > 0;
         std::uint32_t block_offset, quants_offset;
         if constexpr (ITER > 0) {
-            block_offset = real ? block_offsets[slice] : 0;
-            quants_offset = real ? quant_offsets[slice] : 0;
+            block_offset = real ? block_offsets[slice % ITER] : 0;
+            quants_offset = real ? quant_offsets[slice % ITER] : 0;
         } else {
             const int unit = real ? min(fetch.iteration * kWave + lane, units - 1) : 0;
             block_offset = (unit >> 2) * kBlockBytes;
@@ -383,7 +405,9 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
             stage.h0 = make_uint4(h0.x, h0.y, h0.z, h0.w);
             stage.h1 = make_uint4(h1.x, h1.y, h1.z, h1.w);
         }
-        if (--fetch_left > 0) fetch.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+        if (--fetch_left > 0) {
+            fetch.template advance<kHalf>(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+        }
     };
     // STAGES register stages.  Two are requested here; a third only once this wave's
     // activations have arrived (below): weight requests that go out ahead of the activation
@@ -395,8 +419,10 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // below is unrolled over the steps after which (stage, slice) repeats.
     static_assert(STAGES == 2 || STAGES == 3, "two or three stages");
     constexpr int kStages = STAGES;
-    constexpr int kSlices = ITER > 0 ? ITER : 1;
-    constexpr int kPeriod = kStages % kSlices == 0 ? kStages : kStages * kSlices;
+    constexpr int kSlices = PAIRS ? 2 * ITER : ITER > 0 ? ITER : 1;
+    constexpr int kPeriod = kStages % kSlices == 0 ? kStages
+        : kSlices % kStages == 0                   ? kSlices
+                                                   : kStages * kSlices;
     Stage<kQ5> stages[kStages];
     issue(stages[0], 0);
     issue(stages[1], 1 % kSlices);
@@ -445,19 +471,32 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     for (int t = 0; t < T; ++t) acc[t] = 0.0f;
 
     DotCursor work;
+    work.second_minus_first = 0;  // only its row and iteration counters are used in pair mode
     work.start(row_count > 0 ? row_begin : 0, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+    float first_total = 0.0f;  // pair mode: the finished sum of the first projection's row
     // `slice`: for ITER > 0 the slice of its row this step works on
     auto compute = [&](const Stage<kQ5>& stage, int slice) {
         const int iteration = work.iteration;
-        const int raw_unit = iteration * kWave + lane;
+        const int raw_unit = (PAIRS ? iteration % ITER : iteration) * kWave + lane;
         const bool live = raw_unit < units;
         const int unit = min(raw_unit, units - 1);
         if constexpr (ITER > 0) {
-            acc[0] = unit_product(unpack_unit<kQ5>(stage, lane & 3), held[slice], live, acc[0]);
+            acc[0] = unit_product(unpack_unit<kQ5>(stage, lane & 3), held[slice % ITER], live, acc[0]);
         } else {
             accumulate_unit<kQ5, T>(stage, lds, unit, live, blocks, acc);
         }
-        if (iteration == iterations - 1) {
+        if constexpr (PAIRS) {
+            if (iteration == ITER - 1) {
+                first_total = wave_total(acc[0]);
+                acc[0] = 0.0f;
+            } else if (iteration == 2 * ITER - 1) {
+                const float second_total = wave_total(acc[0]);
+                if (lane == 0) {
+                    tail.output[0][work.row] = apply_prologue<kSwiGlu>(first_total, second_total);
+                }
+                acc[0] = 0.0f;
+            }
+        } else if (iteration == iterations - 1) {
             // the row is complete: fixed-order butterfly, lane 0 writes
             float* base = tail.output[0];
             std::int64_t output_dim = tail.output_dim[0];
@@ -476,7 +515,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
                 acc[t] = 0.0f;
             }
         }
-        work.advance(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
+        work.template advance<kHalf>(iterations, stride, data_a, data_b, data_c, bound1, bound2, bound3);
     };
 
     for (int n = 0; n < total; n += kPeriod) {
@@ -550,6 +589,46 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     launch(gemv_dot_kernel<ENC, T, P, 0, 2>);
 }
 
+// Pair mode: `set` holds two projections of one shape and one output (slot 0), one token.
+template <std::uint32_t ENC>
+void launch_pairs(const ProjectionSet& set, const float* input, hipStream_t stream) {
+    const std::int64_t pairs = set.op[0].output_dim;
+    const void* data[4] = {set.op[0].data, set.op[1].data, set.op[0].data, set.op[0].data};
+    DotTail tail{};
+    tail.tokens = 1;
+    tail.output[0] = set.op[0].output;
+    tail.output_dim[0] = pairs;
+    const PackedPointers packed = pack_pointers(data);
+    const std::int64_t blocks = set.input_dim >> 8;
+    const std::size_t lds = static_cast<std::size_t>(token_image_bytes_host(blocks));
+    // workgroups as for the 2 x pairs weight rows of the launch
+    std::int64_t groups = decode_groups(2 * pairs, kDotWaves);
+    if (groups > pairs) groups = pairs;
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), 1), dim3(kDotThreads), lds,
+                           stream, input, packed.a, packed.b, packed.c,
+                           static_cast<int>(set.input_dim), static_cast<int>(pairs / groups),
+                           static_cast<int>(pairs % groups), 0x7fffffff, 0x7fffffff, 0x7fffffff, tail);
+    };
+    const std::int64_t slices = (4 * blocks + kWave - 1) / kWave;
+    const bool small = groups <= compute_units();
+    if (slices == 1) {
+        if (small) {
+            allow_large_lds<gemv_dot_kernel<ENC, 1, kPlain, 1, 3, true>>();
+            launch(gemv_dot_kernel<ENC, 1, kPlain, 1, 3, true>);
+        } else {
+            allow_large_lds<gemv_dot_kernel<ENC, 1, kPlain, 1, 2, true>>();
+            launch(gemv_dot_kernel<ENC, 1, kPlain, 1, 2, true>);
+        }
+    } else if (small) {
+        allow_large_lds<gemv_dot_kernel<ENC, 1, kPlain, 2, 3, true>>();
+        launch(gemv_dot_kernel<ENC, 1, kPlain, 2, 3, true>);
+    } else {
+        allow_large_lds<gemv_dot_kernel<ENC, 1, kPlain, 2, 2, true>>();
+        launch(gemv_dot_kernel<ENC, 1, kPlain, 2, 2, true>);
+    }
+}
+
 template <std::uint32_t ENC, int P>
 void launch_tokens(const ProjectionSet& set, const float* first, const float* second,
                    std::uint8_t* records_out, int tokens, hipStream_t stream) {
@@ -593,6 +672,21 @@ void launch_prologue(const ProjectionSet& set, const float* first, const float* 
 bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim) {
     return (encoding == kEncQ4K || encoding == kEncQ5K) && input_dim % 256 == 0 &&
         token_image_bytes_host(input_dim >> 8) <= 150 * 1024;
+}
+
+bool gemv_dot_pairs_supports(std::uint32_t first_encoding, std::uint32_t second_encoding,
+                             std::int64_t input_dim) {
+    // register-resident activations: rows of at most two 64-unit slices
+    return first_encoding == second_encoding && gemv_dot_supports(first_encoding, input_dim) &&
+        input_dim <= 8192;
+}
+
+void launch_gemv_dot_pairs(const ProjectionSet& set, const float* input, hipStream_t stream) {
+    if (set.op[0].encoding == kEncQ4K) {
+        launch_pairs<kEncQ4K>(set, input, stream);
+    } else {
+        launch_pairs<kEncQ5K>(set, input, stream);
+    }
 }
 
 void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* second,

@@ -16,4 +16,12 @@ void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* 
                      std::uint8_t* records_out, int prologue, std::int64_t rows,
                      hipStream_t stream);
 
+// One token through two projections of one shape and encoding (gate, up) with the SwiGLU
+// activation at the row ends: output r = (up_r gate_r) sigmoid(gate_r), the value the SwiGLU
+// prologue of the projection behind would compute from the two separate outputs.
+// set.op[0]: gate, its `output` the result; set.op[1]: up.
+bool gemv_dot_pairs_supports(std::uint32_t first_encoding, std::uint32_t second_encoding,
+                             std::int64_t input_dim);
+void launch_gemv_dot_pairs(const ProjectionSet& set, const float* input, hipStream_t stream);
+
 }  // namespace nfn

@@ -81,7 +81,7 @@ class LayerCache:
 
 def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
                  pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
-                 attention_workspace=None):
+                 attention_workspace=None, fused_gate_up: bool = False):
     """One token through one layer.
 
     `pending` is the previous layer's down-projection output whose post-feed-forward norm and
@@ -89,6 +89,9 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     and `residual` zeros gives hidden = rms(embedding), the engine's embedding norm,
     resident_glimmer.cpp:1700-1701).  Returns (down, hidden): this layer's owed pair.
     `attention_workspace` (engine_ops.gqa_decode_workspace) selects the split attention form.
+    `fused_gate_up`: the gate and up projections in one call with the SwiGLU activation at the
+    row ends (nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1) where the pair allows it, so
+    that the down projection reads one plain vector; the same bits as the separate calls.
     """
     g = geometry
     # hidden = residual + rms(pending); normalized = rms(hidden, input_norm)
@@ -115,6 +118,10 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
         g.post_norm_eps, g.norm_eps)
+    if fused_gate_up and tile_ops.gate_up_swiglu_supported(weights.mlp_gate, weights.mlp_up):
+        activated = tile_ops.gate_up_swiglu(weights.mlp_gate, weights.mlp_up, normalized)
+        (down,) = tile_ops.multi_linear([weights.mlp_down], activated, workspace)
+        return down, hidden
     mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
                                              workspace)
     (down,) = tile_ops.multi_linear([weights.mlp_down], mlp_gate, workspace, second=mlp_up,

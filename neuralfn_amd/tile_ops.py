@@ -184,6 +184,7 @@ SIGNATURES = {
     "nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1": (
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
+    "nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1": (ctypes.c_int, [_DESC, _DESC, _P, _P, _P]),
     "nfn_native_tile_argmax_rows_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "nfn_native_tile_glimmer_sigmoid_gate_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
     "nfn_native_tile_swiglu_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
@@ -502,6 +503,27 @@ def mmvq_linear(weight: PackedWeight, x, workspace, out=None):
         ctypes.byref(descriptor), x.data_ptr(), out.data_ptr(), workspace.data_ptr(),
         workspace.numel(), stream), "mmvq_linear")
     return out
+
+
+def gate_up_swiglu(gate: PackedWeight, up: PackedWeight, x, out=None):
+    """nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1: one token through the gate and up
+    projections with the SwiGLU activation at the row ends."""
+    import torch
+    stream = _stream_handle()
+    if out is None:
+        out = torch.empty((1, gate.output_dim), dtype=torch.float32, device=x.device)
+    gate_descriptor, up_descriptor = gate.descriptor(stream), up.descriptor(stream)
+    check(load().nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1(
+        ctypes.byref(gate_descriptor), ctypes.byref(up_descriptor), x.data_ptr(), out.data_ptr(),
+        stream), "gate_up_swiglu")
+    return out
+
+
+def gate_up_swiglu_supported(gate: PackedWeight, up: PackedWeight) -> bool:
+    """Whether gate_up_swiglu takes this pair (else: multi_linear, then the swiglu prologue)."""
+    return (gate.encoding == up.encoding and gate.encoding in (kquant.Q4_K, kquant.Q5_K) and
+            gate.output_dim == up.output_dim and gate.input_dim == up.input_dim and
+            gate.input_dim % 256 == 0 and gate.input_dim <= 8192)
 
 
 def quantize_q8_1(x):

@@ -945,6 +945,45 @@ def test_two_decode_layers_against_the_cpu_engine_arithmetic(cuda, oracle):
         assert np.array_equal(bits_of(cache.keys)[untouched], keys[untouched])
 
 
+def test_decode_layer_with_gate_and_up_in_one_call_gives_the_same_bits(cuda, oracle):
+    """decode_layer(fused_gate_up=True) takes gate and up through
+    nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1 and the down projection on its plain
+    output: the layer's two results equal the separate calls' bit for bit."""
+    from neuralfn_amd import decode_layer as dl
+    rng = np.random.default_rng(23)
+    g = dl.LayerGeometry(model_dim=768, query_heads=4, kv_heads=2, head_dim=64, ffn_dim=1280,
+                         sliding_window=128)
+    shapes = dict(q=(g.attention_dim, g.model_dim), k=(g.kv_dim, g.model_dim),
+                  v=(g.kv_dim, g.model_dim), attention_gate=(g.attention_dim, g.model_dim),
+                  output=(g.model_dim, g.attention_dim), mlp_gate=(g.ffn_dim, g.model_dim),
+                  mlp_up=(g.ffn_dim, g.model_dim), mlp_down=(g.model_dim, g.ffn_dim))
+    device = {}
+    for name, (out_dim, in_dim) in shapes.items():
+        encoding = kquant.Q5_K if name in ("mlp_gate", "mlp_up") else kquant.Q4_K
+        packed = kquant.quantize(encoding, (rng.standard_normal((out_dim, in_dim)) * 0.05).astype(np.float32))
+        device[name] = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    for name, width in dict(input_norm=g.model_dim, q_norm=g.head_dim, k_norm=g.head_dim,
+                            post_attention_norm=g.model_dim, pre_feedforward_norm=g.model_dim,
+                            post_feedforward_norm=g.model_dim).items():
+        row = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+        device[name] = tile_ops.PackedWeight.from_numpy(kquant.F32, row.view(np.uint8).copy(), 1, width)
+    weights = dl.LayerWeights(**device)
+    assert tile_ops.gate_up_swiglu_supported(weights.mlp_gate, weights.mlp_up)
+    keys = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+    values = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+    embedding = to_device(rng.standard_normal((1, g.model_dim)).astype(np.float32), cuda)
+    workspace = tile_ops.small_batch_workspace(1, max(g.model_dim, g.ffn_dim))
+    results = []
+    for fused in (False, True):
+        cache = dl.LayerCache(g, cuda)
+        cache.keys.copy_(bf16_tensor(keys, cuda))
+        cache.values.copy_(bf16_tensor(values, cuda))
+        results.append(dl.decode_layer(g, weights, cache, embedding, torch_().zeros_like(embedding),
+                                       None, 150, workspace, fused_gate_up=fused))
+    assert torch_().equal(results[0][0], results[1][0]) and torch_().equal(results[0][1], results[1][1])
+    assert bool(torch_().isfinite(results[1][0]).all())
+
+
 @pytest.mark.parametrize("split", [False, True])
 def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, oracle, split):
     """decode_layer.verify_layer runs a block of tokens through a layer in the batch forms of the

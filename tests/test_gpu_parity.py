@@ -327,6 +327,54 @@ def test_fused_prologue_equals_materialised(cuda, oracle, mixed, prologue, rows)
         assert_bits_equal(b, f, prologue)
 
 
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
+@pytest.mark.parametrize("in_dim,out_dim", [(256, 1), (2304, 70), (4096, 1037), (6656, 16384), (8192, 513)])
+def test_gate_up_swiglu_equals_the_two_calls(cuda, oracle, encoding, in_dim, out_dim):
+    """nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1 = the grouped one-row call on [gate, up]
+    followed by the element-wise SwiGLU, bit for bit; a projection fed from its output equals the
+    SwiGLU-prologue call on the two separate results."""
+    gate = tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, out_dim, in_dim, 91), out_dim, in_dim)
+    up = tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, out_dim, in_dim, 92), out_dim, in_dim)
+    x = to_device(kquant.synthetic_activations(93, 1, in_dim), cuda)
+    workspace = tile_ops.small_batch_workspace(1, max(in_dim, (out_dim + 255) // 256 * 256))
+    separate = tile_ops.multi_linear([gate, up], x, workspace)
+    expected = tile_ops.swiglu(separate[0], separate[1])
+    fused = tile_ops.gate_up_swiglu(gate, up, x)
+    assert_bits_equal(fused, expected, "gate/up with SwiGLU")
+    if out_dim % 256 == 0:
+        down = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, 40, out_dim, 94), 40, out_dim)
+        (by_prologue,) = tile_ops.multi_linear([down], separate[0], workspace, separate[1], "mmq", "swiglu")
+        (plain,) = tile_ops.multi_linear([down], fused, workspace)
+        assert_bits_equal(plain, by_prologue, "the projection behind")
+    exact_gate = oracle.linear(encoding, gate.data.cpu().numpy(), out_dim, in_dim, x.cpu().numpy())
+    exact_up = oracle.linear(encoding, up.data.cpu().numpy(), out_dim, in_dim, x.cpu().numpy())
+    exact = oracle.swiglu(exact_gate, exact_up)
+    assert normalised_error(fused.cpu().numpy(), exact) <= 2 * TOLERANCE
+
+
+def test_gate_up_swiglu_fails_closed(cuda):
+    lib = tile_ops.load()
+    in_dim, out_dim = 512, 24
+    make = lambda e, n, k, seed: tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, k, seed), n, k)
+    gate, up = make(kquant.Q4_K, out_dim, in_dim, 1), make(kquant.Q4_K, out_dim, in_dim, 2)
+    x = to_device(kquant.synthetic_activations(3, 1, 16384), cuda)
+    out = torch_().empty((1, out_dim), dtype=torch_().float32, device=cuda)
+    call = lib.nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1
+    ref = lambda w: ctypes.byref(w.descriptor(0))
+    assert call(ref(gate), ref(up), x.data_ptr(), out.data_ptr(), None) == 0
+    assert call(ref(gate), ref(make(kquant.Q5_K, out_dim, in_dim, 4)), x.data_ptr(), out.data_ptr(), None) == 1
+    assert call(ref(gate), ref(make(kquant.Q4_K, out_dim + 1, in_dim, 5)), x.data_ptr(), out.data_ptr(), None) == 1
+    assert call(ref(gate), ref(make(kquant.Q4_K, out_dim, 256, 6)), x.data_ptr(), out.data_ptr(), None) == 1
+    six = make(kquant.Q6_K, out_dim, in_dim, 7)
+    assert call(ref(six), ref(six), x.data_ptr(), out.data_ptr(), None) == 1
+    wide = make(kquant.Q4_K, 8, 8448, 8)
+    assert call(ref(wide), ref(wide), x.data_ptr(), out.data_ptr(), None) == 1
+    assert call(None, ref(up), x.data_ptr(), out.data_ptr(), None) == 1
+    assert call(ref(gate), ref(up), None, out.data_ptr(), None) == 1
+    assert call(ref(gate), ref(up), x.data_ptr(), None, None) == 1
+    torch_().cuda.synchronize()
+
+
 def test_elementwise_prologues_over_the_float_range(cuda, oracle):
     """The sigmoid of the two element-wise operators (and of the fused prologues, which share
     it) is built from the hardware's exp2 and reciprocal: 2e-6 of the oracle over twenty
