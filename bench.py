@@ -643,7 +643,10 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
     result = {
         "workload": f"{layers} whole decode layers (Q4_K projections incl. attention gate and FFN "
                     f"{MODEL_DIM}<->{FFN_DIM}), one token, HIP-graph replay; local = 2048-key "
-                    "window, global = every key of a 32768-token context"}
+                    "window, global = every key of a 32768-token context; "
+                    "reference_fused_attention = the reference's entry points only, "
+                    "split_attention = with this library's additions (split attention, gate and "
+                    "up in one call with SwiGLU at the row ends)"}
     for kind, keys, local in (("local", 2048, True), ("global", 32768, False)):
         g = dl.LayerGeometry(model_dim=MODEL_DIM, query_heads=ATTN_DIM // 128,
                              kv_heads=KV_DIM // 128, head_dim=128, ffn_dim=FFN_DIM,
