@@ -646,7 +646,8 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
                     "window, global = every key of a 32768-token context; "
                     "reference_fused_attention = the reference's entry points only, "
                     "split_attention = with this library's additions (split attention, gate and "
-                    "up in one call with SwiGLU at the row ends)"}
+                    "up in one call with SwiGLU at the row ends, the first dual norm inside the "
+                    "Q/K/V/gate launch)"}
     for kind, keys, local in (("local", 2048, True), ("global", 32768, False)):
         g = dl.LayerGeometry(model_dim=MODEL_DIM, query_heads=ATTN_DIM // 128,
                              kv_heads=KV_DIM // 128, head_dim=128, ffn_dim=FFN_DIM,
@@ -661,7 +662,7 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
         cache_bytes = layers * 2 * keys * g.kv_dim * 2
         forms = (("reference_fused_attention", None, dl.LAUNCHES_PER_LAYER),
                  ("split_attention", engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim, device),
-                  dl.LAUNCHES_PER_LAYER_SPLIT))
+                  dl.LAUNCHES_PER_LAYER_FUSED))
         for name, attention_workspace, launches in forms:
             def token():
                 pending, residual, pending_norm = embedding, zeros, None
@@ -671,7 +672,8 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
                     pending, residual = dl.decode_layer(g, layer_weights, cache, pending, residual,
                                                         pending_norm, position, workspace, local,
                                                         attention_workspace,
-                                                        fused_gate_up=attention_workspace is not None)
+                                                        fused_gate_up=attention_workspace is not None,
+                                                        fused_input_norm=attention_workspace is not None)
                     pending_norm = layer_weights.post_feedforward_norm
                 last["hidden"] = residual
 

@@ -379,6 +379,34 @@ int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
     void* mmq_workspace,
     int64_t mmq_workspace_nbytes,
     void* cuda_stream);
+/* One row: the two normalisations and the projections of their result in one
+ * launch.  No counterpart in the reference, whose engine calls
+ * nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1 and then the grouped
+ * one-row call on normalized_output (resident_glimmer_cuda.cpp:2890-2956):
+ * here every workgroup of the projection launch normalises the row in its own
+ * prologue (the arithmetic and the float order of the norm kernel,
+ * kernels.cu:2155-2243) and the first also stores the three rows, which saves
+ * the norm kernel's launch in front of a launch of one workgroup per compute
+ * unit.  The same bits as the two calls.  The arguments up to second_centered
+ * are those of the dual RMS call for one row; width a multiple of 256 up to
+ * 8192; 1..4 projections of one encoding (Q4_K or Q5_K) and input_dim = width. */
+int nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
+    float* const* outputs,
+    int64_t operation_count,
+    void* cuda_stream);
 int nfn_mi355_k_quant_mmq_multi_linear_prequantized_float32_v1(
     const NfnNativeTilePackedWeightDescriptorV1* const* descriptors,
     float* const* outputs,

@@ -12,6 +12,7 @@
 #include "gemv_q8.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
+#include "rms_device.hpp"
 
 #include <cmath>
 #include <limits>
@@ -569,6 +570,44 @@ int nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
                                 normalized_output, residual_output, rows, width, first_eps,
                                 second_eps, static_cast<std::uint8_t*>(mmvq_workspace), nullptr,
                                 as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t width, float first_eps, bool first_centered,
+    float second_eps, bool second_centered, const Descriptor* const* descriptors,
+    float* const* outputs, std::int64_t operation_count, void* cuda_stream) {
+    Descriptor first{}, second{};
+    if (descriptors == nullptr || outputs == nullptr || operation_count < 1 ||
+        operation_count > kMaxOperations || width % 256 != 0 ||
+        !dual_rms_arguments_valid(input, first_weight, residual_input, hidden_output,
+                                  second_weight, normalized_output, residual_output, 1, width,
+                                  first_eps, second_eps, &first, &second)) {
+        return kInvalid;
+    }
+    ProjectionSet set{};
+    set.count = static_cast<int>(operation_count);
+    set.input_dim = width;
+    for (std::int64_t index = 0; index < operation_count; ++index) {
+        if (outputs[index] == nullptr ||
+            !validate_k_descriptor(descriptors[index], width, cuda_stream, false)) {
+            return kInvalid;
+        }
+        set.op[index] = make_projection(*descriptors[index], outputs[index]);
+    }
+    if (!gemv_dot_normed_supports(set)) return kInvalid;
+    DualNormArguments norm{};
+    norm.residual = residual_input;
+    norm.first_weight = norm_weight(first_weight != nullptr ? &first : nullptr, first_centered);
+    norm.second_weight = norm_weight(second_weight != nullptr ? &second : nullptr, second_centered);
+    norm.hidden = hidden_output;
+    norm.captured = residual_output;
+    norm.normalized = normalized_output;
+    norm.first_eps = first_eps;
+    norm.second_eps = second_eps;
+    launch_gemv_dot_normed(set, input, norm, as_stream(cuda_stream));
     return launch_status();
 }
 

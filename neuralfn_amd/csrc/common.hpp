@@ -120,7 +120,9 @@ struct ProjectionSet {
 // records that an earlier launch quantized (the prequantized entry point,
 // neuralfn/csrc/native_train/tile_ops.h:698-709).  kHalfImage likewise: the fp16 image of
 // the fp16 small-batch kernel already lies in the workspace (written by the dual RMS kernel).
-enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2, kRecords = 3, kHalfImage = 4 };
+// kDualNorm: the input is the result of the two normalisations of a layer's input, which the
+// decode kernel computes in its own prologue (one row).
+enum Prologue : int { kPlain = 0, kGated = 1, kSwiGlu = 2, kRecords = 3, kHalfImage = 4, kDualNorm = 5 };
 
 #if defined(__HIPCC__)
 

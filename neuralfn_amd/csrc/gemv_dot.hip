@@ -31,6 +31,7 @@
 // c = 256*hi + lo:  y += s*(d*sum_sub sc*dot(q, c) - dmin*sum_sub m*sum(c)).
 #include "common.hpp"
 #include "gemv_dot.hpp"
+#include "rms_device.hpp"
 #include "wave_rows.hpp"
 
 namespace nfn {
@@ -226,6 +227,7 @@ struct DotTail {
     int pad;
     float* output[4];
     std::int64_t output_dim[4];
+    DualNormArguments norm;  // prologue kDualNorm only
 };
 
 
@@ -350,13 +352,21 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // (rows of more than 8,192 columns: eight, i.e. every record of a 16,384-column row)
     constexpr int kEarly = ITER > 0 ? 4 : 8;
     float4 early[kEarly];
+    constexpr int kNormLoaders = kDotThreads / kRmsThreads;
+    DualRmsOperands<kNormLoaders> norm_operands;
+    if constexpr (P == kDualNorm) {
+        // the operands of the two normalisations instead: `first` is the row to normalise
+        dual_rms_request<kNormLoaders>(norm_operands, first, tail.norm.residual,
+                                       tail.norm.first_weight, tail.norm.second_weight, input_dim);
+    } else {
 #pragma unroll
-    for (int e = 0; e < kEarly; ++e) {
-        const int record = min(wave + e * kDotWaves, records - 1);
-        const int token = token_of_record<T>(record, blocks);
-        const int block = record - token * blocks;
-        early[e] = load_activations<P>(pass_first, pass_second,
-                                       static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
+        for (int e = 0; e < kEarly; ++e) {
+            const int record = min(wave + e * kDotWaves, records - 1);
+            const int token = token_of_record<T>(record, blocks);
+            const int block = record - token * blocks;
+            early[e] = load_activations<P>(pass_first, pass_second,
+                                           static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
+        }
     }
 
     // (2) weight loads of the first two (row, slice) pairs.  A stage beyond the wave's
@@ -432,6 +442,21 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // for a later launch that shares this input.
     std::uint8_t* const records_out = tail.records_out;
     const bool keep_records = P != kRecords && records_out != nullptr && blockIdx.x == 0;
+    if constexpr (P == kDualNorm) {
+        // Every workgroup normalises the row for itself (the first one also stores the
+        // results); the normalized row then waits in LDS where the records are made from it.
+        __shared__ __attribute__((aligned(16))) float normalized_row[kRmsOwned * kRmsThreads];
+        __shared__ float norm_partials[kRmsThreads + 1];
+        dual_rms_finish<kNormLoaders>(norm_operands, input_dim, tail.norm.first_eps,
+                                      tail.norm.second_eps, blockIdx.x == 0, tail.norm.hidden,
+                                      tail.norm.captured, tail.norm.normalized, normalized_row,
+                                      norm_partials);
+#pragma unroll
+        for (int e = 0; e < kEarly; ++e) {
+            const int record = min(wave + e * kDotWaves, records - 1);
+            early[e] = *reinterpret_cast<const float4*>(normalized_row + record * 256 + lane * 4);
+        }
+    }
     auto quantize_record = [&](float4 loaded, int record) {
         const int token = token_of_record<T>(record, blocks);
         const int block = record - token * blocks;
@@ -447,13 +472,15 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
         const int record = wave + e * kDotWaves;
         if (record < records) quantize_record(early[e], record);
     }
-    for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
-        const int token = token_of_record<T>(record, blocks);
-        const int block = record - token * blocks;
-        const float4 x = load_activations<P>(
-            pass_first, pass_second,
-            static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
-        quantize_record(x, record);
+    if constexpr (P != kDualNorm) {  // (a normalised row has at most 32 records: all early)
+        for (int record = wave + kEarly * kDotWaves; record < records; record += kDotWaves) {
+            const int token = token_of_record<T>(record, blocks);
+            const int block = record - token * blocks;
+            const float4 x = load_activations<P>(
+                pass_first, pass_second,
+                static_cast<std::int64_t>(token) * input_dim + block * 256 + lane * 4);
+            quantize_record(x, record);
+        }
     }
     if constexpr (kStages == 3) issue(stages[2], 2 % kSlices);
     __syncthreads();
@@ -477,7 +504,7 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
     // `slice`: for ITER > 0 the slice of its row this step works on
     auto compute = [&](const Stage<kQ5>& stage, int slice) {
         const int iteration = work.iteration;
-        const int raw_unit = (PAIRS ? iteration % ITER : iteration) * kWave + lane;
+        const int raw_unit = (PAIRS ? iteration % (ITER > 0 ? ITER : 1) : iteration) * kWave + lane;
         const bool live = raw_unit < units;
         const int unit = min(raw_unit, units - 1);
         if constexpr (ITER > 0) {
@@ -529,7 +556,8 @@ __global__ __launch_bounds__(kDotThreads) void gemv_dot_kernel(
 
 template <std::uint32_t ENC, int T, int P>
 void launch_variant(ProjectionSet set, const float* first, const float* second,
-                    std::uint8_t* records_out, int tokens, hipStream_t stream) {
+                    std::uint8_t* records_out, int tokens, hipStream_t stream,
+                    const DualNormArguments* norm = nullptr) {
     std::int64_t rows = 0;
     int bounds[4] = {0, 0x7fffffff, 0x7fffffff, 0x7fffffff};
     const void* data[4] = {set.op[0].data, set.op[0].data, set.op[0].data, set.op[0].data};
@@ -537,6 +565,7 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
     tail.second = second;
     tail.records_out = records_out;
     tail.tokens = tokens;
+    if (norm != nullptr) tail.norm = *norm;
     for (int index = 0; index < set.count; ++index) {
         bounds[index] = static_cast<int>(rows);
         data[index] = set.op[index].data;
@@ -556,36 +585,38 @@ void launch_variant(ProjectionSet set, const float* first, const float* second,
                            static_cast<int>(rows % groups), bounds[1], bounds[2], bounds[3], tail);
     };
     const std::int64_t slices = (4 * blocks + kWave - 1) / kWave;
+    // (the norm prologue keeps 33 KB of static LDS: less room for the dynamic part)
+    constexpr int kDynamicLds = (P == kDualNorm ? 120 : 160) * 1024;
     if constexpr (T == 1) {
         // one workgroup per compute unit: three stages, the third requested late
         const bool small = groups <= compute_units();
         if (slices == 1) {
             if (small) {
-                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 3>>();
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 3>>(kDynamicLds);
                 launch(gemv_dot_kernel<ENC, T, P, 1, 3>);
             } else {
-                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 2>>();
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 1, 2>>(kDynamicLds);
                 launch(gemv_dot_kernel<ENC, T, P, 1, 2>);
             }
             return;
         }
         if (slices == 2) {
             if (small) {
-                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 3>>();
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 3>>(kDynamicLds);
                 launch(gemv_dot_kernel<ENC, T, P, 2, 3>);
             } else {
-                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 2>>();
+                allow_large_lds<gemv_dot_kernel<ENC, T, P, 2, 2>>(kDynamicLds);
                 launch(gemv_dot_kernel<ENC, T, P, 2, 2>);
             }
             return;
         }
         if (small) {
-            allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 3>>();
+            allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 3>>(kDynamicLds);
             launch(gemv_dot_kernel<ENC, T, P, 0, 3>);
             return;
         }
     }
-    allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 2>>();
+    allow_large_lds<gemv_dot_kernel<ENC, T, P, 0, 2>>(kDynamicLds);
     launch(gemv_dot_kernel<ENC, T, P, 0, 2>);
 }
 
@@ -672,6 +703,24 @@ void launch_prologue(const ProjectionSet& set, const float* first, const float* 
 bool gemv_dot_supports(std::uint32_t encoding, std::int64_t input_dim) {
     return (encoding == kEncQ4K || encoding == kEncQ5K) && input_dim % 256 == 0 &&
         token_image_bytes_host(input_dim >> 8) <= 150 * 1024;
+}
+
+bool gemv_dot_normed_supports(const ProjectionSet& set) {
+    // one launch: one encoding; register-resident activations and norm operands
+    for (int index = 0; index < set.count; ++index) {
+        if (set.op[index].encoding != set.op[0].encoding) return false;
+    }
+    return set.count > 0 && gemv_dot_supports(set.op[0].encoding, set.input_dim) &&
+        set.input_dim <= kRmsOwned * kRmsThreads;
+}
+
+void launch_gemv_dot_normed(const ProjectionSet& set, const float* input,
+                            const DualNormArguments& norm, hipStream_t stream) {
+    if (set.op[0].encoding == kEncQ4K) {
+        launch_variant<kEncQ4K, 1, kDualNorm>(set, input, nullptr, nullptr, 1, stream, &norm);
+    } else {
+        launch_variant<kEncQ5K, 1, kDualNorm>(set, input, nullptr, nullptr, 1, stream, &norm);
+    }
 }
 
 bool gemv_dot_pairs_supports(std::uint32_t first_encoding, std::uint32_t second_encoding,

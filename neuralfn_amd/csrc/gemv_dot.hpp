@@ -16,6 +16,15 @@ void launch_gemv_dot(const ProjectionSet& set, const float* first, const float* 
                      std::uint8_t* records_out, int prologue, std::int64_t rows,
                      hipStream_t stream);
 
+// One token: hidden = residual + rms(input), normalized = rms(hidden) in the launch's own
+// prologue (every workgroup for itself, the first also stores the three rows), then the
+// projections of `set` on the normalized row.  All projections of one encoding, input_dim at
+// most 8192.
+struct DualNormArguments;
+bool gemv_dot_normed_supports(const ProjectionSet& set);
+void launch_gemv_dot_normed(const ProjectionSet& set, const float* input,
+                            const DualNormArguments& norm, hipStream_t stream);
+
 // One token through two projections of one shape and encoding (gate, up) with the SwiGLU
 // activation at the row ends: output r = (up_r gate_r) sigmoid(gate_r), the value the SwiGLU
 // prologue of the projection behind would compute from the two separate outputs.

@@ -23,59 +23,14 @@
 #include "common.hpp"
 #include "f16_decode.hpp"
 #include "kernels.hpp"
+#include "rms_device.hpp"
 #include "wave_rows.hpp"
 
 namespace nfn {
 
 namespace {
 
-constexpr int kRmsThreads = 256;
 constexpr int kBatch = 8;  // columns per thread whose loads are issued together
-
-// Affine weight of one normalisation: a [1, width] packed row, or none.
-struct NormWeight {
-    const std::uint8_t* data;
-    std::uint32_t encoding;
-    int present;
-    int centered;  // the stored weight is (scale - 1)
-};
-
-__device__ __forceinline__ float norm_scale(const NormWeight& weight, std::int64_t column) {
-    if (!weight.present) return 1.0f;
-    float scale = weight_value(weight.encoding, weight.data, column);
-    if (weight.centered) scale += 1.0f;
-    return scale;
-}
-
-// The scales of N columns at once.  The encoding is looked at once, outside the
-// loop, so that for float and bf16 rows (what norm weights are) the N loads are
-// plain and independent and go out together instead of one behind the other's
-// branch.
-template <int N, typename Index>
-__device__ __forceinline__ void norm_scales(const NormWeight& weight, const Index (&columns)[N],
-                                            float (&scale)[N]) {
-    if (!weight.present) {
-#pragma unroll
-        for (int i = 0; i < N; ++i) scale[i] = 1.0f;
-        return;
-    }
-    if (weight.encoding == kEncF32) {
-        const float* values = reinterpret_cast<const float*>(weight.data);
-#pragma unroll
-        for (int i = 0; i < N; ++i) scale[i] = values[columns[i]];
-    } else if (weight.encoding == kEncBF16) {
-        const std::uint16_t* values = reinterpret_cast<const std::uint16_t*>(weight.data);
-#pragma unroll
-        for (int i = 0; i < N; ++i) scale[i] = bf16_to_float(values[columns[i]]);
-    } else {
-#pragma unroll
-        for (int i = 0; i < N; ++i) scale[i] = weight_value(weight.encoding, weight.data, columns[i]);
-    }
-    if (weight.centered) {
-#pragma unroll
-        for (int i = 0; i < N; ++i) scale[i] += 1.0f;
-    }
-}
 
 // 1 / sqrt(mean of squares + eps) of `values[0, width)`, the same number in every thread.
 __device__ __forceinline__ float inverse_rms(const float* values, std::int64_t width, float eps,
@@ -207,28 +162,10 @@ __device__ __forceinline__ float tree_total(float square_sum, float* partials) {
 // does the element-wise arithmetic of its own columns.  The second
 // normalisation needs no second pass over memory.  Same arithmetic, same order,
 // same bits as the kernel above.
-constexpr int kOwned = 32;      // columns per sum
+constexpr int kOwned = kRmsOwned;
 constexpr int kLoaders = 4;     // threads that share the loads of a sum
 constexpr int kWideThreads = kRmsThreads * kLoaders;
 constexpr int kLoaded = kOwned / kLoaders;  // columns per thread
-
-// The halving tree over the 256 sums of threads (0, t), additions in the order of
-// tree_total: (p[t] + p[t+128]) + (p[t+64] + p[t+192]) is its first two levels,
-// the last six run inside the first wave.  Every thread of the workgroup calls it.
-__device__ __forceinline__ float tree_total_wide(float square_sum, float* partials) {
-    if (threadIdx.x < kRmsThreads) partials[threadIdx.x] = square_sum;
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        const float a = partials[threadIdx.x] + partials[threadIdx.x + 128];
-        const float b = partials[threadIdx.x + 64] + partials[threadIdx.x + 192];
-        float value = a + b;
-#pragma unroll
-        for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
-        if (threadIdx.x == 0) partials[kRmsThreads] = value;
-    }
-    __syncthreads();
-    return partials[kRmsThreads];
-}
 
 // HANDOFF 0: nothing more; 1: the activation records of the normalized row (one row);
 // 2: the normalized rows as the fp16 image of the fp16 small-batch kernel, `records` being
@@ -282,7 +219,7 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     for (int i = 0; i < kLoaded; ++i) handed[(q + kLoaders * i) * kRmsThreads + t] = value[i];
     __syncthreads();
     const float first_inverse =
-        1.0f / sqrtf(tree_total_wide(ordered_sum(), partials) / static_cast<float>(width) + first_eps);
+        1.0f / sqrtf(rms_tree_total(ordered_sum(), partials) / static_cast<float>(width) + first_eps);
 
 #pragma unroll
     for (int i = 0; i < kLoaded; ++i) {
@@ -299,7 +236,7 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     }
     __syncthreads();
     const float second_inverse =
-        1.0f / sqrtf(tree_total_wide(ordered_sum(), partials) / static_cast<float>(width) + second_eps);
+        1.0f / sqrtf(rms_tree_total(ordered_sum(), partials) / static_cast<float>(width) + second_eps);
 
     float largest = 0.0f;
 #pragma unroll
@@ -520,16 +457,6 @@ __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
     }
 }
 
-NormWeight norm_weight(const Descriptor* descriptor, bool centered) {
-    NormWeight weight{};
-    if (descriptor != nullptr) {
-        weight.data = descriptor->data;
-        weight.encoding = descriptor->encoding;
-        weight.present = 1;
-        weight.centered = centered ? 1 : 0;
-    }
-    return weight;
-}
 
 }  // namespace
 

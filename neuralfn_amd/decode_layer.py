@@ -81,7 +81,8 @@ class LayerCache:
 
 def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
                  pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
-                 attention_workspace=None, fused_gate_up: bool = False):
+                 attention_workspace=None, fused_gate_up: bool = False,
+                 fused_input_norm: bool = False):
     """One token through one layer.
 
     `pending` is the previous layer's down-projection output whose post-feed-forward norm and
@@ -92,14 +93,21 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     `fused_gate_up`: the gate and up projections in one call with the SwiGLU activation at the
     row ends (nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1) where the pair allows it, so
     that the down projection reads one plain vector; the same bits as the separate calls.
+    `fused_input_norm`: the first dual norm inside the launch of the projections it feeds
+    (nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1) where those allow it; the same bits.
     """
     g = geometry
     # hidden = residual + rms(pending); normalized = rms(hidden, input_norm)
-    hidden, normalized, _ = tile_ops.dual_rms_add_capture(
-        pending, residual, pending_norm, False, weights.input_norm, False,
-        g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps)
-    query, key, value, gate = tile_ops.multi_linear(
-        [weights.q, weights.k, weights.v, weights.attention_gate], normalized, workspace)
+    first_eps = g.post_norm_eps if pending_norm is not None else g.norm_eps
+    attention_inputs = [weights.q, weights.k, weights.v, weights.attention_gate]
+    if fused_input_norm and tile_ops.dual_rms_multi_linear_supported(attention_inputs, g.model_dim):
+        hidden, normalized, _, (query, key, value, gate) = tile_ops.dual_rms_multi_linear(
+            pending, residual, attention_inputs, pending_norm, False, weights.input_norm, False,
+            first_eps, g.norm_eps)
+    else:
+        hidden, normalized, _ = tile_ops.dual_rms_add_capture(
+            pending, residual, pending_norm, False, weights.input_norm, False, first_eps, g.norm_eps)
+        query, key, value, gate = tile_ops.multi_linear(attention_inputs, normalized, workspace)
     # per-head norms and rope in one launch, attention, the cache commit
     query = query.view(g.query_heads, g.head_dim)
     key = key.view(g.kv_heads, g.head_dim)
@@ -187,3 +195,4 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
 
 LAUNCHES_PER_LAYER = 8           # with the reference's fused attention call
 LAUNCHES_PER_LAYER_SPLIT = 9     # with the split attention form (one more: the merge)
+LAUNCHES_PER_LAYER_FUSED = 8     # ... and the first dual norm inside the Q/K/V/gate launch

@@ -185,6 +185,9 @@ SIGNATURES = {
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
     "nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1": (ctypes.c_int, [_DESC, _DESC, _P, _P, _P]),
+    "nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _DESC_ARRAY, _PTR_ARRAY, _I64, _P]),
     "nfn_native_tile_argmax_rows_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _I64, _P]),
     "nfn_native_tile_glimmer_sigmoid_gate_float32_v1": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
     "nfn_native_tile_swiglu_float32": (ctypes.c_int, [_P, _P, _P, _I64, _P]),
@@ -490,6 +493,40 @@ def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = Non
             *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
             "dual_rms_add_capture_mmq_f16")
     return hidden, normalized, captured
+
+
+def dual_rms_multi_linear(x, residual, weights: Sequence[PackedWeight],
+                          first_weight: Optional[PackedWeight] = None, first_centered: bool = False,
+                          second_weight: Optional[PackedWeight] = None,
+                          second_centered: bool = False, first_eps: float = 1e-6,
+                          second_eps: float = 1e-6, outputs=None):
+    """nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1: one row through the two normalisations
+    and the projections of their result in one launch.
+    Returns (hidden, normalized, residual_output, outputs)."""
+    import torch
+    stream = _stream_handle()
+    width = x.shape[1]
+    hidden, normalized, captured = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    if outputs is None:
+        outputs = [torch.empty((1, w.output_dim), dtype=torch.float32, device=x.device)
+                   for w in weights]
+    first = first_weight.descriptor(stream) if first_weight is not None else None
+    second = second_weight.descriptor(stream) if second_weight is not None else None
+    descriptors = [w.descriptor(stream) for w in weights]
+    check(load().nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1(
+        x.data_ptr(), ctypes.byref(first) if first is not None else None, residual.data_ptr(),
+        hidden.data_ptr(), ctypes.byref(second) if second is not None else None,
+        normalized.data_ptr(), captured.data_ptr(), width, first_eps, first_centered, second_eps,
+        second_centered, _descriptor_array(descriptors), _pointer_array(outputs), len(weights),
+        stream), "dual_rms_mmvq_multi_linear")
+    return hidden, normalized, captured, outputs
+
+
+def dual_rms_multi_linear_supported(weights: Sequence[PackedWeight], width: int) -> bool:
+    """Whether dual_rms_multi_linear takes these projections (else: the two calls)."""
+    return (1 <= len(weights) <= 4 and width % 256 == 0 and width <= 8192 and
+            all(w.encoding == weights[0].encoding and w.input_dim == width for w in weights) and
+            weights[0].encoding in (kquant.Q4_K, kquant.Q5_K))
 
 
 def mmvq_linear(weight: PackedWeight, x, workspace, out=None):

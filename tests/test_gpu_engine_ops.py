@@ -945,10 +945,12 @@ def test_two_decode_layers_against_the_cpu_engine_arithmetic(cuda, oracle):
         assert np.array_equal(bits_of(cache.keys)[untouched], keys[untouched])
 
 
-def test_decode_layer_with_gate_and_up_in_one_call_gives_the_same_bits(cuda, oracle):
-    """decode_layer(fused_gate_up=True) takes gate and up through
-    nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1 and the down projection on its plain
-    output: the layer's two results equal the separate calls' bit for bit."""
+def test_decode_layer_with_the_fused_calls_gives_the_same_bits(cuda, oracle):
+    """decode_layer(fused_gate_up=True, fused_input_norm=True) takes gate and up through
+    nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1 (the down projection on its plain output)
+    and the first dual norm inside the Q/K/V/gate launch
+    (nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1): the layer's two results and the
+    committed cache rows equal the separate calls' bit for bit."""
     from neuralfn_amd import decode_layer as dl
     rng = np.random.default_rng(23)
     g = dl.LayerGeometry(model_dim=768, query_heads=4, kv_heads=2, head_dim=64, ffn_dim=1280,
@@ -974,13 +976,18 @@ def test_decode_layer_with_gate_and_up_in_one_call_gives_the_same_bits(cuda, ora
     embedding = to_device(rng.standard_normal((1, g.model_dim)).astype(np.float32), cuda)
     workspace = tile_ops.small_batch_workspace(1, max(g.model_dim, g.ffn_dim))
     results = []
+    assert tile_ops.dual_rms_multi_linear_supported(
+        [weights.q, weights.k, weights.v, weights.attention_gate], g.model_dim)
     for fused in (False, True):
         cache = dl.LayerCache(g, cuda)
         cache.keys.copy_(bf16_tensor(keys, cuda))
         cache.values.copy_(bf16_tensor(values, cuda))
         results.append(dl.decode_layer(g, weights, cache, embedding, torch_().zeros_like(embedding),
-                                       None, 150, workspace, fused_gate_up=fused))
-    assert torch_().equal(results[0][0], results[1][0]) and torch_().equal(results[0][1], results[1][1])
+                                       None, 150, workspace, fused_gate_up=fused,
+                                       fused_input_norm=fused))
+        results[-1] += (cache.keys.clone(), cache.values.clone())
+    for separate, together in zip(results[0], results[1]):
+        assert torch_().equal(separate, together)
     assert bool(torch_().isfinite(results[1][0]).all())
 
 

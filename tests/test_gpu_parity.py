@@ -891,6 +891,72 @@ def test_dual_rms_block_handoff_equals_ordinary_path(cuda, oracle, rows, width):
             assert normalised_error(y.cpu().numpy()[row], exact[row]) <= TOLERANCE
 
 
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
+@pytest.mark.parametrize("width", [256, 4096, 6656, 8192])
+@pytest.mark.parametrize("weights", ["none", "f32", "bf16_centered"])
+def test_dual_rms_inside_the_projection_launch_equals_the_two_calls(cuda, oracle, encoding, width, weights):
+    """nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1: the three rows of the norm kernel and
+    the projections of the normalized row, bit for bit what the dual RMS call followed by the
+    grouped one-row call gives."""
+    rng = np.random.default_rng(width + encoding)
+    x = (rng.standard_normal((1, width)) * 3.0).astype(np.float32)
+    residual = rng.standard_normal((1, width)).astype(np.float32)
+    first = second = None
+    centered = weights == "bf16_centered"
+    if weights != "none":
+        kind = kquant.F32 if weights == "f32" else kquant.BF16
+        make = lambda seed: tile_ops.PackedWeight.from_numpy(
+            kind, kquant.quantize(kind, np.random.default_rng(seed).uniform(-0.3, 0.3, (1, width)).astype(np.float32)
+                                  + (0.0 if centered else 1.0)), 1, width)
+        first, second = make(1), make(2)
+    specs = [129, 33, 70, 300] if width <= 4096 else [4096, 256, 256, 4096]
+    projections = [tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, n, width, 50 + i), n, width)
+                   for i, n in enumerate(specs)]
+    workspace = tile_ops.small_batch_workspace(1, width)
+    arguments = dict(first_weight=first, first_centered=centered, second_weight=second,
+                     second_centered=centered, first_eps=1e-8, second_eps=1e-5)
+    ordinary = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda), **arguments)
+    ordinary_out = tile_ops.multi_linear(projections, ordinary[1], workspace)
+    fused = tile_ops.dual_rms_multi_linear(to_device(x, cuda), to_device(residual, cuda), projections,
+                                           **arguments)
+    for a, b, label in zip(ordinary, fused[:3], ("hidden", "normalized", "capture")):
+        assert_bits_equal(a, b, label)
+    for a, b, n in zip(ordinary_out, fused[3], specs):
+        assert_bits_equal(a, b, f"projection of {n} rows")
+
+
+def test_dual_rms_inside_the_projection_launch_fails_closed(cuda):
+    lib = tile_ops.load()
+    width = 512
+    x = to_device(probe_rms_input(1, width), cuda)
+    rows = [torch_().empty_like(x) for _ in range(3)]
+    make = lambda e, n, k, seed: tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, k, seed), n, k)
+    good, five, six = make(kquant.Q4_K, 24, width, 1), make(kquant.Q5_K, 24, width, 2), make(kquant.Q6_K, 24, width, 3)
+    out = [torch_().empty((1, 24), dtype=torch_().float32, device=cuda) for _ in range(2)]
+    call = lib.nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1
+    head = [x.data_ptr(), None, x.data_ptr(), rows[0].data_ptr(), None, rows[1].data_ptr(), rows[2].data_ptr()]
+    tail = [1e-8, False, 1e-5, False]
+    def run(weights, width_argument=width, count=None, head_arguments=head, tail_arguments=tail):
+        descriptors = tile_ops._descriptor_array([w.descriptor(0) for w in weights])
+        pointers = tile_ops._pointer_array(out[:len(weights)])
+        return call(*head_arguments, width_argument, *tail_arguments, descriptors, pointers,
+                    len(weights) if count is None else count, None)
+    assert run([good, good]) == 0
+    assert run([good, five]) == 1          # two encodings: two launches, not this call
+    assert run([six]) == 1                 # no dot kernel of this form
+    assert run([good], count=0) == 1
+    assert run([good], width_argument=256) == 1   # the projections' input width differs
+    assert run([good], tail_arguments=[0.0, False, 1e-5, False]) == 1
+    assert run([good], head_arguments=[None] + head[1:]) == 1
+    wide = make(kquant.Q4_K, 8, 8448, 4)
+    wide_x = to_device(probe_rms_input(1, 8448), cuda)
+    wide_rows = [torch_().empty_like(wide_x) for _ in range(3)]
+    wide_head = [wide_x.data_ptr(), None, wide_x.data_ptr(), wide_rows[0].data_ptr(), None,
+                 wide_rows[1].data_ptr(), wide_rows[2].data_ptr()]
+    assert run([wide], width_argument=8448, head_arguments=wide_head) == 1
+    torch_().cuda.synchronize()
+
+
 def test_block_handoff_fails_closed(cuda):
     width = 512
     lib = tile_ops.load()
