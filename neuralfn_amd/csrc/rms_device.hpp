@@ -70,21 +70,20 @@ struct DualNormArguments {
 
 // The halving tree over the 256 sums of threads (0, t), additions in the order of the
 // reference's tree: (p[t] + p[t+128]) + (p[t+64] + p[t+192]) is its first two levels, the last
-// six run inside the first wave.  Every thread of the workgroup calls it; `partials` holds
-// kRmsThreads + 1 floats.
+// six run inside a wave.  Every thread of the workgroup calls it; every wave runs the tree
+// for itself on the same 256 numbers (the same operations, the same result), which spares
+// the barrier that handing one wave's total to the others would take.  `partials` holds
+// kRmsThreads floats and may be written again after the workgroup's next barrier.
 __device__ __forceinline__ float rms_tree_total(float square_sum, float* partials) {
     if (threadIdx.x < kRmsThreads) partials[threadIdx.x] = square_sum;
     __syncthreads();
-    if (threadIdx.x < 64) {
-        const float a = partials[threadIdx.x] + partials[threadIdx.x + 128];
-        const float b = partials[threadIdx.x + 64] + partials[threadIdx.x + 192];
-        float value = a + b;
+    const int lane = threadIdx.x & 63;
+    const float a = partials[lane] + partials[lane + 128];
+    const float b = partials[lane + 64] + partials[lane + 192];
+    float value = a + b;
 #pragma unroll
-        for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
-        if (threadIdx.x == 0) partials[kRmsThreads] = value;
-    }
-    __syncthreads();
-    return partials[kRmsThreads];
+    for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
+    return __shfl(value, 0, 64);
 }
 
 // One row of the two normalisations by a workgroup of LOADERS x 256 threads, rows of up to
