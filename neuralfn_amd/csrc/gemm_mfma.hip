@@ -736,6 +736,8 @@ __global__ __launch_bounds__(256) void sum_shares_kernel(const float* __restrict
 // (128-row tiles) workgroup slots; the shares are summed by a second launch in
 // a fixed order.  256-row tiles stay the better choice as long as two shares or
 // more fit; at most 128 rows, or a K too short to split, take 128-row tiles.
+// Narrow projections (an eighth of the units' count in 256-row tiles at most) take
+// 128-row tiles and shares of six blocks or more.
 struct Plan {
     int row_blocks;  // 32-row blocks per wave: 2 = 256-row tiles, 1 = 128-row tiles
     int shares;
@@ -749,6 +751,19 @@ Plan plan(std::uint32_t encoding, std::int64_t rows, std::int64_t output_dim,
     if (tall_tiles >= units) return Plan{2, 1};
     std::int64_t longest = (input_dim >> 8) / 12;  // shares that still get twelve blocks each
     if (longest > kMaxShares) longest = kMaxShares;
+    if (tall_tiles * 8 <= units) {
+        // A narrow projection (a few tiles for the whole chip, e.g. 256 outputs): what it
+        // takes is the length of one workgroup's walk over K, so the shares may be as short
+        // as six blocks and the tiles are the small ones (1,024 x 6,656 -> 256: 53 -> 34 us).
+        std::int64_t shortest = (input_dim >> 8) / 6;
+        if (shortest > kMaxShares) shortest = kMaxShares;
+        if (shortest < 1) shortest = 1;
+        const std::int64_t tiles = (rows + 127) / 128 * n_tiles;
+        std::int64_t shares = units * 3 / tiles;
+        if (shares > shortest) shares = shortest;
+        if (shares < 1) shares = 1;
+        return Plan{1, static_cast<int>(shares)};
+    }
     if (rows > 128) {
         std::int64_t shares = 2 * units / tall_tiles;
         if (shares > longest) shares = longest;

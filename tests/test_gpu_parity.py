@@ -1123,17 +1123,32 @@ def test_prefill_gemm_tall_tiles(cuda, oracle, encoding):
     assert normalised_error(y[picked], expected) <= TOLERANCE
 
 
+def test_prefill_gemm_plans():
+    # Host logic only.  A problem of many tiles but not one per compute unit: shares of at
+    # least twelve 256-value blocks, 256-row tiles while two shares or more fit.
+    wide = 33 * 128
+    assert tile_ops.gemm_plan(kquant.Q4_K, 96, 4096, wide) == (128, 1)    # sixteen blocks: one share
+    assert tile_ops.gemm_plan(kquant.Q4_K, 96, 6144, wide) == (128, 2)
+    assert tile_ops.gemm_plan(kquant.Q4_K, 96, 9216, wide) == (128, 3)
+    assert tile_ops.gemm_plan(kquant.Q4_K, 200, 9216, wide) == (256, 3)
+    assert tile_ops.gemm_plan(kquant.Q4_K, 200, 12544, wide) == (256, 4)
+    assert tile_ops.gemm_plan(kquant.Q4_K, 2048, 6656, 16384) == (256, 1)
+    # A narrow projection (the K and V projections of the workload): small tiles, short shares.
+    assert tile_ops.gemm_plan(kquant.Q4_K, 1024, 6656, 256) == (128, 4)
+    assert tile_ops.gemm_plan(kquant.Q6_K, 2048, 6656, 256) == (128, 4)
+
+
 @pytest.mark.parametrize("rows,in_dim,plan", [
-    (96, 4096, (128, 1)),    # sixteen blocks: too short to give two shares twelve each
-    (96, 6144, (128, 2)),    # 24 blocks -> two shares of 128-row tiles
-    (96, 9216, (128, 3)),    # 36 blocks -> three
-    (200, 9216, (256, 3)),   # more than 128 rows keep 256-row tiles while two shares or more fit
-    (200, 12544, (256, 4)),  # 49 blocks -> four shares of unequal length (13, 12, 12, 12)
+    (96, 1536, (128, 1)),    # six blocks: one share
+    (96, 3072, (128, 2)),    # twelve blocks -> two shares of six
+    (96, 4608, (128, 3)),    # eighteen -> three
+    (200, 6656, (128, 4)),   # 26 blocks -> four shares of unequal length (7, 7, 6, 6)
+    (200, 12544, (128, 4)),  # 49 blocks -> (13, 12, 12, 12)
 ])
 @pytest.mark.parametrize("encoding", ALL_PACKED)
 def test_prefill_gemm_split_k(cuda, oracle, encoding, rows, in_dim, plan):
-    # few tiles and a long K: the launch splits K into shares of at least twelve
-    # 256-value blocks (at most four) and a second launch sums them in share order
+    # few tiles and a long K: the launch splits K into shares (of at least six 256-value
+    # blocks for a narrow projection, at most four) and a second launch sums them in share order
     out_dim = 130
     assert tile_ops.gemm_plan(encoding, rows, in_dim, out_dim) == plan
     packed = kquant.quantize(encoding, kquant.synthetic_weights(70 + encoding, out_dim, in_dim))
