@@ -725,9 +725,12 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
 def memory_rate_extra(device, stream, steps: int, warmup: int) -> dict:
     """What the vendor library's own streaming kernels reach on this GPU: a float sum (read
     only) and a copy (read + write) over buffers below and far above the 256 MB the memory-side
-    cache holds.  The comparator for every HBM-bound figure here, next to the published 8 TB/s."""
+    cache holds, and this library's read-only probe kernel over the same buffers.  The
+    comparators for every HBM-bound figure here, next to the published 8 TB/s."""
     import torch
-    result = {"workload": "torch.sum / Tensor.copy_ over a float32 buffer, TB/s of bytes moved"}
+    from neuralfn_amd import tile_ops
+    result = {"workload": "torch.sum / Tensor.copy_ / this library's read-only probe kernel over a "
+                          "float32 buffer, TB/s of bytes moved"}
     steps, warmup = max(5, steps // 2), max(2, warmup // 2)
     for mib in (256, 2048):
         source = torch.empty(mib * (1 << 20) // 4, dtype=torch.float32, device=device).normal_()
@@ -735,8 +738,16 @@ def memory_rate_extra(device, stream, steps: int, warmup: int) -> dict:
         nbytes = source.numel() * 4
         read_ms = time_replays(lambda: source.sum(), steps, warmup)
         copy_ms = time_replays(lambda: target.copy_(source), steps, warmup)
+        # this library's own read-only kernel (nfn_mi355_read_probe_v1: one workgroup per
+        # compute unit streams its share in 16-byte pieces and stores nothing): what a kernel
+        # of the decode kernels' shape can read at best
+        sink = torch.zeros(1024, dtype=torch.int32, device=device)
+        handle = int(torch.cuda.current_stream().cuda_stream)
+        probe_ms = time_replays(lambda: tile_ops.check(tile_ops.load().nfn_mi355_read_probe_v1(
+            source.data_ptr(), nbytes, sink.data_ptr(), handle), "read probe"), steps, warmup)
         result[f"{mib}_MiB"] = {"sum_read_TB/s": round(nbytes / read_ms / 1e9, 2),
-                                "copy_read_plus_write_TB/s": round(2 * nbytes / copy_ms / 1e9, 2)}
+                                "copy_read_plus_write_TB/s": round(2 * nbytes / copy_ms / 1e9, 2),
+                                "read_probe_TB/s": round(nbytes / probe_ms / 1e9, 2)}
         del source, target
     return result
 
