@@ -518,6 +518,25 @@ def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
         result[f"rows{rows}"] = {"ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
                                  "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
                                  "tokens/s": round(rows / ms * 1e3, 1)}
+    # The verifier's block of 16 rows: beyond the fused call's eight rows, so the reference's own
+    # pair, the small-batch linear (logits to memory) and the row argmax.
+    rows = 16
+    x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
+    workspace = tile_ops.small_batch_workspace(rows, MODEL_DIM, device)
+    logits = torch.empty((rows, VOCAB), dtype=torch.float32, device=device)
+    indices = torch.empty(rows, dtype=torch.int64, device=device)
+    values = torch.empty(rows, dtype=torch.float32, device=device)
+
+    def block():
+        tile_ops.multi_linear([weight], x, workspace, outputs=[logits])
+        tile_ops.argmax_rows(logits, indices, values)
+
+    ms = time_graph(block, stream, steps, warmup)
+    traffic = weight.nbytes + rows * MODEL_DIM * 4 + 2 * rows * VOCAB * 4
+    result["rows16_linear_then_argmax"] = {
+        "ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
+        "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
+        "tokens/s": round(rows / ms * 1e3, 1)}
     return {"workload": f"Q6_K lm_head {MODEL_DIM}->{VOCAB}, fused argmax", **result}
 
 

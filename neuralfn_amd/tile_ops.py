@@ -601,11 +601,13 @@ def linear_q8_1_multi_decode(weights: Sequence[PackedWeight], codes, scales, sum
     return outputs
 
 
-def argmax_rows(values):
+def argmax_rows(values, indices=None, maxima=None):
     import torch
     rows, width = values.shape
-    indices = torch.empty(rows, dtype=torch.int64, device=values.device)
-    maxima = torch.empty(rows, dtype=torch.float32, device=values.device)
+    if indices is None:
+        indices = torch.empty(rows, dtype=torch.int64, device=values.device)
+    if maxima is None:
+        maxima = torch.empty(rows, dtype=torch.float32, device=values.device)
     check(load().nfn_native_tile_argmax_rows_float32_v1(
         values.data_ptr(), indices.data_ptr(), maxima.data_ptr(), rows, width,
         _stream_handle()), "argmax_rows")
