@@ -506,7 +506,9 @@ def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
     from neuralfn_amd import kquant, tile_ops
     weight = random_packed_on_device(kquant.Q6_K, VOCAB, MODEL_DIM, device, 7)
     result = {}
-    for rows in (1, 4):
+    # one row: the streaming dot kernel; four: the int8 matrix-core kernel; eight and sixteen
+    # (a verifier block): the fp16 matrix-core kernel behind its conversion launch
+    for rows in (1, 4, 8, 16):
         x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
         nbytes = tile_ops.load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, VOCAB)
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -518,8 +520,8 @@ def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
         result[f"rows{rows}"] = {"ms": round(ms, 4), "GB/s": round(traffic / ms / 1e6, 1),
                                  "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
                                  "tokens/s": round(rows / ms * 1e3, 1)}
-    # The verifier's block of 16 rows: beyond the fused call's eight rows, so the reference's own
-    # pair, the small-batch linear (logits to memory) and the row argmax.
+    # The same block of 16 rows through the reference's own pair of calls, the small-batch linear
+    # (logits to memory) and the row argmax.
     rows = 16
     x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
     workspace = tile_ops.small_batch_workspace(rows, MODEL_DIM, device)

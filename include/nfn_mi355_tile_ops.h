@@ -783,8 +783,11 @@ int nfn_mi355_abi_version(void);
 /* lm_head GEMV with the argmax fused in: logits never reach memory.  The
  * reference runs mmvq_linear into an 808 KB logits buffer and then
  * argmax_rows over it (resident_glimmer_cuda.cpp:4087-4151, 2661-2704); this
- * is both in one call.  rows 1..8.  Ties go to the lowest index; NaN never
- * wins.  output_indices: int64[rows]; output_values: float[rows]. */
+ * is both in one call.  rows 1..16 (a verifier block); beyond 8 rows for the
+ * four packed formats at an input_dim of at most 16,384, for which the
+ * workspace query, which does not know input_dim, sizes the fp16 copy of the
+ * rows that the 5..16-row form keeps there.  Ties go to the lowest index; NaN
+ * never wins.  output_indices: int64[rows]; output_values: float[rows]. */
 int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(int64_t rows, int64_t output_dim);
 int nfn_mi355_lm_head_argmax_v1(
     const NfnNativeTilePackedWeightDescriptorV1* descriptor,
@@ -806,7 +809,8 @@ int nfn_mi355_lm_head_argmax_v1(
  * and frees nothing.  A problem whose workspace
  * (nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, output_dim)) exceeds that
  * size is refused with NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED; the full
- * 202,048-row vocabulary at 8 rows needs 808,192 bytes and fits.  Every call
+ * 202,048-row vocabulary at 8 rows needs 808,192 bytes and fits, and so do
+ * its 16 rows (786,688 bytes).  Every call
  * on a GPU uses that GPU's one array: calls that overlap on a device
  * (different streams, concurrently replayed graphs) race on it.  The first
  * call on a device looks the array's address up in the runtime

@@ -638,14 +638,33 @@ int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
     return launch_status();
 }
 
+namespace {
+// Widest input the fp16 form of the lm_head takes: the workspace query does not know the
+// input width and sizes that form's fp16 copy of the rows for this one.
+constexpr std::int64_t kLmHeadHalfWidth = 16384;
+constexpr std::int64_t kLmHeadHalfRows = 5;  // rows from which the fp16 form runs
+constexpr std::int64_t kLmHeadOtherRows = 8;  // rows up to which the other forms run
+
+bool lm_head_half_form(const nfn::Descriptor& weight, std::int64_t rows) {
+    return rows >= kLmHeadHalfRows && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
+        nfn::gemv_f16_supports(weight.encoding, weight.input_dim);
+}
+}  // namespace
+
 std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
                                                          std::int64_t output_dim) {
-    if (rows < 1 || rows > 8 || output_dim <= 0) return 0;
-    // room for either kernel's per-workgroup candidates
-    std::int64_t groups = lm_head_f32_blocks(output_dim);
-    if (lm_head_q6_max_groups(output_dim) > groups) groups = lm_head_q6_max_groups(output_dim);
-    if (lm_head_mfma_tiles(output_dim) > groups) groups = lm_head_mfma_tiles(output_dim);
-    const std::int64_t raw = rows * groups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+    if (rows < 1 || rows > 16 || output_dim <= 0) return 0;
+    std::int64_t raw = 0;
+    if (rows <= kLmHeadOtherRows) {
+        // room for either kernel's per-workgroup candidates
+        std::int64_t groups = lm_head_f32_blocks(output_dim);
+        if (lm_head_q6_max_groups(output_dim) > groups) groups = lm_head_q6_max_groups(output_dim);
+        if (lm_head_mfma_tiles(output_dim) > groups) groups = lm_head_mfma_tiles(output_dim);
+        raw = rows * groups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+    }
+    if (rows >= kLmHeadHalfRows) {
+        raw = std::max(raw, lm_head_f16_workspace_bytes(rows, kLmHeadHalfWidth));
+    }
     return (raw + 255) & ~std::int64_t(255);
 }
 
@@ -662,9 +681,16 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
     const std::int64_t required =
         nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    // Two rows and more: the matrix-core kernel (one pass over the weights for
-    // up to four rows).  One row of Q6_K: the streaming dot kernel.
-    if (rows >= 2 && gemv_mfma_supports(normalized.encoding, normalized.input_dim)) {
+    // Five rows and more: the fp16 matrix-core kernel (one pass over the weights for up to
+    // sixteen rows), the only form beyond eight rows.  Two rows and more: the int8
+    // matrix-core kernel (one pass for up to four rows).  One row of Q6_K: the streaming
+    // dot kernel.
+    if (lm_head_half_form(normalized, rows)) {
+        launch_lm_head_f16(normalized, input, rows, workspace, output_indices, output_values,
+                           as_stream(cuda_stream));
+    } else if (rows > kLmHeadOtherRows) {
+        return kInvalid;
+    } else if (rows >= 2 && gemv_mfma_supports(normalized.encoding, normalized.input_dim)) {
         launch_lm_head_mfma(normalized, input, rows, static_cast<LmHeadCandidate*>(workspace),
                             output_indices, output_values, as_stream(cuda_stream));
     } else if (gemv_q6_supports(normalized.encoding, normalized.input_dim)) {

@@ -33,6 +33,7 @@
 #include "common.hpp"
 #include "f16_decode.hpp"
 #include "gemv_f16.hpp"
+#include "lm_head.hpp"
 #include "wave_rows.hpp"
 
 namespace nfn {
@@ -347,10 +348,17 @@ constexpr int kGroupTiles = 2;  // tiles a workgroup accumulates side by side
 // s, so only packed weights stream, kDepth steps (one tile) ahead.  Rows of up
 // to 8,192 columns are one chunk: the fragments are loaded once per launch.
 // After the last chunk the eight waves' partial sums of the group meet in LDS.
-template <std::uint32_t ENC>
+//
+// ARGMAX (the lm_head, one projection): instead of storing the results, the wave that adds up
+// a tile keeps for each of its (row of the tile, token) pairs the best result over the
+// workgroup's tiles, and at the end writes one (value, row) candidate per token:
+// `candidates` is [tokens][kGroupTiles x workgroups].  Ties keep the lower row and NaN never
+// wins, as in the row argmax (neuralfn/csrc/tile_cuda/kernels.cu:1564-1602).
+template <std::uint32_t ENC, bool ARGMAX>
 __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const std::uint8_t* __restrict__ image, const float* __restrict__ inverse_scale, int tokens,
-    std::uint32_t total_tiles, int input_dim, ProjectionSet set) {
+    std::uint32_t total_tiles, int input_dim, LmHeadCandidate* __restrict__ candidates,
+    ProjectionSet set) {
     using Block = PackedBlock<ENC>;
     __shared__ float partial[2 * kGroupTiles * kWaves * kWave * 4];
 
@@ -439,6 +447,9 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     for (int s = 0; s < kDepth; ++s) fetch(stages[s], s);
     fetch_advance();
 
+    float best_value[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    std::int64_t best_row[4] = {0, 0, 0, 0};
+
     for (int group = 0; group < groups; ++group) {
         f32x4 acc[kGroupTiles];
 #pragma unroll
@@ -496,28 +507,85 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int token = 4 * j + r;
-                if (token < tokens && row < op.output_dim) {
-                    op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
-                        sum[r] * token_scale[r];
+                const float result = sum[r] * token_scale[r];
+                if constexpr (ARGMAX) {
+                    // rows past the end and NaN results stand back
+                    better(row < op.output_dim && result == result ? result : -INFINITY, row,
+                           best_value[r], best_row[r]);
+                } else if (token < tokens && row < op.output_dim) {
+                    op.output[static_cast<std::int64_t>(token) * op.output_dim + row] = result;
+                }
+            }
+        }
+    }
+    if constexpr (ARGMAX) {
+        if (wave < kGroupTiles) {  // the waves that added up tiles
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // over the 16 rows of a tile: the lanes of a quarter
+#pragma unroll
+                for (int offset = 8; offset > 0; offset >>= 1) {
+                    const float other_value = __shfl_xor(best_value[r], offset, 64);
+                    const std::int64_t other_row = __shfl_xor(best_row[r], offset, 64);
+                    better(other_value, other_row, best_value[r], best_row[r]);
+                }
+                const int token = 4 * j + r;
+                if (i == 0 && token < tokens) {
+                    LmHeadCandidate candidate;
+                    candidate.index = best_row[r];
+                    candidate.value = best_value[r];
+                    candidate.pad = 0;
+                    candidates[static_cast<std::int64_t>(token) * (kGroupTiles * gridDim.x) +
+                               kGroupTiles * blockIdx.x + wave] = candidate;
                 }
             }
         }
     }
 }
 
+constexpr std::uint32_t kMaxArgmaxGroups = 512;  // workgroups of an lm_head launch at most
+
+// Workgroups of a launch over `tiles` tiles: one per compute unit (persistent), fewer when
+// there are fewer tiles.
+std::uint32_t grid_of(std::uint32_t tiles, bool argmax) {
+    std::uint32_t slots = static_cast<std::uint32_t>(compute_units());
+    if (argmax && slots > kMaxArgmaxGroups) slots = kMaxArgmaxGroups;
+    return tiles < slots ? tiles : slots;
+}
+
+// `candidates` non-null: the lm_head form (one projection), which returns its workgroup count.
 template <std::uint32_t ENC>
-void launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* inverse_scale,
-                     int tokens, hipStream_t stream) {
+std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* inverse_scale,
+                              int tokens, LmHeadCandidate* candidates, hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
-    // persistent grid: one workgroup per compute unit, fewer when there are fewer tiles
-    const std::uint32_t slots = static_cast<std::uint32_t>(compute_units());
-    const std::uint32_t grid = tiles < slots ? tiles : slots;
-    hipLaunchKernelGGL((gemv_f16_kernel<ENC>), dim3(grid), dim3(kThreads), 0, stream, image,
-                       inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), set);
+    const std::uint32_t grid = grid_of(tiles, candidates != nullptr);
+    if (candidates != nullptr) {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, true>), dim3(grid), dim3(kThreads), 0, stream, image,
+                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
+                           set);
+    } else {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, false>), dim3(grid), dim3(kThreads), 0, stream, image,
+                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
+                           set);
+    }
+    return grid;
+}
+
+std::uint32_t launch_by_encoding(const ProjectionSet& group, std::uint32_t encoding,
+                                 const std::uint8_t* image, const float* inverse_scale, int tokens,
+                                 LmHeadCandidate* candidates, hipStream_t stream) {
+    if (encoding == kEncQ4K) {
+        return launch_encoding<kEncQ4K>(group, image, inverse_scale, tokens, candidates, stream);
+    } else if (encoding == kEncQ5K) {
+        return launch_encoding<kEncQ5K>(group, image, inverse_scale, tokens, candidates, stream);
+    } else if (encoding == kEncQ6K) {
+        return launch_encoding<kEncQ6K>(group, image, inverse_scale, tokens, candidates, stream);
+    }
+    return launch_encoding<kEncQ8_0>(group, image, inverse_scale, tokens, candidates, stream);
 }
 
 }  // namespace
@@ -564,16 +632,44 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
             if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
         }
         if (group.count == 0) continue;
-        if (encoding == kEncQ4K) {
-            launch_encoding<kEncQ4K>(group, image, inverse_scale, tokens, stream);
-        } else if (encoding == kEncQ5K) {
-            launch_encoding<kEncQ5K>(group, image, inverse_scale, tokens, stream);
-        } else if (encoding == kEncQ6K) {
-            launch_encoding<kEncQ6K>(group, image, inverse_scale, tokens, stream);
-        } else {
-            launch_encoding<kEncQ8_0>(group, image, inverse_scale, tokens, stream);
-        }
+        launch_by_encoding(group, encoding, image, inverse_scale, tokens, nullptr, stream);
     }
+}
+
+// Workspace of the lm_head form: the fp16 copy and its row scales, then the candidates.
+namespace {
+std::int64_t lm_head_image_bytes(std::int64_t rows, std::int64_t input_dim) {
+    return (rows * input_dim * 2 + rows * 4 + 255) & ~std::int64_t(255);
+}
+}  // namespace
+
+std::int64_t lm_head_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
+    return lm_head_image_bytes(rows, input_dim) +
+        rows * kGroupTiles * kMaxArgmaxGroups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
+}
+
+void launch_lm_head_f16(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                        void* workspace, std::int64_t* indices, float* maxima, hipStream_t stream) {
+    std::uint8_t* image = static_cast<std::uint8_t*>(workspace);
+    float* inverse_scale = reinterpret_cast<float*>(image + rows * descriptor.input_dim * 2);
+    LmHeadCandidate* candidates =
+        reinterpret_cast<LmHeadCandidate*>(image + lm_head_image_bytes(rows, descriptor.input_dim));
+    const int tokens = static_cast<int>(rows);
+    hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows)),
+                       dim3(kImageThreads), 0, stream, input, nullptr, image, inverse_scale, tokens,
+                       static_cast<int>(descriptor.input_dim));
+    ProjectionSet set{};
+    set.count = 1;
+    set.input_dim = descriptor.input_dim;
+    set.op[0].data = descriptor.data;
+    set.op[0].output = nullptr;
+    set.op[0].output_dim = descriptor.output_dim;
+    set.op[0].row_stride = descriptor.row_stride_bytes;
+    set.op[0].encoding = descriptor.encoding;
+    const std::uint32_t groups =
+        launch_by_encoding(set, descriptor.encoding, image, inverse_scale, tokens, candidates, stream);
+    launch_lm_head_final(candidates, static_cast<std::int64_t>(kGroupTiles) * groups, indices, maxima,
+                         rows, stream);
 }
 
 }  // namespace nfn

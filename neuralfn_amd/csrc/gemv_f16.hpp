@@ -17,4 +17,11 @@ std::int64_t gemv_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim)
 void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* second, int prologue,
                      std::int64_t rows, void* workspace, hipStream_t stream);
 
+// lm_head for 5..16 rows: the same two launches, the multiplying one keeping (value, row)
+// candidates per token instead of the logits, and a third that reduces them
+// (lm_head.hip).  `workspace`: lm_head_f16_workspace_bytes(rows, input_dim) bytes.
+std::int64_t lm_head_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim);
+void launch_lm_head_f16(const Descriptor& descriptor, const float* input, std::int64_t rows,
+                        void* workspace, std::int64_t* indices, float* maxima, hipStream_t stream);
+
 }  // namespace nfn

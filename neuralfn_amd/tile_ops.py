@@ -639,7 +639,7 @@ def lm_head_argmax(weight: PackedWeight, x, workspace=None, indices=None, maxima
     if workspace is None:
         nbytes = load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, weight.output_dim)
         if nbytes <= 0:
-            raise ValueError("lm_head_argmax supports 1..8 rows")
+            raise ValueError("lm_head_argmax supports 1..16 rows")
         workspace = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
     if indices is None:
         indices = torch.empty(rows, dtype=torch.int64, device=x.device)

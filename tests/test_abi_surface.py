@@ -188,7 +188,8 @@ def test_other_entry_points_fail_closed(lib):
     assert multi(ctypes.byref(d), ctypes.byref(d), ctypes.byref(d), None, 0x1, 0x2, 0x3, 0x4,
                  0x5, None, None, 2, None) == tile_ops.INVALID           # unused slot not null
     assert lib.nfn_native_tile_argmax_rows_float32_v1(0x1, 0x2, 0x3, 0, 8, None) == tile_ops.INVALID
-    assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(9, 1000) == 0
+    assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(17, 1000) == 0
+    assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(16, 1000) > 0
     assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(512, 6656, 16384, 7) == 0
     assert lib.nfn_mi355_k_quant_gemm_workspace_bytes_v1(512, 100, 16384, 0) == 0
 

@@ -541,8 +541,8 @@ def test_argmax_rows_random_and_nan(cuda, oracle):
     assert indices[3] == min(7, int(np.argmax(values[3])))
 
 
-@pytest.mark.parametrize("rows", [1, 3, 8])
-@pytest.mark.parametrize("encoding", [kquant.Q6_K, kquant.Q4_K, kquant.Q5_K])
+@pytest.mark.parametrize("rows", [1, 3, 5, 8, 16])
+@pytest.mark.parametrize("encoding", [kquant.Q6_K, kquant.Q4_K, kquant.Q5_K, kquant.Q8_0])
 def test_lm_head_fused_argmax_against_oracle(cuda, oracle, encoding, rows):
     out_dim, in_dim = 4099, 1024
     packed = kquant.quantize(encoding, kquant.synthetic_weights(80 + encoding, out_dim, in_dim))
@@ -560,7 +560,7 @@ def test_lm_head_fused_argmax_against_oracle(cuda, oracle, encoding, rows):
             assert logits[row, indices.cpu()[row].item()] >= ordered[0] - 2 * TOLERANCE * scale
 
 
-@pytest.mark.parametrize("rows", [1, 2, 5])
+@pytest.mark.parametrize("rows", [1, 2, 5, 16])
 def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda, rows):
     # Identical vocabulary rows, two in one 32-row tile and one far away: the
     # lowest index must win for every token (all tokens carry the same input).
@@ -633,7 +633,7 @@ def test_q6_k_long_rows_tensor_two_bytes_off_a_word(cuda, oracle):
     assert_bits_equal(a, b, "aligned and shifted tensor")
 
 
-@pytest.mark.parametrize("rows", [1, 3])
+@pytest.mark.parametrize("rows", [1, 3, 8, 16])
 def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
     out_dim, in_dim = 5003, 6656
     packed = kquant.quantize(kquant.Q6_K, kquant.synthetic_weights(83, out_dim, in_dim))
@@ -649,12 +649,12 @@ def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
             assert indices.cpu()[row].item() == oracle.argmax(logits[row])
     # the fused result equals argmax over the unfused logits of the same kernel
     workspace = tile_ops.small_batch_workspace(rows, in_dim)
-    family = "mmvq" if rows == 1 else "mmq"  # one row: dot kernel; more: matrix cores
+    family = "mmvq" if rows == 1 else "mmq"  # one row: dot kernel; more: matrix cores (int8 to four rows, fp16 beyond)
     unfused = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family=family)[0]
     assert torch_().equal(unfused.max(dim=1).values.cpu(), maxima.cpu())
 
 
-@pytest.mark.parametrize("rows", [1, 4])
+@pytest.mark.parametrize("rows", [1, 4, 16])
 def test_lm_head_full_vocabulary_planted_maxima(cuda, oracle, rows):
     # The benchmark's lm_head (Q6_K, 6656 -> 202048, 1.1 GB) with random bytes
     # and planted rows: every token's winner is known, one of them twice (the
@@ -668,6 +668,8 @@ def test_lm_head_full_vocabulary_planted_maxima(cuda, oracle, rows):
     packed = blocks.reshape(out_dim, -1)
     x = kquant.synthetic_activations(95, rows, in_dim, rms_normalize=True)
     planted = {0: [17, 150000], 1: [202047], 2: [101010], 3: [4096]}
+    planted.update({token: [7919 * token + 13] for token in range(4, 16)})
+    planted[9] = [202032, 31]  # the first row of the last 16-row tile, and an earlier row
     expected_index, expected_value = [], []
     for token in range(rows):
         strong = (np.sign(x[token]) * 8.0).astype(np.float32).reshape(1, in_dim)

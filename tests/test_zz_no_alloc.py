@@ -41,13 +41,16 @@ def _case(cuda, oracle, encoding, rows, out_dim, in_dim, seed):
 def test_two_calls_in_a_row_second_smaller(cuda, oracle, encoding):
     _case(cuda, oracle, encoding, 4, 4160, 1024, 900 + encoding)   # many workgroups, four rows
     _case(cuda, oracle, encoding, 1, 520, 1024, 950 + encoding)    # fewer candidates, one row
-    _case(cuda, oracle, encoding, 8, 96, 512, 970 + encoding)      # eight rows, three tiles
+    _case(cuda, oracle, encoding, 8, 96, 512, 970 + encoding)      # eight rows, a few tiles
+    _case(cuda, oracle, encoding, 16, 4160, 1024, 980 + encoding)  # sixteen rows, a tile per workgroup
+    _case(cuda, oracle, encoding, 5, 40, 256, 990 + encoding)      # five rows, three tiles
 
 
 def test_full_vocabulary_fits_and_larger_is_refused(cuda):
     import torch
     lib = tile_ops.load()
     assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(8, 202048) <= tile_ops.LM_HEAD_NO_ALLOC_SCRATCH_BYTES
+    assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(16, 202048) <= tile_ops.LM_HEAD_NO_ALLOC_SCRATCH_BYTES
     # a vocabulary whose candidates do not fit: refused before anything is launched or read
     out_dim, in_dim = 300_000, 256
     assert lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(8, out_dim) > tile_ops.LM_HEAD_NO_ALLOC_SCRATCH_BYTES
@@ -60,7 +63,7 @@ def test_full_vocabulary_fits_and_larger_is_refused(cuda):
     assert status == tile_ops.STATIC_SCRATCH_EXCEEDED
     assert b"scratch" in lib.nfn_native_tile_ops_error_string(status)
     assert lib.nfn_mi355_lm_head_argmax_no_alloc_v1(
-        ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), 9, None) == 1
+        ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), 17, None) == 1
     assert lib.nfn_mi355_lm_head_argmax_no_alloc_v1(
         None, x.data_ptr(), indices.data_ptr(), maxima.data_ptr(), 1, None) == 1
     torch.cuda.synchronize()
