@@ -646,7 +646,9 @@ constexpr std::int64_t kLmHeadHalfRows = 5;  // rows from which the fp16 form ru
 constexpr std::int64_t kLmHeadOtherRows = 8;  // rows up to which the other forms run
 
 bool lm_head_half_form(const nfn::Descriptor& weight, std::int64_t rows) {
+    // (its kernel keeps row numbers in 32 bits)
     return rows >= kLmHeadHalfRows && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
+        weight.output_dim <= std::numeric_limits<std::int32_t>::max() &&
         nfn::gemv_f16_supports(weight.encoding, weight.input_dim);
 }
 }  // namespace

@@ -41,6 +41,7 @@ namespace nfn {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kTileRows = 16;
 constexpr int kWaves = 8;
@@ -447,8 +448,16 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     for (int s = 0; s < kDepth; ++s) fetch(stages[s], s);
     fetch_advance();
 
-    float best_value[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-    std::int64_t best_row[4] = {0, 0, 0, 0};
+    // ARGMAX: the running best of every (lane, result register) of the waves that add up tiles
+    // lives in LDS between tiles, so that the main loop holds no register for it
+    __shared__ f32x4 best_values[ARGMAX ? kGroupTiles * kWave : 1];
+    __shared__ i32x4 best_rows[ARGMAX ? kGroupTiles * kWave : 1];
+    if constexpr (ARGMAX) {
+        if (wave < kGroupTiles) {
+            best_values[wave * kWave + lane] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            best_rows[wave * kWave + lane] = i32x4{0, 0, 0, 0};
+        }
+    }
 
     for (int group = 0; group < groups; ++group) {
         f32x4 acc[kGroupTiles];
@@ -504,36 +513,52 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
             for (int w = 1; w < kWaves; ++w) {
                 sum += *reinterpret_cast<const f32x4*>(mine + (w * kWave + lane) * 4);
             }
+            if constexpr (ARGMAX) {
+                f32x4 best_value = best_values[wave * kWave + lane];
+                i32x4 best_row = best_rows[wave * kWave + lane];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int token = 4 * j + r;
-                const float result = sum[r] * token_scale[r];
-                if constexpr (ARGMAX) {
-                    // rows past the end and NaN results stand back
-                    better(row < op.output_dim && result == result ? result : -INFINITY, row,
-                           best_value[r], best_row[r]);
-                } else if (token < tokens && row < op.output_dim) {
-                    op.output[static_cast<std::int64_t>(token) * op.output_dim + row] = result;
+                for (int r = 0; r < 4; ++r) {
+                    const float result = sum[r] * token_scale[r];
+                    // rows past the end and NaN results stand back; a later tile's rows are
+                    // higher, so that an equal result does not replace an earlier one
+                    const bool wins = row < op.output_dim && result > best_value[r];
+                    best_value[r] = wins ? result : best_value[r];
+                    best_row[r] = wins ? static_cast<int>(row) : best_row[r];
+                }
+                best_values[wave * kWave + lane] = best_value;
+                best_rows[wave * kWave + lane] = best_row;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int token = 4 * j + r;
+                    if (token < tokens && row < op.output_dim) {
+                        op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
+                            sum[r] * token_scale[r];
+                    }
                 }
             }
         }
     }
     if constexpr (ARGMAX) {
         if (wave < kGroupTiles) {  // the waves that added up tiles
+            const f32x4 mine_value = best_values[wave * kWave + lane];
+            const i32x4 mine_row = best_rows[wave * kWave + lane];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
+                float best_value = mine_value[r];
+                std::int64_t best_row = mine_row[r];
                 // over the 16 rows of a tile: the lanes of a quarter
 #pragma unroll
                 for (int offset = 8; offset > 0; offset >>= 1) {
-                    const float other_value = __shfl_xor(best_value[r], offset, 64);
-                    const std::int64_t other_row = __shfl_xor(best_row[r], offset, 64);
-                    better(other_value, other_row, best_value[r], best_row[r]);
+                    const float other_value = __shfl_xor(best_value, offset, 64);
+                    const std::int64_t other_row = __shfl_xor(best_row, offset, 64);
+                    better(other_value, other_row, best_value, best_row);
                 }
                 const int token = 4 * j + r;
                 if (i == 0 && token < tokens) {
                     LmHeadCandidate candidate;
-                    candidate.index = best_row[r];
-                    candidate.value = best_value[r];
+                    candidate.index = best_row;
+                    candidate.value = best_value;
                     candidate.pad = 0;
                     candidates[static_cast<std::int64_t>(token) * (kGroupTiles * gridDim.x) +
                                kGroupTiles * blockIdx.x + wave] = candidate;
