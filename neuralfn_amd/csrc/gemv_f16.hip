@@ -128,8 +128,20 @@ __device__ __forceinline__ f16x8 as_operand(std::uint32_t a, std::uint32_t b, st
     return __builtin_bit_cast(f16x8, u32x4{a, b, c, d});
 }
 
+// kQuadFetch: the packed bytes are fetched by quads of lanes instead of by the lanes that use
+//   them, and change_lanes() moves them there (see the kernel).
+
 template <std::uint32_t ENC>
 struct PackedBlock;
+
+// The value of the lane whose number times four is `source` (any permutation of the lanes).
+__device__ __forceinline__ std::uint32_t from_lane(int source, std::uint32_t value) {
+    return static_cast<std::uint32_t>(__builtin_amdgcn_ds_bpermute(source, static_cast<int>(value)));
+}
+__device__ __forceinline__ u32x4 from_lane(int source, u32x4 value) {
+    return u32x4{from_lane(source, value[0]), from_lane(source, value[1]), from_lane(source, value[2]),
+                 from_lane(source, value[3])};
+}
 
 // Q4_K: a 16-byte piece c of the 128 code bytes holds values 16*(c%2)..+15 of
 // sub-blocks 2*(c/2) (low nibbles) and 2*(c/2)+1 (high nibbles).  Quarter j
@@ -138,6 +150,8 @@ struct PackedBlock;
 template <>
 struct PackedBlock<kEncQ4K> {
     static constexpr int kBytes = 144;
+    static constexpr bool kQuadFetch = false;
+    __device__ __forceinline__ void change_lanes(int) {}
     u32x4 header, piece[2];
     KBlockScales scales[2];
     __device__ __forceinline__ void load(GlobalBytes block, std::uint32_t row, int j) {
@@ -175,6 +189,8 @@ struct PackedBlock<kEncQ4K> {
 template <>
 struct PackedBlock<kEncQ5K> {
     static constexpr int kBytes = 176;
+    static constexpr bool kQuadFetch = false;
+    __device__ __forceinline__ void change_lanes(int) {}
     u32x4 header, fifth, piece[2];
     KBlockScales scales[2];
     int fifth_shift;  // sub-block of the first piece's low nibbles
@@ -220,6 +236,9 @@ struct PackedBlock<kEncQ5K> {
 template <>
 struct PackedBlock<kEncQ6K> {
     static constexpr int kBytes = 210;
+    // its parts are aligned to two bytes only, and a lane's unaligned 16-byte load is slow on
+    // its own; the four of a quad, side by side in one row, are not
+    static constexpr bool kQuadFetch = true;
     u32x4 low_a, low_b, top;
     std::uint32_t sub_scales[2];  // the eight of this lane's half
     std::uint32_t d_bits;
@@ -243,6 +262,14 @@ struct PackedBlock<kEncQ6K> {
         sub_scales[0] = s[0];
         sub_scales[1] = s[1];
         d_bits = *reinterpret_cast<GlobalHalf>(block + (row + 208));
+    }
+    __device__ __forceinline__ void change_lanes(int source) {
+        low_a = from_lane(source, low_a);
+        low_b = from_lane(source, low_b);
+        top = from_lane(source, top);
+        sub_scales[0] = from_lane(source, sub_scales[0]);
+        sub_scales[1] = from_lane(source, sub_scales[1]);
+        d_bits = from_lane(source, d_bits);
     }
     __device__ __forceinline__ void prepare(int j) {
         const float d = half_bits_to_float(d_bits);
@@ -281,6 +308,8 @@ struct PackedBlock<kEncQ6K> {
 template <>
 struct PackedBlock<kEncQ8_0> {
     static constexpr int kBytes = 272;
+    static constexpr bool kQuadFetch = false;
+    __device__ __forceinline__ void change_lanes(int) {}
     std::uint32_t codes[2][8];
     std::uint32_t d_bits[2];
     f16x2 scale[2];
@@ -411,6 +440,13 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     // unconditional (a step without work reads the first bytes of the first
     // projection, one line for the whole wave), so a step waits for nothing but
     // its own.  The fetch cursor walks the same stream, one tile ahead.
+    // kQuadFetch: lane l asks for quarter l % 4 of row l / 4, so that the four lanes of a quad
+    // read neighbouring bytes of one row; the matrix instruction wants quarter l / 16 of row
+    // l % 16 in lane l, and a step's registers change lanes before use (Q6_K at 16 rows,
+    // 6,656 -> 202,048: 299 -> 234 us; the formats with aligned blocks lose 3-7 % to it).
+    const int load_row = Block::kQuadFetch ? lane >> 2 : i;
+    const int load_quarter = Block::kQuadFetch ? lane & 3 : j;
+    const int taken_from = 4 * (4 * i + j);  // the lane that fetched this lane's row and quarter, x 4
     int fetch_group = 0, fetch_chunk = 0, fetch_slot = 0;
     GlobalBytes fetch_tile = nullptr;  // first row of the tile being fetched (uniform)
     std::uint32_t fetch_row = 0;       // this lane's row of it, in bytes
@@ -423,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
         const int last = static_cast<int>(min(static_cast<std::int64_t>(kTileRows - 1), op.output_dim - 1 - row0));
         fetch_tile = (GlobalBytes)op.data + row0 * op.row_stride;
-        fetch_row = static_cast<std::uint32_t>(min(i, last)) * static_cast<std::uint32_t>(op.row_stride);  // rows past the end repeat the last one
+        fetch_row = static_cast<std::uint32_t>(min(load_row, last)) * static_cast<std::uint32_t>(op.row_stride);  // rows past the end repeat the last one
     };
     auto fetch_advance = [&]() {  // to the next (group, chunk, tile of the group)
         if (++fetch_slot >= min(kGroupTiles, tile_count - fetch_group * kGroupTiles)) {
@@ -441,7 +477,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         const bool work = fetch_live && local < count;
         const GlobalBytes source = work
             ? fetch_tile + static_cast<std::int64_t>(begin + local) * Block::kBytes : (GlobalBytes)set.op[0].data;
-        stage.load(source, work ? fetch_row : 0u, work ? j : 0);
+        stage.load(source, work ? fetch_row : 0u, work ? load_quarter : 0);
     };
     PackedBlock<ENC> stages[kDepth];
 #pragma unroll
@@ -475,6 +511,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                     PackedBlock<ENC>& stage = stages[s];
                     if (s < chunk_count) {
                         const f16x8 (&a)[8] = fragments[s];
+                        if constexpr (Block::kQuadFetch) stage.change_lanes(taken_from);
                         stage.prepare(j);
                         f32x4 sum = acc[t];
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[0], stage.template operand<0>(), sum, 0, 0, 0);
