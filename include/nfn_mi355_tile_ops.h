@@ -242,6 +242,26 @@ int nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1(
     float* output,
     void* cuda_stream);
 
+/* The same pair for a block of 5..16 rows (a verifier block) on the fp16
+ * small-batch kernel: output[row][r] = (up * gate) * sigmoid(gate) of the two
+ * projections' results, rows x output_dim floats, which the plain small-batch
+ * call behind then reads (the bits of the SwiGLU call on the separate results).
+ * No counterpart in the reference (it runs the grouped small-batch call and
+ * nfn_native_tile_k_quant_mmq_multi_linear_swiglu_float32_v1,
+ * tile_ops.h:650-684).  input null: the workspace already holds the rows as
+ * nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1 left them.  gate and up: the
+ * same encoding (Q4_K, Q5_K, Q6_K or Q8_0), shape and row stride; the workspace
+ * as for the small-batch calls. */
+int nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1(
+    const NfnNativeTilePackedWeightDescriptorV1* gate,
+    const NfnNativeTilePackedWeightDescriptorV1* up,
+    const float* input,
+    float* output,
+    int64_t rows,
+    void* workspace,
+    int64_t workspace_nbytes,
+    void* cuda_stream);
+
 /* ---- the normalisation step upstream of the decode projections ----------
  * hidden = residual_input + rms(input, first_weight, first_eps);
  * residual_output = hidden; normalized_output = rms(hidden, second_weight,

@@ -23,6 +23,7 @@ namespace {
 
 constexpr std::int64_t kMaxSmallRows = 16;
 constexpr std::int64_t kMaxOperations = 4;
+constexpr std::int64_t kFirstHalfRows = 5;  // rows from which the fp16 matrix-core kernel takes a batch
 // Private activation records of the small-batch path, 576 bytes per token and
 // 256 values (two int8 planes of a 16-bit fixed-point code, group sums, scale,
 // block maximum): 72 bytes per 32 values, the unit the workspace is sized in.
@@ -80,7 +81,6 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // Encodings and widths without either: the float kernel.
     // (two rows are also faster on the dot kernels: they walk the token planes
     // against the same unpacked weights)
-    constexpr std::int64_t kFirstHalfRows = 5;
     const bool one_row_arithmetic = rows <= 2 || verifier;
     ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, half{}, exact{};
     dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = half.input_dim =
@@ -404,6 +404,31 @@ int nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1(const Descriptor* gate, con
     set.op[1] = make_projection(*up, output);
     if (set.op[0].row_stride != set.op[1].row_stride) return kInvalid;
     launch_gemv_dot_pairs(set, input, as_stream(cuda_stream));
+    return launch_status();
+}
+
+int nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1(const Descriptor* gate, const Descriptor* up,
+                                                    const float* input, float* output,
+                                                    std::int64_t rows, void* workspace,
+                                                    std::int64_t workspace_nbytes,
+                                                    void* cuda_stream) {
+    if (gate == nullptr || up == nullptr || output == nullptr || workspace == nullptr ||
+        rows < kFirstHalfRows || rows > kMaxSmallRows ||
+        !validate_k_descriptor(gate, gate->input_dim, cuda_stream, true) ||
+        !validate_k_descriptor(up, gate->input_dim, cuda_stream, true) ||
+        gate->output_dim != up->output_dim ||
+        gate->row_stride_bytes != up->row_stride_bytes ||
+        !gemv_f16_pairs_supports(gate->encoding, up->encoding, gate->input_dim)) {
+        return kInvalid;
+    }
+    const std::int64_t required = small_batch_workspace_bytes(rows, gate->input_dim);
+    if (required == 0 || workspace_nbytes < required) return kInvalid;
+    ProjectionSet set{};
+    set.count = 2;
+    set.input_dim = gate->input_dim;
+    set.op[0] = make_projection(*gate, output);
+    set.op[1] = make_projection(*up, output);
+    launch_gemv_f16_pairs(set, input, rows, workspace, as_stream(cuda_stream));
     return launch_status();
 }
 

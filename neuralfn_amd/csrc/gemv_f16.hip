@@ -384,12 +384,21 @@ constexpr int kGroupTiles = 2;  // tiles a workgroup accumulates side by side
 // workgroup's tiles, and at the end writes one (value, row) candidate per token:
 // `candidates` is [tokens][kGroupTiles x workgroups].  Ties keep the lower row and NaN never
 // wins, as in the row argmax (neuralfn/csrc/tile_cuda/kernels.cu:1564-1602).
-template <std::uint32_t ENC, bool ARGMAX>
+//
+// kPairs (gate and up of an FFN, two projections of one shape): a group is tile T of the first
+// projection beside tile T of the second, and the wave that adds up the first adds up both and
+// stores swiglu(first, second), the value the SwiGLU prologue of the projection behind would
+// compute from the two outputs: one [rows, output_dim] result instead of two.
+enum Mode : int { kStore = 0, kArgmax = 1, kPairs = 2 };
+
+template <std::uint32_t ENC, int MODE>
 __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const std::uint8_t* __restrict__ image, const float* __restrict__ inverse_scale, int tokens,
     std::uint32_t total_tiles, int input_dim, LmHeadCandidate* __restrict__ candidates,
     ProjectionSet set) {
     using Block = PackedBlock<ENC>;
+    constexpr bool ARGMAX = MODE == kArgmax;
+    constexpr bool PAIRS = MODE == kPairs;
     __shared__ float partial[2 * kGroupTiles * kWaves * kWave * 4];
 
     const int lane = threadIdx.x & 63;
@@ -433,7 +442,8 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     // this workgroup's tiles: blockIdx.x + n * gridDim.x
     const int tile_count =
         static_cast<int>((total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x);
-    const int groups = (tile_count + kGroupTiles - 1) / kGroupTiles;
+    // (kPairs: total_tiles counts the tiles of one projection and a group is one of them twice)
+    const int groups = PAIRS ? tile_count : (tile_count + kGroupTiles - 1) / kGroupTiles;
 
     // Every wave walks the same stream of (group, chunk, tile of the group, step)
     // in uniform control flow (a group's tiles: kGroupTiles, fewer in the last group).  Weight loads run kDepth steps ahead; they are
@@ -452,17 +462,17 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     std::uint32_t fetch_row = 0;       // this lane's row of it, in bytes
     bool fetch_live = true;
     auto fetch_setup = [&]() {
-        const int index = fetch_group * kGroupTiles + fetch_slot;
+        const int index = PAIRS ? fetch_group : fetch_group * kGroupTiles + fetch_slot;
         fetch_live = fetch_group < groups && index < tile_count;
         const std::uint32_t tile = blockIdx.x + static_cast<std::uint32_t>(fetch_live ? index : 0) * gridDim.x;
-        const Projection op = tile_projection(set, tile);
-        const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kTileRows;
+        const Projection op = PAIRS ? pick(set, fetch_slot) : tile_projection(set, tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(tile - (PAIRS ? 0u : op.first_tile)) * kTileRows;
         const int last = static_cast<int>(min(static_cast<std::int64_t>(kTileRows - 1), op.output_dim - 1 - row0));
         fetch_tile = (GlobalBytes)op.data + row0 * op.row_stride;
         fetch_row = static_cast<std::uint32_t>(min(load_row, last)) * static_cast<std::uint32_t>(op.row_stride);  // rows past the end repeat the last one
     };
     auto fetch_advance = [&]() {  // to the next (group, chunk, tile of the group)
-        if (++fetch_slot >= min(kGroupTiles, tile_count - fetch_group * kGroupTiles)) {
+        if (++fetch_slot >= (PAIRS ? kGroupTiles : min(kGroupTiles, tile_count - fetch_group * kGroupTiles))) {
             fetch_slot = 0;
             if (++fetch_chunk == chunks) {
                 fetch_chunk = 0;
@@ -499,7 +509,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         f32x4 acc[kGroupTiles];
 #pragma unroll
         for (int t = 0; t < kGroupTiles; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        const int group_tiles = min(kGroupTiles, tile_count - group * kGroupTiles);
+        const int group_tiles = PAIRS ? kGroupTiles : min(kGroupTiles, tile_count - group * kGroupTiles);
         for (int chunk = 0; chunk < chunks; ++chunk) {
             if (chunks > 1 || group == 0) load_fragments(chunk);
             const int chunk_count = min(kDepth, count - chunk * kDepth);  // this wave's blocks of the chunk
@@ -539,6 +549,28 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
             }
         }
         __syncthreads();
+        if constexpr (PAIRS) {
+            if (wave == 0) {
+                const std::uint32_t tile = blockIdx.x + static_cast<std::uint32_t>(group) * gridDim.x;
+                const std::int64_t row = static_cast<std::int64_t>(tile) * kTileRows + i;
+                f32x4 first = *reinterpret_cast<const f32x4*>(buffer + lane * 4);
+                f32x4 second = *reinterpret_cast<const f32x4*>(buffer + (kWaves * kWave + lane) * 4);
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w) {
+                    first += *reinterpret_cast<const f32x4*>(buffer + (w * kWave + lane) * 4);
+                    second += *reinterpret_cast<const f32x4*>(buffer + ((kWaves + w) * kWave + lane) * 4);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int token = 4 * j + r;
+                    if (token < tokens && row < set.op[0].output_dim) {
+                        set.op[0].output[static_cast<std::int64_t>(token) * set.op[0].output_dim + row] =
+                            apply_prologue<kSwiGlu>(first[r] * token_scale[r], second[r] * token_scale[r]);
+                    }
+                }
+            }
+            continue;
+        }
         if (wave < group_tiles) {
             const float* mine = buffer + wave * kWaves * kWave * 4;
             const std::uint32_t tile =
@@ -626,15 +658,26 @@ std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, cons
     }
     const std::uint32_t grid = grid_of(tiles, candidates != nullptr);
     if (candidates != nullptr) {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, true>), dim3(grid), dim3(kThreads), 0, stream, image,
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax>), dim3(grid), dim3(kThreads), 0, stream, image,
                            inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
                            set);
     } else {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, false>), dim3(grid), dim3(kThreads), 0, stream, image,
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kStore>), dim3(grid), dim3(kThreads), 0, stream, image,
                            inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
                            set);
     }
     return grid;
+}
+
+// The pair form: two projections of one shape and encoding, one result.
+template <std::uint32_t ENC>
+void launch_pair(const ProjectionSet& set, const std::uint8_t* image, const float* inverse_scale,
+                 int tokens, hipStream_t stream) {
+    const std::uint32_t tiles =
+        static_cast<std::uint32_t>((set.op[0].output_dim + kTileRows - 1) / kTileRows);
+    hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs>), dim3(grid_of(tiles, false)), dim3(kThreads), 0,
+                       stream, image, inverse_scale, tokens, tiles, static_cast<int>(set.input_dim),
+                       static_cast<LmHeadCandidate*>(nullptr), set);
 }
 
 std::uint32_t launch_by_encoding(const ProjectionSet& group, std::uint32_t encoding,
@@ -695,6 +738,29 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
         }
         if (group.count == 0) continue;
         launch_by_encoding(group, encoding, image, inverse_scale, tokens, nullptr, stream);
+    }
+}
+
+bool gemv_f16_pairs_supports(std::uint32_t first_encoding, std::uint32_t second_encoding,
+                             std::int64_t input_dim) {
+    return first_encoding == second_encoding && gemv_f16_supports(first_encoding, input_dim);
+}
+
+void launch_gemv_f16_pairs(const ProjectionSet& set, const float* input, std::int64_t rows,
+                           void* workspace, hipStream_t stream) {
+    std::uint8_t* image = static_cast<std::uint8_t*>(workspace);
+    float* inverse_scale = reinterpret_cast<float*>(image + rows * set.input_dim * 2);
+    const int tokens = static_cast<int>(rows);
+    if (input != nullptr) {
+        hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows)),
+                           dim3(kImageThreads), 0, stream, input, nullptr, image, inverse_scale, tokens,
+                           static_cast<int>(set.input_dim));
+    }
+    switch (set.op[0].encoding) {
+        case kEncQ4K: launch_pair<kEncQ4K>(set, image, inverse_scale, tokens, stream); break;
+        case kEncQ5K: launch_pair<kEncQ5K>(set, image, inverse_scale, tokens, stream); break;
+        case kEncQ6K: launch_pair<kEncQ6K>(set, image, inverse_scale, tokens, stream); break;
+        default: launch_pair<kEncQ8_0>(set, image, inverse_scale, tokens, stream); break;
     }
 }
 

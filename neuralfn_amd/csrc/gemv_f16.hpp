@@ -17,6 +17,14 @@ std::int64_t gemv_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim)
 void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* second, int prologue,
                      std::int64_t rows, void* workspace, hipStream_t stream);
 
+// Gate and up of an FFN (set.op[0], set.op[1]: one shape, one encoding) with
+// swiglu(gate, up) stored in set.op[0].output instead of the two results.  `input` null: the
+// workspace already holds the converted rows (as with prologue kHalfImage).
+bool gemv_f16_pairs_supports(std::uint32_t first_encoding, std::uint32_t second_encoding,
+                             std::int64_t input_dim);
+void launch_gemv_f16_pairs(const ProjectionSet& set, const float* input, std::int64_t rows,
+                           void* workspace, hipStream_t stream);
+
 // lm_head for 5..16 rows: the same two launches, the multiplying one keeping (value, row)
 // candidates per token instead of the logits, and a third that reduces them
 // (lm_head.hip).  `workspace`: lm_head_f16_workspace_bytes(rows, input_dim) bytes.

@@ -139,7 +139,7 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
 
 def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
                  pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
-                 attention_workspace=None, handoff: bool = False):
+                 attention_workspace=None, handoff: bool = False, fused_gate_up: bool = False):
     """A block of tokens (rows of `pending`, at positions position, position + 1, ...) through
     one layer the way the verifier runs it (resident_glimmer_cuda.cpp:2913-2960, 3437-3520): the
     same operators in their batch forms, a causal block attention over the cache and the
@@ -151,6 +151,10 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     output in `workspace` in the form the projections would convert it to
     (nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1) and the projections behind them
     multiply from it; the same bits, two launches less.
+
+    fused_gate_up (5..16 rows): gate and up in one call that stores swiglu(gate, up)
+    (nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1) where the pair allows it; the down
+    projection then reads that one block of rows plainly; the same bits.
 
     Returns (down, hidden, key_rows, value_rows).
     """
@@ -182,6 +186,11 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
         g.post_norm_eps, g.norm_eps, handoff_workspace=workspace if handoff else None)
+    if fused_gate_up and tile_ops.gate_up_swiglu_rows_supported(weights.mlp_gate, weights.mlp_up, rows):
+        activated = tile_ops.gate_up_swiglu_rows(weights.mlp_gate, weights.mlp_up,
+                                                 None if handoff else normalized, rows, workspace)
+        (down,) = tile_ops.multi_linear([weights.mlp_down], activated, workspace)
+        return down, hidden, key, value
     if handoff:
         mlp_gate, mlp_up = tile_ops.multi_linear_prequantized(
             [weights.mlp_gate, weights.mlp_up], rows, workspace, family="mmq")

@@ -185,6 +185,8 @@ SIGNATURES = {
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
     "nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1": (ctypes.c_int, [_DESC, _DESC, _P, _P, _P]),
+    "nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1": (
+        ctypes.c_int, [_DESC, _DESC, _P, _P, _I64, _P, _I64, _P]),
     "nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1": (
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _DESC_ARRAY, _PTR_ARRAY, _I64, _P]),
@@ -561,6 +563,30 @@ def gate_up_swiglu_supported(gate: PackedWeight, up: PackedWeight) -> bool:
     return (gate.encoding == up.encoding and gate.encoding in (kquant.Q4_K, kquant.Q5_K) and
             gate.output_dim == up.output_dim and gate.input_dim == up.input_dim and
             gate.input_dim % 256 == 0 and gate.input_dim <= 8192)
+
+
+def gate_up_swiglu_rows(gate: PackedWeight, up: PackedWeight, x, rows: int, workspace, out=None):
+    """nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1: a block of 5..16 rows through the gate and
+    up projections with the SwiGLU activation applied to the pair of results.  x None: the
+    workspace holds the rows as dual_rms_add_capture(handoff_workspace=...) left them."""
+    import torch
+    stream = _stream_handle()
+    if out is None:
+        out = torch.empty((rows, gate.output_dim), dtype=torch.float32, device=workspace.device)
+    gate_descriptor, up_descriptor = gate.descriptor(stream), up.descriptor(stream)
+    check(load().nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1(
+        ctypes.byref(gate_descriptor), ctypes.byref(up_descriptor),
+        None if x is None else x.data_ptr(), out.data_ptr(), rows, workspace.data_ptr(),
+        workspace.numel(), stream), "gate_up_swiglu_rows")
+    return out
+
+
+def gate_up_swiglu_rows_supported(gate: PackedWeight, up: PackedWeight, rows: int) -> bool:
+    """Whether gate_up_swiglu_rows takes this pair and row count."""
+    return (5 <= rows <= 16 and gate.encoding == up.encoding and
+            gate.encoding in (kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0) and
+            gate.output_dim == up.output_dim and gate.input_dim == up.input_dim and
+            gate.input_dim % 256 == 0 and gate.input_dim <= 65536)
 
 
 def quantize_q8_1(x):

@@ -1075,6 +1075,18 @@ def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, o
         assert torch_().equal(handed_keys, key_rows) and torch_().equal(handed_values, value_rows)
     assert torch_().equal(handed_pending, pending) and torch_().equal(handed_residual, residual)
 
+    # ... and with gate and up in the one call that stores swiglu(gate, up), with and without
+    # the handoff: the same bits again
+    for handoff in (False, True):
+        fused_pending = to_device(embeddings, cuda)
+        fused_residual, pending_norm = torch_().zeros_like(fused_pending), None
+        for weights, cache in zip(stack, caches()):
+            fused_pending, fused_residual, _, _ = dl.verify_layer(
+                g, weights, cache, fused_pending, fused_residual, pending_norm, position, workspace,
+                True, attention_workspace, handoff=handoff, fused_gate_up=True)
+            pending_norm = weights.post_feedforward_norm
+        assert torch_().equal(fused_pending, pending) and torch_().equal(fused_residual, residual)
+
     def error(actual, expected):
         return float(np.max(np.abs(actual - expected)) / np.max(np.abs(expected)))
 

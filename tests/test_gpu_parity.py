@@ -352,6 +352,79 @@ def test_gate_up_swiglu_equals_the_two_calls(cuda, oracle, encoding, in_dim, out
     assert normalised_error(fused.cpu().numpy(), exact) <= 2 * TOLERANCE
 
 
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0])
+@pytest.mark.parametrize("rows,in_dim,out_dim", [(5, 256, 1), (16, 2304, 70), (8, 6656, 1037), (16, 6656, 16384),
+                                                 (11, 16384, 513)])
+def test_gate_up_swiglu_rows_equals_the_two_calls(cuda, oracle, encoding, rows, in_dim, out_dim):
+    """nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1 = the grouped small-batch call on [gate, up]
+    followed by the element-wise SwiGLU, bit for bit; a projection fed from its output equals the
+    SwiGLU-prologue call on the two separate results."""
+    gate = tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, out_dim, in_dim, 191), out_dim, in_dim)
+    up = tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, out_dim, in_dim, 192), out_dim, in_dim)
+    x = to_device(kquant.synthetic_activations(193, rows, in_dim), cuda)
+    workspace = tile_ops.small_batch_workspace(rows, max(in_dim, (out_dim + 255) // 256 * 256))
+    separate = tile_ops.multi_linear([gate, up], x, workspace)
+    expected = tile_ops.swiglu(separate[0], separate[1])
+    assert tile_ops.gate_up_swiglu_rows_supported(gate, up, rows)
+    fused = tile_ops.gate_up_swiglu_rows(gate, up, x, rows, workspace)
+    assert_bits_equal(fused, expected, "gate/up with SwiGLU")
+    if out_dim % 256 == 0:
+        down = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, 40, out_dim, 194), 40, out_dim)
+        (by_prologue,) = tile_ops.multi_linear([down], separate[0], workspace, separate[1], "mmq", "swiglu")
+        (plain,) = tile_ops.multi_linear([down], fused, workspace)
+        assert_bits_equal(plain, by_prologue, "the projection behind")
+    if out_dim <= 2048:
+        exact_gate = oracle.linear(encoding, gate.data.cpu().numpy(), out_dim, in_dim, x.cpu().numpy())
+        exact_up = oracle.linear(encoding, up.data.cpu().numpy(), out_dim, in_dim, x.cpu().numpy())
+        exact = oracle.swiglu(exact_gate, exact_up)
+        assert normalised_error(fused.cpu().numpy(), exact) <= 2 * TOLERANCE
+
+
+def test_gate_up_swiglu_rows_from_the_norm_handoff(cuda):
+    """With a null input the call multiplies from the fp16 rows the dual norm left in the workspace:
+    the same bits as the call on the normalized rows."""
+    torch = torch_()
+    rows, width, out_dim = 16, 6656, 640
+    rng = np.random.default_rng(7)
+    pending = to_device(rng.standard_normal((rows, width)).astype(np.float32), cuda)
+    residual = to_device(rng.standard_normal((rows, width)).astype(np.float32), cuda)
+    _, first = norm_weight(1.0 + 0.1 * rng.standard_normal(width), kquant.F32, cuda)
+    _, second = norm_weight(1.0 + 0.1 * rng.standard_normal(width), kquant.BF16, cuda)
+    gate = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, out_dim, width, 195), out_dim, width)
+    up = tile_ops.PackedWeight.from_numpy(kquant.Q4_K, random_packed(kquant.Q4_K, out_dim, width, 196), out_dim, width)
+    workspace = tile_ops.small_batch_workspace(rows, width)
+    _, normalized, _ = tile_ops.dual_rms_add_capture(pending, residual, first, False, second, False, 1e-6, 1e-6,
+                                                      handoff_workspace=workspace)
+    handed = tile_ops.gate_up_swiglu_rows(gate, up, None, rows, workspace)
+    ordinary = tile_ops.gate_up_swiglu_rows(gate, up, normalized, rows, workspace)
+    assert_bits_equal(handed, ordinary, "from the handoff")
+
+
+def test_gate_up_swiglu_rows_fails_closed(cuda):
+    lib = tile_ops.load()
+    in_dim, out_dim, rows = 512, 24, 8
+    make = lambda e, n, k, seed: tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, k, seed), n, k)
+    gate, up = make(kquant.Q4_K, out_dim, in_dim, 1), make(kquant.Q4_K, out_dim, in_dim, 2)
+    x = to_device(kquant.synthetic_activations(3, 16, in_dim), cuda)
+    out = torch_().empty((16, out_dim), dtype=torch_().float32, device=cuda)
+    workspace = tile_ops.small_batch_workspace(16, in_dim)
+    call = lib.nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1
+    ref = lambda w: ctypes.byref(w.descriptor(0))
+    arguments = lambda g, u, r=rows, n=workspace.numel(): (ref(g), ref(u), x.data_ptr(), out.data_ptr(), r,
+                                                           workspace.data_ptr(), n, None)
+    assert call(*arguments(gate, up)) == 0
+    assert call(*arguments(gate, make(kquant.Q5_K, out_dim, in_dim, 4))) == 1
+    assert call(*arguments(gate, make(kquant.Q4_K, out_dim + 1, in_dim, 5))) == 1
+    assert call(*arguments(gate, make(kquant.Q4_K, out_dim, 256, 6))) == 1
+    assert call(*arguments(gate, up, 4)) == 1
+    assert call(*arguments(gate, up, 17)) == 1
+    assert call(*arguments(gate, up, rows, 64)) == 1
+    assert call(None, ref(up), x.data_ptr(), out.data_ptr(), rows, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert call(ref(gate), ref(up), x.data_ptr(), None, rows, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert call(ref(gate), ref(up), x.data_ptr(), out.data_ptr(), rows, None, workspace.numel(), None) == 1
+    torch_().cuda.synchronize()
+
+
 def test_gate_up_swiglu_fails_closed(cuda):
     lib = tile_ops.load()
     in_dim, out_dim = 512, 24
