@@ -650,6 +650,32 @@ def test_lm_head_fused_argmax_tie_goes_to_lowest_index(cuda, rows):
     assert indices.cpu().tolist() == [100] * rows
 
 
+def test_lm_head_fused_argmax_fails_closed(cuda):
+    """Row counts and forms the call does not take, refused before any launch (the weights
+    behind these descriptors do not exist)."""
+    lib = tile_ops.load()
+    torch = torch_()
+    out_dim = 4096
+    x = torch.zeros((16, 32768), dtype=torch.float32, device=cuda)
+    indices = torch.full((16,), -7, dtype=torch.int64, device=cuda)
+    maxima = torch.zeros(16, dtype=torch.float32, device=cuda)
+    nbytes = lib.nfn_mi355_lm_head_argmax_workspace_bytes_v1(16, out_dim)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
+
+    def call(encoding, in_dim, rows, size=nbytes):
+        descriptor = tile_ops.make_descriptor(encoding, 0x1000, out_dim, in_dim)
+        return lib.nfn_mi355_lm_head_argmax_v1(ctypes.byref(descriptor), x.data_ptr(), indices.data_ptr(),
+                                               maxima.data_ptr(), rows, workspace.data_ptr(), size, None)
+
+    assert call(kquant.Q6_K, 1024, 17) == 1           # beyond a block of 16
+    assert call(kquant.Q6_K, 1024, 0) == 1
+    assert call(kquant.F32, 1024, 9) == 1             # 9..16 rows: packed formats only
+    assert call(kquant.Q4_K, 32768, 9) == 1           # ... of at most 16,384 columns
+    assert call(kquant.Q6_K, 1024, 16, 4096) == 1     # workspace too small
+    torch.cuda.synchronize()
+    assert int(indices[0]) == -7
+
+
 @pytest.mark.parametrize("shape", [(130, 256), (515, 6656)])
 def test_q8_0_one_token_and_verifier(cuda, oracle, shape):
     out_dim, in_dim = shape
