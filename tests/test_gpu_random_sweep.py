@@ -259,3 +259,41 @@ def test_matrix_core_attention_random_case(cuda, oracle, seed):
             actual = engine_ops.block_attention(*arguments, workspace=lent).cpu().numpy()
             assert np.abs(actual - expected).max() <= 4e-6, \
                 f"{label}, block {rows}/{block_rows}, causal {causal}, split {lent is not None}"
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_lm_head_block_random_case(cuda, seed):
+    """The fused lm_head argmax at 5..16 rows against the logits of the small-batch call, which runs
+    the same kernel and stores them: the value must be the row's largest logit bit for bit and the
+    index the first column that holds it.  Widths off the 16-row tile, K from one block up, ties
+    planted across tiles and workgroups, a NaN logit, one all-NaN row."""
+    import torch
+    rng = np.random.default_rng(7000 + seed)
+    encoding = int(rng.choice(FORMATS))
+    in_dim = 256 * int(rng.choice([1, 2, 5, 8, 26]))
+    out_dim = int(rng.choice([1, 15, 16, 17, 255, 1000, 4097, 8200, 20011]))
+    rows = int(rng.integers(5, 17))
+    w = (rng.standard_normal((out_dim, in_dim)) * 0.05).astype(np.float32)
+    if out_dim > 40:  # equal rows of weights give equal logits: the first of them must win
+        source = int(rng.integers(0, out_dim))
+        for twin in rng.integers(0, out_dim, size=3):
+            w[int(twin)] = w[source]
+    weight = tile_ops.PackedWeight.from_numpy(encoding, kquant.quantize(encoding, w), out_dim, in_dim)
+    x = rng.standard_normal((rows, in_dim)).astype(np.float32)
+    x[0] *= 1e-4
+    x[rows - 1] *= 3e3
+    if seed % 4 == 0:
+        x[1, 3] = np.nan   # every logit of this row is NaN
+    device_x = to_device(x, cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    (logits,) = tile_ops.multi_linear([weight], device_x, workspace)
+    indices, maxima = tile_ops.lm_head_argmax(weight, device_x)
+    logits = logits.cpu().numpy()
+    for row in range(rows):
+        values = logits[row]
+        if np.all(np.isnan(values)):
+            assert int(indices[row]) == 0 and float(maxima[row]) == -np.inf
+            continue
+        best = np.nanmax(values)
+        assert np.float32(maxima[row].item()).view(np.uint32) == np.float32(best).view(np.uint32), (row, seed)
+        assert int(indices[row]) == int(np.flatnonzero(values == best)[0]), (row, seed)
