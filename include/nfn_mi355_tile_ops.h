@@ -798,6 +798,8 @@ int nfn_native_tile_scale_inplace_float32(
 
 /* ==== additions: no counterpart in the reference ========================= */
 
+/* Version of the additions below, 1: an engine that binds any nfn_mi355_* symbol checks it
+ * the way it checks the reference's four version symbols (resident_glimmer_cuda.cpp:496-501). */
 int nfn_mi355_abi_version(void);
 
 /* lm_head GEMV with the argmax fused in: logits never reach memory.  The
