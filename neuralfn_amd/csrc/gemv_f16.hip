@@ -379,7 +379,7 @@ constexpr int kGroupTiles = 2;  // tiles a workgroup accumulates side by side
 // to 8,192 columns are one chunk: the fragments are loaded once per launch.
 // After the last chunk the eight waves' partial sums of the group meet in LDS.
 //
-// ARGMAX (the lm_head, one projection): instead of storing the results, the wave that adds up
+// kArgmax (the lm_head, one projection): instead of storing the results, the wave that adds up
 // a tile keeps for each of its (row of the tile, token) pairs the best result over the
 // workgroup's tiles, and at the end writes one (value, row) candidate per token:
 // `candidates` is [tokens][kGroupTiles x workgroups].  Ties keep the lower row and NaN never
