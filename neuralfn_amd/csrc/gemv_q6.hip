@@ -733,11 +733,10 @@ constexpr int stream_waves(int tokens_per_pass) {
     return tokens_per_pass <= 2 ? 8 : 16;
 }
 
-template <int T, int P, bool ARGMAX>
+template <int T, int P, bool ARGMAX, int W = stream_waves(T)>
 std::int64_t launch_stream(const ProjectionSet& set, const float* first, const float* second,
                            std::uint8_t* records_out, int tokens, LmHeadCandidate* candidates,
                            hipStream_t stream) {
-    constexpr int W = stream_waves(T);
     const std::size_t lds = static_cast<std::size_t>(T) * token_image_bytes(set.input_dim >> 8) +
         W * kStagingBytes;
     auto kernel = gemv_q6_stream_kernel<T, P, ARGMAX, W>;
@@ -773,6 +772,13 @@ std::int64_t launch_tokens(const ProjectionSet& set, const float* first, const f
     const int per_pass = tokens < capacity ? tokens : capacity;
     if (streams(set.input_dim)) {
         if (per_pass <= 1) {
+            // rows of 48 blocks and more: sixteen waves share a workgroup's quantization of the
+            // activations and stream side by side (19,968 -> 6,656: 29.9 -> 27.3 us, 12,288 ->
+            // 6,656: 18.9 -> 16.6 us; rows of 26 blocks lose 10 % to it)
+            if (set.input_dim >= 48 * 256) {
+                return launch_stream<1, P, ARGMAX, 16>(set, first, second, records_out, tokens, candidates,
+                                                       stream);
+            }
             return launch_stream<1, P, ARGMAX>(set, first, second, records_out, tokens, candidates, stream);
         }
         if (per_pass == 2 || capacity < 4) {
