@@ -100,11 +100,14 @@ def make_layers(layers: int, device):
 class DecodeStep:
     """Pre-built ctypes arguments for the two launches of every layer."""
 
-    def __init__(self, layers, rows: int, device):
+    def __init__(self, layers, rows: int, device, family: str = "mmq"):
         import torch
         from neuralfn_amd import kquant, tile_ops
         self.lib = tile_ops.load()
         self.rows = rows
+        # "mmvq": the verifier family, every row in the one-row arithmetic bit for bit
+        self.function = (self.lib.nfn_native_tile_k_quant_mmq_multi_linear_float32_v1 if family == "mmq"
+                         else self.lib.nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1)
         self.layers = layers
         self.workspace = tile_ops.small_batch_workspace(16, MODEL_DIM, device)
         self.hidden = torch.from_numpy(
@@ -122,7 +125,7 @@ class DecodeStep:
 
     def enqueue(self, stream: int) -> None:
         from neuralfn_amd import tile_ops
-        function = self.lib.nfn_native_tile_k_quant_mmq_multi_linear_float32_v1
+        function = self.function
         rows = self.rows
         for index, layer, outs in self.calls:
             qkv = [layer[n].descriptor(stream) for n in ("q", "k", "v")]
@@ -476,6 +479,18 @@ def decode_batch_extra(layers, device, stream, steps: int, warmup: int, headline
                         stream, steps, warmup)
         traffic = len(layers) * layer_algorithmic_bytes(rows)
         result[f"rows{rows}"] = {
+            "ms_per_step": round(ms, 5), "GB/s": round(traffic / ms / 1e6, 1),
+            "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "us_per_launch": round(ms * 1e3 / step.launches_per_step, 3),
+            "tokens/s": round(rows / ms * 1e3, 1)}
+    # the exact verifier's form of a block: the `mmvq` family, whose rows carry the one-row
+    # arithmetic bit for bit (vector-ALU kernels, four rows a pass over the weights)
+    for rows in (4, 16):
+        step = DecodeStep(layers, rows, device, "mmvq")
+        ms = time_graph(lambda: step.enqueue(int(torch.cuda.current_stream().cuda_stream)),
+                        stream, max(5, steps // 2), max(2, warmup // 2))
+        traffic = len(layers) * layer_algorithmic_bytes(rows)
+        result[f"rows{rows}_exact_verifier_family"] = {
             "ms_per_step": round(ms, 5), "GB/s": round(traffic / ms / 1e6, 1),
             "frac_hbm": round(traffic / ms / 1e6 / HBM_PEAK_GBS, 4),
             "us_per_launch": round(ms * 1e3 / step.launches_per_step, 3),
