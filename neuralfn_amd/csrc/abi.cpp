@@ -10,6 +10,7 @@
 #include "gemv_mfma.hpp"
 #include "gemv_q6.hpp"
 #include "gemv_q8.hpp"
+#include "gemv_rows.hpp"
 #include "kernels.hpp"
 #include "lm_head.hpp"
 #include "rms_device.hpp"
@@ -24,6 +25,9 @@ namespace {
 constexpr std::int64_t kMaxSmallRows = 16;
 constexpr std::int64_t kMaxOperations = 4;
 constexpr std::int64_t kFirstHalfRows = 5;  // rows from which the fp16 matrix-core kernel takes a batch
+// rows from which the verifier family's Q4_K / Q5_K projections run on the int8 matrix cores
+// (one pass over the weights behind a quantizer launch; below: the dot kernel's token passes)
+constexpr std::int64_t kFirstVerifierMatrixRows = 5;
 // Private activation records of the small-batch path, 576 bytes per token and
 // 256 values (two int8 planes of a 16-bit fixed-point code, group sums, scale,
 // block maximum): 72 bytes per 32 values, the unit the workspace is sized in.
@@ -82,13 +86,16 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // (two rows are also faster on the dot kernels: they walk the token planes
     // against the same unpacked weights)
     const bool one_row_arithmetic = rows <= 2 || verifier;
-    ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, half{}, exact{};
+    const bool verifier_matrix = verifier && rows >= kFirstVerifierMatrixRows;
+    ProjectionSet dot{}, dot6{}, dot8{}, matrix{}, half{}, exact{}, verifier_rows{};
     dot.input_dim = dot6.input_dim = dot8.input_dim = matrix.input_dim = half.input_dim =
-        exact.input_dim = input_dim;
+        exact.input_dim = verifier_rows.input_dim = input_dim;
     for (int index = 0; index < set.count; ++index) {
         const std::uint32_t encoding = set.op[index].encoding;
         ProjectionSet* target = &exact;
-        if (one_row_arithmetic && gemv_dot_supports(encoding, input_dim)) {
+        if (verifier_matrix && gemv_rows_supports(encoding, input_dim)) {
+            target = &verifier_rows;
+        } else if (one_row_arithmetic && gemv_dot_supports(encoding, input_dim)) {
             target = &dot;
         } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
             target = &dot6;
@@ -110,6 +117,22 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // finds them (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:3649-3666).
     std::uint8_t* records =
         verifier && prologue != kRecords ? static_cast<std::uint8_t*>(workspace) : nullptr;
+    if (verifier_rows.count > 0) {
+        // The matrix-core kernel reads records: a quantizer launch writes them first, and the
+        // dot kernels of the other encodings in this call then read them too.
+        if (prologue != kRecords) {
+            launch_quantize_records(first, second, prologue, rows, input_dim,
+                                    static_cast<std::uint8_t*>(workspace), as_stream(stream));
+        }
+        launch_gemv_rows(verifier_rows, static_cast<const std::uint8_t*>(workspace), rows,
+                         as_stream(stream));
+        if (exact.count == 0) {
+            first = static_cast<const float*>(workspace);
+            second = nullptr;
+            prologue = kRecords;
+            records = nullptr;
+        }
+    }
     if (dot.count > 0) {
         launch_gemv_dot(dot, first, second, records, prologue, rows, as_stream(stream));
     }

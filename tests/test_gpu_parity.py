@@ -585,6 +585,51 @@ def test_decode_dot_kernel_row_lengths(cuda, oracle, encoding, in_dim):
                 assert_bits_equal(whole[row:row + 1].contiguous(), part, f"verifier row {row} of {rows}")
 
 
+@pytest.mark.parametrize("in_dim", [256, 2304, 4096, 6656, 8448, 16384])
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
+def test_verifier_matrix_core_rows_equal_the_one_row_kernel(cuda, oracle, encoding, in_dim):
+    """From five rows on the verifier family's Q4_K / Q5_K projections run on the int8 matrix
+    cores, one pass over the weights: every row must still carry the one-row kernel's bits.
+    Row lengths: one block (15 empty classes), 9 blocks, exactly one 16-block slice, 26 blocks
+    (classes of one and two blocks), 33 and 64 blocks; output widths off the 32-row tile."""
+    out_dims = (40, 8, 70)
+    packed = [random_packed(encoding, n, in_dim, 90 + i) for i, n in enumerate(out_dims)]
+    weights = [tile_ops.PackedWeight.from_numpy(encoding, p, n, in_dim) for p, n in zip(packed, out_dims)]
+    x = kquant.synthetic_activations(91, 16, in_dim)
+    x *= (10.0 ** np.arange(-3, 5).repeat(2))[:, None].astype(np.float32)  # rows of very different size
+    one = tile_ops.small_batch_workspace(1, in_dim)
+    alone = [tile_ops.multi_linear(weights, to_device(x[row:row + 1], cuda), one) for row in range(16)]
+    for y, p, n in zip(alone[3], packed, out_dims):
+        assert normalised_error(y.cpu().numpy(), oracle.linear(encoding, p, n, in_dim, x[3:4])) <= TOLERANCE
+    for rows in (5, 8, 9, 13, 16):
+        workspace = tile_ops.small_batch_workspace(rows, in_dim)
+        batch = tile_ops.multi_linear(weights, to_device(x[:rows], cuda), workspace, family="mmvq")
+        for row in range(rows):
+            for whole, part in zip(batch, alone[row]):
+                assert_bits_equal(whole[row:row + 1].contiguous(), part, f"row {row} of {rows}")
+
+
+@pytest.mark.parametrize("prologue", ["gated", "swiglu"])
+def test_verifier_matrix_core_rows_with_prologues_and_mixed_formats(cuda, prologue):
+    """Fused prologues go through the quantizer launch; the Q6_K and Q8_0 projections of the same
+    call read the records it wrote."""
+    in_dim, rows = 1280, 11
+    specs = [(kquant.Q4_K, 33), (kquant.Q6_K, 40), (kquant.Q5_K, 64), (kquant.Q8_0, 24)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, in_dim, 95 + i), n, in_dim)
+               for i, (e, n) in enumerate(specs)]
+    x = to_device(kquant.synthetic_activations(96, rows, in_dim), cuda)
+    g = to_device(kquant.synthetic_activations(97, rows, in_dim), cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    one = tile_ops.small_batch_workspace(1, in_dim)
+    batch = tile_ops.multi_linear(weights, x, workspace, g, "mmvq", prologue)
+    again = tile_ops.multi_linear_prequantized(weights, rows, workspace)
+    for row in range(rows):
+        alone = tile_ops.multi_linear(weights, x[row:row + 1], one, g[row:row + 1], "mmvq", prologue)
+        for whole, reused, part, (encoding, _) in zip(batch, again, alone, specs):
+            assert_bits_equal(whole[row:row + 1].contiguous(), part, f"{kquant.NAMES[encoding]} row {row}")
+            assert_bits_equal(reused[row:row + 1].contiguous(), part, f"prequantized {kquant.NAMES[encoding]} row {row}")
+
+
 # ------------------------------------------------------------------- argmax
 
 def test_argmax_rows_tie_rule_at_vocabulary_width(cuda):
