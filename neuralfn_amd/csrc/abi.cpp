@@ -33,13 +33,24 @@ constexpr std::int64_t kFirstVerifierMatrixRows = 5;
 // block maximum): 72 bytes per 32 values, the unit the workspace is sized in.
 constexpr std::int64_t kActivationGroupBytes = kActivationRecordBytes / 8;
 
+// Bytes of the activation records of `rows` rows, rounded up to 256.
+std::int64_t record_bytes(std::int64_t rows, std::int64_t input_dim) {
+    const std::int64_t groups = (input_dim + 31) / 32;
+    return (rows * groups * kActivationGroupBytes + 255) & ~std::int64_t(255);
+}
+
+// Records, and behind them, from the row count on at which the verifier family runs on the
+// matrix cores, the same codes in matrix-operand order (gemv_rows.hpp).
 std::int64_t small_batch_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
     if (rows < 1 || rows > kMaxSmallRows || input_dim <= 0 || input_dim % 128 != 0) return 0;
     const std::int64_t groups = (input_dim + 31) / 32;
-    if (groups > std::numeric_limits<std::int64_t>::max() / (kActivationGroupBytes * rows)) {
+    if (groups > std::numeric_limits<std::int64_t>::max() / (2 * kActivationGroupBytes * kMaxSmallRows)) {
         return 0;
     }
-    const std::int64_t raw = rows * groups * kActivationGroupBytes;
+    std::int64_t raw = record_bytes(rows, input_dim);
+    if (rows >= kFirstVerifierMatrixRows && input_dim % 256 == 0) {
+        raw += gemv_rows_image_bytes(input_dim);
+    }
     return (raw + 255) & ~std::int64_t(255);
 }
 
@@ -117,30 +128,33 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     // finds them (neuralfn/csrc/native_gpt2/resident_glimmer_cuda.cpp:3649-3666).
     std::uint8_t* records =
         verifier && prologue != kRecords ? static_cast<std::uint8_t*>(workspace) : nullptr;
-    if (verifier_rows.count > 0) {
-        // The matrix-core kernel reads records: a quantizer launch writes them first, and the
-        // dot kernels of the other encodings in this call then read them too.
+    const float* dot_first = first;
+    const float* dot_second = second;
+    int dot_prologue = prologue;
+    if (verifier_matrix && input_dim % 256 == 0) {
+        // The matrix-core kernel reads the activations in operand order: a quantizer launch
+        // writes that image behind the records (whatever the encodings of this call, so that a
+        // prequantized call behind it finds both), and the dot kernels of the other encodings
+        // read the records instead of quantizing again.
+        std::uint8_t* image = static_cast<std::uint8_t*>(workspace) + record_bytes(rows, input_dim);
         if (prologue != kRecords) {
             launch_quantize_records(first, second, prologue, rows, input_dim,
-                                    static_cast<std::uint8_t*>(workspace), as_stream(stream));
+                                    static_cast<std::uint8_t*>(workspace), image, as_stream(stream));
         }
-        launch_gemv_rows(verifier_rows, static_cast<const std::uint8_t*>(workspace), rows,
-                         as_stream(stream));
-        if (exact.count == 0) {
-            first = static_cast<const float*>(workspace);
-            second = nullptr;
-            prologue = kRecords;
-            records = nullptr;
-        }
+        if (verifier_rows.count > 0) launch_gemv_rows(verifier_rows, image, rows, as_stream(stream));
+        dot_first = static_cast<const float*>(workspace);
+        dot_second = nullptr;
+        dot_prologue = kRecords;
+        records = nullptr;
     }
     if (dot.count > 0) {
-        launch_gemv_dot(dot, first, second, records, prologue, rows, as_stream(stream));
+        launch_gemv_dot(dot, dot_first, dot_second, records, dot_prologue, rows, as_stream(stream));
     }
     if (dot6.count > 0) {
-        launch_gemv_q6(dot6, first, second, records, prologue, rows, as_stream(stream));
+        launch_gemv_q6(dot6, dot_first, dot_second, records, dot_prologue, rows, as_stream(stream));
     }
     if (dot8.count > 0) {
-        launch_gemv_q8(dot8, first, second, records, prologue, rows, as_stream(stream));
+        launch_gemv_q8(dot8, dot_first, dot_second, records, dot_prologue, rows, as_stream(stream));
     }
     if (matrix.count > 0) {
         launch_gemv_mfma(matrix, first, second, prologue, rows, workspace, as_stream(stream));

@@ -13,15 +13,17 @@
 //   * the balanced binary tree over the 64 chains in the order (c, p).
 // Here a workgroup of 8 waves owns 32 consecutive weight rows.  v_mfma_i32_32x32x32_i8 takes
 // the 32 values of a sub-block (K), 32 weight rows (operand B, lane l: row l % 32, values
-// 16 (l / 32)..+15, unpacked from the 16 bytes of codes the lane loaded itself) and the two
-// int8 planes of up to 16 tokens (operand A, read from the activation records a quantizer
-// launch left in the workspace); a second product against the sub-block minimums, spread over
+// 16 (l / 32)..+15; the packed bytes are loaded coalesced and change lanes through a private
+// LDS tile per wave) and the two int8 planes of up to 16 tokens (operand A, fetched in
+// operand order from the image a quantizer launch left in the workspace beside the activation
+// records: lanes that each pick their own 16 bytes out of sixteen records cost the memory
+// pipeline four times the instructions' coalesced rate); a second product against the sub-block minimums, spread over
 // K, gives the sums the minimums multiply.  A lane then holds, for its weight row and up to 8
 // tokens, the integers of a unit, and replays the float tail above.  Wave w takes the classes
 // w and 15 - w (an even share of any row length), keeps the four chains of a class per token
 // in registers, and leaves (c0 + c1) + (c2 + c3) per class, token and row in LDS; after one
 // barrier a thread per (token, row) adds the 16 classes in the tree's order.
-// One pass over the weights for up to 16 tokens, no weight byte through LDS.
+// One pass over the weights for up to 16 tokens.
 #include "common.hpp"
 #include "gemv_rows.hpp"
 #include "wave_rows.hpp"
@@ -32,50 +34,93 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kRowsTile = 32;
 constexpr int kRowsWaves = 8;
 constexpr int kRowsThreads = kRowsWaves * kWave;
 constexpr int kClasses = 16;
 
-// One wave per activation record: the (token, block) records of wave_rows.hpp.
+// Operand image of the activations, written next to the records by the quantizer launch: per
+// block 8 KB of operand-A fragments, [sub-block][lane 0..63][16 bytes] (lane l: matrix row
+// l % 32, values 16 (l / 32)..+15 of the sub-block), so that a wave fetches a fragment with one
+// coalesced load, then the block's 16 token scales.  Matrix row i = 8 a + 4 half + 2 c + plane
+// holds token S * half + 2 a + c, which puts token S * (lane / 32) + slot into output registers
+// 2 * slot (high plane) and 2 * slot + 1 (low plane); S = token slots per lane.
+constexpr int kImageFragments = 8 * 1024;
+constexpr int kImageBlock = kImageFragments + 16 * 4;
+
+__host__ __device__ constexpr int token_slots(int tokens) { return tokens <= 4 ? 2 : tokens <= 8 ? 4 : 8; }
+
+// One wave per activation record: writes the (token, block) record of wave_rows.hpp and the
+// token's share of the block's operand image.
 template <int P>
 __global__ __launch_bounds__(256) void quantize_records_kernel(
     const float* __restrict__ first, const float* __restrict__ second,
-    std::uint8_t* __restrict__ records, int total_records) {
+    std::uint8_t* __restrict__ records, std::uint8_t* __restrict__ image, int blocks, int tokens) {
     const int lane = threadIdx.x & 63;
     const int record = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
-    if (record >= total_records) return;
+    if (record >= blocks * tokens) return;
     const float4 x = load_activations<P>(first, second,
                                          static_cast<std::int64_t>(record) * 256 + lane * 4);
-    store_record(records + static_cast<std::int64_t>(record) * kActRecord, lane,
-                 activation_codes<P>(x));
+    const ActivationCodes codes = activation_codes<P>(x);
+    store_record(records + static_cast<std::int64_t>(record) * kActRecord, lane, codes);
+    const int token = record / blocks;
+    const int block = record - token * blocks;
+    const int slots = token_slots(tokens);
+    const int half = token / slots;
+    const int slot = token - half * slots;
+    const int row = 8 * (slot >> 1) + 4 * half + 2 * (slot & 1);
+    // this lane's values 4 lane..+3: sub-block lane / 8, values 4 (lane % 8)..+3 of it
+    std::uint8_t* block_image = image + static_cast<std::int64_t>(block) * kImageBlock;
+    std::uint8_t* piece = block_image +
+        (((lane >> 3) * 64 + ((lane >> 2) & 1) * 32 + row) * 16) + (lane & 3) * 4;
+    *reinterpret_cast<std::uint32_t*>(piece) = codes.hi;
+    *reinterpret_cast<std::uint32_t*>(piece + 16) = codes.lo;
+    if (lane == 0) {
+        reinterpret_cast<float*>(block_image + kImageFragments)[token] =
+            codes.maximum * (1.0f / kCodeRange);
+    }
 }
+
+template <bool Q5>
+struct RowsFormat {
+    static constexpr int kBlockBytes = Q5 ? 176 : 144;
+    static constexpr int kChunks = kBlockBytes / 16;          // 16-byte chunks of a block
+    static constexpr int kTileChunks = kRowsTile * kChunks;   // of a block of 32 rows
+    static constexpr int kLoads = (kTileChunks + kWave - 1) / kWave;
+    static constexpr int kTileBytes = kRowsTile * kBlockBytes;
+};
 
 template <bool Q5, int S>
 struct RowsStage {
-    uint4 header;   // d, dmin, 12 bytes of scales and minimums
-    uint4 q[4];     // this lane's half of the four 32-byte code groups
-    uint4 high;     // Q5_K: this lane's half of the high-bit bytes
-    v4i a[8];       // operand A of the eight sub-blocks
-    float scale[S]; // the block's activation scale of this lane's tokens
+    v4u chunk[RowsFormat<Q5>::kLoads];     // packed bytes of 32 rows x one block, coalesced
+    v4i a[8];                             // operand A of the eight sub-blocks
+    float scale[S];                       // the block's activation scale of this lane's tokens
 };
 
 __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
 }
 
-// S: token slots per lane.  Token S * (lane / 32) + slot sits in output registers 2 * slot
-// (high plane) and 2 * slot + 1 (low plane) of the lane; tokens = up to 2 * S.
+__device__ __forceinline__ void rows_lds_fence() {
+    // LDS traffic of one wave is in order; this only pins the compiler.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <std::uint32_t ENC, int S>
 __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
-    const std::uint8_t* __restrict__ records, int tokens, int input_dim, std::uint32_t total_tiles,
+    const std::uint8_t* __restrict__ image, int tokens, int input_dim, std::uint32_t total_tiles,
     ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
-    constexpr int kBlockBytes = kQ5 ? 176 : 144;
+    using F = RowsFormat<kQ5>;
+    constexpr int kBlockBytes = F::kBlockBytes;
     constexpr int kQuants = kQ5 ? 48 : 16;
     constexpr int kTokens = 2 * S;
     __shared__ float class_sums[kClasses][kTokens][kRowsTile];
+    __shared__ __attribute__((aligned(16))) std::uint8_t packed_tiles[kRowsWaves][F::kTileBytes];
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -94,23 +139,22 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kRowsTile;
     const int valid_rows =
         static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
-    const std::uint8_t* weight_row =
-        op.data + (row0 + min(j, valid_rows - 1)) * op.row_stride + h * 16;
+    const std::uint8_t* tile_rows = op.data + row0 * op.row_stride;
 
-    // operand A: row i = lane % 32 of the matrix instruction is (token, plane):
-    // i = 8 a + 4 half + 2 c + plane  <->  output register 4 a + 2 c + plane of lane half `half`
-    const int a_plane = j & 1;
-    const int a_slot = 2 * (j >> 3) + ((j >> 1) & 1);
-    const int a_token = min(a_slot < S ? S * ((j >> 2) & 1) + a_slot : 0, tokens - 1);
-    const std::uint8_t* a_row = records +
-        static_cast<std::int64_t>(a_token) * blocks * kActRecord + a_plane * 256 + h * 16;
-    // the scales of this lane's tokens
-    const std::uint8_t* scale_row[S];
+    // the chunks this lane copies per block: chunk n of the 32 x kChunks, 9 (11) to a row
+    std::uint32_t chunk_offset[F::kLoads];
+    int chunk_slot[F::kLoads];
 #pragma unroll
-    for (int slot = 0; slot < S; ++slot) {
-        scale_row[slot] = records +
-            static_cast<std::int64_t>(min(S * h + slot, tokens - 1)) * blocks * kActRecord + kRecordScale;
+    for (int i = 0; i < F::kLoads; ++i) {
+        const int chunk = min(i * kWave + lane, F::kTileChunks - 1);
+        const int row = chunk / F::kChunks;
+        const int col = chunk - row * F::kChunks;
+        chunk_offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
+                static_cast<std::uint32_t>(op.row_stride) + col * 16;
+        chunk_slot[i] = row * kBlockBytes + col * 16;
     }
+    std::uint8_t* const my_tile = packed_tiles[wave];
+    const std::uint8_t* const my_row = my_tile + j * kBlockBytes;
 
     // this wave's steps: the blocks of class `wave`, then those of class 15 - wave
     const int class0 = wave;
@@ -125,22 +169,30 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     auto fetch = [&](RowsStage<kQ5, S>& stage, int step) {
         // (a step past the wave's last repeats it; a wave with no block at all reads the row's last)
         const int block = min(block_of(min(step, max(total - 1, 0))), blocks - 1);
-        const std::uint8_t* weights = weight_row + static_cast<std::int64_t>(block) * kBlockBytes;
-        stage.header = *reinterpret_cast<const uint4*>(weights - h * 16);
+        const std::uint8_t* weights = tile_rows + static_cast<std::int64_t>(block) * kBlockBytes;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            stage.q[p] = *reinterpret_cast<const uint4*>(weights + kQuants + p * 32);
+        for (int i = 0; i < F::kLoads; ++i) {
+            stage.chunk[i] = *reinterpret_cast<const v4u*>(weights + chunk_offset[i]);
         }
-        if constexpr (kQ5) stage.high = *reinterpret_cast<const uint4*>(weights + 16);
-        const std::uint8_t* planes = a_row + static_cast<std::int64_t>(block) * kActRecord;
+        const std::uint8_t* fragments = image + static_cast<std::int64_t>(block) * kImageBlock;
 #pragma unroll
         for (int sub = 0; sub < 8; ++sub) {
-            stage.a[sub] = *reinterpret_cast<const v4i*>(planes + sub * 32);
+            stage.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
         }
+        const float* scales = reinterpret_cast<const float*>(fragments + kImageFragments) + S * h;
+        if constexpr (S >= 4) {
 #pragma unroll
-        for (int slot = 0; slot < S; ++slot) {
-            stage.scale[slot] = *reinterpret_cast<const float*>(
-                scale_row[slot] + static_cast<std::int64_t>(block) * kActRecord);
+            for (int quad = 0; quad < S / 4; ++quad) {
+                const float4 four = *reinterpret_cast<const float4*>(scales + 4 * quad);
+                stage.scale[4 * quad] = four.x;
+                stage.scale[4 * quad + 1] = four.y;
+                stage.scale[4 * quad + 2] = four.z;
+                stage.scale[4 * quad + 3] = four.w;
+            }
+        } else {
+            const float2 two = *reinterpret_cast<const float2*>(scales);
+            stage.scale[0] = two.x;
+            stage.scale[1] = two.y;
         }
     };
 
@@ -152,7 +204,22 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     }
 
     auto compute = [&](const RowsStage<kQ5, S>& stage) {
-        const uint4 head = stage.header;
+        // the packed bytes change lanes through the wave's LDS tile: a lane needs the header
+        // of row j and its half of the row's codes
+#pragma unroll
+        for (int i = 0; i < F::kLoads; ++i) {
+            *reinterpret_cast<v4u*>(my_tile + chunk_slot[i]) = stage.chunk[i];
+        }
+        rows_lds_fence();
+        const uint4 head = *reinterpret_cast<const uint4*>(my_row);
+        uint4 high = make_uint4(0, 0, 0, 0);
+        if constexpr (kQ5) high = *reinterpret_cast<const uint4*>(my_row + 16 + h * 16);
+        uint4 quants[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            quants[p] = *reinterpret_cast<const uint4*>(my_row + kQuants + p * 32 + h * 16);
+        }
+        rows_lds_fence();  // the next block's stores stay behind these reads
         // 6-bit scales and minimums of the eight sub-blocks, four per word
         const std::uint32_t sc_lo = head.y & 0x3f3f3f3fu;
         const std::uint32_t mn_lo = head.z & 0x3f3f3f3fu;
@@ -163,14 +230,14 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const std::uint32_t packed[4] = {stage.q[p].x, stage.q[p].y, stage.q[p].z, stage.q[p].w};
+            const std::uint32_t packed[4] = {quants[p].x, quants[p].y, quants[p].z, quants[p].w};
             v4i low, upper;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 std::uint32_t lo = packed[w] & 0x0f0f0f0fu;
                 std::uint32_t up = (packed[w] >> 4) & 0x0f0f0f0fu;
                 if constexpr (kQ5) {
-                    const std::uint32_t bits[4] = {stage.high.x, stage.high.y, stage.high.z, stage.high.w};
+                    const std::uint32_t bits[4] = {high.x, high.y, high.z, high.w};
                     const std::uint32_t shifted = bits[w] >> (2 * p);
                     lo |= (shifted & 0x01010101u) << 4;
                     up |= (shifted & 0x02020202u) << 3;
@@ -216,19 +283,23 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         }
     };
 
-    RowsStage<kQ5, S> stages[2];
-    fetch(stages[0], 0);
+    // Two named register stages (an array of them indexed in the loop ends up in scratch memory).
+    RowsStage<kQ5, S> even, odd;
+    fetch(even, 0);
     if (count0 == 0) finish_class(class0);
     if (count1 == 0) finish_class(class1);
+    auto finish_step = [&](int step) {
+        if (step == count0 - 1) finish_class(class0);
+        if (step == total - 1 && count1 > 0) finish_class(class1);
+    };
     for (int step = 0; step < total; step += 2) {
-#pragma unroll
-        for (int k = 0; k < 2; ++k) {
-            if (step + k < total) {
-                fetch(stages[1 - k], step + k + 1);
-                compute(stages[k]);
-                if (step + k == count0 - 1) finish_class(class0);
-                if (step + k == total - 1 && count1 > 0) finish_class(class1);
-            }
+        fetch(odd, step + 1);
+        compute(even);
+        finish_step(step);
+        if (step + 1 < total) {
+            fetch(even, step + 2);
+            compute(odd);
+            finish_step(step + 1);
         }
     }
     __syncthreads();
@@ -250,7 +321,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
 }
 
 template <std::uint32_t ENC>
-void launch_encoding(ProjectionSet set, const std::uint8_t* records, int tokens, hipStream_t stream) {
+void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
@@ -259,13 +330,13 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* records, int tokens,
     const dim3 grid(tiles), block(kRowsThreads);
     const int input_dim = static_cast<int>(set.input_dim);
     if (tokens <= 4) {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 2>), grid, block, 0, stream, records, tokens,
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 2>), grid, block, 0, stream, image, tokens,
                            input_dim, tiles, set);
     } else if (tokens <= 8) {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 4>), grid, block, 0, stream, records, tokens,
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 4>), grid, block, 0, stream, image, tokens,
                            input_dim, tiles, set);
     } else {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 8>), grid, block, 0, stream, records, tokens,
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 8>), grid, block, 0, stream, image, tokens,
                            input_dim, tiles, set);
     }
 }
@@ -277,28 +348,33 @@ bool gemv_rows_supports(std::uint32_t encoding, std::int64_t input_dim) {
         input_dim <= (std::int64_t(1) << 20);
 }
 
+std::int64_t gemv_rows_image_bytes(std::int64_t input_dim) {
+    return (input_dim >> 8) * kImageBlock;
+}
+
 void launch_quantize_records(const float* first, const float* second, int prologue,
                              std::int64_t rows, std::int64_t input_dim, std::uint8_t* records,
-                             hipStream_t stream) {
-    const int total = static_cast<int>(rows * (input_dim >> 8));
-    const dim3 grid(static_cast<unsigned>((total + 3) / 4)), block(256);
+                             std::uint8_t* image, hipStream_t stream) {
+    const int blocks = static_cast<int>(input_dim >> 8);
+    const int tokens = static_cast<int>(rows);
+    const dim3 grid(static_cast<unsigned>((blocks * tokens + 3) / 4)), block(256);
     switch (prologue) {
         case kGated:
             hipLaunchKernelGGL((quantize_records_kernel<kGated>), grid, block, 0, stream, first,
-                               second, records, total);
+                               second, records, image, blocks, tokens);
             break;
         case kSwiGlu:
             hipLaunchKernelGGL((quantize_records_kernel<kSwiGlu>), grid, block, 0, stream, first,
-                               second, records, total);
+                               second, records, image, blocks, tokens);
             break;
         default:
             hipLaunchKernelGGL((quantize_records_kernel<kPlain>), grid, block, 0, stream, first,
-                               second, records, total);
+                               second, records, image, blocks, tokens);
             break;
     }
 }
 
-void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* records, std::int64_t rows,
+void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
                       hipStream_t stream) {
     const std::uint32_t encodings[2] = {kEncQ4K, kEncQ5K};
     for (const std::uint32_t encoding : encodings) {
@@ -309,9 +385,9 @@ void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* records, std
         }
         if (group.count == 0) continue;
         if (encoding == kEncQ4K) {
-            launch_encoding<kEncQ4K>(group, records, static_cast<int>(rows), stream);
+            launch_encoding<kEncQ4K>(group, image, static_cast<int>(rows), stream);
         } else {
-            launch_encoding<kEncQ5K>(group, records, static_cast<int>(rows), stream);
+            launch_encoding<kEncQ5K>(group, image, static_cast<int>(rows), stream);
         }
     }
 }
