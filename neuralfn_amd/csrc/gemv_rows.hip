@@ -40,6 +40,7 @@ constexpr int kRowsTile = 32;
 constexpr int kRowsWaves = 8;
 constexpr int kRowsThreads = kRowsWaves * kWave;
 constexpr int kClasses = 16;
+constexpr int kMaxRowsBlocks = 256;  // input_dim up to 65,536: the blocks whose scales a workgroup keeps
 
 // Operand image of the activations, written next to the records by the quantizer launch: per
 // block 8 KB of operand-A fragments, [sub-block][lane 0..63][16 bytes] (lane l: matrix row
@@ -96,7 +97,6 @@ template <bool Q5, int S>
 struct RowsStage {
     v4u chunk[RowsFormat<Q5>::kLoads];     // packed bytes of 32 rows x one block, coalesced
     v4i a[8];                             // operand A of the eight sub-blocks
-    float scale[S];                       // the block's activation scale of this lane's tokens
 };
 
 __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c) {
@@ -141,9 +141,10 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
     const std::uint8_t* tile_rows = op.data + row0 * op.row_stride;
 
-    // the chunks this lane copies per block: chunk n of the 32 x kChunks, 9 (11) to a row
+    // the chunks this lane copies per block: chunk n = 64 i + lane of the 32 x kChunks, 9 (11)
+    // to a row; the LDS tile is the same bytes row after row, so chunk n goes to byte 16 n
+    // (the lanes past the last chunk repeat it)
     std::uint32_t chunk_offset[F::kLoads];
-    int chunk_slot[F::kLoads];
 #pragma unroll
     for (int i = 0; i < F::kLoads; ++i) {
         const int chunk = min(i * kWave + lane, F::kTileChunks - 1);
@@ -151,8 +152,8 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         const int col = chunk - row * F::kChunks;
         chunk_offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
                 static_cast<std::uint32_t>(op.row_stride) + col * 16;
-        chunk_slot[i] = row * kBlockBytes + col * 16;
     }
+    const int last_slot = min((F::kLoads - 1) * kWave + lane, F::kTileChunks - 1) * 16;
     std::uint8_t* const my_tile = packed_tiles[wave];
     const std::uint8_t* const my_row = my_tile + j * kBlockBytes;
 
@@ -179,22 +180,16 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         for (int sub = 0; sub < 8; ++sub) {
             stage.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
         }
-        const float* scales = reinterpret_cast<const float*>(fragments + kImageFragments) + S * h;
-        if constexpr (S >= 4) {
-#pragma unroll
-            for (int quad = 0; quad < S / 4; ++quad) {
-                const float4 four = *reinterpret_cast<const float4*>(scales + 4 * quad);
-                stage.scale[4 * quad] = four.x;
-                stage.scale[4 * quad + 1] = four.y;
-                stage.scale[4 * quad + 2] = four.z;
-                stage.scale[4 * quad + 3] = four.w;
-            }
-        } else {
-            const float2 two = *reinterpret_cast<const float2*>(scales);
-            stage.scale[0] = two.x;
-            stage.scale[1] = two.y;
-        }
     };
+
+    // the activation scales of this wave's blocks, 16 tokens each: once into LDS
+    constexpr int kMaxSteps = kMaxRowsBlocks / kRowsWaves;
+    __shared__ __attribute__((aligned(16))) float step_scales[kRowsWaves][kMaxSteps][16];
+    for (int index = lane; index < total * 16; index += kWave) {
+        const int block = block_of(index >> 4);
+        step_scales[wave][index >> 4][index & 15] = reinterpret_cast<const float*>(
+            image + static_cast<std::int64_t>(block) * kImageBlock + kImageFragments)[index & 15];
+    }
 
     float acc[4][S];
 #pragma unroll
@@ -203,13 +198,14 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         for (int slot = 0; slot < S; ++slot) acc[p][slot] = 0.0f;
     }
 
-    auto compute = [&](const RowsStage<kQ5, S>& stage) {
+    auto compute = [&](const RowsStage<kQ5, S>& stage, int step) {
         // the packed bytes change lanes through the wave's LDS tile: a lane needs the header
         // of row j and its half of the row's codes
 #pragma unroll
-        for (int i = 0; i < F::kLoads; ++i) {
-            *reinterpret_cast<v4u*>(my_tile + chunk_slot[i]) = stage.chunk[i];
+        for (int i = 0; i + 1 < F::kLoads; ++i) {
+            *reinterpret_cast<v4u*>(my_tile + lane * 16 + i * (kWave * 16)) = stage.chunk[i];
         }
+        *reinterpret_cast<v4u*>(my_tile + last_slot) = stage.chunk[F::kLoads - 1];
         rows_lds_fence();
         const uint4 head = *reinterpret_cast<const uint4*>(my_row);
         uint4 high = make_uint4(0, 0, 0, 0);
@@ -219,6 +215,9 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         for (int p = 0; p < 4; ++p) {
             quants[p] = *reinterpret_cast<const uint4*>(my_row + kQuants + p * 32 + h * 16);
         }
+        float scale[S];
+#pragma unroll
+        for (int slot = 0; slot < S; ++slot) scale[slot] = step_scales[wave][step][S * h + slot];
         rows_lds_fence();  // the next block's stores stay behind these reads
         // 6-bit scales and minimums of the eight sub-blocks, four per word
         const std::uint32_t sc_lo = head.y & 0x3f3f3f3fu;
@@ -251,24 +250,46 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
             const int scale_b = static_cast<int>((sc_word >> (16 * (p & 1) + 8)) & 0xffu);
             const int min_a = static_cast<int>((mn_word >> (16 * (p & 1))) & 0xffu);
             const int min_b = static_cast<int>((mn_word >> (16 * (p & 1) + 8)) & 0xffu);
-            const int spread_a = min_a * 0x01010101;
-            const int spread_b = min_b * 0x01010101;
+            const int spread_a = static_cast<int>(__umul24(min_a, 0x010101u)) | (min_a << 24);
+            const int spread_b = static_cast<int>(__umul24(min_b, 0x010101u)) | (min_b << 24);
             const v4i mins_a = {spread_a, spread_a, spread_a, spread_a};
             const v4i mins_b = {spread_b, spread_b, spread_b, spread_b};
+            // the sub-block scales times 256, opaque to the optimizer: it would otherwise factor
+            // scale * (256 * hi + lo) out and pay a full 32-bit multiplication for it
+            int scale_a256, scale_b256;
+            asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_a256) : "v"(scale_a));
+            asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_b256) : "v"(scale_b));
             const v16i dots_a = mfma_i8(stage.a[2 * p], low, zero);
             const v16i dots_b = mfma_i8(stage.a[2 * p + 1], upper, zero);
             // min_a * sum(codes of a) + min_b * sum(codes of b), per plane
             const v16i sums = mfma_i8(stage.a[2 * p + 1], mins_b, mfma_i8(stage.a[2 * p], mins_a, zero));
 #pragma unroll
             for (int slot = 0; slot < S; ++slot) {
-                const int weighted_hi = __mul24(scale_a, dots_a[2 * slot]) + __mul24(scale_b, dots_b[2 * slot]);
-                const int weighted_lo =
-                    __mul24(scale_a, dots_a[2 * slot + 1]) + __mul24(scale_b, dots_b[2 * slot + 1]);
+                float codes;
+                if constexpr (kQ5) {
+                    const int weighted_hi =
+                        __mul24(scale_a, dots_a[2 * slot]) + __mul24(scale_b, dots_b[2 * slot]);
+                    const int weighted_lo =
+                        __mul24(scale_a, dots_a[2 * slot + 1]) + __mul24(scale_b, dots_b[2 * slot + 1]);
+                    codes = fmaf(static_cast<float>(weighted_hi), 256.0f, static_cast<float>(weighted_lo));
+                } else {
+                    // 4-bit codes: 256 * weighted_hi + weighted_lo stays below 2^31
+                    // (2 * 63 * 32 * 15 * (127 * 256 + 128)), and one conversion rounds the
+                    // exact integer as the fused multiply-add of the two exact floats does
+                    // (a chain of multiply-adds: the empty statements keep the optimizer from
+                    // turning it into a tree with one more instruction)
+                    int weighted = __mul24(scale_a256, dots_a[2 * slot]);
+                    asm("" : "+v"(weighted));
+                    weighted += __mul24(scale_b256, dots_b[2 * slot]);
+                    asm("" : "+v"(weighted));
+                    weighted += __mul24(scale_a, dots_a[2 * slot + 1]);
+                    asm("" : "+v"(weighted));
+                    weighted += __mul24(scale_b, dots_b[2 * slot + 1]);
+                    codes = static_cast<float>(weighted);
+                }
                 const int weighted_min = sums[2 * slot] * 256 + sums[2 * slot + 1];
-                const float codes =
-                    fmaf(static_cast<float>(weighted_hi), 256.0f, static_cast<float>(weighted_lo));
                 const float value = fmaf(-dmin, static_cast<float>(weighted_min), d * codes);
-                acc[p][slot] = fmaf(stage.scale[slot], value, acc[p][slot]);
+                acc[p][slot] = fmaf(scale[slot], value, acc[p][slot]);
             }
         }
     };
@@ -294,11 +315,11 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     };
     for (int step = 0; step < total; step += 2) {
         fetch(odd, step + 1);
-        compute(even);
+        compute(even, step);
         finish_step(step);
         if (step + 1 < total) {
             fetch(even, step + 2);
-            compute(odd);
+            compute(odd, step + 1);
             finish_step(step + 1);
         }
     }
@@ -345,7 +366,7 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, h
 
 bool gemv_rows_supports(std::uint32_t encoding, std::int64_t input_dim) {
     return (encoding == kEncQ4K || encoding == kEncQ5K) && input_dim % 256 == 0 &&
-        input_dim <= (std::int64_t(1) << 20);
+        input_dim <= kMaxRowsBlocks * 256;
 }
 
 std::int64_t gemv_rows_image_bytes(std::int64_t input_dim) {
