@@ -409,7 +409,13 @@ int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
  * the norm kernel's launch in front of a launch of one workgroup per compute
  * unit.  The same bits as the two calls.  The arguments up to second_centered
  * are those of the dual RMS call for one row; width a multiple of 256 up to
- * 8192; 1..4 projections of one encoding (Q4_K or Q5_K) and input_dim = width. */
+ * 8192; 1..4 projections of one encoding (Q4_K or Q5_K) and input_dim = width.
+ * No aliasing: every workgroup reads `input` and `residual_input` while the
+ * first one stores the three result rows, so hidden_output, normalized_output,
+ * residual_output and the projection outputs must not overlap either input row
+ * (status 1 otherwise).  A caller that normalises in place, as the engine does
+ * with residual_output == residual_input, keeps its two calls or alternates
+ * between two residual buffers. */
 int nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1(
     const float* input,
     const NfnNativeTilePackedWeightDescriptorV1* first_weight,

@@ -660,6 +660,35 @@ int nfn_mi355_dual_rms_mmvq_multi_linear_float32_v1(
         set.op[index] = make_projection(*descriptors[index], outputs[index]);
     }
     if (!gemv_dot_normed_supports(set)) return kInvalid;
+    // Every workgroup of the launch reads `input` and `residual_input` in its prologue and the
+    // first one stores the three rows: a row stored over one that is still being read would
+    // change what later workgroups normalise.  In-place calls (the engine's residual_output ==
+    // residual_input) therefore keep to the two-call form.
+    const auto overlaps = [width](const float* read, const float* written) {
+        const auto a = reinterpret_cast<std::uintptr_t>(read);
+        const auto b = reinterpret_cast<std::uintptr_t>(written);
+        const std::uintptr_t bytes = static_cast<std::uintptr_t>(width) * sizeof(float);
+        return a < b + bytes && b < a + bytes;
+    };
+    const float* const read_rows[2] = {input, residual_input};
+    const float* const written_rows[3] = {hidden_output, residual_output, normalized_output};
+    for (const float* read : read_rows) {
+        for (const float* written : written_rows) {
+            if (overlaps(read, written)) return kInvalid;
+        }
+    }
+    for (std::int64_t index = 0; index < operation_count; ++index) {
+        // (the projections' outputs are written while other workgroups may still read the rows)
+        const auto out = reinterpret_cast<std::uintptr_t>(outputs[index]);
+        const std::uintptr_t out_bytes =
+            static_cast<std::uintptr_t>(set.op[index].output_dim) * sizeof(float);
+        for (const float* read : read_rows) {
+            const auto a = reinterpret_cast<std::uintptr_t>(read);
+            if (a < out + out_bytes && out < a + static_cast<std::uintptr_t>(width) * sizeof(float)) {
+                return kInvalid;
+            }
+        }
+    }
     DualNormArguments norm{};
     norm.residual = residual_input;
     norm.first_weight = norm_weight(first_weight != nullptr ? &first : nullptr, first_centered);

@@ -139,7 +139,8 @@ def decode_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
 
 def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCache, pending, residual,
                  pending_norm: Optional[PackedWeight], position: int, workspace, local: bool = True,
-                 attention_workspace=None, handoff: bool = False, fused_gate_up: bool = False):
+                 attention_workspace=None, handoff: bool = False, fused_gate_up: bool = False,
+                 family: str = "mmq"):
     """A block of tokens (rows of `pending`, at positions position, position + 1, ...) through
     one layer the way the verifier runs it (resident_glimmer_cuda.cpp:2913-2960, 3437-3520): the
     same operators in their batch forms, a causal block attention over the cache and the
@@ -156,10 +157,18 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     (nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1) where the pair allows it; the down
     projection then reads that one block of rows plainly; the same bits.
 
+    family "mmvq": every projection through the exact verifier's entry points
+    (nfn_native_tile_k_quant_mmvq_multi_linear*_float32_v1), as the engine's speculative decode
+    calls them with exact_verifier_rows (resident_glimmer.cpp:2662-2666,
+    resident_glimmer_cuda.cpp:3526-3532): row r then equals decode_layer's projections bit for
+    bit.  The two additions above belong to the other family and are not combined with it.
+
     Returns (down, hidden, key_rows, value_rows).
     """
     g = geometry
     rows = pending.shape[0]
+    if family == "mmvq" and (handoff or fused_gate_up):
+        raise ValueError("the handoff and the gate/up pair call are forms of the mmq family")
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         pending, residual, pending_norm, False, weights.input_norm, False,
         g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps,
@@ -169,7 +178,8 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
         query, key, value, gate = tile_ops.multi_linear_prequantized(
             attention_inputs, rows, workspace, family="mmq")
     else:
-        query, key, value, gate = tile_ops.multi_linear(attention_inputs, normalized, workspace)
+        query, key, value, gate = tile_ops.multi_linear(attention_inputs, normalized, workspace,
+                                                        family=family)
     query = query.view(rows, g.query_heads, g.head_dim)
     key = key.view(rows, g.kv_heads, g.head_dim)
     value = value.view(rows, g.kv_heads, g.head_dim)
@@ -182,7 +192,7 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
                                            window, g.head_dim ** -0.5, True,
                                            workspace=attention_workspace)
     (projected,) = tile_ops.multi_linear([weights.output], attention.view(rows, g.attention_dim),
-                                         workspace, second=gate, prologue="gated")
+                                         workspace, second=gate, family=family, prologue="gated")
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
         g.post_norm_eps, g.norm_eps, handoff_workspace=workspace if handoff else None)
@@ -196,9 +206,9 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
             [weights.mlp_gate, weights.mlp_up], rows, workspace, family="mmq")
     else:
         mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
-                                                 workspace)
+                                                 workspace, family=family)
     (down,) = tile_ops.multi_linear([weights.mlp_down], mlp_gate, workspace, second=mlp_up,
-                                    prologue="swiglu")
+                                    family=family, prologue="swiglu")
     return down, hidden, key, value
 
 

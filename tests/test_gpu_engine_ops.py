@@ -1090,6 +1090,19 @@ def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, o
     def error(actual, expected):
         return float(np.max(np.abs(actual - expected)) / np.max(np.abs(expected)))
 
+    # the exact verifier's family: every projection of the block carries the one-row kernel's
+    # bits, so what is left between the block and the serial chain is the summation order of
+    # the attention kernels (none while both run on the vector kernel)
+    exact_pending = to_device(embeddings, cuda)
+    exact_residual, pending_norm = torch_().zeros_like(exact_pending), None
+    for weights, cache in zip(stack, caches()):
+        exact_pending, exact_residual, _, _ = dl.verify_layer(
+            g, weights, cache, exact_pending, exact_residual, pending_norm, position, workspace,
+            True, attention_workspace, family="mmvq")
+        pending_norm = weights.post_feedforward_norm
+    assert error(exact_residual.cpu().numpy(), np.stack(serial_hidden)) <= 2e-5
+    assert error(exact_pending.cpu().numpy(), np.stack(serial_down)) <= 2e-5
+
     # the projections of a block (fp16 weights and activations on the matrix cores, 11
     # significant bits each) and of one token (integer codes against 16-bit activation codes)
     # run in different kernels: each within 2e-3 of the float formula, and after two layers

@@ -1094,6 +1094,24 @@ def test_dual_rms_inside_the_projection_launch_fails_closed(cuda):
     assert run([good], width_argument=256) == 1   # the projections' input width differs
     assert run([good], tail_arguments=[0.0, False, 1e-5, False]) == 1
     assert run([good], head_arguments=[None] + head[1:]) == 1
+    # Every workgroup reads the two input rows while the first one stores the three result
+    # rows: in-place calls (the engine's residual_output == residual_input) are refused, as are
+    # results or projection outputs laid over a row that is read.
+    residual_in = to_device(probe_rms_input(1, width), cuda)
+    in_place = [x.data_ptr(), None, residual_in.data_ptr(), rows[0].data_ptr(), None,
+                rows[1].data_ptr(), residual_in.data_ptr()]
+    assert run([good], head_arguments=in_place) == 1
+    over_input = [x.data_ptr(), None, residual_in.data_ptr(), x.data_ptr(), None,
+                  rows[1].data_ptr(), rows[2].data_ptr()]
+    assert run([good], head_arguments=over_input) == 1
+    partly = [x.data_ptr(), None, residual_in.data_ptr(), rows[0].data_ptr(), None,
+              x.data_ptr() + 4 * (width - 1), rows[2].data_ptr()]
+    assert run([good], head_arguments=partly) == 1
+    kept = out[0]
+    out[0] = residual_in[:, :24]  # a projection's output over the residual row
+    assert run([good]) == 0  # (x is both inputs here: not touched)
+    assert run([good], head_arguments=[x.data_ptr(), None, residual_in.data_ptr()] + head[3:]) == 1
+    out[0] = kept
     wide = make(kquant.Q4_K, 8, 8448, 4)
     wide_x = to_device(probe_rms_input(1, 8448), cuda)
     wide_rows = [torch_().empty_like(wide_x) for _ in range(3)]
