@@ -278,8 +278,8 @@ def launch_floor_extra(layers, device, stream, steps: int, warmup: int) -> dict:
     kernel.  The ceiling these two put over the headline is a property of 16 MB launches on
     this chip, not of the kernels."""
     import torch
-    from neuralfn_amd import kquant, tile_ops
-    lib = tile_ops.load()
+    from neuralfn_amd import kquant, probes, tile_ops
+    lib = probes.load()
     qkv = (kquant.packed_nbytes(kquant.Q4_K, ATTN_DIM, MODEL_DIM)
            + 2 * kquant.packed_nbytes(kquant.Q4_K, KV_DIM, MODEL_DIM))
     out = kquant.packed_nbytes(kquant.Q4_K, MODEL_DIM, ATTN_DIM)
@@ -299,7 +299,24 @@ def launch_floor_extra(layers, device, stream, steps: int, warmup: int) -> dict:
     read_ms = time_graph(lambda: enqueue(True), stream, steps, warmup)
     empty_ms = time_graph(lambda: enqueue(False), stream, steps, warmup)
     bytes_per_launch = per_layer / 2
+
+    # Would a launch gain by pulling the next launch's first bytes into its XCD's L2 while it
+    # streams its own (weights are static, so a decode loop could hand the next descriptor set
+    # down as a hint)?  The same chain of launches over equal regions, each also requesting
+    # `rounds` x 512 16-byte pieces per workgroup of the following region (8 rounds = all of it).
+    region = (per_layer // 2) // (16 * CU_COUNT) * (16 * CU_COUNT)
+    def enqueue_chained(rounds: int):
+        handle = int(torch.cuda.current_stream().cuda_stream)
+        for index in range(launches):
+            base = pool.data_ptr() + index * region
+            following = pool.data_ptr() + ((index + 1) % launches) * region
+            tile_ops.check(lib.nfn_mi355_read_probe_chained_v1(
+                base, region, following, rounds, sink.data_ptr(), handle), "chained read probe")
+    chained = {f"prefetch_{rounds}_of_8_rounds": round(
+        time_graph(lambda: enqueue_chained(rounds), stream, steps, warmup) * 1e3 / launches, 3)
+        for rounds in (0, 1, 2, 4, 8)}
     return {
+        "chained_read_only_us_per_launch": chained,
         "workload": f"{launches} launches a HIP-graph replay, one workgroup of 512 per compute unit: "
                     "read only the packed bytes of a decode launch / an empty kernel",
         "read_only_us_per_launch": round(read_ms * 1e3 / launches, 3),
@@ -559,23 +576,31 @@ def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
 
 def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     import torch
-    from neuralfn_amd import kquant, tile_ops
+    from neuralfn_amd import kquant, probes, tile_ops
     gate = random_packed_on_device(kquant.Q4_K, FFN_DIM, MODEL_DIM, device, 8)
+    up = random_packed_on_device(kquant.Q4_K, FFN_DIM, MODEL_DIM, device, 10)
     down = random_packed_on_device(kquant.Q4_K, MODEL_DIM, FFN_DIM, device, 9)
     result = {}
     for mode, name in ((tile_ops.GEMM_F16, "f16"),):
         for rows in (512, 2048):
             x = torch.from_numpy(kquant.synthetic_activations(31, rows, MODEL_DIM)).to(device)
             h = torch.from_numpy(kquant.synthetic_activations(32, rows, FFN_DIM)).to(device)
-            for label, weight, source in (("gate_up", gate, x), ("down", down, h)):
-                out = torch.empty((rows, weight.output_dim), dtype=torch.float32, device=device)
-                nbytes = tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
-                    rows, weight.input_dim, weight.output_dim, mode)
+            # gate_up: both projections of the block's input through the call that converts
+            # the activations once (nfn_mi355_k_quant_gemm_multi_float32_v1), as a SwiGLU
+            # feed-forward block runs them; gate_alone: one of them through the single call
+            for label, weights, source in (("gate_up", [gate, up], x), ("gate_alone", [gate], x),
+                                           ("down", [down], h)):
+                outs = [torch.empty((rows, w.output_dim), dtype=torch.float32, device=device)
+                        for w in weights]
+                nbytes = max(tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
+                    rows, w.input_dim, w.output_dim, mode) for w in weights)
                 workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-                ms = time_graph(
-                    lambda: tile_ops.gemm(weight, source, mode, workspace, out), stream,
-                    max(5, steps // 2), max(2, warmup // 2))
-                flops = 2.0 * rows * weight.input_dim * weight.output_dim
+                if len(weights) == 1:
+                    call = lambda: tile_ops.gemm(weights[0], source, mode, workspace, outs[0])
+                else:
+                    call = lambda: tile_ops.gemm_multi(weights, source, mode, workspace, outs)
+                ms = time_graph(call, stream, max(5, steps // 2), max(2, warmup // 2))
+                flops = sum(2.0 * rows * w.input_dim * w.output_dim for w in weights)
                 tflops = flops / ms / 1e9
                 result[f"{name}_{label}_M{rows}"] = {
                     "ms": round(ms, 4), "TFLOP/s": round(tflops, 1),
@@ -592,7 +617,7 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     result["generic_v1_linear_f32_matrix_cores_gate_M512"] = {
         "ms": round(ms, 4), "TFLOP/s": round(tflops, 2),
         "frac_mfma_f32": round(tflops / MFMA_PEAK_TFLOPS["f32"], 4),
-        "x_workspace_gemm": round(ms / result["f16_gate_up_M512"]["ms"], 1)}
+        "x_workspace_gemm": round(ms / result["f16_gate_alone_M512"]["ms"], 1)}
     # The shader clock while the largest shape runs, and the matrix-core peak at
     # that clock: 256 CUs x 4096 fp16 flop per cycle per CU.
     rows = 2048
@@ -601,7 +626,7 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     nbytes = tile_ops.load().nfn_mi355_k_quant_gemm_workspace_bytes_v1(
         rows, MODEL_DIM, FFN_DIM, tile_ops.GEMM_F16)
     workspace = torch.empty(nbytes, dtype=torch.uint8, device=device)
-    probe = tile_ops.ShaderClockProbe(device)
+    probe = probes.ShaderClockProbe(device)
     for _ in range(10):  # the clock settles under load before the probe's window
         tile_ops.gemm(gate, x, tile_ops.GEMM_F16, workspace, out)
     probe.start(5000)
@@ -626,11 +651,12 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
     # Config 3's int8 leg: what the int8 matrix cores would have to run, from registers
     # (nfn_mi355_mfma_rate_probe_v1), beside the fp16 instruction the GEMM uses.  One step =
     # one 32 x 32 x 32 product per wave = 65,536 flop.
-    lib = tile_ops.load()
+    lib = probes.load()
     sink = torch.zeros(4096, dtype=torch.float32, device=device)
     probe_steps, groups = 20000, 2 * CU_COUNT
     legs = {}
     for mode, label in ((0, "f16_mfma"), (1, "int8_mfma_one_plane_no_rescale"),
+                        (3, "int8_mfma_one_plane_rescaled_per_32"),
                         (2, "int8_mfma_two_planes_rescaled_per_32")):
         def run():
             tile_ops.check(lib.nfn_mi355_mfma_rate_probe_v1(
@@ -640,9 +666,11 @@ def prefill_extra(device, stream, steps: int, warmup: int) -> dict:
         legs[label] = round(65536.0 * probe_steps * groups * 4 / ms / 1e9, 1)
     result["matrix_core_probe_TFLOP/s_equivalent"] = {
         **legs,
-        "note": "useful 32x32x32 products per second x 65,536; the last row is the only int8 form "
-                "whose results can meet the 2e-3 bound (16-bit activation codes), and the reason "
-                "NFN_MI355_GEMM_INT8 stays reserved when it is below the fp16 row"}
+        "note": "useful 32x32x32 products per second x 65,536; one plane rescaled per 32 values is "
+                "config 3's int8 leg as written (8-bit activations per 32-value group, judged "
+                "against the Q8_1 oracle); the last row is the only int8 form whose results can "
+                "meet the 2e-3 bound against the float oracle (16-bit activation codes); "
+                "NFN_MI355_GEMM_INT8 stays reserved while both are below the fp16 row"}
     return {"workload": f"Q4_K SwiGLU FFN projections {MODEL_DIM}<->{FFN_DIM}, dequant-GEMM "
                         "incl. activation conversion", **result}
 
@@ -770,7 +798,7 @@ def memory_rate_extra(device, stream, steps: int, warmup: int) -> dict:
     cache holds, and this library's read-only probe kernel over the same buffers.  The
     comparators for every HBM-bound figure here, next to the published 8 TB/s."""
     import torch
-    from neuralfn_amd import tile_ops
+    from neuralfn_amd import probes, tile_ops
     result = {"workload": "torch.sum / Tensor.copy_ / this library's read-only probe kernel over a "
                           "float32 buffer, TB/s of bytes moved"}
     steps, warmup = max(5, steps // 2), max(2, warmup // 2)
@@ -785,7 +813,7 @@ def memory_rate_extra(device, stream, steps: int, warmup: int) -> dict:
         # of the decode kernels' shape can read at best
         sink = torch.zeros(1024, dtype=torch.int32, device=device)
         handle = int(torch.cuda.current_stream().cuda_stream)
-        probe_ms = time_replays(lambda: tile_ops.check(tile_ops.load().nfn_mi355_read_probe_v1(
+        probe_ms = time_replays(lambda: tile_ops.check(probes.load().nfn_mi355_read_probe_v1(
             source.data_ptr(), nbytes, sink.data_ptr(), handle), "read probe"), steps, warmup)
         result[f"{mib}_MiB"] = {"sum_read_TB/s": round(nbytes / read_ms / 1e9, 2),
                                 "copy_read_plus_write_TB/s": round(2 * nbytes / copy_ms / 1e9, 2),

@@ -804,8 +804,13 @@ int nfn_native_tile_scale_inplace_float32(
 
 /* ==== additions: no counterpart in the reference ========================= */
 
-/* Version of the additions below, 1: an engine that binds any nfn_mi355_* symbol checks it
- * the way it checks the reference's four version symbols (resident_glimmer_cuda.cpp:496-501). */
+/* Version of the additions below, 2: an engine that binds any nfn_mi355_* symbol checks it
+ * the way it checks the reference's four version symbols (resident_glimmer_cuda.cpp:496-501).
+ * Version 2: nfn_mi355_attention_workspace_v1 takes the stream the loan is for as a third
+ * argument (a caller built against the two-argument form must not call it); the measurement
+ * probes live in a library of their own (nfn_mi355_probes.h); the small-batch workspace of
+ * five rows and more also holds the activations in matrix-operand order (the query
+ * nfn_native_tile_k_quant_mmq_workspace_bytes_v1 returns the larger size). */
 int nfn_mi355_abi_version(void);
 
 /* lm_head GEMV with the argmax fused in: logits never reach memory.  The
@@ -979,45 +984,6 @@ int nfn_mi355_dflash_block_attention_split_v1(
  * captured into a graph keep the form they were captured with.  0 on success,
  * 1 for a misaligned pointer, a size without a pointer, or a 33rd loan. */
 int nfn_mi355_attention_workspace_v1(void* workspace, int64_t workspace_nbytes, void* cuda_stream);
-
-/* Shader clock under load, a measurement aid (no counterpart in the reference;
- * for benchmarks that price a kernel against the matrix-core peak at the clock
- * the chip really ran at).  Enqueues one wave that waits about `microseconds`
- * (1..100000) on `cuda_stream` and then writes three uint64 to
- * `cycles_and_ticks` (device memory, 24 bytes): shader cycles, ticks of the
- * constant device clock, and that clock's ticks per second
- * (hipDeviceAttributeWallClockRate).  Launch it on a side stream while the work
- * under test runs on another. */
-int nfn_mi355_shader_clock_probe_v1(
-    uint64_t* cycles_and_ticks,
-    int64_t microseconds,
-    void* cuda_stream);
-
-/* Matrix-core rates from registers, a measurement aid (no counterpart in the
- * reference): `groups` workgroups of four waves each run `steps` steps of one
- * 32 x 32 x 32 product per wave.  mode 0: fp16 operands (two
- * v_mfma_f32_32x32x16_f16); mode 1: int8 operands (one
- * v_mfma_i32_32x32x32_i8); mode 2: the int8 form a K-quant prefill with 16-bit
- * activation codes would need -- two int8 planes into fresh accumulators and,
- * after every 32 values, the rescale of all 16 accumulators by the sub-block's
- * scale.  The benchmark times the three and reports their ratio: the
- * measurement behind the reserved NFN_MI355_GEMM_INT8 mode.  `sink`: device
- * memory of one float per workgroup, never written in practice. */
-int nfn_mi355_mfma_rate_probe_v1(int mode, int steps, int groups, float* sink, void* cuda_stream);
-
-/* The floor under a launch, a measurement aid like the clock probe (no
- * counterpart in the reference): one workgroup per compute unit reads
- * `nbytes` of `data` (16-byte aligned; rounded down to whole 16-byte pieces per
- * workgroup) with plain coalesced loads and stores nothing; with nbytes = 0 it
- * is an empty kernel of the same grid.  Timed back to back in a graph over
- * the bytes a decode launch streams, it is what that launch would cost with
- * no arithmetic at all.  `sink`: device memory of one uint32 per compute unit
- * (1,024 bytes are enough), never written in practice. */
-int nfn_mi355_read_probe_v1(
-    const void* data,
-    int64_t nbytes,
-    uint32_t* sink,
-    void* cuda_stream);
 
 #ifdef __cplusplus
 }

@@ -1,7 +1,8 @@
 """Build recipe for the HIP library and the host-side library (quantizer, GGUF tensor table).
 
 `build_all()` compiles every source for gfx950 with hipcc and links
-`neuralfn_amd/lib/libnfn_mi355_tile_ops.so`; hipcc cross-compiles, so this runs
+`neuralfn_amd/lib/libnfn_mi355_tile_ops.so` (and the benchmark's measurement aids into
+`libnfn_mi355_probes.so`); hipcc cross-compiles, so this runs
 on a machine without a GPU.  Nothing is built at import time: tests, the smoke
 check and the benchmark load what is already built.
 """
@@ -18,6 +19,7 @@ CSRC = PACKAGE / "csrc"
 LIB_DIR = PACKAGE / "lib"
 OBJ_DIR = PACKAGE / "build"
 TILE_OPS_LIB = LIB_DIR / "libnfn_mi355_tile_ops.so"
+PROBES_LIB = LIB_DIR / "libnfn_mi355_probes.so"
 HOST_LIB = LIB_DIR / "libnfn_mi355_kquant_host.so"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -81,6 +83,16 @@ def build_tile_ops(jobs: int = 8) -> Path:
     return TILE_OPS_LIB
 
 
+def build_probes() -> Path:
+    """The benchmark's measurement aids: a library of their own, not part of the product."""
+    LIB_DIR.mkdir(exist_ok=True)
+    OBJ_DIR.mkdir(exist_ok=True)
+    target = OBJ_DIR / "probes.hip.o"
+    _run([HIPCC, *DEVICE_FLAGS, "-c", str(CSRC / "probes" / "probes.hip"), "-o", str(target)])
+    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(PROBES_LIB), str(target)])
+    return PROBES_LIB
+
+
 def build_host() -> Path:
     LIB_DIR.mkdir(exist_ok=True)
     sources = sorted((CSRC / "host").glob("*.cpp"))
@@ -91,10 +103,12 @@ def build_host() -> Path:
 
 def build_all() -> None:
     build_tile_ops()
+    build_probes()
     build_host()
 
 
 if __name__ == "__main__":
     build_all()
     print(TILE_OPS_LIB)
+    print(PROBES_LIB)
     print(HOST_LIB)

@@ -183,7 +183,7 @@ int nfn_native_tile_strict_math_abi_version(void) { return 1; }
 int nfn_native_tile_packed_weight_abi_version(void) { return NFN_NATIVE_TILE_PACKED_WEIGHT_V1; }
 int nfn_native_tile_glimmer_inference_abi_version(void) { return 1; }
 int nfn_native_tile_k_quant_mmq_abi_version(void) { return NFN_NATIVE_TILE_K_QUANT_MMQ_V1; }
-int nfn_mi355_abi_version(void) { return 1; }
+int nfn_mi355_abi_version(void) { return 2; }
 
 const char* nfn_native_tile_ops_error_string(int code) {
     if (code == NFN_MI355_STATUS_STATIC_SCRATCH_EXCEEDED) {
@@ -210,8 +210,10 @@ bool float_matrix_cores_pay(const Descriptor& weight, std::int64_t rows) {
     const double decoded_per_us = weight.encoding == kEncQ4K || weight.encoding == kEncQ5K ? 4.6e5
                                   : weight.encoding == kEncQ6K                             ? 3.0e5
                                                                                            : 2.4e5;
-    const double vector_pass_us = weights / decoded_per_us < 6.0 ? 6.0 : weights / decoded_per_us;
-    const double vector_us = static_cast<double>((rows + 7) / 8) * vector_pass_us;
+    // the vector kernel's passes of eight rows are workgroups of one launch, not launches one
+    // after another: the launch floor counts once
+    const double vector_work_us = static_cast<double>((rows + 7) / 8) * weights / decoded_per_us;
+    const double vector_us = vector_work_us < 6.0 ? 6.0 : vector_work_us;
     const double tile_flop = 128.0 * 64.0 * 2.0 * static_cast<double>(weight.input_dim);
     const double passes = gemm_f32_tile_passes(weight, rows);
     const double alone_us = tile_flop / 3.6e5;
@@ -881,42 +883,6 @@ int nfn_mi355_k_quant_gemm_multi_float32_v1(const Descriptor* const* descriptors
     for (std::int64_t index = 0; index < operation_count; ++index) {
         launch_gemm_f16_converted(normalized[index], outputs[index], rows, workspace, stream);
     }
-    return launch_status();
-}
-
-int nfn_mi355_shader_clock_probe_v1(std::uint64_t* cycles_and_ticks, std::int64_t microseconds,
-                                    void* cuda_stream) {
-    if (cycles_and_ticks == nullptr || microseconds < 1 || microseconds > 100000) return kInvalid;
-    int ticks_per_millisecond = 0;  // the attribute is in kHz
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess ||
-        hipDeviceGetAttribute(&ticks_per_millisecond, hipDeviceAttributeWallClockRate, device) !=
-            hipSuccess ||
-        ticks_per_millisecond <= 0) {
-        return static_cast<int>(hipErrorNotSupported);
-    }
-    launch_clock_probe(cycles_and_ticks, microseconds * ticks_per_millisecond / 1000,
-                       static_cast<std::uint64_t>(ticks_per_millisecond) * 1000,
-                       as_stream(cuda_stream));
-    return launch_status();
-}
-
-int nfn_mi355_mfma_rate_probe_v1(int mode, int steps, int groups, float* sink, void* cuda_stream) {
-    if (mode < 0 || mode > 2 || steps < 1 || steps > (1 << 20) || groups < 1 || groups > 65536 ||
-        sink == nullptr) {
-        return kInvalid;
-    }
-    launch_mfma_rate_probe(mode, steps, groups, sink, as_stream(cuda_stream));
-    return launch_status();
-}
-
-int nfn_mi355_read_probe_v1(const void* data, std::int64_t nbytes, std::uint32_t* sink,
-                            void* cuda_stream) {
-    if (nbytes < 0 || sink == nullptr || (nbytes > 0 && data == nullptr) ||
-        reinterpret_cast<std::uintptr_t>(data) % 16 != 0) {
-        return kInvalid;
-    }
-    launch_read_probe(data, nbytes, sink, as_stream(cuda_stream));
     return launch_status();
 }
 

@@ -409,7 +409,7 @@ __device__ __forceinline__ void k_step(
     const std::uint8_t* a_fetch, std::int64_t row_block_bytes, const std::uint8_t* b_global,
     int fetch_step) {
     WeightFragments ahead;
-    std::uint32_t w[2];
+    std::uint32_t w[2], v[2];
 
     if constexpr (RB == 1) {
         // One row block per wave: 16 slots carry the same side work.
@@ -417,24 +417,24 @@ __device__ __forceinline__ void k_step(
         NFN_SLOT(a_now.r0k0, current.c1, acc[0][1], b_next.prepare_scales(header);
                  ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 1))
         NFN_SLOT(a_now.r0k0, current.c2, acc[0][2], b_next.template group_a<0>(w);
-                 NFN_WRITE8(b_write, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
-        NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_b<0>(w);
-                 NFN_WRITE8(b_write + 64, w); ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
+                 ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
+        NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_a<1>(v);
+                 NFN_WRITE16(b_write, w[0], w[1], v[0], v[1]); ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
                  ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
-        NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<1>(w);
-                 NFN_WRITE8(b_write + 8, w); current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
+        NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<2>(w);
+                 current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
                  a_now.r0k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 0))
-        NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<1>(w);
-                 NFN_WRITE8(b_write + 72, w); current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
-        NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2], b_next.template group_a<2>(w);
-                 NFN_WRITE8(b_write + 16, w); current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2))
-        NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3], b_next.template group_b<2>(w);
-                 NFN_WRITE8(b_write + 80, w); current.c3 = NFN_READ_WEIGHTS(b_read, 3, 2))
-        NFN_SLOT(a_now.r0k2, current.c0, acc[0][0], b_next.template group_a<3>(w);
-                 NFN_WRITE8(b_write + 24, w); ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 3);
+        NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_a<3>(v);
+                 NFN_WRITE16(b_write + 16, w[0], w[1], v[0], v[1]); current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
+        NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2], b_next.template group_b<0>(w);
+                 current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2))
+        NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3], b_next.template group_b<1>(v);
+                 NFN_WRITE16(b_write + 64, w[0], w[1], v[0], v[1]); current.c3 = NFN_READ_WEIGHTS(b_read, 3, 2))
+        NFN_SLOT(a_now.r0k2, current.c0, acc[0][0], b_next.template group_b<2>(w);
+                 ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 3);
                  a_now.r0k1 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 1))
-        NFN_SLOT(a_now.r0k2, current.c1, acc[0][1], b_next.template group_b<3>(w);
-                 NFN_WRITE8(b_write + 88, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 3))
+        NFN_SLOT(a_now.r0k2, current.c1, acc[0][1], b_next.template group_b<3>(v);
+                 NFN_WRITE16(b_write + 80, w[0], w[1], v[0], v[1]); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 3))
         NFN_SLOT(a_now.r0k2, current.c2, acc[0][2], ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 3))
         NFN_SLOT(a_now.r0k2, current.c3, acc[0][3], ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 3))
         __syncthreads();
@@ -455,24 +455,24 @@ __device__ __forceinline__ void k_step(
     NFN_SLOT(a_now.r0k0, current.c1, acc[0][1], b_next.prepare_scales(header);
              ahead.c0 = NFN_READ_WEIGHTS(b_read, 0, 1))
     NFN_SLOT(a_now.r0k0, current.c2, acc[0][2], b_next.template group_a<0>(w);
-             NFN_WRITE8(b_write, w); ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
-    NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_b<0>(w);
-             NFN_WRITE8(b_write + 64, w))
-    NFN_SLOT(a_now.r1k0, current.c0, acc[1][0], b_next.template group_a<1>(w);
-             NFN_WRITE8(b_write + 8, w); ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
+             ahead.c1 = NFN_READ_WEIGHTS(b_read, 1, 1))
+    NFN_SLOT(a_now.r0k0, current.c3, acc[0][3], b_next.template group_a<1>(v);
+             NFN_WRITE16(b_write, w[0], w[1], v[0], v[1]))
+    NFN_SLOT(a_now.r1k0, current.c0, acc[1][0], b_next.template group_a<2>(w);
+             ahead.c2 = NFN_READ_WEIGHTS(b_read, 2, 1);
              a_now.r0k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 0, 0))
-    NFN_SLOT(a_now.r1k0, current.c1, acc[1][1], b_next.template group_b<1>(w);
-             NFN_WRITE8(b_write + 72, w))
-    NFN_SLOT(a_now.r1k0, current.c2, acc[1][2], b_next.template group_a<2>(w);
-             NFN_WRITE8(b_write + 16, w); ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
-    NFN_SLOT(a_now.r1k0, current.c3, acc[1][3], b_next.template group_b<2>(w);
-             NFN_WRITE8(b_write + 80, w))
+    NFN_SLOT(a_now.r1k0, current.c1, acc[1][1], b_next.template group_a<3>(v);
+             NFN_WRITE16(b_write + 16, w[0], w[1], v[0], v[1]))
+    NFN_SLOT(a_now.r1k0, current.c2, acc[1][2], b_next.template group_b<0>(w);
+             ahead.c3 = NFN_READ_WEIGHTS(b_read, 3, 1))
+    NFN_SLOT(a_now.r1k0, current.c3, acc[1][3], b_next.template group_b<1>(v);
+             NFN_WRITE16(b_write + 64, w[0], w[1], v[0], v[1]))
     // K chunk 1: read chunk 2, finish decoding
-    NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_a<3>(w);
-             NFN_WRITE8(b_write + 24, w); current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
+    NFN_SLOT(a_now.r0k1, ahead.c0, acc[0][0], b_next.template group_b<2>(w);
+             current.c0 = NFN_READ_WEIGHTS(b_read, 0, 2);
              a_now.r1k0 = NFN_LOAD_ACTIVATIONS(a_fetch, 1, 0))
-    NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<3>(w);
-             NFN_WRITE8(b_write + 88, w))
+    NFN_SLOT(a_now.r0k1, ahead.c1, acc[0][1], b_next.template group_b<3>(v);
+             NFN_WRITE16(b_write + 80, w[0], w[1], v[0], v[1]))
     NFN_SLOT(a_now.r0k1, ahead.c2, acc[0][2], current.c1 = NFN_READ_WEIGHTS(b_read, 1, 2))
     NFN_SLOT(a_now.r0k1, ahead.c3, acc[0][3], (void)0)
     NFN_SLOT(a_now.r1k1, ahead.c0, acc[1][0], current.c2 = NFN_READ_WEIGHTS(b_read, 2, 2);
@@ -525,7 +525,7 @@ constexpr int kBlockBytes = ENC == kEncQ4K ? 144 : ENC == kEncQ5K ? 176 : ENC ==
 // matrix pipe busy.  With 256-row tiles the Q6_K decode holds too much live
 // state for two.
 template <std::uint32_t ENC, int RB>
-constexpr int kWavesPerSimd = ENC == kEncQ6K ? RB == 1 ? 2 : 1 : RB == 1 ? 3 : 2;
+constexpr int kWavesPerSimd = ENC == kEncQ6K ? RB == 1 ? 2 : 1 : RB == 1 ? (ENC == kEncQ5K ? 2 : 3) : 2;
 
 // RB: 32-row blocks per wave; the workgroup's tile is 128*RB rows by 128 columns.
 template <std::uint32_t ENC, int RB>
@@ -559,8 +559,10 @@ __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<ENC, RB>, kWavesPerSimd<ENC, RB
         static_cast<std::int64_t>(first_block) * 16 * kFragmentBytes + lane * 16;
     constexpr int kStepBytes = (kBK / 16) * kFragmentBytes;
     // weights: thread -> (row, which 16 positions of the two 32-value groups)
-    const int b_row = tid >> 1;
-    const int b_half = tid & 1;
+    // (sixteen consecutive lanes write sixteen consecutive stage rows: with rows of 144 bytes
+    // their 16-byte pieces fall into distinct banks, as the fragment reads do)
+    const int b_row = tid & 127;
+    const int b_half = tid >> 7;
     const std::uint8_t* b_global = weights + min(n0 + b_row, output_dim - 1) * row_stride +
         static_cast<std::int64_t>(first_block) * kBlockBytes<ENC>;
     const int b_target = b_row * kRowBytes + b_half * 32;

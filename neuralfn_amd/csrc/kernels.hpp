@@ -122,16 +122,4 @@ void launch_gqa_decode_split_device_position(
     const NfnNativeTileGlimmerGqaDecodeDescriptorV1& descriptor, const std::int64_t* device_position,
     std::int64_t sliding_window, bool whole_context, float* partials, hipStream_t stream);
 
-// clock_probe.hip — out[0] = shader cycles, out[1] = ticks of the constant
-// clock over a wait of about `ticks` ticks, out[2] = ticks_per_second.
-void launch_clock_probe(std::uint64_t* out, std::int64_t ticks, std::uint64_t ticks_per_second,
-                        hipStream_t stream);
-// clock_probe.hip — one workgroup per compute unit reads `nbytes` (rounded down to a
-// whole 16 bytes per workgroup) and stores nothing; nbytes 0 = an empty kernel.
-void launch_read_probe(const void* data, std::int64_t nbytes, std::uint32_t* sink,
-                       hipStream_t stream);
-// clock_probe.hip — `groups` workgroups of four waves run `steps` 32 x 32 x 32 matrix-core steps
-// each from registers: mode 0 fp16, 1 int8, 2 two int8 planes + the per-32 rescale.
-void launch_mfma_rate_probe(int mode, int steps, int groups, float* sink, hipStream_t stream);
-
 }  // namespace nfn

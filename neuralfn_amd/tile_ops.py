@@ -203,9 +203,6 @@ SIGNATURES = {
         ctypes.c_int, [_DESC, _P, _P, _I64, _P, _I64, ctypes.c_int, _P]),
     "nfn_mi355_k_quant_gemm_multi_float32_v1": (
         ctypes.c_int, [_DESC_ARRAY, _P, _PTR_ARRAY, _I64, _I64, _P, _I64, ctypes.c_int, _P]),
-    "nfn_mi355_shader_clock_probe_v1": (ctypes.c_int, [_P, _I64, _P]),
-    "nfn_mi355_read_probe_v1": (ctypes.c_int, [_P, _I64, _P, _P]),
-    "nfn_mi355_mfma_rate_probe_v1": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int, _P, _P]),
     "nfn_mi355_gqa_decode_split_workspace_bytes_v1": (_I64, [_I64, _I64]),
     "nfn_mi355_attention_workspace_v1": (ctypes.c_int, [_P, _I64, _P]),
     "nfn_mi355_dflash_block_attention_split_v1": (
@@ -742,31 +739,3 @@ def gemm_multi(weights: Sequence[PackedWeight], x, mode: int = GEMM_F16, workspa
         _descriptor_array(descriptors), x.data_ptr(), _pointer_array(outputs), len(weights), rows,
         workspace.data_ptr(), workspace.numel(), mode, stream), "k_quant_gemm_multi")
     return outputs
-
-
-class ShaderClockProbe:
-    """nfn_mi355_shader_clock_probe_v1 on a side stream: the shader clock while other work runs.
-
-    start() enqueues the wait, the caller then runs the work under test on its
-    own stream and synchronizes it, megahertz() waits for the probe and returns
-    shader cycles per second / 1e6 over the probe's window.
-    """
-
-    def __init__(self, device):
-        import torch
-        self._torch = torch
-        self.stream = torch.cuda.Stream(device=device)
-        self.result = torch.zeros(3, dtype=torch.int64, device=device)
-
-    def start(self, microseconds: int) -> None:
-        self.result.zero_()
-        self._torch.cuda.current_stream().synchronize()
-        check(load().nfn_mi355_shader_clock_probe_v1(
-            self.result.data_ptr(), microseconds, int(self.stream.cuda_stream)), "clock probe")
-
-    def megahertz(self) -> float:
-        self.stream.synchronize()
-        cycles, ticks, ticks_per_second = (int(v) for v in self.result.tolist())
-        if ticks <= 0:
-            raise RuntimeError("the clock probe reported no elapsed ticks")
-        return cycles / ticks * ticks_per_second / 1e6

@@ -34,6 +34,21 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     assert set(names) == set(tile_ops.SIGNATURES), "binding and header disagree"
 
 
+def test_the_probes_library_exports_what_its_header_declares():
+    from neuralfn_amd import probes
+    header = ROOT / "include" / "nfn_mi355_probes.h"
+    text = re.sub(r"/\*.*?\*/", "", header.read_text(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(nfn_mi355_[a-z0-9_]+)\s*\(", text)))
+    assert set(names) == set(probes.SIGNATURES)
+    loaded = probes.load()
+    for name in names:
+        assert hasattr(loaded, name), f"{name} is declared but not exported"
+    # and the product library exports none of them
+    product = tile_ops.load()
+    for name in names:
+        assert not hasattr(product, name), f"{name} is a measurement aid inside the product library"
+
+
 def test_versions(lib):
     for name in ("nfn_native_tile_ops_abi_version", "nfn_native_tile_strict_math_abi_version",
                  "nfn_native_tile_packed_weight_abi_version",
@@ -197,3 +212,36 @@ def test_other_entry_points_fail_closed(lib):
 def test_error_string_never_null(lib):
     for code in (0, 1, 2, 98, 719, 12345):
         assert lib.nfn_native_tile_ops_error_string(code)
+
+
+def test_the_reference_engines_own_loader_opens_the_library():
+    """Runtime::Runtime of the reference engine (resident_glimmer_cuda.cpp:329-630), compiled
+    from the reference checkout where it lies (oracle/loader_harness.cpp, `make -C oracle ref`),
+    constructs itself on this library: every required symbol resolves, no optional group is
+    only partly present, the four ABI versions are the ones it insists on.  Its runtime library
+    is the reference's own CPU double (tests/cpp/fake_cuda_runtime.cpp), so no GPU is touched;
+    that double has no graph functions, hence decode_graphs stays off."""
+    loader = ROOT / "oracle" / "_ref" / "libnfn_engine_loader_ref.so"
+    runtime = ROOT / "oracle" / "_ref" / "libnfn_fake_cuda_runtime_ref.so"
+    if not loader.exists() or not runtime.exists():
+        pytest.skip("oracle/_ref is not built: the reference checkout is absent on this machine")
+    harness = ctypes.CDLL(str(loader))
+    harness.nfn_ref_loader_probe.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p,
+                                             ctypes.c_int]
+    harness.nfn_ref_loader_probe.restype = ctypes.c_int
+    report = ctypes.create_string_buffer(4096)
+    status = harness.nfn_ref_loader_probe(str(tile_ops.LIB_PATH.resolve()).encode(),
+                                          str(runtime.resolve()).encode(), report, len(report))
+    text = report.value.decode()
+    assert status == 0, f"the engine's loader refused the library: {text}"
+    bound = dict(line.split("=", 1) for line in text.splitlines() if "=" in line)
+    for group in ("q8_linear", "k_quant_mmq", "k_quant_mmq_gated", "k_quant_mmq_swiglu",
+                  "k_quant_mmvq", "k_quant_mmvq_rows", "k_quant_mmvq_prequantized",
+                  "rms_to_mmvq_handoff", "fused_residual_norm", "short_attention_split",
+                  "cooperative_batch_rms"):
+        assert bound.get(group) == "1", f"the engine did not bind {group}: {text}"
+    assert bound["tile_path"] == str(tile_ops.LIB_PATH.resolve())
+    # a relative path is refused by the engine before it loads anything
+    status = harness.nfn_ref_loader_probe(b"libnfn_mi355_tile_ops.so", str(runtime).encode(),
+                                          report, len(report))
+    assert status == 1 and "absolute" in report.value.decode()
