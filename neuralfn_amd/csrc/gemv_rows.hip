@@ -22,7 +22,9 @@
 // tokens, the integers of a unit, and replays the float tail above.  Wave w takes the classes
 // w and 15 - w (an even share of any row length), keeps the four chains of a class per token
 // in registers, and leaves (c0 + c1) + (c2 + c3) per class, token and row in LDS; after one
-// barrier a thread per (token, row) adds the 16 classes in the tree's order.
+// barrier a thread per (token, row) adds the 16 classes in the tree's order.  A workgroup
+// walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... with the loads of the next tile's
+// first block in flight under the last block of the one before.
 // One pass over the weights for up to 16 tokens.
 #include "common.hpp"
 #include "gemv_rows.hpp"
@@ -119,7 +121,8 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     constexpr int kBlockBytes = F::kBlockBytes;
     constexpr int kQuants = kQ5 ? 48 : 16;
     constexpr int kTokens = 2 * S;
-    __shared__ float class_sums[kClasses][kTokens][kRowsTile];
+    // (two buffers of class sums: the workgroup's waves meet once per tile)
+    __shared__ float class_sums[2][kClasses][kTokens][kRowsTile];
     __shared__ __attribute__((aligned(16))) std::uint8_t packed_tiles[kRowsWaves][F::kTileBytes];
 
     const int lane = threadIdx.x & 63;
@@ -128,36 +131,45 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const int h = lane >> 5;
     const int blocks = input_dim >> 8;
 
-    // the tile's projection and rows (uniform)
-    const std::uint32_t tile = blockIdx.x;
-    int which = 0;
+    // A workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the loads of a
+    // tile's first block go out under the arithmetic of the tile before.
+    const std::uint32_t first_tile = blockIdx.x;
+    const int my_tiles = static_cast<int>((total_tiles - first_tile + gridDim.x - 1) / gridDim.x);
+    auto projection_of = [&](std::uint32_t tile) {
+        int which = 0;
 #pragma unroll
-    for (int index = 1; index < 4; ++index) {
-        if (index < set.count && tile >= set.op[index].first_tile) which = index;
-    }
-    const Projection op = pick(set, which);
-    const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kRowsTile;
-    const int valid_rows =
-        static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
-    const std::uint8_t* tile_rows = op.data + row0 * op.row_stride;
+        for (int index = 1; index < 4; ++index) {
+            if (index < set.count && tile >= set.op[index].first_tile) which = index;
+        }
+        return pick(set, which);
+    };
 
-    // the chunks this lane copies per block: chunk n = 64 i + lane of the 32 x kChunks, 9 (11)
-    // to a row; the LDS tile is the same bytes row after row, so chunk n goes to byte 16 n
-    // (the lanes past the last chunk repeat it)
+    // What the loads of a tile need: its first row and, per lane, where the chunks it copies
+    // per block lie: chunk n = 64 i + lane of the 32 x kChunks, 9 (11) to a row; the LDS tile
+    // is the same bytes row after row, so chunk n goes to byte 16 n (the lanes past the last
+    // chunk repeat it).
+    const std::uint8_t* tile_rows;
     std::uint32_t chunk_offset[F::kLoads];
+    auto aim = [&](std::uint32_t tile) {
+        const Projection op = projection_of(tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kRowsTile;
+        const int valid_rows =
+            static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
+        tile_rows = op.data + row0 * op.row_stride;
 #pragma unroll
-    for (int i = 0; i < F::kLoads; ++i) {
-        const int chunk = min(i * kWave + lane, F::kTileChunks - 1);
-        const int row = chunk / F::kChunks;
-        const int col = chunk - row * F::kChunks;
-        chunk_offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
-                static_cast<std::uint32_t>(op.row_stride) + col * 16;
-    }
+        for (int i = 0; i < F::kLoads; ++i) {
+            const int chunk = min(i * kWave + lane, F::kTileChunks - 1);
+            const int row = chunk / F::kChunks;
+            const int col = chunk - row * F::kChunks;
+            chunk_offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
+                    static_cast<std::uint32_t>(op.row_stride) + col * 16;
+        }
+    };
     const int last_slot = min((F::kLoads - 1) * kWave + lane, F::kTileChunks - 1) * 16;
     std::uint8_t* const my_tile = packed_tiles[wave];
     const std::uint8_t* const my_row = my_tile + j * kBlockBytes;
 
-    // this wave's steps: the blocks of class `wave`, then those of class 15 - wave
+    // this wave's steps of a tile: the blocks of class `wave`, then those of class 15 - wave
     const int class0 = wave;
     const int class1 = kClasses - 1 - wave;
     const int count0 = class0 < blocks ? (blocks - class0 + kClasses - 1) / kClasses : 0;
@@ -167,9 +179,12 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     auto block_of = [&](int step) {
         return step < count0 ? class0 + kClasses * step : class1 + kClasses * (step - count0);
     };
-    auto fetch = [&](RowsStage<kQ5, S>& stage, int step) {
-        // (a step past the wave's last repeats it; a wave with no block at all reads the row's last)
-        const int block = min(block_of(min(step, max(total - 1, 0))), blocks - 1);
+    std::uint32_t fetch_tile = first_tile;
+    int fetch_step = 0;
+    aim(fetch_tile);
+    // the loads of the next step of the walk; past its end the last block again
+    auto fetch = [&](RowsStage<kQ5, S>& stage) {
+        const int block = min(block_of(min(fetch_step, max(total - 1, 0))), blocks - 1);
         const std::uint8_t* weights = tile_rows + static_cast<std::int64_t>(block) * kBlockBytes;
 #pragma unroll
         for (int i = 0; i < F::kLoads; ++i) {
@@ -179,6 +194,11 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
 #pragma unroll
         for (int sub = 0; sub < 8; ++sub) {
             stage.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
+        }
+        if (++fetch_step >= total && fetch_tile + gridDim.x < total_tiles) {
+            fetch_step = 0;
+            fetch_tile += gridDim.x;
+            aim(fetch_tile);
         }
     };
 
@@ -294,50 +314,77 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         }
     };
     // a class is complete: (c0 + c1) + (c2 + c3) per token goes to LDS
+    int parity = 0;
     auto finish_class = [&](int cls) {
 #pragma unroll
         for (int slot = 0; slot < S; ++slot) {
-            class_sums[cls][S * h + slot][j] =
+            class_sums[parity][cls][S * h + slot][j] =
                 (acc[0][slot] + acc[1][slot]) + (acc[2][slot] + acc[3][slot]);
 #pragma unroll
             for (int p = 0; p < 4; ++p) acc[p][slot] = 0.0f;
         }
     };
+    // a tile is complete: after the barrier a thread per (token, row) adds the 16 classes in
+    // the order of the one-row kernel's butterfly
+    std::uint32_t work_tile = first_tile;
+    auto finish_tile = [&]() {
+        __syncthreads();
+        const Projection op = projection_of(work_tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(work_tile - op.first_tile) * kRowsTile;
+        const int valid_rows =
+            static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
+        const int token = static_cast<int>(threadIdx.x) >> 5;
+        if (token < kTokens && token < tokens && j < valid_rows) {
+            float pairs[8];
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                pairs[m] = class_sums[parity][2 * m][token][j] + class_sums[parity][2 * m + 1][token][j];
+            }
+            const float q0 = pairs[0] + pairs[1];
+            const float q1 = pairs[2] + pairs[3];
+            const float q2 = pairs[4] + pairs[5];
+            const float q3 = pairs[6] + pairs[7];
+            op.output[static_cast<std::int64_t>(token) * op.output_dim + row0 + j] = (q0 + q1) + (q2 + q3);
+        }
+        parity ^= 1;
+        work_tile += gridDim.x;
+    };
 
+    if (total == 0) {
+        // (rows of fewer blocks than classes: this wave only takes part in the sums)
+        for (int n = 0; n < my_tiles; ++n) {
+            finish_class(class0);
+            finish_class(class1);
+            finish_tile();
+        }
+        return;
+    }
     // Two named register stages (an array of them indexed in the loop ends up in scratch memory).
     RowsStage<kQ5, S> even, odd;
-    fetch(even, 0);
-    if (count0 == 0) finish_class(class0);
-    if (count1 == 0) finish_class(class1);
-    auto finish_step = [&](int step) {
-        if (step == count0 - 1) finish_class(class0);
-        if (step == total - 1 && count1 > 0) finish_class(class1);
+    fetch(even);
+    int work_step = 0;
+    // (class0 = wave has at least as many blocks as class1 = 15 - wave; a class without
+    // blocks leaves the zeros the sums start from)
+    auto finish_step = [&]() {
+        if (work_step == count0 - 1) finish_class(class0);
+        if (work_step == total - 1) {
+            finish_class(class1);
+            finish_tile();
+            work_step = 0;
+        } else {
+            ++work_step;
+        }
     };
-    for (int step = 0; step < total; step += 2) {
-        fetch(odd, step + 1);
-        compute(even, step);
-        finish_step(step);
-        if (step + 1 < total) {
-            fetch(even, step + 2);
-            compute(odd, step + 1);
-            finish_step(step + 1);
+    const int steps = my_tiles * total;
+    for (int step = 0; step < steps; step += 2) {
+        fetch(odd);
+        compute(even, work_step);
+        finish_step();
+        if (step + 1 < steps) {
+            fetch(even);
+            compute(odd, work_step);
+            finish_step();
         }
-    }
-    __syncthreads();
-
-    // a thread per (token, row): the 16 classes in the order of the one-row kernel's butterfly
-    const int token = static_cast<int>(threadIdx.x) >> 5;
-    if (token < kTokens && token < tokens && j < valid_rows) {
-        float pairs[8];
-#pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            pairs[m] = class_sums[2 * m][token][j] + class_sums[2 * m + 1][token][j];
-        }
-        const float q0 = pairs[0] + pairs[1];
-        const float q1 = pairs[2] + pairs[3];
-        const float q2 = pairs[4] + pairs[5];
-        const float q3 = pairs[6] + pairs[7];
-        op.output[static_cast<std::int64_t>(token) * op.output_dim + row0 + j] = (q0 + q1) + (q2 + q3);
     }
 }
 
@@ -348,7 +395,9 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, h
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kRowsTile - 1) / kRowsTile);
     }
-    const dim3 grid(tiles), block(kRowsThreads);
+    // one workgroup per compute unit walks the tiles; fewer tiles: a workgroup each
+    const std::uint32_t units = static_cast<std::uint32_t>(compute_units());
+    const dim3 grid(tiles < units ? tiles : units), block(kRowsThreads);
     const int input_dim = static_cast<int>(set.input_dim);
     if (tokens <= 4) {
         hipLaunchKernelGGL((gemv_rows_kernel<ENC, 2>), grid, block, 0, stream, image, tokens,
