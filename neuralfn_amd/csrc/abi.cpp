@@ -26,8 +26,10 @@ constexpr std::int64_t kMaxSmallRows = 16;
 constexpr std::int64_t kMaxOperations = 4;
 constexpr std::int64_t kFirstHalfRows = 5;  // rows from which the fp16 matrix-core kernel takes a batch
 // rows from which the verifier family's Q4_K / Q5_K projections run on the int8 matrix cores
-// (one pass over the weights behind a quantizer launch; below: the dot kernel's token passes)
-constexpr std::int64_t kFirstVerifierMatrixRows = 5;
+// (one pass over the weights behind a quantizer launch; below: the dot kernel's token passes,
+// which are faster up to three rows: 9.0 / 12.4 / 13.9 us per launch of the attention
+// projections at 2 / 3 / 4 rows against 12.8 for the matrix-core kernel at any of them)
+constexpr std::int64_t kFirstVerifierMatrixRows = 4;
 // Private activation records of the small-batch path, 576 bytes per token and
 // 256 values (two int8 planes of a 16-bit fixed-point code, group sums, scale,
 // block maximum): 72 bytes per 32 values, the unit the workspace is sized in.

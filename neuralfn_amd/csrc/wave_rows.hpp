@@ -265,11 +265,11 @@ __device__ __forceinline__ WaveRows wave_rows(int group, int wave, int rows_per_
 // once, equally loaded) is fastest until a wave would own more than about three
 // rows; from there the grid grows to up to four workgroups per unit, which a
 // large weight stream needs to keep enough loads in flight.
-inline std::int64_t decode_groups(std::int64_t rows, int waves_per_group) {
+inline std::int64_t decode_groups(std::int64_t rows, int waves_per_group, int most_per_unit = 4) {
     const std::int64_t units = compute_units();
     std::int64_t per_unit = rows / (units * waves_per_group * 3);
     if (per_unit < 1) per_unit = 1;
-    if (per_unit > 4) per_unit = 4;
+    if (per_unit > most_per_unit) per_unit = most_per_unit;
     std::int64_t groups = units * per_unit;
     const std::int64_t useful = (rows + waves_per_group - 1) / waves_per_group;  // a row per wave
     return groups < useful ? groups : useful;

@@ -588,7 +588,7 @@ def test_decode_dot_kernel_row_lengths(cuda, oracle, encoding, in_dim):
 @pytest.mark.parametrize("in_dim", [256, 2304, 4096, 6656, 8448, 16384])
 @pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
 def test_verifier_matrix_core_rows_equal_the_one_row_kernel(cuda, oracle, encoding, in_dim):
-    """From five rows on the verifier family's Q4_K / Q5_K projections run on the int8 matrix
+    """From four rows on the verifier family's Q4_K / Q5_K projections run on the int8 matrix
     cores, one pass over the weights: every row must still carry the one-row kernel's bits.
     Row lengths: one block (15 empty classes), 9 blocks, exactly one 16-block slice, 26 blocks
     (classes of one and two blocks), 33 and 64 blocks; output widths off the 32-row tile."""
@@ -601,7 +601,7 @@ def test_verifier_matrix_core_rows_equal_the_one_row_kernel(cuda, oracle, encodi
     alone = [tile_ops.multi_linear(weights, to_device(x[row:row + 1], cuda), one) for row in range(16)]
     for y, p, n in zip(alone[3], packed, out_dims):
         assert normalised_error(y.cpu().numpy(), oracle.linear(encoding, p, n, in_dim, x[3:4])) <= TOLERANCE
-    for rows in (5, 8, 9, 13, 16):
+    for rows in (4, 5, 8, 9, 13, 16):
         workspace = tile_ops.small_batch_workspace(rows, in_dim)
         batch = tile_ops.multi_linear(weights, to_device(x[:rows], cuda), workspace, family="mmvq")
         for row in range(rows):
