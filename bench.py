@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 # WRITE_SIZE counters of a `--traffic-probe` run, each calibrated on a plain
 # copy of known size; the figures and commands are in
 # profiles/gemv_dot_kernel_decode_attention_projections_rows1_hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_691_496}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {1: 16_690_369}
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "int8": 5000.0, "f32": 157.3}
 CU_COUNT = 256
 F16_FLOP_PER_CYCLE_PER_CU = 4096   # 4 SIMDs x one 32x32x16 fp16 matrix instruction per 32 cycles
