@@ -116,9 +116,12 @@ struct UnitData {
 
 // acc[t] += (activation scale * d) * sum_quarter sc * (256*dot(q,hi) + dot(q,lo) - 32*sum(codes))
 // for unit `unit` (= 4*block + 2*half + sixteen inside the row) and every token.
-template <int T>
+// `later` sends the unit to acc_later instead (a lane of the streaming kernel that is already
+// in the wave's next row); the other accumulator takes a product with zero, which leaves it as it is.
+template <int T, bool TWO = false>
 __device__ __forceinline__ void accumulate_unit(const UnitData& data, std::uint8_t* lds, int blocks,
-                                                int unit, bool live, float (&acc)[T]) {
+                                                int unit, bool live, float (&acc)[T],
+                                                bool later = false, float* acc_later = nullptr) {
     const int units = 4 * blocks;
     const int block = unit >> 2;
     const int sixteen = unit & 1;
@@ -164,7 +167,13 @@ __device__ __forceinline__ void accumulate_unit(const UnitData& data, std::uint8
             unit_value = fmaf(scale_q[k], static_cast<float>(bracket), unit_value);
         }
         const float scale = image.scale[block];
-        acc[t] = fmaf(live ? scale * d : 0.0f, unit_value, acc[t]);
+        const float factor = live ? scale * d : 0.0f;
+        if constexpr (TWO) {
+            acc[t] = fmaf(later ? 0.0f : factor, unit_value, acc[t]);
+            acc_later[t] = fmaf(later ? factor : 0.0f, unit_value, acc_later[t]);
+        } else {
+            acc[t] = fmaf(factor, unit_value, acc[t]);
+        }
     }
 }
 
@@ -603,21 +612,23 @@ __global__ __launch_bounds__(W * kWave) void gemv_q6_stream_kernel(
         const int block_in_row =
             min(stream_block - (in_next ? row_end_block : row_first_block), blocks - 1);
         const int unit = 4 * block_in_row + my_unit;
-        float value[T];
-#pragma unroll
-        for (int t = 0; t < T; ++t) value[t] = 0.0f;
-        accumulate_unit<T>(data, lds, blocks, unit, live, value);
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc_current[t] += in_next ? 0.0f : value[t];
-            acc_next[t] += in_next ? value[t] : 0.0f;
-        }
+        accumulate_unit<T, true>(data, lds, blocks, unit, live, acc_current, in_next, acc_next);
 
         // the current row ends inside this pass: reduce and emit it
         if (row_end_block <= (pass + 1) * kPassBlocks && row < row_count) {
+            // A row that does not start on a pass boundary has its units 4 * row_first_block
+            // lanes further on than a row that does.  The butterfly must see every row the same
+            // way, whatever the wave's range of rows (which changes with the launch's shape and
+            // token count): move unit class u % 64 back to lane u % 64 first.
+            const int turned = (4 * row_first_block) & 63;
 #pragma unroll
             for (int t = 0; t < T; ++t) {
-                const float total_value = wave_total(acc_current[t]);
+                float row_sum = acc_current[t];
+                if (turned != 0) {
+                    row_sum = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(
+                        ((lane + turned) & 63) << 2, __builtin_bit_cast(int, row_sum)));
+                }
+                const float total_value = wave_total(row_sum);
                 if constexpr (ARGMAX) {
                     // rows come in increasing order: a strict comparison keeps the lowest index
                     if (total_value > best_value[t]) {

@@ -609,6 +609,32 @@ def test_verifier_matrix_core_rows_equal_the_one_row_kernel(cuda, oracle, encodi
                 assert_bits_equal(whole[row:row + 1].contiguous(), part, f"row {row} of {rows}")
 
 
+@pytest.mark.parametrize("in_dim,out_dim", [(6656, 3000), (6656, 4608), (13312, 2100), (4096, 2500)])
+def test_q6k_rows_carry_the_same_bits_wherever_their_wave_starts(cuda, oracle, in_dim, out_dim):
+    """The Q6_K streaming kernel hands a wave a contiguous range of rows, and how many depends on
+    the launch (output width, tokens per pass, waves per workgroup, the other projections of the
+    call); a row of 26 or 52 blocks then starts inside a 16-block pass.  Its bits must not depend
+    on where: verifier rows at 2, 4 and 16 tokens equal the one-row call, and a projection alone
+    equals the same projection inside a group."""
+    encoding = kquant.Q6_K
+    packed = random_packed(encoding, out_dim, in_dim, 61)
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    other = tile_ops.PackedWeight.from_numpy(encoding, random_packed(encoding, 256, in_dim, 62), 256, in_dim)
+    x = kquant.synthetic_activations(63, 16, in_dim)
+    one = tile_ops.small_batch_workspace(1, in_dim)
+    alone = [tile_ops.mmvq_linear(weight, to_device(x[row:row + 1], cuda), one) for row in range(16)]
+    picked = np.arange(0, out_dim, 37)
+    expected = oracle.linear(encoding, packed.reshape(out_dim, -1)[picked].reshape(-1), picked.size, in_dim, x[:1])
+    assert normalised_error(alone[0].cpu().numpy()[:, picked], expected) <= TOLERANCE
+    grouped = tile_ops.multi_linear([other, weight], to_device(x[:1], cuda), one, family="mmvq")
+    assert_bits_equal(grouped[1], alone[0], "a projection alone = its place in a group")
+    for rows in (2, 4, 16):
+        workspace = tile_ops.small_batch_workspace(rows, in_dim)
+        batch = tile_ops.multi_linear([weight], to_device(x[:rows], cuda), workspace, family="mmvq")[0]
+        for row in range(rows):
+            assert_bits_equal(batch[row:row + 1].contiguous(), alone[row], f"row {row} of {rows}")
+
+
 @pytest.mark.parametrize("prologue", ["gated", "swiglu"])
 def test_verifier_matrix_core_rows_with_prologues_and_mixed_formats(cuda, prologue):
     """Fused prologues go through the quantizer launch; the Q6_K and Q8_0 projections of the same
