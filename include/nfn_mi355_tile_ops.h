@@ -809,7 +809,7 @@ int nfn_native_tile_scale_inplace_float32(
  * Version 2: nfn_mi355_attention_workspace_v1 takes the stream the loan is for as a third
  * argument (a caller built against the two-argument form must not call it); the measurement
  * probes live in a library of their own (nfn_mi355_probes.h); the small-batch workspace of
- * five rows and more also holds the activations in matrix-operand order (the query
+ * four rows and more also holds the activations in matrix-operand order (the query
  * nfn_native_tile_k_quant_mmq_workspace_bytes_v1 returns the larger size). */
 int nfn_mi355_abi_version(void);
 

@@ -1,30 +1,35 @@
-// Verifier rows (2..16 tokens) of Q4_K / Q5_K projections on the int8 matrix cores, every row
-// in the one-row kernel's arithmetic bit for bit.
+// Verifier rows (4..16 tokens) of K-quant projections on the int8 matrix cores, every row in
+// the one-row kernel's arithmetic bit for bit.
 //
 // The contract (neuralfn/csrc/native_train/tile_ops.h:685-688; the reference's kernel:
 // neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:1753-1925): row t of a batched call equals the
-// one-row call on row t.  The one-row kernel (gemv_dot.hip) gives lane L of a wave the units
-// u = L, L + 64, ... of a weight row (a unit: one 64-value pair of sub-blocks), chains
-//     acc = fmaf(scale, fmaf(-dmin, float(wmin), d * fmaf(float(whi), 256, float(wlo))), acc)
-// over them and sums the 64 lanes in a butterfly.  Everything up to whi / wlo / wmin is exact
-// integer arithmetic, and float addition is commutative, so the result is fixed by
+// one-row call on row t.  The one-row kernels (gemv_dot.hip, gemv_q6.hip, gemv_q8.hip) give
+// lane L of a wave the units u = L, L + 64, ... of a weight row (a unit: 64 values), chain one
+// fused multiply-add per unit,
+//   Q4_K, Q5_K  acc = fmaf(scale, fmaf(-dmin, float(wmin), d * fmaf(float(whi), 256, float(wlo))), acc)
+//   Q6_K        acc = fmaf(scale * d, ((sc0 * float(b0) + sc1 * float(b1)) + ...) in fused steps, acc)
+//   Q8_0        acc = fmaf(scale, fmaf(d1, float(b1), d0 * float(b0)), acc)
+// over them and sum the 64 lanes in a butterfly.  Everything up to the integers in these
+// formulas is exact integer arithmetic, and float addition is commutative, so the result is
+// fixed by
 //   * which terms form a chain: the units 4b + p of the blocks b = c, c + 16, c + 32, ...
-//     ("class" c = 0..15, p = 0..3), in that order,
+//     ("class" c = 0..15, p = 0..3; a block: 256 values), in that order,
 //   * the balanced binary tree over the 64 chains in the order (c, p).
-// Here a workgroup of 8 waves owns 32 consecutive weight rows.  v_mfma_i32_32x32x32_i8 takes
-// the 32 values of a sub-block (K), 32 weight rows (operand B, lane l: row l % 32, values
-// 16 (l / 32)..+15; the packed bytes are loaded coalesced and change lanes through a private
-// LDS tile per wave) and the two int8 planes of up to 16 tokens (operand A, fetched in
-// operand order from the image a quantizer launch left in the workspace beside the activation
-// records: lanes that each pick their own 16 bytes out of sixteen records cost the memory
-// pipeline four times the instructions' coalesced rate); a second product against the sub-block minimums, spread over
-// K, gives the sums the minimums multiply.  A lane then holds, for its weight row and up to 8
-// tokens, the integers of a unit, and replays the float tail above.  Wave w takes the classes
-// w and 15 - w (an even share of any row length), keeps the four chains of a class per token
-// in registers, and leaves (c0 + c1) + (c2 + c3) per class, token and row in LDS; after one
-// barrier a thread per (token, row) adds the 16 classes in the tree's order.  A workgroup
-// walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... with the loads of the next tile's
-// first block in flight under the last block of the one before.
+// Here a workgroup of 8 waves owns 32 consecutive weight rows.  A matrix instruction takes
+// the values of a scale group (K: 32 values, 16 for Q6_K), 32 weight rows (operand B, lane l:
+// row l % 32, half l / 32 of the group; the packed bytes are loaded coalesced and change lanes
+// through a private LDS tile per wave) and the two int8 planes of up to 16 tokens (operand A,
+// fetched in operand order from the image a quantizer launch left in the workspace beside the
+// activation records: lanes that each pick their own 16 bytes out of sixteen records cost the
+// memory pipeline four times the instructions' coalesced rate).  For Q4_K / Q5_K a second
+// product against the sub-block minimums, spread over K, gives the sums the minimums
+// multiply; Q6_K's offset of 32 is taken off the codes before the product.  A lane then holds,
+// for its weight row and up to 8 tokens, the integers of a unit, and replays the float tail
+// above.  Wave w takes the classes w and 15 - w (an even share of any row length), keeps the
+// four chains of a class per token in registers, and leaves (c0 + c1) + (c2 + c3) per class,
+// token and row in LDS; after one barrier a thread per (token, row) adds the 16 classes in the
+// tree's order.  A workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... with the
+// loads of the next tile's first block in flight under the last block of the one before.
 // One pass over the weights for up to 16 tokens.
 #include "common.hpp"
 #include "gemv_rows.hpp"
@@ -86,23 +91,59 @@ __global__ __launch_bounds__(256) void quantize_records_kernel(
     }
 }
 
-template <bool Q5>
+// How a block (256 values of one weight row) lies in memory and in a wave's LDS tile.
+//   Q4_K / Q5_K: 144 / 176 bytes, 16-byte aligned; the tile is the same bytes row after row.
+//   Q8_0: eight 34-byte blocks = 272 bytes; rows are as aligned as the tensor is.
+//   Q6_K: 210 bytes, so every other block starts two bytes past a word.  A block is fetched as
+//     fourteen 16-byte pieces from the word at or before its first byte (pieces 0..12 in a
+//     row, piece 13 from byte 196, so that no load reaches past the word that holds the
+//     block's last byte) and written to its 240-byte LDS slot two bytes down when it started
+//     past a word: in LDS every block starts at byte 16 of its slot.
+template <std::uint32_t ENC>
 struct RowsFormat {
-    static constexpr int kBlockBytes = Q5 ? 176 : 144;
-    static constexpr int kChunks = kBlockBytes / 16;          // 16-byte chunks of a block
-    static constexpr int kTileChunks = kRowsTile * kChunks;   // of a block of 32 rows
+    static constexpr bool kQ6 = ENC == kEncQ6K;
+    static constexpr bool kQ8 = ENC == kEncQ8_0;
+    static constexpr int kBlockBytes = ENC == kEncQ4K ? 144 : ENC == kEncQ5K ? 176 : kQ6 ? 210 : 272;
+    static constexpr int kChunks = kQ6 ? 14 : kBlockBytes / 16;  // 16-byte pieces of a block
+    static constexpr int kTileChunks = kRowsTile * kChunks;      // of a block of 32 rows
     static constexpr int kLoads = (kTileChunks + kWave - 1) / kWave;
-    static constexpr int kTileBytes = kRowsTile * kBlockBytes;
+    static constexpr int kSlotBytes = kQ6 ? 240 : kBlockBytes;   // a row's place in the LDS tile
+    static constexpr int kSlotOrigin = kQ6 ? 16 : 0;             // where the block starts in it
+    static constexpr int kTileBytes = kRowsTile * kSlotBytes;
 };
 
-template <bool Q5, int S>
-struct RowsStage {
-    v4u chunk[RowsFormat<Q5>::kLoads];     // packed bytes of 32 rows x one block, coalesced
-    v4i a[8];                             // operand A of the eight sub-blocks
+struct __attribute__((packed, aligned(2))) RowsPiece {
+    std::uint32_t v[4];
+};
+struct __attribute__((packed, aligned(2))) RowsHalfPiece {
+    std::uint32_t v[2];
+};
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+// The packed bytes of 32 rows x one block as a wave loads them, coalesced: one set of
+// registers (they go to the LDS tile as soon as they arrive, and the next block's request
+// reuses them).
+template <std::uint32_t ENC>
+struct RowsPacked {
+    v4u chunk[RowsFormat<ENC>::kLoads];
+    std::uint32_t shifted;  // Q6_K: bit i = piece i of this lane starts two bytes past a word
+};
+
+// Operand A of the eight 32-value groups of a block: two sets, used by the matrix instructions
+// where they arrive.
+struct RowsOperands {
+    v4i a[8];
 };
 
 __device__ __forceinline__ v16i mfma_i8(v4i a, v4i b, v16i c) {
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+}
+
+// K = 16: operands of 8 bytes a lane (lane l: row l % 32, values 8 (l / 32)..+7)
+__device__ __forceinline__ v16i mfma_i8_k16(v2i a, v2i b, v16i c) {
+    return __builtin_amdgcn_mfma_i32_32x32x16_i8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b),
+                                                 c, 0, 0, 0);
 }
 
 __device__ __forceinline__ void rows_lds_fence() {
@@ -117,7 +158,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const std::uint8_t* __restrict__ image, int tokens, int input_dim, std::uint32_t total_tiles,
     ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
-    using F = RowsFormat<kQ5>;
+    using F = RowsFormat<ENC>;
     constexpr int kBlockBytes = F::kBlockBytes;
     constexpr int kQuants = kQ5 ? 48 : 16;
     constexpr int kTokens = 2 * S;
@@ -144,30 +185,49 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         return pick(set, which);
     };
 
-    // What the loads of a tile need: its first row and, per lane, where the chunks it copies
-    // per block lie: chunk n = 64 i + lane of the 32 x kChunks, 9 (11) to a row; the LDS tile
-    // is the same bytes row after row, so chunk n goes to byte 16 n (the lanes past the last
-    // chunk repeat it).
+    // What the loads of a tile need: its first row and, per lane, where the pieces it copies
+    // per block lie: piece n = 64 i + lane of the 32 x kChunks, kChunks to a row (the lanes
+    // past the last piece repeat it), and where in the LDS tile each goes.
     const std::uint8_t* tile_rows;
     std::uint32_t chunk_offset[F::kLoads];
+    std::uint32_t row_parity = 0;  // Q6_K: bit i = the row of piece i starts two bytes past a word
+    // (Q4_K, Q5_K, Q8_0: the LDS tile is the same bytes row after row, piece n at byte 16 n)
+    std::uint32_t lds_offset[F::kQ6 ? F::kLoads : 1];
+    if constexpr (F::kQ6) {
+#pragma unroll
+        for (int i = 0; i < F::kLoads; ++i) {
+            const int chunk = i * kWave + lane;
+            const int row = chunk / F::kChunks;
+            const int col = chunk - row * F::kChunks;
+            lds_offset[i] = row * F::kSlotBytes + F::kSlotOrigin + (col == 13 ? 196 : col * 16);
+        }
+    }
+    const int last_slot = min((F::kLoads - 1) * kWave + lane, F::kTileChunks - 1) * 16;
     auto aim = [&](std::uint32_t tile) {
         const Projection op = projection_of(tile);
         const std::int64_t row0 = static_cast<std::int64_t>(tile - op.first_tile) * kRowsTile;
         const int valid_rows =
             static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
         tile_rows = op.data + row0 * op.row_stride;
+        row_parity = 0;
 #pragma unroll
         for (int i = 0; i < F::kLoads; ++i) {
             const int chunk = min(i * kWave + lane, F::kTileChunks - 1);
             const int row = chunk / F::kChunks;
             const int col = chunk - row * F::kChunks;
-            chunk_offset[i] = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
-                    static_cast<std::uint32_t>(op.row_stride) + col * 16;
+            const int within = F::kQ6 && col == 13 ? 196 : col * 16;
+            const std::uint32_t row_offset = static_cast<std::uint32_t>(min(row, valid_rows - 1)) *
+                    static_cast<std::uint32_t>(op.row_stride);
+            chunk_offset[i] = row_offset + within;
+            if constexpr (F::kQ6) {
+                const std::uint32_t address_low = static_cast<std::uint32_t>(
+                    reinterpret_cast<std::uintptr_t>(tile_rows)) + row_offset;
+                row_parity |= ((address_low >> 1) & 1u) << i;
+            }
         }
     };
-    const int last_slot = min((F::kLoads - 1) * kWave + lane, F::kTileChunks - 1) * 16;
     std::uint8_t* const my_tile = packed_tiles[wave];
-    const std::uint8_t* const my_row = my_tile + j * kBlockBytes;
+    const std::uint8_t* const my_row = my_tile + j * F::kSlotBytes + F::kSlotOrigin;
 
     // this wave's steps of a tile: the blocks of class `wave`, then those of class 15 - wave
     const int class0 = wave;
@@ -183,17 +243,36 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     int fetch_step = 0;
     aim(fetch_tile);
     // the loads of the next step of the walk; past its end the last block again
-    auto fetch = [&](RowsStage<kQ5, S>& stage) {
+    auto fetch = [&](RowsPacked<ENC>& stage, RowsOperands& operands) {
         const int block = min(block_of(min(fetch_step, max(total - 1, 0))), blocks - 1);
         const std::uint8_t* weights = tile_rows + static_cast<std::int64_t>(block) * kBlockBytes;
+        // (a Q6_K block with an odd index lies two bytes further from a word than its row does)
+        const std::uint32_t shifted = F::kQ6 ? row_parity ^ (0u - static_cast<std::uint32_t>(block & 1)) : 0u;
+        if constexpr (F::kQ6) stage.shifted = shifted;
 #pragma unroll
         for (int i = 0; i < F::kLoads; ++i) {
-            stage.chunk[i] = *reinterpret_cast<const v4u*>(weights + chunk_offset[i]);
+            if constexpr (F::kQ6 || F::kQ8) {
+                // (Q8_0 rows are only as aligned as the tensor; Q6_K pieces start on a word)
+                const std::uint32_t back = F::kQ6 ? ((shifted >> i) & 1u) * 2u : 0u;
+                const RowsPiece piece = *reinterpret_cast<const RowsPiece*>(weights + chunk_offset[i] - back);
+                stage.chunk[i] = v4u{piece.v[0], piece.v[1], piece.v[2], piece.v[3]};
+            } else {
+                stage.chunk[i] = *reinterpret_cast<const v4u*>(weights + chunk_offset[i]);
+            }
         }
         const std::uint8_t* fragments = image + static_cast<std::int64_t>(block) * kImageBlock;
 #pragma unroll
         for (int sub = 0; sub < 8; ++sub) {
-            stage.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
+            if constexpr (F::kQ6) {
+                // the sixteen values 16 s..+15 of a 32-value group are what the image keeps for
+                // lanes 32 s..+31: this lane takes bytes 8 h..+7 of row j's sixteen, for s = 0, 1
+                const std::uint8_t* mine = fragments + sub * 1024 + j * 16 + h * 8;
+                const v2i lower = *reinterpret_cast<const v2i*>(mine);
+                const v2i upper = *reinterpret_cast<const v2i*>(mine + 512);
+                operands.a[sub] = v4i{lower[0], lower[1], upper[0], upper[1]};
+            } else {
+                operands.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
+            }
         }
         if (++fetch_step >= total && fetch_tile + gridDim.x < total_tiles) {
             fetch_step = 0;
@@ -212,98 +291,206 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         for (int slot = 0; slot < S; ++slot) acc[p][slot] = 0.0f;
     }
 
-    auto compute = [&](const RowsStage<kQ5, S>& stage, int step) {
-        // the packed bytes change lanes through the wave's LDS tile: a lane needs the header
-        // of row j and its half of the row's codes
+    // the packed bytes change lanes through the wave's LDS tile
+    auto stage_to_lds = [&](const RowsPacked<ENC>& stage) {
+        if constexpr (F::kQ6) {
 #pragma unroll
-        for (int i = 0; i + 1 < F::kLoads; ++i) {
-            *reinterpret_cast<v4u*>(my_tile + lane * 16 + i * (kWave * 16)) = stage.chunk[i];
-        }
-        *reinterpret_cast<v4u*>(my_tile + last_slot) = stage.chunk[F::kLoads - 1];
-        rows_lds_fence();
-        const uint4 head = *reinterpret_cast<const uint4*>(my_row);
-        uint4 high = make_uint4(0, 0, 0, 0);
-        if constexpr (kQ5) high = *reinterpret_cast<const uint4*>(my_row + 16 + h * 16);
-        uint4 quants[4];
+            for (int i = 0; i < F::kLoads; ++i) {
+                const std::uint32_t back = ((stage.shifted >> i) & 1u) * 2u;
+                RowsPiece piece;
+                piece.v[0] = stage.chunk[i][0];
+                piece.v[1] = stage.chunk[i][1];
+                piece.v[2] = stage.chunk[i][2];
+                piece.v[3] = stage.chunk[i][3];
+                *reinterpret_cast<RowsPiece*>(my_tile + lds_offset[i] - back) = piece;
+            }
+        } else {
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            quants[p] = *reinterpret_cast<const uint4*>(my_row + kQuants + p * 32 + h * 16);
+            for (int i = 0; i + 1 < F::kLoads; ++i) {
+                *reinterpret_cast<v4u*>(my_tile + lane * 16 + i * (kWave * 16)) = stage.chunk[i];
+            }
+            *reinterpret_cast<v4u*>(my_tile + last_slot) = stage.chunk[F::kLoads - 1];
         }
+    };
+
+    auto compute = [&](const RowsOperands& stage, int step) {
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         float scale[S];
 #pragma unroll
         for (int slot = 0; slot < S; ++slot) scale[slot] = step_scales[wave][step][S * h + slot];
-        rows_lds_fence();  // the next block's stores stay behind these reads
-        // 6-bit scales and minimums of the eight sub-blocks, four per word
-        const std::uint32_t sc_lo = head.y & 0x3f3f3f3fu;
-        const std::uint32_t mn_lo = head.z & 0x3f3f3f3fu;
-        const std::uint32_t sc_hi = (head.w & 0x0f0f0f0fu) | ((head.y >> 2) & 0x30303030u);
-        const std::uint32_t mn_hi = ((head.w >> 4) & 0x0f0f0f0fu) | ((head.z >> 2) & 0x30303030u);
-        const float d = half_bits_to_float(head.x & 0xffffu);
-        const float dmin = half_bits_to_float(head.x >> 16);
-        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (F::kQ6) {
+            // Q6_K (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:591-616): per half of 128
+            // values 64 bytes of low nibbles (quarters 0 / 2 in bytes 0..31, 1 / 3 in 32..63) and
+            // 32 bytes of 2-bit tops; 16 int8 sub-scales (half, quarter, sixteen) and d.  This
+            // lane decodes values 8 h..+7 of both sixteens of every quarter of row j.
+            const RowsPiece sub_scales = *reinterpret_cast<const RowsPiece*>(my_row + 192);
+            const float d = half_bits_to_float(*reinterpret_cast<const std::uint16_t*>(my_row + 208));
+            float factor[S];
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const std::uint32_t packed[4] = {quants[p].x, quants[p].y, quants[p].z, quants[p].w};
-            v4i low, upper;
+            for (int slot = 0; slot < S; ++slot) factor[slot] = scale[slot] * d;
+            // The codes go into the product as 4 (q - 32), which is their six bits moved to the
+            // top of a byte with the highest one flipped; the sub-scales as sc / 4, so that
+            // every product sc * bracket keeps its value (both factors are exact) and every
+            // rounding of the one-row kernel's chain happens on the same number.
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                std::uint32_t lo = packed[w] & 0x0f0f0f0fu;
-                std::uint32_t up = (packed[w] >> 4) & 0x0f0f0f0fu;
-                if constexpr (kQ5) {
-                    const std::uint32_t bits[4] = {high.x, high.y, high.z, high.w};
-                    const std::uint32_t shifted = bits[w] >> (2 * p);
-                    lo |= (shifted & 0x01010101u) << 4;
-                    up |= (shifted & 0x02020202u) << 3;
+            for (int half = 0; half < 2; ++half) {
+                float quarter_scale[8];
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const std::uint32_t biased = sub_scales.v[2 * half + w] ^ 0x80808080u;
+#pragma unroll
+                    for (int byte = 0; byte < 4; ++byte) {
+                        quarter_scale[4 * w + byte] =
+                            fmaf(static_cast<float>((biased >> (8 * byte)) & 0xffu), 0.25f, -32.0f);
+                    }
                 }
-                low[w] = static_cast<int>(lo);
-                upper[w] = static_cast<int>(up);
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const std::uint8_t* at = my_row + half * 64 + s * 16 + h * 8;
+                    const RowsHalfPiece low_a = *reinterpret_cast<const RowsHalfPiece*>(at);
+                    const RowsHalfPiece low_b = *reinterpret_cast<const RowsHalfPiece*>(at + 32);
+                    const RowsHalfPiece top =
+                        *reinterpret_cast<const RowsHalfPiece*>(my_row + 128 + half * 32 + s * 16 + h * 8);
+                    v2i codes[4];
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        const std::uint32_t a = low_a.v[w], b = low_b.v[w];
+                        const std::uint32_t t = top.v[w] ^ 0xaaaaaaaau;
+                        codes[0][w] = static_cast<int>(((a << 2) & 0x3c3c3c3cu) | ((t << 6) & 0xc0c0c0c0u));
+                        codes[1][w] = static_cast<int>(((b << 2) & 0x3c3c3c3cu) | ((t << 4) & 0xc0c0c0c0u));
+                        codes[2][w] = static_cast<int>(((a >> 2) & 0x3c3c3c3cu) | ((t << 2) & 0xc0c0c0c0u));
+                        codes[3][w] = static_cast<int>(((b >> 2) & 0x3c3c3c3cu) | (t & 0xc0c0c0c0u));
+                    }
+                    // quarter after quarter, so that one product's sixteen integers are live
+                    float unit_value[S];
+#pragma unroll
+                    for (int slot = 0; slot < S; ++slot) unit_value[slot] = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const v4i both = stage.a[4 * half + k];
+                        const v2i fragment = s == 0 ? v2i{both[0], both[1]} : v2i{both[2], both[3]};
+                        const v16i dots = mfma_i8_k16(fragment, codes[k], zero);
+#pragma unroll
+                        for (int slot = 0; slot < S; ++slot) {
+                            // |4 (256 hi + lo)| <= 4 * 16 * 32 * 32512 < 2^27: exact in int32
+                            const int bracket = (dots[2 * slot] << 8) + dots[2 * slot + 1];
+                            unit_value[slot] =
+                                fmaf(quarter_scale[2 * k + s], static_cast<float>(bracket), unit_value[slot]);
+                        }
+                    }
+#pragma unroll
+                    for (int slot = 0; slot < S; ++slot) {
+                        acc[2 * half + s][slot] = fmaf(factor[slot], unit_value[slot], acc[2 * half + s][slot]);
+                    }
+                }
             }
-            const std::uint32_t sc_word = p < 2 ? sc_lo : sc_hi;
-            const std::uint32_t mn_word = p < 2 ? mn_lo : mn_hi;
-            const int scale_a = static_cast<int>((sc_word >> (16 * (p & 1))) & 0xffu);
-            const int scale_b = static_cast<int>((sc_word >> (16 * (p & 1) + 8)) & 0xffu);
-            const int min_a = static_cast<int>((mn_word >> (16 * (p & 1))) & 0xffu);
-            const int min_b = static_cast<int>((mn_word >> (16 * (p & 1) + 8)) & 0xffu);
-            const int spread_a = static_cast<int>(__umul24(min_a, 0x010101u)) | (min_a << 24);
-            const int spread_b = static_cast<int>(__umul24(min_b, 0x010101u)) | (min_b << 24);
-            const v4i mins_a = {spread_a, spread_a, spread_a, spread_a};
-            const v4i mins_b = {spread_b, spread_b, spread_b, spread_b};
-            // the sub-block scales times 256, opaque to the optimizer: it would otherwise factor
-            // scale * (256 * hi + lo) out and pay a full 32-bit multiplication for it
-            int scale_a256, scale_b256;
-            asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_a256) : "v"(scale_a));
-            asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_b256) : "v"(scale_b));
-            const v16i dots_a = mfma_i8(stage.a[2 * p], low, zero);
-            const v16i dots_b = mfma_i8(stage.a[2 * p + 1], upper, zero);
-            // min_a * sum(codes of a) + min_b * sum(codes of b), per plane
-            const v16i sums = mfma_i8(stage.a[2 * p + 1], mins_b, mfma_i8(stage.a[2 * p], mins_a, zero));
+            rows_lds_fence();  // the next block's stores stay behind these reads
+        } else if constexpr (F::kQ8) {
+            // Q8_0: eight blocks of an fp16 scale and 32 int8 codes; the codes are operand B as
+            // they lie, this lane's sixteen of each block from byte 34 b + 2 + 16 h
 #pragma unroll
-            for (int slot = 0; slot < S; ++slot) {
-                float codes;
-                if constexpr (kQ5) {
-                    const int weighted_hi =
-                        __mul24(scale_a, dots_a[2 * slot]) + __mul24(scale_b, dots_b[2 * slot]);
-                    const int weighted_lo =
-                        __mul24(scale_a, dots_a[2 * slot + 1]) + __mul24(scale_b, dots_b[2 * slot + 1]);
-                    codes = fmaf(static_cast<float>(weighted_hi), 256.0f, static_cast<float>(weighted_lo));
-                } else {
-                    // 4-bit codes: 256 * weighted_hi + weighted_lo stays below 2^31
-                    // (2 * 63 * 32 * 15 * (127 * 256 + 128)), and one conversion rounds the
-                    // exact integer as the fused multiply-add of the two exact floats does
-                    // (a chain of multiply-adds: the empty statements keep the optimizer from
-                    // turning it into a tree with one more instruction)
-                    int weighted = __mul24(scale_a256, dots_a[2 * slot]);
-                    asm("" : "+v"(weighted));
-                    weighted += __mul24(scale_b256, dots_b[2 * slot]);
-                    asm("" : "+v"(weighted));
-                    weighted += __mul24(scale_a, dots_a[2 * slot + 1]);
-                    asm("" : "+v"(weighted));
-                    weighted += __mul24(scale_b, dots_b[2 * slot + 1]);
-                    codes = static_cast<float>(weighted);
+            for (int p = 0; p < 4; ++p) {
+                const std::uint8_t* pair = my_row + 68 * p;
+                const RowsPiece c0 = *reinterpret_cast<const RowsPiece*>(pair + 2 + 16 * h);
+                const RowsPiece c1 = *reinterpret_cast<const RowsPiece*>(pair + 36 + 16 * h);
+                const float d0 = half_bits_to_float(*reinterpret_cast<const std::uint16_t*>(pair));
+                const float d1 = half_bits_to_float(*reinterpret_cast<const std::uint16_t*>(pair + 34));
+                const v16i dots0 = mfma_i8(stage.a[2 * p], v4i{static_cast<int>(c0.v[0]), static_cast<int>(c0.v[1]),
+                                                                static_cast<int>(c0.v[2]), static_cast<int>(c0.v[3])}, zero);
+                const v16i dots1 = mfma_i8(stage.a[2 * p + 1], v4i{static_cast<int>(c1.v[0]), static_cast<int>(c1.v[1]),
+                                                                    static_cast<int>(c1.v[2]), static_cast<int>(c1.v[3])}, zero);
+#pragma unroll
+                for (int slot = 0; slot < S; ++slot) {
+                    // |256 hi + lo| <= 32 * 127 * 32512 < 2^28: exact in int32
+                    const int bracket0 = (dots0[2 * slot] << 8) + dots0[2 * slot + 1];
+                    const int bracket1 = (dots1[2 * slot] << 8) + dots1[2 * slot + 1];
+                    const float value = fmaf(d1, static_cast<float>(bracket1), d0 * static_cast<float>(bracket0));
+                    acc[p][slot] = fmaf(scale[slot], value, acc[p][slot]);
                 }
-                const int weighted_min = sums[2 * slot] * 256 + sums[2 * slot + 1];
-                const float value = fmaf(-dmin, static_cast<float>(weighted_min), d * codes);
-                acc[p][slot] = fmaf(scale[slot], value, acc[p][slot]);
+            }
+            rows_lds_fence();  // the next block's stores stay behind these reads
+        } else {
+            // Q4_K / Q5_K: a lane needs the header of row j and its half of the row's codes
+            const uint4 head = *reinterpret_cast<const uint4*>(my_row);
+            uint4 high = make_uint4(0, 0, 0, 0);
+            if constexpr (kQ5) high = *reinterpret_cast<const uint4*>(my_row + 16 + h * 16);
+            uint4 quants[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                quants[p] = *reinterpret_cast<const uint4*>(my_row + kQuants + p * 32 + h * 16);
+            }
+            rows_lds_fence();  // the next block's stores stay behind these reads
+            // 6-bit scales and minimums of the eight sub-blocks, four per word
+            const std::uint32_t sc_lo = head.y & 0x3f3f3f3fu;
+            const std::uint32_t mn_lo = head.z & 0x3f3f3f3fu;
+            const std::uint32_t sc_hi = (head.w & 0x0f0f0f0fu) | ((head.y >> 2) & 0x30303030u);
+            const std::uint32_t mn_hi = ((head.w >> 4) & 0x0f0f0f0fu) | ((head.z >> 2) & 0x30303030u);
+            const float d = half_bits_to_float(head.x & 0xffffu);
+            const float dmin = half_bits_to_float(head.x >> 16);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const std::uint32_t packed[4] = {quants[p].x, quants[p].y, quants[p].z, quants[p].w};
+                v4i low, upper;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    std::uint32_t lo = packed[w] & 0x0f0f0f0fu;
+                    std::uint32_t up = (packed[w] >> 4) & 0x0f0f0f0fu;
+                    if constexpr (kQ5) {
+                        const std::uint32_t bits[4] = {high.x, high.y, high.z, high.w};
+                        const std::uint32_t shifted = bits[w] >> (2 * p);
+                        lo |= (shifted & 0x01010101u) << 4;
+                        up |= (shifted & 0x02020202u) << 3;
+                    }
+                    low[w] = static_cast<int>(lo);
+                    upper[w] = static_cast<int>(up);
+                }
+                const std::uint32_t sc_word = p < 2 ? sc_lo : sc_hi;
+                const std::uint32_t mn_word = p < 2 ? mn_lo : mn_hi;
+                const int scale_a = static_cast<int>((sc_word >> (16 * (p & 1))) & 0xffu);
+                const int scale_b = static_cast<int>((sc_word >> (16 * (p & 1) + 8)) & 0xffu);
+                const int min_a = static_cast<int>((mn_word >> (16 * (p & 1))) & 0xffu);
+                const int min_b = static_cast<int>((mn_word >> (16 * (p & 1) + 8)) & 0xffu);
+                const int spread_a = static_cast<int>(__umul24(min_a, 0x010101u)) | (min_a << 24);
+                const int spread_b = static_cast<int>(__umul24(min_b, 0x010101u)) | (min_b << 24);
+                const v4i mins_a = {spread_a, spread_a, spread_a, spread_a};
+                const v4i mins_b = {spread_b, spread_b, spread_b, spread_b};
+                // the sub-block scales times 256, opaque to the optimizer: it would otherwise factor
+                // scale * (256 * hi + lo) out and pay a full 32-bit multiplication for it
+                int scale_a256, scale_b256;
+                asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_a256) : "v"(scale_a));
+                asm("v_lshlrev_b32 %0, 8, %1" : "=v"(scale_b256) : "v"(scale_b));
+                const v16i dots_a = mfma_i8(stage.a[2 * p], low, zero);
+                const v16i dots_b = mfma_i8(stage.a[2 * p + 1], upper, zero);
+                // min_a * sum(codes of a) + min_b * sum(codes of b), per plane
+                const v16i sums = mfma_i8(stage.a[2 * p + 1], mins_b, mfma_i8(stage.a[2 * p], mins_a, zero));
+#pragma unroll
+                for (int slot = 0; slot < S; ++slot) {
+                    float codes;
+                    if constexpr (kQ5) {
+                        const int weighted_hi =
+                            __mul24(scale_a, dots_a[2 * slot]) + __mul24(scale_b, dots_b[2 * slot]);
+                        const int weighted_lo =
+                            __mul24(scale_a, dots_a[2 * slot + 1]) + __mul24(scale_b, dots_b[2 * slot + 1]);
+                        codes = fmaf(static_cast<float>(weighted_hi), 256.0f, static_cast<float>(weighted_lo));
+                    } else {
+                        // 4-bit codes: 256 * weighted_hi + weighted_lo stays below 2^31
+                        // (2 * 63 * 32 * 15 * (127 * 256 + 128)), and one conversion rounds the
+                        // exact integer as the fused multiply-add of the two exact floats does
+                        // (a chain of multiply-adds: the empty statements keep the optimizer from
+                        // turning it into a tree with one more instruction)
+                        int weighted = __mul24(scale_a256, dots_a[2 * slot]);
+                        asm("" : "+v"(weighted));
+                        weighted += __mul24(scale_b256, dots_b[2 * slot]);
+                        asm("" : "+v"(weighted));
+                        weighted += __mul24(scale_a, dots_a[2 * slot + 1]);
+                        asm("" : "+v"(weighted));
+                        weighted += __mul24(scale_b, dots_b[2 * slot + 1]);
+                        codes = static_cast<float>(weighted);
+                    }
+                    const int weighted_min = sums[2 * slot] * 256 + sums[2 * slot + 1];
+                    const float value = fmaf(-dmin, static_cast<float>(weighted_min), d * codes);
+                    acc[p][slot] = fmaf(scale[slot], value, acc[p][slot]);
+                }
             }
         }
     };
@@ -353,14 +540,15 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
         }
         return;
     }
-    // Two named register stages (an array of them indexed in the loop ends up in scratch
-    // memory).  The second is requested only when the first has arrived: more requests at the
-    // start of a launch make it slower on this chip, not faster (16 rows of the attention
-    // projections: 14.3 us this way, 15.5 with both stages requested at once).  Past the end of
-    // the walk a request repeats the last block, so that the number of loads in flight is the
-    // same on every path.
-    RowsStage<kQ5, S> even, odd;
-    fetch(even);
+    // One set of registers for the packed bytes, two named ones for the operands (an array of
+    // them indexed in the loop ends up in scratch memory).  A block's loads are requested when
+    // the block before has gone to LDS, so one block's arithmetic covers them; the second is
+    // requested only when the first has arrived: more requests at the start of a launch make
+    // it slower on this chip, not faster.  Past the end of the walk a request repeats the last
+    // block, so that the number of loads in flight is the same on every path.
+    RowsPacked<ENC> packed;
+    RowsOperands even, odd;
+    fetch(packed, even);
     // the activation scales of this wave's blocks, 16 tokens each: once into LDS (requested
     // behind the first block's loads, so that nothing waits for them alone)
     for (int index = lane; index < total * 16; index += kWave) {
@@ -383,11 +571,15 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     };
     const int steps = my_tiles * total;
     for (int step = 0; step < steps; step += 2) {
-        fetch(odd);
+        stage_to_lds(packed);
+        rows_lds_fence();
+        fetch(packed, odd);
         compute(even, work_step);
         finish_step();
         if (step + 1 < steps) {
-            fetch(even);
+            stage_to_lds(packed);
+            rows_lds_fence();
+            fetch(packed, even);
             compute(odd, work_step);
             finish_step();
         }
@@ -420,8 +612,8 @@ void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, h
 }  // namespace
 
 bool gemv_rows_supports(std::uint32_t encoding, std::int64_t input_dim) {
-    return (encoding == kEncQ4K || encoding == kEncQ5K) && input_dim % 256 == 0 &&
-        input_dim <= kMaxRowsBlocks * 256;
+    return (encoding == kEncQ4K || encoding == kEncQ5K || encoding == kEncQ6K || encoding == kEncQ8_0) &&
+        input_dim % 256 == 0 && input_dim <= kMaxRowsBlocks * 256;
 }
 
 std::int64_t gemv_rows_image_bytes(std::int64_t input_dim) {
@@ -452,7 +644,7 @@ void launch_quantize_records(const float* first, const float* second, int prolog
 
 void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
                       hipStream_t stream) {
-    const std::uint32_t encodings[2] = {kEncQ4K, kEncQ5K};
+    const std::uint32_t encodings[4] = {kEncQ4K, kEncQ5K, kEncQ6K, kEncQ8_0};
     for (const std::uint32_t encoding : encodings) {
         ProjectionSet group{};
         group.input_dim = set.input_dim;
@@ -460,10 +652,12 @@ void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::
             if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
         }
         if (group.count == 0) continue;
-        if (encoding == kEncQ4K) {
-            launch_encoding<kEncQ4K>(group, image, static_cast<int>(rows), stream);
-        } else {
-            launch_encoding<kEncQ5K>(group, image, static_cast<int>(rows), stream);
+        const int tokens = static_cast<int>(rows);
+        switch (encoding) {
+            case kEncQ4K: launch_encoding<kEncQ4K>(group, image, tokens, stream); break;
+            case kEncQ5K: launch_encoding<kEncQ5K>(group, image, tokens, stream); break;
+            case kEncQ6K: launch_encoding<kEncQ6K>(group, image, tokens, stream); break;
+            default: launch_encoding<kEncQ8_0>(group, image, tokens, stream); break;
         }
     }
 }

@@ -586,10 +586,11 @@ def test_decode_dot_kernel_row_lengths(cuda, oracle, encoding, in_dim):
 
 
 @pytest.mark.parametrize("in_dim", [256, 2304, 4096, 6656, 8448, 16384])
-@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K])
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0])
 def test_verifier_matrix_core_rows_equal_the_one_row_kernel(cuda, oracle, encoding, in_dim):
-    """From four rows on the verifier family's Q4_K / Q5_K projections run on the int8 matrix
-    cores, one pass over the weights: every row must still carry the one-row kernel's bits.
+    """From four rows on the verifier family's projections run on the int8 matrix cores, one
+    pass over the weights: every row must still carry the one-row kernel's bits (for Q6_K both
+    of its one-row kernels: rows of fewer than 16 blocks and the streaming one).
     Row lengths: one block (15 empty classes), 9 blocks, exactly one 16-block slice, 26 blocks
     (classes of one and two blocks), 33 and 64 blocks; output widths off the 32-row tile."""
     out_dims = (40, 8, 70)
