@@ -926,6 +926,28 @@ def mixed_profile_extra(device, stream, steps: int, warmup: int) -> dict:
                               "frac_hbm": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
                               "tokens/s": round(1e3 / ms, 1)}
 
+    # a verifier block: 16 rows through the same calls, both small-batch families
+    # (mmvq: every row carries the one-row call's bits)
+    x16 = {dim: torch.from_numpy(values[:16].copy()).to(device) for dim, values in inputs.items()}
+    outs16 = [{name: torch.empty((16, w.output_dim), dtype=torch.float32, device=device)
+               for name, w in layer.items()} for layer in layers]
+    workspace16 = tile_ops.small_batch_workspace(16, FFN_DIM)
+    for family, key in (("mmq", "verifier_rows16"), ("mmvq", "verifier_rows16_exact_verifier_family")):
+        def verify(family=family):
+            for layer, out in zip(layers, outs16):
+                tile_ops.multi_linear([layer["q"], layer["k"], layer["v"]], x16[MODEL_DIM], workspace16,
+                                      outputs=[out["q"], out["k"], out["v"]], family=family)
+                tile_ops.multi_linear([layer["o"]], x16[ATTN_DIM], workspace16, outputs=[out["o"]],
+                                      family=family)
+                tile_ops.multi_linear([layer["gate"], layer["up"]], x16[MODEL_DIM], workspace16,
+                                      outputs=[out["gate"], out["up"]], family=family)
+                tile_ops.multi_linear([layer["down"]], x16[FFN_DIM], workspace16, outputs=[out["down"]],
+                                      family=family)
+        ms = time_graph(verify, stream, steps, warmup)
+        result[key] = {"ms": round(ms, 4), "GB/s": round(weight_bytes / ms / 1e6, 1),
+                       "frac_hbm": round(weight_bytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                       "tokens/s": round(16e3 / ms, 1)}
+
     # prefill: 1024 rows through the dequant-GEMM
     rows = 1024
     xs = {dim: torch.from_numpy(values).to(device) for dim, values in inputs.items()}

@@ -88,6 +88,57 @@ def test_small_batch_random_case(cuda, oracle, seed):
         assert np.array_equal(bits(direct), bits(outputs[0])), label
 
 
+def random_bytes(rng, encoding, out_dim, in_dim):
+    """Packed rows of random bytes with the fp16 scales kept finite and small."""
+    elements, nbytes = kquant.BLOCKS[encoding]
+    blocks = rng.integers(0, 256, (out_dim * in_dim // elements, nbytes), dtype=np.uint8)
+    offsets = {kquant.Q4_K: (0, 2), kquant.Q5_K: (0, 2), kquant.Q6_K: (208,), kquant.Q8_0: (0,)}
+    for offset in offsets[encoding]:
+        blocks[:, offset + 1] = (blocks[:, offset + 1] & 0x83) | 0x24
+    return blocks.reshape(-1)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_small_batch_model_sized_case(cuda, oracle, seed):
+    """The sweep above keeps its outputs narrow; a wave's or a workgroup's share of the rows, and
+    with it where a row starts inside a kernel's pass, only changes with thousands of rows.
+    Model-sized projections, random formats, row counts and grouping: against the oracle on a
+    sample of the rows, verifier rows against the one-row call on every row, the one-row call
+    of the group against the single-projection entry point, and the prequantized call."""
+    rng = np.random.default_rng(5000 + seed)
+    in_dim = int(rng.choice([4096, 6656, 8192, 13312, 16384]))
+    rows = int(rng.integers(1, 17))
+    count = int(rng.integers(1, 4))
+    formats = [int(rng.choice(FORMATS)) for _ in range(count)]
+    out_dims = [int(rng.choice([256, 2100, 3000, 4608, 6656, 9000])) for _ in range(count)]
+    family = "mmvq" if seed % 4 else "mmq"
+    packed = [random_bytes(rng, f, n, in_dim) for f, n in zip(formats, out_dims)]
+    weights = [tile_ops.PackedWeight.from_numpy(f, p, n, in_dim) for f, p, n in zip(formats, packed, out_dims)]
+    x = rng.standard_normal((rows, in_dim)).astype(np.float32)
+    device_x = to_device(x, cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    outputs = tile_ops.multi_linear(weights, device_x, workspace, family=family)
+    label = f"K {in_dim} rows {rows} {family} {list(zip(formats, out_dims))}"
+    for f, p, n, y in zip(formats, packed, out_dims, outputs):
+        picked = np.unique(np.concatenate([np.arange(0, n, 97), [n - 1]]))
+        sample = p.reshape(n, -1)[picked].reshape(-1)
+        expected = oracle.linear(f, sample, picked.size, in_dim, x)
+        assert normalised_error(y.cpu().numpy()[:, picked], expected) <= TOLERANCE, label
+    one = tile_ops.small_batch_workspace(1, in_dim)
+    if family == "mmvq":
+        for row in range(rows):
+            single = tile_ops.multi_linear(weights, device_x[row:row + 1], one, family="mmvq")
+            for a, b in zip(outputs, single):
+                assert np.array_equal(bits(a)[row], bits(b)[0]), f"{label} row {row}"
+        reused = tile_ops.multi_linear_prequantized(weights, rows, workspace)
+        for a, b in zip(outputs, reused):
+            assert np.array_equal(bits(a), bits(b)), f"{label} prequantized"
+    first_row = tile_ops.multi_linear(weights, device_x[:1], one, family=family)
+    for weight, grouped in zip(weights, first_row):
+        direct = tile_ops.mmvq_linear(weight, device_x[:1], one)
+        assert np.array_equal(bits(direct), bits(grouped)), f"{label} single projection"
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_gemm_random_case(cuda, oracle, seed):
     rng = np.random.default_rng(2000 + seed)
