@@ -825,6 +825,30 @@ def test_q6_k_long_rows_tensor_two_bytes_off_a_word(cuda, oracle):
     assert_bits_equal(a, b, "aligned and shifted tensor")
 
 
+@pytest.mark.parametrize("encoding,in_dim", [(kquant.Q6_K, 4352), (kquant.Q6_K, 6656), (kquant.Q6_K, 768),
+                                             (kquant.Q8_0, 4352), (kquant.Q8_0, 1280)])
+def test_verifier_matrix_core_rows_tensor_two_bytes_off_a_word(cuda, encoding, in_dim):
+    """The matrix-core rows kernel fetches Q6_K blocks from the word at or before their first
+    byte (rows of an odd number of blocks alternate between the two cases, and so does a tensor
+    that starts two bytes past a word) and Q8_0 rows as they lie: a shifted tensor gives the
+    bits of the aligned one, which the other tests tie to the one-row call."""
+    out_dim = 75
+    packed = random_packed(encoding, out_dim, in_dim, 55)
+    aligned = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    holder = torch_().empty(packed.size + 2, dtype=torch_().uint8, device=cuda)
+    holder[2:].copy_(torch_().from_numpy(packed.reshape(-1)))
+    shifted = tile_ops.PackedWeight(encoding, out_dim, in_dim, holder[2:])
+    assert shifted.data.data_ptr() % 4 == 2
+    for rows in (4, 16):
+        x = to_device(kquant.synthetic_activations(56, rows, in_dim), cuda)
+        workspace = tile_ops.small_batch_workspace(rows, in_dim)
+        a = tile_ops.multi_linear([aligned], x, workspace, family="mmvq")[0]
+        b = tile_ops.multi_linear([shifted], x, workspace, family="mmvq")[0]
+        assert_bits_equal(a, b, f"aligned and shifted tensor, {rows} rows")
+        single = tile_ops.mmvq_linear(shifted, x[rows - 1:rows], workspace)
+        assert_bits_equal(single, a[rows - 1:rows].contiguous(), "the one-row call on the shifted tensor")
+
+
 @pytest.mark.parametrize("rows", [1, 3, 8, 16])
 def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
     out_dim, in_dim = 5003, 6656
