@@ -991,6 +991,81 @@ def test_decode_layer_with_the_fused_calls_gives_the_same_bits(cuda, oracle):
     assert bool(torch_().isfinite(results[1][0]).all())
 
 
+def test_model_sized_layer_fused_calls_and_verifier_families(cuda, oracle):
+    """The fused forms and the two small-batch families on a layer of the benchmark's geometry
+    (6,656 wide, 32 query heads over 2 key/value heads of 128, FFN 16,384, a 2,048-key ring;
+    random packed bytes): launch grids, tiles per workgroup and rows per wave are those of the
+    model, not of the small layers above.  One token: the fused gate/up call and the dual norm
+    inside the Q/K/V/gate launch against the separate calls, bit for bit.  A block of 16: the
+    `mmq` family with and without the norm handoff and the gate/up call, bit for bit; the exact
+    verifier family against the token-at-a-time chain (projections bit-equal, attention to
+    its summation order)."""
+    from neuralfn_amd import decode_layer as dl
+    rng = np.random.default_rng(29)
+    g = dl.LayerGeometry(model_dim=6656, query_heads=32, kv_heads=2, head_dim=128, ffn_dim=16384,
+                         sliding_window=2048)
+    shapes = dict(q=(g.attention_dim, g.model_dim), k=(g.kv_dim, g.model_dim),
+                  v=(g.kv_dim, g.model_dim), attention_gate=(g.attention_dim, g.model_dim),
+                  output=(g.model_dim, g.attention_dim), mlp_gate=(g.ffn_dim, g.model_dim),
+                  mlp_up=(g.ffn_dim, g.model_dim), mlp_down=(g.model_dim, g.ffn_dim))
+    device = {}
+    for index, (name, (out_dim, in_dim)) in enumerate(shapes.items()):
+        device[name] = tile_ops.PackedWeight.from_numpy(
+            kquant.Q4_K, random_packed(kquant.Q4_K, out_dim, in_dim, 300 + index), out_dim, in_dim)
+    for name, width in dict(input_norm=g.model_dim, q_norm=g.head_dim, k_norm=g.head_dim,
+                            post_attention_norm=g.model_dim, pre_feedforward_norm=g.model_dim,
+                            post_feedforward_norm=g.model_dim).items():
+        row = (1.0 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+        device[name] = tile_ops.PackedWeight.from_numpy(kquant.F32, row.view(np.uint8).copy(), 1, width)
+    weights = dl.LayerWeights(**device)
+    keys = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+    values = oracle.to_bf16(rng.standard_normal((g.sliding_window, g.kv_dim)).astype(np.float32))
+    attention_workspace = engine_ops.gqa_decode_workspace(g.query_heads, g.head_dim)
+
+    def cache():
+        made = dl.LayerCache(g, cuda)
+        made.keys.copy_(bf16_tensor(keys, cuda))
+        made.values.copy_(bf16_tensor(values, cuda))
+        return made
+
+    rows, position = 16, 5000
+    embeddings = to_device(rng.standard_normal((rows, g.model_dim)).astype(np.float32), cuda)
+    one = tile_ops.small_batch_workspace(1, g.ffn_dim)
+    serial_cache, serial = cache(), []
+    for row in range(rows):
+        results = []
+        for fused in ((False, True) if row == 0 else (False,)):
+            used = cache() if row == 0 else serial_cache
+            results.append(dl.decode_layer(g, weights, used, embeddings[row:row + 1],
+                                           torch_().zeros_like(embeddings[row:row + 1]), None,
+                                           position + row, one, True, attention_workspace,
+                                           fused_gate_up=fused, fused_input_norm=fused))
+            if row == 0:
+                results[-1] += (used.keys.clone(), used.values.clone())
+        if row == 0:
+            for separate, together in zip(results[0], results[1]):
+                assert torch_().equal(separate, together), "one token: fused calls"
+            serial_cache.keys.copy_(results[0][2])
+            serial_cache.values.copy_(results[0][3])
+        serial.append(results[0][0].cpu().numpy()[0])
+    serial = np.stack(serial)
+
+    block = tile_ops.small_batch_workspace(rows, g.ffn_dim)
+    zero = torch_().zeros_like(embeddings)
+    plain = dl.verify_layer(g, weights, cache(), embeddings, zero, None, position, block, True,
+                            attention_workspace)
+    fused = dl.verify_layer(g, weights, cache(), embeddings, zero, None, position, block, True,
+                            attention_workspace, handoff=True, fused_gate_up=True)
+    for a, b in zip(plain, fused):
+        assert torch_().equal(a, b), "block of 16: handoff and gate/up call"
+    exact = dl.verify_layer(g, weights, cache(), embeddings, zero, None, position, block, True,
+                            attention_workspace, family="mmvq")
+    scale = float(np.max(np.abs(serial)))
+    assert scale > 0 and np.isfinite(scale)
+    assert float(np.max(np.abs(exact[0].cpu().numpy() - serial))) <= 1e-4 * scale
+    assert float(np.max(np.abs(plain[0].cpu().numpy() - serial))) <= 2e-2 * scale
+
+
 @pytest.mark.parametrize("split", [False, True])
 def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, oracle, split):
     """decode_layer.verify_layer runs a block of tokens through a layer in the batch forms of the
