@@ -767,11 +767,14 @@ def decode_layer_extra(device, stream, steps: int, warmup: int) -> dict:
             # (and the one after: gate and up in the call that stores swiglu(gate, up),
             # nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1)
             # (and last the exact verifier's family, every row in the one-row arithmetic bit for
-            # bit: what the engine's speculative decode calls with exact_verifier_rows)
+            # bit: what the engine's speculative decode calls with exact_verifier_rows; then with
+            # the norms handing the rows' records over,
+            # nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1)
             block_forms = [(name, workspace, False, False, "mmq") for name, workspace, _ in forms]
             block_forms.append((forms[-1][0] + "_norm_handoff", forms[-1][1], True, False, "mmq"))
             block_forms.append((forms[-1][0] + "_norm_handoff_gate_up_swiglu", forms[-1][1], True, True, "mmq"))
             block_forms.append((forms[-1][0] + "_exact_verifier_family", forms[-1][1], False, False, "mmvq"))
+            block_forms.append((forms[-1][0] + "_exact_verifier_family_norm_handoff", forms[-1][1], True, False, "mmvq"))
             for name, attention_workspace, handoff, fused_gate_up, family in block_forms:
                 def verify():
                     pending, residual, pending_norm = block, block_zeros, None

@@ -399,6 +399,34 @@ int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
     void* mmq_workspace,
     int64_t mmq_workspace_nbytes,
     void* cuda_stream);
+
+/* The handoff for a block of 4..16 rows in the exact verifier's family.  No counterpart in
+ * the reference: its pair (tile_ops.h:874-894 producer, :698-709 consumer) takes one row,
+ * and the engine's verifier therefore runs the norm and then
+ * nfn_native_tile_k_quant_mmvq_multi_linear_float32_v1, whose first launch here quantizes
+ * the rows.  This producer leaves the activation records of all rows and their
+ * matrix-operand copy in mmvq_workspace, as that launch would, and the reference's own
+ * consumer nfn_native_tile_k_quant_mmvq_multi_linear_prequantized_float32_v1 (same rows, same
+ * workspace) multiplies from them: the bits of the mmvq call on normalized_output, one
+ * launch less per projection group.  width: a multiple of 256, at most 8192; the workspace
+ * at least nfn_native_tile_k_quant_mmq_workspace_bytes_v1(rows, width) bytes. */
+int nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1(
+    const float* input,
+    const NfnNativeTilePackedWeightDescriptorV1* first_weight,
+    const float* residual_input,
+    float* hidden_output,
+    const NfnNativeTilePackedWeightDescriptorV1* second_weight,
+    float* normalized_output,
+    float* residual_output,
+    int64_t rows,
+    int64_t width,
+    float first_eps,
+    bool first_centered,
+    float second_eps,
+    bool second_centered,
+    void* mmvq_workspace,
+    int64_t mmvq_workspace_nbytes,
+    void* cuda_stream);
 /* One row: the two normalisations and the projections of their result in one
  * launch.  No counterpart in the reference, whose engine calls
  * nfn_native_tile_glimmer_dual_rms_add_capture_float32_v1 and then the grouped

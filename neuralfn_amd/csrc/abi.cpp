@@ -733,6 +733,34 @@ int nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
     return launch_status();
 }
 
+int nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1(
+    const float* input, const Descriptor* first_weight, const float* residual_input,
+    float* hidden_output, const Descriptor* second_weight, float* normalized_output,
+    float* residual_output, std::int64_t rows, std::int64_t width, float first_eps,
+    bool first_centered, float second_eps, bool second_centered, void* mmvq_workspace,
+    std::int64_t mmvq_workspace_nbytes, void* cuda_stream) {
+    Descriptor first{}, second{};
+    // Row counts that the exact verifier's entry points run on the matrix-core kernel, rows
+    // that the register-resident norm kernel takes.
+    const bool rows_fit = rows >= kFirstVerifierMatrixRows && rows <= kMaxSmallRows;
+    const std::int64_t required = rows_fit ? small_batch_workspace_bytes(rows, width) : 0;
+    if (mmvq_workspace == nullptr || !rows_fit || width % 256 != 0 || width > 8192 ||
+        required == 0 || mmvq_workspace_nbytes < required ||
+        !dual_rms_arguments_valid(input, first_weight, residual_input, hidden_output,
+                                  second_weight, normalized_output, residual_output, rows, width,
+                                  first_eps, second_eps, &first, &second)) {
+        return kInvalid;
+    }
+    std::uint8_t* records = static_cast<std::uint8_t*>(mmvq_workspace);
+    launch_dual_rms_add_capture(input, first_weight != nullptr ? &first : nullptr, first_centered,
+                                residual_input, hidden_output,
+                                second_weight != nullptr ? &second : nullptr, second_centered,
+                                normalized_output, residual_output, rows, width, first_eps,
+                                second_eps, records, nullptr, as_stream(cuda_stream),
+                                records + record_bytes(rows, width));
+    return launch_status();
+}
+
 namespace {
 // Widest input the fp16 form of the lm_head takes: the workspace query does not know the
 // input width and sizes that form's fp16 copy of the rows for this one.

@@ -49,16 +49,8 @@ constexpr int kRowsThreads = kRowsWaves * kWave;
 constexpr int kClasses = 16;
 constexpr int kMaxRowsBlocks = 256;  // input_dim up to 65,536: the blocks whose scales a workgroup keeps
 
-// Operand image of the activations, written next to the records by the quantizer launch: per
-// block 8 KB of operand-A fragments, [sub-block][lane 0..63][16 bytes] (lane l: matrix row
-// l % 32, values 16 (l / 32)..+15 of the sub-block), so that a wave fetches a fragment with one
-// coalesced load, then the block's 16 token scales.  Matrix row i = 8 a + 4 half + 2 c + plane
-// holds token S * half + 2 a + c, which puts token S * (lane / 32) + slot into output registers
-// 2 * slot (high plane) and 2 * slot + 1 (low plane); S = token slots per lane.
-constexpr int kImageFragments = 8 * 1024;
-constexpr int kImageBlock = kImageFragments + 16 * 4;
-
-__host__ __device__ constexpr int token_slots(int tokens) { return tokens <= 4 ? 2 : tokens <= 8 ? 4 : 8; }
+constexpr int kImageFragments = kRowsImageFragments;
+constexpr int kImageBlock = kRowsImageBlock;
 
 // One wave per activation record: writes the (token, block) record of wave_rows.hpp and the
 // token's share of the block's operand image.
@@ -75,20 +67,7 @@ __global__ __launch_bounds__(256) void quantize_records_kernel(
     store_record(records + static_cast<std::int64_t>(record) * kActRecord, lane, codes);
     const int token = record / blocks;
     const int block = record - token * blocks;
-    const int slots = token_slots(tokens);
-    const int half = token / slots;
-    const int slot = token - half * slots;
-    const int row = 8 * (slot >> 1) + 4 * half + 2 * (slot & 1);
-    // this lane's values 4 lane..+3: sub-block lane / 8, values 4 (lane % 8)..+3 of it
-    std::uint8_t* block_image = image + static_cast<std::int64_t>(block) * kImageBlock;
-    std::uint8_t* piece = block_image +
-        (((lane >> 3) * 64 + ((lane >> 2) & 1) * 32 + row) * 16) + (lane & 3) * 4;
-    *reinterpret_cast<std::uint32_t*>(piece) = codes.hi;
-    *reinterpret_cast<std::uint32_t*>(piece + 16) = codes.lo;
-    if (lane == 0) {
-        reinterpret_cast<float*>(block_image + kImageFragments)[token] =
-            codes.maximum * (1.0f / kCodeRange);
-    }
+    store_operand_image(image, block, token, tokens, lane, codes);
 }
 
 // How a block (256 values of one weight row) lies in memory and in a wave's LDS tile.

@@ -41,14 +41,18 @@ void launch_swiglu(const float* gate, const float* up, float* output, std::int64
 // `records` (may be null, else one row only): the small-batch workspace that
 // receives the activation records of normalized_output.  `half_image` (may be null,
 // else rows of at most 8,192 columns): the small-batch workspace of `rows` rows that
-// receives normalized_output as the fp16 small-batch kernel's image.
+// receives normalized_output as the fp16 small-batch kernel's image.  `operand_image` (may
+// be null; with `records`, rows of at most 8,192 columns): the records are those of all
+// `rows` rows, token by token, and the same codes go to `operand_image` in the order the
+// exact verifier's matrix-core kernel reads them (gemv_rows.hpp).
 void launch_dual_rms_add_capture(const float* input, const Descriptor* first_weight,
                                  bool first_centered, const float* residual_input,
                                  float* hidden_output, const Descriptor* second_weight,
                                  bool second_centered, float* normalized_output,
                                  float* residual_output, std::int64_t rows, std::int64_t width,
                                  float first_eps, float second_eps, std::uint8_t* records,
-                                 std::uint8_t* half_image, hipStream_t stream);
+                                 std::uint8_t* half_image, hipStream_t stream,
+                                 std::uint8_t* operand_image = nullptr);
 
 // One normalisation: output = rms(input, weight, eps) (+ residual_input when
 // given); residual_output (may be null) receives a copy of the input; the

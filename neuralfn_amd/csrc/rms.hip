@@ -22,6 +22,7 @@
 // square root, so the two can differ in the last bits of that one factor.
 #include "common.hpp"
 #include "f16_decode.hpp"
+#include "gemv_rows.hpp"
 #include "kernels.hpp"
 #include "rms_device.hpp"
 #include "wave_rows.hpp"
@@ -169,17 +170,19 @@ constexpr int kLoaded = kOwned / kLoaders;  // columns per thread
 
 // HANDOFF 0: nothing more; 1: the activation records of the normalized row (one row);
 // 2: the normalized rows as the fp16 image of the fp16 small-batch kernel, `records` being
-// the small-batch workspace of gridDim.x rows.
+// the small-batch workspace of gridDim.x rows; 3: the activation records of gridDim.x rows
+// (token by token) and, at `operand_image`, the same codes in matrix-operand order: what
+// the exact verifier's quantizer launch leaves for its matrix-core kernel (gemv_rows.hpp).
 template <int HANDOFF>
 __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     const float* __restrict__ input, NormWeight first_weight,
     const float* __restrict__ residual_input, float* __restrict__ hidden_output,
     NormWeight second_weight, float* __restrict__ normalized_output,
     float* __restrict__ residual_output, int width, float first_eps, float second_eps,
-    std::uint8_t* __restrict__ records) {
+    std::uint8_t* __restrict__ records, std::uint8_t* __restrict__ operand_image) {
     __shared__ float partials[kRmsThreads + 1];
     __shared__ __attribute__((aligned(16))) float handed[kOwned * kRmsThreads];  // [k][t]: column t + 256 k
-    extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF 1: the normalized row
+    extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF 1, 3: the normalized row
     __shared__ float wave_largest[kWideThreads / kWave];
     const std::int64_t row = blockIdx.x;
     const float* source = input + row * width;
@@ -245,7 +248,7 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
         const float result = __fmul_rn(__fmul_rn(value[i], second_inverse), second_scale[i]);
         if (column < width) {
             normalized[column] = result;
-            if constexpr (HANDOFF == 1) staged[column] = result;
+            if constexpr (HANDOFF == 1 || HANDOFF == 3) staged[column] = result;
             // (the sums have read `handed`: tree_total_wide's barriers lie in between)
             if constexpr (HANDOFF == 2) handed[column] = result;
             largest = fmaxf(largest, fabsf(result));
@@ -273,15 +276,22 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
         }
     }
 
-    if constexpr (HANDOFF == 1) {
+    if constexpr (HANDOFF == 1 || HANDOFF == 3) {
         __syncthreads();
         // one wave per 256-value block: the quantizer of the decode kernels
         const int lane = threadIdx.x & 63;
         const int wave = threadIdx.x >> 6;
-        for (int block = wave; block < (width >> 8); block += kWideThreads / kWave) {
+        const int blocks = width >> 8;
+        for (int block = wave; block < blocks; block += kWideThreads / kWave) {
             const float4 x = *reinterpret_cast<const float4*>(staged + block * 256 + lane * 4);
-            store_record(records + static_cast<std::int64_t>(block) * kActRecord, lane,
-                         encode_activations(x));
+            const ActivationCodes codes = encode_activations(x);
+            if constexpr (HANDOFF == 3) {
+                store_record(records + (row * blocks + block) * kActRecord, lane, codes);
+                store_operand_image(operand_image, block, static_cast<int>(row),
+                                    static_cast<int>(gridDim.x), lane, codes);
+            } else {
+                store_record(records + static_cast<std::int64_t>(block) * kActRecord, lane, codes);
+            }
         }
     }
 }
@@ -466,26 +476,34 @@ void launch_dual_rms_add_capture(const float* input, const Descriptor* first_wei
                                  bool second_centered, float* normalized_output,
                                  float* residual_output, std::int64_t rows, std::int64_t width,
                                  float first_eps, float second_eps, std::uint8_t* records,
-                                 std::uint8_t* half_image, hipStream_t stream) {
+                                 std::uint8_t* half_image, hipStream_t stream,
+                                 std::uint8_t* operand_image) {
     const NormWeight first = norm_weight(first_weight, first_centered);
     const NormWeight second = norm_weight(second_weight, second_centered);
     const dim3 grid(static_cast<unsigned>(rows));
     if (width <= kOwned * kRmsThreads) {
         const int columns = static_cast<int>(width);
+        std::uint8_t* const none = nullptr;
         if (half_image != nullptr) {
             hipLaunchKernelGGL((dual_rms_resident_kernel<2>), grid, dim3(kWideThreads), 0, stream, input,
                                first, residual_input, hidden_output, second, normalized_output,
-                               residual_output, columns, first_eps, second_eps, half_image);
+                               residual_output, columns, first_eps, second_eps, half_image, none);
+        } else if (records != nullptr && operand_image != nullptr) {
+            hipLaunchKernelGGL((dual_rms_resident_kernel<3>), grid, dim3(kWideThreads),
+                               static_cast<std::size_t>(columns) * sizeof(float), stream, input,
+                               first, residual_input, hidden_output, second, normalized_output,
+                               residual_output, columns, first_eps, second_eps, records,
+                               operand_image);
         } else if (records != nullptr) {
             hipLaunchKernelGGL((dual_rms_resident_kernel<1>), grid, dim3(kWideThreads),
                                static_cast<std::size_t>(columns) * sizeof(float), stream, input,
                                first, residual_input, hidden_output, second, normalized_output,
-                               residual_output, columns, first_eps, second_eps, records);
+                               residual_output, columns, first_eps, second_eps, records, none);
         } else {
             hipLaunchKernelGGL((dual_rms_resident_kernel<0>), grid, dim3(kWideThreads), 0, stream,
                                input, first, residual_input, hidden_output, second,
                                normalized_output, residual_output, columns, first_eps, second_eps,
-                               records);
+                               records, none);
         }
         return;
     }

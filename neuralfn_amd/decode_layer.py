@@ -161,22 +161,24 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
     (nfn_native_tile_k_quant_mmvq_multi_linear*_float32_v1), as the engine's speculative decode
     calls them with exact_verifier_rows (resident_glimmer.cpp:2662-2666,
     resident_glimmer_cuda.cpp:3526-3532): row r then equals decode_layer's projections bit for
-    bit.  The two additions above belong to the other family and are not combined with it.
+    bit.  With handoff (4..16 rows) the norms leave the rows' activation records and their
+    matrix-operand copy (nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1) for the reference's
+    prequantized consumer; the gate/up pair call belongs to the other family.
 
     Returns (down, hidden, key_rows, value_rows).
     """
     g = geometry
     rows = pending.shape[0]
-    if family == "mmvq" and (handoff or fused_gate_up):
-        raise ValueError("the handoff and the gate/up pair call are forms of the mmq family")
+    if family == "mmvq" and fused_gate_up:
+        raise ValueError("the gate/up pair call is a form of the mmq family")
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         pending, residual, pending_norm, False, weights.input_norm, False,
         g.post_norm_eps if pending_norm is not None else g.norm_eps, g.norm_eps,
-        handoff_workspace=workspace if handoff else None)
+        handoff_workspace=workspace if handoff else None, handoff_family=family)
     attention_inputs = [weights.q, weights.k, weights.v, weights.attention_gate]
     if handoff:
         query, key, value, gate = tile_ops.multi_linear_prequantized(
-            attention_inputs, rows, workspace, family="mmq")
+            attention_inputs, rows, workspace, family=family)
     else:
         query, key, value, gate = tile_ops.multi_linear(attention_inputs, normalized, workspace,
                                                         family=family)
@@ -195,7 +197,8 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
                                          workspace, second=gate, family=family, prologue="gated")
     hidden, normalized, _ = tile_ops.dual_rms_add_capture(
         projected, hidden, weights.post_attention_norm, False, weights.pre_feedforward_norm, False,
-        g.post_norm_eps, g.norm_eps, handoff_workspace=workspace if handoff else None)
+        g.post_norm_eps, g.norm_eps, handoff_workspace=workspace if handoff else None,
+        handoff_family=family)
     if fused_gate_up and tile_ops.gate_up_swiglu_rows_supported(weights.mlp_gate, weights.mlp_up, rows):
         activated = tile_ops.gate_up_swiglu_rows(weights.mlp_gate, weights.mlp_up,
                                                  None if handoff else normalized, rows, workspace)
@@ -203,7 +206,7 @@ def verify_layer(geometry: LayerGeometry, weights: LayerWeights, cache: LayerCac
         return down, hidden, key, value
     if handoff:
         mlp_gate, mlp_up = tile_ops.multi_linear_prequantized(
-            [weights.mlp_gate, weights.mlp_up], rows, workspace, family="mmq")
+            [weights.mlp_gate, weights.mlp_up], rows, workspace, family=family)
     else:
         mlp_gate, mlp_up = tile_ops.multi_linear([weights.mlp_gate, weights.mlp_up], normalized,
                                                  workspace, family=family)

@@ -184,6 +184,9 @@ SIGNATURES = {
     "nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1": (
         ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
                        ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
+    "nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1": (
+        ctypes.c_int, [_P, _DESC, _P, _P, _DESC, _P, _P, _I64, _I64, ctypes.c_float, ctypes.c_bool,
+                       ctypes.c_float, ctypes.c_bool, _P, _I64, _P]),
     "nfn_mi355_k_quant_mmvq_gate_up_swiglu_float32_v1": (ctypes.c_int, [_DESC, _DESC, _P, _P, _P]),
     "nfn_mi355_k_quant_mmq_gate_up_swiglu_float32_v1": (
         ctypes.c_int, [_DESC, _DESC, _P, _P, _I64, _P, _I64, _P]),
@@ -460,12 +463,13 @@ def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = Non
                          first_centered: bool = False,
                          second_weight: Optional[PackedWeight] = None,
                          second_centered: bool = False, first_eps: float = 1e-6,
-                         second_eps: float = 1e-6, handoff_workspace=None):
+                         second_eps: float = 1e-6, handoff_workspace=None,
+                         handoff_family: str = "mmq"):
     """hidden = residual + rms(x, first); normalized = rms(hidden, second).
 
     Returns (hidden, normalized, residual_output).  With `handoff_workspace` the quantized form
     of `normalized` is left there for multi_linear_prequantized: one row, family "mmvq";
-    5..16 rows, family "mmq".
+    5..16 rows, family "mmq" (`handoff_family`), or 4..16 rows, family "mmvq".
     """
     import torch
     rows, width = x.shape
@@ -487,6 +491,10 @@ def dual_rms_add_capture(x, residual, first_weight: Optional[PackedWeight] = Non
         check(load().nfn_native_tile_glimmer_dual_rms_add_capture_mmvq_q8_float32_v1(
             *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
             "dual_rms_add_capture_mmvq_q8")
+    elif handoff_family == "mmvq":
+        check(load().nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1(
+            *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),
+            "dual_rms_add_capture_mmvq_rows")
     else:
         check(load().nfn_mi355_dual_rms_add_capture_mmq_f16_float32_v1(
             *arguments, handoff_workspace.data_ptr(), handoff_workspace.numel(), stream),

@@ -1060,6 +1060,10 @@ def test_model_sized_layer_fused_calls_and_verifier_families(cuda, oracle):
         assert torch_().equal(a, b), "block of 16: handoff and gate/up call"
     exact = dl.verify_layer(g, weights, cache(), embeddings, zero, None, position, block, True,
                             attention_workspace, family="mmvq")
+    handed = dl.verify_layer(g, weights, cache(), embeddings, zero, None, position, block, True,
+                             attention_workspace, family="mmvq", handoff=True)
+    for a, b in zip(exact, handed):
+        assert torch_().equal(a, b), "block of 16, exact family: norm handoff"
     scale = float(np.max(np.abs(serial)))
     assert scale > 0 and np.isfinite(scale)
     assert float(np.max(np.abs(exact[0].cpu().numpy() - serial))) <= 1e-4 * scale

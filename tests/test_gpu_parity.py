@@ -1193,6 +1193,67 @@ def test_dual_rms_inside_the_projection_launch_fails_closed(cuda):
     torch_().cuda.synchronize()
 
 
+@pytest.mark.parametrize("rows,width", [(4, 256), (5, 6656), (9, 2304), (16, 6656), (16, 8192)])
+def test_dual_rms_block_handoff_of_the_exact_family_equals_ordinary_path(cuda, rows, width):
+    """nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1: the norm kernel leaves the rows'
+    activation records and their matrix-operand copy, and the reference's prequantized consumer
+    fed from them gives the bits of the dual RMS followed by the verifier call (and so of the
+    one-row call on every row); rows several orders of magnitude apart keep their own scales."""
+    rng = np.random.default_rng(170 + rows)
+    x = probe_rms_input(rows, width) * (10.0 ** rng.integers(-3, 4, (rows, 1))).astype(np.float32)
+    residual = (rng.standard_normal((rows, width)) *
+                10.0 ** rng.integers(-2, 3, (rows, 1))).astype(np.float32)
+    scale = tile_ops.PackedWeight.from_numpy(
+        kquant.F32, kquant.quantize(kquant.F32, rng.uniform(0.5, 1.5, (1, width)).astype(np.float32)),
+        1, width)
+    specs = [(kquant.Q4_K, 129), (kquant.Q5_K, 33), (kquant.Q6_K, 70), (kquant.Q8_0, 17)]
+    weights = [tile_ops.PackedWeight.from_numpy(e, random_packed(e, n, width, 140 + i), n, width)
+               for i, (e, n) in enumerate(specs)]
+    workspace = tile_ops.small_batch_workspace(rows, width)
+    arguments = dict(first_weight=scale, second_weight=scale, first_eps=1e-8, second_eps=1e-5)
+    ordinary = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda), **arguments)
+    ordinary_out = tile_ops.multi_linear(weights, ordinary[1], workspace, family="mmvq")
+    workspace.zero_()
+    handoff = tile_ops.dual_rms_add_capture(to_device(x, cuda), to_device(residual, cuda),
+                                            handoff_workspace=workspace, handoff_family="mmvq",
+                                            **arguments)
+    handoff_out = tile_ops.multi_linear_prequantized(weights, rows, workspace, family="mmvq")
+    again = tile_ops.multi_linear_prequantized(weights[1:3], rows, workspace, family="mmvq")
+    for a, b, label in zip(ordinary, handoff, ("hidden", "normalized", "capture")):
+        assert_bits_equal(a, b, label)
+    for a, b, (encoding, _) in zip(ordinary_out, handoff_out, specs):
+        assert_bits_equal(a, b, kquant.NAMES[encoding])
+    for a, b in zip(ordinary_out[1:3], again):
+        assert_bits_equal(a, b, "a second consumer of the same rows")
+    one = tile_ops.small_batch_workspace(1, width)
+    alone = tile_ops.multi_linear(weights, ordinary[1][rows - 1:rows].contiguous(), one, family="mmvq")
+    for a, b in zip(handoff_out, alone):
+        assert_bits_equal(a[rows - 1:rows].contiguous(), b, "the one-row call on the last row")
+
+
+def test_block_handoff_of_the_exact_family_fails_closed(cuda):
+    width = 512
+    lib = tile_ops.load()
+    x = to_device(probe_rms_input(16, width), cuda)
+    outputs = [torch_().empty_like(x) for _ in range(3)]
+    workspace = tile_ops.small_batch_workspace(16, width)
+    head = [x.data_ptr(), None, x.data_ptr(), outputs[0].data_ptr(), None, outputs[1].data_ptr(),
+            outputs[2].data_ptr()]
+    tail = [1e-8, False, 1e-5, False]
+    handoff = lib.nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1
+    required = lib.nfn_native_tile_k_quant_mmq_workspace_bytes_v1(8, width)
+    assert handoff(*head, 8, width, *tail, workspace.data_ptr(), required, None) == 0
+    assert handoff(*head, 4, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 0
+    assert handoff(*head, 3, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 17, width, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 8, width, *tail, workspace.data_ptr(), required - 1, None) == 1
+    assert handoff(*head, 8, width, *tail, None, required, None) == 1
+    assert handoff(*head, 8, 384, *tail, workspace.data_ptr(), workspace.numel(), None) == 1
+    assert handoff(*head, 8, 8448, *tail, workspace.data_ptr(), 1 << 30, None) == 1
+    assert handoff(*head, 8, width, 0.0, False, 1e-5, False, workspace.data_ptr(), required, None) == 1
+    torch_().cuda.synchronize()
+
+
 def test_block_handoff_fails_closed(cuda):
     width = 512
     lib = tile_ops.load()
