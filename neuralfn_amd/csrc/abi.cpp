@@ -56,6 +56,12 @@ std::int64_t small_batch_workspace_bytes(std::int64_t rows, std::int64_t input_d
     return (raw + 255) & ~std::int64_t(255);
 }
 
+bool ranges_overlap(const void* a, std::int64_t a_bytes, const void* b, std::int64_t b_bytes) {
+    const std::uintptr_t pa = reinterpret_cast<std::uintptr_t>(a);
+    const std::uintptr_t pb = reinterpret_cast<std::uintptr_t>(b);
+    return pa < pb + static_cast<std::uintptr_t>(b_bytes) && pb < pa + static_cast<std::uintptr_t>(a_bytes);
+}
+
 Projection make_projection(const Descriptor& descriptor, float* output) {
     Projection op{};
     op.data = descriptor.data;
@@ -139,11 +145,28 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
         // prequantized call behind it finds both), and the dot kernels of the other encodings
         // read the records instead of quantizing again.
         std::uint8_t* image = static_cast<std::uint8_t*>(workspace) + record_bytes(rows, input_dim);
+        // The quantizer launch can also prepare the outputs for the kernel's split form, unless
+        // one of them overlaps what that launch reads.
+        ProjectionSet clear{};
         if (prologue != kRecords) {
+            clear = gemv_rows_split_set(verifier_rows);
+            const std::int64_t input_bytes = rows * input_dim * static_cast<std::int64_t>(sizeof(float));
+            for (int index = 0; index < clear.count; ++index) {
+                const std::int64_t bytes =
+                    rows * clear.op[index].output_dim * static_cast<std::int64_t>(sizeof(float));
+                if (ranges_overlap(clear.op[index].output, bytes, first, input_bytes) ||
+                    (second != nullptr && ranges_overlap(clear.op[index].output, bytes, second, input_bytes))) {
+                    clear.count = 0;
+                    break;
+                }
+            }
             launch_quantize_records(first, second, prologue, rows, input_dim,
-                                    static_cast<std::uint8_t*>(workspace), image, as_stream(stream));
+                                    static_cast<std::uint8_t*>(workspace), image, clear,
+                                    as_stream(stream));
         }
-        if (verifier_rows.count > 0) launch_gemv_rows(verifier_rows, image, rows, as_stream(stream));
+        if (verifier_rows.count > 0) {
+            launch_gemv_rows(verifier_rows, image, rows, clear.count > 0, as_stream(stream));
+        }
         dot_first = static_cast<const float*>(workspace);
         dot_second = nullptr;
         dot_prologue = kRecords;

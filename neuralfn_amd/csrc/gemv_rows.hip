@@ -54,10 +54,34 @@ constexpr int kImageBlock = kRowsImageBlock;
 
 // One wave per activation record: writes the (token, block) record of wave_rows.hpp and the
 // token's share of the block's operand image.
+// Workgroups past those of the records fill the outputs of `clear` with -0.0f, 1024 floats a
+// workgroup: the split form of the kernel below adds the two halves of a row's butterfly
+// onto them (-0 + x is x for every x, -0 included).
 template <int P>
 __global__ __launch_bounds__(256) void quantize_records_kernel(
     const float* __restrict__ first, const float* __restrict__ second,
-    std::uint8_t* __restrict__ records, std::uint8_t* __restrict__ image, int blocks, int tokens) {
+    std::uint8_t* __restrict__ records, std::uint8_t* __restrict__ image, int blocks, int tokens,
+    int record_groups, ProjectionSet clear) {
+    if (static_cast<int>(blockIdx.x) >= record_groups) {
+        std::int64_t chunk = static_cast<std::int64_t>(blockIdx.x) - record_groups;
+#pragma unroll
+        for (int index = 0; index < 4; ++index) {
+            if (index >= clear.count) break;
+            const std::int64_t floats = clear.op[index].output_dim * tokens;
+            const std::int64_t chunks = (floats + 1023) >> 10;
+            if (chunk < chunks) {
+                float* output = clear.op[index].output;
+                const std::int64_t begin = (chunk << 10) + threadIdx.x * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (begin + e < floats) output[begin + e] = -0.0f;
+                }
+                return;
+            }
+            chunk -= chunks;
+        }
+        return;
+    }
     const int lane = threadIdx.x & 63;
     const int record = static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6);
     if (record >= blocks * tokens) return;
@@ -132,17 +156,25 @@ __device__ __forceinline__ void rows_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <std::uint32_t ENC, int S>
+// SPLIT: a workgroup computes one half of a row's butterfly, the classes 0..7 (the first
+// left_groups workgroups) or 8..15 (the others), a wave one class, and adds (q0 + q1) or
+// (q2 + q3) onto the output, which the quantizer launch has filled with -0: two terms commute,
+// so the sum is the one-row kernel's whichever half arrives first.  Twice the work units of
+// about half the length, shared out over the workgroups by what the halves cost (a row of 26
+// blocks has 16 on the left and 10 on the right): for tile counts that leave much of the
+// chip idle in the last round of whole tiles (272 tiles on 256 units).
+template <std::uint32_t ENC, int S, bool SPLIT>
 __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const std::uint8_t* __restrict__ image, int tokens, int input_dim, std::uint32_t total_tiles,
-    ProjectionSet set) {
+    std::uint32_t left_groups, ProjectionSet set) {
     constexpr bool kQ5 = ENC == kEncQ5K;
     using F = RowsFormat<ENC>;
     constexpr int kBlockBytes = F::kBlockBytes;
     constexpr int kQuants = kQ5 ? 48 : 16;
     constexpr int kTokens = 2 * S;
     // (two buffers of class sums: the workgroup's waves meet once per tile)
-    __shared__ float class_sums[2][kClasses][kTokens][kRowsTile];
+    constexpr int kOwnClasses = SPLIT ? kClasses / 2 : kClasses;
+    __shared__ float class_sums[2][kOwnClasses][kTokens][kRowsTile];
     __shared__ __attribute__((aligned(16))) std::uint8_t packed_tiles[kRowsWaves][F::kTileBytes];
 
     const int lane = threadIdx.x & 63;
@@ -153,8 +185,11 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
 
     // A workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the loads of a
     // tile's first block go out under the arithmetic of the tile before.
-    const std::uint32_t first_tile = blockIdx.x;
-    const int my_tiles = static_cast<int>((total_tiles - first_tile + gridDim.x - 1) / gridDim.x);
+    const bool right_half = SPLIT && blockIdx.x >= left_groups;
+    const std::uint32_t first_tile = right_half ? blockIdx.x - left_groups : blockIdx.x;
+    const std::uint32_t tile_stride =
+        SPLIT ? (right_half ? gridDim.x - left_groups : left_groups) : gridDim.x;
+    const int my_tiles = static_cast<int>((total_tiles - first_tile + tile_stride - 1) / tile_stride);
     auto projection_of = [&](std::uint32_t tile) {
         int which = 0;
 #pragma unroll
@@ -209,10 +244,18 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const std::uint8_t* const my_row = my_tile + j * F::kSlotBytes + F::kSlotOrigin;
 
     // this wave's steps of a tile: the blocks of class `wave`, then those of class 15 - wave
-    const int class0 = wave;
+    // (SPLIT: the one class 8 (right half) + wave)
+    const int class0 = SPLIT ? (right_half ? 8 : 0) + wave : wave;
     const int class1 = kClasses - 1 - wave;
     const int count0 = class0 < blocks ? (blocks - class0 + kClasses - 1) / kClasses : 0;
-    const int count1 = class1 < blocks ? (blocks - class1 + kClasses - 1) / kClasses : 0;
+    int count1 = class1 < blocks ? (blocks - class1 + kClasses - 1) / kClasses : 0;
+    if constexpr (SPLIT) {
+        // (no second class; a value the optimizer cannot see through, so that the walk below
+        // compiles as it does for two classes: with a known zero it is scheduled with far
+        // more registers, and spills)
+        count1 = 0;
+        asm volatile("" : "+s"(count1));
+    }
     const int total = count0 + count1;
 
     auto block_of = [&](int step) {
@@ -253,9 +296,9 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
                 operands.a[sub] = *reinterpret_cast<const v4i*>(fragments + sub * 1024 + lane * 16);
             }
         }
-        if (++fetch_step >= total && fetch_tile + gridDim.x < total_tiles) {
+        if (++fetch_step >= total && fetch_tile + tile_stride < total_tiles) {
             fetch_step = 0;
-            fetch_tile += gridDim.x;
+            fetch_tile += tile_stride;
             aim(fetch_tile);
         }
     };
@@ -478,7 +521,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     auto finish_class = [&](int cls) {
 #pragma unroll
         for (int slot = 0; slot < S; ++slot) {
-            class_sums[parity][cls][S * h + slot][j] =
+            class_sums[parity][cls & (kOwnClasses - 1)][S * h + slot][j] =
                 (acc[0][slot] + acc[1][slot]) + (acc[2][slot] + acc[3][slot]);
 #pragma unroll
             for (int p = 0; p < 4; ++p) acc[p][slot] = 0.0f;
@@ -495,26 +538,42 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
             static_cast<int>(min(static_cast<std::int64_t>(kRowsTile), op.output_dim - row0));
         const int token = static_cast<int>(threadIdx.x) >> 5;
         if (token < kTokens && token < tokens && j < valid_rows) {
-            float pairs[8];
+            float pairs[kOwnClasses / 2];
 #pragma unroll
-            for (int m = 0; m < 8; ++m) {
+            for (int m = 0; m < kOwnClasses / 2; ++m) {
                 pairs[m] = class_sums[parity][2 * m][token][j] + class_sums[parity][2 * m + 1][token][j];
             }
-            const float q0 = pairs[0] + pairs[1];
-            const float q1 = pairs[2] + pairs[3];
-            const float q2 = pairs[4] + pairs[5];
-            const float q3 = pairs[6] + pairs[7];
-            op.output[static_cast<std::int64_t>(token) * op.output_dim + row0 + j] = (q0 + q1) + (q2 + q3);
+            float* output = op.output + (static_cast<std::int64_t>(token) * op.output_dim + row0 + j);
+            if constexpr (SPLIT) {
+                // this half of the butterfly; the other workgroup's joins it in either order
+                // (a compare-and-swap loop: the sum is a vector-ALU addition like every other)
+                const float mine = (pairs[0] + pairs[1]) + (pairs[2] + pairs[3]);
+                unsigned int* word = reinterpret_cast<unsigned int*>(output);
+                unsigned int seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                while (true) {
+                    const unsigned int wanted = __float_as_uint(__uint_as_float(seen) + mine);
+                    if (__hip_atomic_compare_exchange_strong(word, &seen, wanted, __ATOMIC_RELAXED,
+                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+                        break;
+                    }
+                }
+            } else {
+                const float q0 = pairs[0] + pairs[1];
+                const float q1 = pairs[2] + pairs[3];
+                const float q2 = pairs[4] + pairs[5];
+                const float q3 = pairs[6] + pairs[7];
+                *output = (q0 + q1) + (q2 + q3);
+            }
         }
         parity ^= 1;
-        work_tile += gridDim.x;
+        work_tile += tile_stride;
     };
 
     if (total == 0) {
         // (rows of fewer blocks than classes: this wave only takes part in the sums)
         for (int n = 0; n < my_tiles; ++n) {
             finish_class(class0);
-            finish_class(class1);
+            if constexpr (!SPLIT) finish_class(class1);
             finish_tile();
         }
         return;
@@ -541,7 +600,7 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     auto finish_step = [&]() {
         if (work_step == count0 - 1) finish_class(class0);
         if (work_step == total - 1) {
-            finish_class(class1);
+            if constexpr (!SPLIT) finish_class(class1);
             finish_tile();
             work_step = 0;
         } else {
@@ -565,28 +624,111 @@ __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     }
 }
 
+std::uint32_t tiles_of(const ProjectionSet& set) {
+    std::uint32_t tiles = 0;
+    for (int index = 0; index < set.count; ++index) {
+        tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kRowsTile - 1) / kRowsTile);
+    }
+    return tiles;
+}
+
+// How a launch of `tiles` tiles of rows of `blocks` blocks is shared out.  Costs in blocks a
+// SIMD works through (two of a workgroup's eight waves to a SIMD, waves w and w + 4): a whole
+// tile gives wave w the classes w and 15 - w, the split form the class w (left half) or 8 + w
+// (right half); a block and a half per work unit for its first loads, its barrier and its
+// stores (measured: 1.1 us a block, 1.6 us a unit at 16 tokens).
+struct RowsPlan {
+    bool split;
+    std::uint32_t left_groups;   // split: workgroups on the left halves
+    std::uint32_t groups;        // workgroups of the launch
+};
+
+RowsPlan plan_rows(std::uint32_t tiles, std::int64_t input_dim, bool may_split) {
+    const std::uint32_t units = static_cast<std::uint32_t>(compute_units());
+    const int blocks = static_cast<int>(input_dim >> 8);
+    const auto count = [blocks](int cls) { return cls < blocks ? (blocks - cls + kClasses - 1) / kClasses : 0; };
+    int whole = 0, left = 0, right = 0;
+    for (int simd = 0; simd < 4; ++simd) {
+        const int a = simd, b = simd + 4;
+        const int whole_here = count(a) + count(kClasses - 1 - a) + count(b) + count(kClasses - 1 - b);
+        const int left_here = count(a) + count(b);
+        const int right_here = count(8 + a) + count(8 + b);
+        whole = whole_here > whole ? whole_here : whole;
+        left = left_here > left ? left_here : left;
+        right = right_here > right ? right_here : right;
+    }
+    const auto rounds = [tiles](std::uint32_t groups) { return (tiles + groups - 1) / groups; };
+    RowsPlan plan{false, 0, tiles < units ? tiles : units};
+    if (!may_split || units < 2) return plan;
+    // costs in half blocks
+    const std::uint64_t whole_cost = static_cast<std::uint64_t>(rounds(plan.groups)) * (2 * whole + 3);
+    std::uint64_t best = ~std::uint64_t(0);
+    std::uint32_t best_left = 0, best_right = 0;
+    for (std::uint32_t left_groups = 1; left_groups < units; ++left_groups) {
+        const std::uint32_t l = left_groups < tiles ? left_groups : tiles;
+        const std::uint32_t r = units - left_groups < tiles ? units - left_groups : tiles;
+        const std::uint64_t left_cost = static_cast<std::uint64_t>(rounds(l)) * (2 * left + 3);
+        const std::uint64_t right_cost = static_cast<std::uint64_t>(rounds(r)) * (2 * right + 3);
+        const std::uint64_t cost = left_cost > right_cost ? left_cost : right_cost;
+        if (cost < best) {
+            best = cost;
+            best_left = l;
+            best_right = r;
+        }
+    }
+    // (the split form has to win by a tenth: the model is that coarse)
+    if (best * 10 <= whole_cost * 9) {
+        plan.split = true;
+        plan.left_groups = best_left;
+        plan.groups = best_left + best_right;
+    }
+    return plan;
+}
+
+template <std::uint32_t ENC, bool SPLIT>
+void launch_form(const ProjectionSet& set, const std::uint8_t* image, int tokens, std::uint32_t tiles,
+                 const RowsPlan& plan, hipStream_t stream) {
+    const dim3 grid(plan.groups), block(kRowsThreads);
+    const int input_dim = static_cast<int>(set.input_dim);
+    if (tokens <= 4) {
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 2, SPLIT>), grid, block, 0, stream, image, tokens,
+                           input_dim, tiles, plan.left_groups, set);
+    } else if (tokens <= 8) {
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 4, SPLIT>), grid, block, 0, stream, image, tokens,
+                           input_dim, tiles, plan.left_groups, set);
+    } else {
+        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 8, SPLIT>), grid, block, 0, stream, image, tokens,
+                           input_dim, tiles, plan.left_groups, set);
+    }
+}
+
 template <std::uint32_t ENC>
-void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, hipStream_t stream) {
+void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, bool outputs_cleared,
+                     hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kRowsTile - 1) / kRowsTile);
     }
-    // one workgroup per compute unit walks the tiles; fewer tiles: a workgroup each
-    const std::uint32_t units = static_cast<std::uint32_t>(compute_units());
-    const dim3 grid(tiles < units ? tiles : units), block(kRowsThreads);
-    const int input_dim = static_cast<int>(set.input_dim);
-    if (tokens <= 4) {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 2>), grid, block, 0, stream, image, tokens,
-                           input_dim, tiles, set);
-    } else if (tokens <= 8) {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 4>), grid, block, 0, stream, image, tokens,
-                           input_dim, tiles, set);
+    const RowsPlan plan = plan_rows(tiles, set.input_dim, outputs_cleared);
+    if (plan.split) {
+        launch_form<ENC, true>(set, image, tokens, tiles, plan, stream);
     } else {
-        hipLaunchKernelGGL((gemv_rows_kernel<ENC, 8>), grid, block, 0, stream, image, tokens,
-                           input_dim, tiles, set);
+        launch_form<ENC, false>(set, image, tokens, tiles, plan, stream);
     }
 }
+
+// the projections of one encoding, in the order of the set
+ProjectionSet encoding_group(const ProjectionSet& set, std::uint32_t encoding) {
+    ProjectionSet group{};
+    group.input_dim = set.input_dim;
+    for (int index = 0; index < set.count; ++index) {
+        if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
+    }
+    return group;
+}
+
+constexpr std::uint32_t kRowsEncodings[4] = {kEncQ4K, kEncQ5K, kEncQ6K, kEncQ8_0};
 
 }  // namespace
 
@@ -599,44 +741,55 @@ std::int64_t gemv_rows_image_bytes(std::int64_t input_dim) {
     return (input_dim >> 8) * kImageBlock;
 }
 
+ProjectionSet gemv_rows_split_set(const ProjectionSet& set) {
+    ProjectionSet split{};
+    split.input_dim = set.input_dim;
+    for (const std::uint32_t encoding : kRowsEncodings) {
+        const ProjectionSet group = encoding_group(set, encoding);
+        if (group.count == 0 || !plan_rows(tiles_of(group), set.input_dim, true).split) continue;
+        for (int index = 0; index < group.count; ++index) split.op[split.count++] = group.op[index];
+    }
+    return split;
+}
+
 void launch_quantize_records(const float* first, const float* second, int prologue,
                              std::int64_t rows, std::int64_t input_dim, std::uint8_t* records,
-                             std::uint8_t* image, hipStream_t stream) {
+                             std::uint8_t* image, const ProjectionSet& clear, hipStream_t stream) {
     const int blocks = static_cast<int>(input_dim >> 8);
     const int tokens = static_cast<int>(rows);
-    const dim3 grid(static_cast<unsigned>((blocks * tokens + 3) / 4)), block(256);
+    const int record_groups = (blocks * tokens + 3) / 4;
+    std::int64_t fill_groups = 0;
+    for (int index = 0; index < clear.count; ++index) {
+        fill_groups += (clear.op[index].output_dim * rows + 1023) >> 10;
+    }
+    const dim3 grid(static_cast<unsigned>(record_groups + fill_groups)), block(256);
     switch (prologue) {
         case kGated:
             hipLaunchKernelGGL((quantize_records_kernel<kGated>), grid, block, 0, stream, first,
-                               second, records, image, blocks, tokens);
+                               second, records, image, blocks, tokens, record_groups, clear);
             break;
         case kSwiGlu:
             hipLaunchKernelGGL((quantize_records_kernel<kSwiGlu>), grid, block, 0, stream, first,
-                               second, records, image, blocks, tokens);
+                               second, records, image, blocks, tokens, record_groups, clear);
             break;
         default:
             hipLaunchKernelGGL((quantize_records_kernel<kPlain>), grid, block, 0, stream, first,
-                               second, records, image, blocks, tokens);
+                               second, records, image, blocks, tokens, record_groups, clear);
             break;
     }
 }
 
 void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
-                      hipStream_t stream) {
-    const std::uint32_t encodings[4] = {kEncQ4K, kEncQ5K, kEncQ6K, kEncQ8_0};
-    for (const std::uint32_t encoding : encodings) {
-        ProjectionSet group{};
-        group.input_dim = set.input_dim;
-        for (int index = 0; index < set.count; ++index) {
-            if (set.op[index].encoding == encoding) group.op[group.count++] = set.op[index];
-        }
+                      bool outputs_cleared, hipStream_t stream) {
+    for (const std::uint32_t encoding : kRowsEncodings) {
+        const ProjectionSet group = encoding_group(set, encoding);
         if (group.count == 0) continue;
         const int tokens = static_cast<int>(rows);
         switch (encoding) {
-            case kEncQ4K: launch_encoding<kEncQ4K>(group, image, tokens, stream); break;
-            case kEncQ5K: launch_encoding<kEncQ5K>(group, image, tokens, stream); break;
-            case kEncQ6K: launch_encoding<kEncQ6K>(group, image, tokens, stream); break;
-            default: launch_encoding<kEncQ8_0>(group, image, tokens, stream); break;
+            case kEncQ4K: launch_encoding<kEncQ4K>(group, image, tokens, outputs_cleared, stream); break;
+            case kEncQ5K: launch_encoding<kEncQ5K>(group, image, tokens, outputs_cleared, stream); break;
+            case kEncQ6K: launch_encoding<kEncQ6K>(group, image, tokens, outputs_cleared, stream); break;
+            default: launch_encoding<kEncQ8_0>(group, image, tokens, outputs_cleared, stream); break;
         }
     }
 }

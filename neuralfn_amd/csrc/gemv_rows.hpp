@@ -45,15 +45,22 @@ bool gemv_rows_supports(std::uint32_t encoding, std::int64_t input_dim);
 // Bytes of the operand image of `input_dim` columns (any row count up to 16).
 std::int64_t gemv_rows_image_bytes(std::int64_t input_dim);
 
+// The projections of `set` whose launch adds the two halves of every row's butterfly onto the
+// output (the form that pays when whole tiles would leave most of the chip idle in their last
+// round): their outputs must hold -0.0f when launch_gemv_rows starts.
+ProjectionSet gemv_rows_split_set(const ProjectionSet& set);
+
 // Writes the activation records of `rows` rows (the prologue applied) to `records`
 // (rows * input_dim / 256 records of 576 bytes, token by token) and the same codes in
-// matrix-operand order to `image` (gemv_rows_image_bytes).
+// matrix-operand order to `image` (gemv_rows_image_bytes); fills the outputs (rows x
+// output_dim floats each) of the projections of `clear` with -0.0f.
 void launch_quantize_records(const float* first, const float* second, int prologue,
                              std::int64_t rows, std::int64_t input_dim, std::uint8_t* records,
-                             std::uint8_t* image, hipStream_t stream);
+                             std::uint8_t* image, const ProjectionSet& clear, hipStream_t stream);
 
-// rows 2..16 of the set's Q4_K / Q5_K projections from the operand image.
+// rows 4..16 of the set's projections from the operand image.  outputs_cleared: the outputs of
+// gemv_rows_split_set(set) hold -0.0f (launch_quantize_records ran with that set).
 void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
-                      hipStream_t stream);
+                      bool outputs_cleared, hipStream_t stream);
 
 }  // namespace nfn
