@@ -147,9 +147,12 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
         std::uint8_t* image = static_cast<std::uint8_t*>(workspace) + record_bytes(rows, input_dim);
         // The quantizer launch can also prepare the outputs for the kernel's split form, unless
         // one of them overlaps what that launch reads.
-        ProjectionSet clear{};
-        if (prologue != kRecords) {
-            clear = gemv_rows_split_set(verifier_rows);
+        // (a prequantized call has no such launch: a fill launch of its own where that pays)
+        const bool fill_launch = prologue == kRecords;
+        ProjectionSet clear = gemv_rows_split_set(verifier_rows, fill_launch);
+        if (fill_launch) {
+            launch_fill_outputs(clear, rows, as_stream(stream));
+        } else {
             const std::int64_t input_bytes = rows * input_dim * static_cast<std::int64_t>(sizeof(float));
             for (int index = 0; index < clear.count; ++index) {
                 const std::int64_t bytes =
@@ -165,7 +168,7 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
                                     as_stream(stream));
         }
         if (verifier_rows.count > 0) {
-            launch_gemv_rows(verifier_rows, image, rows, clear.count > 0, as_stream(stream));
+            launch_gemv_rows(verifier_rows, image, rows, clear.count > 0, fill_launch, as_stream(stream));
         }
         dot_first = static_cast<const float*>(workspace);
         dot_second = nullptr;

@@ -643,7 +643,9 @@ struct RowsPlan {
     std::uint32_t groups;        // workgroups of the launch
 };
 
-RowsPlan plan_rows(std::uint32_t tiles, std::int64_t input_dim, bool may_split) {
+// fill_launch: the outputs are filled by a launch of its own (a prequantized call has no
+// quantizer launch to do it), which the split form must win back as well (two blocks' time).
+RowsPlan plan_rows(std::uint32_t tiles, std::int64_t input_dim, bool may_split, bool fill_launch = false) {
     const std::uint32_t units = static_cast<std::uint32_t>(compute_units());
     const int blocks = static_cast<int>(input_dim >> 8);
     const auto count = [blocks](int cls) { return cls < blocks ? (blocks - cls + kClasses - 1) / kClasses : 0; };
@@ -677,6 +679,7 @@ RowsPlan plan_rows(std::uint32_t tiles, std::int64_t input_dim, bool may_split) 
         }
     }
     // (the split form has to win by a tenth: the model is that coarse)
+    if (fill_launch) best += 4;
     if (best * 10 <= whole_cost * 9) {
         plan.split = true;
         plan.left_groups = best_left;
@@ -704,13 +707,13 @@ void launch_form(const ProjectionSet& set, const std::uint8_t* image, int tokens
 
 template <std::uint32_t ENC>
 void launch_encoding(ProjectionSet set, const std::uint8_t* image, int tokens, bool outputs_cleared,
-                     hipStream_t stream) {
+                     bool fill_launch, hipStream_t stream) {
     std::uint32_t tiles = 0;
     for (int index = 0; index < set.count; ++index) {
         set.op[index].first_tile = tiles;
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kRowsTile - 1) / kRowsTile);
     }
-    const RowsPlan plan = plan_rows(tiles, set.input_dim, outputs_cleared);
+    const RowsPlan plan = plan_rows(tiles, set.input_dim, outputs_cleared, fill_launch);
     if (plan.split) {
         launch_form<ENC, true>(set, image, tokens, tiles, plan, stream);
     } else {
@@ -741,12 +744,12 @@ std::int64_t gemv_rows_image_bytes(std::int64_t input_dim) {
     return (input_dim >> 8) * kImageBlock;
 }
 
-ProjectionSet gemv_rows_split_set(const ProjectionSet& set) {
+ProjectionSet gemv_rows_split_set(const ProjectionSet& set, bool fill_launch) {
     ProjectionSet split{};
     split.input_dim = set.input_dim;
     for (const std::uint32_t encoding : kRowsEncodings) {
         const ProjectionSet group = encoding_group(set, encoding);
-        if (group.count == 0 || !plan_rows(tiles_of(group), set.input_dim, true).split) continue;
+        if (group.count == 0 || !plan_rows(tiles_of(group), set.input_dim, true, fill_launch).split) continue;
         for (int index = 0; index < group.count; ++index) split.op[split.count++] = group.op[index];
     }
     return split;
@@ -779,17 +782,30 @@ void launch_quantize_records(const float* first, const float* second, int prolog
     }
 }
 
+void launch_fill_outputs(const ProjectionSet& clear, std::int64_t rows, hipStream_t stream) {
+    std::int64_t fill_groups = 0;
+    for (int index = 0; index < clear.count; ++index) {
+        fill_groups += (clear.op[index].output_dim * rows + 1023) >> 10;
+    }
+    if (fill_groups == 0) return;
+    // (the quantizer kernel with no records to write)
+    hipLaunchKernelGGL((quantize_records_kernel<kPlain>), dim3(static_cast<unsigned>(fill_groups)),
+                       dim3(256), 0, stream, static_cast<const float*>(nullptr),
+                       static_cast<const float*>(nullptr), static_cast<std::uint8_t*>(nullptr),
+                       static_cast<std::uint8_t*>(nullptr), 0, static_cast<int>(rows), 0, clear);
+}
+
 void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
-                      bool outputs_cleared, hipStream_t stream) {
+                      bool outputs_cleared, bool fill_launch, hipStream_t stream) {
     for (const std::uint32_t encoding : kRowsEncodings) {
         const ProjectionSet group = encoding_group(set, encoding);
         if (group.count == 0) continue;
         const int tokens = static_cast<int>(rows);
         switch (encoding) {
-            case kEncQ4K: launch_encoding<kEncQ4K>(group, image, tokens, outputs_cleared, stream); break;
-            case kEncQ5K: launch_encoding<kEncQ5K>(group, image, tokens, outputs_cleared, stream); break;
-            case kEncQ6K: launch_encoding<kEncQ6K>(group, image, tokens, outputs_cleared, stream); break;
-            default: launch_encoding<kEncQ8_0>(group, image, tokens, outputs_cleared, stream); break;
+            case kEncQ4K: launch_encoding<kEncQ4K>(group, image, tokens, outputs_cleared, fill_launch, stream); break;
+            case kEncQ5K: launch_encoding<kEncQ5K>(group, image, tokens, outputs_cleared, fill_launch, stream); break;
+            case kEncQ6K: launch_encoding<kEncQ6K>(group, image, tokens, outputs_cleared, fill_launch, stream); break;
+            default: launch_encoding<kEncQ8_0>(group, image, tokens, outputs_cleared, fill_launch, stream); break;
         }
     }
 }

@@ -48,7 +48,11 @@ std::int64_t gemv_rows_image_bytes(std::int64_t input_dim);
 // The projections of `set` whose launch adds the two halves of every row's butterfly onto the
 // output (the form that pays when whole tiles would leave most of the chip idle in their last
 // round): their outputs must hold -0.0f when launch_gemv_rows starts.
-ProjectionSet gemv_rows_split_set(const ProjectionSet& set);
+// fill_launch: the fill is a launch of its own (launch_fill_outputs), which has to pay too.
+ProjectionSet gemv_rows_split_set(const ProjectionSet& set, bool fill_launch);
+
+// Fills the outputs (rows x output_dim floats each) of the projections of `clear` with -0.0f.
+void launch_fill_outputs(const ProjectionSet& clear, std::int64_t rows, hipStream_t stream);
 
 // Writes the activation records of `rows` rows (the prologue applied) to `records`
 // (rows * input_dim / 256 records of 576 bytes, token by token) and the same codes in
@@ -59,8 +63,9 @@ void launch_quantize_records(const float* first, const float* second, int prolog
                              std::uint8_t* image, const ProjectionSet& clear, hipStream_t stream);
 
 // rows 4..16 of the set's projections from the operand image.  outputs_cleared: the outputs of
-// gemv_rows_split_set(set) hold -0.0f (launch_quantize_records ran with that set).
+// gemv_rows_split_set(set, fill_launch) hold -0.0f (launch_quantize_records or
+// launch_fill_outputs ran with that set).
 void launch_gemv_rows(const ProjectionSet& set, const std::uint8_t* image, std::int64_t rows,
-                      bool outputs_cleared, hipStream_t stream);
+                      bool outputs_cleared, bool fill_launch, hipStream_t stream);
 
 }  // namespace nfn
