@@ -838,7 +838,8 @@ int nfn_native_tile_scale_inplace_float32(
  * argument (a caller built against the two-argument form must not call it); the measurement
  * probes live in a library of their own (nfn_mi355_probes.h); the small-batch workspace of
  * four rows and more also holds the activations in matrix-operand order (the query
- * nfn_native_tile_k_quant_mmq_workspace_bytes_v1 returns the larger size). */
+ * nfn_native_tile_k_quant_mmq_workspace_bytes_v1 returns the larger size);
+ * nfn_mi355_dual_rms_add_capture_mmvq_rows_float32_v1 is new. */
 int nfn_mi355_abi_version(void);
 
 /* lm_head GEMV with the argmax fused in: logits never reach memory.  The
