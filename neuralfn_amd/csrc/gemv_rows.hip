@@ -162,7 +162,7 @@ __device__ __forceinline__ void rows_lds_fence() {
 // so the sum is the one-row kernel's whichever half arrives first.  Twice the work units of
 // about half the length, shared out over the workgroups by what the halves cost (a row of 26
 // blocks has 16 on the left and 10 on the right): for tile counts that leave much of the
-// chip idle in the last round of whole tiles (272 tiles on 256 units).
+// chip idle in the last pass over whole tiles (272 tiles on 256 units).
 template <std::uint32_t ENC, int S, bool SPLIT>
 __global__ __launch_bounds__(kRowsThreads) void gemv_rows_kernel(
     const std::uint8_t* __restrict__ image, int tokens, int input_dim, std::uint32_t total_tiles,
@@ -659,18 +659,18 @@ RowsPlan plan_rows(std::uint32_t tiles, std::int64_t input_dim, bool may_split, 
         left = left_here > left ? left_here : left;
         right = right_here > right ? right_here : right;
     }
-    const auto rounds = [tiles](std::uint32_t groups) { return (tiles + groups - 1) / groups; };
+    const auto passes = [tiles](std::uint32_t groups) { return (tiles + groups - 1) / groups; };
     RowsPlan plan{false, 0, tiles < units ? tiles : units};
     if (!may_split || units < 2) return plan;
     // costs in half blocks
-    const std::uint64_t whole_cost = static_cast<std::uint64_t>(rounds(plan.groups)) * (2 * whole + 3);
+    const std::uint64_t whole_cost = static_cast<std::uint64_t>(passes(plan.groups)) * (2 * whole + 3);
     std::uint64_t best = ~std::uint64_t(0);
     std::uint32_t best_left = 0, best_right = 0;
     for (std::uint32_t left_groups = 1; left_groups < units; ++left_groups) {
         const std::uint32_t l = left_groups < tiles ? left_groups : tiles;
         const std::uint32_t r = units - left_groups < tiles ? units - left_groups : tiles;
-        const std::uint64_t left_cost = static_cast<std::uint64_t>(rounds(l)) * (2 * left + 3);
-        const std::uint64_t right_cost = static_cast<std::uint64_t>(rounds(r)) * (2 * right + 3);
+        const std::uint64_t left_cost = static_cast<std::uint64_t>(passes(l)) * (2 * left + 3);
+        const std::uint64_t right_cost = static_cast<std::uint64_t>(passes(r)) * (2 * right + 3);
         const std::uint64_t cost = left_cost > right_cost ? left_cost : right_cost;
         if (cost < best) {
             best = cost;
