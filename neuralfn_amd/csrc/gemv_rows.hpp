@@ -47,7 +47,7 @@ std::int64_t gemv_rows_image_bytes(std::int64_t input_dim);
 
 // The projections of `set` whose launch adds the two halves of every row's butterfly onto the
 // output (the form that pays when whole tiles would leave most of the chip idle in their last
-// round): their outputs must hold -0.0f when launch_gemv_rows starts.
+// pass): their outputs must hold -0.0f when launch_gemv_rows starts.
 // fill_launch: the fill is a launch of its own (launch_fill_outputs), which has to pay too.
 ProjectionSet gemv_rows_split_set(const ProjectionSet& set, bool fill_launch);
 
