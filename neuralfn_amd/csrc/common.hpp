@@ -151,19 +151,34 @@ __device__ __forceinline__ float bf16_to_float(std::uint32_t bits) {
 // One rotary pair at `position`: angle = position / theta^(2*pair/head_dim) in
 // double, [a, b] -> [a cos - b sin, b cos + a sin]
 // (neuralfn/csrc/native_gpt2/resident_glimmer.cpp:773-800).
-__device__ __forceinline__ void rope_rotate(float& first, float& second, std::int64_t position,
-                                            std::int64_t pair, std::int64_t head_dim, double theta,
-                                            bool inverse) {
+// (in two steps, so that a kernel can work out the angle's sine and cosine -- a few hundred
+// double-precision instructions that depend on the position only -- while its loads are in flight)
+struct RopeAngle {
+    double sine, cosine;
+};
+
+__device__ __forceinline__ RopeAngle rope_angle(std::int64_t position, std::int64_t pair,
+                                                std::int64_t head_dim, double theta, bool inverse) {
     const double inverse_frequency =
         1.0 / pow(theta, static_cast<double>(2 * pair) / static_cast<double>(head_dim));
     double angle = static_cast<double>(position) * inverse_frequency;
     if (inverse) angle = -angle;
-    double sine, cosine;
-    sincos(angle, &sine, &cosine);
+    RopeAngle result;
+    sincos(angle, &result.sine, &result.cosine);
+    return result;
+}
+
+__device__ __forceinline__ void rope_apply(float& first, float& second, const RopeAngle& angle) {
     const float lhs = first;
     const float rhs = second;
-    first = static_cast<float>(lhs * cosine - rhs * sine);
-    second = static_cast<float>(rhs * cosine + lhs * sine);
+    first = static_cast<float>(lhs * angle.cosine - rhs * angle.sine);
+    second = static_cast<float>(rhs * angle.cosine + lhs * angle.sine);
+}
+
+__device__ __forceinline__ void rope_rotate(float& first, float& second, std::int64_t position,
+                                            std::int64_t pair, std::int64_t head_dim, double theta,
+                                            bool inverse) {
+    rope_apply(first, second, rope_angle(position, pair, head_dim, theta, inverse));
 }
 
 // 6-bit scale and minimum of sub-block `index` (resident_glimmer.cpp:178-186).

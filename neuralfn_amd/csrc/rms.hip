@@ -133,26 +133,6 @@ __global__ __launch_bounds__(kRmsThreads) void dual_rms_add_capture_kernel(
     }
 }
 
-// The halving tree over 256 partial sums with the additions in the same order
-// as the loop above: two steps through LDS, the last six inside the first wave
-// (lane t adds the value of lane t + stride, as the tree does).
-__device__ __forceinline__ float tree_total(float square_sum, float* partials) {
-    partials[threadIdx.x] = square_sum;
-    __syncthreads();
-    if (threadIdx.x < 128) partials[threadIdx.x] += partials[threadIdx.x + 128];
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        float value = partials[threadIdx.x] + partials[threadIdx.x + 64];
-#pragma unroll
-        for (int stride = 32; stride > 0; stride /= 2) value += __shfl_down(value, stride, 64);
-        if (threadIdx.x == 0) partials[0] = value;
-    }
-    __syncthreads();
-    const float total = partials[0];
-    __syncthreads();  // partials are reused by the next reduction
-    return total;
-}
-
 // Rows of up to 8192 columns: one workgroup of 1024 threads per row.  The sums
 // keep the 256-thread order above (sum t adds the squares of columns t, t + 256,
 // ... one after another, then the halving tree), but the loads are spread over
@@ -345,7 +325,7 @@ __global__ __launch_bounds__(kRmsThreads) void rms_resident_kernel(
 #pragma unroll
     for (int i = 0; i < kOwned; ++i) square_sum = fmaf(value[i], value[i], square_sum);
     const float inverse =
-        1.0f / sqrtf(tree_total(square_sum, partials) / static_cast<float>(width) + eps);
+        1.0f / sqrtf(rms_tree_total(square_sum, partials) / static_cast<float>(width) + eps);
 #pragma unroll
     for (int i = 0; i < kOwned; ++i) {
         const int column = threadIdx.x + i * kRmsThreads;
@@ -429,7 +409,14 @@ __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
     const float value = inside ? values[clamped[0]] : 0.0f;
     float scale[1];
     norm_scales(is_query ? query_weight : key_weight, clamped, scale);
-    const float inverse = 1.0f / sqrtf(tree_total(fmaf(value, value, 0.0f), partials) /
+    // the rotation's angle depends on the position alone: worked out while the loads above
+    // are in flight (an empty asm keeps the compiler from moving it behind the reduction)
+    RopeAngle angle{0.0, 1.0};
+    if (apply_rope && column < head_dim / 2) {
+        angle = rope_angle(position + row, column, head_dim, theta, false);
+        asm volatile("" : "+v"(angle.sine), "+v"(angle.cosine));
+    }
+    const float inverse = 1.0f / sqrtf(rms_tree_total(fmaf(value, value, 0.0f), partials) /
                                            static_cast<float>(head_dim) + eps);
     float result = __fmul_rn(__fmul_rn(value, inverse), scale[0]);
     if (is_query) result = __fmul_rn(result, query_scale);
@@ -457,7 +444,7 @@ __global__ __launch_bounds__(kRmsThreads) void qk_norm_scale_rope_kernel(
         const int first = interleaved ? 2 * column : column;
         const int second = interleaved ? 2 * column + 1 : column + half;
         float a = normalized[first], b = normalized[second];
-        rope_rotate(a, b, position + row, column, head_dim, theta, false);
+        rope_apply(a, b, angle);
         values[first] = a;
         values[second] = b;
         if (commits) {
