@@ -1304,6 +1304,11 @@ void launch_split(AttentionArguments a, std::int64_t query_rows, std::int64_t ti
     std::int64_t splits = compute_units() / groups;
     if (splits > (grouped ? kMaxSplits : kVectorSplits)) splits = grouped ? kMaxSplits : kVectorSplits;
     if (splits > tiles) splits = tiles;
+    // One query row: at least two tiles a share, two waves a workgroup.  A 2,048-key window
+    // in 16 shares of two waves takes 11.1 us with its merge, in 32 shares of one wave 12.1 us
+    // (12 or 24 shares: 11.7; 8: 11.9); long contexts and blocks are not touched by this
+    // (32,768 keys: 128 shares 15.1 us, 96: 15.4, 64: 17.1; a 16-row block: 8..24 shares 16.1 us).
+    if (query_rows == 1 && grouped && 2 * splits > tiles && tiles >= 4) splits = (tiles + 1) / 2;
     if (splits < 2) splits = 2;
     if (splits > partial_bytes / share_bytes) splits = partial_bytes / share_bytes;
     if (splits < 2) {

@@ -1179,8 +1179,12 @@ def test_verifier_block_through_two_layers_equals_token_at_a_time_decode(cuda, o
             g, weights, cache, exact_pending, exact_residual, pending_norm, position, workspace,
             True, attention_workspace, family="mmvq")
         pending_norm = weights.post_feedforward_norm
-    assert error(exact_residual.cpu().numpy(), np.stack(serial_hidden)) <= 2e-5
-    assert error(exact_pending.cpu().numpy(), np.stack(serial_down)) <= 2e-5
+    # (the two attention forms cut the keys into shares differently, so their partial sums meet
+    # in another order; where such a last-bit difference moves an activation across a
+    # quantization step of the next projection (16-bit codes: 3e-5 of a block's largest value)
+    # it grows to that size, and two layers leave about 1e-4)
+    assert error(exact_residual.cpu().numpy(), np.stack(serial_hidden)) <= 3e-4
+    assert error(exact_pending.cpu().numpy(), np.stack(serial_down)) <= 3e-4
 
     # the projections of a block (fp16 weights and activations on the matrix cores, 11
     # significant bits each) and of one token (integer codes against 16-bit activation codes)
