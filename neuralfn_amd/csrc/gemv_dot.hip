@@ -650,8 +650,9 @@ void launch_pairs(const ProjectionSet& set, const float* input, hipStream_t stre
     const PackedPointers packed = pack_pointers(data);
     const std::int64_t blocks = set.input_dim >> 8;
     const std::size_t lds = static_cast<std::size_t>(token_image_bytes_host(blocks));
-    // workgroups as for the 2 x pairs weight rows of the launch
-    std::int64_t groups = decode_groups(2 * pairs, kDotWaves);
+    // workgroups as for the 2 x pairs weight rows of the launch, two a compute unit at most (gate
+    // and up of 16,384 rows: 24.2 us with two, 24.9 with four, 25.5 with one, 26.7 with six)
+    std::int64_t groups = decode_groups(2 * pairs, kDotWaves, 2);
     if (groups > pairs) groups = pairs;
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(groups), 1), dim3(kDotThreads), lds,
