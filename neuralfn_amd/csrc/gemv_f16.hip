@@ -134,6 +134,22 @@ __device__ __forceinline__ f16x8 as_operand(std::uint32_t a, std::uint32_t b, st
 template <std::uint32_t ENC>
 struct PackedBlock;
 
+// Pieces of a row's packed bytes where a wave has laid them out in LDS (load_tile() below):
+// aligned to two bytes only (a Q6_K block is 210 bytes long, and a tensor may start anywhere).
+struct __attribute__((packed, aligned(2))) TilePiece16 {
+    std::uint32_t v[4];
+};
+struct __attribute__((packed, aligned(2))) TilePiece8 {
+    std::uint32_t v[2];
+};
+struct __attribute__((packed, aligned(2))) TilePiece4 {
+    std::uint32_t v;
+};
+__device__ __forceinline__ u32x4 tile_read16(const std::uint8_t* at) {
+    const TilePiece16 piece = *reinterpret_cast<const TilePiece16*>(at);
+    return u32x4{piece.v[0], piece.v[1], piece.v[2], piece.v[3]};
+}
+
 // The value of the lane whose number times four is `source` (any permutation of the lanes).
 __device__ __forceinline__ std::uint32_t from_lane(int source, std::uint32_t value) {
     return static_cast<std::uint32_t>(__builtin_amdgcn_ds_bpermute(source, static_cast<int>(value)));
@@ -159,6 +175,12 @@ struct PackedBlock<kEncQ4K> {
         const std::uint32_t mine = row + 16 + 16 * j;
         piece[0] = *reinterpret_cast<GlobalVec>(block + mine);
         piece[1] = *reinterpret_cast<GlobalVec>(block + mine + 64);
+    }
+    // the same registers from the block at `at` in LDS
+    __device__ __forceinline__ void load_tile(const std::uint8_t* at, int j) {
+        header = tile_read16(at);
+        piece[0] = tile_read16(at + 16 + 16 * j);
+        piece[1] = tile_read16(at + 80 + 16 * j);
     }
     __device__ __forceinline__ void prepare(int j) {
         scales[0].bits(header, j >> 1);
@@ -200,6 +222,12 @@ struct PackedBlock<kEncQ5K> {
         const std::uint32_t mine = row + 48 + 16 * j;
         piece[0] = *reinterpret_cast<GlobalVec>(block + mine);
         piece[1] = *reinterpret_cast<GlobalVec>(block + mine + 64);
+    }
+    __device__ __forceinline__ void load_tile(const std::uint8_t* at, int j) {
+        header = tile_read16(at);
+        fifth = tile_read16(at + 16 + 16 * (j & 1));
+        piece[0] = tile_read16(at + 48 + 16 * j);
+        piece[1] = tile_read16(at + 112 + 16 * j);
     }
     __device__ __forceinline__ void prepare(int j) {
         scales[0].bits(header, j >> 1);
@@ -263,6 +291,16 @@ struct PackedBlock<kEncQ6K> {
         sub_scales[1] = s[1];
         d_bits = *reinterpret_cast<GlobalHalf>(block + (row + 208));
     }
+    __device__ __forceinline__ void load_tile(const std::uint8_t* at, int j) {
+        const int n = j >> 1, h = j & 1;
+        low_a = tile_read16(at + 64 * n + 16 * h);
+        low_b = tile_read16(at + 64 * n + 16 * h + 32);
+        top = tile_read16(at + 128 + 32 * n + 16 * h);
+        const TilePiece8 s = *reinterpret_cast<const TilePiece8*>(at + 192 + 8 * n);
+        sub_scales[0] = s.v[0];
+        sub_scales[1] = s.v[1];
+        d_bits = *reinterpret_cast<const std::uint16_t*>(at + 208);
+    }
     __device__ __forceinline__ void change_lanes(int source) {
         low_a = from_lane(source, low_a);
         low_b = from_lane(source, low_b);
@@ -310,6 +348,20 @@ struct PackedBlock<kEncQ8_0> {
     static constexpr int kBytes = 272;
     static constexpr bool kQuadFetch = false;
     __device__ __forceinline__ void change_lanes(int) {}
+    __device__ __forceinline__ void load_tile(const std::uint8_t* at, int j) {
+        const std::uint8_t* mine = at + 68 * j;
+        std::uint32_t word[17];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const u32x4 four = tile_read16(mine + 16 * q);
+            word[4 * q] = four[0];
+            word[4 * q + 1] = four[1];
+            word[4 * q + 2] = four[2];
+            word[4 * q + 3] = four[3];
+        }
+        word[16] = reinterpret_cast<const TilePiece4*>(mine + 64)->v;
+        take(word);
+    }
     std::uint32_t codes[2][8];
     std::uint32_t d_bits[2];
     f16x2 scale[2];
@@ -329,6 +381,9 @@ struct PackedBlock<kEncQ8_0> {
             word[4 * q + 3] = four[3];
         }
         word[16] = *reinterpret_cast<GlobalWord>(block + (mine + 64));
+        take(word);
+    }
+    __device__ __forceinline__ void take(const std::uint32_t (&word)[17]) {
         d_bits[0] = word[0] & 0xffffu;
         d_bits[1] = word[8] >> 16;
 #pragma unroll
@@ -391,15 +446,67 @@ constexpr int kGroupTiles = 2;  // tiles a workgroup accumulates side by side
 // compute from the two outputs: one [rows, output_dim] result instead of two.
 enum Mode : int { kStore = 0, kArgmax = 1, kPairs = 2 };
 
-template <std::uint32_t ENC, int MODE>
+// RING: how the packed weights reach the lanes.  In the plain form every lane loads the bytes
+// it decodes, 16 rows x (a quarter of) one block per instruction: a wave instruction touches
+// 16 to 32 cache lines for 1 KB, and the launch is bound by the rate at which the vector
+// cache looks lines up (the Q6_K lm_head read this way and nothing else: 4.05 TB/s).  In the
+// RING form a load instruction brings whole blocks of several rows, every row's block as
+// neighbouring 16-byte pieces (5.4 to 5.7 TB/s for the same bytes), and brings them straight
+// into LDS (global_load_lds_dwordx4: lane l's 16 bytes land at the instruction's LDS address
+// + 16 l; the source may start at any byte), into a ring of block steps that belongs to the
+// wave alone; no register waits for a load.  Every lane then reads its row's pieces from
+// LDS, where two-byte alignment costs nothing.  The arithmetic and its order are those of
+// the plain form.
+template <std::uint32_t ENC>
+struct Ring {
+    static constexpr int kBytes = PackedBlock<ENC>::kBytes;
+    static constexpr int kRowLanes = (kBytes + 15) / 16;  // 16-byte pieces of a row's block
+    static constexpr int kRowPitch = 16 * kRowLanes;      // a row's place in a stage
+    // bytes a row's last piece reaches past its block (Q6_K: 14): the last piece of a
+    // projection's very last block is not loaded this way
+    static constexpr int kOver = kRowPitch - kBytes;
+    static constexpr int kRowsPerLoad = kWave / kRowLanes;
+    static constexpr int kLoads = (kTileRows + kRowsPerLoad - 1) / kRowsPerLoad;  // per block step
+    static constexpr int kStageBytes = kTileRows * kRowPitch;
+    // as many stages as fit beside the kernel's other LDS (36 KB) in the 160 KB of a unit
+    static constexpr int kFit = 120 * 1024 / (kWaves * kStageBytes);
+    static constexpr int kStages = kFit < 6 ? kFit : 6;
+    static constexpr unsigned kLdsBytes = kWaves * kStages * kStageBytes;
+};
+
+// 16 bytes per lane from `source` (this lane's) to the LDS address `target` (uniform) + 16 x
+// lane; counted by vmcnt like any load.  Written out as an instruction because the compiler
+// holds every later LDS read back until all loads of this kind have landed, which would leave
+// the ring one stage deep; the kernel waits by count itself.
+__device__ __forceinline__ void load_to_lds(const __attribute__((address_space(1))) std::uint8_t* source,
+                                            std::uint8_t* target) {
+    const std::uint32_t lds_address = static_cast<std::uint32_t>(
+        reinterpret_cast<std::uintptr_t>((__attribute__((address_space(3))) std::uint8_t*)target));
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(source), "s"(lds_address)
+                 : "memory", "m0");
+}
+
+// A tile of 16 weight rows as both the fetching and the multiplying side see it (uniform).
+struct TileShape {
+    const __attribute__((address_space(1))) std::uint8_t* base;  // its first row
+    std::uint32_t stride;  // bytes between rows
+    int last;              // last row that exists
+    int final_row;         // the projection's last row if it is one of the tile's, else -1
+};
+
+template <std::uint32_t ENC, int MODE, bool RING>
 __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const std::uint8_t* __restrict__ image, const float* __restrict__ inverse_scale, int tokens,
     std::uint32_t total_tiles, int input_dim, LmHeadCandidate* __restrict__ candidates,
     ProjectionSet set) {
     using Block = PackedBlock<ENC>;
+    using Lds = Ring<ENC>;
     constexpr bool ARGMAX = MODE == kArgmax;
     constexpr bool PAIRS = MODE == kPairs;
     __shared__ float partial[2 * kGroupTiles * kWaves * kWave * 4];
+    extern __shared__ __attribute__((aligned(16))) std::uint8_t ring_lds[];  // RING: [wave][stage][row][kRowPitch]
 
     const int lane = threadIdx.x & 63;
     // the wave index is uniform; saying so keeps tile bookkeeping in scalar registers
@@ -407,8 +514,13 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     const int i = lane & 15;
     const int j = lane >> 4;
     const int blocks = input_dim >> 8;
-    const int begin = blocks * wave / kWaves;
-    const int end = blocks * (wave + 1) / kWaves;
+    // K is cut into kWaves shares of blocks * share / kWaves .. blocks * (share + 1) / kWaves;
+    // which wave takes which share is free (sums meet in share order).  Waves w and w + 4 run
+    // on one SIMD, and with this choice the shares that are one block longer than the others
+    // spread over the four SIMDs for every remainder of blocks / 8 (26 blocks: shares 3 and 7).
+    const int share = RING ? (0x63571240 >> (4 * wave)) & 7 : wave;
+    const int begin = blocks * share / kWaves;
+    const int end = blocks * (share + 1) / kWaves;
     const int count = end - begin;
     const int chunks = ((blocks + kWaves - 1) / kWaves + kDepth - 1) / kDepth;  // the same for every wave
 
@@ -444,9 +556,27 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         static_cast<int>((total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x);
     // (kPairs: total_tiles counts the tiles of one projection and a group is one of them twice)
     const int groups = PAIRS ? tile_count : (tile_count + kGroupTiles - 1) / kGroupTiles;
+    auto tiles_of_group = [&](int group) {
+        return PAIRS ? kGroupTiles : min(kGroupTiles, tile_count - group * kGroupTiles);
+    };
+    // tile `slot` of group `group` (both exist)
+    auto tile_shape = [&](int group, int slot) {
+        const int index = PAIRS ? group : group * kGroupTiles + slot;
+        const std::uint32_t tile = blockIdx.x + static_cast<std::uint32_t>(index) * gridDim.x;
+        const Projection op = PAIRS ? pick(set, slot) : tile_projection(set, tile);
+        const std::int64_t row0 = static_cast<std::int64_t>(tile - (PAIRS ? 0u : op.first_tile)) * kTileRows;
+        TileShape shape;
+        shape.last = static_cast<int>(min(static_cast<std::int64_t>(kTileRows - 1), op.output_dim - 1 - row0));
+        shape.base = (GlobalBytes)op.data + row0 * op.row_stride;
+        shape.stride = static_cast<std::uint32_t>(op.row_stride);
+        shape.final_row = row0 + shape.last == op.output_dim - 1 ? shape.last : -1;
+        return shape;
+    };
 
     // Every wave walks the same stream of (group, chunk, tile of the group, step)
-    // in uniform control flow (a group's tiles: kGroupTiles, fewer in the last group).  Weight loads run kDepth steps ahead; they are
+    // in uniform control flow (a group's tiles: kGroupTiles, fewer in the last group).
+    //
+    // Plain form: weight loads run kDepth steps ahead; they are
     // unconditional (a step without work reads the first bytes of the first
     // projection, one line for the whole wave), so a step waits for nothing but
     // its own.  The fetch cursor walks the same stream, one tile ahead.
@@ -454,8 +584,9 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     // read neighbouring bytes of one row; the matrix instruction wants quarter l / 16 of row
     // l % 16 in lane l, and a step's registers change lanes before use (Q6_K at 16 rows,
     // 6,656 -> 202,048: 299 -> 234 us; the formats with aligned blocks lose 3-7 % to it).
-    const int load_row = Block::kQuadFetch ? lane >> 2 : i;
-    const int load_quarter = Block::kQuadFetch ? lane & 3 : j;
+    constexpr bool QUADS = Block::kQuadFetch && !RING;
+    const int load_row = QUADS ? lane >> 2 : i;
+    const int load_quarter = QUADS ? lane & 3 : j;
     const int taken_from = 4 * (4 * i + j);  // the lane that fetched this lane's row and quarter, x 4
     int fetch_group = 0, fetch_chunk = 0, fetch_slot = 0;
     GlobalBytes fetch_tile = nullptr;  // first row of the tile being fetched (uniform)
@@ -464,12 +595,9 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     auto fetch_setup = [&]() {
         const int index = PAIRS ? fetch_group : fetch_group * kGroupTiles + fetch_slot;
         fetch_live = fetch_group < groups && index < tile_count;
-        const std::uint32_t tile = blockIdx.x + static_cast<std::uint32_t>(fetch_live ? index : 0) * gridDim.x;
-        const Projection op = PAIRS ? pick(set, fetch_slot) : tile_projection(set, tile);
-        const std::int64_t row0 = static_cast<std::int64_t>(tile - (PAIRS ? 0u : op.first_tile)) * kTileRows;
-        const int last = static_cast<int>(min(static_cast<std::int64_t>(kTileRows - 1), op.output_dim - 1 - row0));
-        fetch_tile = (GlobalBytes)op.data + row0 * op.row_stride;
-        fetch_row = static_cast<std::uint32_t>(min(load_row, last)) * static_cast<std::uint32_t>(op.row_stride);  // rows past the end repeat the last one
+        const TileShape shape = fetch_live ? tile_shape(fetch_group, fetch_slot) : tile_shape(0, 0);
+        fetch_tile = shape.base;
+        fetch_row = static_cast<std::uint32_t>(min(load_row, shape.last)) * shape.stride;  // rows past the end repeat the last one
     };
     auto fetch_advance = [&]() {  // to the next (group, chunk, tile of the group)
         if (++fetch_slot >= (PAIRS ? kGroupTiles : min(kGroupTiles, tile_count - fetch_group * kGroupTiles))) {
@@ -481,7 +609,6 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         }
         fetch_setup();
     };
-    fetch_setup();
     auto fetch = [&](PackedBlock<ENC>& stage, int s) {
         const int local = fetch_chunk * kDepth + s;  // block of this wave's K range
         const bool work = fetch_live && local < count;
@@ -489,10 +616,98 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
             ? fetch_tile + static_cast<std::int64_t>(begin + local) * Block::kBytes : (GlobalBytes)set.op[0].data;
         stage.load(source, work ? fetch_row : 0u, work ? load_quarter : 0);
     };
-    PackedBlock<ENC> stages[kDepth];
+    PackedBlock<ENC> stages[RING ? 1 : kDepth];
+
+    // RING form: a cursor over the steps that have work runs kStages - 1 of them ahead.  A
+    // step's kLoads instructions each bring the block of kRowsPerLoad rows; lane l of one has
+    // piece l % kRowLanes of row l / kRowLanes.  Past the last step the cursor keeps issuing
+    // (the first 16 bytes of the first projection), so that the count of loads in flight that
+    // a step waits by stays what it is.
+    std::uint8_t* const my_ring = ring_lds + wave * (Lds::kStages * Lds::kStageBytes);
+    const int piece_row = lane / Lds::kRowLanes;
+    const int piece = lane - piece_row * Lds::kRowLanes;
+    int ring_group = 0, ring_chunk = 0, ring_slot = 0, ring_step = -1;
+    int ring_stage = 0;  // where the next step lands
+    bool ring_done = !RING || groups == 0;
+    TileShape ring_tile{};
+    auto ring_next = [&]() {  // to the next step with work
+        while (!ring_done) {
+            if (++ring_step < min(kDepth, count - ring_chunk * kDepth)) return;
+            ring_step = -1;
+            if (++ring_slot >= tiles_of_group(ring_group)) {
+                ring_slot = 0;
+                if (++ring_chunk == chunks) {
+                    ring_chunk = 0;
+                    ++ring_group;
+                }
+            }
+            if (ring_group >= groups) {
+                ring_done = true;
+            } else {
+                ring_tile = tile_shape(ring_group, ring_slot);
+            }
+        }
+    };
+    auto ring_issue = [&]() {
+        // the reads of the step that lay in this stage have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        std::uint8_t* const stage = my_ring + ring_stage * Lds::kStageBytes;
+        ring_stage = ring_stage + 1 == Lds::kStages ? 0 : ring_stage + 1;
+        const bool real = !ring_done;
+        const int block = begin + ring_chunk * kDepth + ring_step;
+        const GlobalBytes base = real
+            ? ring_tile.base + static_cast<std::int64_t>(block) * Block::kBytes : (GlobalBytes)set.op[0].data;
+        const std::uint32_t stride = real ? ring_tile.stride : 0u;
+        const int last = real ? ring_tile.last : 0;
+        const int final_row = Lds::kOver > 0 && real && block == blocks - 1 ? ring_tile.final_row : -1;
+        const std::uint32_t mine = real ? 16u * piece : 0u;
 #pragma unroll
-    for (int s = 0; s < kDepth; ++s) fetch(stages[s], s);
-    fetch_advance();
+        for (int q = 0; q < Lds::kLoads; ++q) {
+            const int row = q * Lds::kRowsPerLoad + piece_row;
+            const int source = min(row, last);  // rows past the end repeat the last one
+            const bool past = source == final_row && piece == Lds::kRowLanes - 1;
+            if (piece_row < Lds::kRowsPerLoad && row < kTileRows && !past) {
+                load_to_lds(base + (static_cast<std::uint32_t>(source) * stride + mine),
+                            stage + q * Lds::kRowsPerLoad * Lds::kRowPitch);
+            }
+        }
+        if constexpr (Lds::kOver > 0) {
+            if (final_row >= 0) {  // the bytes of that last piece that exist, for every row that is the final one
+                static_assert(Lds::kOver == 14, "the last piece holds two bytes of the block");
+                typedef const __attribute__((address_space(1))) std::uint16_t* GlobalHalf;
+                if (lane < kTileRows && min(lane, last) == final_row) {
+                    const std::uint16_t two = *reinterpret_cast<GlobalHalf>(
+                        base + (static_cast<std::uint32_t>(final_row) * stride + Block::kBytes - 2));
+                    *reinterpret_cast<std::uint16_t*>(stage + lane * Lds::kRowPitch + Block::kBytes - 2) = two;
+                }
+            }
+        }
+        ring_next();
+    };
+    int read_stage = 0;  // where the next step to multiply waits
+
+    // RING: the step behind the one being multiplied, read from its stage while that one's
+    // matrix instructions run
+    PackedBlock<ENC> ahead;
+    auto ring_read_ahead = [&]() {
+        ring_issue();
+        // all but the loads of the kStages - 1 steps behind the next one have landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(Lds::kLoads * (Lds::kStages - 1)) : "memory");
+        ahead.load_tile(my_ring + read_stage * Lds::kStageBytes + i * Lds::kRowPitch, j);
+        read_stage = read_stage + 1 == Lds::kStages ? 0 : read_stage + 1;
+    };
+    if constexpr (RING) {
+        if (!ring_done) ring_tile = tile_shape(0, 0);
+        ring_next();
+#pragma unroll
+        for (int s = 0; s < Lds::kStages - 1; ++s) ring_issue();
+        ring_read_ahead();
+    } else {
+        fetch_setup();
+#pragma unroll
+        for (int s = 0; s < kDepth; ++s) fetch(stages[s], s);
+        fetch_advance();
+    }
 
     // ARGMAX: the running best of every (lane, result register) of the waves that add up tiles
     // lives in LDS between tiles, so that the main loop holds no register for it
@@ -509,7 +724,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         f32x4 acc[kGroupTiles];
 #pragma unroll
         for (int t = 0; t < kGroupTiles; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        const int group_tiles = PAIRS ? kGroupTiles : min(kGroupTiles, tile_count - group * kGroupTiles);
+        const int group_tiles = tiles_of_group(group);
         for (int chunk = 0; chunk < chunks; ++chunk) {
             if (chunks > 1 || group == 0) load_fragments(chunk);
             const int chunk_count = min(kDepth, count - chunk * kDepth);  // this wave's blocks of the chunk
@@ -518,10 +733,14 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                 if (t >= group_tiles) break;
 #pragma unroll
                 for (int s = 0; s < kDepth; ++s) {
-                    PackedBlock<ENC>& stage = stages[s];
+                    PackedBlock<ENC>& stage = stages[RING ? 0 : s];
                     if (s < chunk_count) {
                         const f16x8 (&a)[8] = fragments[s];
-                        if constexpr (Block::kQuadFetch) stage.change_lanes(taken_from);
+                        if constexpr (RING) {
+                            stage = ahead;
+                            ring_read_ahead();
+                        }
+                        if constexpr (QUADS) stage.change_lanes(taken_from);
                         stage.prepare(j);
                         f32x4 sum = acc[t];
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[0], stage.template operand<0>(), sum, 0, 0, 0);
@@ -534,9 +753,9 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], stage.template operand<7>(), sum, 0, 0, 0);
                         acc[t] = sum;
                     }
-                    fetch(stage, s);
+                    if constexpr (!RING) fetch(stage, s);
                 }
-                fetch_advance();
+                if constexpr (!RING) fetch_advance();
             }
         }
         // Cross-wave sums in wave order, wave t adds up tile t of the group; the
@@ -545,7 +764,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
 #pragma unroll
         for (int t = 0; t < kGroupTiles; ++t) {
             if (t < group_tiles) {
-                *reinterpret_cast<f32x4*>(buffer + ((t * kWaves + wave) * kWave + lane) * 4) = acc[t];
+                *reinterpret_cast<f32x4*>(buffer + ((t * kWaves + share) * kWave + lane) * 4) = acc[t];
             }
         }
         __syncthreads();
@@ -608,6 +827,8 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
             }
         }
     }
+    // RING: the loads issued past the last step still write this workgroup's LDS
+    if constexpr (RING) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if constexpr (ARGMAX) {
         if (wave < kGroupTiles) {  // the waves that added up tiles
             const f32x4 mine_value = best_values[wave * kWave + lane];
@@ -647,6 +868,15 @@ std::uint32_t grid_of(std::uint32_t tiles, bool argmax) {
     return tiles < slots ? tiles : slots;
 }
 
+// The RING form reads a whole window of Ring::kRowPitch bytes around every block: a
+// projection of one block alone (one row of 256 columns) is shorter than that.
+bool ring_form(const ProjectionSet& set) {
+    for (int index = 0; index < set.count; ++index) {
+        if (set.op[index].output_dim * (set.input_dim / 256) < 2) return false;
+    }
+    return true;
+}
+
 // `candidates` non-null: the lm_head form (one projection), which returns its workgroup count.
 template <std::uint32_t ENC>
 std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, const float* inverse_scale,
@@ -657,14 +887,25 @@ std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, cons
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
     const std::uint32_t grid = grid_of(tiles, candidates != nullptr);
-    if (candidates != nullptr) {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax>), dim3(grid), dim3(kThreads), 0, stream, image,
-                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
-                           set);
+    if (ring_form(set)) {
+        constexpr unsigned kLds = Ring<ENC>::kLdsBytes;
+        if (candidates != nullptr) {
+            hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax, true>), dim3(grid), dim3(kThreads), kLds,
+                               stream, image, inverse_scale, tokens, tiles,
+                               static_cast<int>(set.input_dim), candidates, set);
+        } else {
+            hipLaunchKernelGGL((gemv_f16_kernel<ENC, kStore, true>), dim3(grid), dim3(kThreads), kLds,
+                               stream, image, inverse_scale, tokens, tiles,
+                               static_cast<int>(set.input_dim), candidates, set);
+        }
+    } else if (candidates != nullptr) {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax, false>), dim3(grid), dim3(kThreads), 0, stream,
+                           image, inverse_scale, tokens, tiles, static_cast<int>(set.input_dim),
+                           candidates, set);
     } else {
-        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kStore>), dim3(grid), dim3(kThreads), 0, stream, image,
-                           inverse_scale, tokens, tiles, static_cast<int>(set.input_dim), candidates,
-                           set);
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kStore, false>), dim3(grid), dim3(kThreads), 0, stream,
+                           image, inverse_scale, tokens, tiles, static_cast<int>(set.input_dim),
+                           candidates, set);
     }
     return grid;
 }
@@ -675,9 +916,15 @@ void launch_pair(const ProjectionSet& set, const std::uint8_t* image, const floa
                  int tokens, hipStream_t stream) {
     const std::uint32_t tiles =
         static_cast<std::uint32_t>((set.op[0].output_dim + kTileRows - 1) / kTileRows);
-    hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs>), dim3(grid_of(tiles, false)), dim3(kThreads), 0,
-                       stream, image, inverse_scale, tokens, tiles, static_cast<int>(set.input_dim),
-                       static_cast<LmHeadCandidate*>(nullptr), set);
+    if (ring_form(set)) {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs, true>), dim3(grid_of(tiles, false)), dim3(kThreads),
+                           Ring<ENC>::kLdsBytes, stream, image, inverse_scale, tokens, tiles,
+                           static_cast<int>(set.input_dim), static_cast<LmHeadCandidate*>(nullptr), set);
+    } else {
+        hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs, false>), dim3(grid_of(tiles, false)), dim3(kThreads),
+                           0, stream, image, inverse_scale, tokens, tiles,
+                           static_cast<int>(set.input_dim), static_cast<LmHeadCandidate*>(nullptr), set);
+    }
 }
 
 std::uint32_t launch_by_encoding(const ProjectionSet& group, std::uint32_t encoding,
