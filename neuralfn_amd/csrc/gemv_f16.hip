@@ -622,18 +622,22 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     // step's kLoads instructions each bring the block of kRowsPerLoad rows; lane l of one has
     // piece l % kRowLanes of row l / kRowLanes.  Past the last step the cursor keeps issuing
     // (the first 16 bytes of the first projection), so that the count of loads in flight that
-    // a step waits by stays what it is.
+    // a step waits by stays what it is.  What a step needs is kept ready: a pointer that moves
+    // on by a block, and every lane's offsets from it, which change with the tile only.
     std::uint8_t* const my_ring = ring_lds + wave * (Lds::kStages * Lds::kStageBytes);
     const int piece_row = lane / Lds::kRowLanes;
     const int piece = lane - piece_row * Lds::kRowLanes;
-    int ring_group = 0, ring_chunk = 0, ring_slot = 0, ring_step = -1;
-    int ring_stage = 0;  // where the next step lands
-    bool ring_done = !RING || groups == 0;
-    TileShape ring_tile{};
-    auto ring_next = [&]() {  // to the next step with work
-        while (!ring_done) {
-            if (++ring_step < min(kDepth, count - ring_chunk * kDepth)) return;
-            ring_step = -1;
+    int ring_group = 0, ring_chunk = 0, ring_slot = -1;
+    int ring_step = 0, ring_steps = 0;  // of the cursor's (tile, chunk)
+    int ring_final_step = -1;           // the step that is the projection's very last block, if one is
+    int ring_last = 0, ring_final_row = -1;
+    std::uint32_t ring_stride = 0;
+    int ring_stage = 0;                 // where the next step lands
+    GlobalBytes ring_ptr = (GlobalBytes)set.op[0].data;  // row 0 of the tile, the step's block
+    std::uint32_t ring_bump = 0;                         // what a step moves it by
+    std::uint32_t ring_offset[Lds::kLoads];              // this lane's piece in each instruction
+    auto ring_enter = [&]() {  // the next (tile, chunk) in which this wave has steps
+        for (;;) {
             if (++ring_slot >= tiles_of_group(ring_group)) {
                 ring_slot = 0;
                 if (++ring_chunk == chunks) {
@@ -641,11 +645,33 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                     ++ring_group;
                 }
             }
-            if (ring_group >= groups) {
-                ring_done = true;
-            } else {
-                ring_tile = tile_shape(ring_group, ring_slot);
+            if (ring_group >= groups) {  // done: the same 16 bytes from now on
+                ring_ptr = (GlobalBytes)set.op[0].data;
+                ring_bump = 0;
+                ring_step = 0;
+                ring_steps = 0x7fffffff;
+                ring_final_step = -1;
+#pragma unroll
+                for (int q = 0; q < Lds::kLoads; ++q) ring_offset[q] = 0;
+                return;
             }
+            ring_steps = min(kDepth, count - ring_chunk * kDepth);
+            if (ring_steps > 0) break;
+        }
+        const TileShape shape = tile_shape(ring_group, ring_slot);
+        const int first = begin + ring_chunk * kDepth;
+        ring_ptr = shape.base + static_cast<std::int64_t>(first) * Block::kBytes;
+        ring_bump = Block::kBytes;
+        ring_step = 0;
+        ring_last = shape.last;
+        ring_final_row = shape.final_row;
+        ring_stride = shape.stride;
+        ring_final_step =
+            Lds::kOver > 0 && shape.final_row >= 0 && first + ring_steps == blocks ? ring_steps - 1 : -1;
+#pragma unroll
+        for (int q = 0; q < Lds::kLoads; ++q) {
+            const int row = q * Lds::kRowsPerLoad + piece_row;  // (rows past the end repeat the last one)
+            ring_offset[q] = static_cast<std::uint32_t>(min(row, shape.last)) * shape.stride + 16u * piece;
         }
     };
     auto ring_issue = [&]() {
@@ -653,36 +679,37 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         std::uint8_t* const stage = my_ring + ring_stage * Lds::kStageBytes;
         ring_stage = ring_stage + 1 == Lds::kStages ? 0 : ring_stage + 1;
-        const bool real = !ring_done;
-        const int block = begin + ring_chunk * kDepth + ring_step;
-        const GlobalBytes base = real
-            ? ring_tile.base + static_cast<std::int64_t>(block) * Block::kBytes : (GlobalBytes)set.op[0].data;
-        const std::uint32_t stride = real ? ring_tile.stride : 0u;
-        const int last = real ? ring_tile.last : 0;
-        const int final_row = Lds::kOver > 0 && real && block == blocks - 1 ? ring_tile.final_row : -1;
-        const std::uint32_t mine = real ? 16u * piece : 0u;
+        if (ring_step != ring_final_step) {
 #pragma unroll
-        for (int q = 0; q < Lds::kLoads; ++q) {
-            const int row = q * Lds::kRowsPerLoad + piece_row;
-            const int source = min(row, last);  // rows past the end repeat the last one
-            const bool past = source == final_row && piece == Lds::kRowLanes - 1;
-            if (piece_row < Lds::kRowsPerLoad && row < kTileRows && !past) {
-                load_to_lds(base + (static_cast<std::uint32_t>(source) * stride + mine),
-                            stage + q * Lds::kRowsPerLoad * Lds::kRowPitch);
-            }
-        }
-        if constexpr (Lds::kOver > 0) {
-            if (final_row >= 0) {  // the bytes of that last piece that exist, for every row that is the final one
-                static_assert(Lds::kOver == 14, "the last piece holds two bytes of the block");
-                typedef const __attribute__((address_space(1))) std::uint16_t* GlobalHalf;
-                if (lane < kTileRows && min(lane, last) == final_row) {
-                    const std::uint16_t two = *reinterpret_cast<GlobalHalf>(
-                        base + (static_cast<std::uint32_t>(final_row) * stride + Block::kBytes - 2));
-                    *reinterpret_cast<std::uint16_t*>(stage + lane * Lds::kRowPitch + Block::kBytes - 2) = two;
+            for (int q = 0; q < Lds::kLoads; ++q) {
+                // the lanes of instruction q that have a row of the tile
+                const int rows = min(kTileRows - q * Lds::kRowsPerLoad, Lds::kRowsPerLoad);  // (a constant)
+                if (lane < rows * Lds::kRowLanes) {
+                    load_to_lds(ring_ptr + ring_offset[q], stage + q * Lds::kRowsPerLoad * Lds::kRowPitch);
                 }
             }
+        } else if constexpr (Lds::kOver > 0) {
+            // The projection's very last block: its last piece would reach past the projection.
+            // The lanes that have it stand back, and the bytes of it that exist go by hand
+            // (into every row that repeats the final one).
+            static_assert(Lds::kOver == 14 || Lds::kOver == 0, "the last piece holds two bytes of the block");
+#pragma unroll
+            for (int q = 0; q < Lds::kLoads; ++q) {
+                const int row = q * Lds::kRowsPerLoad + piece_row;
+                const bool past = min(row, ring_last) == ring_final_row && piece == Lds::kRowLanes - 1;
+                if (piece_row < Lds::kRowsPerLoad && row < kTileRows && !past) {
+                    load_to_lds(ring_ptr + ring_offset[q], stage + q * Lds::kRowsPerLoad * Lds::kRowPitch);
+                }
+            }
+            typedef const __attribute__((address_space(1))) std::uint16_t* GlobalHalf;
+            if (lane < kTileRows && min(lane, ring_last) == ring_final_row) {
+                const std::uint16_t two = *reinterpret_cast<GlobalHalf>(
+                    ring_ptr + (static_cast<std::uint32_t>(ring_final_row) * ring_stride + Block::kBytes - 2));
+                *reinterpret_cast<std::uint16_t*>(stage + lane * Lds::kRowPitch + Block::kBytes - 2) = two;
+            }
         }
-        ring_next();
+        ring_ptr += ring_bump;
+        if (++ring_step == ring_steps) ring_enter();
     };
     int read_stage = 0;  // where the next step to multiply waits
 
@@ -697,8 +724,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         read_stage = read_stage + 1 == Lds::kStages ? 0 : read_stage + 1;
     };
     if constexpr (RING) {
-        if (!ring_done) ring_tile = tile_shape(0, 0);
-        ring_next();
+        ring_enter();
 #pragma unroll
         for (int s = 0; s < Lds::kStages - 1; ++s) ring_issue();
         ring_read_ahead();
@@ -733,6 +759,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                 if (t >= group_tiles) break;
 #pragma unroll
                 for (int s = 0; s < kDepth; ++s) {
+                    if (RING && s >= chunk_count) break;  // (the plain form fetches in every step)
                     PackedBlock<ENC>& stage = stages[RING ? 0 : s];
                     if (s < chunk_count) {
                         const f16x8 (&a)[8] = fragments[s];
