@@ -469,6 +469,8 @@ struct Ring {
     static constexpr int kLoads = (kTileRows + kRowsPerLoad - 1) / kRowsPerLoad;  // per block step
     static constexpr int kStageBytes = kTileRows * kRowPitch;
     // as many stages as fit beside the kernel's other LDS (36 KB) in the 160 KB of a unit
+    // (a fifth Q6_K stage in place of the second buffer of partial sums, which costs a second
+    // barrier per group: the lm_head at 16 rows 227 -> 236 us)
     static constexpr int kFit = 120 * 1024 / (kWaves * kStageBytes);
     static constexpr int kStages = kFit < 6 ? kFit : 6;
     static constexpr unsigned kLdsBytes = kWaves * kStages * kStageBytes;
@@ -717,7 +719,6 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     // matrix instructions run
     PackedBlock<ENC> ahead;
     auto ring_read_ahead = [&]() {
-        ring_issue();
         // all but the loads of the kStages - 1 steps behind the next one have landed
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(Lds::kLoads * (Lds::kStages - 1)) : "memory");
         ahead.load_tile(my_ring + read_stage * Lds::kStageBytes + i * Lds::kRowPitch, j);
@@ -726,7 +727,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
     if constexpr (RING) {
         ring_enter();
 #pragma unroll
-        for (int s = 0; s < Lds::kStages - 1; ++s) ring_issue();
+        for (int s = 0; s < Lds::kStages; ++s) ring_issue();
         ring_read_ahead();
     } else {
         fetch_setup();
@@ -765,7 +766,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                         const f16x8 (&a)[8] = fragments[s];
                         if constexpr (RING) {
                             stage = ahead;
-                            ring_read_ahead();
+                            ring_issue();  // into the stage that `ahead` came from
                         }
                         if constexpr (QUADS) stage.change_lanes(taken_from);
                         stage.prepare(j);
@@ -776,6 +777,9 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[3], stage.template operand<3>(), sum, 0, 0, 0);
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[4], stage.template operand<4>(), sum, 0, 0, 0);
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[5], stage.template operand<5>(), sum, 0, 0, 0);
+                        // RING: the next step's registers, as late as its LDS reads still hide
+                        // behind this step's last instructions
+                        if constexpr (RING) ring_read_ahead();
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[6], stage.template operand<6>(), sum, 0, 0, 0);
                         sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[7], stage.template operand<7>(), sum, 0, 0, 0);
                         acc[t] = sum;
@@ -785,7 +789,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                 if constexpr (!RING) fetch_advance();
             }
         }
-        // Cross-wave sums in wave order, wave t adds up tile t of the group; the
+        // Cross-wave sums in share order, wave t adds up tile t of the group; the
         // two buffers alternate so one barrier per group is enough.
         float* buffer = partial + (group & 1) * kGroupTiles * kWaves * kWave * 4;
 #pragma unroll
@@ -895,13 +899,17 @@ std::uint32_t grid_of(std::uint32_t tiles, bool argmax) {
     return tiles < slots ? tiles : slots;
 }
 
-// The RING form reads a whole window of Ring::kRowPitch bytes around every block: a
-// projection of one block alone (one row of 256 columns) is shorter than that.
+// Which form a launch takes (16 rows, graph replay, plain -> RING in us):
+//   Q8_0 6,656 -> 16,384: 34.3 -> 32.9, -> 65,536: 120.7 -> 98.3, 16,384 -> 6,656: 40.4 -> 35.6;
+//   Q6_K 6,656 -> 65,536: 93.4 -> 86.4, 2,048 -> 16,384: 22.6 -> 20.6, the lm_head 245 -> 227,
+//        but 16,384 -> 6,656: 35.0 -> 35.9 (its fragments are loaded per group there);
+//   Q4_K 6,656 -> 16,384: 27.8 -> 30.2, Q5_K: 31.0 -> 33.7 (fewer bytes for the same
+//        arithmetic: the extra instructions of a RING step cost more than its loads save).
+template <std::uint32_t ENC>
 bool ring_form(const ProjectionSet& set) {
-    for (int index = 0; index < set.count; ++index) {
-        if (set.op[index].output_dim * (set.input_dim / 256) < 2) return false;
-    }
-    return true;
+    if (ENC == kEncQ8_0) return true;
+    if (ENC == kEncQ6K) return set.input_dim <= 32 * 256;
+    return false;
 }
 
 // `candidates` non-null: the lm_head form (one projection), which returns its workgroup count.
@@ -914,7 +922,7 @@ std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, cons
         tiles += static_cast<std::uint32_t>((set.op[index].output_dim + kTileRows - 1) / kTileRows);
     }
     const std::uint32_t grid = grid_of(tiles, candidates != nullptr);
-    if (ring_form(set)) {
+    if (ring_form<ENC>(set)) {
         constexpr unsigned kLds = Ring<ENC>::kLdsBytes;
         if (candidates != nullptr) {
             hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax, true>), dim3(grid), dim3(kThreads), kLds,
@@ -943,7 +951,7 @@ void launch_pair(const ProjectionSet& set, const std::uint8_t* image, const floa
                  int tokens, hipStream_t stream) {
     const std::uint32_t tiles =
         static_cast<std::uint32_t>((set.op[0].output_dim + kTileRows - 1) / kTileRows);
-    if (ring_form(set)) {
+    if (ring_form<ENC>(set)) {
         hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs, true>), dim3(grid_of(tiles, false)), dim3(kThreads),
                            Ring<ENC>::kLdsBytes, stream, image, inverse_scale, tokens, tiles,
                            static_cast<int>(set.input_dim), static_cast<LmHeadCandidate*>(nullptr), set);

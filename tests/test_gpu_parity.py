@@ -849,6 +849,44 @@ def test_verifier_matrix_core_rows_tensor_two_bytes_off_a_word(cuda, encoding, i
         assert_bits_equal(single, a[rows - 1:rows].contiguous(), "the one-row call on the shifted tensor")
 
 
+@pytest.mark.parametrize("in_dim", [256, 1024, 6656, 6912])
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q5_K, kquant.Q6_K, kquant.Q8_0])
+def test_fp16_rows_last_row_of_a_tensor_and_shifted_tensors(cuda, encoding, in_dim):
+    """The fp16 small-batch kernel brings Q6_K and Q8_0 blocks into LDS in 16-byte pieces from
+    wherever a row starts; the piece behind a tensor's very last block would reach past the
+    tensor and is fetched another way.  The last row of a tensor gives the bits the same row
+    gives inside a taller tensor (where its blocks go the ordinary way), for a last tile of
+    one row and of several, and a tensor that starts one, two or three bytes past a word gives
+    the bits of the aligned one.  (The other tests tie these bits to the oracle.)"""
+    torch = torch_()
+    tall_dim = 53
+    packed = random_packed(encoding, tall_dim, in_dim, 57)
+    tall = tile_ops.PackedWeight.from_numpy(encoding, packed, tall_dim, in_dim)
+    rows = 16
+    x = to_device(kquant.synthetic_activations(58, rows, in_dim), cuda)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    expected = tile_ops.multi_linear([tall], x, workspace)[0]
+    row_bytes = packed.size // tall_dim
+    for out_dim in (1, 16, 17, 37, 48):
+        short = tile_ops.PackedWeight.from_numpy(encoding, packed.reshape(-1)[:out_dim * row_bytes].copy(),
+                                                 out_dim, in_dim)
+        got = tile_ops.multi_linear([short], x, workspace)[0]
+        assert_bits_equal(got, expected[:, :out_dim].contiguous(), f"a tensor of {out_dim} rows")
+    for shift in (1, 2, 3):
+        if shift != 2 and encoding != kquant.Q8_0 and encoding != kquant.Q6_K:
+            continue
+        holder = torch.empty(packed.size + shift, dtype=torch.uint8, device=cuda)
+        holder[shift:].copy_(torch.from_numpy(packed.reshape(-1)))
+        shifted = tile_ops.PackedWeight(encoding, tall_dim, in_dim, holder[shift:])
+        assert shifted.data.data_ptr() % 4 == shift
+        got = tile_ops.multi_linear([shifted], x, workspace)[0]
+        assert_bits_equal(got, expected, f"a tensor {shift} bytes past a word")
+    # the fused argmax over the short tensors' last tile
+    short = tile_ops.PackedWeight.from_numpy(encoding, packed.reshape(-1)[:37 * row_bytes].copy(), 37, in_dim)
+    indices, maxima = tile_ops.lm_head_argmax(short, x)
+    assert torch.equal(maxima.cpu(), expected[:, :37].max(dim=1).values.cpu())
+
+
 @pytest.mark.parametrize("rows", [1, 3, 8, 16])
 def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
     out_dim, in_dim = 5003, 6656
