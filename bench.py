@@ -547,8 +547,8 @@ def lm_head_extra(device, stream, steps: int, warmup: int) -> dict:
     from neuralfn_amd import kquant, tile_ops
     weight = random_packed_on_device(kquant.Q6_K, VOCAB, MODEL_DIM, device, 7)
     result = {}
-    # one row: the streaming dot kernel; four: the int8 matrix-core kernel; eight and sixteen
-    # (a verifier block): the fp16 matrix-core kernel behind its conversion launch
+    # one row: the streaming dot kernel; four, eight and sixteen (a verifier block): the fp16
+    # matrix-core kernel behind its conversion launch
     for rows in (1, 4, 8, 16):
         x = torch.from_numpy(kquant.synthetic_activations(21, rows, MODEL_DIM, True)).to(device)
         nbytes = tile_ops.load().nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, VOCAB)

@@ -25,6 +25,14 @@ namespace {
 constexpr std::int64_t kMaxSmallRows = 16;
 constexpr std::int64_t kMaxOperations = 4;
 constexpr std::int64_t kFirstHalfRows = 5;  // rows from which the fp16 matrix-core kernel takes a batch
+// ... and Q6_K from three rows: its int8 kernel reads the 210-byte blocks lane by lane, the
+// fp16 one brings them into LDS whole (6,656 -> 4,096 at 4 rows: 22.0 -> 19.2 us, the lm_head at
+// 3 and 4 rows: 257 -> 226 us; Q4_K and Q5_K the other way round: 21.7 -> 27.3 us at
+// 6,656 -> 16,384)
+constexpr std::int64_t kFirstHalfRowsQ6 = 3;
+std::int64_t first_half_rows(std::uint32_t encoding) {
+    return encoding == kEncQ6K ? kFirstHalfRowsQ6 : kFirstHalfRows;
+}
 // rows from which the verifier family's Q4_K / Q5_K projections run on the int8 matrix cores
 // (one pass over the weights behind a quantizer launch; below: the dot kernel's token passes,
 // which are faster up to three rows: 9.0 / 12.4 / 13.9 us per launch of the attention
@@ -99,7 +107,7 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
     if (required == 0 || workspace_nbytes < required) return kInvalid;
     // One or two rows, and the verifier entry points at any row count: the
     // vector-ALU kernels.  Otherwise 3 and 4 rows: the int8 matrix-core kernel,
-    // which quantizes inside the kernel; 5..16 rows: the fp16 matrix-core kernel
+    // which quantizes inside the kernel; 5..16 rows (Q6_K: 3..16): the fp16 matrix-core kernel
     // behind its conversion launch (Q8_0 below five rows: its dot kernel).
     // Encodings and widths without either: the float kernel.
     // (two rows are also faster on the dot kernels: they walk the token planes
@@ -118,7 +126,7 @@ int run_small_batch(bool verifier, const Descriptor* const* descriptors, const f
             target = &dot;
         } else if (one_row_arithmetic && gemv_q6_supports(encoding, input_dim)) {
             target = &dot6;
-        } else if (rows >= kFirstHalfRows && !verifier && gemv_f16_supports(encoding, input_dim)) {
+        } else if (rows >= first_half_rows(encoding) && !verifier && gemv_f16_supports(encoding, input_dim)) {
             target = &half;
         } else if (gemv_q8_supports(encoding, input_dim)) {
             target = &dot8;  // Q8_0 below five rows and in the verifier family: its dot kernel
@@ -791,12 +799,13 @@ namespace {
 // Widest input the fp16 form of the lm_head takes: the workspace query does not know the
 // input width and sizes that form's fp16 copy of the rows for this one.
 constexpr std::int64_t kLmHeadHalfWidth = 16384;
-constexpr std::int64_t kLmHeadHalfRows = 5;  // rows from which the fp16 form runs
+// rows from which the fp16 form runs: those of the small-batch call, so that the fused result
+// is the maximum of that call's logits
 constexpr std::int64_t kLmHeadOtherRows = 8;  // rows up to which the other forms run
 
 bool lm_head_half_form(const nfn::Descriptor& weight, std::int64_t rows) {
     // (its kernel keeps row numbers in 32 bits)
-    return rows >= kLmHeadHalfRows && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
+    return rows >= first_half_rows(weight.encoding) && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
         weight.output_dim <= std::numeric_limits<std::int32_t>::max() &&
         nfn::gemv_f16_supports(weight.encoding, weight.input_dim);
 }
@@ -813,7 +822,7 @@ std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
         if (lm_head_mfma_tiles(output_dim) > groups) groups = lm_head_mfma_tiles(output_dim);
         raw = rows * groups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
     }
-    if (rows >= kLmHeadHalfRows) {
+    if (rows >= kFirstHalfRowsQ6) {  // (the query does not know the encoding either)
         raw = std::max(raw, lm_head_f16_workspace_bytes(rows, kLmHeadHalfWidth));
     }
     return (raw + 255) & ~std::int64_t(255);
@@ -832,8 +841,8 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
     const std::int64_t required =
         nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    // Five rows and more: the fp16 matrix-core kernel (one pass over the weights for up to
-    // sixteen rows), the only form beyond eight rows.  Two rows and more: the int8
+    // Five rows and more (Q6_K: three): the fp16 matrix-core kernel (one pass over the weights
+    // for up to sixteen rows), the only form beyond eight rows.  Two rows and more: the int8
     // matrix-core kernel (one pass for up to four rows).  One row of Q6_K: the streaming
     // dot kernel.
     if (lm_head_half_form(normalized, rows)) {

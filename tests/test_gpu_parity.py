@@ -903,7 +903,7 @@ def test_q6_k_long_rows_lm_head(cuda, oracle, rows):
             assert indices.cpu()[row].item() == oracle.argmax(logits[row])
     # the fused result equals argmax over the unfused logits of the same kernel
     workspace = tile_ops.small_batch_workspace(rows, in_dim)
-    family = "mmvq" if rows == 1 else "mmq"  # one row: dot kernel; more: matrix cores (int8 to four rows, fp16 beyond)
+    family = "mmvq" if rows == 1 else "mmq"  # one row: dot kernel; more: matrix cores (fp16 from three rows of Q6_K)
     unfused = tile_ops.multi_linear([weight], to_device(x, cuda), workspace, family=family)[0]
     assert torch_().equal(unfused.max(dim=1).values.cpu(), maxima.cpu())
 
