@@ -316,6 +316,23 @@ __device__ __forceinline__ float wave_sum(float value) {
     return value;
 }
 
+// 16 bytes per lane from `source` (this lane's) to the LDS address `target` (uniform) + 16 x
+// lane; counted by vmcnt like any load.  Written out as an instruction because the compiler
+// holds every later LDS read back until all loads of this kind have landed, which would leave
+// its ring of stages one deep; the kernels that use it wait by count themselves.
+__device__ __forceinline__ void load_to_lds(const __attribute__((address_space(1))) std::uint8_t* source,
+                                            std::uint8_t* target) {
+    const std::uint32_t lds_address = static_cast<std::uint32_t>(
+        reinterpret_cast<std::uintptr_t>((__attribute__((address_space(3))) std::uint8_t*)target));
+    // (m0 carries the LDS address; it is put back, the compiler keeps no account of it)
+    std::uint32_t kept;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+        : "=&s"(kept)
+        : "v"(source), "s"(lds_address)
+        : "memory");
+}
+
 #endif  // __HIPCC__
 
 }  // namespace nfn

@@ -476,20 +476,6 @@ struct Ring {
     static constexpr unsigned kLdsBytes = kWaves * kStages * kStageBytes;
 };
 
-// 16 bytes per lane from `source` (this lane's) to the LDS address `target` (uniform) + 16 x
-// lane; counted by vmcnt like any load.  Written out as an instruction because the compiler
-// holds every later LDS read back until all loads of this kind have landed, which would leave
-// the ring one stage deep; the kernel waits by count itself.
-__device__ __forceinline__ void load_to_lds(const __attribute__((address_space(1))) std::uint8_t* source,
-                                            std::uint8_t* target) {
-    const std::uint32_t lds_address = static_cast<std::uint32_t>(
-        reinterpret_cast<std::uintptr_t>((__attribute__((address_space(3))) std::uint8_t*)target));
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                 :
-                 : "v"(source), "s"(lds_address)
-                 : "memory", "m0");
-}
-
 // A tile of 16 weight rows as both the fetching and the multiplying side see it (uniform).
 struct TileShape {
     const __attribute__((address_space(1))) std::uint8_t* base;  // its first row
