@@ -18,7 +18,10 @@
 // The K index of a matrix instruction is only a pairing of A and B elements,
 // so every format picks the eight columns a lane contributes from the bytes
 // it already holds; the activation address follows that choice.  Weights are
-// read from HBM once; no weight byte goes through LDS.
+// read from HBM once.  Q4_K and Q5_K bytes go from memory to the registers of
+// the lane that decodes them; Q6_K (rows of up to 8,192 columns) and Q8_0
+// blocks are brought into a per-wave ring in LDS first, whole, and read from
+// there (the RING form below, with the measurements that chose it).
 //
 // Arithmetic it replaces: the reference's small-batch kernel
 // (neuralfn/csrc/tile_cuda/glimmer_k_mmq.cu:1174-1303), which multiplies 8-bit
