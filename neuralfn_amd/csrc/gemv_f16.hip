@@ -914,10 +914,12 @@ std::uint32_t launch_encoding(ProjectionSet set, const std::uint8_t* image, cons
     if (ring_form<ENC>(set)) {
         constexpr unsigned kLds = Ring<ENC>::kLdsBytes;
         if (candidates != nullptr) {
+            allow_large_lds<gemv_f16_kernel<ENC, kArgmax, true>>(kLds);  // (beside 36 KB of static LDS)
             hipLaunchKernelGGL((gemv_f16_kernel<ENC, kArgmax, true>), dim3(grid), dim3(kThreads), kLds,
                                stream, image, inverse_scale, tokens, tiles,
                                static_cast<int>(set.input_dim), candidates, set);
         } else {
+            allow_large_lds<gemv_f16_kernel<ENC, kStore, true>>(kLds);
             hipLaunchKernelGGL((gemv_f16_kernel<ENC, kStore, true>), dim3(grid), dim3(kThreads), kLds,
                                stream, image, inverse_scale, tokens, tiles,
                                static_cast<int>(set.input_dim), candidates, set);
@@ -941,6 +943,7 @@ void launch_pair(const ProjectionSet& set, const std::uint8_t* image, const floa
     const std::uint32_t tiles =
         static_cast<std::uint32_t>((set.op[0].output_dim + kTileRows - 1) / kTileRows);
     if (ring_form<ENC>(set)) {
+        allow_large_lds<gemv_f16_kernel<ENC, kPairs, true>>(Ring<ENC>::kLdsBytes);
         hipLaunchKernelGGL((gemv_f16_kernel<ENC, kPairs, true>), dim3(grid_of(tiles, false)), dim3(kThreads),
                            Ring<ENC>::kLdsBytes, stream, image, inverse_scale, tokens, tiles,
                            static_cast<int>(set.input_dim), static_cast<LmHeadCandidate*>(nullptr), set);
