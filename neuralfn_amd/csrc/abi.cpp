@@ -800,12 +800,16 @@ namespace {
 // input width and sizes that form's fp16 copy of the rows for this one.
 constexpr std::int64_t kLmHeadHalfWidth = 16384;
 // rows from which the fp16 form runs: those of the small-batch call, so that the fused result
-// is the maximum of that call's logits
+// is the maximum of that call's logits; two rows of Q6_K as well (there the small-batch call
+// keeps the one-row arithmetic, which no fused form of two rows has: 249 -> 225 us)
 constexpr std::int64_t kLmHeadOtherRows = 8;  // rows up to which the other forms run
+constexpr std::int64_t kLmHeadFirstHalfRowsQ6 = 2;
 
 bool lm_head_half_form(const nfn::Descriptor& weight, std::int64_t rows) {
+    const std::int64_t first_rows =
+        weight.encoding == nfn::kEncQ6K ? kLmHeadFirstHalfRowsQ6 : first_half_rows(weight.encoding);
     // (its kernel keeps row numbers in 32 bits)
-    return rows >= first_half_rows(weight.encoding) && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
+    return rows >= first_rows && rows <= 16 && weight.input_dim <= kLmHeadHalfWidth &&
         weight.output_dim <= std::numeric_limits<std::int32_t>::max() &&
         nfn::gemv_f16_supports(weight.encoding, weight.input_dim);
 }
@@ -822,7 +826,7 @@ std::int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(std::int64_t rows,
         if (lm_head_mfma_tiles(output_dim) > groups) groups = lm_head_mfma_tiles(output_dim);
         raw = rows * groups * static_cast<std::int64_t>(sizeof(LmHeadCandidate));
     }
-    if (rows >= kFirstHalfRowsQ6) {  // (the query does not know the encoding either)
+    if (rows >= kLmHeadFirstHalfRowsQ6) {  // (the query does not know the encoding either)
         raw = std::max(raw, lm_head_f16_workspace_bytes(rows, kLmHeadHalfWidth));
     }
     return (raw + 255) & ~std::int64_t(255);
@@ -841,7 +845,7 @@ int nfn_mi355_lm_head_argmax_v1(const Descriptor* descriptor, const float* input
     const std::int64_t required =
         nfn_mi355_lm_head_argmax_workspace_bytes_v1(rows, normalized.output_dim);
     if (required == 0 || workspace_nbytes < required) return kInvalid;
-    // Five rows and more (Q6_K: three): the fp16 matrix-core kernel (one pass over the weights
+    // Five rows and more (Q6_K: two): the fp16 matrix-core kernel (one pass over the weights
     // for up to sixteen rows), the only form beyond eight rows.  Two rows and more: the int8
     // matrix-core kernel (one pass for up to four rows).  One row of Q6_K: the streaming
     // dot kernel.
