@@ -848,7 +848,7 @@ int nfn_mi355_abi_version(void);
  * is both in one call.  rows 1..16 (a verifier block); beyond 8 rows for the
  * four packed formats at an input_dim of at most 16,384, for which the
  * workspace query, which does not know input_dim, sizes the fp16 copy of the
- * rows that the 5..16-row form (Q6_K: 3..16) keeps there.  Ties go to the lowest index; NaN
+ * rows that the 5..16-row form (Q6_K: 2..16) keeps there.  Ties go to the lowest index; NaN
  * never wins.  output_indices: int64[rows]; output_values: float[rows]. */
 int64_t nfn_mi355_lm_head_argmax_workspace_bytes_v1(int64_t rows, int64_t output_dim);
 int nfn_mi355_lm_head_argmax_v1(
