@@ -480,8 +480,12 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
     const int j = lane & 31;
     const int kc = lane >> 5;
     const std::int64_t blocks = input_dim >> 8;
-    const std::int64_t begin = blocks * wave / kWaves;
-    const std::int64_t end = blocks * (wave + 1) / kWaves;
+    // K is cut into kWaves shares; which wave takes which is free (the sums meet in share
+    // order).  Waves w and w + 4 run on one SIMD: with this choice the shares that are one
+    // block longer than the others spread over the four SIMDs (26 blocks: shares 3 and 7).
+    const int share = (0x63571240 >> (4 * wave)) & 7;
+    const std::int64_t begin = blocks * share / kWaves;
+    const std::int64_t end = blocks * (share + 1) / kWaves;
     const int count = static_cast<int>(end - begin);
     const int max_count = static_cast<int>((blocks + kWaves - 1) / kWaves);
 
@@ -657,7 +661,7 @@ __global__ __launch_bounds__(kThreads) void gemv_mfma_kernel(
             if (++work_step == steps) {
                 // Cross-wave sum in a fixed order; the two buffers alternate so
                 // one barrier per tile is enough.
-                float* mine = partial + ((parity * kWaves + wave) * kWave + lane) * S;
+                float* mine = partial + ((parity * kWaves + share) * kWave + lane) * S;
 #pragma unroll
                 for (int u = 0; u < S; ++u) mine[u] = acc[u];
                 __syncthreads();
