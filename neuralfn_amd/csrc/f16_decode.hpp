@@ -39,8 +39,9 @@ __device__ __forceinline__ void scale_bytes(std::uint32_t word, f16x2 bias, f16x
 }
 
 // The fp16 copy of a small batch of activation rows that the small-batch kernel reads
-// (gemv_f16.hip): [column / 8][row][8 halfs], every row scaled by a power of two so that its
-// largest magnitude lands near 2^14, and one float per row to multiply results back.
+// (gemv_f16.hip): [column / 8][row][8 halfs], every K share of a row (below) scaled by a power
+// of two so that its largest magnitude lands near 2^14, and one float per row and share,
+// [row][share], to multiply results back.
 struct HalfImageScale {
     float factor, inverse;
 };
@@ -55,6 +56,19 @@ __device__ __forceinline__ HalfImageScale half_image_scale(float largest) {
 }
 __device__ __forceinline__ float largest_of(float4 x, float largest) {
     return fmaxf(largest, fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+}
+// The small-batch kernel's eight waves cut K into shares of whole blocks, share s being blocks
+// blocks * s / 8 .. blocks * (s + 1) / 8, and every (row, share) has a scale of its own: a
+// wave multiplies its partial sums back before the waves' sums meet.  (One scale per row
+// would need the whole row before the first value can be stored; per share, the workgroups
+// that convert a row share nothing.)
+constexpr int kHalfImageShares = 8;
+__host__ __device__ constexpr int half_image_share_begin(int blocks, int share) {
+    return blocks * share / kHalfImageShares;
+}
+// the share that block `block` belongs to
+__host__ __device__ constexpr int half_image_share_of(int block, int blocks) {
+    return (kHalfImageShares * block + kHalfImageShares - 1) / blocks;
 }
 // columns 8 group .. 8 group + 7 of row `row` (a, then b) into the image of `rows` rows
 __device__ __forceinline__ void half_image_store(std::uint8_t* image, int group, int rows, int row,

@@ -1,8 +1,9 @@
 // Small-batch (3..16 rows) GEMV on the fp16 matrix cores.
 //
-// A small launch first turns the activations into fp16, every row scaled by
-// the power of two that brings its largest magnitude into [2^14, 2^15), and
-// stores them in the caller's workspace by groups of eight columns:
+// A small launch first turns the activations into fp16, every K share of a
+// row (the blocks one wave of the main kernel multiplies) scaled by the power
+// of two that brings its largest magnitude into [2^14, 2^15), and stores them
+// in the caller's workspace by groups of eight columns:
 // [column / 8][row][8 values], so that the 16 bytes one lane feeds to a matrix
 // instruction are contiguous and the lanes of a quarter wave read one segment.
 // Fused prologues (sigmoid gate, SwiGLU) are applied there.
@@ -51,20 +52,24 @@ constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kDepth = 4;  // blocks in flight per wave
 
-// ---- activations: fp32 -> row-scaled fp16, [column / 8][row][8] ----------------
+// ---- activations: fp32 -> fp16 scaled per row and K share, [column / 8][row][8] ----
 
-constexpr int kImageThreads = 1024;  // there are at most 16 rows: a large workgroup per row
-constexpr int kImageHeld = 2;  // 8-column groups a thread keeps: rows of up to 16,384 columns are read once
+constexpr int kImageThreads = 256;
+constexpr int kImageHeld = 2;  // 8-column groups a thread keeps: shares of up to 16 blocks are read once
+static_assert(kHalfImageShares == kWaves, "a share of the image is a wave's share of K");
 
-// One workgroup per row.
+// One workgroup per (row, share): blockIdx.x = row * kWaves + share.
 template <int P>
 __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
     const float* __restrict__ first, const float* __restrict__ second,
     std::uint8_t* __restrict__ image, float* __restrict__ inverse_scale, int tokens,
     int input_dim) {
     __shared__ float maxima[kImageThreads / kWave];
-    const int token = blockIdx.x;
-    const int groups = input_dim >> 3;
+    const int token = blockIdx.x / kWaves;
+    const int share = blockIdx.x - token * kWaves;
+    const int blocks = input_dim >> 8;
+    const int group0 = 32 * half_image_share_begin(blocks, share);  // 32 groups of 8 columns a block
+    const int groups = 32 * half_image_share_begin(blocks, share + 1) - group0;
     const std::int64_t base = static_cast<std::int64_t>(token) * input_dim;
     const bool held = groups <= kImageThreads * kImageHeld;  // uniform
     float4 x[kImageHeld][2];
@@ -76,19 +81,19 @@ __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
             x[j][0] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             x[j][1] = x[j][0];
             if (g < groups) {
-                x[j][0] = load_activations<P>(first, second, base + g * 8);
-                x[j][1] = load_activations<P>(first, second, base + g * 8 + 4);
+                x[j][0] = load_activations<P>(first, second, base + (group0 + g) * 8);
+                x[j][1] = load_activations<P>(first, second, base + (group0 + g) * 8 + 4);
             }
         }
 #pragma unroll
         for (int j = 0; j < kImageHeld; ++j) largest = largest_of(x[j][1], largest_of(x[j][0], largest));
     } else {
         for (int g = threadIdx.x; g < groups; g += kImageThreads) {
-            largest = largest_of(load_activations<P>(first, second, base + g * 8), largest);
-            largest = largest_of(load_activations<P>(first, second, base + g * 8 + 4), largest);
+            largest = largest_of(load_activations<P>(first, second, base + (group0 + g) * 8), largest);
+            largest = largest_of(load_activations<P>(first, second, base + (group0 + g) * 8 + 4), largest);
         }
     }
-    // NaN never wins fmaxf: a row with NaN keeps its largest finite magnitude
+    // NaN never wins fmaxf: a share with NaN keeps its largest finite magnitude
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) largest = fmaxf(largest, __shfl_xor(largest, offset));
     if ((threadIdx.x & 63) == 0) maxima[threadIdx.x >> 6] = largest;
@@ -96,9 +101,9 @@ __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
 #pragma unroll
     for (int w = 0; w < kImageThreads / kWave; ++w) largest = fmaxf(largest, maxima[w]);
     const HalfImageScale scale = half_image_scale(largest);
-    if (threadIdx.x == 0) inverse_scale[token] = scale.inverse;
+    if (threadIdx.x == 0) inverse_scale[token * kWaves + share] = scale.inverse;
     auto store = [&](int g, float4 a, float4 b) {
-        half_image_store(image, g, tokens, token, a, b, scale.factor);
+        half_image_store(image, group0 + g, tokens, token, a, b, scale.factor);
     };
     if (held) {
 #pragma unroll
@@ -108,8 +113,8 @@ __global__ __launch_bounds__(kImageThreads) void f16_image_kernel(
         }
     } else {
         for (int g = threadIdx.x; g < groups; g += kImageThreads) {
-            store(g, load_activations<P>(first, second, base + g * 8),
-                  load_activations<P>(first, second, base + g * 8 + 4));
+            store(g, load_activations<P>(first, second, base + (group0 + g) * 8),
+                  load_activations<P>(first, second, base + (group0 + g) * 8 + 4));
         }
     }
 }
@@ -538,10 +543,11 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         }
     };
 
-    // register r of quarter j of the result: token 4j + r
-    float token_scale[4];
+    // register r of quarter j of the result: token 4j + r; what this wave's sums of that token
+    // are multiplied back by (the scale of the token's share of K that the wave has)
+    f32x4 token_scale;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) token_scale[r] = inverse_scale[min(4 * j + r, tokens - 1)];
+    for (int r = 0; r < 4; ++r) token_scale[r] = inverse_scale[min(4 * j + r, tokens - 1) * kWaves + share];
 
     // this workgroup's tiles: blockIdx.x + n * gridDim.x
     const int tile_count =
@@ -785,7 +791,8 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
 #pragma unroll
         for (int t = 0; t < kGroupTiles; ++t) {
             if (t < group_tiles) {
-                *reinterpret_cast<f32x4*>(buffer + ((t * kWaves + share) * kWave + lane) * 4) = acc[t];
+                *reinterpret_cast<f32x4*>(buffer + ((t * kWaves + share) * kWave + lane) * 4) =
+                    acc[t] * token_scale;
             }
         }
         __syncthreads();
@@ -805,7 +812,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                     const int token = 4 * j + r;
                     if (token < tokens && row < set.op[0].output_dim) {
                         set.op[0].output[static_cast<std::int64_t>(token) * set.op[0].output_dim + row] =
-                            apply_prologue<kSwiGlu>(first[r] * token_scale[r], second[r] * token_scale[r]);
+                            apply_prologue<kSwiGlu>(first[r], second[r]);
                     }
                 }
             }
@@ -827,7 +834,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                 i32x4 best_row = best_rows[wave * kWave + lane];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float result = sum[r] * token_scale[r];
+                    const float result = sum[r];
                     // rows past the end and NaN results stand back; a later tile's rows are
                     // higher, so that an equal result does not replace an earlier one
                     const bool wins = row < op.output_dim && result > best_value[r];
@@ -841,8 +848,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
                 for (int r = 0; r < 4; ++r) {
                     const int token = 4 * j + r;
                     if (token < tokens && row < op.output_dim) {
-                        op.output[static_cast<std::int64_t>(token) * op.output_dim + row] =
-                            sum[r] * token_scale[r];
+                        op.output[static_cast<std::int64_t>(token) * op.output_dim + row] = sum[r];
                     }
                 }
             }
@@ -977,7 +983,7 @@ bool gemv_f16_supports(std::uint32_t encoding, std::int64_t input_dim) {
 }
 
 std::int64_t gemv_f16_workspace_bytes(std::int64_t rows, std::int64_t input_dim) {
-    return rows * input_dim * 2 + rows * 4;
+    return rows * input_dim * 2 + rows * kWaves * 4;
 }
 
 void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* second, int prologue,
@@ -986,7 +992,7 @@ void launch_gemv_f16(const ProjectionSet& set, const float* first, const float* 
     float* inverse_scale = reinterpret_cast<float*>(image + rows * set.input_dim * 2);
     const int tokens = static_cast<int>(rows);
     const int input_dim = static_cast<int>(set.input_dim);
-    const dim3 grid(static_cast<unsigned>(rows));
+    const dim3 grid(static_cast<unsigned>(rows * kWaves));
     switch (prologue) {
         case kHalfImage:  // an earlier launch left the image in the workspace
             break;
@@ -1027,7 +1033,7 @@ void launch_gemv_f16_pairs(const ProjectionSet& set, const float* input, std::in
     float* inverse_scale = reinterpret_cast<float*>(image + rows * set.input_dim * 2);
     const int tokens = static_cast<int>(rows);
     if (input != nullptr) {
-        hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows)),
+        hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows * kWaves)),
                            dim3(kImageThreads), 0, stream, input, nullptr, image, inverse_scale, tokens,
                            static_cast<int>(set.input_dim));
     }
@@ -1042,7 +1048,7 @@ void launch_gemv_f16_pairs(const ProjectionSet& set, const float* input, std::in
 // Workspace of the lm_head form: the fp16 copy and its row scales, then the candidates.
 namespace {
 std::int64_t lm_head_image_bytes(std::int64_t rows, std::int64_t input_dim) {
-    return (rows * input_dim * 2 + rows * 4 + 255) & ~std::int64_t(255);
+    return (rows * input_dim * 2 + rows * kWaves * 4 + 255) & ~std::int64_t(255);
 }
 }  // namespace
 
@@ -1058,7 +1064,7 @@ void launch_lm_head_f16(const Descriptor& descriptor, const float* input, std::i
     LmHeadCandidate* candidates =
         reinterpret_cast<LmHeadCandidate*>(image + lm_head_image_bytes(rows, descriptor.input_dim));
     const int tokens = static_cast<int>(rows);
-    hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows)),
+    hipLaunchKernelGGL((f16_image_kernel<kPlain>), dim3(static_cast<unsigned>(rows * kWaves)),
                        dim3(kImageThreads), 0, stream, input, nullptr, image, inverse_scale, tokens,
                        static_cast<int>(descriptor.input_dim));
     ProjectionSet set{};

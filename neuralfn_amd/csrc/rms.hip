@@ -163,7 +163,7 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     __shared__ float partials[kRmsThreads + 1];
     __shared__ __attribute__((aligned(16))) float handed[kOwned * kRmsThreads];  // [k][t]: column t + 256 k
     extern __shared__ __attribute__((aligned(16))) float staged[];  // HANDOFF 1, 3: the normalized row
-    __shared__ float wave_largest[kWideThreads / kWave];
+    __shared__ float share_factor[kHalfImageShares];  // HANDOFF 2: what a share's columns are multiplied by
     const std::int64_t row = blockIdx.x;
     const float* source = input + row * width;
     const float* residual = residual_input + row * width;
@@ -221,7 +221,6 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
     const float second_inverse =
         1.0f / sqrtf(rms_tree_total(ordered_sum(), partials) / static_cast<float>(width) + second_eps);
 
-    float largest = 0.0f;
 #pragma unroll
     for (int i = 0; i < kLoaded; ++i) {
         const int column = t + (q + kLoaders * i) * kRmsThreads;
@@ -231,28 +230,42 @@ __global__ __launch_bounds__(kWideThreads) void dual_rms_resident_kernel(
             if constexpr (HANDOFF == 1 || HANDOFF == 3) staged[column] = result;
             // (the sums have read `handed`: tree_total_wide's barriers lie in between)
             if constexpr (HANDOFF == 2) handed[column] = result;
-            largest = fmaxf(largest, fabsf(result));
         }
     }
 
     if constexpr (HANDOFF == 2) {
-        // what f16_image_kernel would make of the normalized row, bit for bit
-#pragma unroll
-        for (int offset = 32; offset > 0; offset >>= 1) largest = fmaxf(largest, __shfl_xor(largest, offset));
-        if ((threadIdx.x & 63) == 0) wave_largest[threadIdx.x >> 6] = largest;
-        __syncthreads();
-#pragma unroll
-        for (int w = 0; w < kWideThreads / kWave; ++w) largest = fmaxf(largest, wave_largest[w]);
-        const HalfImageScale scale = half_image_scale(largest);
+        // what f16_image_kernel would make of the normalized row, bit for bit: every K share of
+        // the row (f16_decode.hpp) with the scale of its own largest magnitude
+        static_assert(kWideThreads / kWave >= kHalfImageShares, "a wave per share");
+        __syncthreads();  // the row is in `handed`
         const int rows = static_cast<int>(gridDim.x);
+        const int blocks = width >> 8;
         float* inverse_scale =
             reinterpret_cast<float*>(records + static_cast<std::int64_t>(rows) * width * 2);
-        if (threadIdx.x == 0) inverse_scale[row] = scale.inverse;
+        const int share = threadIdx.x >> 6;
+        if (share < kHalfImageShares) {
+            const int end = 256 * half_image_share_begin(blocks, share + 1);
+            float share_largest = 0.0f;
+            for (int column = 256 * half_image_share_begin(blocks, share) + (threadIdx.x & 63); column < end;
+                 column += kWave) {
+                share_largest = fmaxf(share_largest, fabsf(handed[column]));
+            }
+#pragma unroll
+            for (int offset = 32; offset > 0; offset >>= 1) {
+                share_largest = fmaxf(share_largest, __shfl_xor(share_largest, offset));
+            }
+            const HalfImageScale scale = half_image_scale(share_largest);
+            if ((threadIdx.x & 63) == 0) {
+                share_factor[share] = scale.factor;
+                inverse_scale[row * kHalfImageShares + share] = scale.inverse;
+            }
+        }
+        __syncthreads();
         for (int group = threadIdx.x; group < (width >> 3); group += kWideThreads) {
             half_image_store(records, group, rows, static_cast<int>(row),
                              *reinterpret_cast<const float4*>(handed + group * 8),
                              *reinterpret_cast<const float4*>(handed + group * 8 + 4),
-                             scale.factor);
+                             share_factor[half_image_share_of(group >> 5, blocks)]);
         }
     }
 
