@@ -1526,6 +1526,29 @@ def test_prefill_gemm_multi_equals_single_calls(cuda, oracle):
     torch_().cuda.synchronize()
 
 
+@pytest.mark.parametrize("encoding", [kquant.Q4_K, kquant.Q6_K])
+def test_fp16_rows_activation_range(cuda, oracle, encoding):
+    """The fp16 small-batch kernel scales every eighth of K of a row by its own power of two:
+    rows far outside the fp16 range, a zero row, a row whose eighths differ by twelve orders of
+    magnitude and a row with an eighth of zeros keep the bound."""
+    rows, out_dim, in_dim = 8, 96, 2048
+    packed = kquant.quantize(encoding, kquant.synthetic_weights(78, out_dim, in_dim))
+    x = kquant.synthetic_activations(74, rows, in_dim)
+    x *= np.array([1.0, 1.0e6, 1.0e-6, 3.0e20, 2.0e-22, 0.0, 1.0, 1.0], dtype=np.float32)[:, None]
+    x[6, :256] *= 1.0e6
+    x[6, 1280:1536] *= 1.0e-6
+    x[7, 512:768] = 0.0
+    weight = tile_ops.PackedWeight.from_numpy(encoding, packed, out_dim, in_dim)
+    workspace = tile_ops.small_batch_workspace(rows, in_dim)
+    y = tile_ops.multi_linear([weight], to_device(x, cuda), workspace)[0].cpu().numpy()
+    expected = oracle.linear(encoding, packed, out_dim, in_dim, x)
+    for row in range(rows):
+        if row == 5:
+            assert np.all(y[row] == 0.0)
+        else:
+            assert normalised_error(y[row:row + 1], expected[row:row + 1]) <= TOLERANCE
+
+
 def test_prefill_gemm_activation_range(cuda, oracle):
     # rows scaled far outside the fp16 range, and a zero row: the per-row power
     # of two keeps every row at the same relative accuracy
