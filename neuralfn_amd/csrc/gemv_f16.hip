@@ -720,8 +720,13 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         ahead.load_tile(my_ring + read_stage * Lds::kStageBytes + i * Lds::kRowPitch, j);
         read_stage = read_stage + 1 == Lds::kStages ? 0 : read_stage + 1;
     };
+    // RING, rows of one chunk: the launch's only fragments are requested with the first weights,
+    // not behind the wait for them
+    const bool fragments_first = RING && chunks == 1;
     if constexpr (RING) {
         ring_enter();
+        // (ahead of the weights, so that the first step's wait by count covers them)
+        if (fragments_first) load_fragments(0);
 #pragma unroll
         for (int s = 0; s < Lds::kStages; ++s) ring_issue();
         ring_read_ahead();
@@ -749,7 +754,7 @@ __global__ __launch_bounds__(kThreads) void gemv_f16_kernel(
         for (int t = 0; t < kGroupTiles; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         const int group_tiles = tiles_of_group(group);
         for (int chunk = 0; chunk < chunks; ++chunk) {
-            if (chunks > 1 || group == 0) load_fragments(chunk);
+            if (chunks > 1 || (group == 0 && !fragments_first)) load_fragments(chunk);
             const int chunk_count = min(kDepth, count - chunk * kDepth);  // this wave's blocks of the chunk
 #pragma unroll
             for (int t = 0; t < kGroupTiles; ++t) {
